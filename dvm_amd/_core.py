@@ -1,0 +1,421 @@
+"""ctypes binding of libdvm.so (include/dvm_c.h).
+
+Mirrors the classes of the reference's pybind module `_dvm_py`
+(include/dvm_py.h:277-388, src/pybind_api.cc:1066-1116): DataType, NDObject,
+IntArrayRef, ScalarRef, Kernel (graph builder), PyKernel (builder + runner) and
+Device, with the same method names and argument meaning.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+_LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
+_LIB_PATH = os.path.join(_LIB_DIR, "libdvm.so")
+
+
+class _Operand(ctypes.Structure):
+    _fields_ = [("kind", ctypes.c_int), ("obj", ctypes.c_void_p), ("ref", ctypes.c_void_p),
+                ("f", ctypes.c_double), ("i", ctypes.c_int64)]
+
+
+def _load():
+    if not os.path.exists(_LIB_PATH):
+        raise ImportError(
+            "dvm_amd native library missing (%s): run `python -m dvm_amd.build` first" % _LIB_PATH)
+    lib = ctypes.CDLL(_LIB_PATH)
+    vp, ci, cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
+    i64p = ctypes.POINTER(ctypes.c_int64)
+    opp = ctypes.POINTER(_Operand)
+    sig = {
+        "dvm_c_last_error": (ctypes.c_char_p, []),
+        "dvm_rt_new": (vp, [ctypes.c_char_p, ctypes.c_char_p, ci]),
+        "dvm_rt_delete": (None, [vp]),
+        "dvm_rt_reset": (ci, [vp]),
+        "dvm_rt_new_shape": (vp, [vp, i64p, cs]),
+        "dvm_shape_update": (ci, [vp, i64p, cs]),
+        "dvm_rt_new_scalar": (vp, [vp, ci]),
+        "dvm_scalar_update_f": (ci, [vp, ctypes.c_double]),
+        "dvm_scalar_update_i": (ci, [vp, ctypes.c_int64]),
+        "dvm_rt_load": (vp, [vp, vp, ci]),
+        "dvm_rt_store": (vp, [vp, vp]),
+        "dvm_rt_unary": (vp, [vp, ci, vp]),
+        "dvm_rt_binary": (vp, [vp, ci, opp, opp]),
+        "dvm_rt_select": (vp, [vp, vp, vp, vp]),
+        "dvm_rt_cast": (vp, [vp, vp, ci]),
+        "dvm_rt_broadcast": (vp, [vp, vp, vp]),
+        "dvm_rt_full": (vp, [vp, opp, vp, ci]),
+        "dvm_rt_reshape": (vp, [vp, vp, vp]),
+        "dvm_rt_reduce": (vp, [vp, ci, vp, vp, ci]),
+        "dvm_rt_copy": (vp, [vp, vp]),
+        "dvm_rt_matmul": (vp, [vp, vp, vp, ci, ci, vp]),
+        "dvm_rt_set_store_inplace": (ci, [vp, vp]),
+        "dvm_obj_rank": (ci, [vp]),
+        "dvm_obj_shape": (ci, [vp, i64p, cs]),
+        "dvm_obj_dtype": (ci, [vp]),
+        "dvm_rt_input": (ci, [vp, vp, vp, cs]),
+        "dvm_rt_bind_device": (ci, [vp, vp, vp]),
+        "dvm_rt_codegen": (ci, [vp]),
+        "dvm_rt_jit_us": (ctypes.c_double, [vp]),
+        "dvm_rt_run": (ci, [vp, vp, ci]),
+        "dvm_rt_output": (ci, [vp, vp, vp, cs]),
+        "dvm_rt_device_ptr": (vp, [vp, vp]),
+        "dvm_rt_perf": (ci, [vp, ci, ci, ctypes.POINTER(ctypes.c_double)]),
+        "dvm_rt_num_launches": (ci, [vp]),
+        "dvm_rt_workspace_bytes": (cs, [vp]),
+        "dvm_rt_das": (ctypes.c_char_p, [vp]),
+        "dvm_rt_dump": (ctypes.c_char_p, [vp]),
+        "dvm_rt_dump_r": (ctypes.c_char_p, [vp]),
+        "dvm_rt_inspect": (ctypes.c_char_p, [vp]),
+        "dvm_c_f32_to_bf16": (None, [vp, vp, cs]),
+        "dvm_c_bf16_to_f32": (None, [vp, vp, cs]),
+        "dvm_c_has_device": (ci, []),
+        "dvm_c_core_num": (ci, []),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    return lib
+
+
+_lib = _load()
+
+
+def _check(ret):
+    if ret is None or (isinstance(ret, int) and ret != 0 and not isinstance(ret, bool)):
+        raise RuntimeError(_lib.dvm_c_last_error().decode())
+    return ret
+
+
+def _ptr(ret):
+    if not ret:
+        raise RuntimeError(_lib.dvm_c_last_error().decode())
+    return ret
+
+
+class DataType(int):
+    """Element types; values match dvm::DataType (include/dvm.h)."""
+    _names = {0: "bool", 1: "float16", 2: "bfloat16", 3: "float32", 4: "int32", 5: "int64"}
+
+    def __repr__(self):
+        return "DataType." + self._names.get(int(self), str(int(self)))
+
+    __str__ = __repr__
+
+
+DataType.bool = DataType(0)
+DataType.float16 = DataType(1)
+DataType.bfloat16 = DataType(2)
+DataType.float32 = DataType(3)
+DataType.int32 = DataType(4)
+DataType.int64 = DataType(5)
+
+_NP_OF = {0: np.bool_, 1: np.float16, 2: np.uint16, 3: np.float32, 4: np.int32}
+_ITEMSIZE = {0: 1, 1: 2, 2: 2, 3: 4, 4: 4}
+
+
+def _i64(seq):
+    arr = (ctypes.c_int64 * max(1, len(seq)))(*[int(v) for v in seq])
+    return arr, len(seq)
+
+
+class NDObject:
+    def __init__(self, handle):
+        self._h = handle
+
+    def shape(self):
+        buf = (ctypes.c_int64 * 10)()
+        r = _lib.dvm_obj_shape(self._h, buf, 10)
+        return tuple(buf[i] for i in range(r))
+
+    def dtype(self):
+        return DataType(_lib.dvm_obj_dtype(self._h))
+
+
+class IntArrayRef:
+    """A shape (or axis list) whose values can change between codegen calls."""
+
+    def __init__(self, rt, shape=()):
+        arr, n = _i64(shape)
+        self._h = _ptr(_lib.dvm_rt_new_shape(rt, arr, n))
+        self._shape = tuple(int(v) for v in shape)
+
+    def shape(self):
+        return self._shape
+
+    def update(self, shape):
+        arr, n = _i64(shape)
+        _lib.dvm_shape_update(self._h, arr, n)
+        self._shape = tuple(int(v) for v in shape)
+
+
+class ScalarRef:
+    """A scalar whose value is read again at every codegen."""
+
+    def __init__(self, rt, dtype):
+        self._h = _ptr(_lib.dvm_rt_new_scalar(rt, int(dtype)))
+
+    def update(self, value):
+        if isinstance(value, (int, np.integer)) and not isinstance(value, bool):
+            _lib.dvm_scalar_update_i(self._h, int(value))
+        else:
+            _lib.dvm_scalar_update_f(self._h, float(value))
+
+
+_UNARY = ["sqrt", "abs", "log", "exp", "reciprocal", "isfinite", "logical_not", "round", "floor", "ceil", "trunc"]
+_BINARY = ["equal", "not_equal", "greater", "greater_equal", "less", "less_equal", "add", "sub", "mul", "div", "pow",
+           "maximum", "minimum", "logical_and", "logical_or"]
+
+
+class Kernel:
+    """Graph builder; method names follow include/dvm_py.h:301-387."""
+
+    K_VEC, K_CUBE, K_MIX, K_PARAL, K_SEQ, K_SPLIT, K_EAGER = range(7)
+    F_DYN, F_UWS, F_SPEC = 1, 2, 4
+
+    def __init__(self):
+        self._rt = None
+        self._keep = []
+
+    # -- references --
+    def _shape_ref(self, shape):
+        if isinstance(shape, IntArrayRef):
+            return shape
+        ref = IntArrayRef(self._rt, list(shape))
+        self._keep.append(ref)
+        return ref
+
+    def int_array(self):
+        ref = IntArrayRef(self._rt, [])
+        self._keep.append(ref)
+        return ref
+
+    def scalar(self, dtype=DataType.float32):
+        ref = ScalarRef(self._rt, dtype)
+        self._keep.append(ref)
+        return ref
+
+    def _operand(self, v):
+        o = _Operand()
+        if isinstance(v, NDObject):
+            o.kind, o.obj = 0, v._h
+        elif isinstance(v, ScalarRef):
+            o.kind, o.ref = 3, v._h
+        elif isinstance(v, (bool, np.bool_)):
+            o.kind, o.i = 2, int(v)
+        elif isinstance(v, (int, np.integer)):
+            o.kind, o.i = 2, int(v)
+        elif isinstance(v, (float, np.floating)):
+            o.kind, o.f = 1, float(v)
+        else:
+            raise TypeError("unsupported operand: %r" % (v,))
+        return o
+
+    def _wrap(self, h):
+        return NDObject(_ptr(h))
+
+    # -- tensor access --
+    def load(self, shape, type):
+        return self._wrap(_lib.dvm_rt_load(self._rt, self._shape_ref(shape)._h, int(type)))
+
+    def store(self, obj, type=None):
+        if type is not None and int(type) != int(obj.dtype()):
+            obj = self.cast(obj, type)
+        return self._wrap(_lib.dvm_rt_store(self._rt, obj._h))
+
+    def set_store_inplace(self, store):
+        _check(_lib.dvm_rt_set_store_inplace(self._rt, store._h))
+
+    # -- operators --
+    def cast(self, input, type):
+        return self._wrap(_lib.dvm_rt_cast(self._rt, input._h, int(type)))
+
+    def select(self, cond, lhs, rhs):
+        return self._wrap(_lib.dvm_rt_select(self._rt, cond._h, lhs._h, rhs._h))
+
+    def broadcast(self, input, shape):
+        return self._wrap(_lib.dvm_rt_broadcast(self._rt, input._h, self._shape_ref(shape)._h))
+
+    def full(self, scalar, shape, dtype):
+        op = self._operand(scalar)
+        return self._wrap(_lib.dvm_rt_full(self._rt, ctypes.byref(op), self._shape_ref(shape)._h, int(dtype)))
+
+    def reshape(self, input, shape):
+        return self._wrap(_lib.dvm_rt_reshape(self._rt, input._h, self._shape_ref(shape)._h))
+
+    def copy(self, input):
+        return self._wrap(_lib.dvm_rt_copy(self._rt, input._h))
+
+    def _reduce(self, kind, input, dims, keepdims):
+        if isinstance(dims, int):
+            dims = (dims,)
+        return self._wrap(_lib.dvm_rt_reduce(self._rt, kind, input._h, self._shape_ref(dims)._h, int(bool(keepdims))))
+
+    def sum(self, input, dims, keepdims=False):
+        return self._reduce(0, input, dims, keepdims)
+
+    def max(self, input, dims, keepdims=False):
+        return self._reduce(1, input, dims, keepdims)
+
+    def min(self, input, dims, keepdims=False):
+        return self._reduce(2, input, dims, keepdims)
+
+    def matmul(self, lhs, rhs, trans_a, trans_b, bias=None):
+        return self._wrap(_lib.dvm_rt_matmul(self._rt, lhs._h, rhs._h, int(bool(trans_a)), int(bool(trans_b)),
+                                             bias._h if bias is not None else None))
+
+    # -- introspection --
+    def das(self):
+        return _ptr(_lib.dvm_rt_das(self._rt)).decode()
+
+    def dump(self):
+        return _ptr(_lib.dvm_rt_dump(self._rt)).decode()
+
+    def dump_r(self):
+        return _ptr(_lib.dvm_rt_dump_r(self._rt)).decode()
+
+    def inspect(self):
+        return _ptr(_lib.dvm_rt_inspect(self._rt)).decode()
+
+
+def _make_unary(idx):
+    def fn(self, input):
+        return self._wrap(_lib.dvm_rt_unary(self._rt, idx, input._h))
+    return fn
+
+
+def _make_binary(idx):
+    def fn(self, lhs, rhs):
+        a, b = self._operand(lhs), self._operand(rhs)
+        return self._wrap(_lib.dvm_rt_binary(self._rt, idx, ctypes.byref(a), ctypes.byref(b)))
+    return fn
+
+
+for _i, _n in enumerate(_UNARY):
+    setattr(Kernel, _n, _make_unary(_i))
+for _i, _n in enumerate(_BINARY):
+    setattr(Kernel, _n, _make_binary(_i))
+
+
+class PyKernel(Kernel):
+    """Builder plus runner: owns device buffers for the bound numpy inputs and the outputs."""
+
+    def __init__(self, ker_type, run_type, dev_id):
+        Kernel.__init__(self)
+        self._rt = _ptr(_lib.dvm_rt_new(ker_type.encode(), run_type.encode(), int(dev_id)))
+        self._run_type = run_type
+        self._dyn = "dyn" in ker_type
+        self._load_shape = {}   # load handle -> IntArrayRef
+        self._inputs = {}
+
+    def __del__(self):
+        rt, self._rt = getattr(self, "_rt", None), None
+        if rt:
+            _lib.dvm_rt_delete(rt)
+
+    def load(self, shape, type):
+        ref = self._shape_ref(shape)
+        op = Kernel.load(self, ref, type)
+        self._load_shape[op._h] = ref
+        return op
+
+    def reset(self):
+        _check(_lib.dvm_rt_reset(self._rt))
+        self._keep = []
+        self._load_shape = {}
+        self._inputs = {}
+
+    @staticmethod
+    def convert_to_bf16(array):
+        src = np.ascontiguousarray(array, dtype=np.float32)
+        dst = np.empty(src.shape, dtype=np.uint16)
+        _lib.dvm_c_f32_to_bf16(src.ctypes.data, dst.ctypes.data, src.size)
+        return dst
+
+    @staticmethod
+    def convert_from_bf16(array):
+        src = np.ascontiguousarray(array, dtype=np.uint16)
+        dst = np.empty(src.shape, dtype=np.float32)
+        _lib.dvm_c_bf16_to_f32(src.ctypes.data, dst.ctypes.data, src.size)
+        return dst
+
+    def input(self, load, array):
+        """Binds a numpy array (copied to the device), a scalar value, or a shape to a placeholder."""
+        if isinstance(load, ScalarRef):
+            load.update(array)
+            return
+        if isinstance(load, IntArrayRef):
+            load.update(list(array))
+            return
+        arr = np.ascontiguousarray(array)
+        ref = self._load_shape.get(load._h)
+        if ref is not None and tuple(ref.shape()) != tuple(arr.shape):
+            ref.update(list(arr.shape))
+        want = _ITEMSIZE[int(load.dtype())]
+        if arr.dtype.itemsize != want:
+            raise TypeError("array dtype %s does not match the load's element size %d" % (arr.dtype, want))
+        self._inputs[load._h] = arr
+        _check(_lib.dvm_rt_input(self._rt, load._h, arr.ctypes.data, arr.nbytes))
+
+    def bind_device(self, io, device_ptr, shape=None):
+        """Binds caller-owned device memory (e.g. a torch tensor's data_ptr()) to a load or store."""
+        if shape is not None and io._h in self._load_shape:
+            self._load_shape[io._h].update(list(shape))
+        _check(_lib.dvm_rt_bind_device(self._rt, io._h, ctypes.c_void_p(device_ptr)))
+
+    def codegen(self, pass_names=None):
+        _check(_lib.dvm_rt_codegen(self._rt))
+
+    def jit_us(self):
+        return _lib.dvm_rt_jit_us(self._rt)
+
+    def run(self, stream=None, sync=True):
+        _check(_lib.dvm_rt_run(self._rt, ctypes.c_void_p(stream) if stream else None, int(sync)))
+
+    def output(self, store):
+        shape = store.shape()
+        dt = int(store.dtype())
+        out = np.empty(shape, dtype=_NP_OF[dt])
+        _check(_lib.dvm_rt_output(self._rt, store._h, out.ctypes.data, out.nbytes))
+        return out
+
+    def device_ptr(self, io):
+        return _lib.dvm_rt_device_ptr(self._rt, io._h)
+
+    def perf(self, warmup=3, iters=10):
+        out = (ctypes.c_double * 3)()
+        _check(_lib.dvm_rt_perf(self._rt, warmup, iters, out))
+        return (out[0], out[1], out[2])
+
+    def num_launches(self):
+        return _lib.dvm_rt_num_launches(self._rt)
+
+    def workspace_bytes(self):
+        return _lib.dvm_rt_workspace_bytes(self._rt)
+
+    @staticmethod
+    def barrier():
+        pass
+
+    @staticmethod
+    def set_deterministic(enable):
+        pass
+
+
+class Device:
+    @staticmethod
+    def arch():
+        return "gfx950"
+
+    @staticmethod
+    def core_num():
+        return _lib.dvm_c_core_num()
+
+    @staticmethod
+    def soc_name():
+        return "MI355X"
+
+    @staticmethod
+    def available():
+        return bool(_lib.dvm_c_has_device())

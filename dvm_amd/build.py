@@ -1,0 +1,81 @@
+"""Builds the native libraries of the package in-tree.
+
+  dvm_amd/lib/libdvm_hip.so  device layer: HIP interpreter kernels + C ABI (include/dvm_hip.h), hipcc, gfx950
+  dvm_amd/lib/libdvm.so      host library: dvm::Kernel API (include/dvm.h) + flat C ABI (include/dvm_c.h), g++
+
+Run as `python -m dvm_amd.build` (add --force to rebuild everything).
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(ROOT, "csrc")
+LIB = os.path.join(ROOT, "lib")
+OBJ = os.path.join(LIB, "obj")
+
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+HOST_FLAGS = ["-std=c++17", "-O2", "-fPIC", "-fvisibility=hidden", "-Wall"]
+
+
+def _sources(sub, ext):
+    d = os.path.join(CSRC, sub)
+    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(ext))
+
+
+def _deps():
+    out = [os.path.join(CSRC, "isa_gfx950.h")]
+    inc = os.path.join(os.path.dirname(ROOT), "include")
+    out += [os.path.join(inc, f) for f in os.listdir(inc)]
+    out += _sources("host", ".h")
+    return out
+
+
+def _stale(target, sources):
+    if not os.path.exists(target):
+        return True
+    t = os.path.getmtime(target)
+    return any(os.path.getmtime(s) > t for s in sources)
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l and l.strip())
+    if r.returncode != 0:
+        raise RuntimeError("build step failed: %s\n%s" % (" ".join(cmd), err))
+    return err
+
+
+def build(force=False, verbose=False):
+    os.makedirs(OBJ, exist_ok=True)
+    deps = _deps()
+    jobs = []
+    dev_objs, host_objs = [], []
+    for src in _sources("device", ".hip"):
+        obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+        dev_objs.append(obj)
+        if force or _stale(obj, [src] + deps):
+            jobs.append(["hipcc"] + HIP_FLAGS + ["-c", src, "-o", obj])
+    for src in _sources("host", ".cc"):
+        obj = os.path.join(OBJ, os.path.basename(src) + ".o")
+        host_objs.append(obj)
+        if force or _stale(obj, [src] + deps):
+            jobs.append(["g++"] + HOST_FLAGS + ["-c", src, "-o", obj])
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
+        for msg in ex.map(_run, jobs):
+            if verbose and msg:
+                print(msg)
+    hip_so = os.path.join(LIB, "libdvm_hip.so")
+    host_so = os.path.join(LIB, "libdvm.so")
+    if force or _stale(hip_so, dev_objs):
+        _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC"] + dev_objs + ["-o", hip_so])
+    if force or _stale(host_so, host_objs):
+        _run(["g++", "-shared", "-fPIC"] + host_objs + ["-o", host_so, "-ldl", "-lpthread"])
+    return hip_so, host_so
+
+
+if __name__ == "__main__":
+    so = build(force="--force" in sys.argv, verbose=True)
+    print("built", so)

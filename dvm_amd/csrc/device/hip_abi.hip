@@ -1,0 +1,190 @@
+// C ABI of the device layer: VM init / launch geometry / launch, and the thin
+// runtime wrappers the host emitter needs (see include/dvm_hip.h for the
+// reference interfaces each entry point replaces).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include "../../../include/dvm_hip.h"
+#include "../isa_gfx950.h"
+
+extern "C" __global__ void dvm_vm_vec_pw(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_rx(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_ry(const VmParam p);
+
+namespace {
+
+struct DeviceInfo {
+  bool ready = false;
+  int dev = -1;
+  uint32_t cus = 256;
+  uint32_t lds_per_cu = 160 * 1024;
+  uint32_t lds_per_wg = 64 * 1024;
+};
+DeviceInfo g_dev;
+
+__global__ void dvm_fill_u32_kernel(uint32_t *dst, uint32_t value, size_t n) {
+  size_t i = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t stride = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (; i < n; i += stride) dst[i] = value;
+}
+
+// waves per SIMD each interpreter kernel fits at (from its VGPR count)
+uint32_t kernel_waves_per_simd(uint64_t kind) {
+  switch (kind) {
+    case VS_POINTWISE: return 6;
+    case VS_REDX: return 5;
+    case VS_REDY: return 4;
+    default: return 2;
+  }
+}
+
+}  // namespace
+
+extern "C" {
+
+int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
+  int count = 0;
+  hipError_t err = hipGetDeviceCount(&count);
+  if (err != hipSuccess) return static_cast<int>(err);
+  if (dev_id < 0 || dev_id >= count) return static_cast<int>(hipErrorInvalidDevice);
+  err = hipSetDevice(dev_id);
+  if (err != hipSuccess) return static_cast<int>(err);
+  hipDeviceProp_t prop;
+  err = hipGetDeviceProperties(&prop, dev_id);
+  if (err != hipSuccess) return static_cast<int>(err);
+  g_dev.dev = dev_id;
+  g_dev.cus = static_cast<uint32_t>(prop.multiProcessorCount);
+  g_dev.lds_per_cu = static_cast<uint32_t>(prop.maxSharedMemoryPerMultiProcessor);
+  if (g_dev.lds_per_cu == 0) g_dev.lds_per_cu = 64 * 1024;
+  g_dev.lds_per_wg = static_cast<uint32_t>(prop.sharedMemPerBlock);
+  // gfx950 lets one workgroup use the CU's whole 160 KB; the kernels must opt in.
+  const void *kernels[] = {reinterpret_cast<const void *>(dvm_vm_vec_pw), reinterpret_cast<const void *>(dvm_vm_vec_rx),
+                           reinterpret_cast<const void *>(dvm_vm_vec_ry)};
+  for (const void *k : kernels) {
+    if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(g_dev.lds_per_cu)) ==
+        hipSuccess) {
+      g_dev.lds_per_wg = g_dev.lds_per_cu;
+    } else {
+      (void)hipGetLastError();
+    }
+  }
+  g_dev.ready = true;
+  if (conf != nullptr) {
+    conf->core_num = g_dev.cus;
+    conf->local_mem_size = g_dev.lds_per_wg;
+    conf->default_threads = 256;
+    conf->wave_size = static_cast<uint64_t>(prop.warpSize);
+    conf->l2_bytes = static_cast<uint64_t>(prop.l2CacheSize);
+    conf->xcd_num = 8;
+  }
+  return 0;
+}
+
+uint64_t dvm_hip_select_block_thread(uint64_t kind, uint64_t item_num, uint64_t threads, uint32_t lds_bytes) {
+  if (threads == 0) threads = 256;
+  const uint64_t waves_per_wg = (threads + 63) / 64;
+  uint64_t wg_per_cu = (4ull * kernel_waves_per_simd(kind)) / waves_per_wg;
+  if (lds_bytes > 0) {
+    const uint64_t by_lds = g_dev.lds_per_cu / lds_bytes;
+    if (by_lds < wg_per_cu) wg_per_cu = by_lds;
+  }
+  if (wg_per_cu == 0) wg_per_cu = 1;
+  uint64_t blocks = static_cast<uint64_t>(g_dev.cus) * wg_per_cu;
+  if (blocks > item_num) blocks = item_num;
+  if (blocks == 0) blocks = 1;
+  return (blocks << 32) | threads;
+}
+
+int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, uint32_t lds_bytes, void *stream) {
+  if (param == nullptr || block_dim == 0 || threads == 0 || threads > 1024 || (threads & 63u) != 0) {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  if (lds_bytes > g_dev.lds_per_wg) return static_cast<int>(hipErrorInvalidValue);
+  VmParam p;
+  memcpy(&p, param, sizeof(p));
+  const VVecHeader *h = reinterpret_cast<const VVecHeader *>(p.w);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (h->entry == VE_VECTOR) {
+    // Reject blobs whose tables would be read outside the 4 KB argument.
+    const uint64_t mem_end = static_cast<uint64_t>(h->mem_off) + static_cast<uint64_t>(h->n_mem) * (sizeof(VMemDesc) / 8);
+    const uint64_t code_end = static_cast<uint64_t>(h->code_off) + h->n_code;
+    if (mem_end > DVM_PARAM_WORDS || code_end > DVM_PARAM_WORDS || h->n_code == 0 ||
+        VI_OP(p.w[code_end - 1]) != VOP_END || h->n_kdim > DVM_VEC_MAXR || h->n_rdim > DVM_VEC_MAXR) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+    switch (h->sched) {
+      case VS_POINTWISE:
+        hipLaunchKernelGGL(dvm_vm_vec_pw, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        break;
+      case VS_REDX:
+        hipLaunchKernelGGL(dvm_vm_vec_rx, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        break;
+      case VS_REDY:
+        hipLaunchKernelGGL(dvm_vm_vec_ry, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        break;
+      default:
+        return static_cast<int>(hipErrorInvalidValue);
+    }
+  } else {
+    return static_cast<int>(hipErrorInvalidValue);
+  }
+  return static_cast<int>(hipGetLastError());
+}
+
+int dvm_hip_fill_u32(void *dst, uint32_t value, size_t bytes, void *stream) {
+  if (bytes == 0) return 0;
+  if (dst == nullptr || (bytes & 3u) != 0) return static_cast<int>(hipErrorInvalidValue);
+  const size_t n = bytes / 4;
+  size_t blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(dvm_fill_u32_kernel, dim3(static_cast<uint32_t>(blocks)), dim3(256), 0,
+                     reinterpret_cast<hipStream_t>(stream), static_cast<uint32_t *>(dst), value, n);
+  return static_cast<int>(hipGetLastError());
+}
+
+int dvm_hip_get_device_count(uint32_t *count) {
+  int n = 0;
+  hipError_t err = hipGetDeviceCount(&n);
+  if (err != hipSuccess) {
+    (void)hipGetLastError();
+    n = 0;
+  }
+  if (count != nullptr) *count = static_cast<uint32_t>(n);
+  return static_cast<int>(err);
+}
+int dvm_hip_set_device(int device_id) { return static_cast<int>(hipSetDevice(device_id)); }
+int dvm_hip_get_device(int *device_id) { return static_cast<int>(hipGetDevice(device_id)); }
+int dvm_hip_create_stream(void **stream) { return static_cast<int>(hipStreamCreate(reinterpret_cast<hipStream_t *>(stream))); }
+int dvm_hip_destroy_stream(void *stream) { return static_cast<int>(hipStreamDestroy(reinterpret_cast<hipStream_t>(stream))); }
+int dvm_hip_synchronize_stream(void *stream) {
+  hipError_t err = hipStreamSynchronize(reinterpret_cast<hipStream_t>(stream));
+  if (err != hipSuccess) (void)hipGetLastError();  // do not leave the error for the next call
+  return static_cast<int>(err);
+}
+int dvm_hip_malloc(void **ptr, size_t size) { return static_cast<int>(hipMalloc(ptr, size)); }
+int dvm_hip_free(void *ptr) { return static_cast<int>(hipFree(ptr)); }
+int dvm_hip_malloc_host(void **ptr, size_t size) { return static_cast<int>(hipHostMalloc(ptr, size, hipHostMallocDefault)); }
+int dvm_hip_free_host(void *ptr) { return static_cast<int>(hipHostFree(ptr)); }
+int dvm_hip_mem_to_dev(void *dst, const void *src, size_t count) {
+  return static_cast<int>(hipMemcpy(dst, src, count, hipMemcpyHostToDevice));
+}
+int dvm_hip_mem_from_dev(void *dst, const void *src, size_t count) {
+  return static_cast<int>(hipMemcpy(dst, src, count, hipMemcpyDeviceToHost));
+}
+int dvm_hip_mem_to_dev_async(void *dst, const void *src, size_t count, void *stream) {
+  return static_cast<int>(hipMemcpyAsync(dst, src, count, hipMemcpyHostToDevice, reinterpret_cast<hipStream_t>(stream)));
+}
+int dvm_hip_memset(void *dst, int value, size_t size) { return static_cast<int>(hipMemset(dst, value, size)); }
+int dvm_hip_create_event(void **event) { return static_cast<int>(hipEventCreate(reinterpret_cast<hipEvent_t *>(event))); }
+int dvm_hip_destroy_event(void *event) { return static_cast<int>(hipEventDestroy(reinterpret_cast<hipEvent_t>(event))); }
+int dvm_hip_record_event(void *event, void *stream) {
+  return static_cast<int>(hipEventRecord(reinterpret_cast<hipEvent_t>(event), reinterpret_cast<hipStream_t>(stream)));
+}
+int dvm_hip_synchronize_event(void *event) { return static_cast<int>(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event))); }
+int dvm_hip_event_elapsed_time(float *ms, void *start, void *end) {
+  return static_cast<int>(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(end)));
+}
+const char *dvm_hip_error_string(int code) { return hipGetErrorString(static_cast<hipError_t>(code)); }
+
+}  // extern "C"

@@ -1,0 +1,790 @@
+// gfx950 vector VM: persistent interpreter kernels for fused
+// load / elementwise / cast / broadcast / reduce / store programs.
+//
+// Replaces the reference's generic interpreter (src/vm_gpu.cu:1552-1617 and the
+// RunOp switch at :941-1548) with a register-resident design for CDNA4:
+//  * a lane owns U slabs of E=8 consecutive elements of the innermost axis per
+//    instruction; slab u of all lanes is contiguous, so every global access is
+//    a coalesced 128-bit access and U of them are in flight per lane;
+//  * values stay in an accumulator (U*E VGPRs); local memory holds only the
+//    few values that must outlive an instruction chain and the reduce partials
+//    that cross waves;
+//  * broadcast operands are never materialised: they are stride-0 operands;
+//  * a reduce and its consumers run in one launch as consecutive sweeps over
+//    the reduce index space of the workgroup's outputs;
+//  * decoding is wave-uniform (scalar unit): the cost of one dispatch is spread
+//    over U*E*64 elements.
+// Numerics follow the reference device functors (src/vm_gpu.cu:198-329): fp16
+// and bf16 arithmetic is one fp32 operation rounded once, sums accumulate in
+// fp64 (src/vm_gpu.cu:779-866), float->int is C truncation, round is
+// half-to-even.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../isa_gfx950.h"
+
+namespace {
+
+constexpr int E = DVM_VEC_E;
+constexpr int U = DVM_VEC_U;
+
+typedef float vf8 __attribute__((ext_vector_type(8)));
+typedef float vf4 __attribute__((ext_vector_type(4)));
+typedef uint32_t vu4 __attribute__((ext_vector_type(4)));
+typedef uint32_t vu2 __attribute__((ext_vector_type(2)));
+typedef _Float16 vh8 __attribute__((ext_vector_type(8)));
+
+#define DVM_GLOBAL __attribute__((address_space(1)))
+#define FOR_U _Pragma("unroll") for (int u = 0; u < U; ++u)
+#define FOR_E _Pragma("unroll") for (int e = 0; e < E; ++e)
+
+struct Acc {
+  vf8 v[U];
+};
+
+// packed per-slab valid counts: 4 bits per slab
+constexpr uint32_t kAllOnes = U == 4 ? 0x1111u : (U == 2 ? 0x11u : 0x1u);
+constexpr uint32_t kAllFull = kAllOnes * 8u;
+
+__device__ __forceinline__ uint32_t uni(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, const VDim &d) { return (__umulhi(n, d.magic) + n) >> d.shift; }
+
+__device__ __forceinline__ float round_f16(float x) { return static_cast<float>(static_cast<_Float16>(x)); }
+
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float x) {
+  uint32_t u = __float_as_uint(x);
+  uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
+  r = (x != x) ? 0x7fc00000u : r;              // NaN stays NaN
+  return r >> 16;
+}
+__device__ __forceinline__ float round_bf16(float x) { return __uint_as_float(f32_to_bf16_bits(x) << 16); }
+
+__device__ __forceinline__ void apply_rnd(Acc &a, uint32_t rnd) {
+  if (rnd == VRND_NONE) return;
+  if (rnd == VRND_F16) {
+    FOR_U FOR_E a.v[u][e] = round_f16(a.v[u][e]);
+  } else {
+    FOR_U FOR_E a.v[u][e] = round_bf16(a.v[u][e]);
+  }
+}
+
+// ---- memory operands -------------------------------------------------------
+
+__device__ __forceinline__ float elem_load(uint64_t base, uint32_t dtype, uint64_t off) {
+  switch (dtype) {
+    case VDT_F32:
+      return reinterpret_cast<const DVM_GLOBAL float *>(base)[off];
+    case VDT_I32:
+      return __int_as_float(reinterpret_cast<const DVM_GLOBAL int32_t *>(base)[off]);
+    case VDT_F16:
+      return static_cast<float>(reinterpret_cast<const DVM_GLOBAL _Float16 *>(base)[off]);
+    case VDT_BF16:
+      return __uint_as_float(static_cast<uint32_t>(reinterpret_cast<const DVM_GLOBAL uint16_t *>(base)[off]) << 16);
+    default:  // VDT_BOOL
+      return reinterpret_cast<const DVM_GLOBAL uint8_t *>(base)[off] != 0 ? 1.0f : 0.0f;
+  }
+}
+
+__device__ __forceinline__ void elem_store(uint64_t base, uint32_t dtype, uint64_t off, float v) {
+  switch (dtype) {
+    case VDT_F32:
+      reinterpret_cast<DVM_GLOBAL float *>(base)[off] = v;
+      break;
+    case VDT_I32:
+      reinterpret_cast<DVM_GLOBAL int32_t *>(base)[off] = __float_as_int(v);
+      break;
+    case VDT_F16:
+      reinterpret_cast<DVM_GLOBAL _Float16 *>(base)[off] = static_cast<_Float16>(v);
+      break;
+    case VDT_BF16:
+      reinterpret_cast<DVM_GLOBAL uint16_t *>(base)[off] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+      break;
+    default:
+      reinterpret_cast<DVM_GLOBAL uint8_t *>(base)[off] = v != 0.0f ? 1 : 0;
+      break;
+  }
+}
+
+// Slow path of a slab: scalar per-element accesses (ragged tail, unaligned rows, stride-0 operand).
+__device__ __forceinline__ vf8 slab_load_slow(const VMemDesc &m, uint64_t off, int nv) {
+  vf8 out = 0.0f;
+  if (!(m.flags & VMF_VEC)) {
+    out = elem_load(m.addr, m.dtype, off);
+    return out;
+  }
+  FOR_E {
+    if (e < nv) out[e] = elem_load(m.addr, m.dtype, off + e);
+  }
+  return out;
+}
+
+__device__ __forceinline__ void slab_store_slow(const VMemDesc &m, uint64_t off, int nv, vf8 in) {
+  if (!(m.flags & VMF_VEC)) {
+    elem_store(m.addr, m.dtype, off, in[0]);
+    return;
+  }
+  FOR_E {
+    if (e < nv) elem_store(m.addr, m.dtype, off + e, in[e]);
+  }
+}
+
+// Loads the U slabs of operand `m`. nvp holds 4 bits per slab: elements inside the tensor (0 = skip).
+__device__ __forceinline__ void mem_load(const VMemDesc &m, const uint64_t (&off)[U], uint32_t nvp, Acc &out) {
+  const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
+  const uint32_t dtype = m.dtype;
+  if (fast && nvp == kAllFull) {  // whole instruction on the wide path: issue every load before any use
+    if (dtype == VDT_F32 || dtype == VDT_I32) {
+      vf4 a[U], b[U];
+      FOR_U {
+        const DVM_GLOBAL vf4 *p = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off[u] * 4);
+        a[u] = p[0];
+        b[u] = p[1];
+      }
+      FOR_U out.v[u] = __builtin_shufflevector(a[u], b[u], 0, 1, 2, 3, 4, 5, 6, 7);
+    } else if (dtype == VDT_BF16) {
+      vu4 a[U];
+      FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(m.addr + off[u] * 2);
+      FOR_U {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          out.v[u][2 * i] = __uint_as_float(a[u][i] << 16);
+          out.v[u][2 * i + 1] = __uint_as_float(a[u][i] & 0xffff0000u);
+        }
+      }
+    } else if (dtype == VDT_F16) {
+      vh8 a[U];
+      FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off[u] * 2);
+      FOR_U out.v[u] = __builtin_convertvector(a[u], vf8);
+    } else {
+      vu2 a[U];
+      FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vu2 *>(m.addr + off[u]);
+      FOR_U {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          out.v[u][e] = ((a[u][0] >> (8 * e)) & 0xffu) ? 1.0f : 0.0f;
+          out.v[u][e + 4] = ((a[u][1] >> (8 * e)) & 0xffu) ? 1.0f : 0.0f;
+        }
+      }
+    }
+    return;
+  }
+  FOR_U {
+    const int nv = static_cast<int>((nvp >> (4 * u)) & 0xfu);
+    out.v[u] = 0.0f;
+    if (nv == 0) continue;
+    if (fast && nv == E) {
+      if (dtype == VDT_F32 || dtype == VDT_I32) {
+        const DVM_GLOBAL vf4 *p = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off[u] * 4);
+        out.v[u] = __builtin_shufflevector(p[0], p[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        continue;
+      }
+      if (dtype == VDT_F16) {
+        out.v[u] = __builtin_convertvector(*reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off[u] * 2), vf8);
+        continue;
+      }
+    }
+    out.v[u] = slab_load_slow(m, off[u], nv);
+  }
+}
+
+__device__ __forceinline__ void mem_store(const VMemDesc &m, const uint64_t (&off)[U], uint32_t nvp, const Acc &in) {
+  const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
+  const uint32_t dtype = m.dtype;
+  FOR_U {
+    const int nv = static_cast<int>((nvp >> (4 * u)) & 0xfu);
+    if (nv == 0) continue;
+    if (fast && nv == E) {
+      if (dtype == VDT_F32 || dtype == VDT_I32) {
+        DVM_GLOBAL vf4 *p = reinterpret_cast<DVM_GLOBAL vf4 *>(m.addr + off[u] * 4);
+        p[0] = __builtin_shufflevector(in.v[u], in.v[u], 0, 1, 2, 3);
+        p[1] = __builtin_shufflevector(in.v[u], in.v[u], 4, 5, 6, 7);
+      } else if (dtype == VDT_BF16) {
+        vu4 a;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          a[i] = f32_to_bf16_bits(in.v[u][2 * i]) | (f32_to_bf16_bits(in.v[u][2 * i + 1]) << 16);
+        *reinterpret_cast<DVM_GLOBAL vu4 *>(m.addr + off[u] * 2) = a;
+      } else if (dtype == VDT_F16) {
+        *reinterpret_cast<DVM_GLOBAL vh8 *>(m.addr + off[u] * 2) = __builtin_convertvector(in.v[u], vh8);
+      } else {
+        vu2 a = 0u;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[0] |= (in.v[u][e] != 0.0f ? 1u : 0u) << (8 * e);
+          a[1] |= (in.v[u][e + 4] != 0.0f ? 1u : 0u) << (8 * e);
+        }
+        *reinterpret_cast<DVM_GLOBAL vu2 *>(m.addr + off[u]) = a;
+      }
+    } else {
+      slab_store_slow(m, off[u], nv, in.v[u]);
+    }
+  }
+}
+
+// ---- reduce helpers ----------------------------------------------------------
+
+__device__ __forceinline__ double red_combine(uint32_t kind, double r, double v) {
+  if (kind == VR_SUM) return r + v;
+  if (kind == VR_MAX) return (v > r || v != v) ? v : r;  // NaN propagates, as NumPy's max/min
+  return (v < r || v != v) ? v : r;
+}
+
+__device__ __forceinline__ double red_identity(uint32_t kind) {
+  if (kind == VR_SUM) return 0.0;
+  if (kind == VR_MAX) return -__builtin_huge_val();
+  return __builtin_huge_val();
+}
+
+__device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
+  int lo = __double2loint(v), hi = __double2hiint(v);
+  lo = __shfl_xor(lo, mask, 64);
+  hi = __shfl_xor(hi, mask, 64);
+  return __hiloint2double(hi, lo);
+}
+
+// REDX keeps one fp64 partial per slot (the elements of an instruction are
+// combined pairwise first); REDY keeps one per element of the lane's group.
+template <int SCHED>
+struct RedAcc {
+  double v[SCHED == VS_REDY ? E : 1];
+};
+
+template <int SCHED>
+__device__ __forceinline__ void red_init(RedAcc<SCHED> &r, uint32_t kind) {
+  const double idv = red_identity(kind);
+#pragma unroll
+  for (int e = 0; e < (SCHED == VS_REDY ? E : 1); ++e) r.v[e] = idv;
+}
+
+// fp32 combine of the elements of one slab (NaN-propagating for max/min).
+__device__ __forceinline__ float red_combine_f32(uint32_t kind, float r, float v) {
+  if (kind == VR_SUM) return r + v;
+  if (kind == VR_MAX) return (v > r || v != v) ? v : r;
+  return (v < r || v != v) ? v : r;
+}
+
+template <int SCHED>
+__device__ __forceinline__ void red_accumulate(RedAcc<SCHED> &r, uint32_t kind, const Acc &x, uint32_t nvp) {
+  FOR_U {
+    const int nv = static_cast<int>((nvp >> (4 * u)) & 0xfu);
+    if constexpr (SCHED == VS_REDY) {
+      FOR_E {
+        if (e < nv) r.v[e] = red_combine(kind, r.v[e], static_cast<double>(x.v[u][e]));
+      }
+    } else {
+      // The 8 elements of a slab are combined pairwise in fp32 (the blocking NumPy's
+      // float32 sum uses as well), every further step accumulates in fp64.
+      const float idv = static_cast<float>(red_identity(kind));
+      float d[E];
+      FOR_E d[e] = e < nv ? x.v[u][e] : idv;
+#pragma unroll
+      for (int w = 1; w < E; w <<= 1)
+#pragma unroll
+        for (int e = 0; e + w < E; e += 2 * w) d[e] = red_combine_f32(kind, d[e], d[e + w]);
+      if (nv > 0) r.v[0] = red_combine(kind, r.v[0], static_cast<double>(d[0]));
+    }
+  }
+}
+
+// Combines one slot's partials across the lanes that share an output; every
+// one of those lanes ends up with the result.
+template <int SCHED>
+__device__ __forceinline__ void red_finalize(RedAcc<SCHED> &r, uint32_t rk, uint32_t tlog, bool team_is_block,
+                                             uint32_t tid, uint32_t nthreads, uint32_t k_local, uint32_t r_local,
+                                             double *scratch) {
+  if constexpr (SCHED == VS_REDX) {
+    double t = r.v[0];
+    const uint32_t span = team_is_block ? 64u : (1u << tlog);
+    for (uint32_t msk = 1; msk < span; msk <<= 1) t = red_combine(rk, t, shfl_xor_f64(t, msk));
+    if (team_is_block) {
+      const uint32_t nw = (nthreads + 63u) >> 6;
+      __syncthreads();
+      if ((tid & 63u) == 0) scratch[tid >> 6] = t;
+      __syncthreads();
+      t = scratch[0];
+      for (uint32_t j = 1; j < nw; ++j) t = red_combine(rk, t, scratch[j]);
+    }
+    r.v[0] = t;
+  } else if constexpr (SCHED == VS_REDY) {
+    const uint32_t tx = 1u << tlog, ty = nthreads >> tlog;
+    if (ty > 1) {
+      FOR_E {
+        __syncthreads();
+        scratch[r_local * tx + k_local] = r.v[e];
+        __syncthreads();
+        double t = scratch[k_local];
+        for (uint32_t j = 1; j < ty; ++j) t = red_combine(rk, t, scratch[j * tx + k_local]);
+        r.v[e] = t;
+      }
+    }
+  }
+}
+
+// ---- S registers (one float per lane, VGPRs) -----------------------------------
+
+struct SRegs {
+  float s0, s1, s2, s3, s4, s5, s6, s7;
+};
+
+__device__ __forceinline__ float sreg_read(const SRegs &sr, uint32_t idx) {
+  switch (idx) {
+    case 0: return sr.s0;
+    case 1: return sr.s1;
+    case 2: return sr.s2;
+    case 3: return sr.s3;
+    case 4: return sr.s4;
+    case 5: return sr.s5;
+    case 6: return sr.s6;
+    default: return sr.s7;
+  }
+}
+
+__device__ __forceinline__ void sreg_write(SRegs &sr, uint32_t idx, float v) {
+  switch (idx) {
+    case 0: sr.s0 = v; break;
+    case 1: sr.s1 = v; break;
+    case 2: sr.s2 = v; break;
+    case 3: sr.s3 = v; break;
+    case 4: sr.s4 = v; break;
+    case 5: sr.s5 = v; break;
+    case 6: sr.s6 = v; break;
+    default: sr.s7 = v; break;
+  }
+}
+
+// ---- V registers (U*E values per lane, local memory) -----------------------------
+// A slot is U planes of 16 bytes per lane; slab u of slot s lives at
+// plane[(s*U + u) * nthreads + tid]. A lane only touches its own column, so no
+// barrier is needed. fp32 values take two slots, fp16/bf16-representable
+// values are packed into one.
+__device__ __forceinline__ void vreg_store(vf4 *planes, uint32_t slot, uint32_t fmt, uint32_t nthreads, uint32_t tid,
+                                           const Acc &a) {
+  if (fmt == VF_F32) {
+    FOR_U {
+      planes[(slot * U + u) * nthreads + tid] = __builtin_shufflevector(a.v[u], a.v[u], 0, 1, 2, 3);
+      planes[((slot + 1) * U + u) * nthreads + tid] = __builtin_shufflevector(a.v[u], a.v[u], 4, 5, 6, 7);
+    }
+  } else if (fmt == VF_F16) {
+    FOR_U {
+      vh8 hv = __builtin_convertvector(a.v[u], vh8);
+      planes[(slot * U + u) * nthreads + tid] = *reinterpret_cast<vf4 *>(&hv);
+    }
+  } else {
+    FOR_U {
+      vu4 b;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        b[i] = (__float_as_uint(a.v[u][2 * i]) >> 16) | (__float_as_uint(a.v[u][2 * i + 1]) & 0xffff0000u);
+      planes[(slot * U + u) * nthreads + tid] = *reinterpret_cast<vf4 *>(&b);
+    }
+  }
+}
+
+__device__ __forceinline__ void vreg_load(const vf4 *planes, uint32_t slot, uint32_t fmt, uint32_t nthreads, uint32_t tid,
+                                          Acc &a) {
+  if (fmt == VF_F32) {
+    FOR_U {
+      const vf4 lo = planes[(slot * U + u) * nthreads + tid];
+      const vf4 hi = planes[((slot + 1) * U + u) * nthreads + tid];
+      a.v[u] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  } else if (fmt == VF_F16) {
+    FOR_U {
+      vf4 raw = planes[(slot * U + u) * nthreads + tid];
+      a.v[u] = __builtin_convertvector(*reinterpret_cast<vh8 *>(&raw), vf8);
+    }
+  } else {
+    FOR_U {
+      vf4 raw = planes[(slot * U + u) * nthreads + tid];
+      vu4 b = *reinterpret_cast<vu4 *>(&raw);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        a.v[u][2 * i] = __uint_as_float(b[i] << 16);
+        a.v[u][2 * i + 1] = __uint_as_float(b[i] & 0xffff0000u);
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ VMemDesc load_desc(const uint32_t *prog32, uint32_t mem_off_words, uint32_t idx) {
+  const uint32_t *d = prog32 + 2 * mem_off_words + idx * (sizeof(VMemDesc) / 4);
+  VMemDesc m;
+  m.addr = static_cast<uint64_t>(uni(d[0])) | (static_cast<uint64_t>(uni(d[1])) << 32);
+  m.dtype = uni(d[2]);
+  m.flags = uni(d[3]);
+#pragma unroll
+  for (int i = 0; i < DVM_VEC_MAXR; ++i) {
+    m.kstride[i] = uni(d[4 + i]);
+    m.rstride[i] = uni(d[4 + DVM_VEC_MAXR + i]);
+  }
+  return m;
+}
+
+// Splits a flat index of an index space into its coordinates and returns the
+// element offset sum(coord * stride). The innermost-axis coordinate counts
+// E-groups when `inner` is set and is converted to elements.
+__device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim (&dims)[DVM_VEC_MAXR], uint32_t ndim,
+                                                 const uint32_t (&stride)[DVM_VEC_MAXR], bool inner) {
+  uint64_t off = 0;
+#pragma unroll
+  for (int i = 0; i < DVM_VEC_MAXR; ++i) {
+    if (i < static_cast<int>(ndim)) {
+      uint32_t c = n;
+      if (i + 1 < static_cast<int>(ndim)) {
+        const uint32_t q = fast_div(n, dims[i]);
+        c = n - q * dims[i].extent;
+        n = q;
+      }
+      if (i == 0 && inner) c *= E;
+      off += static_cast<uint64_t>(c) * stride[i];
+    }
+  }
+  return off;
+}
+
+// Valid element count (0..E) of the E-group with flat index n in a space whose first axis counts groups.
+__device__ __forceinline__ uint32_t group_valid(uint32_t n, const VDim (&dims)[DVM_VEC_MAXR], uint32_t ndim,
+                                                uint32_t inner_extent) {
+  uint32_t c = n;
+  if (ndim > 1) c = n - fast_div(n, dims[0]) * dims[0].extent;
+  const uint32_t left = inner_extent - c * E;
+  return left < static_cast<uint32_t>(E) ? left : static_cast<uint32_t>(E);
+}
+
+template <int SCHED>
+__device__ __forceinline__ void vm_vector(const VmParam &p) {
+  extern __shared__ double lds[];
+  __shared__ uint32_t prog32[DVM_PARAM_BYTES / 4];
+  // The blob arrives as a kernel argument; decoding from there would cost a
+  // dependent scalar-memory round trip per access, so each workgroup copies it
+  // into local memory once and decodes from there.
+  {
+    const uint32_t *src = reinterpret_cast<const uint32_t *>(p.w);
+    for (uint32_t i = threadIdx.x; i < DVM_PARAM_BYTES / 4; i += blockDim.x) prog32[i] = src[i];
+    __syncthreads();
+  }
+  VVecHeader h;
+  {
+    uint32_t *hw = reinterpret_cast<uint32_t *>(&h);
+#pragma unroll
+    for (int i = 0; i < static_cast<int>(sizeof(VVecHeader) / 4); ++i) hw[i] = uni(prog32[i]);
+  }
+  const uint32_t mem_off = h.mem_off;
+  const uint32_t *code32 = prog32 + 2 * h.code_off;
+
+  const uint32_t tid = threadIdx.x;
+  const uint32_t nthreads = blockDim.x;
+  const uint32_t tlog = h.team_log2;
+  const bool team_is_block = h.team_is_block != 0;
+  vf4 *planes = reinterpret_cast<vf4 *>(lds + nthreads);  // first nthreads doubles: reduce scratch
+
+  // lane -> (kept local index, reduce local index)
+  uint32_t k_local, r_local, k_per_wg, r_step;
+  if constexpr (SCHED == VS_POINTWISE) {
+    k_local = tid; r_local = 0; k_per_wg = nthreads * U; r_step = 1;
+  } else if constexpr (SCHED == VS_REDX) {
+    if (team_is_block) {
+      k_local = 0; r_local = tid; k_per_wg = 1; r_step = nthreads;
+    } else {
+      k_local = tid >> tlog; r_local = tid & ((1u << tlog) - 1u); k_per_wg = nthreads >> tlog; r_step = 1u << tlog;
+    }
+  } else {
+    k_local = tid & ((1u << tlog) - 1u); r_local = tid >> tlog; k_per_wg = 1u << tlog; r_step = nthreads >> tlog;
+  }
+  const uint32_t n_rounds = SCHED == VS_POINTWISE ? 1u : (h.n_ridx + r_step * U - 1) / (r_step * U);
+  constexpr bool inner_red = SCHED == VS_REDX;
+
+  SRegs sr;
+  sr.s0 = sr.s1 = sr.s2 = sr.s3 = sr.s4 = sr.s5 = sr.s6 = sr.s7 = 0.0f;
+  Acc acc;
+  FOR_U acc.v[u] = 0.0f;
+  uint32_t mask = 0;
+  RedAcc<SCHED> racc0, racc1;
+  red_init<SCHED>(racc0, VR_SUM);
+  red_init<SCHED>(racc1, VR_SUM);
+
+  for (uint32_t item = blockIdx.x; item < h.n_items; item += gridDim.x) {
+    // position of the lane in the kept space (POINTWISE: of slab 0; slab u is nthreads further each)
+    const uint32_t kidx = item * k_per_wg + k_local;
+    const bool kvalid = kidx < h.n_kidx;
+    uint32_t nvp_out;  // valid counts outside sweeps
+    if constexpr (SCHED == VS_POINTWISE) {
+      nvp_out = 0;
+      FOR_U {
+        const uint32_t ku = kidx + u * nthreads;
+        const uint32_t nv = ku < h.n_kidx ? group_valid(ku, h.kdims, h.n_kdim, h.inner_extent) : 0u;
+        nvp_out |= nv << (4 * u);
+      }
+    } else {
+      const uint32_t nv = !kvalid ? 0u : (inner_red ? 1u : group_valid(kidx, h.kdims, h.n_kdim, h.inner_extent));
+      nvp_out = nv * kAllOnes;
+    }
+
+    bool in_sweep = false;
+    uint32_t nvp = nvp_out;
+    uint32_t round = 0, sweep_pc = 0, slot_kinds = 0;
+    uint32_t ridx = r_local;  // reduce-space index of slab 0 in the current round
+
+    uint32_t pc = 0;
+    while (true) {
+      const uint32_t w0 = uni(code32[2 * pc]);
+      const uint32_t imm = uni(code32[2 * pc + 1]);
+      ++pc;
+      const uint32_t op = w0 & 0xffu;
+      if (op == VOP_END) break;
+      const uint32_t sub = (w0 >> 8) & 0xffu, a = w0 >> 24;
+
+      if (op >= VOP_SRC_BASE) {
+        // ---- fetch the source operand ----
+        Acc src;
+        const uint32_t kind = (w0 >> 16) & 0xfu;
+        if (kind == VK_MEM) {
+          const VMemDesc m = load_desc(prog32, mem_off, a);
+          uint64_t off[U];
+          if constexpr (SCHED == VS_POINTWISE) {
+            FOR_U {
+              const uint32_t ku = kidx + u * nthreads;
+              off[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
+            }
+          } else {
+            const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
+            FOR_U {
+              off[u] = koff;
+              if (in_sweep) {
+                const uint32_t ru = ridx + u * r_step;
+                off[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+              }
+            }
+          }
+          mem_load(m, off, nvp, src);
+        } else if (kind == VK_SREG) {
+          const float v = sreg_read(sr, a);
+          FOR_U src.v[u] = v;
+        } else if (kind == VK_IMM) {
+          const float v = __uint_as_float(imm);
+          FOR_U src.v[u] = v;
+        } else if (kind == VK_REG) {
+          vreg_load(planes, a, sub >> 6, nthreads, tid, src);
+        } else {
+          src = acc;
+        }
+
+        switch (op) {
+          case VOP_LD:
+            acc = src;
+            break;
+          case VOP_BINF: {
+            switch (sub & 0x3fu) {
+              case VB_ADD: FOR_U acc.v[u] = acc.v[u] + src.v[u]; break;
+              case VB_SUB: FOR_U acc.v[u] = acc.v[u] - src.v[u]; break;
+              case VB_RSUB: FOR_U acc.v[u] = src.v[u] - acc.v[u]; break;
+              case VB_MUL: FOR_U acc.v[u] = acc.v[u] * src.v[u]; break;
+              case VB_DIV: FOR_U acc.v[u] = acc.v[u] / src.v[u]; break;
+              case VB_RDIV: FOR_U acc.v[u] = src.v[u] / acc.v[u]; break;
+              // on NaN the second operand wins, as in the reference functors (src/vm_gpu.cu:222-233)
+              case VB_MIN: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] < src.v[u][e] ? acc.v[u][e] : src.v[u][e]; break;
+              case VB_MAX: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] > src.v[u][e] ? acc.v[u][e] : src.v[u][e]; break;
+              case VB_AND: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f && src.v[u][e] != 0.0f) ? 1.0f : 0.0f; break;
+              case VB_OR: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f || src.v[u][e] != 0.0f) ? 1.0f : 0.0f; break;
+              case VB_POW: FOR_U FOR_E acc.v[u][e] = powf(acc.v[u][e], src.v[u][e]); break;
+              default: FOR_U FOR_E acc.v[u][e] = powf(src.v[u][e], acc.v[u][e]); break;
+            }
+            apply_rnd(acc, (w0 >> 20) & 0x3u);
+            break;
+          }
+          case VOP_BINI: {
+            switch (sub & 0x3fu) {
+              case VBI_ADD: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(acc.v[u][e]) + __float_as_uint(src.v[u][e])); break;
+              case VBI_SUB: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(acc.v[u][e]) - __float_as_uint(src.v[u][e])); break;
+              case VBI_RSUB: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(src.v[u][e]) - __float_as_uint(acc.v[u][e])); break;
+              case VBI_MUL: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(acc.v[u][e]) * __float_as_uint(src.v[u][e])); break;
+              case VBI_MIN: FOR_U FOR_E acc.v[u][e] = __int_as_float(min(__float_as_int(acc.v[u][e]), __float_as_int(src.v[u][e]))); break;
+              default: FOR_U FOR_E acc.v[u][e] = __int_as_float(max(__float_as_int(acc.v[u][e]), __float_as_int(src.v[u][e]))); break;
+            }
+            break;
+          }
+          case VOP_CMP: {
+            switch (sub & 0x3fu) {
+              case VCMP_EQ: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] == src.v[u][e] ? 1.0f : 0.0f; break;
+              case VCMP_NE: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] != src.v[u][e] ? 1.0f : 0.0f; break;
+              case VCMP_GT: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] > src.v[u][e] ? 1.0f : 0.0f; break;
+              case VCMP_GE: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] >= src.v[u][e] ? 1.0f : 0.0f; break;
+              case VCMP_LT: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] < src.v[u][e] ? 1.0f : 0.0f; break;
+              case VCMP_LE: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] <= src.v[u][e] ? 1.0f : 0.0f; break;
+              case VCMP_INT + VCMP_EQ: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) == __float_as_int(src.v[u][e]) ? 1 : 0); break;
+              case VCMP_INT + VCMP_NE: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) != __float_as_int(src.v[u][e]) ? 1 : 0); break;
+              case VCMP_INT + VCMP_GT: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) > __float_as_int(src.v[u][e]) ? 1 : 0); break;
+              case VCMP_INT + VCMP_GE: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) >= __float_as_int(src.v[u][e]) ? 1 : 0); break;
+              case VCMP_INT + VCMP_LT: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) < __float_as_int(src.v[u][e]) ? 1 : 0); break;
+              default: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) <= __float_as_int(src.v[u][e]) ? 1 : 0); break;
+            }
+            break;
+          }
+          case VOP_MSK: {
+            // 1/0 in either container: a zero has no bits set below the sign
+            mask = 0;
+            FOR_U FOR_E mask |= ((__float_as_uint(src.v[u][e]) << 1) != 0 ? 1u : 0u) << (u * E + e);
+            break;
+          }
+          default: {  // VOP_MOVM
+            FOR_U FOR_E acc.v[u][e] = ((mask >> (u * E + e)) & 1u) ? src.v[u][e] : acc.v[u][e];
+            break;
+          }
+        }
+        continue;
+      }
+
+      switch (op) {
+        case VOP_LDR:
+          vreg_load(planes, a, sub, nthreads, tid, acc);
+          break;
+        case VOP_LDS: {
+          const float v = sreg_read(sr, a);
+          FOR_U acc.v[u] = v;
+          break;
+        }
+        case VOP_LDI: {
+          const float v = __uint_as_float(imm);
+          FOR_U acc.v[u] = v;
+          break;
+        }
+        case VOP_STR:
+          vreg_store(planes, a, sub, nthreads, tid, acc);
+          break;
+        case VOP_STS:
+          sreg_write(sr, a, acc.v[0][0]);
+          break;
+        case VOP_ST: {
+          const VMemDesc m = load_desc(prog32, mem_off, a);
+          uint64_t off[U];
+          uint32_t nvs = nvp;
+          if constexpr (SCHED == VS_POINTWISE) {
+            FOR_U {
+              const uint32_t ku = kidx + u * nthreads;
+              off[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
+            }
+          } else {
+            const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
+            FOR_U {
+              off[u] = koff;
+              if (in_sweep) {
+                const uint32_t ru = ridx + u * r_step;
+                off[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+              }
+            }
+            if (!in_sweep) nvs = r_local == 0 ? (nvp & 0xfu) : 0u;  // one lane per output, one slab
+          }
+          mem_store(m, off, nvs, acc);
+          break;
+        }
+        case VOP_UN: {
+          switch (sub) {
+            case VU_SQRT: FOR_U FOR_E acc.v[u][e] = sqrtf(acc.v[u][e]); break;
+            case VU_ABS: FOR_U FOR_E acc.v[u][e] = fabsf(acc.v[u][e]); break;
+            case VU_LOG: FOR_U FOR_E acc.v[u][e] = logf(acc.v[u][e]); break;
+            case VU_EXP: FOR_U FOR_E acc.v[u][e] = expf(acc.v[u][e]); break;
+            case VU_ISFINITE: FOR_U FOR_E acc.v[u][e] = isfinite(acc.v[u][e]) ? 1.0f : 0.0f; break;
+            case VU_ROUND: FOR_U FOR_E acc.v[u][e] = rintf(acc.v[u][e]); break;
+            case VU_FLOOR: FOR_U FOR_E acc.v[u][e] = floorf(acc.v[u][e]); break;
+            case VU_CEIL: FOR_U FOR_E acc.v[u][e] = ceilf(acc.v[u][e]); break;
+            case VU_TRUNC: FOR_U FOR_E acc.v[u][e] = truncf(acc.v[u][e]); break;
+            default:  // VU_IABS, wraps for INT32_MIN like the reference (src/vm_gpu.cu:262-266)
+              FOR_U FOR_E {
+                const uint32_t x = __float_as_uint(acc.v[u][e]);
+                acc.v[u][e] = __uint_as_float(static_cast<int32_t>(x) < 0 ? 0u - x : x);
+              }
+              break;
+          }
+          apply_rnd(acc, (w0 >> 20) & 0x3u);
+          break;
+        }
+        case VOP_CAST: {
+          if (sub == VC_F2I) {
+            FOR_U FOR_E acc.v[u][e] = __int_as_float(static_cast<int32_t>(acc.v[u][e]));
+          } else if (sub == VC_I2F) {
+            FOR_U FOR_E acc.v[u][e] = static_cast<float>(__float_as_int(acc.v[u][e]));
+            apply_rnd(acc, (w0 >> 20) & 0x3u);
+          } else if (sub == VC_RND) {
+            apply_rnd(acc, (w0 >> 20) & 0x3u);
+          } else {
+            FOR_U FOR_E acc.v[u][e] = acc.v[u][e] != 0.0f ? 1.0f : 0.0f;
+          }
+          break;
+        }
+        default:
+          break;
+      }
+
+      if constexpr (SCHED != VS_POINTWISE) {
+        switch (op) {
+          case VOP_RED: {
+            if (a == 0) {
+              red_accumulate<SCHED>(racc0, sub, acc, nvp);
+            } else {
+              red_accumulate<SCHED>(racc1, sub, acc, nvp);
+            }
+            break;
+          }
+          case VOP_SWEEP: {
+            in_sweep = true;
+            round = 0;
+            sweep_pc = pc;
+            slot_kinds = imm;
+            red_init<SCHED>(racc0, slot_kinds & 0xfu);
+            red_init<SCHED>(racc1, (slot_kinds >> 4) & 0xfu);
+            ridx = r_local;
+            break;
+          }
+          case VOP_ENDSWEEP: {
+            ++round;
+            if (round < n_rounds) {
+              ridx += r_step * U;
+              pc = sweep_pc;
+            } else {
+              in_sweep = false;
+              const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
+              if (k0 <= VR_MIN) red_finalize<SCHED>(racc0, k0, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
+              if (k1 <= VR_MIN) red_finalize<SCHED>(racc1, k1, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
+            }
+            break;
+          }
+          case VOP_FIN: {
+            if constexpr (SCHED == VS_REDY) {
+              vf8 t;
+              FOR_E t[e] = static_cast<float>(a == 0 ? racc0.v[e] : racc1.v[e]);
+              FOR_U acc.v[u] = t;
+            } else {
+              const float t = static_cast<float>(a == 0 ? racc0.v[0] : racc1.v[0]);
+              FOR_U acc.v[u] = t;
+            }
+            break;
+          }
+          default:
+            break;
+        }
+
+        // valid counts of the round's slabs
+        if (op == VOP_SWEEP || op == VOP_ENDSWEEP) {
+          if (in_sweep) {
+            nvp = 0;
+            FOR_U {
+              const uint32_t ru = ridx + u * r_step;
+              uint32_t nv = 0;
+              if (kvalid && ru < h.n_ridx) nv = inner_red ? group_valid(ru, h.rdims, h.n_rdim, h.inner_extent) : (nvp_out & 0xfu);
+              nvp |= nv << (4 * u);
+            }
+          } else {
+            nvp = nvp_out;
+          }
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_pw(const VmParam p) { vm_vector<VS_POINTWISE>(p); }
+extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_rx(const VmParam p) { vm_vector<VS_REDX>(p); }
+extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_ry(const VmParam p) { vm_vector<VS_REDY>(p); }

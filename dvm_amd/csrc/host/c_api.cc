@@ -1,0 +1,584 @@
+// Flat C ABI + runner over dvm::Kernel (see include/dvm_c.h).
+#include "../../../include/dvm_c.h"
+
+#include <chrono>
+#include <cstring>
+#include <map>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "ir.h"
+#include "system.h"
+
+using namespace dvm;
+
+struct dvm_shape {
+  std::vector<int64_t> dims;
+  IntArrayRef ref;
+  void Set(const int64_t *d, size_t n) {
+    dims.assign(d, d + n);
+    if (dims.capacity() < static_cast<size_t>(kMaxRank)) dims.reserve(kMaxRank);
+    ref.data = dims.data();
+    ref.size = dims.size();
+  }
+};
+
+struct dvm_scalar {
+  ScalarRef ref;
+};
+
+namespace {
+
+thread_local std::string g_last_error;
+
+struct Buffer {
+  void *ptr = nullptr;
+  size_t bytes = 0;
+  bool owned = false;
+};
+
+struct WsAlloc : public WsAllocator {
+  dvm_rt *rt;
+  void *Alloc(size_t size) override;
+};
+
+}  // namespace
+
+struct dvm_rt {
+  Kernel kernel;
+  KernelType ktype = kSplit;
+  uint32_t flags = 0;
+  bool das_mode = false;
+  void *stream = nullptr;
+  std::vector<std::unique_ptr<dvm_shape>> shapes;
+  std::vector<std::unique_ptr<dvm_scalar>> scalars;
+  std::vector<NDObject *> loads, stores;
+  std::map<NDObject *, Buffer> buffers;
+  Buffer workspace;
+  uint64_t fake_addr = 0x1000;
+  double jit_us = 0.0;
+  WsAlloc ws_alloc;
+
+  const DeviceApi &Api() const { return g_system.Api(); }
+
+  void *AllocDevice(size_t bytes) {
+    if (das_mode) {
+      void *p = reinterpret_cast<void *>(fake_addr);
+      fake_addr += (bytes + 0xfff) & ~static_cast<uint64_t>(0xfff);
+      return p;
+    }
+    void *p = nullptr;
+    int rc = Api().malloc(&p, bytes == 0 ? 16 : bytes);
+    if (rc != 0) throw std::runtime_error(std::string("device allocation failed: ") + Api().error_string(rc));
+    return p;
+  }
+
+  void Release(Buffer &b) {
+    if (b.owned && b.ptr != nullptr && !das_mode) Api().free(b.ptr);
+    b = Buffer();
+  }
+
+  void Ensure(NDObject *o, size_t bytes) {
+    Buffer &b = buffers[o];
+    if (b.ptr != nullptr && (!b.owned || b.bytes >= bytes)) return;
+    Release(b);
+    b.ptr = AllocDevice(bytes);
+    b.bytes = bytes;
+    b.owned = true;
+  }
+
+  void FreeAll() {
+    for (auto &kv : buffers) Release(kv.second);
+    buffers.clear();
+    Release(workspace);
+  }
+};
+
+namespace {
+
+void *WsAlloc::Alloc(size_t size) {
+  Buffer &w = rt->workspace;
+  if (w.ptr == nullptr || w.bytes < size) {
+    rt->Release(w);
+    w.ptr = rt->AllocDevice(size);
+    w.bytes = size;
+    w.owned = true;
+  }
+  return w.ptr;
+}
+
+template <typename F>
+auto Guard(F f, decltype(f()) on_error) -> decltype(f()) {
+  try {
+    return f();
+  } catch (const std::exception &e) {
+    g_last_error = e.what();
+    return on_error;
+  }
+}
+
+NDObject *Obj(dvm_obj *o) { return reinterpret_cast<NDObject *>(o); }
+dvm_obj *Handle(NDObject *o) { return reinterpret_cast<dvm_obj *>(o); }
+
+void ParseKernelType(const std::string &s, KernelType *type, uint32_t *flags) {
+  std::string name = s, opts;
+  auto pos = s.find(':');
+  if (pos != std::string::npos) {
+    name = s.substr(0, pos);
+    opts = s.substr(pos + 1);
+  }
+  if (name.empty() || name == "vector") {
+    *type = kVector;
+  } else if (name == "split") {
+    *type = kSplit;
+  } else if (name == "mix") {
+    *type = kMix;
+  } else if (name == "cube") {
+    *type = kCube;
+  } else {
+    throw std::runtime_error("DVM EXCEPTION. reason: kernel type '" + name + "' is not supported by the gfx950 backend");
+  }
+  *flags = 0;
+  size_t start = 0;
+  while (start < opts.size()) {
+    size_t end = opts.find(',', start);
+    if (end == std::string::npos) end = opts.size();
+    const std::string f = opts.substr(start, end - start);
+    if (f == "dyn") {
+      *flags |= kDynamic;
+    } else if (f == "uws") {
+      *flags |= kUnifyWS;
+    } else if (!f.empty()) {
+      throw std::runtime_error("DVM EXCEPTION. reason: kernel flag '" + f + "' is not supported by the gfx950 backend");
+    }
+    start = end + 1;
+  }
+}
+
+template <BinaryType kOp>
+NDObject *BinaryDispatch(Kernel &k, const dvm_operand *l, const dvm_operand *r) {
+  auto with_rhs = [&](auto lhs) -> NDObject * {
+    switch (r->kind) {
+      case 0: return k.Binary<kOp>(lhs, Obj(r->obj));
+      default: throw std::runtime_error("DVM EXCEPTION. reason: binary operator needs a tensor operand");
+    }
+  };
+  if (l->kind == 0) {
+    NDObject *lhs = Obj(l->obj);
+    switch (r->kind) {
+      case 0: return k.Binary<kOp>(lhs, Obj(r->obj));
+      case 1: return k.Binary<kOp>(lhs, static_cast<float>(r->f));
+      case 2: return k.Binary<kOp>(lhs, static_cast<int32_t>(r->i));
+      case 3: return k.Binary<kOp>(lhs, &r->ref->ref);
+      default: break;
+    }
+  } else if (l->kind == 1) {
+    return with_rhs(static_cast<float>(l->f));
+  } else if (l->kind == 2) {
+    return with_rhs(static_cast<int32_t>(l->i));
+  } else if (l->kind == 3) {
+    return with_rhs(&l->ref->ref);
+  }
+  throw std::runtime_error("DVM EXCEPTION. reason: bad operand kind");
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *dvm_c_last_error(void) { return g_last_error.c_str(); }
+
+dvm_rt *dvm_rt_new(const char *ker_type, const char *run_mode, int dev_id) {
+  return Guard(
+      [&]() -> dvm_rt * {
+        std::unique_ptr<dvm_rt> rt(new dvm_rt());
+        ParseKernelType(ker_type != nullptr ? ker_type : "", &rt->ktype, &rt->flags);
+        const std::string mode = run_mode != nullptr ? run_mode : "dev";
+        rt->das_mode = mode == "das";
+        if (!rt->das_mode && mode != "dev") throw std::runtime_error("DVM EXCEPTION. reason: run mode '" + mode + "' is not supported");
+        rt->ws_alloc.rt = rt.get();
+        (void)dev_id;
+        rt->kernel.Reset(rt->ktype, rt->flags);
+        if (!rt->das_mode) {
+          if (!g_system.HasDevice()) {
+            throw std::runtime_error(std::string("DVM EXCEPTION. reason: no MI355X device layer: ") + g_system.LoadError());
+          }
+          int rc = rt->Api().create_stream(&rt->stream);
+          if (rc != 0) throw std::runtime_error(std::string("stream creation failed: ") + rt->Api().error_string(rc));
+        }
+        return rt.release();
+      },
+      nullptr);
+}
+
+void dvm_rt_delete(dvm_rt *rt) {
+  if (rt == nullptr) return;
+  rt->FreeAll();
+  if (rt->stream != nullptr) rt->Api().destroy_stream(rt->stream);
+  delete rt;
+}
+
+int dvm_rt_reset(dvm_rt *rt) {
+  return Guard(
+      [&]() {
+        rt->FreeAll();
+        rt->loads.clear();
+        rt->stores.clear();
+        rt->kernel.Reset(rt->ktype, rt->flags);
+        return 0;
+      },
+      -1);
+}
+
+dvm_shape *dvm_rt_new_shape(dvm_rt *rt, const int64_t *dims, size_t n) {
+  return Guard(
+      [&]() {
+        rt->shapes.emplace_back(new dvm_shape());
+        rt->shapes.back()->dims.reserve(kMaxRank);
+        rt->shapes.back()->Set(dims, n);
+        return rt->shapes.back().get();
+      },
+      static_cast<dvm_shape *>(nullptr));
+}
+
+int dvm_shape_update(dvm_shape *s, const int64_t *dims, size_t n) {
+  s->Set(dims, n);
+  return 0;
+}
+
+dvm_scalar *dvm_rt_new_scalar(dvm_rt *rt, int dtype) {
+  return Guard(
+      [&]() {
+        rt->scalars.emplace_back(new dvm_scalar());
+        dvm_scalar *s = rt->scalars.back().get();
+        if (dtype == kInt32) {
+          s->ref = 0;
+        } else {
+          s->ref = 0.0f;
+        }
+        return s;
+      },
+      static_cast<dvm_scalar *>(nullptr));
+}
+
+int dvm_scalar_update_f(dvm_scalar *s, double v) {
+  if (s->ref.type == kInt32) {
+    s->ref = static_cast<int32_t>(v);
+  } else {
+    s->ref = static_cast<float>(v);
+  }
+  return 0;
+}
+
+int dvm_scalar_update_i(dvm_scalar *s, int64_t v) {
+  if (s->ref.type == kInt32) {
+    s->ref = static_cast<int32_t>(v);
+  } else {
+    s->ref = static_cast<float>(v);
+  }
+  return 0;
+}
+
+dvm_obj *dvm_rt_load(dvm_rt *rt, dvm_shape *shape, int dtype) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.Load(nullptr, &shape->ref, static_cast<DataType>(dtype));
+        rt->loads.push_back(o);
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_store(dvm_rt *rt, dvm_obj *x) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.Store(nullptr, Obj(x));
+        rt->stores.push_back(o);
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_unary(dvm_rt *rt, int unary_type, dvm_obj *x) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.Unary(unary_type, Obj(x));
+        if (o == nullptr) throw std::runtime_error("DVM EXCEPTION. reason: bad unary operator");
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_binary(dvm_rt *rt, int binary_type, const dvm_operand *lhs, const dvm_operand *rhs) {
+  return Guard(
+      [&]() {
+        Kernel &k = rt->kernel;
+        NDObject *o = nullptr;
+        switch (binary_type) {
+          case kEqual: o = BinaryDispatch<kEqual>(k, lhs, rhs); break;
+          case kNotEqual: o = BinaryDispatch<kNotEqual>(k, lhs, rhs); break;
+          case kGreater: o = BinaryDispatch<kGreater>(k, lhs, rhs); break;
+          case kGreaterEqual: o = BinaryDispatch<kGreaterEqual>(k, lhs, rhs); break;
+          case kLess: o = BinaryDispatch<kLess>(k, lhs, rhs); break;
+          case kLessEqual: o = BinaryDispatch<kLessEqual>(k, lhs, rhs); break;
+          case kAdd: o = BinaryDispatch<kAdd>(k, lhs, rhs); break;
+          case kSub: o = BinaryDispatch<kSub>(k, lhs, rhs); break;
+          case kMul: o = BinaryDispatch<kMul>(k, lhs, rhs); break;
+          case kDiv: o = BinaryDispatch<kDiv>(k, lhs, rhs); break;
+          case kPow: o = BinaryDispatch<kPow>(k, lhs, rhs); break;
+          case kMaximum: o = BinaryDispatch<kMaximum>(k, lhs, rhs); break;
+          case kMinimum: o = BinaryDispatch<kMinimum>(k, lhs, rhs); break;
+          case kLogicalAnd: o = BinaryDispatch<kLogicalAnd>(k, lhs, rhs); break;
+          case kLogicalOr: o = BinaryDispatch<kLogicalOr>(k, lhs, rhs); break;
+          default: throw std::runtime_error("DVM EXCEPTION. reason: bad binary operator");
+        }
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_select(dvm_rt *rt, dvm_obj *cond, dvm_obj *lhs, dvm_obj *rhs) {
+  return Guard([&]() { return Handle(rt->kernel.Select(Obj(cond), Obj(lhs), Obj(rhs))); }, static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_cast(dvm_rt *rt, dvm_obj *x, int dtype) {
+  return Guard([&]() { return Handle(rt->kernel.Cast(Obj(x), static_cast<DataType>(dtype))); }, static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_broadcast(dvm_rt *rt, dvm_obj *x, dvm_shape *shape) {
+  return Guard([&]() { return Handle(rt->kernel.Broadcast(Obj(x), &shape->ref)); }, static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_full(dvm_rt *rt, const dvm_operand *value, dvm_shape *shape, int dtype) {
+  return Guard(
+      [&]() {
+        const DataType t = static_cast<DataType>(dtype);
+        switch (value->kind) {
+          case 1: return Handle(rt->kernel.Broadcast(static_cast<float>(value->f), &shape->ref, t));
+          case 2: return Handle(rt->kernel.Broadcast(static_cast<int32_t>(value->i), &shape->ref, t));
+          case 3: return Handle(rt->kernel.Broadcast(&value->ref->ref, &shape->ref, t));
+          default: throw std::runtime_error("DVM EXCEPTION. reason: full needs a scalar value");
+        }
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_reshape(dvm_rt *rt, dvm_obj *x, dvm_shape *shape) {
+  return Guard([&]() { return Handle(rt->kernel.Reshape(Obj(x), &shape->ref)); }, static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_reduce(dvm_rt *rt, int reduce_type, dvm_obj *x, dvm_shape *dims, int keepdims) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.Reduce(reduce_type, Obj(x), &dims->ref, keepdims != 0);
+        if (o == nullptr) throw std::runtime_error("DVM EXCEPTION. reason: sum needs an fp32 input (cast first)");
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_copy(dvm_rt *rt, dvm_obj *x) {
+  return Guard([&]() { return Handle(rt->kernel.Copy(Obj(x))); }, static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int trans_b, dvm_obj *bias) {
+  return Guard(
+      [&]() { return Handle(rt->kernel.MatMul(Obj(lhs), Obj(rhs), trans_a != 0, trans_b != 0, Obj(bias))); },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store) {
+  return Guard(
+      [&]() {
+        rt->kernel.SetStoreInplace(Obj(store));
+        return 0;
+      },
+      -1);
+}
+
+int dvm_obj_rank(const dvm_obj *o) { return reinterpret_cast<const NDObject *>(o)->rank(); }
+
+int dvm_obj_shape(const dvm_obj *o, int64_t *dims, size_t cap) {
+  const NDObject *n = reinterpret_cast<const NDObject *>(o);
+  const size_t r = n->shape_ref_->size;
+  for (size_t i = 0; i < r && i < cap; ++i) dims[i] = n->shape_ref_->data[i];
+  return static_cast<int>(r);
+}
+
+int dvm_obj_dtype(const dvm_obj *o) { return reinterpret_cast<const NDObject *>(o)->type_id_; }
+
+int dvm_rt_input(dvm_rt *rt, dvm_obj *load, const void *host, size_t bytes) {
+  return Guard(
+      [&]() {
+        NDObject *o = Obj(load);
+        rt->Ensure(o, bytes);
+        if (!rt->das_mode && bytes > 0) {
+          int rc = rt->Api().mem_to_dev(rt->buffers[o].ptr, host, bytes);
+          if (rc != 0) throw std::runtime_error(std::string("host to device copy failed: ") + rt->Api().error_string(rc));
+        }
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_bind_device(dvm_rt *rt, dvm_obj *io, void *device_ptr) {
+  return Guard(
+      [&]() {
+        Buffer &b = rt->buffers[Obj(io)];
+        rt->Release(b);
+        b.ptr = device_ptr;
+        b.owned = false;
+        b.bytes = 0;
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_codegen(dvm_rt *rt) {
+  return Guard(
+      [&]() {
+        const auto t0 = std::chrono::steady_clock::now();
+        rt->kernel.Normalize();
+        const auto t1 = std::chrono::steady_clock::now();
+        // outputs take their size from the inferred shapes
+        for (NDObject *s : rt->stores) {
+          const size_t bytes = static_cast<size_t>(s->numel()) * DTypeSize(s->type_id_);
+          rt->Ensure(s, bytes);
+        }
+        std::vector<RelocEntry> relocs;
+        relocs.reserve(rt->buffers.size());
+        for (auto &kv : rt->buffers) relocs.emplace_back(kv.first, kv.second.ptr);
+        for (NDObject *l : rt->loads) {
+          if (rt->buffers.find(l) == rt->buffers.end()) throw std::runtime_error("DVM EXCEPTION. reason: a load has no input bound");
+        }
+        const auto t2 = std::chrono::steady_clock::now();
+        rt->kernel.CodeGen(relocs.data(), relocs.size(), &rt->ws_alloc);
+        const auto t3 = std::chrono::steady_clock::now();
+        rt->jit_us = std::chrono::duration<double, std::micro>((t1 - t0) + (t3 - t2)).count();
+        return 0;
+      },
+      -1);
+}
+
+double dvm_rt_jit_us(const dvm_rt *rt) { return rt->jit_us; }
+
+int dvm_rt_run(dvm_rt *rt, void *stream, int sync) {
+  return Guard(
+      [&]() {
+        if (rt->das_mode) return 0;
+        void *s = stream != nullptr ? stream : rt->stream;
+        int rc = rt->kernel.Launch(s);
+        if (rc != 0) throw std::runtime_error(std::string("launch failed: ") + rt->Api().error_string(rc));
+        if (sync != 0) {
+          rc = rt->Api().synchronize_stream(s);
+          if (rc != 0) throw std::runtime_error(std::string("kernel execution failed: ") + rt->Api().error_string(rc));
+        }
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_output(dvm_rt *rt, dvm_obj *store, void *host, size_t bytes) {
+  return Guard(
+      [&]() {
+        if (rt->das_mode) {
+          std::memset(host, 0, bytes);
+          return 0;
+        }
+        auto it = rt->buffers.find(Obj(store));
+        if (it == rt->buffers.end()) throw std::runtime_error("DVM EXCEPTION. reason: store has no buffer");
+        if (bytes > 0) {
+          int rc = rt->Api().mem_from_dev(host, it->second.ptr, bytes);
+          if (rc != 0) throw std::runtime_error(std::string("device to host copy failed: ") + rt->Api().error_string(rc));
+        }
+        return 0;
+      },
+      -1);
+}
+
+void *dvm_rt_device_ptr(dvm_rt *rt, dvm_obj *io) {
+  auto it = rt->buffers.find(Obj(io));
+  return it == rt->buffers.end() ? nullptr : it->second.ptr;
+}
+
+int dvm_rt_perf(dvm_rt *rt, int warmup, int iters, double out[3]) {
+  return Guard(
+      [&]() {
+        if (rt->das_mode) {
+          out[0] = out[1] = out[2] = 0.0;
+          return 0;
+        }
+        const DeviceApi &api = rt->Api();
+        for (int i = 0; i < warmup; ++i) {
+          int rc = rt->kernel.Launch(rt->stream);
+          if (rc != 0) throw std::runtime_error(std::string("launch failed: ") + api.error_string(rc));
+        }
+        api.synchronize_stream(rt->stream);
+        std::vector<void *> ev(2 * static_cast<size_t>(iters), nullptr);
+        for (auto &e : ev) api.create_event(&e);
+        for (int i = 0; i < iters; ++i) {
+          api.record_event(ev[2 * i], rt->stream);
+          int rc = rt->kernel.Launch(rt->stream);
+          api.record_event(ev[2 * i + 1], rt->stream);
+          if (rc != 0) throw std::runtime_error(std::string("launch failed: ") + api.error_string(rc));
+        }
+        int rc = api.synchronize_stream(rt->stream);
+        if (rc != 0) throw std::runtime_error(std::string("kernel execution failed: ") + api.error_string(rc));
+        double mn = 1e30, mx = 0.0, sum = 0.0;
+        for (int i = 0; i < iters; ++i) {
+          float ms = 0.0f;
+          api.event_elapsed_time(&ms, ev[2 * i], ev[2 * i + 1]);
+          const double us = ms * 1000.0;
+          mn = std::min(mn, us);
+          mx = std::max(mx, us);
+          sum += us;
+        }
+        for (auto &e : ev) api.destroy_event(e);
+        out[0] = mn;
+        out[1] = mx;
+        out[2] = iters > 0 ? sum / iters : 0.0;
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_num_launches(const dvm_rt *rt) {
+  int n = 0;
+  for (const Program &p : rt->kernel.GetImpl()->programs_) n += (p.skip ? 0 : 1) + static_cast<int>(p.fills.size());
+  return n;
+}
+
+size_t dvm_rt_workspace_bytes(const dvm_rt *rt) { return rt->kernel.GetImpl()->ws_bytes_; }
+
+const char *dvm_rt_das(dvm_rt *rt) {
+  return Guard([&]() { return rt->kernel.Das(); }, static_cast<const char *>(nullptr));
+}
+const char *dvm_rt_dump(dvm_rt *rt) {
+  return Guard([&]() { return rt->kernel.Dump(); }, static_cast<const char *>(nullptr));
+}
+const char *dvm_rt_dump_r(dvm_rt *rt) {
+  return Guard([&]() { return rt->kernel.DumpR(); }, static_cast<const char *>(nullptr));
+}
+const char *dvm_rt_inspect(dvm_rt *rt) {
+  return Guard([&]() { return rt->kernel.Inspect(); }, static_cast<const char *>(nullptr));
+}
+
+void dvm_c_f32_to_bf16(const float *src, uint16_t *dst, size_t n) {
+  for (size_t i = 0; i < n; ++i) dst[i] = F32ToBF16Bits(src[i]);
+}
+void dvm_c_bf16_to_f32(const uint16_t *src, float *dst, size_t n) {
+  for (size_t i = 0; i < n; ++i) dst[i] = BF16BitsToF32(src[i]);
+}
+
+int dvm_c_has_device(void) {
+  g_system.Init();
+  return g_system.HasDevice() ? 1 : 0;
+}
+int dvm_c_core_num(void) {
+  g_system.Init();
+  return static_cast<int>(g_system.core_num);
+}
+
+}  // extern "C"

@@ -1,0 +1,1629 @@
+// Graph -> sub-kernels -> gfx950 tile bytecode.
+//
+// Role in the reference: shape normalisation (src/ops.cc Normalize family),
+// the split kernel's graph cutter (src/xkernel.cc:1980-2119), domain / tiling
+// (src/kernel.cc:765-1194), liveness + buffer allocation (src/kernel.cc:196-317,
+// 1285-1332) and the Emit methods (src/ops.cc). The gfx950 target differs in
+// what a sub-kernel may contain: a reduce and its consumers stay in one launch
+// (consecutive sweeps of one workgroup-resident program), broadcasts are
+// stride-0 operands, and intermediate values live in lane registers, so the
+// "tiling" step is an index-space analysis instead of a local-memory planner:
+//   1. every tensor dim of every value is unified into domain axes;
+//   2. axes are ordered, merged where all memory operands allow it, and split
+//      into a kept list and a reduced list;
+//   3. a schedule (pointwise / reduce over the innermost axis / reduce with
+//      the innermost axis kept) and its launch geometry are chosen;
+//   4. the operator DAG is linearised into accumulator-machine code, section
+//      by section (code outside sweeps works on the kept space, a sweep walks
+//      the reduce space), values that cannot stay in a register across a
+//      sweep are recomputed from their loads.
+#include <algorithm>
+#include <chrono>
+#include <cmath>
+#include <cstring>
+#include <stdexcept>
+
+#include "ir.h"
+#include "system.h"
+
+namespace dvm {
+
+VKernel::~VKernel() {
+  for (NDObject *o : ops_) delete o;
+}
+
+NDObject *VKernel::Append(NDObject *op) {
+  op->id = static_cast<int>(ops_.size());
+  ops_.push_back(op);
+  normalized_ = false;
+  compiled_ = false;
+  return op;
+}
+
+// ---- shape inference -----------------------------------------------------------------
+
+namespace {
+
+void BroadcastShapes(const NDObject *a, const NDObject *b, int64_t *out, size_t *out_rank) {
+  const size_t ra = a->shape_ref_->size, rb = b->shape_ref_->size;
+  const size_t r = std::max(ra, rb);
+  for (size_t i = 0; i < r; ++i) {
+    const int64_t da = i + ra >= r ? a->shape_ref_->data[i + ra - r] : 1;
+    const int64_t db = i + rb >= r ? b->shape_ref_->data[i + rb - r] : 1;
+    if (da != db && da != 1 && db != 1) Throw("operands cannot be broadcast together");
+    out[i] = da == 1 ? db : da;
+  }
+  *out_rank = r;
+}
+
+}  // namespace
+
+void VKernel::Normalize() {
+  for (NDObject *o : ops_) {
+    switch (o->kind) {
+      case kObjLoad:
+        if (o->shape_ref_->size > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
+        break;
+      case kObjStore:
+      case kObjUnary:
+      case kObjBinaryS:
+      case kObjCompareS:
+      case kObjCast:
+      case kObjCopy:
+        o->SetShape(o->in[0]->shape_ref_->data, o->in[0]->shape_ref_->size);
+        break;
+      case kObjBinary:
+      case kObjCompare: {
+        size_t r;
+        BroadcastShapes(o->in[0], o->in[1], o->shape_, &r);
+        o->own_ref_.size = r;
+        break;
+      }
+      case kObjSelect: {
+        NDObject tmp(kObjCopy, o->type_id_);
+        size_t r;
+        BroadcastShapes(o->in[0], o->in[1], tmp.shape_, &r);
+        tmp.own_ref_.size = r;
+        BroadcastShapes(&tmp, o->in[2], o->shape_, &r);
+        o->own_ref_.size = r;
+        break;
+      }
+      case kObjBroadcast: {
+        const size_t r = o->aux_ref->size;
+        const size_t ri = o->in[0]->shape_ref_->size;
+        if (r > static_cast<size_t>(kMaxRank) || ri > r) Throw("bad broadcast target");
+        for (size_t i = 0; i < r; ++i) {
+          int64_t d = o->aux_ref->data[i];
+          if (d == -1) {
+            if (i + ri < r) Throw("bad broadcast target");
+            d = o->in[0]->shape_ref_->data[i + ri - r];
+          }
+          o->shape_[i] = d;
+        }
+        o->own_ref_.size = r;
+        break;
+      }
+      case kObjBroadcastS:
+        if (o->aux_ref->size > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
+        o->SetShape(o->aux_ref->data, o->aux_ref->size);
+        break;
+      case kObjReduce: {
+        const NDObject *x = o->in[0];
+        const size_t r = x->shape_ref_->size;
+        bool red[kMaxRank] = {false};
+        for (size_t i = 0; i < o->aux_ref->size; ++i) {
+          int64_t d = o->aux_ref->data[i];
+          if (d < 0) d += static_cast<int64_t>(r);
+          if (d < 0 || d >= static_cast<int64_t>(r)) Throw("reduce axis out of range");
+          red[d] = true;
+        }
+        size_t n = 0;
+        for (size_t i = 0; i < r; ++i) {
+          if (red[i]) {
+            if (o->keepdims) o->shape_[n++] = 1;
+          } else {
+            o->shape_[n++] = x->shape_ref_->data[i];
+          }
+        }
+        o->own_ref_.size = n;
+        break;
+      }
+      case kObjReshape: {
+        const size_t r = o->aux_ref->size;
+        if (r > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
+        int64_t known = 1;
+        int infer = -1;
+        for (size_t i = 0; i < r; ++i) {
+          o->shape_[i] = o->aux_ref->data[i];
+          if (o->shape_[i] == -1) {
+            infer = static_cast<int>(i);
+          } else {
+            known *= o->shape_[i];
+          }
+        }
+        o->own_ref_.size = r;
+        const int64_t total = o->in[0]->numel();
+        if (infer >= 0) o->shape_[infer] = known == 0 ? 0 : total / known;
+        if (o->numel() != total) Throw("reshape changes the number of elements");
+        break;
+      }
+      case kObjMatMul: {
+        const NDObject *a = o->in[0], *b = o->in[1];
+        const size_t ra = a->shape_ref_->size, rb = b->shape_ref_->size;
+        if (ra < 2 || rb < 2) Throw("matmul operands need rank >= 2");
+        const int64_t m = o->trans_a ? a->dim(ra - 1) : a->dim(ra - 2);
+        const int64_t ka = o->trans_a ? a->dim(ra - 2) : a->dim(ra - 1);
+        const int64_t kb = o->trans_b ? b->dim(rb - 1) : b->dim(rb - 2);
+        const int64_t n = o->trans_b ? b->dim(rb - 2) : b->dim(rb - 1);
+        if (ka != kb) Throw("matmul inner dimensions differ");
+        const size_t ba = ra - 2, bb = rb - 2, br = std::max(ba, bb);
+        if (br + 2 > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
+        for (size_t i = 0; i < br; ++i) {
+          const int64_t da = i + ba >= br ? a->dim(i + ba - br) : 1;
+          const int64_t db = i + bb >= br ? b->dim(i + bb - br) : 1;
+          if (da != db && da != 1 && db != 1) Throw("matmul batch dimensions cannot be broadcast");
+          o->shape_[i] = da == 1 ? db : da;
+        }
+        o->shape_[br] = m;
+        o->shape_[br + 1] = n;
+        o->own_ref_.size = br + 2;
+        break;
+      }
+    }
+  }
+  normalized_ = true;
+}
+
+// ---- compiler ------------------------------------------------------------------------
+
+namespace {
+
+constexpr int kMaxNodes = 160;     // nodes of one sub-kernel
+constexpr int kMaxAxes = 24;       // domain axes before merging
+constexpr int E = DVM_VEC_E;
+constexpr int U = DVM_VEC_U;
+
+enum AKind : uint8_t { AK_MEM, AK_SCALAR, AK_OP, AK_ALIAS, AK_REDUCE, AK_OUT };
+
+struct ANode {
+  AKind kind;
+  NDObject *op;         // originating operator (for AK_MEM of a cross-kernel value: the producer or the reshape view)
+  DataType dtype;
+  int nin;
+  int in[3];
+  int rank;
+  const int64_t *dims;  // API shape, outermost first
+  int axis[kMaxRank];   // domain axis per dim, -1 for extent 1
+  // memory leaves / outputs
+  int addr_op;          // load/store operator supplying the address, or -1
+  int ws_slot;          // workspace slot, or -1
+  int mem_idx;          // descriptor index in the program
+  // emission state
+  bool has_inner;       // varies along the innermost domain axis
+  bool fd;              // has a reduced axis
+  int level;
+  int sec;              // section the value is computed in
+  int uses;             // remaining uses in the section being emitted
+  int reg;              // S register (has_inner false) or V slot, -1 when not in a register
+  uint8_t reg_fmt;
+  bool in_cone;
+  int last_sec;         // last section with a consumer
+};
+
+struct Axis {
+  int64_t extent;
+  bool reduced;
+  uint32_t before;  // axes that must be outside (more significant than) this one
+};
+
+struct Dim {  // merged domain dim
+  int64_t extent;
+  bool reduced;
+  int first_axis, last_axis;  // merged range in ordered-axis space (outer .. inner)
+};
+
+uint32_t FloatBits(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  return u;
+}
+
+VDim MakeVDim(uint32_t d) {
+  VDim v;
+  v.extent = d;
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;
+  v.shift = s;
+  v.magic = static_cast<uint32_t>((((1ull << 32) * ((1ull << s) - d)) / (d == 0 ? 1 : d)) + 1);
+  v.pad = 0;
+  return v;
+}
+
+uint32_t MemDType(DataType t) {
+  switch (t) {
+    case kBool: return VDT_BOOL;
+    case kFloat16: return VDT_F16;
+    case kBFloat16: return VDT_BF16;
+    case kFloat32: return VDT_F32;
+    case kInt32: return VDT_I32;
+    default: Throw("tensor type without a device form");
+  }
+}
+
+uint32_t RndOf(DataType t) { return t == kFloat16 ? VRND_F16 : (t == kBFloat16 ? VRND_BF16 : VRND_NONE); }
+
+bool IsPointwiseKind(ObjKind k) {
+  switch (k) {
+    case kObjUnary:
+    case kObjBinary:
+    case kObjBinaryS:
+    case kObjCompare:
+    case kObjCompareS:
+    case kObjSelect:
+    case kObjCast:
+    case kObjCopy:
+    case kObjBroadcast:
+    case kObjStore:
+      return true;
+    default:
+      return false;
+  }
+}
+
+// A reshape that only inserts or removes extent-1 dims keeps every element's coordinates.
+bool IsSqueezeReshape(const NDObject *o) {
+  const NDObject *x = o->in[0];
+  int i = 0, j = 0;
+  const int ri = x->rank(), ro = o->rank();
+  while (true) {
+    while (i < ri && x->dim(i) == 1) ++i;
+    while (j < ro && o->dim(j) == 1) ++j;
+    if (i == ri || j == ro) break;
+    if (x->dim(i) != o->dim(j)) return false;
+    ++i;
+    ++j;
+  }
+  return i == ri && j == ro;
+}
+
+}  // namespace
+
+class Compiler {
+ public:
+  explicit Compiler(VKernel *k) : k_(k), n_(static_cast<int>(k->ops_.size())) {}
+
+  size_t Run() {
+    try {
+      return RunOnce(false);
+    } catch (const std::runtime_error &) {
+      // maximal fusion did not fit the VM: cut after every reduce instead
+      return RunOnce(true);
+    }
+  }
+
+  size_t RunOnce(bool conservative) {
+    conservative_ = conservative;
+    area_.assign(n_, -1);
+    live_.assign(n_, 0);
+    mat_.assign(n_, 0);
+    ws_slot_.assign(n_, -1);
+    store_of_.assign(n_, -1);
+    MarkLive();
+    Partition();
+    k_->programs_.clear();
+    k_->ws_sizes_.clear();
+    k_->ws_offsets_.clear();
+    PlanMaterialisation();
+    for (int a = 0; a < n_areas_; ++a) CompileArea(a);
+    size_t total = 0;
+    for (size_t i = 0; i < k_->ws_sizes_.size(); ++i) {
+      k_->ws_offsets_.push_back(total);
+      total += (k_->ws_sizes_[i] + 255) & ~static_cast<size_t>(255);
+    }
+    k_->ws_bytes_ = total;
+    return total;
+  }
+
+ private:
+  VKernel *k_;
+  int n_;
+  std::vector<int> area_, ws_slot_, store_of_;
+  std::vector<char> live_, mat_;
+  int n_areas_ = 0;
+  struct AreaInfo {
+    bool cube = false;
+    bool has_reduce = false;
+    const NDObject *reduce = nullptr;
+    int rank = 0;
+    int64_t dom[kMaxRank];
+    const NDObject *cube_op = nullptr;
+  };
+  std::vector<AreaInfo> areas_;
+
+  // ---------- liveness ----------
+  void MarkLive() {
+    for (int i = n_ - 1; i >= 0; --i) {
+      NDObject *o = k_->ops_[i];
+      if (o->kind == kObjStore) live_[i] = 1;
+      if (!live_[i]) continue;
+      for (int j = 0; j < o->nin; ++j)
+        if (o->in[j] != nullptr) live_[o->in[j]->id] = 1;
+    }
+  }
+
+  // ---------- partition into sub-kernels ----------
+  static bool IsLeaf(const NDObject *o) { return o->kind == kObjLoad || o->kind == kObjBroadcastS; }
+
+  // A view: reshape of a materialised value (or of a load) that is read through its new shape.
+  bool IsView(const NDObject *o) const { return o->kind == kObjReshape && !IsSqueezeReshape(o); }
+
+  // The operator whose buffer a view chain ends at.
+  const NDObject *ViewRoot(const NDObject *o) const {
+    while (IsView(o)) o = o->in[0];
+    return o;
+  }
+
+  bool DomCompatible(const AreaInfo &ai, const int64_t *dims, int rank) const {
+    const int r = std::max(ai.rank, rank);
+    for (int i = 0; i < r; ++i) {
+      const int64_t da = i + ai.rank >= r ? ai.dom[i + ai.rank - r] : 1;
+      const int64_t db = i + rank >= r ? dims[i + rank - r] : 1;
+      if (da != db && da != 1 && db != 1) return false;
+    }
+    return true;
+  }
+
+  void DomMerge(AreaInfo &ai, const int64_t *dims, int rank) {
+    const int r = std::max(ai.rank, rank);
+    int64_t out[kMaxRank];
+    for (int i = 0; i < r; ++i) {
+      const int64_t da = i + ai.rank >= r ? ai.dom[i + ai.rank - r] : 1;
+      const int64_t db = i + rank >= r ? dims[i + rank - r] : 1;
+      out[i] = da == 1 ? db : da;
+    }
+    std::memcpy(ai.dom, out, sizeof(int64_t) * r);
+    ai.rank = r;
+  }
+
+  static bool SameReduce(const NDObject *a, const NDObject *b) {
+    const NDObject *xa = a->in[0], *xb = b->in[0];
+    if (xa->rank() != xb->rank()) return false;
+    for (int i = 0; i < xa->rank(); ++i)
+      if (xa->dim(i) != xb->dim(i)) return false;
+    bool ra[kMaxRank] = {false}, rb[kMaxRank] = {false};
+    for (size_t i = 0; i < a->aux_ref->size; ++i) {
+      int64_t d = a->aux_ref->data[i];
+      ra[d < 0 ? d + xa->rank() : d] = true;
+    }
+    for (size_t i = 0; i < b->aux_ref->size; ++i) {
+      int64_t d = b->aux_ref->data[i];
+      rb[d < 0 ? d + xb->rank() : d] = true;
+    }
+    for (int i = 0; i < xa->rank(); ++i)
+      if (xa->dim(i) != 1 && ra[i] != rb[i]) return false;
+    return true;
+  }
+
+  bool CanJoin(int a, const NDObject *o) {
+    if (a >= static_cast<int>(areas_.size())) return true;  // a fresh sub-kernel
+    const AreaInfo &ai = areas_[a];
+    if (o->kind == kObjMatMul) return false;
+    if (ai.cube) {
+      if (!IsPointwiseKind(o->kind)) return false;
+      // the epilogue works on the matmul's own output domain
+      const NDObject *c = ai.cube_op;
+      if (o->rank() != c->rank()) return false;
+      for (int i = 0; i < o->rank(); ++i)
+        if (o->dim(i) != c->dim(i)) return false;
+      return true;
+    }
+    if (o->kind == kObjReduce) {
+      if (ai.has_reduce && !SameReduce(ai.reduce, o)) return false;
+      return DomCompatible(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
+    }
+    return DomCompatible(ai, o->shape_ref_->data, o->rank());
+  }
+
+  void Join(int a, const NDObject *o) {
+    while (a >= static_cast<int>(areas_.size())) areas_.push_back(AreaInfo());
+    AreaInfo &ai = areas_[a];
+    if (o->kind == kObjMatMul) {
+      ai.cube = true;
+      ai.cube_op = o;
+      return;
+    }
+    if (ai.cube) return;
+    if (o->kind == kObjReduce) {
+      if (!ai.has_reduce) {
+        ai.has_reduce = true;
+        ai.reduce = o;
+      }
+      DomMerge(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
+    }
+    DomMerge(ai, o->shape_ref_->data, o->rank());
+  }
+
+  void Partition() {
+    areas_.clear();
+    const bool fuse = !conservative_;
+    for (int i = 0; i < n_; ++i) {
+      NDObject *o = k_->ops_[i];
+      if (!live_[i] || IsLeaf(o)) continue;
+      if (IsView(o)) continue;  // read through by its consumers
+      int a = 0;
+      for (int j = 0; j < o->nin; ++j) {
+        const NDObject *v = o->in[j];
+        if (v == nullptr || IsLeaf(v)) continue;
+        bool cut = false;
+        if (IsView(v)) {
+          v = ViewRoot(v);
+          if (IsLeaf(v)) continue;
+          cut = true;
+        }
+        if (o->kind == kObjMatMul) cut = true;
+        if (!fuse && v->kind == kObjReduce) cut = true;  // the reference's rule: a reduce ends its sub-kernel
+        a = std::max(a, area_[v->id] + (cut ? 1 : 0));
+      }
+      if (o->kind == kObjMatMul) a = std::max(a, static_cast<int>(areas_.size()));
+      while (!CanJoin(a, o)) ++a;
+      area_[i] = a;
+      Join(a, o);
+    }
+    n_areas_ = static_cast<int>(areas_.size());
+  }
+
+  // ---------- which values cross sub-kernels ----------
+  void PlanMaterialisation() {
+    for (int i = 0; i < n_; ++i) {
+      NDObject *o = k_->ops_[i];
+      if (!live_[i]) continue;
+      if (o->kind == kObjStore) store_of_[o->in[0]->id] = i;
+    }
+    for (int i = 0; i < n_; ++i) {
+      NDObject *o = k_->ops_[i];
+      if (!live_[i] || IsLeaf(o)) continue;
+      for (int j = 0; j < o->nin; ++j) {
+        const NDObject *v = o->in[j];
+        if (v == nullptr) continue;
+        const NDObject *root = ViewRoot(v);
+        if (IsLeaf(root) || root->kind == kObjLoad) continue;
+        const int user_area = IsView(o) ? -2 : area_[i];
+        if (IsView(v) || (user_area != -2 && area_[root->id] != user_area)) mat_[root->id] = 1;
+      }
+    }
+    for (int i = 0; i < n_; ++i) {
+      if (!mat_[i]) continue;
+      NDObject *o = k_->ops_[i];
+      if (store_of_[i] >= 0 && area_[store_of_[i]] == area_[i]) continue;  // later kernels read the user's output
+      ws_slot_[i] = static_cast<int>(k_->ws_sizes_.size());
+      k_->ws_sizes_.push_back(static_cast<size_t>(std::max<int64_t>(o->numel(), 1)) * DTypeSize(o->type_id_));
+    }
+  }
+
+  // ---------- one sub-kernel ----------
+  ANode nodes_[kMaxNodes];
+  int nn_ = 0;
+  std::vector<int> node_of_;  // op id -> node (per area)
+  Axis axes_[kMaxAxes];
+  int n_axes_ = 0;
+  int order_[kMaxAxes];       // ordered axes, outermost first
+  int pos_[kMaxAxes];         // axis -> position in order_
+  Dim dims_[kMaxAxes];
+  int n_dims_ = 0;
+  int dim_of_axis_[kMaxAxes]; // ordered position -> merged dim
+  // kept / reduced lists, innermost first (indices into dims_)
+  int klist_[DVM_VEC_MAXR], rlist_[DVM_VEC_MAXR];
+  int nk_ = 0, nr_ = 0;
+  // program under construction
+  Program *prog_ = nullptr;
+  VVecHeader hdr_;
+  VMemDesc mems_[DVM_VEC_MAXMEM];
+  int n_mem_ = 0;
+  std::vector<uint64_t> code_;
+  bool conservative_ = false;
+  bool single_round_ = false;
+  int acc_node_ = -1;
+  uint32_t sreg_used_ = 0;
+  uint32_t vslot_used_ = 0;
+  int max_vslot_ = 0;
+  int vslot_limit_ = 0;
+  int cur_sec_ = 0;
+
+  int AddNode(AKind kind, NDObject *op, DataType t, const int64_t *dims, int rank) {
+    if (nn_ >= kMaxNodes) Throw("sub-kernel too large");
+    ANode &n = nodes_[nn_];
+    std::memset(&n, 0, sizeof(n));
+    n.kind = kind;
+    n.op = op;
+    n.dtype = t;
+    n.dims = dims;
+    n.rank = rank;
+    n.addr_op = -1;
+    n.ws_slot = -1;
+    n.mem_idx = -1;
+    n.reg = -1;
+    for (int i = 0; i < kMaxRank; ++i) n.axis[i] = -1;
+    return nn_++;
+  }
+
+  // Leaf node for an operand coming from outside the sub-kernel.
+  int LeafFor(NDObject *v) {
+    if (node_of_[v->id] >= 0) return node_of_[v->id];
+    int idx;
+    if (v->kind == kObjBroadcastS) {
+      idx = AddNode(AK_SCALAR, v, v->type_id_, v->shape_ref_->data, v->rank());
+    } else {
+      idx = AddNode(AK_MEM, v, v->type_id_, v->shape_ref_->data, v->rank());
+      const NDObject *root = ViewRoot(v);
+      if (root->kind == kObjLoad) {
+        nodes_[idx].addr_op = root->id;
+      } else if (ws_slot_[root->id] >= 0) {
+        nodes_[idx].ws_slot = ws_slot_[root->id];
+      } else {
+        nodes_[idx].addr_op = store_of_[root->id];
+      }
+    }
+    node_of_[v->id] = idx;
+    return idx;
+  }
+
+  void Fail(const char *why) { Throw(std::string("cannot compile sub-kernel: ") + why); }
+
+  void CompileArea(int a);
+  void CompileCube(int a);
+  void BuildNodes(int a);
+  void UnifyAxes();
+  void OrderAndMerge();
+  void ChooseSchedule();
+  void EmitProgram();
+  void FinishProgram();
+
+  // union-find over (node, dim) variables
+  std::vector<int> uf_;
+  int Find(int x) {
+    while (uf_[x] != x) {
+      uf_[x] = uf_[uf_[x]];
+      x = uf_[x];
+    }
+    return x;
+  }
+  void Union(int a, int b) {
+    a = Find(a);
+    b = Find(b);
+    if (a != b) uf_[b] = a;
+  }
+  int Var(int node, int dim) const { return node * kMaxRank + dim; }
+  void UnifyAligned(int out, int in);
+
+  // emission helpers
+  void Emit(uint32_t op, uint32_t sub, uint32_t kind, uint32_t rnd, uint32_t a, uint32_t imm) {
+    code_.push_back(VI_MAKE(op, sub, kind, rnd, a, imm));
+  }
+  int Resolve(int v) const {
+    while (nodes_[v].kind == AK_ALIAS) v = nodes_[v].in[0];
+    return v;
+  }
+  int MemIndex(int v);
+  bool SimpleOperand(int v);
+  void EmitOperandInsn(uint32_t op, uint32_t sub, uint32_t rnd, int v);
+  void EmitValue(int v);
+  void ComputeInto(int v);
+  void BeforeOverwrite();
+  void SaveAcc(int v);
+  void ConsumeUse(int v);
+  void ReleaseReg(int v);
+  int AllocSReg();
+  int AllocVSlot(int n);
+  void CountCone(int v);
+  void EmitSection(int sec);
+  int n_sec_ = 1;
+};
+
+// ---------- node construction ----------
+
+void Compiler::BuildNodes(int a) {
+  nn_ = 0;
+  node_of_.assign(n_, -1);
+  for (int i = 0; i < n_; ++i) {
+    if (area_[i] != a) continue;
+    NDObject *o = k_->ops_[i];
+    int in_idx[3] = {-1, -1, -1};
+    for (int j = 0; j < o->nin; ++j) {
+      NDObject *v = o->in[j];
+      if (v == nullptr) continue;
+      if (node_of_[v->id] >= 0 && area_[v->id] == a) {
+        in_idx[j] = node_of_[v->id];
+      } else {
+        in_idx[j] = LeafFor(v);
+      }
+    }
+    AKind kind = AK_OP;
+    if (o->kind == kObjCopy || o->kind == kObjBroadcast || o->kind == kObjReshape) kind = AK_ALIAS;
+    if (o->kind == kObjReduce) kind = AK_REDUCE;
+    if (o->kind == kObjStore) kind = AK_OUT;
+    if (o->kind == kObjCast) {
+      // widening conversions do not change the register value
+      const DataType s = o->in[0]->type_id_, d = o->type_id_;
+      const bool nop = (d == kFloat32 && (s == kFloat16 || s == kBFloat16)) || (s == kBool && d != kInt32);
+      if (nop) kind = AK_ALIAS;
+    }
+    const int idx = AddNode(kind, o, o->type_id_, o->shape_ref_->data, o->rank());
+    ANode &n = nodes_[idx];
+    n.nin = o->nin;
+    for (int j = 0; j < 3; ++j) n.in[j] = in_idx[j];
+    if (kind == AK_OUT) n.addr_op = i;
+    node_of_[i] = idx;
+    // a value later sub-kernels read and that the user does not store: write it to workspace
+    if (mat_[i] && ws_slot_[i] >= 0) {
+      const int out = AddNode(AK_OUT, o, o->type_id_, o->shape_ref_->data, o->rank());
+      nodes_[out].nin = 1;
+      nodes_[out].in[0] = idx;
+      nodes_[out].ws_slot = ws_slot_[i];
+    }
+  }
+}
+
+// Unifies the dims of `in` with the right-aligned dims of `out` (NumPy broadcasting).
+void Compiler::UnifyAligned(int out, int in) {
+  const ANode &o = nodes_[out], &x = nodes_[in];
+  for (int i = 0; i < x.rank; ++i) {
+    const int oi = i + o.rank - x.rank;
+    if (oi < 0) {
+      if (x.dims[i] != 1) Fail("operand rank exceeds result rank");
+      continue;
+    }
+    if (x.dims[i] != 1 && x.dims[i] == o.dims[oi]) Union(Var(out, oi), Var(in, i));
+  }
+}
+
+void Compiler::UnifyAxes() {
+  uf_.resize(static_cast<size_t>(nn_) * kMaxRank);
+  for (size_t i = 0; i < uf_.size(); ++i) uf_[i] = static_cast<int>(i);
+  std::vector<char> reduced_var(uf_.size(), 0);
+  for (int i = 0; i < nn_; ++i) {
+    ANode &n = nodes_[i];
+    switch (n.kind) {
+      case AK_MEM:
+      case AK_SCALAR:
+        break;
+      case AK_OUT:
+        for (int d = 0; d < n.rank; ++d) Union(Var(i, d), Var(n.in[0], d));
+        break;
+      case AK_REDUCE: {
+        const ANode &x = nodes_[n.in[0]];
+        bool red[kMaxRank] = {false};
+        for (size_t j = 0; j < n.op->aux_ref->size; ++j) {
+          int64_t d = n.op->aux_ref->data[j];
+          red[d < 0 ? d + x.rank : d] = true;
+        }
+        int od = 0;
+        for (int d = 0; d < x.rank; ++d) {
+          if (red[d]) {
+            if (x.dims[d] != 1) reduced_var[Var(n.in[0], d)] = 1;
+            if (n.op->keepdims) ++od;
+          } else {
+            Union(Var(i, od), Var(n.in[0], d));
+            ++od;
+          }
+        }
+        break;
+      }
+      case AK_ALIAS:
+        if (n.op->kind == kObjReshape) {
+          const ANode &x = nodes_[n.in[0]];
+          int a = 0, b = 0;
+          while (true) {
+            while (a < x.rank && x.dims[a] == 1) ++a;
+            while (b < n.rank && n.dims[b] == 1) ++b;
+            if (a == x.rank || b == n.rank) break;
+            Union(Var(i, b), Var(n.in[0], a));
+            ++a;
+            ++b;
+          }
+        } else {
+          UnifyAligned(i, n.in[0]);
+        }
+        break;
+      case AK_OP:
+        for (int j = 0; j < n.nin; ++j)
+          if (n.in[j] >= 0) UnifyAligned(i, n.in[j]);
+        break;
+    }
+  }
+  // classes with extent > 1 become domain axes
+  n_axes_ = 0;
+  std::vector<int> axis_of(uf_.size(), -1);
+  for (int i = 0; i < nn_; ++i) {
+    ANode &n = nodes_[i];
+    for (int d = 0; d < n.rank; ++d) {
+      if (n.dims[d] == 1) continue;
+      const int root = Find(Var(i, d));
+      if (axis_of[root] < 0) {
+        if (n_axes_ >= kMaxAxes) Fail("too many axes");
+        axis_of[root] = n_axes_;
+        axes_[n_axes_].extent = n.dims[d];
+        axes_[n_axes_].reduced = false;
+        axes_[n_axes_].before = 0;
+        ++n_axes_;
+      }
+      if (axes_[axis_of[root]].extent != n.dims[d]) Fail("inconsistent axis extents");
+      n.axis[d] = axis_of[root];
+    }
+  }
+  for (size_t v = 0; v < uf_.size(); ++v) {
+    if (!reduced_var[v]) continue;
+    const int ax = axis_of[Find(static_cast<int>(v))];
+    if (ax >= 0) axes_[ax].reduced = true;
+  }
+  // every reduce must reduce exactly the reduced axes present in its input
+  for (int i = 0; i < nn_; ++i) {
+    const ANode &n = nodes_[i];
+    if (n.kind != AK_REDUCE) continue;
+    const ANode &x = nodes_[n.in[0]];
+    uint32_t in_axes = 0, out_axes = 0;
+    for (int d = 0; d < x.rank; ++d)
+      if (x.axis[d] >= 0) in_axes |= 1u << x.axis[d];
+    for (int d = 0; d < n.rank; ++d)
+      if (n.axis[d] >= 0) out_axes |= 1u << n.axis[d];
+    for (int ax = 0; ax < n_axes_; ++ax) {
+      const bool in_has = (in_axes >> ax) & 1u, out_has = (out_axes >> ax) & 1u;
+      if (in_has && axes_[ax].reduced == out_has) Fail("reduces over different axes in one sub-kernel");
+    }
+  }
+  // no value may have the same axis twice
+  for (int i = 0; i < nn_; ++i) {
+    uint32_t seen = 0;
+    for (int d = 0; d < nodes_[i].rank; ++d) {
+      const int ax = nodes_[i].axis[d];
+      if (ax < 0) continue;
+      if ((seen >> ax) & 1u) Fail("axis used twice by one value");
+      seen |= 1u << ax;
+    }
+  }
+}
+
+void Compiler::OrderAndMerge() {
+  // order constraints: within a value, an earlier dim is outside a later dim
+  for (int i = 0; i < nn_; ++i) {
+    const ANode &n = nodes_[i];
+    uint32_t outer = 0;
+    for (int d = 0; d < n.rank; ++d) {
+      if (n.axis[d] < 0) continue;
+      axes_[n.axis[d]].before |= outer;
+      outer |= 1u << n.axis[d];
+    }
+  }
+  uint32_t placed = 0;
+  for (int k = 0; k < n_axes_; ++k) {
+    int pick = -1;
+    for (int ax = 0; ax < n_axes_; ++ax) {
+      if ((placed >> ax) & 1u) continue;
+      if ((axes_[ax].before & ~placed) == 0) {
+        pick = ax;
+        break;
+      }
+    }
+    if (pick < 0) Fail("values disagree on the order of axes");
+    order_[k] = pick;
+    pos_[pick] = k;
+    placed |= 1u << pick;
+  }
+  // merge neighbours that every memory operand either holds contiguously or lacks
+  n_dims_ = 0;
+  for (int k = 0; k < n_axes_; ++k) {
+    bool merge = false;
+    if (k > 0) {
+      const int a0 = order_[k - 1], a1 = order_[k];
+      merge = axes_[a0].reduced == axes_[a1].reduced;
+      for (int i = 0; i < nn_ && merge; ++i) {
+        const ANode &n = nodes_[i];
+        if (n.kind != AK_MEM && n.kind != AK_OUT) continue;
+        int d0 = -1, d1 = -1;
+        for (int d = 0; d < n.rank; ++d) {
+          if (n.axis[d] == a0) d0 = d;
+          if (n.axis[d] == a1) d1 = d;
+        }
+        if ((d0 < 0) != (d1 < 0)) merge = false;
+        if (d0 >= 0 && d1 >= 0) {
+          // contiguous only if nothing of extent > 1 lies between them
+          for (int d = d0 + 1; d < d1; ++d)
+            if (n.dims[d] != 1) merge = false;
+        }
+      }
+    }
+    if (merge) {
+      dims_[n_dims_ - 1].extent *= axes_[order_[k]].extent;
+      dims_[n_dims_ - 1].last_axis = k;
+    } else {
+      dims_[n_dims_].extent = axes_[order_[k]].extent;
+      dims_[n_dims_].reduced = axes_[order_[k]].reduced;
+      dims_[n_dims_].first_axis = dims_[n_dims_].last_axis = k;
+      ++n_dims_;
+    }
+    dim_of_axis_[k] = n_dims_ - 1;
+  }
+  if (n_dims_ == 0) {  // every extent is 1
+    dims_[0].extent = 1;
+    dims_[0].reduced = false;
+    dims_[0].first_axis = dims_[0].last_axis = -1;
+    n_dims_ = 1;
+  }
+  nk_ = nr_ = 0;
+  for (int d = n_dims_ - 1; d >= 0; --d) {
+    if (dims_[d].reduced) {
+      if (nr_ >= DVM_VEC_MAXR) Fail("too many reduced dims");
+      rlist_[nr_++] = d;
+    } else {
+      if (nk_ >= DVM_VEC_MAXR) Fail("too many kept dims");
+      klist_[nk_++] = d;
+    }
+  }
+}
+
+// ---------- schedule and geometry ----------
+
+namespace {
+uint32_t Pow2Ceil(uint64_t v) {
+  uint32_t p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+uint32_t Log2(uint32_t v) {
+  uint32_t l = 0;
+  while ((1u << l) < v) ++l;
+  return l;
+}
+}  // namespace
+
+void Compiler::ChooseSchedule() {
+  std::memset(&hdr_, 0, sizeof(hdr_));
+  hdr_.entry = VE_VECTOR;
+  const int inner = n_dims_ - 1;
+  const bool inner_red = dims_[inner].reduced;
+  hdr_.inner_extent = static_cast<uint32_t>(dims_[inner].extent);
+  hdr_.inner_reduced = inner_red ? 1 : 0;
+  const uint64_t inner_groups = (static_cast<uint64_t>(dims_[inner].extent) + E - 1) / E;
+  uint64_t n_k = 1, n_r = 1;
+  for (int i = 0; i < nk_; ++i) {
+    const uint64_t ext = klist_[i] == inner ? inner_groups : static_cast<uint64_t>(dims_[klist_[i]].extent);
+    hdr_.kdims[i] = MakeVDim(static_cast<uint32_t>(ext));
+    n_k *= ext;
+  }
+  for (int i = 0; i < nr_; ++i) {
+    const uint64_t ext = rlist_[i] == inner ? inner_groups : static_cast<uint64_t>(dims_[rlist_[i]].extent);
+    hdr_.rdims[i] = MakeVDim(static_cast<uint32_t>(ext));
+    n_r *= ext;
+  }
+  for (int i = nk_; i < DVM_VEC_MAXR; ++i) hdr_.kdims[i] = MakeVDim(1);
+  for (int i = nr_; i < DVM_VEC_MAXR; ++i) hdr_.rdims[i] = MakeVDim(1);
+  if (n_k >= (1ull << 31) || n_r >= (1ull << 31)) Fail("index space above 2^31 groups");
+  for (int d = 0; d < n_dims_; ++d)
+    if (dims_[d].extent >= (1ll << 32)) Fail("axis extent above 2^32");
+  hdr_.n_kdim = nk_;
+  hdr_.n_rdim = nr_;
+  hdr_.n_kidx = static_cast<uint32_t>(n_k);
+  hdr_.n_ridx = static_cast<uint32_t>(n_r);
+  uint32_t threads = 256;
+  single_round_ = true;
+  if (nr_ == 0) {
+    hdr_.sched = VS_POINTWISE;
+    if (n_k <= 64 * U) threads = 64;
+    else if (n_k <= 128 * U) threads = 128;
+    hdr_.n_items = static_cast<uint32_t>((n_k + static_cast<uint64_t>(threads) * U - 1) / (threads * U));
+    n_sec_ = 1;
+  } else if (inner_red) {
+    hdr_.sched = VS_REDX;
+    // lanes that share one output: enough to cover the reduce space in one round if possible
+    uint32_t team = Pow2Ceil((n_r + U - 1) / U);
+    if (team > 1024) team = 1024;
+    if (team > 64) {
+      hdr_.team_is_block = 1;
+      threads = team;
+      hdr_.team_log2 = Log2(team);
+      hdr_.n_items = static_cast<uint32_t>(n_k);
+    } else {
+      hdr_.team_is_block = 0;
+      hdr_.team_log2 = Log2(team);
+      threads = n_k * team >= 256 ? 256 : std::max<uint32_t>(64, Pow2Ceil(n_k * team));
+      const uint32_t per_wg = threads / team;
+      hdr_.n_items = static_cast<uint32_t>((n_k + per_wg - 1) / per_wg);
+    }
+    single_round_ = n_r <= static_cast<uint64_t>(team) * U;
+  } else {
+    hdr_.sched = VS_REDY;
+    uint32_t tx = n_k >= 64 ? 64 : Pow2Ceil(n_k);
+    uint32_t ty = 256 / tx;
+    const uint64_t items = (n_k + tx - 1) / tx;
+    if (items < 128 && n_r > 256) ty = 1024 / tx;  // few outputs: give each more lanes along the reduce space
+    while (ty > 1 && static_cast<uint64_t>(ty) * U > 2 * n_r) ty >>= 1;
+    threads = std::max<uint32_t>(64, tx * ty);
+    ty = threads / tx;
+    hdr_.team_log2 = Log2(tx);
+    hdr_.n_items = static_cast<uint32_t>(items);
+    single_round_ = n_r <= static_cast<uint64_t>(ty) * U;
+  }
+  prog_->threads = threads;
+}
+
+// ---------- emission ----------
+
+int Compiler::MemIndex(int v) {
+  ANode &n = nodes_[v];
+  if (n.mem_idx >= 0) return n.mem_idx;
+  if (n_mem_ >= DVM_VEC_MAXMEM) Fail("too many memory operands");
+  VMemDesc &m = mems_[n_mem_];
+  std::memset(&m, 0, sizeof(m));
+  m.dtype = MemDType(n.dtype);
+  // element stride of every axis the operand has (row-major over its own shape)
+  int64_t stride = 1;
+  int64_t dim_stride[kMaxAxes];
+  bool dim_has[kMaxAxes] = {false};
+  for (int d = n.rank - 1; d >= 0; --d) {
+    if (n.axis[d] >= 0) {
+      const int p = pos_[n.axis[d]];
+      const int md = dim_of_axis_[p];
+      dim_has[md] = true;
+      if (p == dims_[md].last_axis) dim_stride[md] = stride;  // the innermost axis of a merged dim carries its stride
+    }
+    stride *= n.dims[d];
+  }
+  const int inner = n_dims_ - 1;
+  bool aligned = true;
+  const int64_t isz = static_cast<int64_t>(DTypeSize(n.dtype));
+  const int64_t need = isz * E >= 16 ? 16 : isz * E;
+  for (int i = 0; i < nk_; ++i) {
+    const int md = klist_[i];
+    if (!dim_has[md]) continue;
+    if (dim_stride[md] >= (1ll << 32)) Fail("stride above 2^32");
+    m.kstride[i] = static_cast<uint32_t>(dim_stride[md]);
+    if (md != inner && (dim_stride[md] * isz) % need != 0) aligned = false;
+  }
+  for (int i = 0; i < nr_; ++i) {
+    const int md = rlist_[i];
+    if (!dim_has[md]) continue;
+    if (dim_stride[md] >= (1ll << 32)) Fail("stride above 2^32");
+    m.rstride[i] = static_cast<uint32_t>(dim_stride[md]);
+    if (md != inner && (dim_stride[md] * isz) % need != 0) aligned = false;
+  }
+  if (dim_has[inner] && dims_[inner].first_axis >= 0) {
+    if (dim_stride[inner] != 1) Fail("innermost axis is not contiguous");
+    m.flags |= VMF_VEC;
+    if (aligned) m.flags |= VMF_ALIGNED;
+  }
+  Program::Patch p;
+  p.word = static_cast<uint32_t>(n_mem_);
+  p.op_id = n.addr_op;
+  p.ws_slot = n.ws_slot;
+  prog_->patches.push_back(p);
+  n.mem_idx = n_mem_++;
+  return n.mem_idx;
+}
+
+int Compiler::AllocSReg() {
+  for (int i = 0; i < DVM_VEC_NSREG; ++i) {
+    if (!((sreg_used_ >> i) & 1u)) {
+      sreg_used_ |= 1u << i;
+      return i;
+    }
+  }
+  Fail("out of S registers");
+  return -1;
+}
+
+int Compiler::AllocVSlot(int n) {
+  for (int i = 0; i + n <= vslot_limit_; ++i) {
+    const uint32_t msk = ((1u << n) - 1u) << i;
+    if ((vslot_used_ & msk) == 0) {
+      vslot_used_ |= msk;
+      max_vslot_ = std::max(max_vslot_, i + n);
+      return i;
+    }
+  }
+  Fail("out of V register slots");
+  return -1;
+}
+
+void Compiler::ReleaseReg(int v) {
+  ANode &n = nodes_[v];
+  if (n.reg < 0) return;
+  if (!n.has_inner) {
+    sreg_used_ &= ~(1u << n.reg);
+  } else {
+    const int cnt = n.reg_fmt == VF_F32 ? 2 : 1;
+    vslot_used_ &= ~(((1u << cnt) - 1u) << n.reg);
+  }
+  n.reg = -1;
+}
+
+void Compiler::SaveAcc(int v) {
+  ANode &n = nodes_[v];
+  if (n.reg >= 0) return;
+  if (!n.has_inner) {
+    n.reg = AllocSReg();
+    Emit(VOP_STS, 0, 0, 0, n.reg, 0);
+  } else {
+    n.reg_fmt = n.dtype == kFloat16 ? VF_F16 : (n.dtype == kBFloat16 ? VF_BF16 : VF_F32);
+    if (n.dtype == kBool) n.reg_fmt = VF_F16;
+    n.reg = AllocVSlot(n.reg_fmt == VF_F32 ? 2 : 1);
+    Emit(VOP_STR, n.reg_fmt, 0, 0, n.reg, 0);
+  }
+}
+
+// Called before an instruction replaces the accumulator by an unrelated value.
+void Compiler::BeforeOverwrite() {
+  if (acc_node_ < 0) return;
+  ANode &n = nodes_[acc_node_];
+  if (n.kind == AK_MEM || n.kind == AK_SCALAR) return;  // cheaper to fetch again than to park
+  const bool needed_later = n.last_sec > cur_sec_ && (!n.fd || single_round_);
+  if ((n.uses > 0 || needed_later) && n.reg < 0) SaveAcc(acc_node_);
+}
+
+void Compiler::ConsumeUse(int v) {
+  ANode &n = nodes_[v];
+  if (n.uses > 0) --n.uses;
+  const bool needed_later = n.last_sec > cur_sec_ && (!n.fd || single_round_);
+  if (n.uses == 0 && !needed_later && n.reg >= 0) ReleaseReg(v);
+}
+
+bool Compiler::SimpleOperand(int v) {
+  const ANode &n = nodes_[v];
+  if (n.reg >= 0) return true;
+  if (acc_node_ == v) return false;
+  return n.kind == AK_MEM || n.kind == AK_SCALAR;
+}
+
+// acc = acc (op) value-of-v, v being a simple operand.
+void Compiler::EmitOperandInsn(uint32_t op, uint32_t sub, uint32_t rnd, int v) {
+  ANode &n = nodes_[v];
+  if (n.reg >= 0) {
+    if (!n.has_inner) {
+      Emit(op, sub, VK_SREG, rnd, n.reg, 0);
+    } else {
+      Emit(op, sub | (static_cast<uint32_t>(n.reg_fmt) << 6), VK_REG, rnd, n.reg, 0);
+    }
+  } else if (n.kind == AK_MEM) {
+    Emit(op, sub, VK_MEM, rnd, MemIndex(v), 0);
+  } else if (n.kind == AK_SCALAR) {
+    Emit(op, sub, VK_IMM, rnd, 0, ScalarToContainer(n.op->scalar.Get(), n.dtype));
+  } else {
+    Fail("operand is not addressable");
+  }
+  ConsumeUse(v);
+}
+
+// Puts value v into the accumulator.
+void Compiler::EmitValue(int v) {
+  v = Resolve(v);
+  if (acc_node_ == v) return;
+  ANode &n = nodes_[v];
+  if (n.reg >= 0) {
+    BeforeOverwrite();
+    if (!n.has_inner) {
+      Emit(VOP_LDS, 0, 0, 0, n.reg, 0);
+    } else {
+      Emit(VOP_LDR, n.reg_fmt, 0, 0, n.reg, 0);
+    }
+    acc_node_ = v;
+    return;
+  }
+  ComputeInto(v);
+  acc_node_ = v;
+}
+
+namespace {
+uint32_t BinSubF(int op, bool reversed) {
+  switch (op) {
+    case kAdd: return VB_ADD;
+    case kSub: return reversed ? VB_RSUB : VB_SUB;
+    case kMul: return VB_MUL;
+    case kDiv: return reversed ? VB_RDIV : VB_DIV;
+    case kPow: return reversed ? VB_RPOW : VB_POW;
+    case kMaximum: return VB_MAX;
+    case kMinimum: return VB_MIN;
+    case kLogicalAnd: return VB_AND;
+    case kLogicalOr: return VB_OR;
+    default: Throw("binary operator without a device form");
+  }
+}
+uint32_t BinSubI(int op, bool reversed) {
+  switch (op) {
+    case kAdd: return VBI_ADD;
+    case kSub: return reversed ? VBI_RSUB : VBI_SUB;
+    case kMul: return VBI_MUL;
+    case kMaximum: return VBI_MAX;
+    case kMinimum: return VBI_MIN;
+    default: Throw("binary operator without an int32 form");
+  }
+}
+uint32_t CmpSub(int op, bool reversed, bool is_int) {
+  static const uint32_t rev[6] = {VCMP_EQ, VCMP_NE, VCMP_LT, VCMP_LE, VCMP_GT, VCMP_GE};
+  uint32_t t = static_cast<uint32_t>(op);  // kEqual..kLessEqual == VCMP_EQ..VCMP_LE
+  if (reversed) t = rev[t];
+  return t + (is_int ? VCMP_INT : 0);
+}
+bool NeedsRounding(int op) { return op == kAdd || op == kSub || op == kMul || op == kDiv || op == kPow; }
+}  // namespace
+
+// Emits the code that computes v (not in a register, not in the accumulator).
+void Compiler::ComputeInto(int v) {
+  ANode &n = nodes_[v];
+  NDObject *o = n.op;
+  switch (n.kind) {
+    case AK_MEM:
+      BeforeOverwrite();
+      Emit(VOP_LD, 0, VK_MEM, 0, MemIndex(v), 0);
+      return;
+    case AK_SCALAR:
+      BeforeOverwrite();
+      Emit(VOP_LDI, 0, 0, 0, 0, ScalarToContainer(o->scalar.Get(), n.dtype));
+      return;
+    case AK_REDUCE:
+      Fail("reduce result used before it is complete");
+      return;
+    default:
+      break;
+  }
+  const bool is_int = (o->kind == kObjCompare || o->kind == kObjCompareS || o->kind == kObjBinary ||
+                       o->kind == kObjBinaryS || o->kind == kObjUnary)
+                          ? nodes_[Resolve(n.in[0])].dtype == kInt32
+                          : false;
+  switch (o->kind) {
+    case kObjUnary: {
+      const int x = Resolve(n.in[0]);
+      EmitValue(x);
+      ConsumeUse(x);
+      BeforeOverwrite();
+      uint32_t sub;
+      bool rnd = false;
+      switch (o->op) {
+        case kSqrt: sub = VU_SQRT; rnd = true; break;
+        case kAbs: sub = is_int ? VU_IABS : VU_ABS; break;
+        case kLog: sub = VU_LOG; rnd = true; break;
+        case kExp: sub = VU_EXP; rnd = true; break;
+        case kIsFinite: sub = VU_ISFINITE; break;
+        case kRound: sub = VU_ROUND; break;
+        case kFloor: sub = VU_FLOOR; break;
+        case kCeil: sub = VU_CEIL; break;
+        case kTrunc: sub = VU_TRUNC; break;
+        default: Throw("unary operator without a device form");
+      }
+      Emit(VOP_UN, sub, 0, rnd ? RndOf(n.dtype) : 0, 0, 0);
+      return;
+    }
+    case kObjCast: {
+      const int x = Resolve(n.in[0]);
+      const DataType s = nodes_[x].dtype, d = n.dtype;
+      EmitValue(x);
+      ConsumeUse(x);
+      BeforeOverwrite();
+      if (d == kInt32) {
+        Emit(VOP_CAST, VC_F2I, 0, 0, 0, 0);
+      } else if (s == kInt32) {
+        Emit(VOP_CAST, VC_I2F, 0, RndOf(d), 0, 0);
+      } else if (d == kBool) {
+        Emit(VOP_CAST, VC_F2B, 0, 0, 0, 0);
+      } else {
+        Emit(VOP_CAST, VC_RND, 0, RndOf(d), 0, 0);
+      }
+      return;
+    }
+    case kObjBinaryS:
+    case kObjCompareS: {
+      const int x = Resolve(n.in[0]);
+      EmitValue(x);
+      ConsumeUse(x);
+      BeforeOverwrite();
+      const uint32_t imm = ScalarToContainer(o->scalar.Get(), nodes_[x].dtype);
+      if (o->kind == kObjCompareS) {
+        Emit(VOP_CMP, CmpSub(o->op, o->scalar_left, is_int), VK_IMM, 0, 0, imm);
+      } else if (is_int) {
+        Emit(VOP_BINI, BinSubI(o->op, o->scalar_left), VK_IMM, 0, 0, imm);
+      } else {
+        Emit(VOP_BINF, BinSubF(o->op, o->scalar_left), VK_IMM, NeedsRounding(o->op) ? RndOf(n.dtype) : 0, 0, imm);
+      }
+      return;
+    }
+    case kObjBinary:
+    case kObjCompare: {
+      int a = Resolve(n.in[0]), b = Resolve(n.in[1]);
+      bool reversed = false;
+      uint32_t opc, sub, rnd = 0;
+      auto pick = [&](bool rev) {
+        if (o->kind == kObjCompare) {
+          opc = VOP_CMP;
+          sub = CmpSub(o->op, rev, is_int);
+        } else if (is_int) {
+          opc = VOP_BINI;
+          sub = BinSubI(o->op, rev);
+        } else {
+          opc = VOP_BINF;
+          sub = BinSubF(o->op, rev);
+          rnd = NeedsRounding(o->op) ? RndOf(n.dtype) : 0;
+        }
+      };
+      if (a == b) {
+        EmitValue(a);
+        ConsumeUse(a);
+        ConsumeUse(a);
+        BeforeOverwrite();
+        pick(false);
+        Emit(opc, sub, VK_ACC, rnd, 0, 0);
+        return;
+      }
+      if (acc_node_ == b) {
+        std::swap(a, b);
+        reversed = true;
+      }
+      if (acc_node_ == a) {
+        if (!SimpleOperand(b)) {
+          // computing b would clobber a: park a, compute b, then use a as the operand
+          SaveAcc(a);
+          EmitValue(b);
+          std::swap(a, b);
+          reversed = !reversed;
+        }
+      } else if (SimpleOperand(b)) {
+        EmitValue(a);
+      } else if (SimpleOperand(a)) {
+        EmitValue(b);
+        std::swap(a, b);
+        reversed = true;
+      } else {
+        EmitValue(b);
+        SaveAcc(b);
+        EmitValue(a);
+      }
+      ConsumeUse(a);
+      BeforeOverwrite();
+      pick(reversed);
+      EmitOperandInsn(opc, sub, rnd, b);
+      return;
+    }
+    case kObjSelect: {
+      const int c = Resolve(n.in[0]), x = Resolve(n.in[1]), y = Resolve(n.in[2]);
+      if (!SimpleOperand(c)) {
+        EmitValue(c);
+        SaveAcc(c);
+      }
+      if (!SimpleOperand(x)) {
+        EmitValue(x);
+        SaveAcc(x);
+      }
+      EmitValue(y);
+      ConsumeUse(y);
+      BeforeOverwrite();
+      EmitOperandInsn(VOP_MSK, 0, 0, c);
+      EmitOperandInsn(VOP_MOVM, 0, 0, x);
+      return;
+    }
+    default:
+      Fail("operator without a vector form");
+  }
+}
+
+// Counts, for the section being emitted, how often each value of the cone is read.
+void Compiler::CountCone(int v) {
+  v = Resolve(v);
+  ANode &n = nodes_[v];
+  ++n.uses;
+  if (n.in_cone) return;
+  n.in_cone = true;
+  if (n.reg >= 0 || n.kind == AK_MEM || n.kind == AK_SCALAR || n.kind == AK_REDUCE) return;
+  for (int j = 0; j < n.nin; ++j)
+    if (n.in[j] >= 0) CountCone(n.in[j]);
+}
+
+void Compiler::EmitSection(int sec) {
+  cur_sec_ = sec;
+  const bool sweep = (sec & 1) != 0;
+  for (int i = 0; i < nn_; ++i) {
+    nodes_[i].uses = 0;
+    nodes_[i].in_cone = false;
+  }
+  if (!sweep && sec > 0) {
+    // results of the previous sweep's reduces become register values
+    for (int i = 0; i < nn_; ++i) {
+      ANode &n = nodes_[i];
+      if (n.kind != AK_REDUCE || n.sec != sec - 1) continue;
+      BeforeOverwrite();
+      Emit(VOP_FIN, 0, 0, 0, n.reg_fmt, 0);
+      acc_node_ = i;
+      SaveAcc(i);
+    }
+  }
+  // sinks of this section, in node order
+  int sinks[kMaxNodes];
+  int ns = 0;
+  for (int i = 0; i < nn_; ++i) {
+    const ANode &n = nodes_[i];
+    if ((n.kind == AK_REDUCE || n.kind == AK_OUT) && n.sec == sec) sinks[ns++] = i;
+  }
+  // values computed here that a later section reads from a register
+  int keep[kMaxNodes];
+  int nkp = 0;
+  for (int i = 0; i < nn_; ++i) {
+    const ANode &n = nodes_[i];
+    if (n.sec != sec || n.last_sec <= sec) continue;
+    if (n.kind == AK_MEM) {
+      // an operand that does not vary inside the sweeps is loaded once per output into an S register
+      if (sweep || n.has_inner || n_sec_ == 1) continue;
+      if (__builtin_popcount(sreg_used_) >= DVM_VEC_NSREG - 3) continue;
+      keep[nkp++] = i;
+      continue;
+    }
+    if (n.kind != AK_OP) continue;
+    if (n.fd && !single_round_) continue;  // recomputed by the later sweep
+    keep[nkp++] = i;
+  }
+  if (sweep) {
+    uint32_t kinds = 0xff;
+    int slot = 0;
+    for (int i = 0; i < ns; ++i) {
+      ANode &n = nodes_[sinks[i]];
+      if (n.kind != AK_REDUCE) continue;
+      if (slot >= DVM_VEC_NSLOT) Fail("more than two reduces in one sweep");
+      const uint32_t rk = n.op->op == kSum ? VR_SUM : (n.op->op == kMax ? VR_MAX : VR_MIN);
+      kinds = (kinds & ~(0xfu << (4 * slot))) | (rk << (4 * slot));
+      n.reg_fmt = static_cast<uint8_t>(slot);  // slot number until the result is fetched
+      ++slot;
+    }
+    BeforeOverwrite();
+    Emit(VOP_SWEEP, 0, 0, 0, 0, kinds);
+    if (!single_round_) acc_node_ = -1;
+  }
+  for (int i = 0; i < ns; ++i) CountCone(nodes_[sinks[i]].in[0]);
+  for (int i = 0; i < nkp; ++i) CountCone(keep[i]);
+  for (int i = 0; i < ns; ++i) {
+    ANode &n = nodes_[sinks[i]];
+    const int x = Resolve(n.in[0]);
+    EmitValue(x);
+    if (n.kind == AK_REDUCE) {
+      const uint32_t rk = n.op->op == kSum ? VR_SUM : (n.op->op == kMax ? VR_MAX : VR_MIN);
+      Emit(VOP_RED, rk, 0, 0, n.reg_fmt, 0);
+    } else {
+      Emit(VOP_ST, 0, 0, 0, MemIndex(sinks[i]), 0);
+    }
+    ConsumeUse(x);
+  }
+  for (int i = 0; i < nkp; ++i) {
+    const int v = keep[i];
+    if (nodes_[v].reg < 0) {
+      EmitValue(v);
+      SaveAcc(v);
+    }
+    ConsumeUse(v);
+  }
+  if (sweep) {
+    if (!single_round_) BeforeOverwrite();
+    Emit(VOP_ENDSWEEP, 0, 0, 0, 0, 0);
+    if (!single_round_) acc_node_ = -1;
+  }
+}
+
+void Compiler::EmitProgram() {
+  const int inner = n_dims_ - 1;
+  const int inner_first = dims_[inner].first_axis, inner_last = dims_[inner].last_axis;
+  // classify values
+  for (int i = 0; i < nn_; ++i) {
+    ANode &n = nodes_[i];
+    n.has_inner = false;
+    n.fd = false;
+    for (int d = 0; d < n.rank; ++d) {
+      if (n.axis[d] < 0) continue;
+      const int p = pos_[n.axis[d]];
+      if (inner_first >= 0 && p >= inner_first && p <= inner_last) n.has_inner = true;
+      if (axes_[n.axis[d]].reduced) n.fd = true;
+    }
+    // Only a value that is the same for every slab of a lane fits an S register: slabs differ in
+    // the kept position (pointwise) or in the reduce position (sweeps).
+    if (n.fd || nr_ == 0) n.has_inner = true;
+  }
+  int max_level = 0;
+  for (int i = 0; i < nn_; ++i) {
+    ANode &n = nodes_[i];
+    n.level = 0;
+    for (int j = 0; j < n.nin; ++j) {
+      if (n.in[j] < 0) continue;
+      const ANode &x = nodes_[n.in[j]];
+      n.level = std::max(n.level, x.level + (x.kind == AK_REDUCE ? 1 : 0));
+    }
+    if (n.kind == AK_REDUCE) {
+      // the reduce runs in the sweep of its input's level
+      n.sec = 2 * n.level + 1;
+    } else if (nr_ == 0) {
+      n.sec = 0;
+    } else {
+      n.sec = 2 * n.level + (n.fd ? 1 : 0);
+    }
+    max_level = std::max(max_level, n.level);
+  }
+  // aliases inherit the class of what they resolve to
+  for (int i = 0; i < nn_; ++i) {
+    ANode &n = nodes_[i];
+    if (n.kind == AK_ALIAS) {
+      const ANode &r = nodes_[Resolve(i)];
+      n.sec = r.sec;
+    }
+  }
+  // an output's section is that of the value it stores
+  n_sec_ = nr_ == 0 ? 1 : 2 * (max_level + 1);
+  for (int i = 0; i < nn_; ++i) nodes_[i].last_sec = -1;
+  for (int i = 0; i < nn_; ++i) {
+    ANode &n = nodes_[i];
+    if (n.kind == AK_ALIAS) continue;
+    const int my_sec = n.sec;
+    for (int j = 0; j < n.nin; ++j) {
+      if (n.in[j] < 0) continue;
+      ANode &x = nodes_[Resolve(n.in[j])];
+      x.last_sec = std::max(x.last_sec, my_sec);
+    }
+  }
+  // values recomputed by a later sweep pull their own inputs forward
+  if (!single_round_) {
+    for (int pass = 0; pass < nn_; ++pass) {
+      bool changed = false;
+      for (int i = nn_ - 1; i >= 0; --i) {
+        ANode &n = nodes_[i];
+        if (n.kind != AK_OP || !n.fd) continue;
+        for (int j = 0; j < n.nin; ++j) {
+          if (n.in[j] < 0) continue;
+          ANode &x = nodes_[Resolve(n.in[j])];
+          if (x.last_sec < n.last_sec) {
+            x.last_sec = n.last_sec;
+            changed = true;
+          }
+        }
+      }
+      if (!changed) break;
+    }
+  }
+  // local memory budget for V registers
+  const uint32_t per_slot = static_cast<uint32_t>(U) * 16u * prog_->threads;
+  const uint32_t budget = g_system.lds_per_wg > 80 * 1024 ? 72 * 1024 : g_system.lds_per_wg - 8 * 1024;
+  vslot_limit_ = std::min<int>(DVM_VEC_NREG, static_cast<int>(budget / per_slot));
+  sreg_used_ = vslot_used_ = 0;
+  max_vslot_ = 0;
+  acc_node_ = -1;
+  code_.clear();
+  n_mem_ = 0;
+  for (int s = 0; s < n_sec_; ++s) EmitSection(s);
+  Emit(VOP_END, 0, 0, 0, 0, 0);
+}
+
+void Compiler::FinishProgram() {
+  hdr_.n_mem = n_mem_;
+  hdr_.n_code = static_cast<uint32_t>(code_.size());
+  hdr_.mem_off = sizeof(VVecHeader) / 8;
+  hdr_.code_off = hdr_.mem_off + n_mem_ * (sizeof(VMemDesc) / 8);
+  hdr_.n_vslot = max_vslot_;
+  if (hdr_.code_off + code_.size() > DVM_PARAM_WORDS) Fail("program larger than 4 KB");
+  std::memset(&prog_->blob, 0, sizeof(VmParam));
+  std::memcpy(prog_->blob.w, &hdr_, sizeof(hdr_));
+  std::memcpy(prog_->blob.w + hdr_.mem_off, mems_, sizeof(VMemDesc) * n_mem_);
+  std::memcpy(prog_->blob.w + hdr_.code_off, code_.data(), 8 * code_.size());
+  prog_->lds_bytes = prog_->threads * 8 + static_cast<uint32_t>(max_vslot_) * U * 16 * prog_->threads;
+  uint64_t gt = (static_cast<uint64_t>(std::min<uint32_t>(hdr_.n_items, g_system.core_num * 4)) << 32) | prog_->threads;
+  if (g_system.HasDevice()) {
+    gt = g_system.Api().select_block_thread(hdr_.sched, hdr_.n_items, prog_->threads, prog_->lds_bytes);
+  }
+  prog_->grid = static_cast<uint32_t>(gt >> 32);
+  if (prog_->grid == 0) prog_->grid = 1;
+}
+
+void Compiler::CompileArea(int a) {
+  k_->programs_.emplace_back();
+  prog_ = &k_->programs_.back();
+  if (areas_[a].cube) {
+    CompileCube(a);
+    return;
+  }
+  BuildNodes(a);
+  // an empty domain: nothing to run, outputs that still have elements are zero-filled
+  bool empty = false;
+  for (int i = 0; i < nn_; ++i) {
+    int64_t n = 1;
+    for (int d = 0; d < nodes_[i].rank; ++d) n *= nodes_[i].dims[d];
+    if (n == 0) empty = true;
+  }
+  if (empty) {
+    prog_->skip = true;
+    for (int i = 0; i < nn_; ++i) {
+      const ANode &n = nodes_[i];
+      if (n.kind != AK_OUT) continue;
+      int64_t cnt = 1;
+      for (int d = 0; d < n.rank; ++d) cnt *= n.dims[d];
+      if (cnt == 0) continue;
+      Program::Fill f;
+      f.op_id = n.addr_op;
+      f.ws_slot = n.ws_slot;
+      f.value = 0;
+      f.bytes = (static_cast<size_t>(cnt) * DTypeSize(n.dtype) + 3) & ~static_cast<size_t>(3);
+      prog_->fills.push_back(f);
+    }
+    return;
+  }
+  UnifyAxes();
+  OrderAndMerge();
+  ChooseSchedule();
+  // a stored value must span the index space it is stored from, or it would be written several times
+  for (int i = 0; i < nn_; ++i) {
+    const ANode &n = nodes_[i];
+    if (n.kind != AK_OUT) continue;
+    uint32_t have = 0;
+    bool fd = false;
+    for (int d = 0; d < n.rank; ++d) {
+      if (n.axis[d] < 0) continue;
+      have |= 1u << n.axis[d];
+      if (axes_[n.axis[d]].reduced) fd = true;
+    }
+    for (int ax = 0; ax < n_axes_; ++ax) {
+      if ((have >> ax) & 1u) continue;
+      if (!axes_[ax].reduced || fd) Fail("output smaller than the kernel domain");
+    }
+  }
+  EmitProgram();
+  FinishProgram();
+}
+
+void Compiler::CompileCube(int /*a*/) { Fail("matmul kernels are not available yet"); }
+
+size_t VKernel::CodeGen(bool /*pre*/) {
+  if (!normalized_) Normalize();
+  Compiler c(this);
+  const size_t ws = c.Run();
+  compiled_ = true;
+  return ws;
+}
+
+void VKernel::BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *alloc, void *workspace) {
+  for (size_t i = 0; i < n; ++i) {
+    if (relocs[i].io != nullptr) relocs[i].io->addr = relocs[i].addr;
+  }
+  if (ws_bytes_ > 0) {
+    if (workspace != nullptr) {
+      ws_base_ = workspace;
+    } else if (alloc != nullptr) {
+      ws_base_ = alloc->Alloc(ws_bytes_);
+    }
+    if (ws_base_ == nullptr) Throw("kernel needs workspace but none was provided");
+  }
+  for (Program &p : programs_) {
+    if (p.skip) continue;
+    const VVecHeader *h = reinterpret_cast<const VVecHeader *>(p.blob.w);
+    VMemDesc *mems = reinterpret_cast<VMemDesc *>(p.blob.w + h->mem_off);
+    for (const Program::Patch &pt : p.patches) {
+      uint64_t addr = 0;
+      if (pt.op_id >= 0) {
+        addr = reinterpret_cast<uint64_t>(ops_[pt.op_id]->addr);
+      } else if (pt.ws_slot >= 0) {
+        addr = reinterpret_cast<uint64_t>(ws_base_) + ws_offsets_[pt.ws_slot];
+      }
+      if (addr == 0) Throw("a tensor address is missing at launch");
+      VMemDesc &m = mems[pt.word];
+      m.addr = addr;
+      if ((addr & 15u) != 0) m.flags &= ~static_cast<uint32_t>(VMF_ALIGNED);
+    }
+  }
+}
+
+int VKernel::Launch(void *stream) {
+  if (!compiled_) Throw("Launch before CodeGen");
+  if (!g_system.HasDevice()) {
+    Throw(std::string("no MI355X device layer: ") + g_system.LoadError());
+  }
+  const DeviceApi &api = g_system.Api();
+  for (Program &p : programs_) {
+    for (const Program::Fill &f : p.fills) {
+      void *dst = f.op_id >= 0 ? ops_[f.op_id]->addr
+                               : static_cast<void *>(static_cast<char *>(ws_base_) + ws_offsets_[f.ws_slot]);
+      int rc = api.fill_u32(dst, f.value, f.bytes, stream);
+      if (rc != 0) return rc;
+    }
+    if (p.skip) continue;
+    int rc = api.launch_vm(&p.blob, p.grid, p.threads, p.lds_bytes, stream);
+    if (rc != 0) return rc;
+  }
+  return 0;
+}
+
+}  // namespace dvm

@@ -1,0 +1,194 @@
+// Text forms of a kernel: operator graph dump and bytecode disassembly.
+// Role in the reference: VKernel::DumpGraph and Code::Das (src/code.cc:27-1498).
+// The disassembly is one instruction per line, "<mnemonic>.<type> operands";
+// tests pin fusion decisions by counting these mnemonics.
+#include <cstdio>
+#include <sstream>
+
+#include "ir.h"
+#include "system.h"
+
+namespace dvm {
+
+namespace {
+
+const char *DTypeName(DataType t) {
+  switch (t) {
+    case kBool: return "bool";
+    case kFloat16: return "fp16";
+    case kBFloat16: return "bf16";
+    case kFloat32: return "fp32";
+    case kInt32: return "int32";
+    case kInt64: return "int64";
+    default: return "?";
+  }
+}
+
+const char *kUnaryNames[] = {"Sqrt", "Abs", "Log", "Exp", "Reciprocal", "IsFinite", "LogicalNot", "Round", "Floor", "Ceil", "Trunc"};
+const char *kBinaryNames[] = {"Equal", "NotEqual", "Greater", "GreaterEqual", "Less", "LessEqual", "Add", "Sub",
+                              "Mul", "Div", "Pow", "Maximum", "Minimum", "LogicalAnd", "LogicalOr"};
+const char *kReduceNames[] = {"Sum", "Max", "Min"};
+
+void PrintShape(std::ostringstream &os, const NDObject *o) {
+  os << "[";
+  for (int i = 0; i < o->rank(); ++i) os << (i ? "," : "") << o->dim(i);
+  os << "]";
+}
+
+const char *kMemTypes[] = {"bool", "fp16", "bf16", "fp32", "int32"};
+const char *kBinF[] = {"Add", "Sub", "RSub", "Mul", "Div", "RDiv", "Min", "Max", "And", "Or", "Pow", "RPow"};
+const char *kBinI[] = {"Add", "Sub", "RSub", "Mul", "Min", "Max"};
+const char *kUn[] = {"Sqrt", "Abs", "Log", "Exp", "IsFinite", "Round", "Floor", "Ceil", "Trunc", "Abs"};
+const char *kCmp[] = {"Eq", "Ne", "Gt", "Ge", "Lt", "Le"};
+const char *kRnd[] = {"fp32", "fp16", "bf16", "?"};
+const char *kRed[] = {"sum", "max", "min"};
+const char *kFmt[] = {"fp32", "fp16", "bf16", "?"};
+
+void PrintSrc(std::ostringstream &os, uint64_t w) {
+  char buf[64];
+  switch (VI_KIND(w)) {
+    case VK_REG: os << "v" << VI_A(w) << "." << kFmt[(VI_SUB(w) >> 6) & 3]; break;
+    case VK_SREG: os << "s" << VI_A(w); break;
+    case VK_MEM: os << "m" << VI_A(w); break;
+    case VK_ACC: os << "acc"; break;
+    default:
+      std::snprintf(buf, sizeof(buf), "#0x%08x", VI_IMM(w));
+      os << buf;
+      break;
+  }
+}
+
+}  // namespace
+
+std::string &VKernel::DumpGraph(bool ref_shapes) {
+  (void)ref_shapes;  // compute shapes and API shapes coincide on this backend
+  std::ostringstream os;
+  os << "kernel " << (name_.empty() ? "dvm" : name_) << " type=" << static_cast<int>(ktype_) << " flags=" << flags_ << "\n";
+  for (const NDObject *o : ops_) {
+    os << "%" << o->id << " = ";
+    switch (o->kind) {
+      case kObjLoad: os << "Load"; break;
+      case kObjStore: os << "Store"; break;
+      case kObjUnary: os << kUnaryNames[o->op]; break;
+      case kObjBinary: os << kBinaryNames[o->op]; break;
+      case kObjBinaryS: os << kBinaryNames[o->op] << "S" << (o->scalar_left ? "(scalar-left)" : ""); break;
+      case kObjCompare: os << kBinaryNames[o->op]; break;
+      case kObjCompareS: os << kBinaryNames[o->op] << "S" << (o->scalar_left ? "(scalar-left)" : ""); break;
+      case kObjSelect: os << "Select"; break;
+      case kObjCast: os << "Cast"; break;
+      case kObjBroadcast: os << "Broadcast"; break;
+      case kObjBroadcastS: os << "BroadcastS"; break;
+      case kObjReduce: os << "Reduce" << kReduceNames[o->op] << (o->keepdims ? "(keepdims)" : ""); break;
+      case kObjReshape: os << "Reshape"; break;
+      case kObjCopy: os << "Copy"; break;
+      case kObjMatMul: os << "MatMul" << (o->trans_a ? "T" : "N") << (o->trans_b ? "T" : "N"); break;
+    }
+    os << "." << DTypeName(o->type_id_) << "(";
+    for (int i = 0; i < o->nin; ++i) {
+      if (o->in[i] != nullptr) os << (i ? ", " : "") << "%" << o->in[i]->id;
+    }
+    os << ") ";
+    if (normalized_) PrintShape(os, o);
+    os << "\n";
+  }
+  dump_str_ = os.str();
+  return dump_str_;
+}
+
+std::string &VKernel::DisAssemble() {
+  std::ostringstream os;
+  if (!compiled_) {
+    dump_str_ = "<not compiled>\n";
+    return dump_str_;
+  }
+  int idx = 0;
+  for (const Program &p : programs_) {
+    os << "== sub-kernel " << idx++ << " ==\n";
+    if (p.skip) {
+      os << "idle (empty domain), " << p.fills.size() << " clean fill(s)\n";
+      continue;
+    }
+    const VVecHeader *h = reinterpret_cast<const VVecHeader *>(p.blob.w);
+    if (h->entry == VE_VECTOR) {
+      static const char *sched[] = {"pointwise", "reduce-x", "reduce-y"};
+      os << "entry vector sched=" << sched[h->sched] << " blocks=" << p.grid << " threads=" << p.threads
+         << " lds=" << p.lds_bytes << " items=" << h->n_items << " kept=" << h->n_kidx << " red=" << h->n_ridx
+         << " inner=" << h->inner_extent << " team=" << (h->team_is_block ? p.threads : (1u << h->team_log2))
+         << " vslots=" << h->n_vslot << "\n";
+      os << "  kdims:";
+      for (uint32_t i = 0; i < h->n_kdim; ++i) os << " " << h->kdims[i].extent;
+      os << "  rdims:";
+      for (uint32_t i = 0; i < h->n_rdim; ++i) os << " " << h->rdims[i].extent;
+      os << "\n";
+      const VMemDesc *mems = reinterpret_cast<const VMemDesc *>(p.blob.w + h->mem_off);
+      for (uint32_t i = 0; i < h->n_mem; ++i) {
+        char buf[32];
+        std::snprintf(buf, sizeof(buf), "0x%llx", static_cast<unsigned long long>(mems[i].addr));
+        os << "  m" << i << ": " << kMemTypes[mems[i].dtype] << " @" << buf << ((mems[i].flags & VMF_VEC) ? " vec" : " bcast")
+           << ((mems[i].flags & VMF_ALIGNED) ? " aligned" : "") << " k[";
+        for (uint32_t j = 0; j < h->n_kdim; ++j) os << (j ? "," : "") << mems[i].kstride[j];
+        os << "] r[";
+        for (uint32_t j = 0; j < h->n_rdim; ++j) os << (j ? "," : "") << mems[i].rstride[j];
+        os << "]\n";
+      }
+      const uint64_t *code = p.blob.w + h->code_off;
+      for (uint32_t i = 0; i < h->n_code; ++i) {
+        const uint64_t w = code[i];
+        const uint32_t sub = VI_SUB(w);
+        os << "  ";
+        switch (VI_OP(w)) {
+          case VOP_END: os << "end"; break;
+          case VOP_LDR: os << "mov acc, v" << VI_A(w) << "." << kFmt[sub & 3]; break;
+          case VOP_LDS: os << "mov acc, s" << VI_A(w); break;
+          case VOP_LDI: {
+            char buf[32];
+            std::snprintf(buf, sizeof(buf), "#0x%08x", VI_IMM(w));
+            os << "broadcast_s acc, " << buf;
+            break;
+          }
+          case VOP_STR: os << "mov v" << VI_A(w) << "." << kFmt[sub & 3] << ", acc"; break;
+          case VOP_STS: os << "mov s" << VI_A(w) << ", acc"; break;
+          case VOP_ST: os << "store." << kMemTypes[mems[VI_A(w)].dtype] << " m" << VI_A(w) << ", acc"; break;
+          case VOP_UN: os << kUn[sub] << "." << (sub == VU_IABS ? "int32" : kRnd[VI_RND(w)]) << " acc"; break;
+          case VOP_CAST: {
+            static const char *names[] = {"cast.f2i", "cast.i2f", "cast.round", "cast.f2b"};
+            os << names[sub] << "." << kRnd[VI_RND(w)] << " acc";
+            break;
+          }
+          case VOP_RED: os << "reduce_" << kRed[sub] << " r" << VI_A(w) << ", acc"; break;
+          case VOP_SWEEP: os << "sweep slots=" << kRed[(VI_IMM(w) & 0xf) < 3 ? (VI_IMM(w) & 0xf) : 0]
+                             << ((VI_IMM(w) & 0xf) < 3 ? "" : "(none)"); break;
+          case VOP_ENDSWEEP: os << "endsweep"; break;
+          case VOP_FIN: os << "mov acc, r" << VI_A(w); break;
+          case VOP_LD: os << "load." << kMemTypes[mems[VI_A(w)].dtype] << " acc, m" << VI_A(w); break;
+          case VOP_BINF: os << kBinF[sub & 0x3f] << "." << kRnd[VI_RND(w)] << " acc, "; PrintSrc(os, w); break;
+          case VOP_BINI: os << kBinI[sub & 0x3f] << ".int32 acc, "; PrintSrc(os, w); break;
+          case VOP_CMP: os << "Cmp" << kCmp[sub & 7] << "." << ((sub & VCMP_INT) ? "int32" : "fp32") << " acc, "; PrintSrc(os, w); break;
+          case VOP_MSK: os << "mask "; PrintSrc(os, w); break;
+          case VOP_MOVM: os << "select acc, "; PrintSrc(os, w); break;
+          default: os << "?"; break;
+        }
+        os << "\n";
+      }
+    } else {
+      os << "entry type " << h->entry << " blocks=" << p.grid << " threads=" << p.threads << "\n";
+    }
+  }
+  dump_str_ = os.str();
+  return dump_str_;
+}
+
+std::string &VKernel::Inspect() {
+  std::ostringstream os;
+  if (!g_system.HasDevice()) os << "warning: LaunchNone (" << g_system.LoadError() << ")\n";
+  if (!compiled_) os << "warning: not compiled\n";
+  for (const NDObject *o : ops_) {
+    if ((o->kind == kObjLoad || o->kind == kObjStore) && o->addr == nullptr) {
+      os << "note: %" << o->id << " has no address yet\n";
+    }
+  }
+  dump_str_ = os.str();
+  return dump_str_;
+}
+
+}  // namespace dvm

@@ -1,0 +1,713 @@
+// dvm::Kernel: graph building and the dtype lowering rules.
+//
+// The rules restate the reference's Kernel methods for a target without native
+// bool / bf16 arithmetic (src/dvm.cc:1245-1447, GetBinaryS :586-676, PowS
+// :255-279, NoLossCast :425-443, cast routing table :416-423): they fix the
+// numerics of a graph (where values are rounded, which operations run in
+// fp32), so they are kept operation for operation. int64 tensors, views,
+// gathers and collectives are not implemented by this backend and raise.
+#include <chrono>
+#include <cmath>
+#include <cstring>
+#include <type_traits>
+
+#include "ir.h"
+#include "system.h"
+
+namespace dvm {
+
+// ---- fp16 / bf16 codecs -------------------------------------------------------
+
+uint16_t F32ToF16Bits(float f) {
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  const uint32_t sign = (x >> 16) & 0x8000u;
+  x &= 0x7fffffffu;
+  if (x >= 0x7f800000u) return static_cast<uint16_t>(sign | (x > 0x7f800000u ? 0x7e00u : 0x7c00u));
+  if (x >= 0x477ff000u) return static_cast<uint16_t>(sign | 0x7c00u);  // rounds to infinity
+  if (x < 0x38800000u) {
+    // result is subnormal or zero: let an fp32 add do the round-to-nearest-even
+    float v;
+    std::memcpy(&v, &x, 4);
+    float magic = 0.5f;  // 2^-1: adding it aligns the 10 result bits at the bottom of the mantissa
+    v += magic;
+    uint32_t r;
+    std::memcpy(&r, &v, 4);
+    return static_cast<uint16_t>(sign | (r - 0x3f000000u));
+  }
+  const uint32_t odd = (x >> 13) & 1u;
+  x += 0xc8000fffu + odd;  // rebias the exponent (-112 << 23) and round to nearest even
+  return static_cast<uint16_t>(sign | (x >> 13));
+}
+
+float F16BitsToF32(uint16_t h) {
+  const uint32_t sign = static_cast<uint32_t>(h & 0x8000u) << 16;
+  uint32_t em = h & 0x7fffu;
+  uint32_t out;
+  if (em >= 0x7c00u) {
+    out = sign | 0x7f800000u | ((em & 0x3ffu) << 13);
+  } else if (em >= 0x0400u) {
+    out = sign | ((em << 13) + 0x38000000u);
+  } else if (em == 0) {
+    out = sign;
+  } else {
+    // subnormal: value = em * 2^-24
+    float v = static_cast<float>(em) * 5.9604644775390625e-08f;
+    std::memcpy(&out, &v, 4);
+    out |= sign;
+  }
+  float f;
+  std::memcpy(&f, &out, 4);
+  return f;
+}
+
+uint16_t F32ToBF16Bits(float f) {
+  if (std::isnan(f)) return 0x7fc0u;
+  uint32_t x;
+  std::memcpy(&x, &f, 4);
+  x += 0x7fffu + ((x >> 16) & 1u);
+  return static_cast<uint16_t>(x >> 16);
+}
+
+float BF16BitsToF32(uint16_t h) {
+  uint32_t x = static_cast<uint32_t>(h) << 16;
+  float f;
+  std::memcpy(&f, &x, 4);
+  return f;
+}
+
+Float16::Float16(float v) : value_(F32ToF16Bits(v)) {}
+Float16::Float16(int32_t v) : value_(F32ToF16Bits(static_cast<float>(v))) {}
+Float16::operator float() const { return F16BitsToF32(value_); }
+Float16::operator int32_t() const { return static_cast<int32_t>(F16BitsToF32(value_)); }
+BFloat16::BFloat16(float v) : value_(F32ToBF16Bits(v)) {}
+BFloat16::BFloat16(int32_t v) : value_(F32ToBF16Bits(static_cast<float>(v))) {}
+BFloat16::operator float() const { return BF16BitsToF32(value_); }
+BFloat16::operator int32_t() const { return static_cast<int32_t>(BF16BitsToF32(value_)); }
+
+namespace {
+
+float ScalarAsFloat(const ScalarRef &s) {
+  switch (s.type) {
+    case kFloat32: return s.f32;
+    case kInt32: return static_cast<float>(s.i32);
+    case kInt64: return static_cast<float>(s.i64);
+    case kFloat16: return F16BitsToF32(s.f16);
+    case kBFloat16: return BF16BitsToF32(s.f16);
+    default: return 0.0f;
+  }
+}
+
+uint32_t FloatBits(float f) {
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  return u;
+}
+
+}  // namespace
+
+uint32_t ScalarToContainer(const ScalarRef &s, DataType t) {
+  switch (t) {
+    case kFloat16: {
+      if (s.type == kFloat16) return FloatBits(F16BitsToF32(s.f16));
+      return FloatBits(F16BitsToF32(F32ToF16Bits(ScalarAsFloat(s))));
+    }
+    case kBFloat16: {
+      if (s.type == kBFloat16) return FloatBits(BF16BitsToF32(s.f16));
+      return FloatBits(BF16BitsToF32(F32ToBF16Bits(ScalarAsFloat(s))));
+    }
+    case kFloat32:
+      return FloatBits(ScalarAsFloat(s));
+    case kInt32: {
+      int32_t v;
+      if (s.type == kInt32) {
+        v = s.i32;
+      } else if (s.type == kInt64) {
+        v = static_cast<int32_t>(s.i64);
+      } else {
+        v = static_cast<int32_t>(ScalarAsFloat(s));
+      }
+      return static_cast<uint32_t>(v);
+    }
+    case kBool:
+      return FloatBits(ScalarAsFloat(s) != 0.0f ? 1.0f : 0.0f);
+    default:
+      Throw("scalar for an unsupported tensor type");
+  }
+}
+
+// ---- Comm (single GPU: nothing to connect) ------------------------------------------
+
+Comm::~Comm() {}
+bool Comm::Init(int /*rank_id*/, int rank_size, int /*comm_type*/, const uint32_t * /*group_ranks*/) {
+  return rank_size == 1;
+}
+void Comm::Init(void * /*hccl_comm*/) {}
+
+// ---- Kernel ------------------------------------------------------------------------
+
+namespace {
+
+[[noreturn]] void Unsupported(const char *what) {
+  Throw(std::string(what) + " is not supported by the gfx950 backend");
+}
+
+struct Operand {
+  NDObject *obj = nullptr;
+  ScalarOperand sc;
+  bool IsObj() const { return obj != nullptr; }
+};
+
+template <typename T>
+Operand MakeOperand(T v) {
+  Operand o;
+  if constexpr (std::is_same<T, NDObject *>::value) {
+    o.obj = v;
+  } else if constexpr (std::is_same<T, ScalarRef *>::value) {
+    o.sc.ref = v;
+  } else {
+    o.sc.imm = v;
+  }
+  return o;
+}
+
+bool IsCompare(int op) { return op <= kLessEqual; }
+
+// Intermediate type of one conversion step from `from` towards `to` (row = from, column = to).
+const DataType kCastRoute[kDataTypeEnd][kDataTypeEnd] = {
+    /* bool  */ {kBool, kFloat16, kFloat16, kFloat16, kFloat16, kFloat16},
+    /* f16   */ {kBool, kFloat16, kFloat32, kFloat32, kInt32, kFloat32},
+    /* bf16  */ {kFloat32, kFloat32, kBFloat16, kFloat32, kInt32, kFloat32},
+    /* f32   */ {kFloat16, kFloat16, kBFloat16, kFloat32, kInt32, kInt64},
+    /* i32   */ {kFloat16, kFloat16, kFloat32, kFloat32, kInt32, kInt64},
+    /* i64   */ {kBool, kFloat32, kFloat32, kFloat32, kInt32, kInt64},
+};
+
+class Builder {
+ public:
+  explicit Builder(VKernel *k) : k_(k) {}
+
+  NDObject *New(ObjKind kind, DataType t, NDObject *a = nullptr, NDObject *b = nullptr, NDObject *c = nullptr) {
+    NDObject *o = new NDObject(kind, t);
+    o->in[0] = a;
+    o->in[1] = b;
+    o->in[2] = c;
+    o->nin = c != nullptr ? 3 : (b != nullptr ? 2 : (a != nullptr ? 1 : 0));
+    return k_->Append(o);
+  }
+
+  NDObject *CastStep(NDObject *x, DataType t, bool noloss) {
+    NDObject *o = New(kObjCast, t, x);
+    o->noloss_cast = noloss;
+    return o;
+  }
+
+  // Conversion that cannot lose information on the values it is used for
+  // (bool <-> arithmetic types); a cast back over such a cast is elided.
+  NDObject *NoLossCast(NDObject *x, DataType t) {
+    DataType cur = x->type_id_;
+    while (cur != t) {
+      const DataType step = kCastRoute[cur][t];
+      if (x->kind == kObjCast && x->noloss_cast && x->in[0]->type_id_ == step) {
+        x = x->in[0];
+      } else {
+        x = CastStep(x, step, true);
+      }
+      cur = step;
+    }
+    return x;
+  }
+
+  static bool IsBoolResult(const NDObject *x) {
+    if (x->kind == kObjCompare || x->kind == kObjCompareS) return true;
+    if (x->kind == kObjBinary) return x->op == kLogicalAnd || x->op == kLogicalOr;
+    return false;
+  }
+
+  NDObject *Cast(NDObject *x, DataType t) {
+    if (x->type_id_ == t) return x;
+    if (t == kInt64 || x->type_id_ == kInt64) Unsupported("int64 tensors");
+    if (t == kBool && !IsBoolResult(x)) {
+      ScalarOperand zero;
+      zero.imm = 0;
+      x = ScalarBinary(kNotEqual, zero, x, true);
+    }
+    DataType cur = x->type_id_;
+    while (cur != t) {
+      const DataType step = kCastRoute[cur][t];
+      x = CastStep(x, step, false);
+      cur = step;
+    }
+    return x;
+  }
+
+  NDObject *BroadcastScalar(const ScalarOperand &s, IntArrayRef *shape, DataType t) {
+    if (t == kBool) return Cast(BroadcastScalar(s, shape, kFloat16), kBool);
+    if (t == kInt64) Unsupported("int64 tensors");
+    NDObject *o = New(kObjBroadcastS, t);
+    o->scalar = s;
+    o->aux_ref = shape;
+    return o;
+  }
+
+  NDObject *Unary(int op, NDObject *x) {
+    switch (x->type_id_) {
+      case kBool: {
+        NDObject *r = Unary(op, NoLossCast(x, kFloat16));
+        return NoLossCast(r, kBool);
+      }
+      case kBFloat16:
+        return Cast(Unary(op, Cast(x, kFloat32)), kBFloat16);
+      case kFloat16:
+        if (op >= kRound && op <= kTrunc) return Cast(Unary(op, Cast(x, kFloat32)), kFloat16);
+        break;
+      case kInt64:
+        Unsupported("int64 tensors");
+      default:
+        break;
+    }
+    if (op == kLogicalNot) {
+      ScalarOperand one;
+      one.imm = 1;
+      return ScalarBinaryOrFallback(kSub, one, x, false);
+    }
+    if (op == kReciprocal) {
+      ScalarOperand one;
+      one.imm = 1;
+      return ScalarBinaryOrFallback(kDiv, one, x, false);
+    }
+    if (x->type_id_ == kInt32 && op != kAbs) Throw("unary operator without an int32 form");
+    NDObject *o = New(kObjUnary, x->type_id_, x);
+    o->op = static_cast<uint8_t>(op);
+    return o;
+  }
+
+  NDObject *TensorBinary(int op, NDObject *l, NDObject *r) {
+    switch (l->type_id_) {
+      case kBool: {
+        NDObject *res = TensorBinary(op, NoLossCast(l, kFloat16), NoLossCast(r, kFloat16));
+        return NoLossCast(res, kBool);
+      }
+      case kBFloat16:
+        if (op == kPow || op == kDiv) {
+          return Cast(TensorBinary(op, Cast(l, kFloat32), Cast(r, kFloat32)), kBFloat16);
+        }
+        break;
+      case kFloat16:
+        if (op == kPow) return Cast(TensorBinary(op, Cast(l, kFloat32), Cast(r, kFloat32)), kFloat16);
+        break;
+      case kInt64:
+        Unsupported("int64 tensors");
+      default:
+        break;
+    }
+    if (IsCompare(op)) {
+      NDObject *o = New(kObjCompare, l->type_id_, l, r);
+      o->op = static_cast<uint8_t>(op);
+      return NoLossCast(o, kBool);
+    }
+    if (l->type_id_ == kInt32 && (op == kDiv || op == kPow)) Throw("binary operator without an int32 form");
+    NDObject *o = New(kObjBinary, l->type_id_, l, r);
+    o->op = static_cast<uint8_t>(op);
+    return o;
+  }
+
+  NDObject *NewBinaryS(int op, NDObject *x, const ScalarOperand &s, bool scalar_left) {
+    NDObject *o = New(kObjBinaryS, x->type_id_, x);
+    o->op = static_cast<uint8_t>(op);
+    o->scalar = s;
+    o->scalar_left = scalar_left;
+    return o;
+  }
+
+  // x ^ n for an integer n by repeated squaring.
+  NDObject *PowInt(NDObject *x, const ScalarOperand &s, int32_t n) {
+    uint32_t it = n < 0 ? 0u - static_cast<uint32_t>(n) : static_cast<uint32_t>(n);
+    if (it == 0) {
+      ScalarOperand one;
+      one.imm = s.imm.type == kInt32 ? ScalarRef(1) : ScalarRef(1.0f);
+      return BroadcastScalar(one, x->shape_ref_, x->type_id_);
+    }
+    NDObject *res = nullptr;
+    if (it == 1) {
+      res = New(kObjCopy, x->type_id_, x);
+    } else {
+      while (it != 0) {
+        if (it & 1u) res = res == nullptr ? x : TensorBinary(kMul, res, x);
+        if (it != 1) x = TensorBinary(kMul, x, x);
+        it >>= 1;
+      }
+    }
+    if (n < 0) res = Unary(kReciprocal, res);
+    return res;
+  }
+
+  // Tensor (op) scalar when the operation has a scalar form; null otherwise.
+  // rhs_val: the scalar is the right operand.
+  NDObject *ScalarBinary(int op, const ScalarOperand &s, NDObject *x, bool rhs_val) {
+    if (x->type_id_ == kInt64) Unsupported("int64 tensors");
+    const bool is_ref = s.ref != nullptr;
+    switch (op) {
+      case kAdd:
+      case kMul:
+      case kMinimum:
+      case kMaximum:
+        return NewBinaryS(op, x, s, false);
+      case kDiv: {
+        if (x->type_id_ == kBFloat16) return Cast(ScalarBinary(op, s, Cast(x, kFloat32), rhs_val), kBFloat16);
+        if (x->type_id_ == kInt32) Throw("binary operator without an int32 form");
+        return NewBinaryS(op, x, s, !rhs_val);
+      }
+      case kEqual:
+      case kNotEqual:
+      case kGreater:
+      case kGreaterEqual:
+      case kLess:
+      case kLessEqual: {
+        NDObject *o = New(kObjCompareS, x->type_id_, x);
+        o->op = static_cast<uint8_t>(op);
+        o->scalar = s;
+        o->scalar_left = !rhs_val;
+        return NoLossCast(o, kBool);
+      }
+      case kPow: {
+        if (is_ref) return nullptr;
+        const float v = ScalarAsFloat(s.imm);
+        if (rhs_val) {
+          const bool integral = s.imm.type == kInt32 || std::floor(v) == v;
+          if (integral && std::fabs(v) < 2147483648.0f) return PowInt(x, s, static_cast<int32_t>(v));
+          return nullptr;
+        }
+        if (v > 0.0f) {
+          if (x->type_id_ != kFloat32) {
+            ScalarOperand f;
+            f.imm = v;
+            const DataType orig = x->type_id_;
+            return Cast(ScalarBinary(kPow, f, Cast(x, kFloat32), false), orig);
+          }
+          ScalarOperand lg;
+          lg.imm = std::log(v);
+          return Unary(kExp, NewBinaryS(kMul, x, lg, false));
+        }
+        return nullptr;
+      }
+      case kSub: {
+        if (is_ref) return nullptr;
+        ScalarOperand neg = s;
+        if (rhs_val) {
+          switch (neg.imm.type) {
+            case kFloat32: neg.imm.f32 = -neg.imm.f32; break;
+            case kInt32: neg.imm.i32 = static_cast<int32_t>(0u - static_cast<uint32_t>(neg.imm.i32)); break;
+            case kInt64: neg.imm.i64 = -neg.imm.i64; break;
+            default: neg.imm.f16 ^= 0x8000u; break;
+          }
+          return NewBinaryS(kAdd, x, neg, false);
+        }
+        ScalarOperand m1;
+        switch (s.imm.type) {
+          case kInt32: m1.imm = -1; break;
+          case kInt64: m1.imm = static_cast<int64_t>(-1); break;
+          case kFloat16: m1.imm = Float16(-1.0f); break;
+          case kBFloat16: m1.imm = BFloat16(-1.0f); break;
+          default: m1.imm = -1.0f; break;
+        }
+        return NewBinaryS(kAdd, NewBinaryS(kMul, x, m1, false), s, false);
+      }
+      default:
+        return nullptr;
+    }
+  }
+
+  NDObject *ScalarBinaryOrFallback(int op, const ScalarOperand &s, NDObject *x, bool rhs_val) {
+    if (x->type_id_ == kBool) {
+      NDObject *r = ScalarBinaryOrFallback(op, s, NoLossCast(x, kFloat16), rhs_val);
+      return NoLossCast(r, kBool);
+    }
+    NDObject *o = ScalarBinary(op, s, x, rhs_val);
+    if (o != nullptr) return o;
+    NDObject *b = BroadcastScalar(s, x->shape_ref_, x->type_id_);
+    return rhs_val ? TensorBinary(op, x, b) : TensorBinary(op, b, x);
+  }
+
+  NDObject *Binary(int op, const Operand &l, const Operand &r) {
+    if (l.IsObj() && r.IsObj()) return TensorBinary(op, l.obj, r.obj);
+    if (l.IsObj()) return ScalarBinaryOrFallback(op, r.sc, l.obj, true);
+    if (r.IsObj()) return ScalarBinaryOrFallback(op, l.sc, r.obj, false);
+    Throw("binary operator needs at least one tensor operand");
+  }
+
+ private:
+  VKernel *k_;
+};
+
+}  // namespace
+
+Kernel::Kernel() : kernel_(nullptr) {}
+Kernel::~Kernel() { delete kernel_; }
+Kernel &Kernel::operator=(Kernel &other) {
+  if (this != &other) {
+    delete kernel_;
+    kernel_ = other.kernel_;
+    other.kernel_ = nullptr;
+  }
+  return *this;
+}
+Kernel::Kernel(Kernel &other) : kernel_(other.kernel_) { other.kernel_ = nullptr; }
+
+void Kernel::Reset(KernelType type, uint32_t flags) {
+  g_system.Init();
+  delete kernel_;
+  switch (type) {
+    case kVector:
+    case kCube:
+    case kMix:
+    case kSplit:
+      break;
+    default:
+      kernel_ = nullptr;
+      Unsupported("this kernel type");
+  }
+  kernel_ = new VKernel(type, flags);
+}
+
+void Kernel::Clone(const Kernel &base, CloneHelper &helper) {
+  VKernel *src = base.GetImpl();
+  delete kernel_;
+  kernel_ = new VKernel(src->KType(), src->Flags());
+  for (NDObject *o : src->ops_) {
+    NDObject *c = new NDObject(o->kind, o->type_id_);
+    c->op = o->op;
+    c->scalar_left = o->scalar_left;
+    c->keepdims = o->keepdims;
+    c->trans_a = o->trans_a;
+    c->trans_b = o->trans_b;
+    c->inplace = o->inplace;
+    c->noloss_cast = o->noloss_cast;
+    c->nin = o->nin;
+    for (int i = 0; i < o->nin; ++i) c->in[i] = helper.GetClone(o->in[i]);
+    c->scalar.imm = o->scalar.imm;
+    c->scalar.ref = o->scalar.ref != nullptr ? helper.GetClone(o->scalar.ref) : nullptr;
+    c->aux_ref = o->aux_ref != nullptr ? helper.GetClone(o->aux_ref) : nullptr;
+    c->addr = o->addr;
+    if (o->kind == kObjLoad) c->shape_ref_ = c->aux_ref;
+    kernel_->Append(c);
+    helper.SetClone(o, c);
+  }
+}
+
+void Kernel::SetNameHint(const char *name, const char *fullname) {
+  kernel_->name_ = name != nullptr ? name : "";
+  kernel_->fullname_ = fullname != nullptr ? fullname : "";
+}
+
+NDObject *Kernel::Load(void *addr, IntArrayRef *shape, DataType type) {
+  if (type == kInt64) Unsupported("int64 tensors");
+  NDObject *o = new NDObject(kObjLoad, type);
+  o->addr = addr;
+  o->aux_ref = shape;
+  o->shape_ref_ = shape;
+  return kernel_->Append(o);
+}
+
+NDObject *Kernel::Load(void *addr, IntArrayRef *shape, IntArrayRef *stride, DataType type) {
+  if (stride != nullptr) Unsupported("a strided load");
+  return Load(addr, shape, type);
+}
+
+NDObject *Kernel::GlobalAccess(void *, IntArrayRef *, DataType) { Unsupported("GlobalAccess"); }
+NDObject *Kernel::GatherLoad(void *, IntArrayRef *, NDObject *, int, DataType, GatherMode) { Unsupported("GatherLoad"); }
+NDObject *Kernel::SliceLoad(void *, IntArrayRef *, IntArrayRef *, IntArrayRef *, DataType) { Unsupported("SliceLoad"); }
+NDObject *Kernel::StridedSliceLoad(void *, IntArrayRef *, IntArrayRef *, IntArrayRef *, IntArrayRef *, DataType) {
+  Unsupported("StridedSliceLoad");
+}
+NDObject *Kernel::MultiLoad(void *, IntArrayRef *, DataType, const Comm *) { Unsupported("MultiLoad"); }
+
+NDObject *Kernel::Store(void *addr, NDObject *input) {
+  Builder b(kernel_);
+  if (input->IsLoad()) input = b.New(kObjCopy, input->type_id_, input);
+  NDObject *o = b.New(kObjStore, input->type_id_, input);
+  o->addr = addr;
+  return o;
+}
+
+NDObject *Kernel::Store(void *addr, NDObject *input, IntArrayRef *stride) {
+  if (stride != nullptr) Unsupported("a strided store");
+  return Store(addr, input);
+}
+
+NDObject *Kernel::PadStore(void *, NDObject *, int64_t) { Unsupported("PadStore"); }
+void Kernel::SetStoreInplace(NDObject *store) { store->inplace = true; }
+void Kernel::SetStoreTemp(NDObject *) { Unsupported("SetStoreTemp"); }
+void Kernel::SetLoadBind(NDObject *, NDObject *) { Unsupported("SetLoadBind"); }
+
+NDObject *Kernel::_Unary(int op_type, NDObject *input) {
+  if (op_type < 0 || op_type >= kUnaryTypeEnd) return nullptr;
+  return Builder(kernel_).Unary(op_type, input);
+}
+
+template <UnaryType op_type>
+NDObject *Kernel::Unary(NDObject *input) {
+  return _Unary(op_type, input);
+}
+
+template <typename L, typename R>
+NDObject *Kernel::_Binary(int op_type, L lhs, R rhs) {
+  if (op_type < 0 || op_type >= kBinaryTypeEnd) return nullptr;
+  return Builder(kernel_).Binary(op_type, MakeOperand(lhs), MakeOperand(rhs));
+}
+
+template <BinaryType op_type, typename L, typename R>
+NDObject *Kernel::Binary(L lhs, R rhs) {
+  return _Binary<L, R>(op_type, lhs, rhs);
+}
+
+#define DVM_INST_UNARY(op) template NDObject *Kernel::Unary<op>(NDObject *);
+DVM_INST_UNARY(kSqrt) DVM_INST_UNARY(kAbs) DVM_INST_UNARY(kLog) DVM_INST_UNARY(kExp) DVM_INST_UNARY(kReciprocal)
+DVM_INST_UNARY(kIsFinite) DVM_INST_UNARY(kLogicalNot) DVM_INST_UNARY(kRound) DVM_INST_UNARY(kFloor)
+DVM_INST_UNARY(kCeil) DVM_INST_UNARY(kTrunc)
+#undef DVM_INST_UNARY
+
+#define DVM_INST_BINARY_T(L, R) template NDObject *Kernel::_Binary<L, R>(int, L, R);
+DVM_INST_BINARY_T(NDObject *, NDObject *)
+DVM_INST_BINARY_T(NDObject *, float) DVM_INST_BINARY_T(NDObject *, int32_t) DVM_INST_BINARY_T(NDObject *, int64_t)
+DVM_INST_BINARY_T(NDObject *, Float16) DVM_INST_BINARY_T(NDObject *, BFloat16) DVM_INST_BINARY_T(NDObject *, ScalarRef *)
+DVM_INST_BINARY_T(float, NDObject *) DVM_INST_BINARY_T(int32_t, NDObject *) DVM_INST_BINARY_T(int64_t, NDObject *)
+DVM_INST_BINARY_T(Float16, NDObject *) DVM_INST_BINARY_T(BFloat16, NDObject *) DVM_INST_BINARY_T(ScalarRef *, NDObject *)
+#undef DVM_INST_BINARY_T
+
+#define DVM_INST_BINARY(op)                                              \
+  template NDObject *Kernel::Binary<op>(NDObject *, NDObject *);         \
+  template NDObject *Kernel::Binary<op>(NDObject *, float);              \
+  template NDObject *Kernel::Binary<op>(NDObject *, int32_t);            \
+  template NDObject *Kernel::Binary<op>(NDObject *, int64_t);            \
+  template NDObject *Kernel::Binary<op>(NDObject *, Float16);            \
+  template NDObject *Kernel::Binary<op>(NDObject *, BFloat16);           \
+  template NDObject *Kernel::Binary<op>(NDObject *, ScalarRef *);        \
+  template NDObject *Kernel::Binary<op>(float, NDObject *);              \
+  template NDObject *Kernel::Binary<op>(int32_t, NDObject *);            \
+  template NDObject *Kernel::Binary<op>(int64_t, NDObject *);            \
+  template NDObject *Kernel::Binary<op>(Float16, NDObject *);            \
+  template NDObject *Kernel::Binary<op>(BFloat16, NDObject *);           \
+  template NDObject *Kernel::Binary<op>(ScalarRef *, NDObject *);
+DVM_INST_BINARY(kEqual) DVM_INST_BINARY(kNotEqual) DVM_INST_BINARY(kGreater) DVM_INST_BINARY(kGreaterEqual)
+DVM_INST_BINARY(kLess) DVM_INST_BINARY(kLessEqual) DVM_INST_BINARY(kAdd) DVM_INST_BINARY(kSub) DVM_INST_BINARY(kMul)
+DVM_INST_BINARY(kDiv) DVM_INST_BINARY(kPow) DVM_INST_BINARY(kMaximum) DVM_INST_BINARY(kMinimum)
+DVM_INST_BINARY(kLogicalAnd) DVM_INST_BINARY(kLogicalOr)
+#undef DVM_INST_BINARY
+
+NDObject *Kernel::_Reduce(int op_type, NDObject *input, IntArrayRef *dims, bool keepdims) {
+  if (op_type == kSum && input->type_id_ != kFloat32) return nullptr;  // callers cast to fp32 first
+  if (input->type_id_ == kInt64 || input->type_id_ == kBool) Throw("reduce over an unsupported tensor type");
+  NDObject *o = Builder(kernel_).New(kObjReduce, input->type_id_, input);
+  o->op = static_cast<uint8_t>(op_type);
+  o->aux_ref = dims;
+  o->keepdims = keepdims;
+  return o;
+}
+
+NDObject *Kernel::Select(NDObject *cond, NDObject *lhs, NDObject *rhs) {
+  Builder b(kernel_);
+  if (lhs->type_id_ == kInt64) Unsupported("int64 tensors");
+  if (cond->type_id_ != lhs->type_id_) cond = b.NoLossCast(cond, lhs->type_id_);
+  return b.New(kObjSelect, lhs->type_id_, cond, lhs, rhs);
+}
+
+NDObject *Kernel::Cast(NDObject *input, DataType type) { return Builder(kernel_).Cast(input, type); }
+
+NDObject *Kernel::Broadcast(NDObject *input, IntArrayRef *shape) {
+  Builder b(kernel_);
+  if (input->type_id_ == kBool) {
+    NDObject *r = Broadcast(b.NoLossCast(input, kFloat16), shape);
+    return b.NoLossCast(r, kBool);
+  }
+  NDObject *o = b.New(kObjBroadcast, input->type_id_, input);
+  o->aux_ref = shape;
+  return o;
+}
+
+template <typename T>
+NDObject *Kernel::Broadcast(T val, IntArrayRef *shape, DataType type) {
+  return Builder(kernel_).BroadcastScalar(MakeOperand(val).sc, shape, type);
+}
+template NDObject *Kernel::Broadcast<float>(float, IntArrayRef *, DataType);
+template NDObject *Kernel::Broadcast<int32_t>(int32_t, IntArrayRef *, DataType);
+template NDObject *Kernel::Broadcast<int64_t>(int64_t, IntArrayRef *, DataType);
+template NDObject *Kernel::Broadcast<Float16>(Float16, IntArrayRef *, DataType);
+template NDObject *Kernel::Broadcast<BFloat16>(BFloat16, IntArrayRef *, DataType);
+template NDObject *Kernel::Broadcast<ScalarRef *>(ScalarRef *, IntArrayRef *, DataType);
+
+NDObject *Kernel::Reshape(NDObject *input, IntArrayRef *shape) {
+  NDObject *o = Builder(kernel_).New(kObjReshape, input->type_id_, input);
+  o->aux_ref = shape;
+  return o;
+}
+
+NDObject *Kernel::Copy(NDObject *input) { return Builder(kernel_).New(kObjCopy, input->type_id_, input); }
+
+NDObject *Kernel::MatMul(NDObject *lhs, NDObject *rhs, bool trans_a, bool trans_b, NDObject *bias) {
+  if (lhs->type_id_ != rhs->type_id_ || (lhs->type_id_ != kFloat16 && lhs->type_id_ != kBFloat16)) {
+    Throw("matmul needs two fp16 or two bf16 operands");
+  }
+  NDObject *o = Builder(kernel_).New(kObjMatMul, lhs->type_id_, lhs, rhs, bias);
+  o->trans_a = trans_a;
+  o->trans_b = trans_b;
+  return o;
+}
+
+NDObject *Kernel::Permute(NDObject *, IntArrayRef *) { Unsupported("Permute"); }
+NDObject *Kernel::Slice(NDObject *, IntArrayRef *, IntArrayRef *) { Unsupported("Slice"); }
+NDObject *Kernel::Slice(NDObject *, int, ScalarRef *, ScalarRef *) { Unsupported("Slice"); }
+NDObject *Kernel::Concat(NDObject **, size_t, int) { Unsupported("Concat"); }
+NDObject **Kernel::Split(NDObject *, int, int64_t, size_t) { Unsupported("Split"); }
+template <typename T>
+NDObject *Kernel::OneHot(NDObject *, IntArrayRef *, int, T, T) {
+  Unsupported("OneHot");
+}
+template NDObject *Kernel::OneHot<float>(NDObject *, IntArrayRef *, int, float, float);
+template NDObject *Kernel::OneHot<int32_t>(NDObject *, IntArrayRef *, int, int32_t, int32_t);
+template NDObject *Kernel::OneHot<Float16>(NDObject *, IntArrayRef *, int, Float16, Float16);
+template NDObject *Kernel::OneHot<BFloat16>(NDObject *, IntArrayRef *, int, BFloat16, BFloat16);
+NDObject *Kernel::ElemAny(NDObject *) { Unsupported("ElemAny"); }
+NDObject *Kernel::GroupedMatMul(NDObject *, NDObject *, bool, bool, NDObject *, NDObject *, GmmSplitType, GmmListType) {
+  Unsupported("GroupedMatMul");
+}
+NDObject *Kernel::_AllReduce(int, NDObject *, const Comm *) { Unsupported("AllReduce (single-GPU backend)"); }
+NDObject *Kernel::AllGather(NDObject *, const Comm *) { Unsupported("AllGather (single-GPU backend)"); }
+NDObject *Kernel::AllGatherV2(NDObject *, const Comm *) { Unsupported("AllGatherV2 (single-GPU backend)"); }
+NDObject *Kernel::ReduceScatter(NDObject *, const Comm *) { Unsupported("ReduceScatter (single-GPU backend)"); }
+NDObject *Kernel::ExtOut(NDObject *, int) { Unsupported("ExtOut"); }
+void Kernel::SpecNext() { Unsupported("speculative kernels"); }
+void Kernel::ParallelAdd(KernelType, uint32_t, size_t) { Unsupported("parallel kernels"); }
+void Kernel::SequenceAdd(KernelType, uint32_t) { Unsupported("sequence kernels"); }
+void Kernel::Clear() {}
+
+void Kernel::Normalize() { kernel_->Normalize(); }
+
+size_t Kernel::PreCodeGen() {
+  kernel_->Normalize();
+  return kernel_->CodeGen(true);
+}
+
+void Kernel::CodeGen(const RelocEntry *relocs, size_t reloc_size, WsAllocator *ws_alloc) {
+  const auto t0 = std::chrono::steady_clock::now();
+  kernel_->CodeGen(false);
+  kernel_->BindAddresses(relocs, reloc_size, ws_alloc, nullptr);
+  kernel_->last_codegen_us_ =
+      std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count();
+}
+
+int Kernel::Launch(void *stream) { return kernel_->Launch(stream); }
+
+int Kernel::Launch(const RelocEntry *relocs, size_t reloc_size, void *workspace, void *stream) {
+  kernel_->BindAddresses(relocs, reloc_size, nullptr, workspace);
+  return kernel_->Launch(stream);
+}
+
+IntArrayRef *Kernel::GetShape(NDObject *op) { return op->shape_ref_; }
+DataType Kernel::GetDType(NDObject *op) { return op->type_id_; }
+const char *Kernel::Dump() const { return kernel_->DumpGraph(false).c_str(); }
+const char *Kernel::DumpR() const { return kernel_->DumpGraph(true).c_str(); }
+const char *Kernel::Das() const { return kernel_->DisAssemble().c_str(); }
+const char *Kernel::Inspect() const { return kernel_->Inspect().c_str(); }
+
+}  // namespace dvm

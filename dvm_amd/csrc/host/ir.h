@@ -1,0 +1,181 @@
+// Host-side IR of the gfx950 backend: operator nodes, the kernel object behind
+// dvm::Kernel, and the compiled sub-kernel programs.
+//
+// Role in the reference: NDObject hierarchy (src/ops.h:444-554), VKernel and
+// its subclasses (src/kernel.h:52-104, src/xkernel.h), Code (src/code.h:90-286).
+// Here one node class covers every operator kind and one kernel class covers
+// the vector / split / mix kernel types; the graph is cut into sub-kernels by
+// fusability on the gfx950 VM, not by the reference's local-memory tile model.
+#ifndef DVM_AMD_HOST_IR_H_
+#define DVM_AMD_HOST_IR_H_
+
+#include <cstdint>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "../../../include/dvm.h"
+#include "../isa_gfx950.h"
+
+namespace dvm {
+
+constexpr int kMaxRank = 10;  // same limit as the reference (src/ops.h:165)
+
+enum ObjKind : uint8_t {
+  kObjLoad = 0,
+  kObjStore,
+  kObjUnary,
+  kObjBinary,
+  kObjBinaryS,   // tensor (op) scalar
+  kObjCompare,
+  kObjCompareS,  // tensor (cmp) scalar
+  kObjSelect,
+  kObjCast,
+  kObjBroadcast,
+  kObjBroadcastS,  // scalar fill
+  kObjReduce,
+  kObjReshape,
+  kObjCopy,
+  kObjMatMul,
+};
+
+// A scalar operand: an immediate fixed at build time or a ScalarRef re-read at every code generation.
+struct ScalarOperand {
+  ScalarRef imm;
+  ScalarRef *ref = nullptr;
+  const ScalarRef &Get() const { return ref != nullptr ? *ref : imm; }
+};
+
+class NDObject {
+ public:
+  NDObject(ObjKind k, DataType t) : kind(k), type_id_(t) {
+    own_ref_.data = shape_;
+    own_ref_.size = 0;
+    shape_ref_ = &own_ref_;
+  }
+  ObjKind kind;
+  DataType type_id_;
+  uint8_t op = 0;          // UnaryType / BinaryType / ReduceType
+  bool scalar_left = false;  // kObjBinaryS / kObjCompareS: scalar is the left operand
+  bool keepdims = false;
+  bool trans_a = false, trans_b = false;
+  bool inplace = false;
+  bool noloss_cast = false;
+  int nin = 0;
+  NDObject *in[3] = {nullptr, nullptr, nullptr};
+  ScalarOperand scalar;
+  IntArrayRef *aux_ref = nullptr;  // reduce axes / broadcast target / reshape target / user shape of a load
+  void *addr = nullptr;            // load / store address (may arrive later through a RelocEntry)
+  int id = -1;                     // position in the kernel's operator list
+
+  // Shape as the API sees it, outermost first. Loads point at the caller's
+  // IntArrayRef (dynamic shapes), every other node at its own storage.
+  IntArrayRef *shape_ref_;
+  IntArrayRef own_ref_;
+  int64_t shape_[kMaxRank];
+
+  int rank() const { return static_cast<int>(shape_ref_->size); }
+  int64_t dim(int i) const { return shape_ref_->data[i]; }
+  int64_t numel() const {
+    int64_t n = 1;
+    for (size_t i = 0; i < shape_ref_->size; ++i) n *= shape_ref_->data[i];
+    return n;
+  }
+  void SetShape(const int64_t *d, size_t n) {
+    std::memcpy(shape_, d, sizeof(int64_t) * n);
+    own_ref_.size = n;
+  }
+  bool IsLoad() const { return kind == kObjLoad; }
+};
+
+inline size_t DTypeSize(DataType t) {
+  switch (t) {
+    case kBool: return 1;
+    case kFloat16:
+    case kBFloat16: return 2;
+    case kInt64: return 8;
+    default: return 4;
+  }
+}
+
+// One launch of the device VM.
+struct Program {
+  VmParam blob;
+  uint32_t grid = 0;
+  uint32_t threads = 0;
+  uint32_t lds_bytes = 0;
+  bool skip = false;       // nothing to do (an extent is zero)
+  // addresses inside the blob that depend on relocation: (word offset, op) pairs
+  struct Patch {
+    uint32_t word;
+    int op_id;       // load/store node whose address goes there, or -1
+    int ws_slot;     // or the workspace slot
+  };
+  std::vector<Patch> patches;
+  // pre-launch fills (zero-size reduce identities, clean kernels)
+  struct Fill {
+    int op_id;
+    int ws_slot;
+    uint32_t value;
+    size_t bytes;
+  };
+  std::vector<Fill> fills;
+};
+
+// Host fp16 / bf16 codecs (same results as the reference's, src/dvm.cc:78-186).
+uint16_t F32ToF16Bits(float f);
+float F16BitsToF32(uint16_t h);
+uint16_t F32ToBF16Bits(float f);
+float BF16BitsToF32(uint16_t h);
+
+// Value of a scalar operand as the 32-bit register pattern of a tensor of
+// type `t`: the value is first converted to `t` exactly like the reference's
+// EncodeScalar (src/dvm.cc:186-223), then widened to the VM's container
+// (fp32 bits for bool/f16/bf16/f32 tensors, two's complement for int32).
+uint32_t ScalarToContainer(const ScalarRef &s, DataType t);
+
+struct DeviceApi;  // bound C ABI of libdvm_hip.so (system.cc)
+
+class VKernel {
+ public:
+  VKernel(KernelType t, uint32_t f) : ktype_(t), flags_(f) {}
+  ~VKernel();
+
+  KernelType KType() const { return ktype_; }
+  uint32_t Flags() const { return flags_; }
+  bool IsDynamic() const { return (flags_ & kDynamic) != 0; }
+
+  NDObject *Append(NDObject *op);
+  void Normalize();
+  // Compiles every sub-kernel. With `pre` set no addresses are needed yet; returns the workspace size.
+  size_t CodeGen(bool pre);
+  void BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *alloc, void *workspace);
+  int Launch(void *stream);
+
+  std::string &DumpGraph(bool ref_shapes);
+  std::string &DisAssemble();
+  std::string &Inspect();
+
+  std::vector<NDObject *> ops_;
+  std::vector<Program> programs_;
+  size_t ws_bytes_ = 0;
+  std::vector<size_t> ws_offsets_;  // per workspace slot
+  std::vector<size_t> ws_sizes_;
+  void *ws_base_ = nullptr;
+  std::string name_, fullname_;
+  double last_codegen_us_ = 0.0;  // wall time of the last Normalize+CodeGen, for JIT latency reports
+
+ private:
+  KernelType ktype_;
+  uint32_t flags_;
+  bool normalized_ = false;
+  bool compiled_ = false;
+  std::string dump_str_;
+  friend class Compiler;
+};
+
+[[noreturn]] void Throw(const std::string &msg);
+
+}  // namespace dvm
+
+#endif  // DVM_AMD_HOST_IR_H_

@@ -1,0 +1,164 @@
+// Tile bytecode for the gfx950 device VM. Shared by the host emitter and the
+// HIP interpreter kernels, so it is plain C structs and enums only.
+//
+// This plays the role the reference's src/isa.h plays for its targets
+// (instruction ids src/isa.h:59-228, entry word src/isa.h:2388-2448), but the
+// unit of interpretation is different: values live in per-lane registers, an
+// instruction works on E consecutive elements per lane, and operands are
+// addressed through stride descriptors instead of tile buffers in local
+// memory.
+#ifndef DVM_ISA_GFX950_H_
+#define DVM_ISA_GFX950_H_
+
+#include <stdint.h>
+
+#define DVM_PARAM_BYTES 4096          // program blob travels as a kernel argument
+#define DVM_PARAM_WORDS (DVM_PARAM_BYTES / 8)
+#define DVM_VEC_E 8                   // consecutive elements per lane per slab (one or two 128-bit accesses)
+#define DVM_VEC_U 2                   // slabs per lane per instruction
+#define DVM_VEC_NREG 16               // V register slots per lane (local memory, sized per program)
+#define DVM_VEC_NSREG 8               // one-float S registers per lane (VGPRs)
+#define DVM_VEC_NSLOT 2               // concurrent reduce accumulators per sweep
+#define DVM_VEC_MAXR 4                // max kept dims and max reduced dims after merging
+#define DVM_VEC_MAXMEM 24             // memory operand descriptors per program
+
+// ---- entry types ---------------------------------------------------------
+enum {
+  VE_VECTOR = 1,  // pointwise / broadcast / reduce program (vm_vector)
+  VE_CUBE = 2,    // MFMA matmul tile loop + interpreted epilogue (vm_cube)
+  VE_ATTN = 3,    // two MFMA stages with online softmax between them (vm_attn)
+};
+
+// ---- element types of memory operands ------------------------------------
+enum {
+  VDT_BOOL = 0,  // uint8 0/1 in memory, 0.0f/1.0f in registers
+  VDT_F16 = 1,
+  VDT_BF16 = 2,
+  VDT_F32 = 3,
+  VDT_I32 = 4,
+};
+
+// ---- schedules -------------------------------------------------------------
+enum {
+  VS_POINTWISE = 0,  // lanes enumerate the whole (kept) index space, no reduce
+  VS_REDX = 1,       // innermost axis is reduced: a team of lanes strides the reduce space of one output
+  VS_REDY = 2,       // innermost axis is kept: lanes own output groups, wave rows partition the reduce space
+};
+
+// ---- opcodes ---------------------------------------------------------------
+// The interpreter is an accumulator machine. Per lane, `acc` holds U slabs of E
+// elements (U*E values); one instruction transforms all of them. Opcodes below
+// VOP_SRC_BASE take no source operand, the others fetch one (kind field).
+enum {
+  VOP_END = 0,
+  VOP_LDR = 1,       // acc = vreg[a]
+  VOP_LDS = 2,       // acc = splat(sreg[a])
+  VOP_LDI = 3,       // acc = splat(imm)
+  VOP_STR = 4,       // vreg[a] = acc           (sub: VF_F32 two slots, VF_16 one slot of packed halves)
+  VOP_STS = 5,       // sreg[a] = acc[0][0]
+  VOP_ST = 6,        // mem[a] = acc
+  VOP_UN = 7,        // acc = f(acc), sub = VU_*
+  VOP_CAST = 8,      // container conversion, sub = VC_*
+  VOP_RED = 9,       // slot[a] (sub = VR_*) accumulates acc      (inside a sweep)
+  VOP_SWEEP = 10,    // start of a loop over the reduce index space; imm = slot kinds, 4 bits each
+  VOP_ENDSWEEP = 11, // next round, or fall through and combine the slots across lanes
+  VOP_FIN = 12,      // acc = combined slot[a]
+  VOP_SRC_BASE = 16,
+  VOP_LD = 16,       // acc = mem[a]             (kind is always VK_MEM)
+  VOP_BINF = 17,     // acc = acc (sub = VB_*) src, float class
+  VOP_BINI = 18,     // acc = acc (sub = VBI_*) src, int32 class
+  VOP_CMP = 19,      // acc = acc (sub = VCMP_*, +8 for int32) src ? 1 : 0 in the operand's container
+  VOP_MSK = 20,      // mask = src != 0          (per element predicate)
+  VOP_MOVM = 21,     // acc = mask ? src : acc
+};
+
+// source kinds (bits 16..19)
+enum { VK_REG = 0, VK_IMM = 1, VK_MEM = 2, VK_ACC = 3, VK_SREG = 4 };
+// result rounding (bits 20..21): value is rounded to that format and widened back
+enum { VRND_NONE = 0, VRND_F16 = 1, VRND_BF16 = 2 };
+// V register storage formats
+enum { VF_F32 = 0, VF_F16 = 1, VF_BF16 = 2 };
+
+// float binary sub-ops (R* = operands reversed: src op acc)
+enum {
+  VB_ADD = 0, VB_SUB, VB_RSUB, VB_MUL, VB_DIV, VB_RDIV, VB_MIN, VB_MAX, VB_AND, VB_OR, VB_POW, VB_RPOW,
+};
+// int32 binary sub-ops
+enum { VBI_ADD = 0, VBI_SUB, VBI_RSUB, VBI_MUL, VBI_MIN, VBI_MAX };
+// unary sub-ops
+enum {
+  VU_SQRT = 0, VU_ABS, VU_LOG, VU_EXP, VU_ISFINITE, VU_ROUND, VU_FLOOR, VU_CEIL, VU_TRUNC, VU_IABS,
+};
+// compare sub-ops (same order as dvm::BinaryType kEqual..kLessEqual); +VCMP_INT for int32 operands
+enum { VCMP_EQ = 0, VCMP_NE, VCMP_GT, VCMP_GE, VCMP_LT, VCMP_LE, VCMP_INT = 8 };
+// cast kinds
+enum {
+  VC_F2I = 0,    // float container -> int32 (C truncation)
+  VC_I2F = 1,    // int32 -> float (then optional rounding via rnd field)
+  VC_RND = 2,    // float -> float rounded per rnd field (f32->f16, f32->bf16)
+  VC_F2B = 3,    // float -> bool container (x != 0 ? 1.0 : 0.0)
+};
+// reduce kinds
+enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
+
+// instruction word:
+//   [7:0] opcode  [15:8] sub  [19:16] src kind  [21:20] rnd
+//   [31:24] a (register / memory operand / slot index)   [63:32] imm32
+#define VI_MAKE(op, sub, kind, rnd, a, imm)                                                     \
+  ((uint64_t)(op) | ((uint64_t)(sub) << 8) | ((uint64_t)(kind) << 16) | ((uint64_t)(rnd) << 20) | \
+   ((uint64_t)(a) << 24) | ((uint64_t)(uint32_t)(imm) << 32))
+#define VI_OP(w) ((uint32_t)(w) & 0xffu)
+#define VI_SUB(w) (((uint32_t)(w) >> 8) & 0xffu)
+#define VI_KIND(w) (((uint32_t)(w) >> 16) & 0xfu)
+#define VI_RND(w) (((uint32_t)(w) >> 20) & 0x3u)
+#define VI_A(w) (((uint32_t)(w) >> 24) & 0xffu)
+#define VI_IMM(w) ((uint32_t)((w) >> 32))
+
+// One axis of an index space, with the constants of a multiply-shift division
+// (q = (mulhi(n, magic) + n) >> shift, valid for n < 2^31).
+typedef struct {
+  uint32_t extent;  // for the innermost domain axis: number of E-groups
+  uint32_t magic;
+  uint32_t shift;
+  uint32_t pad;
+} VDim;
+
+// A memory operand: base address plus element strides against the kept list
+// and the reduced list (position 0 = fastest varying). The stride of the
+// innermost domain axis is 0 (operand broadcast along it: one element is
+// loaded and replicated) or 1 (E consecutive elements).
+typedef struct {
+  uint64_t addr;
+  uint32_t dtype;                  // VDT_*
+  uint32_t flags;                  // VMF_*
+  uint32_t kstride[DVM_VEC_MAXR];
+  uint32_t rstride[DVM_VEC_MAXR];
+} VMemDesc;
+enum { VMF_VEC = 1 /* innermost stride 1 */, VMF_ALIGNED = 2 /* every E-group starts 16-byte aligned */ };
+
+typedef struct {
+  uint32_t entry;        // VE_VECTOR
+  uint32_t sched;        // VS_*
+  uint32_t n_mem;
+  uint32_t n_code;       // instruction words
+  uint32_t n_kdim;
+  uint32_t n_rdim;
+  uint32_t team_log2;    // REDX: lanes per team; REDY: lanes along the kept space (tx)
+  uint32_t team_is_block;// REDX: team spans the whole workgroup
+  uint32_t n_kidx;       // size of the kept index space (groups if the innermost axis is kept)
+  uint32_t n_ridx;       // size of the reduced index space (groups if the innermost axis is reduced)
+  uint32_t inner_extent; // elements along the innermost domain axis
+  uint32_t inner_reduced;// innermost axis belongs to the reduced list
+  uint32_t n_items;      // work items (grid-strided over workgroups)
+  uint32_t mem_off;      // word offset of VMemDesc[n_mem]
+  uint32_t code_off;     // word offset of the instruction words
+  uint32_t n_vslot;      // V register slots in use (each U*16 bytes per lane of local memory)
+  VDim kdims[DVM_VEC_MAXR];
+  VDim rdims[DVM_VEC_MAXR];
+} VVecHeader;            // 64 + 128 = 192 bytes
+
+typedef struct {
+  uint64_t w[DVM_PARAM_WORDS];
+} VmParam;
+
+#endif  // DVM_ISA_GFX950_H_

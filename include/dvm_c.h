@@ -1,0 +1,103 @@
+/* Flat C ABI over dvm::Kernel plus a small runner (device buffers, launch,
+ * timing), bound by the Python package with ctypes.
+ *
+ * It stands where the reference's pybind module stands: the `Kernel` builder
+ * methods of include/dvm_py.h:277-388 and the `PyKernel` runner of
+ * src/pybind_api.cc:410-907 (input / codegen / run / output / perf / das).
+ * Handles are opaque pointers owned by the runner they came from. Functions
+ * that return a pointer return NULL on error, the others a non-zero code;
+ * dvm_c_last_error() then holds the message (per thread).
+ */
+#ifndef DVM_C_H_
+#define DVM_C_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+#pragma GCC visibility push(default)
+
+typedef struct dvm_rt dvm_rt;          /* a kernel plus its runner                        */
+typedef struct dvm_obj dvm_obj;        /* an operator node (dvm::NDObject)                */
+typedef struct dvm_shape dvm_shape;    /* an updatable shape (dvm::IntArrayRef + storage) */
+typedef struct dvm_scalar dvm_scalar;  /* an updatable scalar (dvm::ScalarRef)            */
+
+/* One operand of a binary operator. kind: 0 tensor (obj), 1 float immediate (f),
+ * 2 int32 immediate (i), 3 scalar reference (ref). */
+typedef struct {
+  int kind;
+  dvm_obj *obj;
+  dvm_scalar *ref;
+  double f;
+  int64_t i;
+} dvm_operand;
+
+const char *dvm_c_last_error(void);
+
+/* ker_type: "vector", "split", "mix", "cube" optionally followed by ":dyn" (src/pybind_api.cc:117-154).
+ * run_mode: "dev" (needs a GPU) or "das" (code generation and disassembly only, fake addresses). */
+dvm_rt *dvm_rt_new(const char *ker_type, const char *run_mode, int dev_id);
+void dvm_rt_delete(dvm_rt *rt);
+int dvm_rt_reset(dvm_rt *rt);
+
+dvm_shape *dvm_rt_new_shape(dvm_rt *rt, const int64_t *dims, size_t n);
+int dvm_shape_update(dvm_shape *s, const int64_t *dims, size_t n);
+dvm_scalar *dvm_rt_new_scalar(dvm_rt *rt, int dtype);
+int dvm_scalar_update_f(dvm_scalar *s, double v);
+int dvm_scalar_update_i(dvm_scalar *s, int64_t v);
+
+dvm_obj *dvm_rt_load(dvm_rt *rt, dvm_shape *shape, int dtype);
+dvm_obj *dvm_rt_store(dvm_rt *rt, dvm_obj *x);
+dvm_obj *dvm_rt_unary(dvm_rt *rt, int unary_type, dvm_obj *x);
+dvm_obj *dvm_rt_binary(dvm_rt *rt, int binary_type, const dvm_operand *lhs, const dvm_operand *rhs);
+dvm_obj *dvm_rt_select(dvm_rt *rt, dvm_obj *cond, dvm_obj *lhs, dvm_obj *rhs);
+dvm_obj *dvm_rt_cast(dvm_rt *rt, dvm_obj *x, int dtype);
+dvm_obj *dvm_rt_broadcast(dvm_rt *rt, dvm_obj *x, dvm_shape *shape);
+dvm_obj *dvm_rt_full(dvm_rt *rt, const dvm_operand *value, dvm_shape *shape, int dtype);
+dvm_obj *dvm_rt_reshape(dvm_rt *rt, dvm_obj *x, dvm_shape *shape);
+dvm_obj *dvm_rt_reduce(dvm_rt *rt, int reduce_type, dvm_obj *x, dvm_shape *dims, int keepdims);
+dvm_obj *dvm_rt_copy(dvm_rt *rt, dvm_obj *x);
+dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int trans_b, dvm_obj *bias);
+int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store);
+
+int dvm_obj_rank(const dvm_obj *o);
+int dvm_obj_shape(const dvm_obj *o, int64_t *dims, size_t cap);
+int dvm_obj_dtype(const dvm_obj *o);
+
+/* Copies `bytes` of host data into a device buffer owned by the runner and binds it to the load. */
+int dvm_rt_input(dvm_rt *rt, dvm_obj *load, const void *host, size_t bytes);
+/* Binds a caller-owned device buffer to a load or store (no copy, no ownership). */
+int dvm_rt_bind_device(dvm_rt *rt, dvm_obj *io, void *device_ptr);
+/* Normalize + allocate unbound outputs + CodeGen with relocations. */
+int dvm_rt_codegen(dvm_rt *rt);
+/* Host wall time of the last Normalize + CodeGen in microseconds. */
+double dvm_rt_jit_us(const dvm_rt *rt);
+/* Launch on the runner's stream (or on `stream` if not NULL) and, with sync != 0, wait. */
+int dvm_rt_run(dvm_rt *rt, void *stream, int sync);
+int dvm_rt_output(dvm_rt *rt, dvm_obj *store, void *host, size_t bytes);
+void *dvm_rt_device_ptr(dvm_rt *rt, dvm_obj *io);
+/* warmup + iters timed launches with events: out = {min, max, mean} microseconds (src/pybind_api.cc:751-767). */
+int dvm_rt_perf(dvm_rt *rt, int warmup, int iters, double out[3]);
+/* Number of device launches one run() issues. */
+int dvm_rt_num_launches(const dvm_rt *rt);
+size_t dvm_rt_workspace_bytes(const dvm_rt *rt);
+
+const char *dvm_rt_das(dvm_rt *rt);
+const char *dvm_rt_dump(dvm_rt *rt);
+const char *dvm_rt_dump_r(dvm_rt *rt);
+const char *dvm_rt_inspect(dvm_rt *rt);
+
+/* Host codecs used for bf16 numpy round trips (src/pybind_api.cc:584-609). */
+void dvm_c_f32_to_bf16(const float *src, uint16_t *dst, size_t n);
+void dvm_c_bf16_to_f32(const uint16_t *src, float *dst, size_t n);
+
+int dvm_c_has_device(void);
+int dvm_c_core_num(void);
+
+#pragma GCC visibility pop
+#ifdef __cplusplus
+}
+#endif
+#endif /* DVM_C_H_ */

@@ -1,0 +1,82 @@
+/* C ABI of the gfx950 device layer (libdvm_hip.so).
+ *
+ * These are the entry points the reference's host code binds for its device
+ * backend: the three device-VM functions of src/vm_gpu.h:153-155 and the
+ * runtime wrappers of src/runtime.h:34-84. Plain C types only, so the host
+ * emitter (or any other caller) needs no HIP headers. Every function returns
+ * 0 on success or the HIP error code, unless stated otherwise. No function
+ * throws.
+ */
+#ifndef DVM_HIP_H_
+#define DVM_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Limits of the device the VM was initialised on.
+ * Replaces dvm::gpu::SysConfig (src/vm_gpu.h:147-151). */
+typedef struct {
+  uint64_t core_num;        /* compute units */
+  uint64_t local_mem_size;  /* LDS bytes one workgroup may use */
+  uint64_t default_threads; /* default workgroup size */
+  uint64_t wave_size;       /* 64 on gfx950 */
+  uint64_t l2_bytes;        /* L2 size per XCD */
+  uint64_t xcd_num;         /* accelerator dies (L2 domains) */
+} dvm_hip_sysconfig;
+
+/* Queries device `dev_id`, loads the VM kernels and fills `conf`.
+ * Replaces dvm::gpu::InitVM (src/vm_gpu.h:153). */
+int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf);
+
+/* Launch geometry for a program of interpreter kind `kind` (the schedule id
+ * of a vector program, or 16 + entry type for the matmul kernels) over
+ * `item_num` work items, each workgroup having `threads` lanes and
+ * `lds_bytes` of local memory: returns (workgroups << 32) | threads, the
+ * number of workgroups that are resident at once, capped by `item_num`.
+ * Replaces dvm::gpu::SelectBlockThread (src/vm_gpu.h:154). */
+uint64_t dvm_hip_select_block_thread(uint64_t kind, uint64_t item_num, uint64_t threads, uint32_t lds_bytes);
+
+/* Launches the device VM on one 4096-byte program blob (`param` is host
+ * memory, copied into the kernel arguments). The entry type in the blob's
+ * first word selects the interpreter kernel.
+ * Replaces dvm::gpu::LaunchVM (src/vm_gpu.h:155). */
+int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, uint32_t lds_bytes, void *stream);
+
+/* Fills `bytes` bytes at device address `dst` with the 32-bit pattern `value`
+ * on `stream` using a fill kernel (safe under graph capture, unlike a memset
+ * node). Used where the reference launches its clean kernels
+ * (src/ops.cc:551-606, src/kernel.cc:23-75). `bytes` must be a multiple of 4. */
+int dvm_hip_fill_u32(void *dst, uint32_t value, size_t bytes, void *stream);
+
+/* Runtime wrappers: the dvm::rt functions of src/runtime.h:34-84. */
+int dvm_hip_get_device_count(uint32_t *count);
+int dvm_hip_set_device(int device_id);
+int dvm_hip_get_device(int *device_id);
+int dvm_hip_create_stream(void **stream);
+int dvm_hip_destroy_stream(void *stream);
+int dvm_hip_synchronize_stream(void *stream);
+int dvm_hip_malloc(void **ptr, size_t size);
+int dvm_hip_free(void *ptr);
+int dvm_hip_malloc_host(void **ptr, size_t size);
+int dvm_hip_free_host(void *ptr);
+int dvm_hip_mem_to_dev(void *dst, const void *src, size_t count);
+int dvm_hip_mem_from_dev(void *dst, const void *src, size_t count);
+int dvm_hip_mem_to_dev_async(void *dst, const void *src, size_t count, void *stream);
+int dvm_hip_memset(void *dst, int value, size_t size);
+int dvm_hip_create_event(void **event);
+int dvm_hip_destroy_event(void *event);
+int dvm_hip_record_event(void *event, void *stream);
+int dvm_hip_synchronize_event(void *event);
+int dvm_hip_event_elapsed_time(float *ms, void *start, void *end);
+
+/* Text for an error code returned by any function above (static storage). */
+const char *dvm_hip_error_string(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DVM_HIP_H_ */
