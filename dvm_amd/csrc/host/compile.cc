@@ -20,6 +20,7 @@
 #include <algorithm>
 #include <chrono>
 #include <cmath>
+#include <cstdlib>
 #include <cstring>
 #include <stdexcept>
 
@@ -292,17 +293,26 @@ class Compiler {
  public:
   explicit Compiler(VKernel *k) : k_(k), n_(static_cast<int>(k->ops_.size())) {}
 
+  // Partition modes, tried in order until every sub-kernel compiles: 0 joins an operator to its
+  // producers' sub-kernel whenever the hard rules allow, 1 also requires broadcast-compatible
+  // shapes, 2 additionally ends a sub-kernel after every reduce (the reference's rule), 3 gives
+  // every operator its own sub-kernel.
   size_t Run() {
-    try {
-      return RunOnce(false);
-    } catch (const std::runtime_error &) {
-      // maximal fusion did not fit the VM: cut after every reduce instead
-      return RunOnce(true);
+    for (int mode = k_->part_mode_; mode < 3; ++mode) {
+      try {
+        const size_t ws = RunOnce(mode);
+        k_->part_mode_ = mode;
+        return ws;
+      } catch (const std::runtime_error &) {
+      }
     }
+    k_->part_mode_ = 3;
+    return RunOnce(3);
   }
 
-  size_t RunOnce(bool conservative) {
-    conservative_ = conservative;
+  size_t RunOnce(int mode) {
+    mode_ = mode;
+    conservative_ = mode >= 2;
     area_.assign(n_, -1);
     live_.assign(n_, 0);
     mat_.assign(n_, 0);
@@ -419,9 +429,9 @@ class Compiler {
     }
     if (o->kind == kObjReduce) {
       if (ai.has_reduce && !SameReduce(ai.reduce, o)) return false;
-      return DomCompatible(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
+      return mode_ == 0 || DomCompatible(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
     }
-    return DomCompatible(ai, o->shape_ref_->data, o->rank());
+    return mode_ == 0 || DomCompatible(ai, o->shape_ref_->data, o->rank());
   }
 
   void Join(int a, const NDObject *o) {
@@ -446,11 +456,30 @@ class Compiler {
   void Partition() {
     areas_.clear();
     const bool fuse = !conservative_;
+    // Operators that share no tensor (directly or through other operators) never share a
+    // sub-kernel: connected components are numbered first, each gets its own range of areas.
+    std::vector<int> comp(n_);
+    for (int i = 0; i < n_; ++i) comp[i] = i;
+    auto find = [&](int x) {
+      while (comp[x] != x) x = comp[x] = comp[comp[x]];
+      return x;
+    };
+    for (int i = 0; i < n_; ++i) {
+      NDObject *o = k_->ops_[i];
+      if (!live_[i]) continue;
+      for (int j = 0; j < o->nin; ++j) {
+        if (o->in[j] == nullptr || o->in[j]->kind == kObjBroadcastS) continue;
+        comp[find(i)] = find(o->in[j]->id);
+      }
+    }
+    std::vector<int> comp_base(n_, -1);
     for (int i = 0; i < n_; ++i) {
       NDObject *o = k_->ops_[i];
       if (!live_[i] || IsLeaf(o)) continue;
       if (IsView(o)) continue;  // read through by its consumers
-      int a = 0;
+      const int c = find(i);
+      if (comp_base[c] < 0) comp_base[c] = static_cast<int>(areas_.size());
+      int a = comp_base[c];
       for (int j = 0; j < o->nin; ++j) {
         const NDObject *v = o->in[j];
         if (v == nullptr || IsLeaf(v)) continue;
@@ -461,10 +490,10 @@ class Compiler {
           cut = true;
         }
         if (o->kind == kObjMatMul) cut = true;
-        if (!fuse && v->kind == kObjReduce) cut = true;  // the reference's rule: a reduce ends its sub-kernel
+        if (!fuse && v->kind == kObjReduce && o->kind != kObjStore) cut = true;  // the reference's rule: a reduce ends its sub-kernel
         a = std::max(a, area_[v->id] + (cut ? 1 : 0));
       }
-      if (o->kind == kObjMatMul) a = std::max(a, static_cast<int>(areas_.size()));
+      if (o->kind == kObjMatMul || (mode_ >= 3 && o->kind != kObjStore)) a = std::max(a, static_cast<int>(areas_.size()));
       while (!CanJoin(a, o)) ++a;
       area_[i] = a;
       Join(a, o);
@@ -521,6 +550,7 @@ class Compiler {
   int n_mem_ = 0;
   std::vector<uint64_t> code_;
   bool conservative_ = false;
+  int mode_ = 0;
   bool single_round_ = false;
   int acc_node_ = -1;
   uint32_t sreg_used_ = 0;
@@ -567,7 +597,21 @@ class Compiler {
     return idx;
   }
 
-  void Fail(const char *why) { Throw(std::string("cannot compile sub-kernel: ") + why); }
+  int cur_area_ = 0;
+  void Fail(const char *why) {
+    std::string msg = "cannot compile sub-kernel " + std::to_string(cur_area_) + " (partition mode " +
+                      std::to_string(mode_) + "): " + why;
+    if (std::getenv("DVM_DEBUG") != nullptr) {
+      msg += "\n nodes:";
+      for (int i = 0; i < nn_; ++i) {
+        msg += "\n  n" + std::to_string(i) + " kind=" + std::to_string(nodes_[i].kind) + " op=%" +
+               std::to_string(nodes_[i].op != nullptr ? nodes_[i].op->id : -1) + " dims=[";
+        for (int d = 0; d < nodes_[i].rank; ++d) msg += std::to_string(nodes_[i].dims[d]) + ":" + std::to_string(nodes_[i].axis[d]) + " ";
+        msg += "] in=" + std::to_string(nodes_[i].in[0]) + "," + std::to_string(nodes_[i].in[1]);
+      }
+    }
+    Throw(msg);
+  }
 
   void CompileArea(int a);
   void CompileCube(int a);
@@ -728,6 +772,22 @@ void Compiler::UnifyAxes() {
         for (int j = 0; j < n.nin; ++j)
           if (n.in[j] >= 0) UnifyAligned(i, n.in[j]);
         break;
+    }
+  }
+  // Reduces that share a sub-kernel have the same input shape and axes: their inputs walk the
+  // same index space even when no operator relates them, so their dims are unified by position.
+  {
+    int first = -1;
+    for (int i = 0; i < nn_; ++i) {
+      if (nodes_[i].kind != AK_REDUCE) continue;
+      if (first < 0) {
+        first = nodes_[i].in[0];
+        continue;
+      }
+      const ANode &x = nodes_[nodes_[i].in[0]], &f = nodes_[first];
+      if (x.rank != f.rank) Fail("reduces of different rank in one sub-kernel");
+      for (int d = 0; d < x.rank; ++d)
+        if (x.dims[d] != 1 && x.dims[d] == f.dims[d]) Union(Var(nodes_[i].in[0], d), Var(first, d));
     }
   }
   // classes with extent > 1 become domain axes
@@ -1165,7 +1225,7 @@ void Compiler::ComputeInto(int v) {
   }
   const bool is_int = (o->kind == kObjCompare || o->kind == kObjCompareS || o->kind == kObjBinary ||
                        o->kind == kObjBinaryS || o->kind == kObjUnary)
-                          ? nodes_[Resolve(n.in[0])].dtype == kInt32
+                          ? o->in[0]->type_id_ == kInt32
                           : false;
   switch (o->kind) {
     case kObjUnary: {
@@ -1192,7 +1252,7 @@ void Compiler::ComputeInto(int v) {
     }
     case kObjCast: {
       const int x = Resolve(n.in[0]);
-      const DataType s = nodes_[x].dtype, d = n.dtype;
+      const DataType s = o->in[0]->type_id_, d = n.dtype;
       EmitValue(x);
       ConsumeUse(x);
       BeforeOverwrite();
@@ -1213,7 +1273,7 @@ void Compiler::ComputeInto(int v) {
       EmitValue(x);
       ConsumeUse(x);
       BeforeOverwrite();
-      const uint32_t imm = ScalarToContainer(o->scalar.Get(), nodes_[x].dtype);
+      const uint32_t imm = ScalarToContainer(o->scalar.Get(), o->in[0]->type_id_);
       if (o->kind == kObjCompareS) {
         Emit(VOP_CMP, CmpSub(o->op, o->scalar_left, is_int), VK_IMM, 0, 0, imm);
       } else if (is_int) {
@@ -1511,6 +1571,7 @@ void Compiler::FinishProgram() {
 }
 
 void Compiler::CompileArea(int a) {
+  cur_area_ = a;
   k_->programs_.emplace_back();
   prog_ = &k_->programs_.back();
   if (areas_[a].cube) {

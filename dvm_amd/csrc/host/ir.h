@@ -163,6 +163,7 @@ class VKernel {
   std::vector<size_t> ws_sizes_;
   void *ws_base_ = nullptr;
   std::string name_, fullname_;
+  int part_mode_ = 0;             // partition mode that compiled last time (see Compiler::Run)
   double last_codegen_us_ = 0.0;  // wall time of the last Normalize+CodeGen, for JIT latency reports
 
  private:

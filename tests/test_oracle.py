@@ -1,0 +1,214 @@
+"""Pins the CPU oracle (oracle/dvm_oracle.c + oracle/oracle.py) without a GPU.
+
+Checks, chosen so that a plausible mistake (wrong rounding mode, dropped NaN case,
+wrong operand order, truncation vs rounding) fails one of them:
+  * fp16 codec: every one of the 65536 bit patterns round-trips through fp32 exactly as
+    numpy.float16 does; random and tie fp32 values round like numpy (round to nearest even);
+  * bf16 codec: closed form on ties, carries into the exponent, inf, NaN (host form -> 0x7fc0,
+    src/dvm.cc:173-186), and the bf16 truncation trick of the reference's tester (python/dvm/tester.py:93-99);
+  * the constants of the reference's own tests: 0.5 / 0.4 element-wise table (tests/ut/test_elemwise.py:24-54),
+    0.1 + 0.3 (examples/01_add.py:27-34), pow special values [-2, 9, -64, 1, nan, 3]
+    (tests/ut/test_elemwise.py:235-246), sum of 64 x 0.01 = 0.64 (tests/ut/test_reduce.py:74-83),
+    add->sum 40.96 (tests/ut/test_reduce.py:232-241);
+  * int32 wrap-around like NumPy (tests/ut/test_elemwise.py:295-428), float -> int32 truncation,
+    round half to even (tests/ut/test_elemwise.py:456-468);
+  * lowering rules against NumPy: logical ops over bool / fp16 / fp32, compares of mixed dtypes,
+    scalar-left sub / div, pow by integer and scalar ** x;
+  * sum against float64 NumPy sums, max / min exact, matmul against np.matmul on fp32 copies
+    (tests/ut/test_matmul.py:34-36), batch-norm restatement against the float64 closed form.
+"""
+import numpy as np
+import pytest
+
+from oracle import oracle as ora
+from oracle.oracle import OracleKernel
+
+
+def test_f16_all_bit_patterns():
+    bits = np.arange(65536, dtype=np.uint16)
+    ref = bits.view(np.float16).astype(np.float32)
+    got = ora.f16_bits_to_f32(bits)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    back = ora.f32_to_f16_bits(ref)
+    nan = np.isnan(ref)
+    assert np.array_equal(back[~nan], bits[~nan])
+    assert np.all((back[nan] & 0x7c00) == 0x7c00) and np.all((back[nan] & 0x3ff) != 0)
+
+
+def test_f32_to_f16_rounding_matches_numpy():
+    rng = np.random.default_rng(7)
+    x = np.concatenate([
+        rng.normal(0, 1, 200000), rng.normal(0, 1e-5, 50000), rng.normal(0, 3e4, 50000),
+        np.array([65504.0, 65519.9, 65520.0, 65536.0, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8, 6.1e-5, -0.0, np.inf, -np.inf]),
+    ]).astype(np.float32)
+    # exact ties between neighbouring halves
+    h = rng.integers(0x0001, 0x7bff, 20000).astype(np.uint16)
+    a = h.view(np.float16).astype(np.float32)
+    b = (h + 1).astype(np.uint16).view(np.float16).astype(np.float32)
+    x = np.concatenate([x, (a + b) / 2, -(a + b) / 2]).astype(np.float32)
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    assert np.array_equal(ora.f32_to_f16_bits(x), want)
+
+
+def test_bf16_codec():
+    def bits(v):
+        return int(ora.f32_to_bf16_bits(np.array([v], np.float32))[0])
+    assert bits(1.0) == 0x3f80
+    assert bits(np.float32(1.0) + np.float32(2 ** -8)) == 0x3f80       # tie -> even (down)
+    assert bits(np.float32(1.0) + np.float32(3 * 2 ** -8)) == 0x3f82   # tie -> even (up)
+    assert bits(np.float32(1.0) + np.float32(2 ** -8) + np.float32(2 ** -20)) == 0x3f81
+    assert bits(np.array([0x3fffffff], np.uint32).view(np.float32)[0]) == 0x4000  # carry into the exponent
+    assert bits(np.inf) == 0x7f80 and bits(-np.inf) == 0xff80
+    assert bits(np.nan) == 0x7fc0
+    x = np.random.default_rng(3).normal(0, 10, 100000).astype(np.float32)
+    u = x.view(np.uint32).astype(np.uint64)
+    want = ((u + 0x7fff + ((u >> 16) & 1)) >> 16).astype(np.uint16)
+    assert np.array_equal(ora.f32_to_bf16_bits(x), want)
+    # values that are already bf16 (the reference tester's truncation) convert exactly
+    t = (x.view(np.uint32) & 0xFFFF0000).view(np.float32)
+    assert np.array_equal(ora.bf16_bits_to_f32(ora.f32_to_bf16_bits(t)), t)
+
+
+@pytest.mark.parametrize("dt", [np.float16, np.float32])
+def test_elementwise_constants(dt):
+    k = OracleKernel()
+    x = np.full([32, 1024], 0.5, dt)
+    y = np.full([32, 1024], 0.4, dt)
+    a, b = k.load(x), k.load(y)
+    eps = 1e-3 if dt == np.float16 else 1e-6
+    for got, want in [(k.sqrt(a), np.sqrt(x)), (k.abs(a), np.abs(x)), (k.log(a), np.log(x)), (k.exp(a), np.exp(x)),
+                      (k.reciprocal(a), np.reciprocal(x)), (k.add(a, b), x + y), (k.sub(a, b), x - y),
+                      (k.div(a, b), x / y), (k.mul(a, b), x * y), (k.maximum(a, b), np.maximum(x, y)),
+                      (k.minimum(a, b), np.minimum(x, y))]:
+        assert np.allclose(k.output(got).astype(np.float32), want.astype(np.float32), rtol=eps, atol=eps)
+    # fp16 arithmetic is "fp32 op, round once": identical to numpy's half arithmetic, bit for bit
+    if dt == np.float16:
+        rng = np.random.default_rng(5)
+        p, q = rng.normal(0, 1, 4096).astype(dt), rng.normal(0, 1, 4096).astype(dt)
+        for f, g in [(k.add, np.add), (k.sub, np.subtract), (k.mul, np.multiply), (k.div, np.divide)]:
+            assert np.array_equal(k.output(f(k.load(p), k.load(q))).view(np.uint16), g(p, q).view(np.uint16))
+
+
+def test_add_example_and_reduce_constants():
+    k = OracleKernel()
+    x, y = np.full([32, 32], 0.1, np.float32), np.full([32, 32], 0.3, np.float32)
+    assert np.array_equal(k.output(k.add(k.load(x), k.load(y))), x + y)
+    z = k.load(np.full([64, 1001], 0.01, np.float32))
+    assert np.allclose(k.output(k.sum(z, (0,), False)), 0.64, rtol=1e-6)
+    a = k.load(np.full([32, 2048], 0.01, np.float32))
+    assert np.allclose(k.output(k.sum(k.add(a, a), (1,), True)), 40.96, rtol=1e-6)
+
+
+def test_pow_special_values():
+    k = OracleKernel()
+    a = np.array([-2, -3, -4, 0, -2, 9], np.float32)
+    b = np.array([1, 2, 3, 0, 0.5, 0.5], np.float32)
+    got = k.output(k.pow(k.load(a), k.load(b)))
+    assert np.allclose(got, [-2, 9, -64, 1, np.nan, 3], equal_nan=True)
+    x = np.abs(np.random.default_rng(1).normal(0, 1, 1000) - 2).astype(np.float32)
+    for s in (0, 1.2, 5, -7, -3):
+        assert np.allclose(k.output(k.pow(k.load(x), s)), np.power(x, np.float32(s)), rtol=1e-5, atol=1e-5)
+    assert np.allclose(k.output(k.pow(0.91, k.load(x))), np.power(np.float32(0.91), x), rtol=1e-5, atol=1e-6)
+
+
+def test_int32_wraparound_and_casts():
+    rng = np.random.default_rng(2)
+    x = rng.integers(-2 ** 30, 2 ** 30, [32, 1024]).astype(np.int32)
+    y = rng.integers(-2 ** 30, 2 ** 30, [32, 1024]).astype(np.int32)
+    k = OracleKernel()
+    a, b = k.load(x), k.load(y)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(k.output(k.add(a, b)), x + y)
+        assert np.array_equal(k.output(k.sub(a, b)), x - y)
+        assert np.array_equal(k.output(k.mul(a, b)), x * y)
+        assert np.array_equal(k.output(k.add(a, 11111)), x + np.int32(11111))
+    assert np.array_equal(k.output(k.maximum(a, b)), np.maximum(x, y))
+    assert np.array_equal(k.output(k.abs(a)), np.abs(x))
+    f = rng.normal(0, 100, 10000).astype(np.float32)
+    assert np.array_equal(k.output(k.cast(k.load(f), "int32")), np.trunc(f).astype(np.int32))
+    assert np.array_equal(k.output(k.cast(k.load(x[0]), "float32")), x[0].astype(np.float32))
+    h = rng.normal(0, 10, 10000).astype(np.float16)
+    assert np.array_equal(k.output(k.cast(k.load(h), "int32")), np.trunc(h.astype(np.float32)).astype(np.int32))
+    r = np.array([0.5, 1.5, 2.5, -0.5, -1.5, 2.4999, 3.5001], np.float32)
+    assert np.array_equal(k.output(k.round(k.load(r))), np.round(r))
+    assert np.array_equal(k.output(k.floor(k.load(f))), np.floor(f))
+    assert np.array_equal(k.output(k.ceil(k.load(f))), np.ceil(f))
+    assert np.array_equal(k.output(k.trunc(k.load(f))), np.trunc(f))
+
+
+@pytest.mark.parametrize("dt", [np.bool_, np.float16, np.float32])
+def test_logical_rules(dt):
+    rng = np.random.default_rng(4)
+    x = rng.choice([True, False], [128, 777]).astype(dt)
+    y = rng.choice([True, False], [128, 777]).astype(dt)
+    k = OracleKernel()
+    a, b = k.load(x), k.load(y)
+    assert np.array_equal(k.output(k.logical_and(a, b)).astype(bool), np.logical_and(x, y))
+    assert np.array_equal(k.output(k.logical_or(a, b)).astype(bool), np.logical_or(x, y))
+    assert np.array_equal(k.output(k.logical_not(a)).astype(bool), np.logical_not(x))
+
+
+def test_compare_select_scalar_rules():
+    rng = np.random.default_rng(6)
+    xi = rng.integers(-1024, 1024, [128, 77]).astype(np.int32)
+    yi = rng.integers(-1024, 1024, [128, 77]).astype(np.int32)
+    xf = rng.normal(0, 1, [128, 77]).astype(np.float32)
+    yf = rng.normal(0, 1, [128, 77]).astype(np.float32)
+    k = OracleKernel()
+    g = k.greater(k.load(xi), k.load(yi))
+    l = k.less(k.load(xf), k.load(yf))
+    assert g.t == ora.BOOL and np.array_equal(k.output(g), xi > yi)
+    assert np.array_equal(k.output(k.logical_and(g, l)), np.logical_and(xi > yi, xf < yf))
+    assert np.array_equal(k.output(k.select(l, k.load(xf), k.load(yf))), np.where(xf < yf, xf, yf))
+    assert np.array_equal(k.output(k.greater_equal(0.25, k.load(xf))), 0.25 >= xf)
+    assert np.array_equal(k.output(k.sub(0.1, k.load(xf))), xf * np.float32(-1.0) + np.float32(0.1))
+    assert np.array_equal(k.output(k.sub(k.load(xf), 0.1)), xf + np.float32(-0.1))
+    assert np.array_equal(k.output(k.div(2.0, k.load(xf))), np.float32(2.0) / xf)
+    hf = xf.astype(np.float16)
+    assert np.array_equal(k.output(k.div(2.0, k.load(hf))).view(np.uint16), (np.float16(2.0) / hf).view(np.uint16))
+    assert np.array_equal(k.output(k.isfinite(k.load(np.array([1, np.inf, -np.inf, np.nan], np.float32)))), [1, 0, 0, 0])
+
+
+def test_reduce_against_float64():
+    rng = np.random.default_rng(8)
+    x = rng.normal(-0.5, 0.5, [6, 4, 2, 5, 1, 3, 8]).astype(np.float32)
+    k = OracleKernel()
+    for dims in [(0,), (6,), (1, 3), (0, 2, 5), (0, 1, 2, 3, 4, 5, 6)]:
+        for keep in (True, False):
+            want = np.sum(x.astype(np.float64), axis=dims, keepdims=keep).astype(np.float32)
+            assert np.array_equal(k.output(k.sum(k.load(x), dims, keep)), want)
+            assert np.array_equal(k.output(k.max(k.load(x), dims, keep)), np.max(x, axis=dims, keepdims=keep))
+            assert np.array_equal(k.output(k.min(k.load(x), dims, keep)), np.min(x, axis=dims, keepdims=keep))
+    nanx = np.array([[1.0, np.nan, 3.0], [1.0, 2.0, 3.0]], np.float32)
+    assert np.array_equal(k.output(k.max(k.load(nanx), (1,), False)), np.max(nanx, 1), equal_nan=True)
+
+
+def test_matmul_against_numpy():
+    np.random.seed(1)
+    for dt, eps in [(np.float16, 1e-3), ("bfloat16", 5e-3)]:
+        a = np.random.normal(0, 0.1, (64, 96)).astype(np.float32)
+        b = np.random.normal(0, 0.1, (96, 48)).astype(np.float32)
+        k = OracleKernel()
+        la = k.load(a.astype(np.float16) if dt == np.float16 else a, None if dt == np.float16 else dt)
+        lb = k.load(b.astype(np.float16) if dt == np.float16 else b, None if dt == np.float16 else dt)
+        want = np.matmul(la.a, lb.a)
+        assert np.allclose(k.output(k.matmul(la, lb, False, False)).astype(np.float32), want, rtol=eps, atol=eps)
+        lbt = k.load(np.ascontiguousarray(lb.a.T), None if dt == np.float16 else dt) if dt != np.float16 else k.load(np.ascontiguousarray(lb.a.T).astype(np.float16))
+        assert np.array_equal(k.output(k.matmul(la, lbt, False, True)), k.output(k.matmul(la, lb, False, False)))
+    # an exactly representable case: no tolerance
+    a = np.arange(12, dtype=np.float32).reshape(3, 4).astype(np.float16)
+    b = np.arange(8, dtype=np.float32).reshape(4, 2).astype(np.float16)
+    k = OracleKernel()
+    assert np.array_equal(k.output(k.matmul(k.load(a), k.load(b), False, False)), (a.astype(np.float32) @ b.astype(np.float32)).astype(np.float16))
+
+
+def test_batchnorm_restatement():
+    rng = np.random.default_rng(1002)
+    x = rng.normal(0, 1, [4, 16, 7, 9]).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, [16]).astype(np.float32)
+    b = rng.normal(0, 0.1, [16]).astype(np.float32)
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean((0, 2, 3), keepdims=True)) / np.sqrt(x64.var((0, 2, 3), keepdims=True) + 1e-5)
+    want = want * g[None, :, None, None] + b[None, :, None, None]
+    assert np.allclose(ora.batchnorm_nchw(x, g, b, 1e-5), want, rtol=1e-5, atol=1e-5)

@@ -1,0 +1,218 @@
+"""GPU parity: broadcast, reduce, reshape, graph cutting and dynamic shapes (reference tests cited per case)."""
+import numpy as np
+import pytest
+
+from dvm_amd.tester import Tester
+from tests.util import run_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def test_add_example():  # examples/01_add.py:19-34 (BASELINE config 1)
+    import dvm_amd as dvm
+
+    @dvm.kernel
+    def my_add(k, x, y):
+        return k.store(k.add(k.load(x, dvm.float32), k.load(y, dvm.float32)))
+    x, y = np.full([32, 32], 0.1, np.float32), np.full([32, 32], 0.3, np.float32)
+    assert np.array_equal(my_add(x, y), x + y)
+    x, y = np.full([32, 1], 0.2, np.float32), np.full([32, 512], 0.7, np.float32)
+    assert np.array_equal(my_add(x, y), x + y)  # same kernel object, new shapes
+
+
+@pytest.mark.parametrize("case", [((32, 1), (32, 512)), ((1, 512), (32, 512)), ((4, 1, 7, 1), (4, 3, 7, 5)), ((1,), (33, 9)),
+                                  ((2, 3, 1, 5), (2, 3, 4, 5)), ((16, 1, 131), (16, 4, 131))])
+@pytest.mark.parametrize("dt", [np.float32, np.float16, np.int32, np.bool_])
+def test_broadcast(case, dt):  # tests/ut/test_broadcast.py:24-165
+    src, dst = case
+    rng = np.random.default_rng(len(dst))
+    x = (rng.normal(0, 10, src)).astype(dt)
+    run_parity(lambda k, a: k.broadcast(a, list(dst)), [x], golden=np.broadcast_to(x, dst), eps=0)
+    if dt not in (np.bool_,):
+        y = (rng.normal(0, 10, dst)).astype(dt)
+        with np.errstate(over="ignore"):
+            run_parity(lambda k, a, b: k.add(a, b), [x, y], golden=x + y, eps=0 if dt == np.int32 else None)
+
+
+def test_broadcast_scalar_and_bf16():  # tests/ut/test_broadcast.py:257-277
+    run_parity(lambda k, a: k.add(k.full(0.3, [3, 10], "float32"), a), [np.zeros([3, 10], np.float32)], golden=np.full([3, 10], np.float32(0.3)))
+    x = np.random.default_rng(2).normal(0, 1, [7, 1]).astype(np.float32)
+    outs = run_parity(lambda k, a: k.broadcast(a, [7, 33]), [x], dtypes=["bfloat16"], eps=0)
+    assert outs[0].shape == (7, 33)
+
+
+@pytest.mark.parametrize("dim", [64, 256, 251])
+def test_sum_last_axis(dim):  # tests/ut/test_reduce.py:24-33
+    x = np.random.default_rng(dim).normal(-0.5, 0.5, [10, dim]).astype(np.float32)
+    run_parity(lambda k, a: [k.sum(a, (1,), True), k.sum(a, (1,), False)], [x],
+               golden=[np.sum(x, 1, keepdims=True), np.sum(x, 1)])
+
+
+@pytest.mark.parametrize("shape", [(10, 6, 64), (10, 6, 60), (10, 2, 6128)])
+def test_sum_middle_axis(shape):  # tests/ut/test_reduce.py:36-45
+    x = np.random.default_rng(shape[2]).normal(-0.5, 0.5, shape).astype(np.float32)
+    run_parity(lambda k, a: k.sum(a, (1,), False), [x], golden=np.sum(x, 1))
+
+
+@pytest.mark.parametrize("ij", [(1, 1), (3, 5), (7, 9), (13, 11), (17, 3), (5, 31), (9, 9)])
+def test_sum_023(ij):  # tests/ut/test_reduce.py:48-58
+    x = np.random.default_rng(ij[0]).normal(-0.5, 0.5, [3, 1280, ij[0], ij[1]]).astype(np.float32)
+    run_parity(lambda k, a: k.sum(a, (0, 2, 3), True), [x], golden=np.sum(x, (0, 2, 3), keepdims=True), eps=1e-4)
+
+
+@pytest.mark.parametrize("dims", [(0,), (6,), (1, 3), (0, 2, 5), (2, 4, 6), (0, 1, 2, 3, 4, 5, 6), (1, 2), (3, 5, 6)])
+def test_sum_rank7(dims):  # tests/ut/test_reduce.py:61-71
+    x = np.random.default_rng(len(dims)).normal(-0.5, 0.5, [6, 4, 2, 5, 1, 3, 8]).astype(np.float32)
+    run_parity(lambda k, a: [k.sum(a, dims, True), k.sum(a, dims, False)], [x],
+               golden=[np.sum(x, dims, keepdims=True), np.sum(x, dims)], eps=1e-5)
+
+
+@pytest.mark.parametrize("dim", [1001, 1024])
+def test_sum_axis0_constant(dim):  # tests/ut/test_reduce.py:74-83
+    x = np.full([64, dim], 0.01, np.float32)
+    run_parity(lambda k, a: k.sum(a, (0,), False), [x], golden=np.full([dim], 0.64, np.float32))
+
+
+@pytest.mark.parametrize("shape,dims", [((4096, 40000), (1,)), ((1024, 1000), (0, 1)), ((32, 2048), (1,)), ((3, 20000), (0,)),
+                                        ((2048, 3201), (1,)), ((7, 5, 3), (1,)), ((128, 1), (0,)), ((1, 4096), (1,))])
+def test_sum_regression_shapes(shape, dims):  # tests/ut/test_reduce.py:86-108, tests/st/test_bugfix.py:20-53,98
+    x = np.random.default_rng(shape[0]).normal(-0.5, 0.5, shape).astype(np.float32)
+    run_parity(lambda k, a: k.sum(a, dims, False), [x], golden=np.sum(x.astype(np.float64), dims).astype(np.float32), eps=1e-4)
+
+
+@pytest.mark.parametrize("shape,dims", [((77, 513), (1,)), ((77, 513), (0,)), ((3, 1280, 7, 9), (0, 2, 3)), ((6, 4, 2, 5, 1, 3, 8), (1, 3))])
+@pytest.mark.parametrize("dt", [np.float32, np.float16])
+def test_max_min(shape, dims, dt):  # ops the reference's CUDA VM lacks; NumPy golden, exact (tests/ut/test_reduce.py:86-133)
+    x = np.random.default_rng(shape[0]).normal(-0.5, 0.5, shape).astype(dt)
+    run_parity(lambda k, a: [k.max(a, dims, True), k.min(a, dims, False)], [x],
+               golden=[np.max(x, dims, keepdims=True), np.min(x, dims)], eps=0)
+
+
+def test_fused_reduce_graphs():  # tests/ut/test_reduce.py:232-308
+    x = np.full([32, 2048], 0.01, np.float32)
+    run_parity(lambda k, a: k.sum(k.add(a, a), (1,), True), [x], golden=np.full([32, 1], 40.96, np.float32))
+    y = np.random.default_rng(1).uniform(0, 1, [1024, 1000]).astype(np.float32)
+    run_parity(lambda k, a: k.sum(k.copy(a), (0, 1), False), [y], golden=np.sum(y.astype(np.float64), (0, 1)).astype(np.float32), eps=1e-4)
+    b = np.random.default_rng(2).normal(0, 1, [1, 64, 1, 1]).astype(np.float32)
+    z = np.random.default_rng(3).normal(0, 1, [3, 64, 7, 9]).astype(np.float32)
+
+    def g(k, p, q):
+        s = k.add(k.broadcast(p, [3, 64, 7, 9]), q)
+        return [k.sum(s, (0, 2, 3), True), s]
+    run_parity(g, [b, z], ker="split", golden=[np.sum((b + z).astype(np.float64), (0, 2, 3), keepdims=True).astype(np.float32), b + z], eps=1e-4)
+
+
+def test_reduce_then_consumers_split_graph():  # tests/ut/test_eager_fusion.py:25-212 (graph-cutting cases)
+    rng = np.random.default_rng(4)
+    x = rng.normal(0, 1, [64, 300]).astype(np.float32)
+
+    def softmax(k, a):
+        m = k.max(a, (1,), True)
+        e = k.exp(k.sub(a, m))
+        return [k.div(e, k.sum(e, (1,), True)), m]
+    ex = np.exp(x - x.max(1, keepdims=True))
+    run_parity(softmax, [x], ker="split", golden=[ex / ex.sum(1, keepdims=True), x.max(1, keepdims=True)], eps=1e-5)
+
+    # a reduce result that two consumers and a store share; a dead node; a shared load
+    def g(k, a):
+        s = k.sum(a, (1,), True)
+        _dead = k.exp(a)
+        return [k.mul(a, s), k.add(s, 1.0), k.sub(a, k.mul(s, 1.0 / 300))]
+    s = x.astype(np.float64).sum(1, keepdims=True).astype(np.float32)
+    run_parity(g, [x], ker="split", golden=[x * s, s + 1, x - s * np.float32(1.0 / 300)], eps=1e-4)
+
+    # reduces over different axes of one input cannot share a kernel: the graph is cut, results still right
+    def g2(k, a):
+        return [k.sum(a, (0,), True), k.sum(a, (1,), True), k.add(k.sum(a, (1,), True), k.sum(k.mul(a, a), (1,), True))]
+    run_parity(g2, [x], ker="split", eps=1e-4,
+               golden=[x.astype(np.float64).sum(0, keepdims=True), x.astype(np.float64).sum(1, keepdims=True),
+                       (x.astype(np.float64).sum(1, keepdims=True) + (x.astype(np.float64) ** 2).sum(1, keepdims=True))])
+
+
+def test_reshape_graphs():  # tests/ut/test_reshape.py:24-160
+    for dims in [(2,), (1,)]:
+        b = np.full((10, 3, 1), 0.1, np.float32)
+        run_parity(lambda k, a: k.sum(k.reshape(k.broadcast(a, [10, 3, 4]), [1, 10, 12]), dims, True), [b], ker="split",
+                   golden=np.sum(np.broadcast_to(b, (10, 3, 4)).reshape(1, 10, 12), dims, keepdims=True))
+    x = np.full((16, 16), 81.0, np.float32)
+    run_parity(lambda k, a: k.sqrt(k.reshape(k.sqrt(a), [32, 8])), [x], ker="split", golden=np.full((32, 8), 3.0, np.float32))
+    run_parity(lambda k, a: k.cast(k.sqrt(k.reshape(k.sqrt(a), [32, 8])), "float16"), [x], ker="split", golden=np.full((32, 8), 3.0, np.float16))
+    rng = np.random.default_rng(5)
+    c, p, q = rng.choice([True, False], (3, 3)), np.full((9,), 1.0, np.float32), np.full((3, 3), 2.0, np.float32)
+    run_parity(lambda k, cc, pp, qq: k.select(cc, k.reshape(pp, [3, 3]), qq), [c, p, q], ker="split", golden=np.where(c, p.reshape(3, 3), q))
+    y = np.full([1, 8], 0.3, np.float32)
+    run_parity(lambda k, a: k.broadcast(k.reshape(k.broadcast(a, [10, 8]), [10, 1, 8]), [10, 4, 8]), [y], ker="split", golden=np.full([10, 4, 8], np.float32(0.3)))
+    z = np.full([10, 3, 4], 0.3, np.float32)
+    run_parity(lambda k, a: k.broadcast(k.reshape(a, [1, 10, 12]), [8, 10, 12]), [z], ker="split", golden=np.full([8, 10, 12], np.float32(0.3)))
+    a = rng.uniform(0.1, 1, (54, 89)).astype(np.float32)
+    run_parity(lambda k, v: k.add(k.sqrt(k.reshape(v, [89, 54])), k.reshape(k.reciprocal(v), [89, 54])), [a], ker="split",
+               golden=(np.sqrt(a) + np.reciprocal(a)).reshape(89, 54))
+
+
+@pytest.mark.parametrize("shape", [(13, 131), (128, 7), (5, 1023), (1, 1), (2, 3, 5, 7)])
+@pytest.mark.parametrize("dt", [np.float32, np.float16, np.int32, np.bool_])
+def test_unaligned_shapes(shape, dt):  # tests/ut/test_unalign.py:25-72, tests/ut/test_misc.py:26
+    rng = np.random.default_rng(shape[-1])
+    x = rng.normal(0, 10, shape).astype(dt)
+    y = rng.normal(0, 10, shape).astype(dt)
+    if dt == np.bool_:
+        run_parity(lambda k, a, b: [k.copy(a), k.logical_or(a, b)], [x, y], golden=[x, np.logical_or(x, y)])
+    else:
+        with np.errstate(over="ignore"):
+            run_parity(lambda k, a, b: [k.copy(a), k.mul(a, b)], [x, y], golden=[x, x * y], eps=0 if dt == np.int32 else None)
+
+
+def _dyn_sum_kernel():
+    t = Tester("vector:dyn")
+    x = t.load([1, 1, 4096], "float16")
+    y = t.load([1, 1, 4096], "float16")
+    s = t.add(x, y)
+    f = t.cast(s, "float32")
+    outs = [t.store(s), t.store(f), t.store(t.sum(t.mul(f, f), (2,), True))]
+    return t, (x, y), outs
+
+
+def test_dynamic_shapes():  # tests/ut/test_dynamic_shape.py:68-114,137-162 (closest reference test to BASELINE config 3)
+    t, (x, y), outs = _dyn_sum_kernel()
+    for rows in (2685, 2686, 2687, 1, 64):
+        np.random.seed(rows)
+        a = Tester.fast_random_normal(0, 1, [1, rows, 4096]).astype(np.float16)
+        b = Tester.fast_random_normal(0, 1, [1, rows, 4096]).astype(np.float16)
+        t.input(x, a)
+        t.input(y, b)
+        t.run()
+        s = a + b
+        assert np.array_equal(t.output(outs[0]), s)
+        assert np.array_equal(t.output(outs[1]), s.astype(np.float32))
+        want = np.sum(s.astype(np.float64) ** 2, 2, keepdims=True)
+        assert np.allclose(t.output(outs[2]), want, rtol=1e-4, atol=1e-4)
+
+
+def test_scalar_ref_updates():  # tests/ut/test_elemwise.py:500-532
+    t = Tester("vector:dyn")
+    x = t.load([1024], "float32")
+    sf = t.scalar()
+    si = t.scalar("int32" if False else t.cast.__self__ and 4)  # an int32 scalar reference
+    xi = t.load([1024], "int32")
+    o1 = t.store(t.mul(x, sf))
+    o2 = t.store(t.add(xi, si))
+    a = np.random.default_rng(0).normal(-10, 10, [1024]).astype(np.float32)
+    ai = np.random.default_rng(1).integers(-100, 100, [1024]).astype(np.int32)
+    for fv, iv in [(0.5, 3), (-2.25, -7), (10.0, 11111)]:
+        t.input(x, a)
+        t.input(xi, ai)
+        sf.update(fv)
+        si.update(iv)
+        t.run()
+        assert np.array_equal(t.output(o1), a * np.float32(fv))
+        assert np.array_equal(t.output(o2), ai + np.int32(iv))
+
+
+def test_zero_size():  # tests/ut/test_codegen.py:116-164
+    t = Tester("vector")
+    x = t.load(np.zeros([0, 16], np.float32))
+    s = t.store(t.sum(x, (0,), False))
+    e = t.store(t.add(x, 1.0))
+    t.run()
+    assert np.array_equal(t.output(s), np.zeros([16], np.float32))
+    assert t.output(e).shape == (0, 16)

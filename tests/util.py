@@ -1,0 +1,50 @@
+"""Shared parity harness: one graph-building function runs on the HIP path
+(dvm_amd.tester.Tester, through the C ABI) and on the CPU oracle
+(oracle.oracle.OracleKernel); outputs are compared with each other and, when
+given, with a NumPy golden."""
+import numpy as np
+
+from dvm_amd import DataType
+from dvm_amd.tester import Tester
+from oracle.oracle import OracleKernel
+
+DEFAULT_EPS = {int(DataType.float32): 1e-5, int(DataType.float16): 1e-3, int(DataType.bfloat16): 1e-2}
+
+
+def run_parity(build, arrays, dtypes=None, ker="vector", eps=None, golden=None, golden_eps=None):
+    """build(k, *inputs) -> value or list of values. Returns the HIP outputs."""
+    dtypes = dtypes or [None] * len(arrays)
+    t, o = Tester(ker), OracleKernel()
+    t_in = [t.load(a, d) for a, d in zip(arrays, dtypes)]
+    o_in = [o.load(a, d) for a, d in zip(arrays, dtypes)]
+    t_out, o_out = build(t, *t_in), build(o, *o_in)
+    if not isinstance(t_out, (list, tuple)):
+        t_out, o_out = [t_out], [o_out]
+    stores = [t.store(x) for x in t_out]
+    refs = [o.output(o.store(x)) for x in o_out]
+    t.run()
+    outs = []
+    for i, (s, ref) in enumerate(zip(stores, refs)):
+        out = t.output(s)
+        dt = int(s.dtype())
+        if dt == int(DataType.bfloat16):
+            out = Tester.convert_from_bf16(out)
+        assert out.shape == ref.shape, "output %d: shape %s vs oracle %s" % (i, out.shape, ref.shape)
+        if dt in (int(DataType.int32), int(DataType.bool)):
+            assert np.array_equal(out, ref), "output %d differs from the oracle (bit-exact required)\n%s" % (i, t.das())
+        else:
+            e = eps if eps is not None else DEFAULT_EPS[dt]
+            assert np.allclose(out.astype(np.float32), ref.astype(np.float32), rtol=e, atol=e, equal_nan=True), (
+                "output %d differs from the oracle beyond %g: max abs diff %g\n%s"
+                % (i, e, np.nanmax(np.abs(out.astype(np.float64) - ref.astype(np.float64))), t.das()))
+        outs.append(out)
+    if golden is not None:
+        g = golden if isinstance(golden, (list, tuple)) else [golden]
+        for i, (out, gi) in enumerate(zip(outs, g)):
+            if gi is None:
+                continue
+            dt = int(stores[i].dtype())
+            e = golden_eps if golden_eps is not None else (eps if eps is not None else DEFAULT_EPS.get(dt, 0))
+            assert np.allclose(out, gi, rtol=e, atol=e, equal_nan=True), (
+                "output %d differs from the NumPy golden beyond %g\n%s" % (i, e, t.das()))
+    return outs
