@@ -1,0 +1,193 @@
+"""Benchmark of the DVM hot path on one MI355X.
+
+Headline (BASELINE.json configs[1]): fused batch-norm forward with training statistics, fp32 NCHW
+[32,256,56,56], one launch of the vector VM. `value` is algorithmic GB/s: the tensor is read once
+and written once (2 x 102 760 448 B + 2 KB parameters = 205 522 944 B per step) over the wall time
+of K steps with inputs resident in HBM. The same JSON line carries the roofline figure of the kernel
+(HIP events on the launch stream), a CPU baseline (the C oracle on this box's host, one core) and,
+under "configs", the other BASELINE configs (latency / JIT microseconds / GB/s).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+METRIC = "fused-op HBM GB/s (% roofline) + matmul TFLOPS (% MFMA peak); JIT us/shape"
+
+
+def bn_graph(t, x, g, b, n_red, eps):
+    """mean / biased variance over N,H,W in one sweep (sum x, sum x^2, fp64 accumulation), then
+    y = x * scale + shift with per-channel scale = gamma / sqrt(var + eps), shift = beta - mean * scale."""
+    inv = 1.0 / n_red
+    mean = t.mul(t.sum(x, (0, 2, 3), True), inv)
+    ex2 = t.mul(t.sum(t.mul(x, x), (0, 2, 3), True), inv)
+    var = t.sub(ex2, t.mul(mean, mean))
+    scale = t.div(g, t.sqrt(t.add(var, eps)))
+    shift = t.sub(b, t.mul(mean, scale))
+    return t.add(t.mul(x, scale), shift)
+
+
+def bench_batchnorm(steps, warmup):
+    from dvm_amd.tester import Tester
+    n, c, h, w = 32, 256, 56, 56
+    rng = np.random.default_rng(1002)
+    x = rng.standard_normal([n, c, h, w], dtype=np.float32)
+    g = rng.uniform(0.5, 1.5, [1, c, 1, 1]).astype(np.float32)
+    b = rng.normal(0, 0.1, [1, c, 1, 1]).astype(np.float32)
+    t = Tester("split:dyn")
+    lx, lg, lb = t.load(x), t.load(g), t.load(b)
+    out = t.store(bn_graph(t, lx, lg, lb, n * h * w, 1e-5))
+    t.codegen()
+    jit_cold = t.jit_us()
+    t.codegen()
+    jit_warm = t.jit_us()
+    launches = t.num_launches()
+    for _ in range(warmup):
+        t.bare_run()
+    # K timed steps: asynchronous launches, one synchronisation at the end
+    from dvm_amd import _core
+    t0 = time.perf_counter()
+    for _ in range(steps - 1):
+        _core.PyKernel.run(t, sync=False)
+    _core.PyKernel.run(t, sync=True)
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / steps * 1e3
+    ev_min, ev_max, ev_mean = t.perf(warmup=3, iters=max(20, steps))
+    got = t.output(out)
+    alg_bytes = 2 * x.nbytes + g.nbytes + b.nbytes
+    # parity gate before any number counts
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean((0, 2, 3), keepdims=True)) / np.sqrt(x64.var((0, 2, 3), keepdims=True) + 1e-5) * g + b
+    err = float(np.max(np.abs(got - want) / (np.abs(want) + 1.0)))
+    if not np.allclose(got, want, rtol=1e-5, atol=1e-5):
+        raise RuntimeError("batch-norm result differs from the NumPy golden: max rel err %g" % err)
+    return {
+        "x": x, "g": g, "b": b, "alg_bytes": alg_bytes, "ms_per_step": ms_per_step, "kernel_us_mean": ev_mean,
+        "kernel_us_min": ev_min, "jit_us_cold": jit_cold, "jit_us_warm": jit_warm, "launches": launches, "max_rel_err": err,
+    }
+
+
+def cpu_baseline_batchnorm(x, g, b, alg_bytes):
+    from oracle import oracle as ora
+    ora.batchnorm_nchw(x[:2], g, b, 1e-5)  # warm-up on a slice
+    reps = 3
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        ora.batchnorm_nchw(x, g, b, 1e-5)
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": round(alg_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": "full [32,256,56,56] tensor, scalar C oracle (oracle/dvm_oracle.c ora_batchnorm_nchw), mean of %d runs, %.2f s each" % (reps, dt)}
+
+
+def bench_add():
+    """configs[0]: fp32 [32,32] add; launch latency and JIT microseconds (a plumbing check)."""
+    from dvm_amd.tester import Tester
+    x, y = np.full([32, 32], 0.1, np.float32), np.full([32, 32], 0.3, np.float32)
+    t = Tester("split:dyn")
+    out = t.store(t.add(t.load(x), t.load(y)))
+    t.codegen()
+    cold = t.jit_us()
+    t.codegen()
+    warm = t.jit_us()
+    t.run()
+    assert np.array_equal(t.output(out), x + y)
+    mn, _, mean = t.perf(warmup=3, iters=50)
+    return {"kernel_us_mean": round(mean, 2), "kernel_us_min": round(mn, 2), "jit_us_cold": round(cold, 2), "jit_us_warm": round(warm, 2)}
+
+
+def bench_rmsnorm(calls=200):
+    """configs[2]: bf16 residual-add + RMSNorm + cast, R ~ U{1..8192} per call, 200 seeded calls."""
+    from dvm_amd.tester import Tester
+    rng = np.random.default_rng(1003)
+    rows = rng.integers(1, 8193, calls)
+    rmax = int(rows.max())
+    xs = Tester.convert_to_bf16(rng.standard_normal([rmax, 4096], dtype=np.float32))
+    rs = Tester.convert_to_bf16(rng.standard_normal([rmax, 4096], dtype=np.float32))
+    wv = rng.uniform(0.9, 1.1, [4096]).astype(np.float32)
+    t = Tester("split:dyn")
+    x, r, w = t.load([1, 4096], "bfloat16"), t.load([1, 4096], "bfloat16"), t.load([4096], "float32")
+    hf = t.cast(t.add(x, r), "float32")
+    ss = t.sum(t.mul(hf, hf), (1,), True)
+    rstd = t.div(1.0, t.sqrt(t.add(t.mul(ss, 1.0 / 4096), 1e-6)))
+    out = t.store(t.cast(t.mul(t.mul(hf, rstd), w), "bfloat16"))
+    t.input(w, wv)
+    jit, gbs, big_gbs, big_frac = [], [], [], []
+    total_bytes = 0
+    total_us = 0.0
+    checked = 0
+    for i, R in enumerate(rows):
+        R = int(R)
+        t.input(x, xs[:R])
+        t.input(r, rs[:R])
+        t.codegen()
+        jit.append(t.jit_us())
+        mn, _, mean = t.perf(warmup=1, iters=5)
+        nbytes = 24576 * R + 16384
+        total_bytes += nbytes
+        total_us += mean
+        gbs.append(nbytes / mean / 1e3)
+        if R >= 512:
+            big_gbs.append(nbytes / mean / 1e3)
+        if i % 40 == 0:  # parity spot checks against the NumPy golden (1e-2)
+            got = Tester.convert_from_bf16(t.output(out))
+            hh = Tester.convert_from_bf16(Tester.convert_to_bf16(Tester.convert_from_bf16(xs[:R]) + Tester.convert_from_bf16(rs[:R]))).astype(np.float64)
+            want = hh / np.sqrt((hh * hh).mean(1, keepdims=True) + 1e-6) * wv
+            if not np.allclose(got, want, rtol=1e-2, atol=1e-2):
+                raise RuntimeError("RMSNorm result differs from the NumPy golden at R=%d" % R)
+            checked += 1
+    jit_sorted = sorted(jit[1:])
+    return {
+        "calls": calls, "sum_alg_GB": round(total_bytes / 1e9, 3), "aggregate_GBps": round(total_bytes / total_us / 1e3, 1),
+        "aggregate_frac_of_8TBps": round(total_bytes / total_us / 1e3 / HBM_PEAK_GBS, 4),
+        "R>=512_median_GBps": round(float(np.median(big_gbs)), 1), "R>=512_median_frac": round(float(np.median(big_gbs)) / HBM_PEAK_GBS, 4),
+        "jit_us_first": round(jit[0], 2), "jit_us_median": round(jit_sorted[len(jit_sorted) // 2], 2), "jit_us_max": round(jit_sorted[-1], 2),
+        "launches_per_call": t.num_launches(), "parity_checked_calls": checked,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
+    ap.add_argument("--only-headline", action="store_true", help="omit the other BASELINE configs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the DVM hot path is a single-device operator JIT (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    import dvm_amd as dvm
+    if not dvm.Device.available():
+        print("bench.py needs an MI355X and the built HIP device layer (dvm_amd/lib/libdvm_hip.so)", file=sys.stderr)
+        sys.exit(1)
+    bn = bench_batchnorm(args.steps, args.warmup)
+    value = bn["alg_bytes"] / (bn["ms_per_step"] * 1e-3) / 1e9
+    achieved = bn["alg_bytes"] / (bn["kernel_us_mean"] * 1e-6) / 1e9
+    line = {
+        "metric": METRIC, "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(bn["ms_per_step"], 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "BASELINE configs[1]: fused batch-norm forward (training statistics), fp32 NCHW [32,256,56,56], eps=1e-5, one launch",
+                   "algorithmic_bytes_per_step": bn["alg_bytes"], "launches_per_step": bn["launches"],
+                   "jit_us_cold": round(bn["jit_us_cold"], 2), "jit_us_warm": round(bn["jit_us_warm"], 2),
+                   "parity_max_rel_err_vs_numpy_f64": bn["max_rel_err"]},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "dvm_vm_vec_rx", "kernel_us_mean": round(bn["kernel_us_mean"], 2), "kernel_us_min": round(bn["kernel_us_min"], 2)},
+    }
+    if not args.skip_cpu:
+        line["cpu_baseline"] = cpu_baseline_batchnorm(bn["x"], bn["g"], bn["b"], bn["alg_bytes"])
+    if not args.only_headline:
+        line["configs"] = {"add_fp32_32x32": bench_add(), "residual_rmsnorm_bf16_dynamic": bench_rmsnorm()}
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
