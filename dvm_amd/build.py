@@ -15,8 +15,13 @@ CSRC = os.path.join(ROOT, "csrc")
 LIB = os.path.join(ROOT, "lib")
 OBJ = os.path.join(LIB, "obj")
 
+# The interpreter kernels branch on wave-uniform values only (every per-lane condition lives in an
+# out-of-line helper), so the CFG structurizer is told to leave uniform regions alone: the
+# dispatch then compiles to real scalar branches instead of a chain of predicate checks.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
-             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+             "-mllvm", "-structurizecfg-skip-uniform-regions=true",
+             "-mllvm", "-structurizecfg-relaxed-uniform-regions=true"]
 HOST_FLAGS = ["-std=c++17", "-O2", "-fPIC", "-fvisibility=hidden", "-Wall"]
 
 

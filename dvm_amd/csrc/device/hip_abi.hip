@@ -32,7 +32,7 @@ __global__ void dvm_fill_u32_kernel(uint32_t *dst, uint32_t value, size_t n) {
 // waves per SIMD each interpreter kernel fits at (from its VGPR count)
 uint32_t kernel_waves_per_simd(uint64_t kind) {
   switch (kind) {
-    case VS_POINTWISE: return 6;
+    case VS_POINTWISE: return 5;
     case VS_REDX: return 5;
     case VS_REDY: return 4;
     default: return 2;

@@ -69,6 +69,24 @@ __device__ __forceinline__ void apply_rnd(Acc &a, uint32_t rnd) {
   }
 }
 
+// Library functions with internal (per-lane) branches stay out of the interpreter loop.
+__device__ __attribute__((noinline)) vf8 slab_exp(vf8 x) {
+  FOR_E x[e] = expf(x[e]);
+  return x;
+}
+__device__ __attribute__((noinline)) vf8 slab_log(vf8 x) {
+  FOR_E x[e] = logf(x[e]);
+  return x;
+}
+__device__ __attribute__((noinline)) vf8 slab_pow(vf8 x, vf8 y) {
+  FOR_E x[e] = powf(x[e], y[e]);
+  return x;
+}
+__device__ __attribute__((noinline)) vf8 slab_sqrt(vf8 x) {
+  FOR_E x[e] = sqrtf(x[e]);
+  return x;
+}
+
 // ---- memory operands -------------------------------------------------------
 
 __device__ __forceinline__ float elem_load(uint64_t base, uint32_t dtype, uint64_t off) {
@@ -129,96 +147,136 @@ __device__ __forceinline__ void slab_store_slow(const VMemDesc &m, uint64_t off,
   }
 }
 
-// Loads the U slabs of operand `m`. nvp holds 4 bits per slab: elements inside the tensor (0 = skip).
-__device__ __forceinline__ void mem_load(const VMemDesc &m, const uint64_t (&off)[U], uint32_t nvp, Acc &out) {
-  const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
-  const uint32_t dtype = m.dtype;
-  if (fast && nvp == kAllFull) {  // whole instruction on the wide path: issue every load before any use
-    if (dtype == VDT_F32 || dtype == VDT_I32) {
-      vf4 a[U], b[U];
-      FOR_U {
-        const DVM_GLOBAL vf4 *p = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off[u] * 4);
-        a[u] = p[0];
-        b[u] = p[1];
-      }
-      FOR_U out.v[u] = __builtin_shufflevector(a[u], b[u], 0, 1, 2, 3, 4, 5, 6, 7);
-    } else if (dtype == VDT_BF16) {
-      vu4 a[U];
-      FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(m.addr + off[u] * 2);
-      FOR_U {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          out.v[u][2 * i] = __uint_as_float(a[u][i] << 16);
-          out.v[u][2 * i + 1] = __uint_as_float(a[u][i] & 0xffff0000u);
-        }
-      }
-    } else if (dtype == VDT_F16) {
-      vh8 a[U];
-      FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off[u] * 2);
-      FOR_U out.v[u] = __builtin_convertvector(a[u], vf8);
-    } else {
-      vu2 a[U];
-      FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vu2 *>(m.addr + off[u]);
-      FOR_U {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          out.v[u][e] = ((a[u][0] >> (8 * e)) & 0xffu) ? 1.0f : 0.0f;
-          out.v[u][e + 4] = ((a[u][1] >> (8 * e)) & 0xffu) ? 1.0f : 0.0f;
-        }
-      }
-    }
-    return;
-  }
+// The interpreter loop must contain uniform branches only: one divergent branch anywhere in it makes
+// the compiler linearise the whole dispatch (every handler guarded by predicate checks, register
+// copies on every path). Per-lane conditions therefore live in these out-of-line slow paths, which
+// take and return the accumulator by value (VGPRs), and the loop picks between the wide path and
+// them with a wave-wide vote.
+__device__ __forceinline__ bool wave_all(bool c) { return __builtin_amdgcn_ballot_w64(!c) == 0; }
+
+struct Offs {
+  uint64_t v[U];
+};
+
+__device__ __attribute__((noinline)) Acc mem_load_slow(uint64_t addr, uint32_t dtype, uint32_t flags, Offs off, uint32_t nvp) {
+  VMemDesc m;
+  m.addr = addr;
+  m.dtype = dtype;
+  m.flags = flags;
+  const bool fast = (flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
+  Acc out;
   FOR_U {
     const int nv = static_cast<int>((nvp >> (4 * u)) & 0xfu);
     out.v[u] = 0.0f;
     if (nv == 0) continue;
     if (fast && nv == E) {
       if (dtype == VDT_F32 || dtype == VDT_I32) {
-        const DVM_GLOBAL vf4 *p = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off[u] * 4);
+        const DVM_GLOBAL vf4 *p = reinterpret_cast<const DVM_GLOBAL vf4 *>(addr + off.v[u] * 4);
         out.v[u] = __builtin_shufflevector(p[0], p[1], 0, 1, 2, 3, 4, 5, 6, 7);
         continue;
       }
       if (dtype == VDT_F16) {
-        out.v[u] = __builtin_convertvector(*reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off[u] * 2), vf8);
+        out.v[u] = __builtin_convertvector(*reinterpret_cast<const DVM_GLOBAL vh8 *>(addr + off.v[u] * 2), vf8);
         continue;
       }
     }
-    out.v[u] = slab_load_slow(m, off[u], nv);
+    out.v[u] = slab_load_slow(m, off.v[u], nv);
   }
+  return out;
 }
 
-__device__ __forceinline__ void mem_store(const VMemDesc &m, const uint64_t (&off)[U], uint32_t nvp, const Acc &in) {
-  const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
-  const uint32_t dtype = m.dtype;
+__device__ __attribute__((noinline)) void mem_store_slow(uint64_t addr, uint32_t dtype, uint32_t flags, Offs off, uint32_t nvp, Acc in) {
+  VMemDesc m;
+  m.addr = addr;
+  m.dtype = dtype;
+  m.flags = flags;
   FOR_U {
     const int nv = static_cast<int>((nvp >> (4 * u)) & 0xfu);
     if (nv == 0) continue;
-    if (fast && nv == E) {
-      if (dtype == VDT_F32 || dtype == VDT_I32) {
-        DVM_GLOBAL vf4 *p = reinterpret_cast<DVM_GLOBAL vf4 *>(m.addr + off[u] * 4);
-        p[0] = __builtin_shufflevector(in.v[u], in.v[u], 0, 1, 2, 3);
-        p[1] = __builtin_shufflevector(in.v[u], in.v[u], 4, 5, 6, 7);
-      } else if (dtype == VDT_BF16) {
-        vu4 a;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-          a[i] = f32_to_bf16_bits(in.v[u][2 * i]) | (f32_to_bf16_bits(in.v[u][2 * i + 1]) << 16);
-        *reinterpret_cast<DVM_GLOBAL vu4 *>(m.addr + off[u] * 2) = a;
-      } else if (dtype == VDT_F16) {
-        *reinterpret_cast<DVM_GLOBAL vh8 *>(m.addr + off[u] * 2) = __builtin_convertvector(in.v[u], vh8);
-      } else {
-        vu2 a = 0u;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          a[0] |= (in.v[u][e] != 0.0f ? 1u : 0u) << (8 * e);
-          a[1] |= (in.v[u][e + 4] != 0.0f ? 1u : 0u) << (8 * e);
-        }
-        *reinterpret_cast<DVM_GLOBAL vu2 *>(m.addr + off[u]) = a;
-      }
-    } else {
-      slab_store_slow(m, off[u], nv, in.v[u]);
+    slab_store_slow(m, off.v[u], nv, in.v[u]);
+  }
+}
+
+// Wide path of a load: every lane of the wave owns U full, aligned slabs. All loads are issued before any use.
+__device__ __forceinline__ void mem_load_wide(const VMemDesc &m, const Offs &off, Acc &out) {
+  const uint32_t dtype = m.dtype;
+  if (dtype == VDT_F32 || dtype == VDT_I32) {
+    vf4 a[U], b[U];
+    FOR_U {
+      const DVM_GLOBAL vf4 *p = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off.v[u] * 4);
+      a[u] = p[0];
+      b[u] = p[1];
     }
+    FOR_U out.v[u] = __builtin_shufflevector(a[u], b[u], 0, 1, 2, 3, 4, 5, 6, 7);
+  } else if (dtype == VDT_BF16) {
+    vu4 a[U];
+    FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(m.addr + off.v[u] * 2);
+    FOR_U {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        out.v[u][2 * i] = __uint_as_float(a[u][i] << 16);
+        out.v[u][2 * i + 1] = __uint_as_float(a[u][i] & 0xffff0000u);
+      }
+    }
+  } else if (dtype == VDT_F16) {
+    vh8 a[U];
+    FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off.v[u] * 2);
+    FOR_U out.v[u] = __builtin_convertvector(a[u], vf8);
+  } else {
+    vu2 a[U];
+    FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vu2 *>(m.addr + off.v[u]);
+    FOR_U {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        out.v[u][e] = ((a[u][0] >> (8 * e)) & 0xffu) ? 1.0f : 0.0f;
+        out.v[u][e + 4] = ((a[u][1] >> (8 * e)) & 0xffu) ? 1.0f : 0.0f;
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ void mem_store_wide(const VMemDesc &m, const Offs &off, const Acc &in) {
+  const uint32_t dtype = m.dtype;
+  FOR_U {
+    if (dtype == VDT_F32 || dtype == VDT_I32) {
+      DVM_GLOBAL vf4 *p = reinterpret_cast<DVM_GLOBAL vf4 *>(m.addr + off.v[u] * 4);
+      p[0] = __builtin_shufflevector(in.v[u], in.v[u], 0, 1, 2, 3);
+      p[1] = __builtin_shufflevector(in.v[u], in.v[u], 4, 5, 6, 7);
+    } else if (dtype == VDT_BF16) {
+      vu4 a;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        a[i] = f32_to_bf16_bits(in.v[u][2 * i]) | (f32_to_bf16_bits(in.v[u][2 * i + 1]) << 16);
+      *reinterpret_cast<DVM_GLOBAL vu4 *>(m.addr + off.v[u] * 2) = a;
+    } else if (dtype == VDT_F16) {
+      *reinterpret_cast<DVM_GLOBAL vh8 *>(m.addr + off.v[u] * 2) = __builtin_convertvector(in.v[u], vh8);
+    } else {
+      vu2 a = 0u;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        a[0] |= (in.v[u][e] != 0.0f ? 1u : 0u) << (8 * e);
+        a[1] |= (in.v[u][e + 4] != 0.0f ? 1u : 0u) << (8 * e);
+      }
+      *reinterpret_cast<DVM_GLOBAL vu2 *>(m.addr + off.v[u]) = a;
+    }
+  }
+}
+
+__device__ __forceinline__ void mem_load(const VMemDesc &m, const Offs &off, uint32_t nvp, Acc &out) {
+  const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
+  if (fast && wave_all(nvp == kAllFull)) {
+    mem_load_wide(m, off, out);
+  } else {
+    out = mem_load_slow(m.addr, m.dtype, m.flags, off, nvp);
+  }
+}
+
+__device__ __forceinline__ void mem_store(const VMemDesc &m, const Offs &off, uint32_t nvp, const Acc &in) {
+  const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
+  if (fast && wave_all(nvp == kAllFull)) {
+    mem_store_wide(m, off, in);
+  } else {
+    mem_store_slow(m.addr, m.dtype, m.flags, off, nvp, in);
   }
 }
 
@@ -257,42 +315,56 @@ __device__ __forceinline__ void red_init(RedAcc<SCHED> &r, uint32_t kind) {
   for (int e = 0; e < (SCHED == VS_REDY ? E : 1); ++e) r.v[e] = idv;
 }
 
-// fp32 combine of the elements of one slab (NaN-propagating for max/min).
-__device__ __forceinline__ float red_combine_f32(uint32_t kind, float r, float v) {
-  if (kind == VR_SUM) return r + v;
-  if (kind == VR_MAX) return (v > r || v != v) ? v : r;
+// One reduce step for a fixed kind; the kind is resolved once per instruction, outside the element loops.
+template <int KIND, typename T>
+__device__ __forceinline__ T red_op(T r, T v) {
+  if constexpr (KIND == VR_SUM) return r + v;
+  if constexpr (KIND == VR_MAX) return (v > r || v != v) ? v : r;  // NaN propagates, as NumPy's max/min
   return (v < r || v != v) ? v : r;
 }
 
-template <int SCHED>
-__device__ __forceinline__ void red_accumulate(RedAcc<SCHED> &r, uint32_t kind, const Acc &x, uint32_t nvp) {
+template <int SCHED, int KIND>
+__device__ __forceinline__ void red_accumulate_k(RedAcc<SCHED> &r, const Acc &x, uint32_t nvp) {
+  constexpr float idv = KIND == VR_SUM ? 0.0f : (KIND == VR_MAX ? -__builtin_huge_valf() : __builtin_huge_valf());
   FOR_U {
     const int nv = static_cast<int>((nvp >> (4 * u)) & 0xfu);
     if constexpr (SCHED == VS_REDY) {
       FOR_E {
-        if (e < nv) r.v[e] = red_combine(kind, r.v[e], static_cast<double>(x.v[u][e]));
+        const double t = red_op<KIND>(r.v[e], static_cast<double>(x.v[u][e]));
+        r.v[e] = e < nv ? t : r.v[e];
       }
     } else {
-      // The 8 elements of a slab are combined pairwise in fp32 (the blocking NumPy's
-      // float32 sum uses as well), every further step accumulates in fp64.
-      const float idv = static_cast<float>(red_identity(kind));
+      // The 8 elements of a slab are combined pairwise in fp32 (the blocking NumPy's float32 sum
+      // uses as well); every further step accumulates in fp64.
       float d[E];
-      FOR_E d[e] = e < nv ? x.v[u][e] : idv;
+      FOR_E d[e] = e < nv ? x.v[u][e] : idv;  // selects, not branches
 #pragma unroll
       for (int w = 1; w < E; w <<= 1)
 #pragma unroll
-        for (int e = 0; e + w < E; e += 2 * w) d[e] = red_combine_f32(kind, d[e], d[e + w]);
-      if (nv > 0) r.v[0] = red_combine(kind, r.v[0], static_cast<double>(d[0]));
+        for (int e = 0; e + w < E; e += 2 * w) d[e] = red_op<KIND>(d[e], d[e + w]);
+      const double t = red_op<KIND>(r.v[0], static_cast<double>(d[0]));
+      r.v[0] = nv > 0 ? t : r.v[0];
     }
+  }
+}
+
+template <int SCHED>
+__device__ __forceinline__ void red_accumulate(RedAcc<SCHED> &r, uint32_t kind, const Acc &x, uint32_t nvp) {
+  if (kind == VR_SUM) {
+    red_accumulate_k<SCHED, VR_SUM>(r, x, nvp);
+  } else if (kind == VR_MAX) {
+    red_accumulate_k<SCHED, VR_MAX>(r, x, nvp);
+  } else {
+    red_accumulate_k<SCHED, VR_MIN>(r, x, nvp);
   }
 }
 
 // Combines one slot's partials across the lanes that share an output; every
 // one of those lanes ends up with the result.
 template <int SCHED>
-__device__ __forceinline__ void red_finalize(RedAcc<SCHED> &r, uint32_t rk, uint32_t tlog, bool team_is_block,
-                                             uint32_t tid, uint32_t nthreads, uint32_t k_local, uint32_t r_local,
-                                             double *scratch) {
+__device__ __attribute__((noinline)) RedAcc<SCHED> red_finalize(RedAcc<SCHED> r, uint32_t rk, uint32_t tlog, bool team_is_block,
+                                                                uint32_t tid, uint32_t nthreads, uint32_t k_local,
+                                                                uint32_t r_local, double *scratch) {
   if constexpr (SCHED == VS_REDX) {
     double t = r.v[0];
     const uint32_t span = team_is_block ? 64u : (1u << tlog);
@@ -319,6 +391,7 @@ __device__ __forceinline__ void red_finalize(RedAcc<SCHED> &r, uint32_t rk, uint
       }
     }
   }
+  return r;
 }
 
 // ---- S registers (one float per lane, VGPRs) -----------------------------------
@@ -460,8 +533,14 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   // dependent scalar-memory round trip per access, so each workgroup copies it
   // into local memory once and decodes from there.
   {
+    // uniform trip count and clamped indices: no per-lane branch (lanes past the end rewrite the last word)
     const uint32_t *src = reinterpret_cast<const uint32_t *>(p.w);
-    for (uint32_t i = threadIdx.x; i < DVM_PARAM_BYTES / 4; i += blockDim.x) prog32[i] = src[i];
+    const uint32_t trips = (DVM_PARAM_BYTES / 4 + blockDim.x - 1) / blockDim.x;
+    for (uint32_t t = 0; t < trips; ++t) {
+      uint32_t i = t * blockDim.x + threadIdx.x;
+      i = i < DVM_PARAM_BYTES / 4 ? i : DVM_PARAM_BYTES / 4 - 1;
+      prog32[i] = src[i];
+    }
     __syncthreads();
   }
   VVecHeader h;
@@ -513,11 +592,14 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       nvp_out = 0;
       FOR_U {
         const uint32_t ku = kidx + u * nthreads;
-        const uint32_t nv = ku < h.n_kidx ? group_valid(ku, h.kdims, h.n_kdim, h.inner_extent) : 0u;
+        // computed for a clamped index and masked afterwards: a select, never a per-lane branch
+        const uint32_t in_range = ku < h.n_kidx ? 0xfu : 0u;
+        const uint32_t nv = group_valid(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, h.inner_extent) & in_range;
         nvp_out |= nv << (4 * u);
       }
     } else {
-      const uint32_t nv = !kvalid ? 0u : (inner_red ? 1u : group_valid(kidx, h.kdims, h.n_kdim, h.inner_extent));
+      const uint32_t nv_in = inner_red ? 1u : group_valid(kvalid ? kidx : 0u, h.kdims, h.n_kdim, h.inner_extent);
+      const uint32_t nv = nv_in & (kvalid ? 0xfu : 0u);
       nvp_out = nv * kAllOnes;
     }
 
@@ -536,26 +618,78 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       const uint32_t sub = (w0 >> 8) & 0xffu, a = w0 >> 24;
 
       if (op >= VOP_SRC_BASE) {
-        // ---- fetch the source operand ----
-        Acc src;
         const uint32_t kind = (w0 >> 16) & 0xfu;
+        // ---- scalar source (immediate or S register): no need to widen it to U*E values ----
+        if ((kind == VK_IMM || kind == VK_SREG) && (op == VOP_BINF || op == VOP_BINI || op == VOP_CMP)) {
+          const float sv = kind == VK_IMM ? __uint_as_float(imm) : sreg_read(sr, a);
+          if (op == VOP_BINF) {
+            switch (sub & 0x3fu) {
+              case VB_ADD: FOR_U acc.v[u] = acc.v[u] + sv; break;
+              case VB_SUB: FOR_U acc.v[u] = acc.v[u] - sv; break;
+              case VB_RSUB: FOR_U acc.v[u] = sv - acc.v[u]; break;
+              case VB_MUL: FOR_U acc.v[u] = acc.v[u] * sv; break;
+              case VB_DIV: FOR_U acc.v[u] = acc.v[u] / sv; break;
+              case VB_RDIV: FOR_U acc.v[u] = sv / acc.v[u]; break;
+              case VB_MIN: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] < sv ? acc.v[u][e] : sv; break;
+              case VB_MAX: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] > sv ? acc.v[u][e] : sv; break;
+              case VB_AND: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f && sv != 0.0f) ? 1.0f : 0.0f; break;
+              case VB_OR: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f || sv != 0.0f) ? 1.0f : 0.0f; break;
+              case VB_POW: FOR_U acc.v[u] = slab_pow(acc.v[u], vf8(sv)); break;
+              default: FOR_U acc.v[u] = slab_pow(vf8(sv), acc.v[u]); break;
+            }
+            apply_rnd(acc, (w0 >> 20) & 0x3u);
+          } else if (op == VOP_BINI) {
+            const uint32_t si = __float_as_uint(sv);
+            switch (sub & 0x3fu) {
+              case VBI_ADD: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(acc.v[u][e]) + si); break;
+              case VBI_SUB: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(acc.v[u][e]) - si); break;
+              case VBI_RSUB: FOR_U FOR_E acc.v[u][e] = __uint_as_float(si - __float_as_uint(acc.v[u][e])); break;
+              case VBI_MUL: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(acc.v[u][e]) * si); break;
+              case VBI_MIN: FOR_U FOR_E acc.v[u][e] = __int_as_float(min(__float_as_int(acc.v[u][e]), static_cast<int32_t>(si))); break;
+              default: FOR_U FOR_E acc.v[u][e] = __int_as_float(max(__float_as_int(acc.v[u][e]), static_cast<int32_t>(si))); break;
+            }
+          } else {
+            const int32_t si = __float_as_int(sv);
+            switch (sub & 0x3fu) {
+              case VCMP_EQ: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] == sv ? 1.0f : 0.0f; break;
+              case VCMP_NE: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] != sv ? 1.0f : 0.0f; break;
+              case VCMP_GT: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] > sv ? 1.0f : 0.0f; break;
+              case VCMP_GE: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] >= sv ? 1.0f : 0.0f; break;
+              case VCMP_LT: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] < sv ? 1.0f : 0.0f; break;
+              case VCMP_LE: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] <= sv ? 1.0f : 0.0f; break;
+              case VCMP_INT + VCMP_EQ: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) == si ? 1 : 0); break;
+              case VCMP_INT + VCMP_NE: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) != si ? 1 : 0); break;
+              case VCMP_INT + VCMP_GT: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) > si ? 1 : 0); break;
+              case VCMP_INT + VCMP_GE: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) >= si ? 1 : 0); break;
+              case VCMP_INT + VCMP_LT: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) < si ? 1 : 0); break;
+              default: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) <= si ? 1 : 0); break;
+            }
+          }
+          continue;
+        }
+        // ---- fetch a full-width source operand ----
+        Acc src;
         if (kind == VK_MEM) {
           const VMemDesc m = load_desc(prog32, mem_off, a);
-          uint64_t off[U];
+          Offs off;
           if constexpr (SCHED == VS_POINTWISE) {
             FOR_U {
               const uint32_t ku = kidx + u * nthreads;
-              off[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
+              off.v[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
             }
           } else {
             const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
             FOR_U {
-              off[u] = koff;
+              off.v[u] = koff;
               if (in_sweep) {
                 const uint32_t ru = ridx + u * r_step;
-                off[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+                off.v[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
               }
             }
+          }
+          if (op == VOP_LD) {
+            mem_load(m, off, nvp, acc);
+            continue;
           }
           mem_load(m, off, nvp, src);
         } else if (kind == VK_SREG) {
@@ -569,11 +703,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
         } else {
           src = acc;
         }
-
         switch (op) {
-          case VOP_LD:
-            acc = src;
-            break;
           case VOP_BINF: {
             switch (sub & 0x3fu) {
               case VB_ADD: FOR_U acc.v[u] = acc.v[u] + src.v[u]; break;
@@ -587,8 +717,8 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               case VB_MAX: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] > src.v[u][e] ? acc.v[u][e] : src.v[u][e]; break;
               case VB_AND: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f && src.v[u][e] != 0.0f) ? 1.0f : 0.0f; break;
               case VB_OR: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f || src.v[u][e] != 0.0f) ? 1.0f : 0.0f; break;
-              case VB_POW: FOR_U FOR_E acc.v[u][e] = powf(acc.v[u][e], src.v[u][e]); break;
-              default: FOR_U FOR_E acc.v[u][e] = powf(src.v[u][e], acc.v[u][e]); break;
+              case VB_POW: FOR_U acc.v[u] = slab_pow(acc.v[u], src.v[u]); break;
+              default: FOR_U acc.v[u] = slab_pow(src.v[u], acc.v[u]); break;
             }
             apply_rnd(acc, (w0 >> 20) & 0x3u);
             break;
@@ -657,20 +787,20 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
           break;
         case VOP_ST: {
           const VMemDesc m = load_desc(prog32, mem_off, a);
-          uint64_t off[U];
+          Offs off;
           uint32_t nvs = nvp;
           if constexpr (SCHED == VS_POINTWISE) {
             FOR_U {
               const uint32_t ku = kidx + u * nthreads;
-              off[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
+              off.v[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
             }
           } else {
             const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
             FOR_U {
-              off[u] = koff;
+              off.v[u] = koff;
               if (in_sweep) {
                 const uint32_t ru = ridx + u * r_step;
-                off[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+                off.v[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
               }
             }
             if (!in_sweep) nvs = r_local == 0 ? (nvp & 0xfu) : 0u;  // one lane per output, one slab
@@ -680,10 +810,10 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
         }
         case VOP_UN: {
           switch (sub) {
-            case VU_SQRT: FOR_U FOR_E acc.v[u][e] = sqrtf(acc.v[u][e]); break;
+            case VU_SQRT: FOR_U acc.v[u] = slab_sqrt(acc.v[u]); break;
             case VU_ABS: FOR_U FOR_E acc.v[u][e] = fabsf(acc.v[u][e]); break;
-            case VU_LOG: FOR_U FOR_E acc.v[u][e] = logf(acc.v[u][e]); break;
-            case VU_EXP: FOR_U FOR_E acc.v[u][e] = expf(acc.v[u][e]); break;
+            case VU_LOG: FOR_U acc.v[u] = slab_log(acc.v[u]); break;
+            case VU_EXP: FOR_U acc.v[u] = slab_exp(acc.v[u]); break;
             case VU_ISFINITE: FOR_U FOR_E acc.v[u][e] = isfinite(acc.v[u][e]) ? 1.0f : 0.0f; break;
             case VU_ROUND: FOR_U FOR_E acc.v[u][e] = rintf(acc.v[u][e]); break;
             case VU_FLOOR: FOR_U FOR_E acc.v[u][e] = floorf(acc.v[u][e]); break;
@@ -744,8 +874,8 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             } else {
               in_sweep = false;
               const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
-              if (k0 <= VR_MIN) red_finalize<SCHED>(racc0, k0, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
-              if (k1 <= VR_MIN) red_finalize<SCHED>(racc1, k1, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
+              if (k0 <= VR_MIN) racc0 = red_finalize<SCHED>(racc0, k0, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
+              if (k1 <= VR_MIN) racc1 = red_finalize<SCHED>(racc1, k1, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
             }
             break;
           }
@@ -770,8 +900,9 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             nvp = 0;
             FOR_U {
               const uint32_t ru = ridx + u * r_step;
-              uint32_t nv = 0;
-              if (kvalid && ru < h.n_ridx) nv = inner_red ? group_valid(ru, h.rdims, h.n_rdim, h.inner_extent) : (nvp_out & 0xfu);
+              const bool ok = kvalid && ru < h.n_ridx;
+              uint32_t nv = inner_red ? group_valid(ok ? ru : 0u, h.rdims, h.n_rdim, h.inner_extent) : (nvp_out & 0xfu);
+              nv &= ok ? 0xfu : 0u;
               nvp |= nv << (4 * u);
             }
           } else {
