@@ -11,6 +11,12 @@
 extern "C" __global__ void dvm_vm_vec_pw(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_rx(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_ry(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_bf16_big(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_f16_big(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_bf16_mid(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_f16_mid(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_bf16_small(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_f16_small(const VmParam p);
 
 namespace {
 
@@ -60,7 +66,13 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
   g_dev.lds_per_wg = static_cast<uint32_t>(prop.sharedMemPerBlock);
   // gfx950 lets one workgroup use the CU's whole 160 KB; the kernels must opt in.
   const void *kernels[] = {reinterpret_cast<const void *>(dvm_vm_vec_pw), reinterpret_cast<const void *>(dvm_vm_vec_rx),
-                           reinterpret_cast<const void *>(dvm_vm_vec_ry)};
+                           reinterpret_cast<const void *>(dvm_vm_vec_ry),
+                           reinterpret_cast<const void *>(dvm_vm_cube_bf16_big),
+                           reinterpret_cast<const void *>(dvm_vm_cube_f16_big),
+                           reinterpret_cast<const void *>(dvm_vm_cube_bf16_mid),
+                           reinterpret_cast<const void *>(dvm_vm_cube_f16_mid),
+                           reinterpret_cast<const void *>(dvm_vm_cube_bf16_small),
+                           reinterpret_cast<const void *>(dvm_vm_cube_f16_small)};
   for (const void *k : kernels) {
     if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(g_dev.lds_per_cu)) ==
         hipSuccess) {
@@ -126,6 +138,27 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
       default:
         return static_cast<int>(hipErrorInvalidValue);
     }
+  } else if (h->entry == VE_CUBE) {
+    const VCubeHeader *c = reinterpret_cast<const VCubeHeader *>(p.w);
+    const uint64_t mem_end = static_cast<uint64_t>(c->mem_off) + static_cast<uint64_t>(c->n_mem) * (sizeof(VCubeMem) / 8);
+    const uint64_t code_end = static_cast<uint64_t>(c->code_off) + c->n_code;
+    const uint32_t bt = c->tile == 0 ? 256u : (c->tile == 1 ? 128u : 64u);
+    // The tile loop trusts the header: check it describes the launch it gets.
+    if (mem_end > DVM_PARAM_WORDS || code_end > DVM_PARAM_WORDS || c->n_code == 0 || VI_OP(p.w[code_end - 1]) != VOP_END ||
+        c->tile > 2 || threads != 256 || c->m == 0 || c->n == 0 || c->nb0 == 0 || c->nb1 == 0 ||
+        c->tiles_m != (c->m + bt - 1) / bt || c->tiles_n != (c->n + bt - 1) / bt || lds_bytes < 2u * (2u * bt) * 72u * 2u ||
+        c->a_addr == 0 || c->b_addr == 0 || (c->dtype != VDT_F16 && c->dtype != VDT_BF16)) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+    if (c->fast && (c->k % 64 != 0 || c->k == 0 || c->lda % 8 != 0 || c->ldb % 8 != 0 ||
+                    (c->a_addr & 15u) != 0 || (c->b_addr & 15u) != 0)) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+    const bool bf = c->dtype == VDT_BF16;
+    void (*kern)(const VmParam) = c->tile == 0   ? (bf ? dvm_vm_cube_bf16_big : dvm_vm_cube_f16_big)
+                                  : c->tile == 1 ? (bf ? dvm_vm_cube_bf16_mid : dvm_vm_cube_f16_mid)
+                                                 : (bf ? dvm_vm_cube_bf16_small : dvm_vm_cube_f16_small);
+    hipLaunchKernelGGL(kern, dim3(block_dim), dim3(256), lds_bytes, s, p);
   } else {
     return static_cast<int>(hipErrorInvalidValue);
   }

@@ -3,6 +3,7 @@
 // The disassembly is one instruction per line, "<mnemonic>.<type> operands";
 // tests pin fusion decisions by counting these mnemonics.
 #include <cstdio>
+#include <functional>
 #include <sstream>
 
 #include "ir.h"
@@ -108,6 +109,46 @@ std::string &VKernel::DisAssemble() {
       os << "idle (empty domain), " << p.fills.size() << " clean fill(s)\n";
       continue;
     }
+    auto print_code = [&os](const uint64_t *code, uint32_t n_code, const std::function<uint32_t(uint32_t)> &mem_dtype) {
+      for (uint32_t i = 0; i < n_code; ++i) {
+        const uint64_t w = code[i];
+        const uint32_t sub = VI_SUB(w);
+        os << "  ";
+        switch (VI_OP(w)) {
+          case VOP_END: os << "end"; break;
+          case VOP_LDR: os << "mov acc, v" << VI_A(w) << "." << kFmt[sub & 3]; break;
+          case VOP_LDS: os << "mov acc, s" << VI_A(w); break;
+          case VOP_LDI: {
+            char buf[32];
+            std::snprintf(buf, sizeof(buf), "#0x%08x", VI_IMM(w));
+            os << "broadcast_s acc, " << buf;
+            break;
+          }
+          case VOP_STR: os << "mov v" << VI_A(w) << "." << kFmt[sub & 3] << ", acc"; break;
+          case VOP_STS: os << "mov s" << VI_A(w) << ", acc"; break;
+          case VOP_ST: os << "store." << kMemTypes[mem_dtype(VI_A(w))] << " m" << VI_A(w) << ", acc"; break;
+          case VOP_UN: os << kUn[sub] << "." << (sub == VU_IABS ? "int32" : kRnd[VI_RND(w)]) << " acc"; break;
+          case VOP_CAST: {
+            static const char *names[] = {"cast.f2i", "cast.i2f", "cast.round", "cast.f2b"};
+            os << names[sub] << "." << kRnd[VI_RND(w)] << " acc";
+            break;
+          }
+          case VOP_RED: os << "reduce_" << kRed[sub] << " r" << VI_A(w) << ", acc"; break;
+          case VOP_SWEEP: os << "sweep slots=" << kRed[(VI_IMM(w) & 0xf) < 3 ? (VI_IMM(w) & 0xf) : 0]
+                             << ((VI_IMM(w) & 0xf) < 3 ? "" : "(none)"); break;
+          case VOP_ENDSWEEP: os << "endsweep"; break;
+          case VOP_FIN: os << "mov acc, r" << VI_A(w); break;
+          case VOP_LD: os << "load." << kMemTypes[mem_dtype(VI_A(w))] << " acc, m" << VI_A(w); break;
+          case VOP_BINF: os << kBinF[sub & 0x3f] << "." << kRnd[VI_RND(w)] << " acc, "; PrintSrc(os, w); break;
+          case VOP_BINI: os << kBinI[sub & 0x3f] << ".int32 acc, "; PrintSrc(os, w); break;
+          case VOP_CMP: os << "Cmp" << kCmp[sub & 7] << "." << ((sub & VCMP_INT) ? "int32" : "fp32") << " acc, "; PrintSrc(os, w); break;
+          case VOP_MSK: os << "mask "; PrintSrc(os, w); break;
+          case VOP_MOVM: os << "select acc, "; PrintSrc(os, w); break;
+          default: os << "?"; break;
+        }
+        os << "\n";
+      }
+    };
     const VVecHeader *h = reinterpret_cast<const VVecHeader *>(p.blob.w);
     if (h->entry == VE_VECTOR) {
       static const char *sched[] = {"pointwise", "reduce-x", "reduce-y"};
@@ -131,45 +172,22 @@ std::string &VKernel::DisAssemble() {
         for (uint32_t j = 0; j < h->n_rdim; ++j) os << (j ? "," : "") << mems[i].rstride[j];
         os << "]\n";
       }
-      const uint64_t *code = p.blob.w + h->code_off;
-      for (uint32_t i = 0; i < h->n_code; ++i) {
-        const uint64_t w = code[i];
-        const uint32_t sub = VI_SUB(w);
-        os << "  ";
-        switch (VI_OP(w)) {
-          case VOP_END: os << "end"; break;
-          case VOP_LDR: os << "mov acc, v" << VI_A(w) << "." << kFmt[sub & 3]; break;
-          case VOP_LDS: os << "mov acc, s" << VI_A(w); break;
-          case VOP_LDI: {
-            char buf[32];
-            std::snprintf(buf, sizeof(buf), "#0x%08x", VI_IMM(w));
-            os << "broadcast_s acc, " << buf;
-            break;
-          }
-          case VOP_STR: os << "mov v" << VI_A(w) << "." << kFmt[sub & 3] << ", acc"; break;
-          case VOP_STS: os << "mov s" << VI_A(w) << ", acc"; break;
-          case VOP_ST: os << "store." << kMemTypes[mems[VI_A(w)].dtype] << " m" << VI_A(w) << ", acc"; break;
-          case VOP_UN: os << kUn[sub] << "." << (sub == VU_IABS ? "int32" : kRnd[VI_RND(w)]) << " acc"; break;
-          case VOP_CAST: {
-            static const char *names[] = {"cast.f2i", "cast.i2f", "cast.round", "cast.f2b"};
-            os << names[sub] << "." << kRnd[VI_RND(w)] << " acc";
-            break;
-          }
-          case VOP_RED: os << "reduce_" << kRed[sub] << " r" << VI_A(w) << ", acc"; break;
-          case VOP_SWEEP: os << "sweep slots=" << kRed[(VI_IMM(w) & 0xf) < 3 ? (VI_IMM(w) & 0xf) : 0]
-                             << ((VI_IMM(w) & 0xf) < 3 ? "" : "(none)"); break;
-          case VOP_ENDSWEEP: os << "endsweep"; break;
-          case VOP_FIN: os << "mov acc, r" << VI_A(w); break;
-          case VOP_LD: os << "load." << kMemTypes[mems[VI_A(w)].dtype] << " acc, m" << VI_A(w); break;
-          case VOP_BINF: os << kBinF[sub & 0x3f] << "." << kRnd[VI_RND(w)] << " acc, "; PrintSrc(os, w); break;
-          case VOP_BINI: os << kBinI[sub & 0x3f] << ".int32 acc, "; PrintSrc(os, w); break;
-          case VOP_CMP: os << "Cmp" << kCmp[sub & 7] << "." << ((sub & VCMP_INT) ? "int32" : "fp32") << " acc, "; PrintSrc(os, w); break;
-          case VOP_MSK: os << "mask "; PrintSrc(os, w); break;
-          case VOP_MOVM: os << "select acc, "; PrintSrc(os, w); break;
-          default: os << "?"; break;
-        }
-        os << "\n";
+      print_code(p.blob.w + h->code_off, h->n_code, [&](uint32_t m) { return mems[m].dtype; });
+    } else if (h->entry == VE_CUBE) {
+      const VCubeHeader *c = reinterpret_cast<const VCubeHeader *>(p.blob.w);
+      static const int tile[] = {256, 128, 64};
+      os << "entry cube " << kMemTypes[c->dtype] << " m=" << c->m << " n=" << c->n << " k=" << c->k << " trans_a=" << c->trans_a
+         << " trans_b=" << c->trans_b << " batch=" << c->nb0 << "x" << c->nb1 << " tile=" << tile[c->tile] << " blocks=" << p.grid
+         << " lds=" << p.lds_bytes << (c->fast ? " fast" : " guarded") << "\n";
+      const VCubeMem *cm = reinterpret_cast<const VCubeMem *>(p.blob.w + c->mem_off);
+      for (uint32_t i = 0; i < c->n_mem; ++i) {
+        char buf[32];
+        std::snprintf(buf, sizeof(buf), "0x%llx", static_cast<unsigned long long>(cm[i].addr));
+        os << "  m" << i << ": " << kMemTypes[cm[i].dtype] << " @" << buf << " strides n=" << cm[i].stride_n << " m=" << cm[i].stride_m
+           << " b=" << cm[i].stride_b0 << "," << cm[i].stride_b1 << "\n";
       }
+      os << "  mmad acc, A, B\n";
+      print_code(p.blob.w + c->code_off, c->n_code, [&](uint32_t m) { return cm[m].dtype; });
     } else {
       os << "entry type " << h->entry << " blocks=" << p.grid << " threads=" << p.threads << "\n";
     }

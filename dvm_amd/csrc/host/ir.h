@@ -107,10 +107,13 @@ struct Program {
   bool skip = false;       // nothing to do (an extent is zero)
   // addresses inside the blob that depend on relocation: (word offset, op) pairs
   struct Patch {
-    uint32_t word;
+    uint32_t word;   // 64-bit word of the blob that receives the address
     int op_id;       // load/store node whose address goes there, or -1
     int ws_slot;     // or the workspace slot
+    uint8_t role;    // kPatchVecMem: a VMemDesc (alignment flag follows the address); kPatchCubeOperand:
+                     // a matmul operand (the fast path needs 16-byte alignment); kPatchPlain: nothing else
   };
+  enum : uint8_t { kPatchVecMem = 0, kPatchCubeOperand = 1, kPatchPlain = 2 };
   std::vector<Patch> patches;
   // pre-launch fills (zero-size reduce identities, clean kernels)
   struct Fill {

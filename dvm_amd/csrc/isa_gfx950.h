@@ -157,6 +157,44 @@ typedef struct {
   VDim rdims[DVM_VEC_MAXR];
 } VVecHeader;            // 64 + 128 = 192 bytes
 
+// ---- matmul programs (VE_CUBE) ---------------------------------------------------
+// C[b][m][n] = sum_k A[b][m][k] * B[b][k][n], fp32 accumulation on MFMA, then an epilogue program
+// in the vector VM's instruction words runs on every accumulator fragment (acc = the 16 values a
+// lane holds of one 32x32 tile) before anything is stored: VOP_CAST / VOP_UN / VOP_BINF / VOP_BINI /
+// VOP_CMP / VOP_MSK / VOP_MOVM with VK_IMM, VK_ACC, VK_MEM (stride-addressed, so a bias row is a
+// stride-0 operand) or VK_REG (two fragment-sized temporaries), VOP_STR / VOP_LDR on those
+// temporaries, VOP_ST to one or more outputs.
+#define DVM_CUBE_MAXMEM 12
+#define DVM_CUBE_NTEMP 2
+
+typedef struct {
+  uint64_t addr;
+  uint32_t dtype;     // VDT_*
+  uint32_t flags;
+  uint32_t stride_n;  // element strides against the output's n, m and the two batch axes (0 = broadcast)
+  uint32_t stride_m;
+  uint32_t stride_b0;
+  uint32_t stride_b1;
+} VCubeMem;
+
+typedef struct {
+  uint32_t entry;      // VE_CUBE
+  uint32_t dtype;      // VDT_F16 or VDT_BF16 (operand type; accumulation is fp32)
+  uint32_t m, n, k;
+  uint32_t trans_a;    // A is stored [k][m]
+  uint32_t trans_b;    // B is stored [n][k]
+  uint32_t lda, ldb;   // leading dimensions in elements
+  uint32_t nb0, nb1;   // batch extents (outer, inner); 1 when absent
+  uint32_t a_sb0, a_sb1, b_sb0, b_sb1;  // batch strides in elements (0 = broadcast)
+  uint32_t tile;       // block tile: 0 = 256x256, 1 = 128x128, 2 = 64x64
+  uint32_t tiles_m, tiles_n;
+  uint32_t n_mem, n_code;
+  uint32_t mem_off, code_off;  // word offsets
+  uint32_t fast;       // k is a multiple of 64 and every 8-element operand chunk is 16-byte aligned: full tiles take the vector path
+  uint32_t pad;
+  uint64_t a_addr, b_addr;
+} VCubeHeader;
+
 typedef struct {
   uint64_t w[DVM_PARAM_WORDS];
 } VmParam;

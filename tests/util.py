@@ -11,17 +11,26 @@ from oracle.oracle import OracleKernel
 DEFAULT_EPS = {int(DataType.float32): 1e-5, int(DataType.float16): 1e-3, int(DataType.bfloat16): 1e-2}
 
 
-def run_parity(build, arrays, dtypes=None, ker="vector", eps=None, golden=None, golden_eps=None):
-    """build(k, *inputs) -> value or list of values. Returns the HIP outputs."""
+def run_parity(build, arrays, dtypes=None, ker="vector", eps=None, golden=None, golden_eps=None, use_oracle=True):
+    """build(k, *inputs) -> value or list of values. Returns the HIP outputs.
+
+    use_oracle=False (sizes the scalar oracle cannot finish in seconds) checks against the golden only."""
     dtypes = dtypes or [None] * len(arrays)
-    t, o = Tester(ker), OracleKernel()
+    assert use_oracle or golden is not None
+    t = Tester(ker)
     t_in = [t.load(a, d) for a, d in zip(arrays, dtypes)]
-    o_in = [o.load(a, d) for a, d in zip(arrays, dtypes)]
-    t_out, o_out = build(t, *t_in), build(o, *o_in)
+    t_out = build(t, *t_in)
     if not isinstance(t_out, (list, tuple)):
-        t_out, o_out = [t_out], [o_out]
+        t_out = [t_out]
     stores = [t.store(x) for x in t_out]
-    refs = [o.output(o.store(x)) for x in o_out]
+    if use_oracle:
+        o = OracleKernel()
+        o_out = build(o, *[o.load(a, d) for a, d in zip(arrays, dtypes)])
+        if not isinstance(o_out, (list, tuple)):
+            o_out = [o_out]
+        refs = [o.output(o.store(x)) for x in o_out]
+    else:
+        refs = [None] * len(stores)
     t.run()
     outs = []
     for i, (s, ref) in enumerate(zip(stores, refs)):
@@ -29,6 +38,9 @@ def run_parity(build, arrays, dtypes=None, ker="vector", eps=None, golden=None, 
         dt = int(s.dtype())
         if dt == int(DataType.bfloat16):
             out = Tester.convert_from_bf16(out)
+        if ref is None:
+            outs.append(out)
+            continue
         assert out.shape == ref.shape, "output %d: shape %s vs oracle %s" % (i, out.shape, ref.shape)
         if dt in (int(DataType.int32), int(DataType.bool)):
             assert np.array_equal(out, ref), "output %d differs from the oracle (bit-exact required)\n%s" % (i, t.das())
