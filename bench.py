@@ -152,6 +152,37 @@ def bench_rmsnorm(calls=200):
     }
 
 
+def bench_matmul(m=8192, n=4096, k=4096, iters=20):
+    """configs[4]: bf16 A[m,k] x B[k,n], fp32 accumulate, epilogue bias add + SiLU + cast to bf16, one launch."""
+    from dvm_amd.tester import Tester
+    rng = np.random.default_rng(1005)
+    a = Tester.convert_to_bf16((rng.standard_normal([m, k], dtype=np.float32) / 8.0))
+    b = Tester.convert_to_bf16((rng.standard_normal([k, n], dtype=np.float32) / 8.0))
+    bias = (rng.standard_normal([n], dtype=np.float32) * np.float32(np.sqrt(0.1)))
+    t = Tester("mix")
+    x, y, bb = t.load(a.shape, "bfloat16"), t.load(b.shape, "bfloat16"), t.load(bias)
+    t.input(x, a)
+    t.input(y, b)
+    h = t.add(t.cast(t.matmul(x, y, False, False), "float32"), bb)
+    out = t.store(t.cast(t.div(h, t.add(t.exp(t.mul(h, -1.0)), 1.0)), "bfloat16"))
+    t.codegen()
+    cold = t.jit_us()
+    t.run()
+    got = Tester.convert_from_bf16(t.output(out))
+    # parity on sampled rows against the NumPy golden (bf16 tolerance 1e-2)
+    rows = rng.integers(0, m, 16)
+    af, bf = Tester.convert_from_bf16(a[rows]).astype(np.float64), Tester.convert_from_bf16(b).astype(np.float64)
+    hh = Tester.convert_from_bf16(Tester.convert_to_bf16((af @ bf).astype(np.float32))).astype(np.float64) + bias
+    want = hh / (1.0 + np.exp(-hh))
+    if not np.allclose(got[rows], want, rtol=1e-2, atol=1e-2):
+        raise RuntimeError("matmul epilogue result differs from the NumPy golden")
+    mn, _, mean = t.perf(warmup=3, iters=iters)
+    flops = 2.0 * m * n * k
+    return {"shape": [m, n, k], "kernel_us_mean": round(mean, 2), "kernel_us_min": round(mn, 2), "TFLOPs": round(flops / mean / 1e6, 1),
+            "frac_of_2.5PFLOPs": round(flops / mean / 1e6 / 2500.0, 4), "launches": t.num_launches(), "jit_us_cold": round(cold, 2),
+            "parity_rows_checked": len(rows)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -185,7 +216,8 @@ def main():
     if not args.skip_cpu:
         line["cpu_baseline"] = cpu_baseline_batchnorm(bn["x"], bn["g"], bn["b"], bn["alg_bytes"])
     if not args.only_headline:
-        line["configs"] = {"add_fp32_32x32": bench_add(), "residual_rmsnorm_bf16_dynamic": bench_rmsnorm()}
+        line["configs"] = {"add_fp32_32x32": bench_add(), "residual_rmsnorm_bf16_dynamic": bench_rmsnorm(),
+                           "matmul_bias_silu_bf16_8192x4096x4096": bench_matmul()}
     print(json.dumps(line))
 
 

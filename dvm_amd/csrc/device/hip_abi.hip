@@ -5,18 +5,33 @@
 #include <stdint.h>
 #include <string.h>
 
+#include <vector>
+
 #include "../../../include/dvm_hip.h"
 #include "../isa_gfx950.h"
 
 extern "C" __global__ void dvm_vm_vec_pw(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_rx(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_ry(const VmParam p);
-extern "C" __global__ void dvm_vm_cube_bf16_big(const VmParam p);
-extern "C" __global__ void dvm_vm_cube_f16_big(const VmParam p);
-extern "C" __global__ void dvm_vm_cube_bf16_mid(const VmParam p);
-extern "C" __global__ void dvm_vm_cube_f16_mid(const VmParam p);
-extern "C" __global__ void dvm_vm_cube_bf16_small(const VmParam p);
-extern "C" __global__ void dvm_vm_cube_f16_small(const VmParam p);
+#define DVM_CUBE_DECL(prefix)                                \
+  extern "C" __global__ void prefix##_nn(const VmParam p); \
+  extern "C" __global__ void prefix##_nt(const VmParam p); \
+  extern "C" __global__ void prefix##_tn(const VmParam p); \
+  extern "C" __global__ void prefix##_tt(const VmParam p);
+DVM_CUBE_DECL(dvm_vm_cube_bf16_big)
+DVM_CUBE_DECL(dvm_vm_cube_f16_big)
+DVM_CUBE_DECL(dvm_vm_cube_bf16_mid)
+DVM_CUBE_DECL(dvm_vm_cube_f16_mid)
+DVM_CUBE_DECL(dvm_vm_cube_bf16_small)
+DVM_CUBE_DECL(dvm_vm_cube_f16_small)
+
+typedef void (*CubeKernel)(const VmParam);
+#define DVM_CUBE_ROW(prefix) {prefix##_nn, prefix##_nt, prefix##_tn, prefix##_tt}
+// [tile][bf16][trans_a * 2 + trans_b]
+static const CubeKernel kCubeKernels[3][2][4] = {
+    {DVM_CUBE_ROW(dvm_vm_cube_f16_big), DVM_CUBE_ROW(dvm_vm_cube_bf16_big)},
+    {DVM_CUBE_ROW(dvm_vm_cube_f16_mid), DVM_CUBE_ROW(dvm_vm_cube_bf16_mid)},
+    {DVM_CUBE_ROW(dvm_vm_cube_f16_small), DVM_CUBE_ROW(dvm_vm_cube_bf16_small)}};
 
 namespace {
 
@@ -65,14 +80,11 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
   if (g_dev.lds_per_cu == 0) g_dev.lds_per_cu = 64 * 1024;
   g_dev.lds_per_wg = static_cast<uint32_t>(prop.sharedMemPerBlock);
   // gfx950 lets one workgroup use the CU's whole 160 KB; the kernels must opt in.
-  const void *kernels[] = {reinterpret_cast<const void *>(dvm_vm_vec_pw), reinterpret_cast<const void *>(dvm_vm_vec_rx),
-                           reinterpret_cast<const void *>(dvm_vm_vec_ry),
-                           reinterpret_cast<const void *>(dvm_vm_cube_bf16_big),
-                           reinterpret_cast<const void *>(dvm_vm_cube_f16_big),
-                           reinterpret_cast<const void *>(dvm_vm_cube_bf16_mid),
-                           reinterpret_cast<const void *>(dvm_vm_cube_f16_mid),
-                           reinterpret_cast<const void *>(dvm_vm_cube_bf16_small),
-                           reinterpret_cast<const void *>(dvm_vm_cube_f16_small)};
+  std::vector<const void *> kernels = {reinterpret_cast<const void *>(dvm_vm_vec_pw), reinterpret_cast<const void *>(dvm_vm_vec_rx),
+                                       reinterpret_cast<const void *>(dvm_vm_vec_ry)};
+  for (const auto &tile : kCubeKernels)
+    for (const auto &dt : tile)
+      for (CubeKernel k : dt) kernels.push_back(reinterpret_cast<const void *>(k));
   for (const void *k : kernels) {
     if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(g_dev.lds_per_cu)) ==
         hipSuccess) {
@@ -146,18 +158,15 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
     // The tile loop trusts the header: check it describes the launch it gets.
     if (mem_end > DVM_PARAM_WORDS || code_end > DVM_PARAM_WORDS || c->n_code == 0 || VI_OP(p.w[code_end - 1]) != VOP_END ||
         c->tile > 2 || threads != 256 || c->m == 0 || c->n == 0 || c->nb0 == 0 || c->nb1 == 0 ||
-        c->tiles_m != (c->m + bt - 1) / bt || c->tiles_n != (c->n + bt - 1) / bt || lds_bytes < 2u * (2u * bt) * 72u * 2u ||
+        c->tiles_m != (c->m + bt - 1) / bt || c->tiles_n != (c->n + bt - 1) / bt || lds_bytes < DVM_CUBE_LDS_BYTES(bt) ||
         c->a_addr == 0 || c->b_addr == 0 || (c->dtype != VDT_F16 && c->dtype != VDT_BF16)) {
       return static_cast<int>(hipErrorInvalidValue);
     }
-    if (c->fast && (c->k % 64 != 0 || c->k == 0 || c->lda % 8 != 0 || c->ldb % 8 != 0 ||
+    if (c->fast && (c->lda >= (1u << 22) || c->ldb >= (1u << 22) || c->k % 64 != 0 || c->k == 0 || c->lda % 8 != 0 || c->ldb % 8 != 0 ||
                     (c->a_addr & 15u) != 0 || (c->b_addr & 15u) != 0)) {
       return static_cast<int>(hipErrorInvalidValue);
     }
-    const bool bf = c->dtype == VDT_BF16;
-    void (*kern)(const VmParam) = c->tile == 0   ? (bf ? dvm_vm_cube_bf16_big : dvm_vm_cube_f16_big)
-                                  : c->tile == 1 ? (bf ? dvm_vm_cube_bf16_mid : dvm_vm_cube_f16_mid)
-                                                 : (bf ? dvm_vm_cube_bf16_small : dvm_vm_cube_f16_small);
+    const CubeKernel kern = kCubeKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0][(c->trans_a ? 2 : 0) + (c->trans_b ? 1 : 0)];
     hipLaunchKernelGGL(kern, dim3(block_dim), dim3(256), lds_bytes, s, p);
   } else {
     return static_cast<int>(hipErrorInvalidValue);

@@ -1,19 +1,24 @@
-// gfx950 matmul VM: MFMA tile loop with an interpreted epilogue applied from registers.
+// gfx950 matmul VM: MFMA tile loop followed by an interpreted epilogue on the tile, before anything
+// reaches memory.
 //
 // Role in the reference: the cube kernels (device semantics src/vm_aic.cce:34-470: fp32
 // accumulation, one rounding to the operand type on write-out) plus the mix kernel's post-fusion
 // vector program (src/xkernel.cc:304-360). The reference's CUDA backend has no matmul at all
 // (src/system.cc:290-294); this kernel is specific to CDNA4:
-//  * v_mfma_f32_32x32x16 (bf16 / f16), 64-wide waves, each wave owns a (TM*32) x (TN*32) block of
-//    accumulators that never leaves registers until the epilogue has run;
-//  * operand tiles are staged through local memory with k contiguous and rows padded by 16 bytes,
-//    so every fragment read is one conflict-free 128-bit access; operands whose k axis is strided
-//    in memory (B of an NN product, A of a TN product) are transposed in registers on the way in;
-//  * local memory is double buffered, the next tile's global loads are in flight while the MFMAs
-//    of the current one run;
-//  * the epilogue decodes the vector VM's instruction words (wave-uniform) and works on the 16
-//    accumulator values a lane holds of one 32x32 tile, so bias add, activation and casts cost no
-//    extra pass over memory.
+//  * v_mfma_f32_32x32x16 (bf16 / f16), 64-wide waves, 2 x 2 waves per workgroup, each wave owning a
+//    (TM*32) x (TN*32) block of fp32 accumulators that stays in registers for the whole k loop;
+//  * operand tiles are staged through local memory with k contiguous: rows of 64 elements (128
+//    bytes, no padding) whose eight 16-byte chunks are XOR-swizzled by the row number, so that the
+//    fragment reads (32 consecutive rows, one chunk), the straight tile copies (one row, eight
+//    chunks) and the transposing copies (rows 8 apart, one chunk) are all free of bank conflicts;
+//  * operands whose k axis is strided in memory (B of an NN product, A of a TN product) are read
+//    along their contiguous axis and transposed in registers, 8x8 elements per lane, on the way in;
+//  * local memory is double buffered and fragments are double buffered in registers: the global
+//    loads of tile t+1 and the fragment reads of step s+1 are in flight while the MFMAs of step s run;
+//  * the epilogue runs in two passes over half tiles: accumulators go to local memory once, row
+//    major, and come back as slabs of 8 consecutive columns per lane, so every memory operand of the
+//    epilogue and every store is a coalesced 128-bit access; the epilogue program is the vector
+//    VM's instruction words, decoded wave-uniformly.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -24,12 +29,15 @@ namespace {
 #define DVM_GLOBAL __attribute__((address_space(1)))
 
 typedef float vf16 __attribute__((ext_vector_type(16)));
+typedef float vf4 __attribute__((ext_vector_type(4)));
 typedef uint32_t vu4 __attribute__((ext_vector_type(4)));
+typedef uint32_t vu2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
-constexpr int BK = 64;          // k extent of a staged tile
-constexpr int LDS_ROW = BK + 8; // elements per padded row (144 bytes)
+constexpr int BK = 64;   // k extent of a staged tile = one 128-byte row of 16-bit elements
+constexpr int SL = 2;    // slabs of 8 columns the epilogue interpreter handles per walk of the program
+constexpr int NTEMP = DVM_CUBE_NTEMP;
 
 __device__ __forceinline__ uint32_t uni(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 
@@ -51,72 +59,80 @@ __device__ __forceinline__ vf16 mfma(vu4 a, vu4 b, vf16 c) {
   }
 }
 
-// ---- staging one operand tile: ROWS rows (m or n) x BK (k), k contiguous in local memory -------------
-// Source with k contiguous (A when !trans_a, B when trans_b): 16-byte chunks copied as they are.
-// Source with k strided (row index contiguous): 8x8 element blocks, transposed in registers.
-template <int ROWS>
+// Element offset of 16-byte chunk `chunk` (0..7) of row `row` inside a staged tile.
+__device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk) {
+  return row * BK + ((chunk ^ ((row ^ (row >> 3)) & 7u)) << 3);
+}
+
+// ---- staging one operand tile: ROWS rows (m or n) x BK (k) ---------------------------------------------
+// KC source (k contiguous in memory: A when !trans_a, B when trans_b): 16-byte chunks copied as they are.
+// KS source (k strided, the row index contiguous): 8x8 element blocks, transposed in registers.
+template <int ROWS, bool KC>
 struct Stage {
-  static constexpr int CHUNKS = ROWS * BK / 8 / 256;  // 16-byte chunks per thread
-  // a k-strided source moves whole 8x8 blocks (8 chunks): ROWS blocks per tile, one per thread for
-  // the first ROWS threads
-  vu4 r[CHUNKS < 8 ? 8 : CHUNKS];
+  static constexpr int CHUNKS = ROWS * BK / 8 / 256;  // 16-byte chunks per thread when all 256 threads copy
+  // a KS source moves whole 8x8 blocks (8 chunks): ROWS blocks per tile, one per thread for the first ROWS threads
+  static constexpr int N = KC ? CHUNKS : 8;
+  vu4 r[N];
+
+  // Byte offset of this lane's first chunk from the tile's origin; the rest of every address is
+  // wave-uniform, so one register per operand addresses all its loads.
+  static __device__ __forceinline__ uint32_t lane_offset(uint32_t ld, uint32_t tid) {
+    if constexpr (KC) {
+      return ((tid >> 3) * ld + ((tid & 7u) << 3)) * 2u;
+    } else {
+      const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
+      return (kb * 8u * ld + rb * 8u) * 2u;
+    }
+  }
+
+  // origin: address of element (row0, k0) of the operand; voff: lane_offset()
+  __device__ __forceinline__ void load(uint64_t origin, uint32_t ld, uint32_t voff, uint32_t tid) {
+    const DVM_GLOBAL char *base = reinterpret_cast<const DVM_GLOBAL char *>(origin);
+    if constexpr (KC) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        r[i] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(base + static_cast<uint64_t>(i) * 32u * ld * 2u + voff);
+      }
+    } else {
+      static_assert(ROWS <= 256, "one block per thread");
+      if (ROWS == 256 || tid < ROWS) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          r[j] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(base + static_cast<uint64_t>(j) * ld * 2u + voff);
+        }
+      }
+    }
+  }
+
+  __device__ __forceinline__ void store(uint16_t *tile, uint32_t tid) const {
+    if constexpr (KC) {
+#pragma unroll
+      for (int i = 0; i < N; ++i) {
+        const uint32_t c = tid + 256u * i;
+        *reinterpret_cast<vu4 *>(tile + tile_off(c >> 3, c & 7u)) = r[i];
+      }
+    } else {
+      if (ROWS == 256 || tid < ROWS) {
+        const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
+        // r[j] holds k = kb*8 + j, rows rb*8 .. +7; the tile wants, per row, k = kb*8 .. +7
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          vu4 o;
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) {
+            const uint32_t lo = r[2 * jj][i >> 1], hi = r[2 * jj + 1][i >> 1];
+            // bytes of the result, least significant first: (i odd ? upper : lower) half of lo, then of hi
+            o[jj] = __builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
+          }
+          *reinterpret_cast<vu4 *>(tile + tile_off(rb * 8 + i, kb)) = o;
+        }
+      }
+    }
+  }
 };
 
-// k-contiguous source, every chunk in range and 16-byte aligned
-template <int ROWS>
-__device__ __forceinline__ void stage_load_kc(Stage<ROWS> &s, uint64_t base, uint32_t ld, uint32_t row0, uint32_t k0, uint32_t tid) {
-#pragma unroll
-  for (int i = 0; i < Stage<ROWS>::CHUNKS; ++i) {
-    const uint32_t c = tid + 256u * i;
-    const uint32_t row = c / (BK / 8), kc = (c % (BK / 8)) * 8;
-    s.r[i] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(base + (static_cast<uint64_t>(row0 + row) * ld + k0 + kc) * 2);
-  }
-}
-
-template <int ROWS>
-__device__ __forceinline__ void stage_store_kc(const Stage<ROWS> &s, uint16_t *tile, uint32_t tid) {
-#pragma unroll
-  for (int i = 0; i < Stage<ROWS>::CHUNKS; ++i) {
-    const uint32_t c = tid + 256u * i;
-    const uint32_t row = c / (BK / 8), kc = (c % (BK / 8)) * 8;
-    *reinterpret_cast<vu4 *>(tile + row * LDS_ROW + kc) = s.r[i];
-  }
-}
-
-// k-strided source (memory is [k][row]): thread t < ROWS handles the 8x8 block (kb, rb) = (t / (ROWS/8), t % (ROWS/8))
-template <int ROWS>
-__device__ __forceinline__ void stage_load_ks(Stage<ROWS> &s, uint64_t base, uint32_t ld, uint32_t row0, uint32_t k0, uint32_t tid) {
-  static_assert(ROWS <= 256, "one block per thread");
-  if (tid < ROWS) {
-    const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      s.r[j] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(base + (static_cast<uint64_t>(k0 + kb * 8 + j) * ld + row0 + rb * 8) * 2);
-    }
-  }
-}
-
-template <int ROWS>
-__device__ __forceinline__ void stage_store_ks(const Stage<ROWS> &s, uint16_t *tile, uint32_t tid) {
-  if (tid < ROWS) {
-    const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
-    // in[j][i]: k = kb*8 + j, row = rb*8 + i  ->  out row i holds k = kb*8 .. +7
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      vu4 o = 0u;
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t w = s.r[j][i / 2];
-        const uint32_t e = (i & 1) ? (w >> 16) : (w & 0xffffu);
-        o[j / 2] |= e << (16 * (j & 1));
-      }
-      *reinterpret_cast<vu4 *>(tile + (rb * 8 + i) * LDS_ROW + kb * 8) = o;
-    }
-  }
-}
-
-// Generic staging of one tile straight into local memory, element by element (edges, unaligned or
-// odd leading dimensions). Slow, correct for every shape.
+// Generic staging of one tile straight into local memory, element by element (edge tiles, odd
+// leading dimensions, unaligned operands). Slow, correct for every shape.
 template <int ROWS>
 __device__ __attribute__((noinline)) void stage_generic(uint16_t *tile, uint64_t base, uint32_t ld, uint32_t row0, uint32_t k0,
                                                         uint32_t rows, uint32_t kext, uint32_t k_contig, uint32_t tid) {
@@ -128,100 +144,151 @@ __device__ __attribute__((noinline)) void stage_generic(uint16_t *tile, uint64_t
       const uint64_t idx = k_contig ? static_cast<uint64_t>(gr) * ld + gk : static_cast<uint64_t>(gk) * ld + gr;
       v = reinterpret_cast<const DVM_GLOBAL uint16_t *>(base)[idx];
     }
-    tile[row * LDS_ROW + kk] = v;
+    tile[tile_off(row, kk >> 3) + (kk & 7u)] = v;
   }
 }
 
-// ---- epilogue -------------------------------------------------------------------------------------
+// ---- epilogue ---------------------------------------------------------------------------------------
+// A slab is 8 consecutive columns of one row of the output; the interpreter works on SL slabs at a
+// time, held as one 16-wide vector of fp32 containers (element s*8 + e = column e of slab s) so that
+// values travel between the out-of-line helpers in registers.
+static_assert(SL == 2, "the slab vector is 16 wide");
+typedef vf16 Slabs;
 
-struct Frag {
-  vf16 v;
-};
+#define FOR_SE _Pragma("unroll") for (int q = 0; q < SL * 8; ++q)
 
-__device__ __forceinline__ float elem_load(uint64_t base, uint32_t dtype, uint64_t off) {
-  switch (dtype) {
-    case VDT_F32: return reinterpret_cast<const DVM_GLOBAL float *>(base)[off];
-    case VDT_I32: return __int_as_float(reinterpret_cast<const DVM_GLOBAL int32_t *>(base)[off]);
-    case VDT_F16: return static_cast<float>(reinterpret_cast<const DVM_GLOBAL _Float16 *>(base)[off]);
-    case VDT_BF16: return __uint_as_float(static_cast<uint32_t>(reinterpret_cast<const DVM_GLOBAL uint16_t *>(base)[off]) << 16);
-    default: return reinterpret_cast<const DVM_GLOBAL uint8_t *>(base)[off] != 0 ? 1.0f : 0.0f;
-  }
+__device__ __forceinline__ float cvt_in(uint32_t dtype, uint32_t bits16) {
+  return dtype == VDT_F16 ? static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16))) : __uint_as_float(bits16 << 16);
 }
 
-__device__ __forceinline__ void elem_store(uint64_t base, uint32_t dtype, uint64_t off, float v) {
-  switch (dtype) {
-    case VDT_F32: reinterpret_cast<DVM_GLOBAL float *>(base)[off] = v; break;
-    case VDT_I32: reinterpret_cast<DVM_GLOBAL int32_t *>(base)[off] = __float_as_int(v); break;
-    case VDT_F16: reinterpret_cast<DVM_GLOBAL _Float16 *>(base)[off] = static_cast<_Float16>(v); break;
-    case VDT_BF16: reinterpret_cast<DVM_GLOBAL uint16_t *>(base)[off] = static_cast<uint16_t>(f32_to_bf16_bits(v)); break;
-    default: reinterpret_cast<DVM_GLOBAL uint8_t *>(base)[off] = v != 0.0f ? 1 : 0; break;
-  }
-}
-
-// Memory operand of the epilogue for the fragment whose lane column is `col` and whose 16 rows are
-// row_base + 8*(r/4) + (r%4). Out-of-range positions read 0 / are not written.
-__device__ __attribute__((noinline)) Frag frag_load(uint64_t addr, uint32_t dtype, uint32_t sn, uint32_t sm, uint64_t boff,
-                                                   uint32_t row_base, uint32_t col, uint32_t m, uint32_t n) {
-  Frag f;
+// row0/row1: output rows of the two slabs, col: first column, ncol: columns inside the output (0..8),
+// rows_ok: bit s set when slab s is inside the output.
+__device__ __attribute__((noinline)) Slabs epi_load(uint64_t addr, uint32_t dtype, uint32_t sn, uint32_t sm, uint64_t boff, uint32_t row0,
+                                                   uint32_t row1, uint32_t col, uint32_t ncol, uint32_t rows_ok) {
+  Slabs out;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const uint32_t row = row_base + 8 * (r / 4) + (r % 4);
-    float v = 0.0f;
-    if (row < m && col < n) v = elem_load(addr, dtype, boff + static_cast<uint64_t>(row) * sm + static_cast<uint64_t>(col) * sn);
-    f.v[r] = v;
+  for (int s = 0; s < SL; ++s) {
+    const bool ok = (rows_ok >> s) & 1u;
+    const uint64_t off = boff + static_cast<uint64_t>(s == 0 ? row0 : row1) * sm + static_cast<uint64_t>(col) * sn;
+    const uint32_t esz = (dtype == VDT_F32 || dtype == VDT_I32) ? 4u : (dtype == VDT_BOOL ? 1u : 2u);
+    const bool vec = ok && sn == 1 && ncol == 8 && ((addr + off * esz) & 15u) == 0;
+    if (vec && esz == 4) {
+      const vu4 a = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + off * 4), b = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + off * 4 + 16);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        out[s * 8 + e] = __uint_as_float(a[e]);
+        out[s * 8 + 4 + e] = __uint_as_float(b[e]);
+      }
+    } else if (vec && esz == 2) {
+      const vu4 a = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + off * 2);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[s * 8 + e] = cvt_in(dtype, (a[e >> 1] >> (16 * (e & 1))) & 0xffffu);
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float v = 0.0f;
+        if (ok && static_cast<uint32_t>(e) < ncol) {
+          const uint64_t o = off + static_cast<uint64_t>(e) * sn;
+          switch (dtype) {
+            case VDT_F32: v = reinterpret_cast<const DVM_GLOBAL float *>(addr)[o]; break;
+            case VDT_I32: v = __int_as_float(reinterpret_cast<const DVM_GLOBAL int32_t *>(addr)[o]); break;
+            case VDT_F16:
+            case VDT_BF16: v = cvt_in(dtype, reinterpret_cast<const DVM_GLOBAL uint16_t *>(addr)[o]); break;
+            default: v = reinterpret_cast<const DVM_GLOBAL uint8_t *>(addr)[o] != 0 ? 1.0f : 0.0f; break;
+          }
+        }
+        out[s * 8 + e] = v;
+      }
+    }
   }
-  return f;
+  return out;
 }
 
-__device__ __attribute__((noinline)) void frag_store(uint64_t addr, uint32_t dtype, uint32_t sn, uint32_t sm, uint64_t boff,
-                                                    uint32_t row_base, uint32_t col, uint32_t m, uint32_t n, Frag f) {
+__device__ __attribute__((noinline)) void epi_store(uint64_t addr, uint32_t dtype, uint32_t sn, uint32_t sm, uint64_t boff, uint32_t row0,
+                                                   uint32_t row1, uint32_t col, uint32_t ncol, uint32_t rows_ok, Slabs x) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const uint32_t row = row_base + 8 * (r / 4) + (r % 4);
-    if (row < m && col < n) elem_store(addr, dtype, boff + static_cast<uint64_t>(row) * sm + static_cast<uint64_t>(col) * sn, f.v[r]);
+  for (int s = 0; s < SL; ++s) {
+    if (!((rows_ok >> s) & 1u) || ncol == 0) continue;
+    const uint64_t off = boff + static_cast<uint64_t>(s == 0 ? row0 : row1) * sm + static_cast<uint64_t>(col) * sn;
+    const uint32_t esz = (dtype == VDT_F32 || dtype == VDT_I32) ? 4u : (dtype == VDT_BOOL ? 1u : 2u);
+    const bool vec = sn == 1 && ncol == 8 && ((addr + off * esz) & 15u) == 0;
+    if (vec && esz == 4) {
+      vu4 a, b;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        a[e] = __float_as_uint(x[s * 8 + e]);
+        b[e] = __float_as_uint(x[s * 8 + 4 + e]);
+      }
+      *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + off * 4) = a;
+      *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + off * 4 + 16) = b;
+    } else if (vec && esz == 2) {
+      vu4 a;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        uint32_t lo, hi;
+        if (dtype == VDT_F16) {
+          lo = __builtin_bit_cast(uint16_t, static_cast<_Float16>(x[s * 8 + 2 * e]));
+          hi = __builtin_bit_cast(uint16_t, static_cast<_Float16>(x[s * 8 + 2 * e + 1]));
+        } else {
+          lo = f32_to_bf16_bits(x[s * 8 + 2 * e]);
+          hi = f32_to_bf16_bits(x[s * 8 + 2 * e + 1]);
+        }
+        a[e] = lo | (hi << 16);
+      }
+      *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + off * 2) = a;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        if (static_cast<uint32_t>(e) >= ncol) continue;
+        const uint64_t o = off + static_cast<uint64_t>(e) * sn;
+        const float v = x[s * 8 + e];
+        switch (dtype) {
+          case VDT_F32: reinterpret_cast<DVM_GLOBAL float *>(addr)[o] = v; break;
+          case VDT_I32: reinterpret_cast<DVM_GLOBAL int32_t *>(addr)[o] = __float_as_int(v); break;
+          case VDT_F16: reinterpret_cast<DVM_GLOBAL _Float16 *>(addr)[o] = static_cast<_Float16>(v); break;
+          case VDT_BF16: reinterpret_cast<DVM_GLOBAL uint16_t *>(addr)[o] = static_cast<uint16_t>(f32_to_bf16_bits(v)); break;
+          default: reinterpret_cast<DVM_GLOBAL uint8_t *>(addr)[o] = v != 0.0f ? 1 : 0; break;
+        }
+      }
+    }
   }
 }
 
-__device__ __attribute__((noinline)) vf16 frag_exp(vf16 x) {
-#pragma unroll
-  for (int r = 0; r < 16; ++r) x[r] = expf(x[r]);
+__device__ __attribute__((noinline)) Slabs epi_exp(Slabs x) {
+  FOR_SE x[q] = expf(x[q]);
   return x;
 }
-__device__ __attribute__((noinline)) vf16 frag_log(vf16 x) {
-#pragma unroll
-  for (int r = 0; r < 16; ++r) x[r] = logf(x[r]);
+__device__ __attribute__((noinline)) Slabs epi_log(Slabs x) {
+  FOR_SE x[q] = logf(x[q]);
   return x;
 }
-__device__ __attribute__((noinline)) vf16 frag_pow(vf16 x, vf16 y) {
-#pragma unroll
-  for (int r = 0; r < 16; ++r) x[r] = powf(x[r], y[r]);
+__device__ __attribute__((noinline)) Slabs epi_pow(Slabs x, Slabs y) {
+  FOR_SE x[q] = powf(x[q], y[q]);
   return x;
 }
-__device__ __attribute__((noinline)) vf16 frag_sqrt(vf16 x) {
-#pragma unroll
-  for (int r = 0; r < 16; ++r) x[r] = sqrtf(x[r]);
+__device__ __attribute__((noinline)) Slabs epi_sqrt(Slabs x) {
+  FOR_SE x[q] = sqrtf(x[q]);
   return x;
 }
 
-#define FOR_R _Pragma("unroll") for (int r = 0; r < 16; ++r)
-
-__device__ __forceinline__ void apply_rnd(vf16 &a, uint32_t rnd) {
+__device__ __forceinline__ void apply_rnd(Slabs &a, uint32_t rnd) {
   if (rnd == VRND_F16) {
-    FOR_R a[r] = round_f16(a[r]);
+    FOR_SE a[q] = round_f16(a[q]);
   } else if (rnd == VRND_BF16) {
-    FOR_R a[r] = round_bf16(a[r]);
+    FOR_SE a[q] = round_bf16(a[q]);
   }
 }
 
-// Runs the epilogue program on one accumulator fragment.
 struct EpiArgs {
-  uint32_t m, n, mem_off, code_off;
+  uint32_t mem_off, code_off, batch0, batch1;
 };
 
-__device__ __attribute__((noinline)) void run_epilogue(vf16 acc, const uint32_t *prog32, EpiArgs h, uint32_t batch0, uint32_t batch1,
-                                                      uint32_t row_base, uint32_t col) {
+// Runs the epilogue program on SL slabs whose accumulator values are in `acc`.
+__device__ __forceinline__ void run_epilogue(Slabs acc, const uint32_t *prog32, const EpiArgs &h, uint32_t row0, uint32_t row1, uint32_t col,
+                                             uint32_t ncol, uint32_t rows_ok) {
   const uint32_t *code32 = prog32 + 2 * h.code_off;
-  vf16 t0 = 0.0f, t1 = 0.0f;
+  static_assert(NTEMP == 4, "temporaries are named registers");
+  Slabs t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
   uint32_t mask = 0;
   uint32_t pc = 0;
   while (true) {
@@ -233,23 +300,21 @@ __device__ __attribute__((noinline)) void run_epilogue(vf16 acc, const uint32_t 
     const uint32_t sub = (w0 >> 8) & 0xffu, a = w0 >> 24, rnd = (w0 >> 20) & 0x3u;
     if (op >= VOP_SRC_BASE || op == VOP_ST) {
       const uint32_t kind = op == VOP_ST ? static_cast<uint32_t>(VK_MEM) : ((w0 >> 16) & 0xfu);
-      vf16 src;
+      Slabs src;
       if (kind == VK_MEM) {
         const uint32_t *d = prog32 + 2 * h.mem_off + a * (sizeof(VCubeMem) / 4);
         const uint64_t addr = static_cast<uint64_t>(uni(d[0])) | (static_cast<uint64_t>(uni(d[1])) << 32);
         const uint32_t dtype = uni(d[2]), sn = uni(d[4]), sm = uni(d[5]), sb0 = uni(d[6]), sb1 = uni(d[7]);
-        const uint64_t boff = static_cast<uint64_t>(batch0) * sb0 + static_cast<uint64_t>(batch1) * sb1;
+        const uint64_t boff = static_cast<uint64_t>(h.batch0) * sb0 + static_cast<uint64_t>(h.batch1) * sb1;
         if (op == VOP_ST) {
-          Frag f;
-          f.v = acc;
-          frag_store(addr, dtype, sn, sm, boff, row_base, col, h.m, h.n, f);
+          epi_store(addr, dtype, sn, sm, boff, row0, row1, col, ncol, rows_ok, acc);
           continue;
         }
-        src = frag_load(addr, dtype, sn, sm, boff, row_base, col, h.m, h.n).v;
+        src = epi_load(addr, dtype, sn, sm, boff, row0, row1, col, ncol, rows_ok);
       } else if (kind == VK_IMM) {
         src = __uint_as_float(imm);
       } else if (kind == VK_REG) {
-        src = a == 0 ? t0 : t1;
+        src = a == 0 ? t0 : (a == 1 ? t1 : (a == 2 ? t2 : t3));
       } else {
         src = acc;
       }
@@ -265,81 +330,80 @@ __device__ __attribute__((noinline)) void run_epilogue(vf16 acc, const uint32_t 
             case VB_MUL: acc = acc * src; break;
             case VB_DIV: acc = acc / src; break;
             case VB_RDIV: acc = src / acc; break;
-            case VB_MIN: FOR_R acc[r] = acc[r] < src[r] ? acc[r] : src[r]; break;
-            case VB_MAX: FOR_R acc[r] = acc[r] > src[r] ? acc[r] : src[r]; break;
-            case VB_AND: FOR_R acc[r] = (acc[r] != 0.0f && src[r] != 0.0f) ? 1.0f : 0.0f; break;
-            case VB_OR: FOR_R acc[r] = (acc[r] != 0.0f || src[r] != 0.0f) ? 1.0f : 0.0f; break;
-            case VB_POW: acc = frag_pow(acc, src); break;
-            default: acc = frag_pow(src, acc); break;
+            case VB_MIN: FOR_SE acc[q] = acc[q] < src[q] ? acc[q] : src[q]; break;
+            case VB_MAX: FOR_SE acc[q] = acc[q] > src[q] ? acc[q] : src[q]; break;
+            case VB_AND: FOR_SE acc[q] = (acc[q] != 0.0f && src[q] != 0.0f) ? 1.0f : 0.0f; break;
+            case VB_OR: FOR_SE acc[q] = (acc[q] != 0.0f || src[q] != 0.0f) ? 1.0f : 0.0f; break;
+            case VB_POW: acc = epi_pow(acc, src); break;
+            default: acc = epi_pow(src, acc); break;
           }
           apply_rnd(acc, rnd);
           break;
         case VOP_BINI:
           switch (sub & 0x3fu) {
-            case VBI_ADD: FOR_R acc[r] = __uint_as_float(__float_as_uint(acc[r]) + __float_as_uint(src[r])); break;
-            case VBI_SUB: FOR_R acc[r] = __uint_as_float(__float_as_uint(acc[r]) - __float_as_uint(src[r])); break;
-            case VBI_RSUB: FOR_R acc[r] = __uint_as_float(__float_as_uint(src[r]) - __float_as_uint(acc[r])); break;
-            case VBI_MUL: FOR_R acc[r] = __uint_as_float(__float_as_uint(acc[r]) * __float_as_uint(src[r])); break;
-            case VBI_MIN: FOR_R acc[r] = __int_as_float(min(__float_as_int(acc[r]), __float_as_int(src[r]))); break;
-            default: FOR_R acc[r] = __int_as_float(max(__float_as_int(acc[r]), __float_as_int(src[r]))); break;
+            case VBI_ADD: FOR_SE acc[q] = __uint_as_float(__float_as_uint(acc[q]) + __float_as_uint(src[q])); break;
+            case VBI_SUB: FOR_SE acc[q] = __uint_as_float(__float_as_uint(acc[q]) - __float_as_uint(src[q])); break;
+            case VBI_RSUB: FOR_SE acc[q] = __uint_as_float(__float_as_uint(src[q]) - __float_as_uint(acc[q])); break;
+            case VBI_MUL: FOR_SE acc[q] = __uint_as_float(__float_as_uint(acc[q]) * __float_as_uint(src[q])); break;
+            case VBI_MIN: FOR_SE acc[q] = __int_as_float(min(__float_as_int(acc[q]), __float_as_int(src[q]))); break;
+            default: FOR_SE acc[q] = __int_as_float(max(__float_as_int(acc[q]), __float_as_int(src[q]))); break;
           }
           break;
         case VOP_CMP: {
           const uint32_t t = sub & 0x7u;
           if (sub & VCMP_INT) {
-            FOR_R {
-              const int32_t x = __float_as_int(acc[r]), y = __float_as_int(src[r]);
+            FOR_SE {
+              const int32_t x = __float_as_int(acc[q]), y = __float_as_int(src[q]);
               const bool c = t == VCMP_EQ ? x == y : t == VCMP_NE ? x != y : t == VCMP_GT ? x > y : t == VCMP_GE ? x >= y : t == VCMP_LT ? x < y : x <= y;
-              acc[r] = __int_as_float(c ? 1 : 0);
+              acc[q] = __int_as_float(c ? 1 : 0);
             }
           } else {
-            FOR_R {
-              const float x = acc[r], y = src[r];
+            FOR_SE {
+              const float x = acc[q], y = src[q];
               const bool c = t == VCMP_EQ ? x == y : t == VCMP_NE ? x != y : t == VCMP_GT ? x > y : t == VCMP_GE ? x >= y : t == VCMP_LT ? x < y : x <= y;
-              acc[r] = c ? 1.0f : 0.0f;
+              acc[q] = c ? 1.0f : 0.0f;
             }
           }
           break;
         }
         case VOP_MSK:
           mask = 0;
-          FOR_R mask |= ((__float_as_uint(src[r]) << 1) != 0 ? 1u : 0u) << r;
+          FOR_SE mask |= ((__float_as_uint(src[q]) << 1) != 0 ? 1u : 0u) << q;
           break;
         default:  // VOP_MOVM
-          FOR_R acc[r] = ((mask >> r) & 1u) ? src[r] : acc[r];
+          FOR_SE acc[q] = ((mask >> q) & 1u) ? src[q] : acc[q];
           break;
       }
       continue;
     }
     switch (op) {
       case VOP_LDR:
-        acc = a == 0 ? t0 : t1;
+        acc = a == 0 ? t0 : (a == 1 ? t1 : (a == 2 ? t2 : t3));
         break;
       case VOP_LDI:
         acc = __uint_as_float(imm);
         break;
       case VOP_STR:
-        if (a == 0) {
-          t0 = acc;
-        } else {
-          t1 = acc;
-        }
+        if (a == 0) t0 = acc;
+        else if (a == 1) t1 = acc;
+        else if (a == 2) t2 = acc;
+        else t3 = acc;
         break;
       case VOP_UN:
         switch (sub) {
-          case VU_SQRT: acc = frag_sqrt(acc); break;
-          case VU_ABS: FOR_R acc[r] = fabsf(acc[r]); break;
-          case VU_LOG: acc = frag_log(acc); break;
-          case VU_EXP: acc = frag_exp(acc); break;
-          case VU_ISFINITE: FOR_R acc[r] = isfinite(acc[r]) ? 1.0f : 0.0f; break;
-          case VU_ROUND: FOR_R acc[r] = rintf(acc[r]); break;
-          case VU_FLOOR: FOR_R acc[r] = floorf(acc[r]); break;
-          case VU_CEIL: FOR_R acc[r] = ceilf(acc[r]); break;
-          case VU_TRUNC: FOR_R acc[r] = truncf(acc[r]); break;
+          case VU_SQRT: acc = epi_sqrt(acc); break;
+          case VU_ABS: FOR_SE acc[q] = fabsf(acc[q]); break;
+          case VU_LOG: acc = epi_log(acc); break;
+          case VU_EXP: acc = epi_exp(acc); break;
+          case VU_ISFINITE: FOR_SE acc[q] = isfinite(acc[q]) ? 1.0f : 0.0f; break;
+          case VU_ROUND: FOR_SE acc[q] = rintf(acc[q]); break;
+          case VU_FLOOR: FOR_SE acc[q] = floorf(acc[q]); break;
+          case VU_CEIL: FOR_SE acc[q] = ceilf(acc[q]); break;
+          case VU_TRUNC: FOR_SE acc[q] = truncf(acc[q]); break;
           default:
-            FOR_R {
-              const uint32_t x = __float_as_uint(acc[r]);
-              acc[r] = __uint_as_float(static_cast<int32_t>(x) < 0 ? 0u - x : x);
+            FOR_SE {
+              const uint32_t x = __float_as_uint(acc[q]);
+              acc[q] = __uint_as_float(static_cast<int32_t>(x) < 0 ? 0u - x : x);
             }
             break;
         }
@@ -347,14 +411,14 @@ __device__ __attribute__((noinline)) void run_epilogue(vf16 acc, const uint32_t 
         break;
       case VOP_CAST:
         if (sub == VC_F2I) {
-          FOR_R acc[r] = __int_as_float(static_cast<int32_t>(acc[r]));
+          FOR_SE acc[q] = __int_as_float(static_cast<int32_t>(acc[q]));
         } else if (sub == VC_I2F) {
-          FOR_R acc[r] = static_cast<float>(__float_as_int(acc[r]));
+          FOR_SE acc[q] = static_cast<float>(__float_as_int(acc[q]));
           apply_rnd(acc, rnd);
         } else if (sub == VC_RND) {
           apply_rnd(acc, rnd);
         } else {
-          FOR_R acc[r] = acc[r] != 0.0f ? 1.0f : 0.0f;
+          FOR_SE acc[q] = acc[q] != 0.0f ? 1.0f : 0.0f;
         }
         break;
       default:
@@ -363,10 +427,49 @@ __device__ __attribute__((noinline)) void run_epilogue(vf16 acc, const uint32_t 
   }
 }
 
-// TM x TN 32x32 MFMA tiles per wave, 2 x 2 waves per workgroup.
-template <bool IS_BF16, int TM, int TN>
+// Second half of a pass: the half tile sits in local memory, row major with PITCH floats per row;
+// every lane takes slabs of 8 columns and walks the epilogue program over them.
+template <int ROWS, int BN, int TM>
+__device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
+                                                        uint32_t pass, uint32_t m, uint32_t n) {
+  constexpr int PITCH = BN + 4;
+  constexpr int GROUPS = BN / 8;               // slabs per row
+  constexpr int PER_THREAD = ROWS * GROUPS / 256;  // slabs per thread
+  static_assert(PER_THREAD % SL == 0, "slab count per thread");
+  constexpr int ROWS_PER_STEP = 256 / GROUPS;  // rows one step of all 256 threads covers
+  const uint32_t tid = threadIdx.x;
+  const uint32_t g = tid % GROUPS, r0 = tid / GROUPS;
+  constexpr int HALF = ROWS / 2;  // local rows [0, HALF) belong to the upper pair of waves, the rest to the lower pair
+  const uint32_t col = n0 + g * 8;
+  const uint32_t ncol = col >= n ? 0u : (n - col < 8u ? n - col : 8u);
+  for (int it = 0; it < PER_THREAD / SL; ++it) {
+    Slabs acc;
+    uint32_t row[SL], rows_ok = 0;
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+      const uint32_t lr = (it * SL + s) * ROWS_PER_STEP + r0;  // local row of the dump
+      const uint32_t wm = lr / HALF, rr = lr % HALF;
+      row[s] = m0 + wm * (TM * 32) + pass * HALF + rr;
+      rows_ok |= (row[s] < m ? 1u : 0u) << s;
+      const vf4 lo = *reinterpret_cast<const vf4 *>(dump + lr * PITCH + g * 8), hi = *reinterpret_cast<const vf4 *>(dump + lr * PITCH + g * 8 + 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[s * 8 + e] = lo[e];
+        acc[s * 8 + 4 + e] = hi[e];
+      }
+    }
+    run_epilogue(acc, prog32, ea, row[0], row[1], col, ncol, rows_ok);
+  }
+}
+
+// TM x TN 32x32 MFMA tiles per wave, 2 x 2 waves per workgroup; A_KC / B_KC: the operand's k axis is
+// contiguous in memory.
+template <bool IS_BF16, int TM, int TN, bool A_KC, bool B_KC>
 __device__ __forceinline__ void vm_cube(const VmParam &p) {
   constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
+  constexpr int PASSES = TM >= 2 ? 2 : 1;
+  constexpr int PROWS = BM / PASSES;  // rows of the tile one epilogue pass covers
+  constexpr int PITCH = BN + 4;
   extern __shared__ double lds_raw[];
   __shared__ uint32_t prog32[DVM_PARAM_BYTES / 4];
   {
@@ -386,9 +489,9 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
     for (int i = 0; i < static_cast<int>(sizeof(VCubeHeader) / 4); ++i) hw[i] = uni(prog32[i]);
   }
   uint16_t *lds = reinterpret_cast<uint16_t *>(lds_raw);
-  // two buffers of [A tile | B tile]; offsets in elements from `lds`, so every access stays a local-memory access
-  constexpr uint32_t kBufElems = (BM + BN) * LDS_ROW;
-  constexpr uint32_t kBOff = BM * LDS_ROW;
+  float *dump = reinterpret_cast<float *>(lds_raw);
+  // [A buffer 0 | A buffer 1 | B buffer 0 | B buffer 1], offsets in elements
+  constexpr uint32_t kABuf = BM * BK, kBBuf = BN * BK, kBBase = 2 * kABuf;
 
   const uint32_t tid = threadIdx.x;
   const uint32_t wave = tid >> 6, lane = tid & 63u;
@@ -396,12 +499,21 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
   const uint32_t tiles_per_batch = h.tiles_m * h.tiles_n;
   const uint32_t n_tiles = tiles_per_batch * h.nb0 * h.nb1;
   const uint32_t nk = (h.k + BK - 1) / BK;
-  const bool a_kc = h.trans_a == 0, b_kc = h.trans_b != 0;
+
+  // Fragment reads: fragment i of this wave is rows r0 + 32*i of the staged tile (r0 = the lane's row
+  // in fragment 0), and step kk wants chunk 2*kk + lane/32 of that row. With the swizzle of tile_off
+  // the element offset is (r0 + 32*i) * 64 + ((x ^ c) ), x = ((lane/32) ^ swz(r0)) * 8 per lane and
+  // c = (kk * 16) ^ ((i & 1) * 32) a constant: one XOR per read instead of one register per address.
+  const uint32_t a_r0 = wm * TM * 32 + (lane & 31u), b_r0 = wn * TN * 32 + (lane & 31u);
+  const uint32_t a_x = ((lane >> 5) ^ ((a_r0 ^ (a_r0 >> 3)) & 7u)) << 3, b_x = ((lane >> 5) ^ ((b_r0 ^ (b_r0 >> 3)) & 7u)) << 3;
+  const uint32_t a_row = a_r0 * BK, b_row = kBBase + b_r0 * BK;
+  auto frag_off = [](uint32_t row, uint32_t x, int f, int kk) -> uint32_t {
+    return row + static_cast<uint32_t>(f) * 32u * BK + (x ^ static_cast<uint32_t>((kk << 4) ^ ((f & 1) << 5)));
+  };
 
   for (uint32_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
     const uint32_t batch = t / tiles_per_batch, tt = t % tiles_per_batch;
     const uint32_t bi0 = batch / h.nb1, bi1 = batch % h.nb1;
-    // neighbouring workgroups share a row of A tiles: walk n fastest
     const uint32_t tm = tt / h.tiles_n, tn = tt % h.tiles_n;
     const uint32_t m0 = tm * BM, n0 = tn * BN;
     const uint64_t a_base = h.a_addr + (static_cast<uint64_t>(bi0) * h.a_sb0 + static_cast<uint64_t>(bi1) * h.a_sb1) * 2;
@@ -414,55 +526,71 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       for (int j = 0; j < TN; ++j) acc[i][j] = 0.0f;
 
     if (h.fast && m0 + BM <= h.m && n0 + BN <= h.n) {
-      Stage<BM> sa;
-      Stage<BN> sb;
-      if (a_kc) stage_load_kc<BM>(sa, a_base, h.lda, m0, 0, tid); else stage_load_ks<BM>(sa, a_base, h.lda, m0, 0, tid);
-      if (b_kc) stage_load_kc<BN>(sb, b_base, h.ldb, n0, 0, tid); else stage_load_ks<BN>(sb, b_base, h.ldb, n0, 0, tid);
-      if (a_kc) stage_store_kc<BM>(sa, lds, tid); else stage_store_ks<BM>(sa, lds, tid);
-      if (b_kc) stage_store_kc<BN>(sb, lds + kBOff, tid); else stage_store_ks<BN>(sb, lds + kBOff, tid);
+      Stage<BM, A_KC> sa;
+      Stage<BN, B_KC> sb;
+      // address of element (row0, k) of each operand, k advancing by BK per step
+      const uint64_t a_org = a_base + (A_KC ? static_cast<uint64_t>(m0) * h.lda : static_cast<uint64_t>(m0)) * 2;
+      const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb : static_cast<uint64_t>(n0)) * 2;
+      const uint64_t a_step = (A_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.lda) * 2;
+      const uint64_t b_step = (B_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.ldb) * 2;
+      const uint32_t a_voff = Stage<BM, A_KC>::lane_offset(h.lda, tid), b_voff = Stage<BN, B_KC>::lane_offset(h.ldb, tid);
+      sa.load(a_org, h.lda, a_voff, tid);
+      sb.load(b_org, h.ldb, b_voff, tid);
+      sa.store(lds, tid);
+      sb.store(lds + kBBase, tid);
       __syncthreads();
+      vu4 af[2][TM], bf[2][TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const vu4 *>(lds + frag_off(a_row, a_x, i, 0));
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const vu4 *>(lds + frag_off(b_row, b_x, j, 0));
       for (uint32_t kt = 0; kt < nk; ++kt) {
         const uint32_t cur = kt & 1u;
         const bool more = kt + 1 < nk;
+        const uint16_t *abuf = lds + cur * kABuf, *bbuf = lds + cur * kBBuf;
         if (more) {
-          const uint32_t k0 = (kt + 1) * BK;
-          if (a_kc) stage_load_kc<BM>(sa, a_base, h.lda, m0, k0, tid); else stage_load_ks<BM>(sa, a_base, h.lda, m0, k0, tid);
-          if (b_kc) stage_load_kc<BN>(sb, b_base, h.ldb, n0, k0, tid); else stage_load_ks<BN>(sb, b_base, h.ldb, n0, k0, tid);
+          sa.load(a_org + (kt + 1) * a_step, h.lda, a_voff, tid);
+          sb.load(b_org + (kt + 1) * b_step, h.ldb, b_voff, tid);
         }
-        const uint16_t *at = lds + cur * kBufElems + (wm * TM * 32 + (lane & 31u)) * LDS_ROW + (lane >> 5) * 8;
-        const uint16_t *bt = lds + cur * kBufElems + kBOff + (wn * TN * 32 + (lane & 31u)) * LDS_ROW + (lane >> 5) * 8;
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
-          vu4 af[TM], bf[TN];
+          constexpr int LAST = BK / 16 - 1;
+          if (kk < LAST) {
 #pragma unroll
-          for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const vu4 *>(at + i * 32 * LDS_ROW + kk * 16);
+            for (int i = 0; i < TM; ++i) af[(kk + 1) & 1][i] = *reinterpret_cast<const vu4 *>(abuf + frag_off(a_row, a_x, i, kk + 1));
 #pragma unroll
-          for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const vu4 *>(bt + j * 32 * LDS_ROW + kk * 16);
+            for (int j = 0; j < TN; ++j) bf[(kk + 1) & 1][j] = *reinterpret_cast<const vu4 *>(bbuf + frag_off(b_row, b_x, j, kk + 1));
+          } else if (more) {
+            // the next tile goes to the other buffer while the last MFMAs of this one run
+            sa.store(lds + (cur ^ 1u) * kABuf, tid);
+            sb.store(lds + kBBase + (cur ^ 1u) * kBBuf, tid);
+          }
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = mfma<IS_BF16>(af[i], bf[j], acc[i][j]);
-        }
-        if (more) {
-          if (a_kc) stage_store_kc<BM>(sa, lds + (cur ^ 1u) * kBufElems, tid); else stage_store_ks<BM>(sa, lds + (cur ^ 1u) * kBufElems, tid);
-          if (b_kc) stage_store_kc<BN>(sb, lds + (cur ^ 1u) * kBufElems + kBOff, tid); else stage_store_ks<BN>(sb, lds + (cur ^ 1u) * kBufElems + kBOff, tid);
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma<IS_BF16>(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
         }
         __syncthreads();
+        if (more) {
+          const uint16_t *an = lds + (cur ^ 1u) * kABuf, *bn = lds + (cur ^ 1u) * kBBuf;
+#pragma unroll
+          for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const vu4 *>(an + frag_off(a_row, a_x, i, 0));
+#pragma unroll
+          for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const vu4 *>(bn + frag_off(b_row, b_x, j, 0));
+        }
       }
     } else {
       for (uint32_t kt = 0; kt < nk; ++kt) {
-        stage_generic<BM>(lds, a_base, h.lda, m0, kt * BK, h.m, h.k, a_kc ? 1u : 0u, tid);
-        stage_generic<BN>(lds + kBOff, b_base, h.ldb, n0, kt * BK, h.n, h.k, b_kc ? 1u : 0u, tid);
+        stage_generic<BM>(lds, a_base, h.lda, m0, kt * BK, h.m, h.k, A_KC ? 1u : 0u, tid);
+        stage_generic<BN>(lds + kBBase, b_base, h.ldb, n0, kt * BK, h.n, h.k, B_KC ? 1u : 0u, tid);
         __syncthreads();
-        const uint16_t *at = lds + (wm * TM * 32 + (lane & 31u)) * LDS_ROW + (lane >> 5) * 8;
-        const uint16_t *bt = lds + kBOff + (wn * TN * 32 + (lane & 31u)) * LDS_ROW + (lane >> 5) * 8;
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
           vu4 af[TM], bf[TN];
 #pragma unroll
-          for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const vu4 *>(at + i * 32 * LDS_ROW + kk * 16);
+          for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const vu4 *>(lds + frag_off(a_row, a_x, i, kk));
 #pragma unroll
-          for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const vu4 *>(bt + j * 32 * LDS_ROW + kk * 16);
+          for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const vu4 *>(lds + frag_off(b_row, b_x, j, kk));
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -472,25 +600,42 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       }
     }
 
-    // epilogue, fragment by fragment, straight from the accumulators
-    const EpiArgs ea = {h.m, h.n, h.mem_off, h.code_off};
+    // epilogue: accumulators -> local memory (row major), then slabs through the program
+    const EpiArgs ea = {h.mem_off, h.code_off, bi0, bi1};
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    for (int ps = 0; ps < PASSES; ++ps) {
+      constexpr int FR = TM / PASSES;  // fragment rows of a wave per pass
 #pragma unroll
-      for (int j = 0; j < TN; ++j) {
-        const uint32_t row_base = m0 + (wm * TM + i) * 32 + (lane >> 5) * 4;
-        const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31u);
-        run_epilogue(acc[i][j], prog32, ea, bi0, bi1, row_base, col);
+      for (int fi = 0; fi < FR; ++fi) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const vf16 &c = acc[ps * FR + fi][j];
+          // lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4 of the fragment
+          float *dst = dump + (wm * (PROWS / 2) + fi * 32 + (lane >> 5) * 4) * PITCH + (wn * TN + j) * 32 + (lane & 31u);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) dst[(8 * (r / 4) + (r % 4)) * PITCH] = c[r];
+        }
       }
+      __syncthreads();
+      epilogue_pass<PROWS, BN, TM>(dump, prog32, ea, m0, n0, ps, h.m, h.n);
+      __syncthreads();
     }
   }
 }
 
 }  // namespace
 
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_cube_bf16_big(const VmParam p) { vm_cube<true, 4, 4>(p); }
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_cube_f16_big(const VmParam p) { vm_cube<false, 4, 4>(p); }
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_cube_bf16_mid(const VmParam p) { vm_cube<true, 2, 2>(p); }
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_cube_f16_mid(const VmParam p) { vm_cube<false, 2, 2>(p); }
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_cube_bf16_small(const VmParam p) { vm_cube<true, 1, 1>(p); }
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_cube_f16_small(const VmParam p) { vm_cube<false, 1, 1>(p); }
+#define DVM_CUBE_KERNEL(name, bf, tm, akc, bkc) \
+  extern "C" __global__ void __launch_bounds__(256) name(const VmParam p) { vm_cube<bf, tm, tm, akc, bkc>(p); }
+#define DVM_CUBE_LAYOUTS(prefix, bf, tm)            \
+  DVM_CUBE_KERNEL(prefix##_nn, bf, tm, true, false) \
+  DVM_CUBE_KERNEL(prefix##_nt, bf, tm, true, true)  \
+  DVM_CUBE_KERNEL(prefix##_tn, bf, tm, false, false) \
+  DVM_CUBE_KERNEL(prefix##_tt, bf, tm, false, true)
+
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_big, true, 4)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_big, false, 4)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_mid, true, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_mid, false, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_small, true, 1)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_small, false, 1)

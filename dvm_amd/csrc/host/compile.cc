@@ -1746,7 +1746,7 @@ void Compiler::CompileCube(int a) {
   h.tiles_m = static_cast<uint32_t>((M + bt - 1) / bt);
   h.tiles_n = static_cast<uint32_t>((N + bt - 1) / bt);
   if (tiles(bt) >= (1ull << 31)) Fail("too many matmul tiles");
-  h.fast = (K % 64 == 0 && K > 0 && h.lda % 8 == 0 && h.ldb % 8 == 0 && h.a_sb0 % 8 == 0 &&
+  h.fast = (K % 64 == 0 && K > 0 && h.lda < (1u << 22) && h.ldb < (1u << 22) && h.lda % 8 == 0 && h.ldb % 8 == 0 && h.a_sb0 % 8 == 0 &&
             h.a_sb1 % 8 == 0 && h.b_sb0 % 8 == 0 && h.b_sb1 % 8 == 0)
                ? 1
                : 0;
@@ -1811,7 +1811,7 @@ void Compiler::CompileCube(int a) {
   std::memcpy(prog_->blob.w + h.mem_off, cmems_, sizeof(VCubeMem) * n_mem_);
   std::memcpy(prog_->blob.w + h.code_off, code_.data(), 8 * code_.size());
   prog_->threads = 256;
-  prog_->lds_bytes = static_cast<uint32_t>(2 * (2 * bt) * (64 + 8) * 2);
+  prog_->lds_bytes = DVM_CUBE_LDS_BYTES(static_cast<uint32_t>(bt));
   prog_->grid = static_cast<uint32_t>(tiles(bt));
 }
 

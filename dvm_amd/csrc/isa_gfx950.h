@@ -162,10 +162,10 @@ typedef struct {
 // in the vector VM's instruction words runs on every accumulator fragment (acc = the 16 values a
 // lane holds of one 32x32 tile) before anything is stored: VOP_CAST / VOP_UN / VOP_BINF / VOP_BINI /
 // VOP_CMP / VOP_MSK / VOP_MOVM with VK_IMM, VK_ACC, VK_MEM (stride-addressed, so a bias row is a
-// stride-0 operand) or VK_REG (two fragment-sized temporaries), VOP_STR / VOP_LDR on those
+// stride-0 operand) or VK_REG (DVM_CUBE_NTEMP temporaries), VOP_STR / VOP_LDR on those
 // temporaries, VOP_ST to one or more outputs.
 #define DVM_CUBE_MAXMEM 12
-#define DVM_CUBE_NTEMP 2
+#define DVM_CUBE_NTEMP 4
 
 typedef struct {
   uint64_t addr;
@@ -194,6 +194,13 @@ typedef struct {
   uint32_t pad;
   uint64_t a_addr, b_addr;
 } VCubeHeader;
+
+// Dynamic local memory a VE_CUBE launch needs for block tile `bt` (256, 128 or 64): the double-buffered
+// operand tiles of the k loop, or the half tile of fp32 accumulators the epilogue reads back.
+#define DVM_CUBE_LDS_BYTES(bt) \
+  ((2u * (2u * (bt)) * 64u * 2u) > (((bt) >= 128u ? (bt) / 2u : (bt)) * ((bt) + 4u) * 4u) \
+       ? (2u * (2u * (bt)) * 64u * 2u) \
+       : (((bt) >= 128u ? (bt) / 2u : (bt)) * ((bt) + 4u) * 4u))
 
 typedef struct {
   uint64_t w[DVM_PARAM_WORDS];
