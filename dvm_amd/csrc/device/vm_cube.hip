@@ -22,6 +22,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "../isa_gfx950.h"
 
 namespace {
@@ -36,19 +38,25 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 
 constexpr int BK = 64;   // k extent of a staged tile = one 128-byte row of 16-bit elements
-constexpr int SL = 2;    // slabs of 8 columns the epilogue interpreter handles per walk of the program
 constexpr int NTEMP = DVM_CUBE_NTEMP;
 
 __device__ __forceinline__ uint32_t uni(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 
 __device__ __forceinline__ float round_f16(float x) { return static_cast<float>(static_cast<_Float16>(x)); }
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float x) {
-  uint32_t u = __float_as_uint(x);
-  uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);
-  r = (x != x) ? 0x7fc00000u : r;
-  return r >> 16;
+// gfx950 converts fp32 to bf16 in hardware (round to nearest even, NaN stays NaN): v_cvt_pk_bf16_f32
+typedef float vf2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float x) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(x)); }
+__device__ __forceinline__ float round_bf16(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  const vf2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
-__device__ __forceinline__ float round_bf16(float x) { return __uint_as_float(f32_to_bf16_bits(x) << 16); }
+__device__ __forceinline__ uint32_t pack_f16(float lo, float hi) {
+  const vf2 v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, half2v));
+}
 
 template <bool IS_BF16>
 __device__ __forceinline__ vf16 mfma(vu4 a, vu4 b, vf16 c) {
@@ -150,127 +158,269 @@ __device__ __attribute__((noinline)) void stage_generic(uint16_t *tile, uint64_t
 
 // ---- epilogue ---------------------------------------------------------------------------------------
 // A slab is 8 consecutive columns of one row of the output; the interpreter works on SL slabs at a
-// time, held as one 16-wide vector of fp32 containers (element s*8 + e = column e of slab s) so that
-// values travel between the out-of-line helpers in registers.
-static_assert(SL == 2, "the slab vector is 16 wide");
-typedef vf16 Slabs;
+// time (4 when a lane has that many per pass, else 2), held as one vector of fp32 containers
+// (element s*8 + e = column e of slab s): with one wave per SIMD the independent elements are what
+// hides the VALU latency.
+typedef float vf32 __attribute__((ext_vector_type(32)));
+template <int SL> struct SlabVec;
+template <> struct SlabVec<2> { typedef vf16 type; };
+template <> struct SlabVec<4> { typedef vf32 type; };
 
 #define FOR_SE _Pragma("unroll") for (int q = 0; q < SL * 8; ++q)
+
+struct SlabRows {
+  uint32_t row[4];  // output row of each slab
+  uint32_t ok;      // bit s: slab s is inside the output
+};
+
+typedef float vf8 __attribute__((ext_vector_type(8)));
+
+__device__ __forceinline__ bool wave_all(bool c) { return __builtin_amdgcn_ballot_w64(!c) == 0; }
 
 __device__ __forceinline__ float cvt_in(uint32_t dtype, uint32_t bits16) {
   return dtype == VDT_F16 ? static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits16))) : __uint_as_float(bits16 << 16);
 }
 
-// row0/row1: output rows of the two slabs, col: first column, ncol: columns inside the output (0..8),
-// rows_ok: bit s set when slab s is inside the output.
-__device__ __attribute__((noinline)) Slabs epi_load(uint64_t addr, uint32_t dtype, uint32_t sn, uint32_t sm, uint64_t boff, uint32_t row0,
-                                                   uint32_t row1, uint32_t col, uint32_t ncol, uint32_t rows_ok) {
-  Slabs out;
+__device__ __forceinline__ uint32_t elem_size(uint32_t dtype) {
+  return (dtype == VDT_F32 || dtype == VDT_I32) ? 4u : (dtype == VDT_BOOL ? 1u : 2u);
+}
+
+// One slab, element by element, with every guard: edges, strided or unaligned operands.
+__device__ __attribute__((noinline)) vf8 slab_load_slow(uint64_t addr, uint32_t dtype, uint32_t sn, uint64_t off, uint32_t ncol, uint32_t ok) {
+  vf8 out;
 #pragma unroll
-  for (int s = 0; s < SL; ++s) {
-    const bool ok = (rows_ok >> s) & 1u;
-    const uint64_t off = boff + static_cast<uint64_t>(s == 0 ? row0 : row1) * sm + static_cast<uint64_t>(col) * sn;
-    const uint32_t esz = (dtype == VDT_F32 || dtype == VDT_I32) ? 4u : (dtype == VDT_BOOL ? 1u : 2u);
-    const bool vec = ok && sn == 1 && ncol == 8 && ((addr + off * esz) & 15u) == 0;
-    if (vec && esz == 4) {
-      const vu4 a = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + off * 4), b = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + off * 4 + 16);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        out[s * 8 + e] = __uint_as_float(a[e]);
-        out[s * 8 + 4 + e] = __uint_as_float(b[e]);
-      }
-    } else if (vec && esz == 2) {
-      const vu4 a = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + off * 2);
-#pragma unroll
-      for (int e = 0; e < 8; ++e) out[s * 8 + e] = cvt_in(dtype, (a[e >> 1] >> (16 * (e & 1))) & 0xffffu);
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float v = 0.0f;
-        if (ok && static_cast<uint32_t>(e) < ncol) {
-          const uint64_t o = off + static_cast<uint64_t>(e) * sn;
-          switch (dtype) {
-            case VDT_F32: v = reinterpret_cast<const DVM_GLOBAL float *>(addr)[o]; break;
-            case VDT_I32: v = __int_as_float(reinterpret_cast<const DVM_GLOBAL int32_t *>(addr)[o]); break;
-            case VDT_F16:
-            case VDT_BF16: v = cvt_in(dtype, reinterpret_cast<const DVM_GLOBAL uint16_t *>(addr)[o]); break;
-            default: v = reinterpret_cast<const DVM_GLOBAL uint8_t *>(addr)[o] != 0 ? 1.0f : 0.0f; break;
-          }
-        }
-        out[s * 8 + e] = v;
+  for (int e = 0; e < 8; ++e) {
+    float v = 0.0f;
+    if (ok != 0 && static_cast<uint32_t>(e) < ncol) {
+      const uint64_t o = off + static_cast<uint64_t>(e) * sn;
+      switch (dtype) {
+        case VDT_F32: v = reinterpret_cast<const DVM_GLOBAL float *>(addr)[o]; break;
+        case VDT_I32: v = __int_as_float(reinterpret_cast<const DVM_GLOBAL int32_t *>(addr)[o]); break;
+        case VDT_F16:
+        case VDT_BF16: v = cvt_in(dtype, reinterpret_cast<const DVM_GLOBAL uint16_t *>(addr)[o]); break;
+        default: v = reinterpret_cast<const DVM_GLOBAL uint8_t *>(addr)[o] != 0 ? 1.0f : 0.0f; break;
       }
     }
+    out[e] = v;
   }
   return out;
 }
 
-__device__ __attribute__((noinline)) void epi_store(uint64_t addr, uint32_t dtype, uint32_t sn, uint32_t sm, uint64_t boff, uint32_t row0,
-                                                   uint32_t row1, uint32_t col, uint32_t ncol, uint32_t rows_ok, Slabs x) {
+__device__ __attribute__((noinline)) void slab_store_slow(uint64_t addr, uint32_t dtype, uint32_t sn, uint64_t off, uint32_t ncol, uint32_t ok, vf8 x) {
+  if (ok == 0) return;
 #pragma unroll
-  for (int s = 0; s < SL; ++s) {
-    if (!((rows_ok >> s) & 1u) || ncol == 0) continue;
-    const uint64_t off = boff + static_cast<uint64_t>(s == 0 ? row0 : row1) * sm + static_cast<uint64_t>(col) * sn;
-    const uint32_t esz = (dtype == VDT_F32 || dtype == VDT_I32) ? 4u : (dtype == VDT_BOOL ? 1u : 2u);
-    const bool vec = sn == 1 && ncol == 8 && ((addr + off * esz) & 15u) == 0;
-    if (vec && esz == 4) {
-      vu4 a, b;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        a[e] = __float_as_uint(x[s * 8 + e]);
-        b[e] = __float_as_uint(x[s * 8 + 4 + e]);
-      }
-      *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + off * 4) = a;
-      *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + off * 4 + 16) = b;
-    } else if (vec && esz == 2) {
-      vu4 a;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        uint32_t lo, hi;
-        if (dtype == VDT_F16) {
-          lo = __builtin_bit_cast(uint16_t, static_cast<_Float16>(x[s * 8 + 2 * e]));
-          hi = __builtin_bit_cast(uint16_t, static_cast<_Float16>(x[s * 8 + 2 * e + 1]));
-        } else {
-          lo = f32_to_bf16_bits(x[s * 8 + 2 * e]);
-          hi = f32_to_bf16_bits(x[s * 8 + 2 * e + 1]);
-        }
-        a[e] = lo | (hi << 16);
-      }
-      *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + off * 2) = a;
-    } else {
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        if (static_cast<uint32_t>(e) >= ncol) continue;
-        const uint64_t o = off + static_cast<uint64_t>(e) * sn;
-        const float v = x[s * 8 + e];
-        switch (dtype) {
-          case VDT_F32: reinterpret_cast<DVM_GLOBAL float *>(addr)[o] = v; break;
-          case VDT_I32: reinterpret_cast<DVM_GLOBAL int32_t *>(addr)[o] = __float_as_int(v); break;
-          case VDT_F16: reinterpret_cast<DVM_GLOBAL _Float16 *>(addr)[o] = static_cast<_Float16>(v); break;
-          case VDT_BF16: reinterpret_cast<DVM_GLOBAL uint16_t *>(addr)[o] = static_cast<uint16_t>(f32_to_bf16_bits(v)); break;
-          default: reinterpret_cast<DVM_GLOBAL uint8_t *>(addr)[o] = v != 0.0f ? 1 : 0; break;
-        }
-      }
+  for (int e = 0; e < 8; ++e) {
+    if (static_cast<uint32_t>(e) >= ncol) continue;
+    const uint64_t o = off + static_cast<uint64_t>(e) * sn;
+    const float v = x[e];
+    switch (dtype) {
+      case VDT_F32: reinterpret_cast<DVM_GLOBAL float *>(addr)[o] = v; break;
+      case VDT_I32: reinterpret_cast<DVM_GLOBAL int32_t *>(addr)[o] = __float_as_int(v); break;
+      case VDT_F16: reinterpret_cast<DVM_GLOBAL _Float16 *>(addr)[o] = static_cast<_Float16>(v); break;
+      case VDT_BF16: reinterpret_cast<DVM_GLOBAL uint16_t *>(addr)[o] = static_cast<uint16_t>(f32_to_bf16_bits(v)); break;
+      default: reinterpret_cast<DVM_GLOBAL uint8_t *>(addr)[o] = v != 0.0f ? 1 : 0; break;
     }
   }
 }
 
-__device__ __attribute__((noinline)) Slabs epi_exp(Slabs x) {
-  FOR_SE x[q] = expf(x[q]);
-  return x;
-}
-__device__ __attribute__((noinline)) Slabs epi_log(Slabs x) {
-  FOR_SE x[q] = logf(x[q]);
-  return x;
-}
-__device__ __attribute__((noinline)) Slabs epi_pow(Slabs x, Slabs y) {
-  FOR_SE x[q] = powf(x[q], y[q]);
-  return x;
-}
-__device__ __attribute__((noinline)) Slabs epi_sqrt(Slabs x) {
-  FOR_SE x[q] = sqrtf(x[q]);
-  return x;
+// Memory operand of the epilogue for SL slabs. col: first column of the slabs, ncol: columns inside
+// the output (0..8). The whole wave takes one of three routes (the decision is a wave vote, so the
+// common routes carry no per-lane control flow): 128-bit accesses when every lane's slabs are full,
+// contiguous and 16-byte aligned; one element per slab when the operand does not vary along a row
+// (a column of biases, a scalar); the guarded element loop otherwise.
+template <int SL>
+__device__ __forceinline__ typename SlabVec<SL>::type epi_load(uint64_t addr, uint32_t dtype, uint32_t sn, uint32_t sm, uint64_t boff,
+                                                                const SlabRows &rows, uint32_t col, uint32_t ncol) {
+  typename SlabVec<SL>::type out;
+  const uint32_t esz = elem_size(dtype);
+  const uint32_t full = (1u << SL) - 1u;
+  const uint64_t col_off = boff + static_cast<uint64_t>(col) * sn;
+  const bool wide = sn == 1 && esz != 1 && ((static_cast<uint64_t>(sm) * esz) & 15u) == 0 &&
+                    wave_all(rows.ok == full && ncol == 8 && ((addr + col_off * esz) & 15u) == 0);
+  if (wide) {
+    // an operand that does not vary with the row (a bias row) is fetched once
+    const int distinct = sm == 0 ? 1 : SL;
+    if (esz == 4) {
+#pragma unroll
+      for (int s = 0; s < SL; ++s) {
+        if (s < distinct) {
+          const uint64_t o = (col_off + static_cast<uint64_t>(rows.row[s]) * sm) * 4;
+          const vu4 a = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + o), b = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + o + 16);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            out[s * 8 + e] = __uint_as_float(a[e]);
+            out[s * 8 + 4 + e] = __uint_as_float(b[e]);
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) out[s * 8 + e] = out[e];
+        }
+      }
+    } else {
+      const bool f16 = dtype == VDT_F16;
+#pragma unroll
+      for (int s = 0; s < SL; ++s) {
+        if (s < distinct) {
+          const vu4 a = *reinterpret_cast<const DVM_GLOBAL vu4 *>(addr + (col_off + static_cast<uint64_t>(rows.row[s]) * sm) * 2);
+          if (f16) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              out[s * 8 + e] = static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>((a[e >> 1] >> (16 * (e & 1))) & 0xffffu)));
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) out[s * 8 + e] = __uint_as_float((e & 1) ? (a[e >> 1] & 0xffff0000u) : (a[e >> 1] << 16));
+          }
+        } else {
+#pragma unroll
+          for (int e = 0; e < 8; ++e) out[s * 8 + e] = out[e];
+        }
+      }
+    }
+    return out;
+  }
+  if (sn == 0 && wave_all(rows.ok == full)) {
+#pragma unroll
+    for (int s = 0; s < SL; ++s) {
+      const uint64_t o = col_off + static_cast<uint64_t>(rows.row[s]) * sm;
+      float v;
+      switch (dtype) {
+        case VDT_F32: v = reinterpret_cast<const DVM_GLOBAL float *>(addr)[o]; break;
+        case VDT_I32: v = __int_as_float(reinterpret_cast<const DVM_GLOBAL int32_t *>(addr)[o]); break;
+        case VDT_F16:
+        case VDT_BF16: v = cvt_in(dtype, reinterpret_cast<const DVM_GLOBAL uint16_t *>(addr)[o]); break;
+        default: v = reinterpret_cast<const DVM_GLOBAL uint8_t *>(addr)[o] != 0 ? 1.0f : 0.0f; break;
+      }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[s * 8 + e] = v;
+    }
+    return out;
+  }
+#pragma unroll
+  for (int s = 0; s < SL; ++s) {
+    const vf8 v = slab_load_slow(addr, dtype, sn, col_off + static_cast<uint64_t>(rows.row[s]) * sm, ncol, (rows.ok >> s) & 1u);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) out[s * 8 + e] = v[e];
+  }
+  return out;
 }
 
+template <int SL>
+__device__ __forceinline__ void epi_store(uint64_t addr, uint32_t dtype, uint32_t sn, uint32_t sm, uint64_t boff, const SlabRows &rows,
+                                          uint32_t col, uint32_t ncol, const typename SlabVec<SL>::type &x) {
+  const uint32_t esz = elem_size(dtype);
+  const uint32_t full = (1u << SL) - 1u;
+  const uint64_t col_off = boff + static_cast<uint64_t>(col) * sn;
+  const bool wide = sn == 1 && esz != 1 && ((static_cast<uint64_t>(sm) * esz) & 15u) == 0 &&
+                    wave_all(rows.ok == full && ncol == 8 && ((addr + col_off * esz) & 15u) == 0);
+  if (wide) {
+    if (esz == 4) {
+#pragma unroll
+      for (int s = 0; s < SL; ++s) {
+        const uint64_t o = (col_off + static_cast<uint64_t>(rows.row[s]) * sm) * 4;
+        vu4 a, b;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          a[e] = __float_as_uint(x[s * 8 + e]);
+          b[e] = __float_as_uint(x[s * 8 + 4 + e]);
+        }
+        *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + o) = a;
+        *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + o + 16) = b;
+      }
+    } else if (dtype == VDT_F16) {
+#pragma unroll
+      for (int s = 0; s < SL; ++s) {
+        vu4 a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[e] = pack_f16(x[s * 8 + 2 * e], x[s * 8 + 2 * e + 1]);
+        *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + (col_off + static_cast<uint64_t>(rows.row[s]) * sm) * 2) = a;
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < SL; ++s) {
+        vu4 a;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a[e] = pack_bf16(x[s * 8 + 2 * e], x[s * 8 + 2 * e + 1]);
+        *reinterpret_cast<DVM_GLOBAL vu4 *>(addr + (col_off + static_cast<uint64_t>(rows.row[s]) * sm) * 2) = a;
+      }
+    }
+    return;
+  }
+#pragma unroll
+  for (int s = 0; s < SL; ++s) {
+    vf8 v;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) v[e] = x[s * 8 + e];
+    slab_store_slow(addr, dtype, sn, col_off + static_cast<uint64_t>(rows.row[s]) * sm, ncol, (rows.ok >> s) & 1u, v);
+  }
+}
+
+// out-of-line math on 16 values at a time (arguments and results travel in registers)
+__device__ __attribute__((noinline)) vf16 math_exp(vf16 x) {
+#pragma unroll
+  for (int q = 0; q < 16; ++q) x[q] = expf(x[q]);
+  return x;
+}
+__device__ __attribute__((noinline)) vf16 math_log(vf16 x) {
+#pragma unroll
+  for (int q = 0; q < 16; ++q) x[q] = logf(x[q]);
+  return x;
+}
+__device__ __attribute__((noinline)) vf16 math_pow(vf16 x, vf16 y) {
+#pragma unroll
+  for (int q = 0; q < 16; ++q) x[q] = powf(x[q], y[q]);
+  return x;
+}
+__device__ __attribute__((noinline)) vf16 math_sqrt(vf16 x) {
+#pragma unroll
+  for (int q = 0; q < 16; ++q) x[q] = sqrtf(x[q]);
+  return x;
+}
+template <int SL, typename V, typename F>
+__device__ __forceinline__ V by_halves(V x, F f) {
+  if constexpr (SL == 2) {
+    return f(x);
+  } else {
+    vf16 lo, hi;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      lo[q] = x[q];
+      hi[q] = x[16 + q];
+    }
+    lo = f(lo);
+    hi = f(hi);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      x[q] = lo[q];
+      x[16 + q] = hi[q];
+    }
+    return x;
+  }
+}
+template <int SL, typename V>
+__device__ __forceinline__ V slab_pow(V x, V y) {
+  if constexpr (SL == 2) {
+    return math_pow(x, y);
+  } else {
+    vf16 xl, xh, yl, yh;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      xl[q] = x[q];
+      xh[q] = x[16 + q];
+      yl[q] = y[q];
+      yh[q] = y[16 + q];
+    }
+    xl = math_pow(xl, yl);
+    xh = math_pow(xh, yh);
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      x[q] = xl[q];
+      x[16 + q] = xh[q];
+    }
+    return x;
+  }
+}
+
+template <int SL, typename Slabs>
 __device__ __forceinline__ void apply_rnd(Slabs &a, uint32_t rnd) {
   if (rnd == VRND_F16) {
     FOR_SE a[q] = round_f16(a[q]);
@@ -284,8 +434,10 @@ struct EpiArgs {
 };
 
 // Runs the epilogue program on SL slabs whose accumulator values are in `acc`.
-__device__ __forceinline__ void run_epilogue(Slabs acc, const uint32_t *prog32, const EpiArgs &h, uint32_t row0, uint32_t row1, uint32_t col,
-                                             uint32_t ncol, uint32_t rows_ok) {
+template <int SL>
+__device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, const uint32_t *prog32, const EpiArgs &h, const SlabRows &rows,
+                                             uint32_t col, uint32_t ncol) {
+  typedef typename SlabVec<SL>::type Slabs;
   const uint32_t *code32 = prog32 + 2 * h.code_off;
   static_assert(NTEMP == 4, "temporaries are named registers");
   Slabs t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
@@ -307,10 +459,10 @@ __device__ __forceinline__ void run_epilogue(Slabs acc, const uint32_t *prog32, 
         const uint32_t dtype = uni(d[2]), sn = uni(d[4]), sm = uni(d[5]), sb0 = uni(d[6]), sb1 = uni(d[7]);
         const uint64_t boff = static_cast<uint64_t>(h.batch0) * sb0 + static_cast<uint64_t>(h.batch1) * sb1;
         if (op == VOP_ST) {
-          epi_store(addr, dtype, sn, sm, boff, row0, row1, col, ncol, rows_ok, acc);
+          epi_store<SL>(addr, dtype, sn, sm, boff, rows, col, ncol, acc);
           continue;
         }
-        src = epi_load(addr, dtype, sn, sm, boff, row0, row1, col, ncol, rows_ok);
+        src = epi_load<SL>(addr, dtype, sn, sm, boff, rows, col, ncol);
       } else if (kind == VK_IMM) {
         src = __uint_as_float(imm);
       } else if (kind == VK_REG) {
@@ -334,10 +486,10 @@ __device__ __forceinline__ void run_epilogue(Slabs acc, const uint32_t *prog32, 
             case VB_MAX: FOR_SE acc[q] = acc[q] > src[q] ? acc[q] : src[q]; break;
             case VB_AND: FOR_SE acc[q] = (acc[q] != 0.0f && src[q] != 0.0f) ? 1.0f : 0.0f; break;
             case VB_OR: FOR_SE acc[q] = (acc[q] != 0.0f || src[q] != 0.0f) ? 1.0f : 0.0f; break;
-            case VB_POW: acc = epi_pow(acc, src); break;
-            default: acc = epi_pow(src, acc); break;
+            case VB_POW: acc = slab_pow<SL>(acc, src); break;
+            default: acc = slab_pow<SL>(src, acc); break;
           }
-          apply_rnd(acc, rnd);
+          apply_rnd<SL>(acc, rnd);
           break;
         case VOP_BINI:
           switch (sub & 0x3fu) {
@@ -391,10 +543,10 @@ __device__ __forceinline__ void run_epilogue(Slabs acc, const uint32_t *prog32, 
         break;
       case VOP_UN:
         switch (sub) {
-          case VU_SQRT: acc = epi_sqrt(acc); break;
+          case VU_SQRT: acc = by_halves<SL>(acc, math_sqrt); break;
           case VU_ABS: FOR_SE acc[q] = fabsf(acc[q]); break;
-          case VU_LOG: acc = epi_log(acc); break;
-          case VU_EXP: acc = epi_exp(acc); break;
+          case VU_LOG: acc = by_halves<SL>(acc, math_log); break;
+          case VU_EXP: acc = by_halves<SL>(acc, math_exp); break;
           case VU_ISFINITE: FOR_SE acc[q] = isfinite(acc[q]) ? 1.0f : 0.0f; break;
           case VU_ROUND: FOR_SE acc[q] = rintf(acc[q]); break;
           case VU_FLOOR: FOR_SE acc[q] = floorf(acc[q]); break;
@@ -407,16 +559,16 @@ __device__ __forceinline__ void run_epilogue(Slabs acc, const uint32_t *prog32, 
             }
             break;
         }
-        apply_rnd(acc, rnd);
+        apply_rnd<SL>(acc, rnd);
         break;
       case VOP_CAST:
         if (sub == VC_F2I) {
           FOR_SE acc[q] = __int_as_float(static_cast<int32_t>(acc[q]));
         } else if (sub == VC_I2F) {
           FOR_SE acc[q] = static_cast<float>(__float_as_int(acc[q]));
-          apply_rnd(acc, rnd);
+          apply_rnd<SL>(acc, rnd);
         } else if (sub == VC_RND) {
-          apply_rnd(acc, rnd);
+          apply_rnd<SL>(acc, rnd);
         } else {
           FOR_SE acc[q] = acc[q] != 0.0f ? 1.0f : 0.0f;
         }
@@ -435,6 +587,7 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
   constexpr int PITCH = BN + 4;
   constexpr int GROUPS = BN / 8;               // slabs per row
   constexpr int PER_THREAD = ROWS * GROUPS / 256;  // slabs per thread
+  constexpr int SL = PER_THREAD % 4 == 0 ? 4 : 2;
   static_assert(PER_THREAD % SL == 0, "slab count per thread");
   constexpr int ROWS_PER_STEP = 256 / GROUPS;  // rows one step of all 256 threads covers
   const uint32_t tid = threadIdx.x;
@@ -443,14 +596,15 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
   const uint32_t col = n0 + g * 8;
   const uint32_t ncol = col >= n ? 0u : (n - col < 8u ? n - col : 8u);
   for (int it = 0; it < PER_THREAD / SL; ++it) {
-    Slabs acc;
-    uint32_t row[SL], rows_ok = 0;
+    typename SlabVec<SL>::type acc;
+    SlabRows rows;
+    rows.ok = 0;
 #pragma unroll
     for (int s = 0; s < SL; ++s) {
       const uint32_t lr = (it * SL + s) * ROWS_PER_STEP + r0;  // local row of the dump
       const uint32_t wm = lr / HALF, rr = lr % HALF;
-      row[s] = m0 + wm * (TM * 32) + pass * HALF + rr;
-      rows_ok |= (row[s] < m ? 1u : 0u) << s;
+      rows.row[s] = m0 + wm * (TM * 32) + pass * HALF + rr;
+      rows.ok |= (rows.row[s] < m ? 1u : 0u) << s;
       const vf4 lo = *reinterpret_cast<const vf4 *>(dump + lr * PITCH + g * 8), hi = *reinterpret_cast<const vf4 *>(dump + lr * PITCH + g * 8 + 4);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -458,7 +612,7 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
         acc[s * 8 + 4 + e] = hi[e];
       }
     }
-    run_epilogue(acc, prog32, ea, row[0], row[1], col, ncol, rows_ok);
+    run_epilogue<SL>(acc, prog32, ea, rows, col, ncol);
   }
 }
 
@@ -473,11 +627,15 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
   extern __shared__ double lds_raw[];
   __shared__ uint32_t prog32[DVM_PARAM_BYTES / 4];
   {
+    // only the words the program occupies are read: the argument segment is far away
     const uint32_t *src = reinterpret_cast<const uint32_t *>(p.w);
-    const uint32_t trips = (DVM_PARAM_BYTES / 4 + 255) / 256;
+    const VCubeHeader *hp = reinterpret_cast<const VCubeHeader *>(p.w);
+    uint32_t used = (hp->code_off + hp->n_code) * 2;
+    used = used < DVM_PARAM_BYTES / 4 ? used : DVM_PARAM_BYTES / 4;
+    const uint32_t trips = (used + 255) / 256;
     for (uint32_t t = 0; t < trips; ++t) {
       uint32_t i = t * 256 + threadIdx.x;
-      i = i < DVM_PARAM_BYTES / 4 ? i : DVM_PARAM_BYTES / 4 - 1;
+      i = i < used ? i : used - 1;
       prog32[i] = src[i];
     }
     __syncthreads();
@@ -538,47 +696,106 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       sb.load(b_org, h.ldb, b_voff, tid);
       sa.store(lds, tid);
       sb.store(lds + kBBase, tid);
+      if (nk > 1) {
+        sa.load(a_org + a_step, h.lda, a_voff, tid);
+        sb.load(b_org + b_step, h.ldb, b_voff, tid);
+      }
       __syncthreads();
       vu4 af[2][TM], bf[2][TN];
+      auto read_frags = [&](int fb, uint32_t buf, int kk) {
+        const uint16_t *ab = lds + buf * kABuf, *bb = lds + buf * kBBuf;
 #pragma unroll
-      for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const vu4 *>(lds + frag_off(a_row, a_x, i, 0));
+        for (int i = 0; i < TM; ++i) af[fb][i] = *reinterpret_cast<const vu4 *>(ab + frag_off(a_row, a_x, i, kk));
 #pragma unroll
-      for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const vu4 *>(lds + frag_off(b_row, b_x, j, 0));
-      for (uint32_t kt = 0; kt < nk; ++kt) {
+        for (int j = 0; j < TN; ++j) bf[fb][j] = *reinterpret_cast<const vu4 *>(bb + frag_off(b_row, b_x, j, kk));
+      };
+      auto mfmas = [&](int fb) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j) acc[i][j] = mfma<IS_BF16>(af[fb][i], bf[fb][j], acc[i][j]);
+      };
+      // One k tile (4 steps of 16). Step s runs its MFMAs on fragment buffer s&1 while the reads of
+      // step s+1 land in the other one. Tile kt+1 is written to the other local-memory buffer during
+      // step 2 (its global loads were issued a tile earlier), the workgroup meets before step 3, and
+      // step 3 overlaps the first fragment reads of tile kt+1 and the global loads of tile kt+2.
+      // The group barriers pin that interleaving: the scheduler would otherwise serialise each read
+      // against its use to save registers, and with one wave per SIMD nothing else hides the latency.
+      auto k_tile = [&](uint32_t kt, auto has_next, auto has_next2) {
+        constexpr bool NEXT = decltype(has_next)::value, NEXT2 = decltype(has_next2)::value;
+        constexpr int NF = TM + TN, NM = TM * TN;
         const uint32_t cur = kt & 1u;
-        const bool more = kt + 1 < nk;
-        const uint16_t *abuf = lds + cur * kABuf, *bbuf = lds + cur * kBBuf;
-        if (more) {
-          sa.load(a_org + (kt + 1) * a_step, h.lda, a_voff, tid);
-          sb.load(b_org + (kt + 1) * b_step, h.ldb, b_voff, tid);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(1, cur, 1);
+        mfmas(0);
+#pragma unroll
+        for (int q = 0; q < NF; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
+        __builtin_amdgcn_sched_group_barrier(0x008, NM - NF > 0 ? NM - NF : 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(0, cur, 2);
+        mfmas(1);
 #pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-          constexpr int LAST = BK / 16 - 1;
-          if (kk < LAST) {
+        for (int q = 0; q < NF; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, NM - NF > 0 ? NM - NF : 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        read_frags(1, cur, 3);
+        if constexpr (NEXT) {
+          sa.store(lds + (cur ^ 1u) * kABuf, tid);
+          sb.store(lds + kBBase + (cur ^ 1u) * kBBuf, tid);
+        }
+        mfmas(0);
 #pragma unroll
-            for (int i = 0; i < TM; ++i) af[(kk + 1) & 1][i] = *reinterpret_cast<const vu4 *>(abuf + frag_off(a_row, a_x, i, kk + 1));
+        for (int q = 0; q < NF; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        if constexpr (NEXT) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j) bf[(kk + 1) & 1][j] = *reinterpret_cast<const vu4 *>(bbuf + frag_off(b_row, b_x, j, kk + 1));
-          } else if (more) {
-            // the next tile goes to the other buffer while the last MFMAs of this one run
-            sa.store(lds + (cur ^ 1u) * kABuf, tid);
-            sb.store(lds + kBBase + (cur ^ 1u) * kBBuf, tid);
+          for (int q = 0; q < (NM - NF > 0 ? NM - NF : 1); ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, (Stage<BM, A_KC>::N + Stage<BN, B_KC>::N + (NM - NF > 0 ? NM - NF : 1) - 1) / (NM - NF > 0 ? NM - NF : 1), 0);
           }
-#pragma unroll
-          for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = mfma<IS_BF16>(af[kk & 1][i], bf[kk & 1][j], acc[i][j]);
         }
-        __syncthreads();
-        if (more) {
-          const uint16_t *an = lds + (cur ^ 1u) * kABuf, *bn = lds + (cur ^ 1u) * kBBuf;
-#pragma unroll
-          for (int i = 0; i < TM; ++i) af[0][i] = *reinterpret_cast<const vu4 *>(an + frag_off(a_row, a_x, i, 0));
-#pragma unroll
-          for (int j = 0; j < TN; ++j) bf[0][j] = *reinterpret_cast<const vu4 *>(bn + frag_off(b_row, b_x, j, 0));
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (NEXT) __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (NEXT) read_frags(0, cur ^ 1u, 0);
+        if constexpr (NEXT2) {
+          sa.load(a_org + (kt + 2) * a_step, h.lda, a_voff, tid);
+          sb.load(b_org + (kt + 2) * b_step, h.ldb, b_voff, tid);
         }
+        mfmas(1);
+        if constexpr (NEXT) {
+#pragma unroll
+          for (int q = 0; q < NF; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+        }
+        if constexpr (NEXT2) {
+#pragma unroll
+          for (int q = 0; q < (NM - NF > 0 ? NM - NF : 1); ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, (Stage<BM, A_KC>::N + Stage<BN, B_KC>::N + (NM - NF > 0 ? NM - NF : 1) - 1) / (NM - NF > 0 ? NM - NF : 1), 0);
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      };
+      read_frags(0, 0, 0);
+      uint32_t kt = 0;
+      for (; kt + 2 < nk; ++kt) k_tile(kt, std::true_type{}, std::true_type{});
+      if (kt + 1 < nk) {
+        k_tile(kt, std::true_type{}, std::false_type{});
+        ++kt;
       }
+      k_tile(kt, std::false_type{}, std::false_type{});
+      __syncthreads();
     } else {
       for (uint32_t kt = 0; kt < nk; ++kt) {
         stage_generic<BM>(lds, a_base, h.lda, m0, kt * BK, h.m, h.k, A_KC ? 1u : 0u, tid);

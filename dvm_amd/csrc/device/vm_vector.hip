@@ -52,13 +52,15 @@ __device__ __forceinline__ uint32_t fast_div(uint32_t n, const VDim &d) { return
 
 __device__ __forceinline__ float round_f16(float x) { return static_cast<float>(static_cast<_Float16>(x)); }
 
-__device__ __forceinline__ uint32_t f32_to_bf16_bits(float x) {
-  uint32_t u = __float_as_uint(x);
-  uint32_t r = u + 0x7fffu + ((u >> 16) & 1u);  // round to nearest even
-  r = (x != x) ? 0x7fc00000u : r;              // NaN stays NaN
-  return r >> 16;
+// gfx950 converts fp32 to bf16 in hardware (round to nearest even, NaN stays NaN): v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float x) { return __builtin_bit_cast(uint16_t, static_cast<__bf16>(x)); }
+__device__ __forceinline__ float round_bf16(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
+typedef float vf2_t __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  const vf2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
-__device__ __forceinline__ float round_bf16(float x) { return __uint_as_float(f32_to_bf16_bits(x) << 16); }
 
 __device__ __forceinline__ void apply_rnd(Acc &a, uint32_t rnd) {
   if (rnd == VRND_NONE) return;
@@ -246,7 +248,7 @@ __device__ __forceinline__ void mem_store_wide(const VMemDesc &m, const Offs &of
       vu4 a;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        a[i] = f32_to_bf16_bits(in.v[u][2 * i]) | (f32_to_bf16_bits(in.v[u][2 * i + 1]) << 16);
+        a[i] = pack_bf16(in.v[u][2 * i], in.v[u][2 * i + 1]);
       *reinterpret_cast<DVM_GLOBAL vu4 *>(m.addr + off.v[u] * 2) = a;
     } else if (dtype == VDT_F16) {
       *reinterpret_cast<DVM_GLOBAL vh8 *>(m.addr + off.v[u] * 2) = __builtin_convertvector(in.v[u], vh8);
@@ -534,11 +536,15 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   // into local memory once and decodes from there.
   {
     // uniform trip count and clamped indices: no per-lane branch (lanes past the end rewrite the last word)
+    // only the words the program occupies are read: the argument segment is far away
     const uint32_t *src = reinterpret_cast<const uint32_t *>(p.w);
-    const uint32_t trips = (DVM_PARAM_BYTES / 4 + blockDim.x - 1) / blockDim.x;
+    const VVecHeader *hp = reinterpret_cast<const VVecHeader *>(p.w);
+    uint32_t used = (hp->code_off + hp->n_code) * 2;
+    used = used < DVM_PARAM_BYTES / 4 ? used : DVM_PARAM_BYTES / 4;
+    const uint32_t trips = (used + blockDim.x - 1) / blockDim.x;
     for (uint32_t t = 0; t < trips; ++t) {
       uint32_t i = t * blockDim.x + threadIdx.x;
-      i = i < DVM_PARAM_BYTES / 4 ? i : DVM_PARAM_BYTES / 4 - 1;
+      i = i < used ? i : used - 1;
       prog32[i] = src[i];
     }
     __syncthreads();

@@ -1743,6 +1743,13 @@ void Compiler::CompileCube(int a) {
     h.tile = 2;
     bt = 64;
   }
+  if (const char *e = std::getenv("DVM_CUBE_TILE")) {  // tuning override: 256, 128 or 64
+    const int v = std::atoi(e);
+    if (v == 256 || v == 128 || v == 64) {
+      bt = v;
+      h.tile = v == 256 ? 0 : (v == 128 ? 1 : 2);
+    }
+  }
   h.tiles_m = static_cast<uint32_t>((M + bt - 1) / bt);
   h.tiles_n = static_cast<uint32_t>((N + bt - 1) / bt);
   if (tiles(bt) >= (1ull << 31)) Fail("too many matmul tiles");
