@@ -183,6 +183,36 @@ def bench_matmul(m=8192, n=4096, k=4096, iters=20):
             "parity_rows_checked": len(rows)}
 
 
+def bench_attention(b=8, h=32, s=2048, d=128, iters=10):
+    """configs[3]: fused attention softmax(Q K^T / sqrt(d)) V, fp16, one launch; FLOPs = 4*b*h*s*s*d."""
+    import math
+    from dvm_amd.tester import Tester
+    rng = np.random.default_rng(1004)
+    q, k, v = (rng.standard_normal((b, h, s, d), dtype=np.float32).astype(np.float16) for _ in range(3))
+    t = Tester("mix")
+    sc = t.mul(t.matmul(t.load(q), t.load(k), False, True), 1.0 / math.sqrt(d))
+    x = t.cast(sc, "float32")
+    x = t.sub(x, t.max(x, (3,), True))
+    e = t.exp(x)
+    p = t.cast(t.div(e, t.sum(e, (3,), True)), "float16")
+    out = t.store(t.matmul(p, t.load(v), False, False))
+    t.codegen()
+    cold = t.jit_us()
+    t.run()
+    got = t.output(out)
+    for bi, hi in ((0, 0), (b - 1, h - 1)):  # parity on two heads against the NumPy golden (1e-2)
+        sm = (q[bi, hi].astype(np.float64) @ k[bi, hi].astype(np.float64).T) / math.sqrt(d)
+        sm = np.exp(sm - sm.max(-1, keepdims=True))
+        want = (sm / sm.sum(-1, keepdims=True)) @ v[bi, hi].astype(np.float64)
+        if not np.allclose(got[bi, hi], want, rtol=1e-2, atol=1e-2):
+            raise RuntimeError("attention result differs from the NumPy golden")
+    mn, _, mean = t.perf(warmup=2, iters=iters)
+    flops = 4.0 * b * h * s * s * d
+    return {"shape": [b, h, s, d], "kernel_us_mean": round(mean, 2), "kernel_us_min": round(mn, 2), "TFLOPs": round(flops / mean / 1e6, 1),
+            "frac_of_2.5PFLOPs": round(flops / mean / 1e6 / 2500.0, 4), "launches": t.num_launches(), "jit_us_cold": round(cold, 2),
+            "parity_heads_checked": 2}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -217,6 +247,7 @@ def main():
         line["cpu_baseline"] = cpu_baseline_batchnorm(bn["x"], bn["g"], bn["b"], bn["alg_bytes"])
     if not args.only_headline:
         line["configs"] = {"add_fp32_32x32": bench_add(), "residual_rmsnorm_bf16_dynamic": bench_rmsnorm(),
+                           "attention_fp16_b8_h32_s2048_d128": bench_attention(),
                            "matmul_bias_silu_bf16_8192x4096x4096": bench_matmul()}
     print(json.dumps(line))
 

@@ -25,6 +25,9 @@ DVM_CUBE_DECL(dvm_vm_cube_f16_mid)
 DVM_CUBE_DECL(dvm_vm_cube_bf16_small)
 DVM_CUBE_DECL(dvm_vm_cube_f16_small)
 
+extern "C" __global__ void dvm_vm_attn_f16(const VmParam p);
+extern "C" __global__ void dvm_vm_attn_bf16(const VmParam p);
+
 typedef void (*CubeKernel)(const VmParam);
 #define DVM_CUBE_ROW(prefix) {prefix##_nn, prefix##_nt, prefix##_tn, prefix##_tt}
 // [tile][bf16][trans_a * 2 + trans_b]
@@ -85,6 +88,8 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
   for (const auto &tile : kCubeKernels)
     for (const auto &dt : tile)
       for (CubeKernel k : dt) kernels.push_back(reinterpret_cast<const void *>(k));
+  kernels.push_back(reinterpret_cast<const void *>(dvm_vm_attn_f16));
+  kernels.push_back(reinterpret_cast<const void *>(dvm_vm_attn_bf16));
   for (const void *k : kernels) {
     if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(g_dev.lds_per_cu)) ==
         hipSuccess) {
@@ -168,6 +173,16 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
     }
     const CubeKernel kern = kCubeKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0][(c->trans_a ? 2 : 0) + (c->trans_b ? 1 : 0)];
     hipLaunchKernelGGL(kern, dim3(block_dim), dim3(256), lds_bytes, s, p);
+  } else if (h->entry == VE_ATTN) {
+    const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.w);
+    // the kernel has no guards of its own beyond the query tail: the header must fit it exactly
+    if (a->d != DVM_ATTN_D || a->skv == 0 || a->skv % DVM_ATTN_BKV != 0 || a->sq == 0 || a->nb == 0 ||
+        a->q_blocks != (a->sq + DVM_ATTN_BQ - 1) / DVM_ATTN_BQ || static_cast<uint64_t>(a->nb) * a->q_blocks != block_dim || threads != 256 ||
+        lds_bytes < DVM_ATTN_LDS_BYTES || a->q_addr == 0 || a->k_addr == 0 || a->v_addr == 0 || a->o_addr == 0 ||
+        ((a->q_addr | a->k_addr | a->v_addr | a->o_addr) & 15u) != 0 || (a->dtype != VDT_F16 && a->dtype != VDT_BF16)) {
+      return static_cast<int>(hipErrorInvalidValue);
+    }
+    hipLaunchKernelGGL(a->dtype == VDT_BF16 ? dvm_vm_attn_bf16 : dvm_vm_attn_f16, dim3(block_dim), dim3(256), lds_bytes, s, p);
   } else {
     return static_cast<int>(hipErrorInvalidValue);
   }

@@ -1,0 +1,269 @@
+// gfx950 fused attention: two MFMA stages with the softmax between them, one launch.
+//
+// Role in the reference: none on any backend. The reference runs examples/03_attention.py:39-50 as
+// three sub-kernels (Q K^T on the cube unit, the softmax as a vector kernel over the full score
+// matrix, P V on the cube unit; the cut rule is src/xkernel.cc:2097-2107), so the [sq][skv] scores
+// travel through memory twice. This kernel keeps them in registers:
+//  * a workgroup (4 waves) owns 256 query rows of one (batch, head), a wave 64 of them; the keys are
+//    walked in blocks of 64 with a running row max and row sum (online softmax);
+//  * stage 1 computes the TRANSPOSED scores S^T = K Q^T with v_mfma_f32_32x32x16: in the MFMA result
+//    layout a lane then holds one query (column) and 16 keys (rows) per tile, so the row max, the row
+//    sum and the rescale factor of a query are per-lane values: no cross-lane reduction except one
+//    exchange between the two half-waves;
+//  * the probabilities go to the second MFMA straight from those registers: O^T += V^T P^T sums
+//    over keys, and the order of that sum is free, so the keys a lane happens to hold are fed as they
+//    are and the V^T fragment is read in the matching (permuted) key order;
+//  * K is staged in local memory as it lies in memory (head dimension contiguous), V transposed in
+//    registers on the way in (keys contiguous), both in the XOR-swizzled tile layout of the matmul
+//    kernel and double buffered, the loads of block j+1 in flight during block j;
+//  * Q fragments are read from memory once and stay in registers.
+// Scores stay in fp32 between the stages (the three-kernel graph rounds them to the operand type);
+// the result agrees with the NumPy golden of examples/03_attention.py:20-28 within its 1e-2.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../isa_gfx950.h"
+
+namespace {
+
+#define DVM_GLOBAL __attribute__((address_space(1)))
+
+typedef float vf16 __attribute__((ext_vector_type(16)));
+typedef float vf2 __attribute__((ext_vector_type(2)));
+typedef uint32_t vu4 __attribute__((ext_vector_type(4)));
+typedef uint32_t vu2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+constexpr int D = DVM_ATTN_D;      // head dimension
+constexpr int BKV = DVM_ATTN_BKV;  // keys per block
+constexpr int WQ = 64;             // query rows per wave
+constexpr int ROW = 64;            // elements per local-memory tile row (128 bytes)
+
+__device__ __forceinline__ uint32_t uni(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
+template <bool IS_BF16>
+__device__ __forceinline__ vf16 mfma(vu4 a, vu4 b, vf16 c) {
+  if constexpr (IS_BF16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<bf16x8 *>(&a), *reinterpret_cast<bf16x8 *>(&b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(*reinterpret_cast<half8 *>(&a), *reinterpret_cast<half8 *>(&b), c, 0, 0, 0);
+  }
+}
+
+template <bool IS_BF16>
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  const vf2 v = {lo, hi};
+  if constexpr (IS_BF16) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+  } else {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, half2v));
+  }
+}
+
+// Element offset of 16-byte chunk `chunk` (0..7) of row `row` in a tile of 64-element rows.
+__device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk) {
+  return row * ROW + ((chunk ^ ((row ^ (row >> 3)) & 7u)) << 3);
+}
+
+// Local memory per buffer: K block as two tiles [64 keys][64 d] (d halves), V^T block as one tile [128 d][64 keys].
+constexpr uint32_t kKTile = BKV * ROW;           // elements of one K half tile
+constexpr uint32_t kVOff = 2 * kKTile;           // V^T tile after the two K half tiles
+constexpr uint32_t kBuf = 2 * kKTile + D * ROW;  // elements per buffer
+
+template <bool IS_BF16>
+__device__ __forceinline__ void vm_attn(const VmParam &p) {
+  extern __shared__ double lds_raw[];
+  uint16_t *lds = reinterpret_cast<uint16_t *>(lds_raw);
+  const VAttnHeader *hp = reinterpret_cast<const VAttnHeader *>(p.w);
+  const uint32_t sq = hp->sq, skv = hp->skv, q_blocks = hp->q_blocks;
+  const float scale = hp->scale;
+  const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+  const uint32_t lj = lane & 31u, lh = lane >> 5;
+  const uint32_t b = blockIdx.x / q_blocks, qb = blockIdx.x % q_blocks;
+  const uint64_t q_base = hp->q_addr + static_cast<uint64_t>(b) * sq * D * 2;
+  const uint64_t k_base = hp->k_addr + static_cast<uint64_t>(b) * skv * D * 2;
+  const uint64_t v_base = hp->v_addr + static_cast<uint64_t>(b) * skv * D * 2;
+  const uint64_t o_base = hp->o_addr + static_cast<uint64_t>(b) * sq * D * 2;
+  const uint32_t q0 = qb * DVM_ATTN_BQ + wave * WQ;
+
+  // Q fragments (B operand of stage 1): lane (j, h) holds Q[q0 + 32*qt + j][16*kk + 8*h .. +7]; rows
+  // past the end repeat the last row (their results are never stored)
+  vu4 qf[2][D / 16];
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    uint32_t row = q0 + 32 * qt + lj;
+    row = row < sq ? row : sq - 1;
+#pragma unroll
+    for (int kk = 0; kk < D / 16; ++kk)
+      qf[qt][kk] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(q_base + (static_cast<uint64_t>(row) * D + 16 * kk + 8 * lh) * 2);
+  }
+
+  // staging: K block = 64 keys x 128 d = 1024 chunks of 16 bytes, 4 per thread, copied as they are;
+  // V block = 128 (8x8 blocks along d: 16) x (along keys: 8) blocks, one per thread for the first 128
+  vu4 ks[4], vs[8];
+  const uint32_t v_kb = tid >> 4, v_db = tid & 15u;  // 8x8 block of V this thread transposes (tid < 128)
+  auto load_kv = [&](uint32_t key0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t c = tid + 256u * i;  // chunk: key = c / 16, d chunk = c % 16
+      ks[i] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(k_base + (static_cast<uint64_t>(key0 + (c >> 4)) * D + ((c & 15u) << 3)) * 2);
+    }
+    if (tid < 128) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j)
+        vs[j] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(v_base + (static_cast<uint64_t>(key0 + v_kb * 8 + j) * D + v_db * 8) * 2);
+    }
+  };
+  auto store_kv = [&](uint32_t buf) {
+    uint16_t *base = lds + buf * kBuf;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t c = tid + 256u * i;
+      const uint32_t key = c >> 4, dc = c & 15u;
+      *reinterpret_cast<vu4 *>(base + (dc >> 3) * kKTile + tile_off(key, dc & 7u)) = ks[i];
+    }
+    if (tid < 128) {
+      // vs[j] holds key v_kb*8 + j, d = v_db*8 .. +7; row d of V^T wants keys v_kb*8 .. +7
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        vu4 o;
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj) {
+          const uint32_t lo = vs[2 * jj][i >> 1], hi = vs[2 * jj + 1][i >> 1];
+          o[jj] = __builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
+        }
+        *reinterpret_cast<vu4 *>(base + kVOff + tile_off(v_db * 8 + i, v_kb)) = o;
+      }
+    }
+  };
+
+  vf16 o_acc[D / 32][2];
+#pragma unroll
+  for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) o_acc[dt][qt] = 0.0f;
+  float m_run[2] = {-1.0e30f, -1.0e30f}, l_run[2] = {0.0f, 0.0f};
+  const float c_log2 = scale * 1.44269504088896340736f;  // scores are handled in the log2 domain
+
+  // Fragment reads. For row = 32*t + j of a tile the swizzle is swz0 ^ 4*(t & 1) with swz0 = (j ^ j>>3) & 7,
+  // so every read address is a per-lane base plus (x ^ constant) plus a constant: no register per address.
+  const uint32_t swz0 = (lj ^ (lj >> 3)) & 7u;
+  const uint32_t lane_row = lj * ROW;
+  const uint32_t k_x = (lh ^ swz0) << 3;  // K fragment: chunk 2*(kk&3) + h
+  const uint32_t v_x = swz0 << 3;         // V^T fragment: whole chunks, the half-wave picks 4 elements inside
+  const uint32_t n_blocks = skv / BKV;
+  load_kv(0);
+  store_kv(0);
+  if (n_blocks > 1) load_kv(BKV);
+  __syncthreads();
+  for (uint32_t kb = 0; kb < n_blocks; ++kb) {
+    const uint32_t cur = kb & 1u;
+    const uint16_t *kbuf = lds + cur * kBuf, *vbuf = lds + cur * kBuf + kVOff;
+    // stage 1: S^T[key][query] for 2 key tiles x 2 query tiles
+    vf16 s[2][2];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) s[kt][qt] = 0.0f;
+#pragma unroll
+    for (int kk = 0; kk < D / 16; ++kk) {
+      vu4 kf[2];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+        kf[kt] = *reinterpret_cast<const vu4 *>(kbuf + (kk >> 2) * kKTile + kt * 32 * ROW + lane_row + (k_x ^ static_cast<uint32_t>((((kk & 3) * 2) ^ (4 * kt)) << 3)));
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) s[kt][qt] = mfma<IS_BF16>(kf[kt], qf[qt][kk], s[kt][qt]);
+      if (kk & 1) __builtin_amdgcn_sched_barrier(0);  // keep the fragment reads near their use: registers are scarce
+    }
+    // the next block goes to the other buffer while the softmax runs
+    if (kb + 1 < n_blocks) store_kv(cur ^ 1u);
+    __builtin_amdgcn_sched_barrier(0);
+    // softmax of this block, per query (= per lane, both half-waves share a query)
+    vu4 pf[2][2][2];  // [key tile][16-key step][query tile]: B operand of stage 2
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) {
+      float mx = s[0][qt][0];
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kt][qt][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run[qt], mx * c_log2);
+      const float alpha = exp2f(m_run[qt] - m_new);
+      m_run[qt] = m_new;
+      float sum = 0.0f;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float pv = exp2f(s[kt][qt][r] * c_log2 - m_new);
+          s[kt][qt][r] = pv;
+          sum += pv;
+        }
+#pragma unroll
+        for (int st = 0; st < 2; ++st)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pf[kt][st][qt][e] = pack2<IS_BF16>(s[kt][qt][8 * st + 2 * e], s[kt][qt][8 * st + 2 * e + 1]);
+      }
+      l_run[qt] = l_run[qt] * alpha + sum;
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt) o_acc[dt][qt] = o_acc[dt][qt] * alpha;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    // stage 2: O^T[d][query] += V^T[d][key] P^T[key][query]. Step (kt, st) contracts the 16 keys the
+    // lane's registers 8*st .. 8*st+7 of tile kt hold: keys 32*kt + 16*st + {0..3, 8..11} + 4*h.
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+#pragma unroll
+      for (int st = 0; st < 2; ++st) {
+        vu4 vf[D / 32];
+#pragma unroll
+        for (int dt = 0; dt < D / 32; ++dt) {
+          const int c0 = kt * 4 + st * 2;  // chunk of keys 32*kt + 16*st .. +7, the next chunk holds +8 .. +15
+          const uint16_t *rowp = vbuf + dt * 32 * ROW + lane_row + 4 * lh;
+          const vu2 a = *reinterpret_cast<const vu2 *>(rowp + (v_x ^ static_cast<uint32_t>((c0 ^ (4 * (dt & 1))) << 3)));
+          const vu2 bq = *reinterpret_cast<const vu2 *>(rowp + (v_x ^ static_cast<uint32_t>(((c0 + 1) ^ (4 * (dt & 1))) << 3)));
+          vf[dt] = vu4{a[0], a[1], bq[0], bq[1]};
+        }
+#pragma unroll
+        for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+          for (int qt = 0; qt < 2; ++qt) o_acc[dt][qt] = mfma<IS_BF16>(vf[dt], pf[kt][st][qt], o_acc[dt][qt]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+    __syncthreads();
+    if (kb + 2 < n_blocks) load_kv((kb + 2) * BKV);
+  }
+
+  // O[query][d] = O^T / l, rounded once to the operand type. Lane (j, h) holds, per d tile and register
+  // group g, d = 32*dt + 8*g + 4*h + 0..3: four consecutive values = one 8-byte store.
+#pragma unroll
+  for (int qt = 0; qt < 2; ++qt) {
+    const float l = l_run[qt] + __shfl_xor(l_run[qt], 32);
+    const float inv = 1.0f / l;
+    const uint32_t row = q0 + 32 * qt + lj;
+    if (row < sq) {
+#pragma unroll
+      for (int dt = 0; dt < D / 32; ++dt) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          vu2 w;
+          w[0] = pack2<IS_BF16>(o_acc[dt][qt][4 * g] * inv, o_acc[dt][qt][4 * g + 1] * inv);
+          w[1] = pack2<IS_BF16>(o_acc[dt][qt][4 * g + 2] * inv, o_acc[dt][qt][4 * g + 3] * inv);
+          *reinterpret_cast<DVM_GLOBAL vu2 *>(o_base + (static_cast<uint64_t>(row) * D + dt * 32 + 8 * g + 4 * lh) * 2) = w;
+        }
+      }
+    }
+  }
+}
+
+}  // namespace
+
+extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_f16(const VmParam p) { vm_attn<false>(p); }
+extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_bf16(const VmParam p) { vm_attn<true>(p); }

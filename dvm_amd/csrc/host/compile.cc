@@ -320,6 +320,9 @@ class Compiler {
     ws_slot_.assign(n_, -1);
     store_of_.assign(n_, -1);
     MarkLive();
+    attn_groups_.clear();
+    attn_of_.assign(n_, -1);
+    if (mode_ == 0) DetectAttention();
     Partition();
     k_->programs_.clear();
     k_->ws_sizes_.clear();
@@ -348,8 +351,20 @@ class Compiler {
     int rank = 0;
     int64_t dom[kMaxRank];
     const NDObject *cube_op = nullptr;
+    int attn = -1;  // index into attn_groups_ when the sub-kernel is one fused attention
   };
   std::vector<AreaInfo> areas_;
+
+  // softmax(Q K^T * scale) V written as matmul / mul / cast / max / sub / exp / sum / div / cast /
+  // matmul (examples/03_attention.py:30-50): recognised as a whole and run by the fused kernel.
+  struct AttnGroup {
+    NDObject *m1, *m2, *q, *k, *v;
+    float scale;
+    int area;
+  };
+  std::vector<AttnGroup> attn_groups_;
+  std::vector<int> attn_of_;
+  void DetectAttention();
 
   // ---------- liveness ----------
   void MarkLive() {
@@ -419,6 +434,7 @@ class Compiler {
     if (a >= static_cast<int>(areas_.size())) return true;  // a fresh sub-kernel
     const AreaInfo &ai = areas_[a];
     if (o->kind == kObjMatMul) return false;
+    if (ai.attn >= 0) return o->kind == kObjStore && o->in[0] == attn_groups_[ai.attn].m2;
     if (ai.cube) {
       if (!IsPointwiseKind(o->kind)) return false;
       if (mode_ >= 2 && !(o->kind == kObjStore && o->in[0] == ai.cube_op)) return false;  // plain matmul, epilogue on its own
@@ -481,6 +497,16 @@ class Compiler {
       if (IsView(o)) continue;  // read through by its consumers
       const int c = find(i);
       if (comp_base[c] < 0) comp_base[c] = static_cast<int>(areas_.size());
+      if (attn_of_[i] >= 0) {
+        AttnGroup &g = attn_groups_[attn_of_[i]];
+        if (g.area < 0) {
+          g.area = static_cast<int>(areas_.size());
+          areas_.push_back(AreaInfo());
+          areas_.back().attn = attn_of_[i];
+        }
+        area_[i] = g.area;
+        continue;
+      }
       int a = comp_base[c];
       for (int j = 0; j < o->nin; ++j) {
         const NDObject *v = o->in[j];
@@ -617,6 +643,7 @@ class Compiler {
 
   void CompileArea(int a);
   void CompileCube(int a);
+  void CompileAttn(int g);
   void BuildNodes(int a);
   void UnifyAxes();
   void OrderAndMerge();
@@ -1588,6 +1615,10 @@ void Compiler::CompileArea(int a) {
   k_->programs_.emplace_back();
   prog_ = &k_->programs_.back();
   cube_mode_ = false;
+  if (areas_[a].attn >= 0) {
+    CompileAttn(areas_[a].attn);
+    return;
+  }
   if (areas_[a].cube) {
     CompileCube(a);
     return;
@@ -1822,6 +1853,111 @@ void Compiler::CompileCube(int a) {
   prog_->grid = static_cast<uint32_t>(tiles(bt));
 }
 
+
+// ---------- fused attention ----------
+
+void Compiler::DetectAttention() {
+  std::vector<int> uses(n_, 0);
+  for (int i = 0; i < n_; ++i) {
+    if (!live_[i]) continue;
+    const NDObject *o = k_->ops_[i];
+    for (int j = 0; j < o->nin; ++j)
+      if (o->in[j] != nullptr) ++uses[o->in[j]->id];
+  }
+  auto last_axis_keep = [](const NDObject *r) {
+    if (!r->keepdims || r->aux_ref == nullptr || r->aux_ref->size != 1) return false;
+    const int64_t ax = r->aux_ref->data[0];
+    return ax == -1 || ax == r->in[0]->rank() - 1;
+  };
+  for (int i = 0; i < n_; ++i) {
+    if (!live_[i]) continue;
+    NDObject *m2 = k_->ops_[i];
+    if (m2->kind != kObjMatMul || m2->trans_a || m2->trans_b || m2->in[2] != nullptr) continue;
+    if (m2->type_id_ != kFloat16 && m2->type_id_ != kBFloat16) continue;
+    NDObject *p = m2->in[0], *v = m2->in[1];
+    if (p->kind != kObjCast || p->in[0]->type_id_ != kFloat32 || uses[p->id] != 1) continue;
+    NDObject *dv = p->in[0];
+    if (dv->kind != kObjBinary || dv->op != kDiv || uses[dv->id] != 1) continue;
+    NDObject *e = dv->in[0], *sm = dv->in[1];
+    if (sm->kind != kObjReduce || sm->op != kSum || sm->in[0] != e || uses[sm->id] != 1 || !last_axis_keep(sm)) continue;
+    if (e->kind != kObjUnary || e->op != kExp || uses[e->id] != 2) continue;
+    NDObject *sb = e->in[0];
+    if (sb->kind != kObjBinary || sb->op != kSub || uses[sb->id] != 1) continue;
+    NDObject *x = sb->in[0], *mx = sb->in[1];
+    if (mx->kind != kObjReduce || mx->op != kMax || mx->in[0] != x || uses[mx->id] != 1 || !last_axis_keep(mx)) continue;
+    if (x->kind != kObjCast || x->type_id_ != kFloat32 || uses[x->id] != 2) continue;
+    NDObject *sc = x->in[0];
+    NDObject *m1 = sc;
+    float scale = 1.0f;
+    NDObject *mul = nullptr;
+    if (sc->kind == kObjBinaryS && sc->op == kMul && uses[sc->id] == 1) {
+      mul = sc;
+      m1 = sc->in[0];
+      const uint32_t bits = ScalarToContainer(sc->scalar.Get(), sc->in[0]->type_id_);
+      std::memcpy(&scale, &bits, 4);
+    }
+    if (m1->kind != kObjMatMul || m1->trans_a || !m1->trans_b || m1->in[2] != nullptr || uses[m1->id] != 1) continue;
+    if (m1->type_id_ != m2->type_id_) continue;
+    NDObject *q = m1->in[0], *kk = m1->in[1];
+    if (q->kind != kObjLoad || kk->kind != kObjLoad || v->kind != kObjLoad) continue;
+    const int r = q->rank();
+    if (kk->rank() != r || v->rank() != r || r < 2) continue;
+    bool ok = q->dim(r - 1) == DVM_ATTN_D && kk->dim(r - 1) == DVM_ATTN_D && v->dim(r - 1) == DVM_ATTN_D && kk->dim(r - 2) == v->dim(r - 2) &&
+              kk->dim(r - 2) % DVM_ATTN_BKV == 0 && kk->dim(r - 2) > 0 && q->dim(r - 2) > 0;
+    for (int d = 0; d < r - 2 && ok; ++d) ok = q->dim(d) == kk->dim(d) && q->dim(d) == v->dim(d) && q->dim(d) > 0;
+    if (!ok || q->numel() >= (1ll << 31) || kk->numel() >= (1ll << 31)) continue;
+    AttnGroup g = {m1, m2, q, kk, v, scale, -1};
+    const int gi = static_cast<int>(attn_groups_.size());
+    attn_groups_.push_back(g);
+    NDObject *members[] = {m1, mul, x, mx, sb, e, sm, dv, p, m2};
+    for (NDObject *mbr : members)
+      if (mbr != nullptr) attn_of_[mbr->id] = gi;
+  }
+}
+
+void Compiler::CompileAttn(int gi) {
+  const AttnGroup &g = attn_groups_[gi];
+  const int r = g.q->rank();
+  VAttnHeader h;
+  std::memset(&h, 0, sizeof(h));
+  h.entry = VE_ATTN;
+  h.dtype = MemDType(g.m2->type_id_);
+  int64_t nb = 1;
+  for (int d = 0; d < r - 2; ++d) nb *= g.q->dim(d);
+  h.nb = static_cast<uint32_t>(nb);
+  h.sq = static_cast<uint32_t>(g.q->dim(r - 2));
+  h.skv = static_cast<uint32_t>(g.k->dim(r - 2));
+  h.d = DVM_ATTN_D;
+  h.scale = g.scale;
+  h.q_blocks = (h.sq + DVM_ATTN_BQ - 1) / DVM_ATTN_BQ;
+  if (static_cast<uint64_t>(h.nb) * h.q_blocks >= (1ull << 31)) Fail("too many attention blocks");
+  std::memset(&prog_->blob, 0, sizeof(VmParam));
+  std::memcpy(prog_->blob.w, &h, sizeof(h));
+  auto patch = [&](size_t byte_off, int op_id, int ws_slot) {
+    Program::Patch p;
+    p.word = static_cast<uint32_t>(byte_off / 8);
+    p.op_id = op_id;
+    p.ws_slot = ws_slot;
+    p.role = Program::kPatchAligned16;
+    prog_->patches.push_back(p);
+  };
+  patch(offsetof(VAttnHeader, q_addr), g.q->id, -1);
+  patch(offsetof(VAttnHeader, k_addr), g.k->id, -1);
+  patch(offsetof(VAttnHeader, v_addr), g.v->id, -1);
+  // the result goes to the user's store when there is one in this sub-kernel, else to workspace
+  const int m2 = g.m2->id;
+  if (store_of_[m2] >= 0 && area_[store_of_[m2]] == area_[m2]) {
+    patch(offsetof(VAttnHeader, o_addr), store_of_[m2], -1);
+  } else if (ws_slot_[m2] >= 0) {
+    patch(offsetof(VAttnHeader, o_addr), -1, ws_slot_[m2]);
+  } else {
+    Fail("attention result has no destination");
+  }
+  prog_->threads = 256;
+  prog_->lds_bytes = DVM_ATTN_LDS_BYTES;
+  prog_->grid = h.nb * h.q_blocks;
+}
+
 size_t VKernel::CodeGen(bool /*pre*/) {
   if (!normalized_) Normalize();
   Compiler c(this);
@@ -1858,6 +1994,8 @@ void VKernel::BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *all
           reinterpret_cast<VMemDesc *>(p.blob.w + pt.word)->flags &= ~static_cast<uint32_t>(VMF_ALIGNED);
         } else if (pt.role == Program::kPatchCubeOperand) {
           reinterpret_cast<VCubeHeader *>(p.blob.w)->fast = 0;
+        } else if (pt.role == Program::kPatchAligned16) {
+          Throw("fused attention needs 16-byte aligned tensors");
         }
       }
     }

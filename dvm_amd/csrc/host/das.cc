@@ -188,6 +188,11 @@ std::string &VKernel::DisAssemble() {
       }
       os << "  mmad acc, A, B\n";
       print_code(p.blob.w + c->code_off, c->n_code, [&](uint32_t m) { return cm[m].dtype; });
+    } else if (h->entry == VE_ATTN) {
+      const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.blob.w);
+      os << "entry attention " << kMemTypes[a->dtype] << " batch=" << a->nb << " sq=" << a->sq << " skv=" << a->skv << " d=" << a->d
+         << " scale=" << a->scale << " blocks=" << p.grid << " lds=" << p.lds_bytes << "\n";
+      os << "  mmad s, K, Q^T\n  online_softmax p, s\n  mmad o, V^T, p\n  store o\n";
     } else {
       os << "entry type " << h->entry << " blocks=" << p.grid << " threads=" << p.threads << "\n";
     }

@@ -111,9 +111,10 @@ struct Program {
     int op_id;       // load/store node whose address goes there, or -1
     int ws_slot;     // or the workspace slot
     uint8_t role;    // kPatchVecMem: a VMemDesc (alignment flag follows the address); kPatchCubeOperand:
-                     // a matmul operand (the fast path needs 16-byte alignment); kPatchPlain: nothing else
+                     // a matmul operand (the fast path needs 16-byte alignment); kPatchPlain: nothing else;
+                     // kPatchAligned16: an operand of the fused attention kernel, which only has 128-bit accesses
   };
-  enum : uint8_t { kPatchVecMem = 0, kPatchCubeOperand = 1, kPatchPlain = 2 };
+  enum : uint8_t { kPatchVecMem = 0, kPatchCubeOperand = 1, kPatchPlain = 2, kPatchAligned16 = 3 };
   std::vector<Patch> patches;
   // pre-launch fills (zero-size reduce identities, clean kernels)
   struct Fill {

@@ -202,6 +202,27 @@ typedef struct {
        ? (2u * (2u * (bt)) * 64u * 2u) \
        : (((bt) >= 128u ? (bt) / 2u : (bt)) * ((bt) + 4u) * 4u))
 
+// ---- fused attention programs (VE_ATTN) -------------------------------------------
+// O[b] = softmax(Q[b] K[b]^T * scale) V[b] for nb independent (batch, head) pairs, all operands row
+// major with the head dimension contiguous: Q [nb][sq][d], K [nb][skv][d], V [nb][skv][d], O [nb][sq][d].
+// One workgroup owns DVM_ATTN_BQ query rows and walks the keys in blocks of DVM_ATTN_BKV with an
+// online softmax (running row max and sum), so the [sq][skv] score matrix never exists in memory.
+#define DVM_ATTN_BQ 256
+#define DVM_ATTN_BKV 64
+#define DVM_ATTN_D 128
+#define DVM_ATTN_LDS_BYTES (2u * 2u * DVM_ATTN_BKV * DVM_ATTN_D * 2u)
+
+typedef struct {
+  uint32_t entry;   // VE_ATTN
+  uint32_t dtype;   // VDT_F16 or VDT_BF16
+  uint32_t nb;      // batch * heads
+  uint32_t sq, skv; // query rows, keys (skv a multiple of DVM_ATTN_BKV)
+  uint32_t d;       // head dimension (DVM_ATTN_D)
+  float scale;      // applied to Q K^T before the softmax
+  uint32_t q_blocks;  // ceil(sq / DVM_ATTN_BQ)
+  uint64_t q_addr, k_addr, v_addr, o_addr;
+} VAttnHeader;
+
 typedef struct {
   uint64_t w[DVM_PARAM_WORDS];
 } VmParam;

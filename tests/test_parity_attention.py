@@ -1,0 +1,87 @@
+"""GPU parity: attention. The graph of examples/03_attention.py runs as three sub-kernels when the
+fused kernel does not apply, as one fused launch when it does; both against the example's NumPy
+golden (1e-2), the unfused one also against the CPU oracle."""
+import math
+
+import numpy as np
+import pytest
+
+from dvm_amd.tester import Tester
+from tests.util import run_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def np_attention(q, k, v):  # examples/03_attention.py:20-28, batched
+    scale = 1.0 / math.sqrt(q.shape[-1])
+    s = np.matmul(q.astype(np.float32), np.swapaxes(k.astype(np.float32), -1, -2)) * scale
+    s = s - s.max(-1, keepdims=True)
+    p = np.exp(s)
+    p = p / p.sum(-1, keepdims=True)
+    return np.matmul(p, v.astype(np.float32))
+
+
+def attention_graph(k, q, kk, v, scale, rank, dt="float16"):  # examples/03_attention.py:30-50
+    s = k.mul(k.matmul(q, kk, False, True), scale)
+    x = k.cast(s, "float32")
+    x = k.sub(x, k.max(x, (rank - 1,), True))
+    e = k.exp(x)
+    p = k.cast(k.div(e, k.sum(e, (rank - 1,), True)), dt)
+    return k.matmul(p, v, False, False)
+
+
+def _bf16(x):
+    return Tester.convert_from_bf16(Tester.convert_to_bf16(x.astype(np.float32)))
+
+
+def test_attention_example_small():  # examples/03_attention.py:52-63: too small for the fused kernel
+    rng = np.random.default_rng(0)
+    q, k, v = (rng.normal(0, 0.02, s).astype(np.float16) for s in ((4, 8), (6, 8), (6, 12)))
+    run_parity(lambda kk, a, b, c: attention_graph(kk, a, b, c, 1.0 / math.sqrt(8), 2), [q, k, v], ker="mix",
+               golden=np_attention(q, k, v).astype(np.float16), eps=1e-2)
+
+
+def _fused(q, k, v, dt="float16"):
+    t = Tester("mix")
+    dts = dt if dt == "bfloat16" else None
+    out = t.store(attention_graph(t, t.load(q, dts), t.load(k, dts), t.load(v, dts), 1.0 / math.sqrt(q.shape[-1]), q.ndim, dt))
+    t.run()
+    assert "entry attention" in t.das() and t.num_launches() == 1, t.das()
+    o = t.output(out)
+    return Tester.convert_from_bf16(o) if dt == "bfloat16" else o
+
+
+@pytest.mark.parametrize("shape", [((2, 3), 256, 192), ((1,), 64, 64), ((3,), 100, 128), ((2, 2), 300, 2048), ((), 513, 640)])
+@pytest.mark.parametrize("dt", ["float16", "bfloat16"])
+def test_attention_fused(shape, dt):
+    batch, sq, skv = shape
+    rng = np.random.default_rng(sq)
+    conv = (lambda x: x.astype(np.float16)) if dt == "float16" else _bf16
+    q, k, v = (conv(rng.standard_normal(batch + (n, 128))) for n in (sq, skv, skv))
+    got = _fused(q, k, v, dt)
+    want = np_attention(q, k, v)
+    assert got.shape == want.shape
+    assert np.allclose(got, want, rtol=1e-2, atol=1e-2), np.abs(got - want).max()
+
+
+def test_attention_fused_constant_values_and_key_order():
+    # softmax weights sum to one: with every row of V equal to c the output rows are c, at any size;
+    # and the result does not depend on the order of the keys
+    rng = np.random.default_rng(5)
+    q, k = (rng.standard_normal((4, 512, 128)).astype(np.float16) for _ in range(2))
+    c = rng.standard_normal(128).astype(np.float16)
+    got = _fused(q, k, np.broadcast_to(c, (4, 512, 128)).copy())
+    assert np.allclose(got, c, rtol=2e-3, atol=2e-3)
+    v = rng.standard_normal((4, 512, 128)).astype(np.float16)
+    perm = rng.permutation(512)
+    a, b = _fused(q, k, v), _fused(q, k[:, perm], v[:, perm])
+    assert np.allclose(a, b, rtol=5e-3, atol=5e-3)
+
+
+def test_attention_full_size_heads():  # BASELINE config 4 shape, three sampled heads against the golden
+    rng = np.random.default_rng(1004)
+    q, k, v = (rng.standard_normal((8, 32, 2048, 128), dtype=np.float32).astype(np.float16) for _ in range(3))
+    got = _fused(q, k, v)
+    for b, h in ((0, 0), (3, 17), (7, 31)):
+        want = np_attention(q[b, h], k[b, h], v[b, h])
+        assert np.allclose(got[b, h], want, rtol=1e-2, atol=1e-2), (b, h, np.abs(got[b, h] - want).max())
