@@ -19,6 +19,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+# HBM bytes one launch of the headline kernel moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of
+# `bench.py --traffic-probe`, each scaled by the same counter's reading for a plain copy of known size
+# (207.2 MB fetched + 118.4 MB written). A counter cannot be read from inside this script: the figure is
+# re-measured and updated whenever the kernel's schedule changes.
+HEADLINE_TRAFFIC_BYTES = 325.7e6
 METRIC = "fused-op HBM GB/s (% roofline) + matmul TFLOPS (% MFMA peak); JIT us/shape"
 
 
@@ -77,10 +82,12 @@ def bench_batchnorm(steps, warmup):
 def cpu_baseline_batchnorm(x, g, b, alg_bytes):
     from oracle import oracle as ora
     ora.batchnorm_nchw(x[:2], g, b, 1e-5)  # warm-up on a slice
-    reps = 3
+    # about 10 s of CPU work on the full tensor
+    reps = 0
     t0 = time.perf_counter()
-    for _ in range(reps):
+    while reps < 3 or time.perf_counter() - t0 < 10.0:
         ora.batchnorm_nchw(x, g, b, 1e-5)
+        reps += 1
     dt = (time.perf_counter() - t0) / reps
     return {"value": round(alg_bytes / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": "full [32,256,56,56] tensor, scalar C oracle (oracle/dvm_oracle.c ora_batchnorm_nchw), mean of %d runs, %.2f s each" % (reps, dt)}
@@ -213,6 +220,22 @@ def bench_attention(b=8, h=32, s=2048, d=128, iters=10):
             "parity_heads_checked": 2}
 
 
+def traffic_probe():
+    """For the counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): five launches of the headline kernel
+    and five launches of a plain copy of the same tensor through the pointwise VM kernel, whose traffic is
+    known (102 760 448 B read, as many written); the copy calibrates the counters' unit."""
+    from dvm_amd.tester import Tester
+    bn = bench_batchnorm(5, 2)
+    t = Tester("split")
+    out = t.store(t.copy(t.load(bn["x"])))
+    t.codegen()
+    for _ in range(5):
+        t.bare_run()
+    t.run()
+    assert np.array_equal(t.output(out), bn["x"])
+    print(json.dumps({"probe": "traffic", "copy_bytes_each_way": int(bn["x"].nbytes)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -220,6 +243,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true", help="omit the other BASELINE configs")
+    ap.add_argument("--traffic-probe", action="store_true", help="launch the headline kernel and a plain copy only (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the DVM hot path is a single-device operator JIT (run with --gpus 1)", file=sys.stderr)
@@ -228,6 +252,9 @@ def main():
     if not dvm.Device.available():
         print("bench.py needs an MI355X and the built HIP device layer (dvm_amd/lib/libdvm_hip.so)", file=sys.stderr)
         sys.exit(1)
+    if args.traffic_probe:
+        traffic_probe()
+        return
     bn = bench_batchnorm(args.steps, args.warmup)
     value = bn["alg_bytes"] / (bn["ms_per_step"] * 1e-3) / 1e9
     achieved = bn["alg_bytes"] / (bn["kernel_us_mean"] * 1e-6) / 1e9
@@ -240,7 +267,7 @@ def main():
                    "jit_us_cold": round(bn["jit_us_cold"], 2), "jit_us_warm": round(bn["jit_us_warm"], 2),
                    "parity_max_rel_err_vs_numpy_f64": bn["max_rel_err"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": HEADLINE_TRAFFIC_BYTES,
                      "kernel": "dvm_vm_vec_rx", "kernel_us_mean": round(bn["kernel_us_mean"], 2), "kernel_us_min": round(bn["kernel_us_min"], 2)},
     }
     if not args.skip_cpu:
