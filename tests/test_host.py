@@ -214,3 +214,49 @@ def test_product_never_imports_the_oracle():
             if f.endswith((".py", ".cc", ".h", ".hip")):
                 text = open(os.path.join(dirpath, f), errors="ignore").read()
                 assert "oracle" not in text.lower(), os.path.join(dirpath, f)
+
+
+def test_matmul_epilogue_is_one_cube_program():
+    # examples/04_matmul_post_fusion.py: bias add, SiLU and the cast ride in the matmul's sub-kernel
+    t = Tester("mix", run_mode="das")
+    a, b = t.load(np.zeros([512, 256], np.float32), "bfloat16"), t.load(np.zeros([256, 384], np.float32), "bfloat16")
+    h = t.add(t.cast(t.matmul(a, b, False, False), "float32"), t.load(np.zeros([384], np.float32)))
+    t.store(t.cast(t.div(h, t.add(t.exp(t.mul(h, -1.0)), 1.0)), "bfloat16"))
+    t.codegen()
+    das = t.das()
+    assert das.count("== sub-kernel") == 1 and "entry cube bf16 m=512 n=384 k=256" in das, das
+    assert "mmad acc, A, B" in das and "Exp.fp32 acc" in das and "store.bf16" in das and "strides n=1 m=0" in das, das
+    # the fp32 accumulators are rounded to the operand type before the epilogue sees them (src/vm_aic.cce:34-470)
+    assert das.index("cast.round.bf16") < das.index("Add.fp32"), das
+
+
+def test_matmul_tile_follows_problem_size():
+    for (m, n), tile in (((8192, 4096), 256), ((2048, 2048), 128), ((256, 256), 64)):
+        t = Tester("mix", run_mode="das")
+        t.store(t.matmul(t.load(np.zeros([m, 64], np.float16)), t.load(np.zeros([n, 64], np.float16)), False, True))
+        t.codegen()
+        assert "tile=%d" % tile in t.das() and "trans_b=1" in t.das(), t.das()
+    # an odd leading dimension cannot use 128-bit operand loads
+    t = Tester("mix", run_mode="das")
+    t.store(t.matmul(t.load(np.zeros([211, 211], np.float16)), t.load(np.zeros([211, 230], np.float16)), False, False))
+    t.codegen()
+    assert "guarded" in t.das(), t.das()
+
+
+def _attention(t, sq, skv, d):
+    q, k, v = (t.load(np.zeros([2, n, d], np.float16)) for n in (sq, skv, skv))
+    x = t.cast(t.mul(t.matmul(q, k, False, True), 0.125), "float32")
+    x = t.sub(x, t.max(x, (2,), True))
+    e = t.exp(x)
+    t.store(t.matmul(t.cast(t.div(e, t.sum(e, (2,), True)), "float16"), v, False, False))
+    t.codegen()
+    return t.das()
+
+
+def test_attention_graph_is_recognised():
+    das = _attention(Tester("mix", run_mode="das"), 300, 192, 128)
+    assert das.count("== sub-kernel") == 1 and "entry attention fp16 batch=2 sq=300 skv=192 d=128 scale=0.125" in das, das
+    # other head sizes or ragged key counts run as matmul, softmax, matmul
+    for sq, skv, d in ((300, 192, 64), (300, 100, 128)):
+        das = _attention(Tester("mix", run_mode="das"), sq, skv, d)
+        assert das.count("== sub-kernel") == 3 and das.count("entry cube") == 2 and "entry attention" not in das, das
