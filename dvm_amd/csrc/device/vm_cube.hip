@@ -73,67 +73,89 @@ __device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk) {
 }
 
 // ---- staging one operand tile: ROWS rows (m or n) x BK (k) ---------------------------------------------
-// KC source (k contiguous in memory: A when !trans_a, B when trans_b): 16-byte chunks copied as they are.
-// KS source (k strided, the row index contiguous): 8x8 element blocks, transposed in registers.
+// KC source (k contiguous in memory: A when !trans_a, B when trans_b): the tile is a straight copy, so it
+// goes from memory to local memory directly (global_load_lds_dwordx4: a wave's 64 x 16 bytes land in 1 KB
+// of consecutive local memory, the swizzle is applied by choosing which chunk each lane fetches); no
+// registers, no ds_write, and the data may be in flight for a whole k tile.
+// KS source (k strided, the row index contiguous): 8x8 element blocks through registers, transposed on
+// the way (v_perm_b32), then written with ds_write_b128.
+struct LaneOffsets {
+  uint32_t v[2];
+};
+
 template <int ROWS, bool KC>
-struct Stage {
-  static constexpr int CHUNKS = ROWS * BK / 8 / 256;  // 16-byte chunks per thread when all 256 threads copy
-  // a KS source moves whole 8x8 blocks (8 chunks): ROWS blocks per tile, one per thread for the first ROWS threads
-  static constexpr int N = KC ? CHUNKS : 8;
+struct Stage;
+
+template <int ROWS>
+struct Stage<ROWS, true> {
+  static constexpr int N = ROWS * BK / 8 / 256;  // 16-byte chunks per thread
+  static constexpr int N_LOADS = N, N_WRITES = 0;
+
+  // Chunk position p = 256*i + tid of the tile holds row p/8, logical chunk (p%8) ^ swizzle(row): with
+  // row = 32*i + tid/8 the swizzle only depends on the parity of i, hence two byte offsets per lane.
+  static __device__ __forceinline__ LaneOffsets lane_offset(uint32_t ld, uint32_t tid) {
+    LaneOffsets o;
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+      const uint32_t row = 32u * par + (tid >> 3);
+      const uint32_t logical = (tid & 7u) ^ ((row ^ (row >> 3)) & 7u);
+      o.v[par] = ((tid >> 3) * ld + (logical << 3)) * 2u;
+    }
+    return o;
+  }
+
+  // origin: address of element (row0, k0) of the operand
+  __device__ __forceinline__ void fetch(uint64_t origin, uint32_t ld, const LaneOffsets &lane, uint32_t tid, uint16_t *tile) {
+    const DVM_GLOBAL char *base = reinterpret_cast<const DVM_GLOBAL char *>(origin);
+    const uint32_t wave_first = uni(tid >> 6) * 64u;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const DVM_GLOBAL char *src = base + static_cast<uint64_t>(i) * 32u * ld * 2u + lane.v[i & 1];
+      uint16_t *dst = tile + (static_cast<uint32_t>(i) * 256u + wave_first) * 8u;
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(src), (__attribute__((address_space(3))) void *)(dst), 16, 0, 0);
+    }
+  }
+  __device__ __forceinline__ void commit(uint16_t *, uint32_t) const {}
+};
+
+template <int ROWS>
+struct Stage<ROWS, false> {
+  static_assert(ROWS <= 256, "one 8x8 block per thread");
+  static constexpr int N = 8;
+  static constexpr int N_LOADS = 8, N_WRITES = 8;
   vu4 r[N];
 
-  // Byte offset of this lane's first chunk from the tile's origin; the rest of every address is
-  // wave-uniform, so one register per operand addresses all its loads.
-  static __device__ __forceinline__ uint32_t lane_offset(uint32_t ld, uint32_t tid) {
-    if constexpr (KC) {
-      return ((tid >> 3) * ld + ((tid & 7u) << 3)) * 2u;
-    } else {
-      const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
-      return (kb * 8u * ld + rb * 8u) * 2u;
-    }
+  static __device__ __forceinline__ LaneOffsets lane_offset(uint32_t ld, uint32_t tid) {
+    const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
+    LaneOffsets o;
+    o.v[0] = o.v[1] = (kb * 8u * ld + rb * 8u) * 2u;
+    return o;
   }
 
-  // origin: address of element (row0, k0) of the operand; voff: lane_offset()
-  __device__ __forceinline__ void load(uint64_t origin, uint32_t ld, uint32_t voff, uint32_t tid) {
+  __device__ __forceinline__ void fetch(uint64_t origin, uint32_t ld, const LaneOffsets &lane, uint32_t tid, uint16_t *) {
     const DVM_GLOBAL char *base = reinterpret_cast<const DVM_GLOBAL char *>(origin);
-    if constexpr (KC) {
+    if (ROWS == 256 || tid < ROWS) {
 #pragma unroll
-      for (int i = 0; i < N; ++i) {
-        r[i] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(base + static_cast<uint64_t>(i) * 32u * ld * 2u + voff);
-      }
-    } else {
-      static_assert(ROWS <= 256, "one block per thread");
-      if (ROWS == 256 || tid < ROWS) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          r[j] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(base + static_cast<uint64_t>(j) * ld * 2u + voff);
-        }
+      for (int j = 0; j < 8; ++j) {
+        r[j] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(base + static_cast<uint64_t>(j) * ld * 2u + lane.v[0]);
       }
     }
   }
 
-  __device__ __forceinline__ void store(uint16_t *tile, uint32_t tid) const {
-    if constexpr (KC) {
+  __device__ __forceinline__ void commit(uint16_t *tile, uint32_t tid) const {
+    if (ROWS == 256 || tid < ROWS) {
+      const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
+      // r[j] holds k = kb*8 + j, rows rb*8 .. +7; the tile wants, per row, k = kb*8 .. +7
 #pragma unroll
-      for (int i = 0; i < N; ++i) {
-        const uint32_t c = tid + 256u * i;
-        *reinterpret_cast<vu4 *>(tile + tile_off(c >> 3, c & 7u)) = r[i];
-      }
-    } else {
-      if (ROWS == 256 || tid < ROWS) {
-        const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
-        // r[j] holds k = kb*8 + j, rows rb*8 .. +7; the tile wants, per row, k = kb*8 .. +7
+      for (int i = 0; i < 8; ++i) {
+        vu4 o;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          vu4 o;
-#pragma unroll
-          for (int jj = 0; jj < 4; ++jj) {
-            const uint32_t lo = r[2 * jj][i >> 1], hi = r[2 * jj + 1][i >> 1];
-            // bytes of the result, least significant first: (i odd ? upper : lower) half of lo, then of hi
-            o[jj] = __builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
-          }
-          *reinterpret_cast<vu4 *>(tile + tile_off(rb * 8 + i, kb)) = o;
+        for (int jj = 0; jj < 4; ++jj) {
+          const uint32_t lo = r[2 * jj][i >> 1], hi = r[2 * jj + 1][i >> 1];
+          // bytes of the result, least significant first: (i odd ? upper : lower) half of lo, then of hi
+          o[jj] = __builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
         }
+        *reinterpret_cast<vu4 *>(tile + tile_off(rb * 8 + i, kb)) = o;
       }
     }
   }
@@ -669,10 +691,18 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
     return row + static_cast<uint32_t>(f) * 32u * BK + (x ^ static_cast<uint32_t>((kk << 4) ^ ((f & 1) << 5)));
   };
 
-  for (uint32_t t = blockIdx.x; t < n_tiles; t += gridDim.x) {
+  for (uint32_t t0 = blockIdx.x; t0 < n_tiles; t0 += gridDim.x) {
+    // Tile order. Workgroups are dealt to the 8 XCDs round robin, each XCD has its own L2: workgroup w
+    // takes position (w % 8) * (n_tiles / 8) + w / 8, so an XCD works through one contiguous eighth of the
+    // order; the order itself walks 8-tile-wide column bands row by row, which makes the 32 tiles an XCD has
+    // in flight a 4 x 8 block (12 operand panels to fetch instead of 18 for two full rows of 16).
+    uint32_t t = t0;
+    if ((n_tiles & 7u) == 0 && gridDim.x == n_tiles) t = (t0 & 7u) * (n_tiles >> 3) + (t0 >> 3);
     const uint32_t batch = t / tiles_per_batch, tt = t % tiles_per_batch;
     const uint32_t bi0 = batch / h.nb1, bi1 = batch % h.nb1;
-    const uint32_t tm = tt / h.tiles_n, tn = tt % h.tiles_n;
+    const uint32_t band = tt / (h.tiles_m * 8u), in_band = tt % (h.tiles_m * 8u);
+    const uint32_t band_w = h.tiles_n - band * 8u < 8u ? h.tiles_n - band * 8u : 8u;
+    const uint32_t tm = in_band / band_w, tn = band * 8u + in_band % band_w;
     const uint32_t m0 = tm * BM, n0 = tn * BN;
     const uint64_t a_base = h.a_addr + (static_cast<uint64_t>(bi0) * h.a_sb0 + static_cast<uint64_t>(bi1) * h.a_sb1) * 2;
     const uint64_t b_base = h.b_addr + (static_cast<uint64_t>(bi0) * h.b_sb0 + static_cast<uint64_t>(bi1) * h.b_sb1) * 2;
@@ -691,15 +721,16 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb : static_cast<uint64_t>(n0)) * 2;
       const uint64_t a_step = (A_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.lda) * 2;
       const uint64_t b_step = (B_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.ldb) * 2;
-      const uint32_t a_voff = Stage<BM, A_KC>::lane_offset(h.lda, tid), b_voff = Stage<BN, B_KC>::lane_offset(h.ldb, tid);
-      sa.load(a_org, h.lda, a_voff, tid);
-      sb.load(b_org, h.ldb, b_voff, tid);
-      sa.store(lds, tid);
-      sb.store(lds + kBBase, tid);
+      const LaneOffsets a_voff = Stage<BM, A_KC>::lane_offset(h.lda, tid), b_voff = Stage<BN, B_KC>::lane_offset(h.ldb, tid);
+      sa.fetch(a_org, h.lda, a_voff, tid, lds);
+      sb.fetch(b_org, h.ldb, b_voff, tid, lds + kBBase);
+      sa.commit(lds, tid);
+      sb.commit(lds + kBBase, tid);
       if (nk > 1) {
-        sa.load(a_org + a_step, h.lda, a_voff, tid);
-        sb.load(b_org + b_step, h.ldb, b_voff, tid);
+        sa.fetch(a_org + a_step, h.lda, a_voff, tid, lds + kABuf);
+        sb.fetch(b_org + b_step, h.ldb, b_voff, tid, lds + kBBase + kBBuf);
       }
+      __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): direct loads are not waited for by the barrier itself
       __syncthreads();
       vu4 af[2][TM], bf[2][TN];
       auto read_frags = [&](int fb, uint32_t buf, int kk) {
@@ -716,15 +747,24 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
           for (int j = 0; j < TN; ++j) acc[i][j] = mfma<IS_BF16>(af[fb][i], bf[fb][j], acc[i][j]);
       };
       // One k tile (4 steps of 16). Step s runs its MFMAs on fragment buffer s&1 while the reads of
-      // step s+1 land in the other one. Tile kt+1 is written to the other local-memory buffer during
-      // step 2 (its global loads were issued a tile earlier), the workgroup meets before step 3, and
-      // step 3 overlaps the first fragment reads of tile kt+1 and the global loads of tile kt+2.
+      // step s+1 land in the other one. A k-strided operand's tile kt+1 is written to the other
+      // local-memory buffer during step 1 (its global loads were issued three steps earlier) and the
+      // global loads of its tile kt+2 follow in step 2; the workgroup meets before step 3, which overlaps
+      // the first fragment reads of tile kt+1 and sends the direct loads of tile kt+2 of a k-contiguous
+      // operand into the buffer that has just been read for the last time (a whole tile of slack).
       // The group barriers pin that interleaving: the scheduler would otherwise serialise each read
       // against its use to save registers, and with one wave per SIMD nothing else hides the latency.
       auto k_tile = [&](uint32_t kt, auto has_next, auto has_next2) {
         constexpr bool NEXT = decltype(has_next)::value, NEXT2 = decltype(has_next2)::value;
         constexpr int NF = TM + TN, NM = TM * TN;
         const uint32_t cur = kt & 1u;
+        constexpr int NREST = NM - NF > 0 ? NM - NF : 1;  // MFMAs left in a step after the fragment reads
+        // staging instructions per such MFMA: ds_write of a k-strided operand (step 1), its global loads
+        // (step 2), direct-to-LDS loads of a k-contiguous operand (step 3)
+        constexpr int NW = ((A_KC ? 0 : 8) + (B_KC ? 0 : 8) + NREST - 1) / NREST;
+        constexpr int NL = ((A_KC ? 0 : 8) + (B_KC ? 0 : 8) + NREST - 1) / NREST;
+        constexpr int ND = ((A_KC ? Stage<BM, true>::N : 0) + (B_KC ? Stage<BN, true>::N : 0) + NREST - 1) / NREST;
+        // step 0
         __builtin_amdgcn_sched_barrier(0);
         read_frags(1, cur, 1);
         mfmas(0);
@@ -734,42 +774,61 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_group_barrier(0x008, NM - NF > 0 ? NM - NF : 0, 0);
+        // step 1: tile kt+1 (loaded during the previous tile) goes to the other buffer
         __builtin_amdgcn_sched_barrier(0);
         read_frags(0, cur, 2);
+        if constexpr (NEXT) {
+          sa.commit(lds + (cur ^ 1u) * kABuf, tid);
+          sb.commit(lds + kBBase + (cur ^ 1u) * kBBuf, tid);
+        }
         mfmas(1);
 #pragma unroll
         for (int q = 0; q < NF; ++q) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        __builtin_amdgcn_sched_group_barrier(0x008, NM - NF > 0 ? NM - NF : 0, 0);
+        if constexpr (NEXT && NW > 0) {
+#pragma unroll
+          for (int q = 0; q < NREST; ++q) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x200, NW, 0);
+          }
+        }
+        // step 2: the staging registers are free again: tile kt+2 starts its way from memory
         __builtin_amdgcn_sched_barrier(0);
         read_frags(1, cur, 3);
-        if constexpr (NEXT) {
-          sa.store(lds + (cur ^ 1u) * kABuf, tid);
-          sb.store(lds + kBBase + (cur ^ 1u) * kBBuf, tid);
-        }
+        if constexpr (NEXT2 && !A_KC) sa.fetch(a_org + (kt + 2) * a_step, h.lda, a_voff, tid, lds);
+        if constexpr (NEXT2 && !B_KC) sb.fetch(b_org + (kt + 2) * b_step, h.ldb, b_voff, tid, lds);
         mfmas(0);
 #pragma unroll
         for (int q = 0; q < NF; ++q) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
-        if constexpr (NEXT) {
+        if constexpr (NEXT2 && NL > 0) {
 #pragma unroll
-          for (int q = 0; q < (NM - NF > 0 ? NM - NF : 1); ++q) {
+          for (int q = 0; q < NREST; ++q) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x200, (Stage<BM, A_KC>::N + Stage<BN, B_KC>::N + (NM - NF > 0 ? NM - NF : 1) - 1) / (NM - NF > 0 ? NM - NF : 1), 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, NL, 0);
           }
         }
+        // step 3: every wave has read its last fragments of this buffer and written its share of the
+        // next one a step ago; meet, then start on the next tile's fragments under the last MFMAs
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (NEXT) __syncthreads();
+        if constexpr (NEXT) {
+          // the direct loads of tile kt+1 (issued a tile ago) must have landed before anyone reads them; the
+          // only younger memory operations of this wave are the step-2 loads of a k-strided operand
+          if constexpr (A_KC || B_KC) {
+            constexpr int YOUNGER = (BM == 256 && BN == 256 && NEXT2) ? ((A_KC ? 0 : 8) + (B_KC ? 0 : 8)) : 0;
+            __builtin_amdgcn_s_waitcnt((YOUNGER & 0xf) | ((YOUNGER >> 4) << 14) | (7 << 4) | (15 << 8));
+          }
+          __syncthreads();
+        }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (NEXT) read_frags(0, cur ^ 1u, 0);
-        if constexpr (NEXT2) {
-          sa.load(a_org + (kt + 2) * a_step, h.lda, a_voff, tid);
-          sb.load(b_org + (kt + 2) * b_step, h.ldb, b_voff, tid);
-        }
+        // this buffer has been read for the last time: tile kt+2 of a k-contiguous operand starts its way into it
+        if constexpr (NEXT2 && A_KC) sa.fetch(a_org + (kt + 2) * a_step, h.lda, a_voff, tid, lds + cur * kABuf);
+        if constexpr (NEXT2 && B_KC) sb.fetch(b_org + (kt + 2) * b_step, h.ldb, b_voff, tid, lds + kBBase + cur * kBBuf);
         mfmas(1);
         if constexpr (NEXT) {
 #pragma unroll
@@ -778,11 +837,11 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
           }
         }
-        if constexpr (NEXT2) {
+        if constexpr (NEXT2 && ND > 0) {
 #pragma unroll
-          for (int q = 0; q < (NM - NF > 0 ? NM - NF : 1); ++q) {
+          for (int q = 0; q < NREST; ++q) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x020, (Stage<BM, A_KC>::N + Stage<BN, B_KC>::N + (NM - NF > 0 ? NM - NF : 1) - 1) / (NM - NF > 0 ? NM - NF : 1), 0);
+            __builtin_amdgcn_sched_group_barrier(0x020, ND, 0);
           }
         }
         __builtin_amdgcn_sched_barrier(0);
