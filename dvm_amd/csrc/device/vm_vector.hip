@@ -527,6 +527,71 @@ __device__ __forceinline__ uint32_t group_valid(uint32_t n, const VDim (&dims)[D
   return left < static_cast<uint32_t>(E) ? left : static_cast<uint32_t>(E);
 }
 
+// Arithmetic on one value per lane, for instructions flagged VI_UNIFORM. Out of line: these run once per
+// output (the scalar section between sweeps), never per element.
+__device__ __attribute__((noinline)) float uniform_binary(uint32_t op, uint32_t sub, float x, float y) {
+  if (op == VOP_BINF) {
+    switch (sub & 0x3fu) {
+      case VB_ADD: return x + y;
+      case VB_SUB: return x - y;
+      case VB_RSUB: return y - x;
+      case VB_MUL: return x * y;
+      case VB_DIV: return x / y;
+      case VB_RDIV: return y / x;
+      case VB_MIN: return x < y ? x : y;
+      case VB_MAX: return x > y ? x : y;
+      case VB_AND: return (x != 0.0f && y != 0.0f) ? 1.0f : 0.0f;
+      case VB_OR: return (x != 0.0f || y != 0.0f) ? 1.0f : 0.0f;
+      case VB_POW: return powf(x, y);
+      default: return powf(y, x);
+    }
+  }
+  const uint32_t xi = __float_as_uint(x), yi = __float_as_uint(y);
+  const int32_t xs = __float_as_int(x), ys = __float_as_int(y);
+  if (op == VOP_BINI) {
+    switch (sub & 0x3fu) {
+      case VBI_ADD: return __uint_as_float(xi + yi);
+      case VBI_SUB: return __uint_as_float(xi - yi);
+      case VBI_RSUB: return __uint_as_float(yi - xi);
+      case VBI_MUL: return __uint_as_float(xi * yi);
+      case VBI_MIN: return __int_as_float(min(xs, ys));
+      default: return __int_as_float(max(xs, ys));
+    }
+  }
+  const uint32_t t = sub & 0x7u;
+  if (sub & VCMP_INT) {
+    const bool c = t == VCMP_EQ ? xs == ys : t == VCMP_NE ? xs != ys : t == VCMP_GT ? xs > ys : t == VCMP_GE ? xs >= ys : t == VCMP_LT ? xs < ys : xs <= ys;
+    return __int_as_float(c ? 1 : 0);
+  }
+  const bool c = t == VCMP_EQ ? x == y : t == VCMP_NE ? x != y : t == VCMP_GT ? x > y : t == VCMP_GE ? x >= y : t == VCMP_LT ? x < y : x <= y;
+  return c ? 1.0f : 0.0f;
+}
+
+__device__ __attribute__((noinline)) float uniform_unary(uint32_t sub, float x) {
+  switch (sub) {
+    case VU_SQRT: return sqrtf(x);
+    case VU_ABS: return fabsf(x);
+    case VU_LOG: return logf(x);
+    case VU_EXP: return expf(x);
+    case VU_ISFINITE: return isfinite(x) ? 1.0f : 0.0f;
+    case VU_ROUND: return rintf(x);
+    case VU_FLOOR: return floorf(x);
+    case VU_CEIL: return ceilf(x);
+    case VU_TRUNC: return truncf(x);
+    default: {
+      const uint32_t v = __float_as_uint(x);
+      return __uint_as_float(static_cast<int32_t>(v) < 0 ? 0u - v : v);
+    }
+  }
+}
+
+__device__ __forceinline__ float uniform_cast(uint32_t sub, float x) {
+  if (sub == VC_F2I) return __int_as_float(static_cast<int32_t>(x));
+  if (sub == VC_I2F) return static_cast<float>(__float_as_int(x));
+  if (sub == VC_RND) return x;
+  return x != 0.0f ? 1.0f : 0.0f;
+}
+
 template <int SCHED>
 __device__ __forceinline__ void vm_vector(const VmParam &p) {
   extern __shared__ double lds[];
@@ -613,6 +678,8 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     uint32_t nvp = nvp_out;
     uint32_t round = 0, sweep_pc = 0, slot_kinds = 0;
     uint32_t ridx = r_local;  // reduce-space index of slab 0 in the current round
+    Offs last_off;            // element offsets of the last memory instruction (VI_SAME_OFFS reuses them)
+    FOR_U last_off.v[u] = 0;
 
     uint32_t pc = 0;
     while (true) {
@@ -623,6 +690,24 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       if (op == VOP_END) break;
       const uint32_t sub = (w0 >> 8) & 0xffu, a = w0 >> 24;
 
+      // ---- one value per lane (VI_UNIFORM): compute element 0 and copy it ----
+      if (w0 & VI_UNIFORM) {
+        const uint32_t kind = (w0 >> 16) & 0xfu;
+        float x = acc.v[0][0];
+        if (op >= VOP_SRC_BASE) {
+          const float sv = kind == VK_IMM ? __uint_as_float(imm) : (kind == VK_SREG ? sreg_read(sr, a) : x);
+          x = uniform_binary(op, sub, x, sv);
+        } else if (op == VOP_UN) {
+          x = uniform_unary(sub, x);
+        } else {
+          x = uniform_cast(sub, x);
+        }
+        const uint32_t rnd = (w0 >> 20) & 0x3u;
+        const bool rounds = op == VOP_BINF || op == VOP_UN || (op == VOP_CAST && (sub == VC_I2F || sub == VC_RND));
+        if (rounds) x = rnd == VRND_F16 ? round_f16(x) : (rnd == VRND_BF16 ? round_bf16(x) : x);
+        FOR_U acc.v[u] = x;
+        continue;
+      }
       if (op >= VOP_SRC_BASE) {
         const uint32_t kind = (w0 >> 16) & 0xfu;
         // ---- scalar source (immediate or S register): no need to widen it to U*E values ----
@@ -677,21 +762,24 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
         Acc src;
         if (kind == VK_MEM) {
           const VMemDesc m = load_desc(prog32, mem_off, a);
-          Offs off;
-          if constexpr (SCHED == VS_POINTWISE) {
-            FOR_U {
-              const uint32_t ku = kidx + u * nthreads;
-              off.v[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
-            }
-          } else {
-            const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
-            FOR_U {
-              off.v[u] = koff;
-              if (in_sweep) {
-                const uint32_t ru = ridx + u * r_step;
-                off.v[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+          Offs off = last_off;
+          if (!(w0 & VI_SAME_OFFS)) {
+            if constexpr (SCHED == VS_POINTWISE) {
+              FOR_U {
+                const uint32_t ku = kidx + u * nthreads;
+                off.v[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
+              }
+            } else {
+              const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
+              FOR_U {
+                off.v[u] = koff;
+                if (in_sweep) {
+                  const uint32_t ru = ridx + u * r_step;
+                  off.v[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+                }
               }
             }
+            last_off = off;
           }
           if (op == VOP_LD) {
             mem_load(m, off, nvp, acc);
@@ -795,20 +883,27 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
           const VMemDesc m = load_desc(prog32, mem_off, a);
           Offs off;
           uint32_t nvs = nvp;
-          if constexpr (SCHED == VS_POINTWISE) {
-            FOR_U {
-              const uint32_t ku = kidx + u * nthreads;
-              off.v[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
-            }
+          if (w0 & VI_SAME_OFFS) {
+            off = last_off;
           } else {
-            const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
-            FOR_U {
-              off.v[u] = koff;
-              if (in_sweep) {
-                const uint32_t ru = ridx + u * r_step;
-                off.v[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+            if constexpr (SCHED == VS_POINTWISE) {
+              FOR_U {
+                const uint32_t ku = kidx + u * nthreads;
+                off.v[u] = space_offset(ku < h.n_kidx ? ku : 0u, h.kdims, h.n_kdim, m.kstride, true);
+              }
+            } else {
+              const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
+              FOR_U {
+                off.v[u] = koff;
+                if (in_sweep) {
+                  const uint32_t ru = ridx + u * r_step;
+                  off.v[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+                }
               }
             }
+            last_off = off;
+          }
+          if constexpr (SCHED != VS_POINTWISE) {
             if (!in_sweep) nvs = r_local == 0 ? (nvp & 0xfu) : 0u;  // one lane per output, one slab
           }
           mem_store(m, off, nvs, acc);

@@ -670,8 +670,27 @@ class Compiler {
 
   // emission helpers
   void Emit(uint32_t op, uint32_t sub, uint32_t kind, uint32_t rnd, uint32_t a, uint32_t imm) {
-    code_.push_back(VI_MAKE(op, sub, kind, rnd, a, imm));
+    uint64_t w = VI_MAKE(op, sub, kind, rnd, a, imm);
+    if (!cube_mode_) {
+      const bool mem = op == VOP_ST || (op >= VOP_SRC_BASE && kind == VK_MEM);
+      if (mem) {
+        // consecutive memory instructions of one round that walk memory identically share their offsets
+        if (last_mem_ >= 0 && std::memcmp(mems_[last_mem_].kstride, mems_[a].kstride, sizeof(mems_[a].kstride)) == 0 &&
+            std::memcmp(mems_[last_mem_].rstride, mems_[a].rstride, sizeof(mems_[a].rstride)) == 0) {
+          w |= VI_SAME_OFFS;
+        }
+        last_mem_ = static_cast<int>(a);
+      } else if (op == VOP_SWEEP || op == VOP_ENDSWEEP) {
+        last_mem_ = -1;
+      } else if (uniform_emit_ && (op == VOP_UN || op == VOP_CAST ||
+                                   ((op == VOP_BINF || op == VOP_BINI || op == VOP_CMP) && (kind == VK_IMM || kind == VK_SREG || kind == VK_ACC)))) {
+        w |= VI_UNIFORM;
+      }
+    }
+    code_.push_back(w);
   }
+  int last_mem_ = -1;         // memory operand of the last memory instruction emitted in this round, or -1
+  bool uniform_emit_ = false; // the value being computed is the same in every element of a lane's accumulator
   int Resolve(int v) const {
     while (nodes_[v].kind == AK_ALIAS) v = nodes_[v].in[0];
     return v;
@@ -1248,6 +1267,12 @@ bool NeedsRounding(int op) { return op == kAdd || op == kSub || op == kMul || op
 void Compiler::ComputeInto(int v) {
   ANode &n = nodes_[v];
   NDObject *o = n.op;
+  // outside the sweeps of a reduce kernel, a value without the innermost axis is one number per lane
+  struct UniformScope {
+    bool &flag, saved;
+    UniformScope(bool &f, bool v) : flag(f), saved(f) { flag = v; }
+    ~UniformScope() { flag = saved; }
+  } scope(uniform_emit_, !cube_mode_ && nr_ > 0 && (cur_sec_ & 1) == 0 && !n.has_inner && n.kind == AK_OP);
   switch (n.kind) {
     case AK_MEM:
       BeforeOverwrite();
@@ -1415,6 +1440,7 @@ void Compiler::CountCone(int v) {
 
 void Compiler::EmitSection(int sec) {
   cur_sec_ = sec;
+  last_mem_ = -1;
   const bool sweep = (sec & 1) != 0;
   for (int i = 0; i < nn_; ++i) {
     nodes_[i].uses = 0;

@@ -102,8 +102,14 @@ enum {
 enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 
 // instruction word:
-//   [7:0] opcode  [15:8] sub  [19:16] src kind  [21:20] rnd
+//   [7:0] opcode  [15:8] sub  [19:16] src kind  [21:20] rnd  [22] VI_UNIFORM  [23] VI_SAME_OFFS
 //   [31:24] a (register / memory operand / slot index)   [63:32] imm32
+// VI_UNIFORM (vector VM, arithmetic without a memory or V-register operand): every element of the lane's
+// accumulator holds the same value, the instruction may compute one and copy it.
+// VI_SAME_OFFS (vector VM, memory instructions): the operand has the strides of the previous memory
+// instruction of the same round, whose element offsets are reused.
+#define VI_UNIFORM (1u << 22)
+#define VI_SAME_OFFS (1u << 23)
 #define VI_MAKE(op, sub, kind, rnd, a, imm)                                                     \
   ((uint64_t)(op) | ((uint64_t)(sub) << 8) | ((uint64_t)(kind) << 16) | ((uint64_t)(rnd) << 20) | \
    ((uint64_t)(a) << 24) | ((uint64_t)(uint32_t)(imm) << 32))
