@@ -13,9 +13,11 @@
 //  * the probabilities go to the second MFMA straight from those registers: O^T += V^T P^T sums
 //    over keys, and the order of that sum is free, so the keys a lane happens to hold are fed as they
 //    are and the V^T fragment is read in the matching (permuted) key order;
-//  * K is staged in local memory as it lies in memory (head dimension contiguous), V transposed in
-//    registers on the way in (keys contiguous), both in the XOR-swizzled tile layout of the matmul
-//    kernel and double buffered, the loads of block j+1 in flight during block j;
+//  * K and V blocks go from memory to local memory directly (global_load_lds_dwordx4), as they lie in
+//    memory (head dimension contiguous), in the XOR-swizzled tile layout of the matmul kernel, double
+//    buffered, block j+1 in flight during the whole of block j: no staging registers, no ds_write;
+//  * the V^T fragments stage 2 needs (keys contiguous per lane) come out of that layout with
+//    ds_read_b64_tr_b16, the transposing local-memory read of gfx950;
 //  * Q fragments are read from memory once and stay in registers.
 // Scores stay in fp32 between the stages (the three-kernel graph rounds them to the operand type);
 // the result agrees with the NumPy golden of examples/03_attention.py:20-28 within its 1e-2.
@@ -32,6 +34,7 @@ typedef float vf16 __attribute__((ext_vector_type(16)));
 typedef float vf2 __attribute__((ext_vector_type(2)));
 typedef uint32_t vu4 __attribute__((ext_vector_type(4)));
 typedef uint32_t vu2 __attribute__((ext_vector_type(2)));
+typedef short v4s __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
@@ -53,6 +56,12 @@ __device__ __forceinline__ vf16 mfma(vu4 a, vu4 b, vf16 c) {
   }
 }
 
+// 2^x for x <= 0 (scores minus their running maximum): the bare hardware instruction; results below the
+// normal range flush to zero, which is what a softmax weight of that size amounts to anyway.
+__device__ __forceinline__ float exp2_neg(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ bool wave_all(bool c) { return __builtin_amdgcn_ballot_w64(!c) == 0; }
+
 template <bool IS_BF16>
 __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   const vf2 v = {lo, hi};
@@ -68,10 +77,10 @@ __device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk) {
   return row * ROW + ((chunk ^ ((row ^ (row >> 3)) & 7u)) << 3);
 }
 
-// Local memory per buffer: K block as two tiles [64 keys][64 d] (d halves), V^T block as one tile [128 d][64 keys].
-constexpr uint32_t kKTile = BKV * ROW;           // elements of one K half tile
-constexpr uint32_t kVOff = 2 * kKTile;           // V^T tile after the two K half tiles
-constexpr uint32_t kBuf = 2 * kKTile + D * ROW;  // elements per buffer
+// Local memory per buffer: K block and V block, each as two tiles [64 keys][64 d] (d halves).
+constexpr uint32_t kKTile = BKV * ROW;  // elements of one half tile
+constexpr uint32_t kVOff = 2 * kKTile;  // V block after the K block
+constexpr uint32_t kBuf = 4 * kKTile;   // elements per buffer
 
 template <bool IS_BF16>
 __device__ __forceinline__ void vm_attn(const VmParam &p) {
@@ -101,42 +110,28 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
       qf[qt][kk] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(q_base + (static_cast<uint64_t>(row) * D + 16 * kk + 8 * lh) * 2);
   }
 
-  // staging: K block = 64 keys x 128 d = 1024 chunks of 16 bytes, 4 per thread, copied as they are;
-  // V block = 128 (8x8 blocks along d: 16) x (along keys: 8) blocks, one per thread for the first 128
-  vu4 ks[4], vs[8];
-  const uint32_t v_kb = tid >> 4, v_db = tid & 15u;  // 8x8 block of V this thread transposes (tid < 128)
-  auto load_kv = [&](uint32_t key0) {
+  // Staging. A block of K or V is 64 keys x 128 d = two half tiles (d < 64, d >= 64) of 64 rows x 8 chunks of
+  // 16 bytes. Chunk position p = 256*i + tid (i = 0..3) of a block is half tile i/2, key 32*(i&1) + tid/8,
+  // physical chunk tid%8; the lane fetches the logical chunk that belongs there (physical ^ swizzle(key)),
+  // and a wave's 64 chunks land in 1 KB of consecutive local memory.
+  uint32_t ld_off[2];  // byte offset of the lane's chunk inside a block, for even / odd i
+#pragma unroll
+  for (int par = 0; par < 2; ++par) {
+    const uint32_t key = 32u * par + (tid >> 3);
+    const uint32_t logical = (tid & 7u) ^ ((key ^ (key >> 3)) & 7u);
+    ld_off[par] = ((tid >> 3) * D + (logical << 3)) * 2u;
+  }
+  const uint32_t wave_first = uni(wave) * 64u;
+  auto fetch_kv = [&](uint32_t key0, uint32_t buf) {
+    uint16_t *kdst = lds + buf * kBuf, *vdst = lds + buf * kBuf + kVOff;
+    const DVM_GLOBAL char *ksrc = reinterpret_cast<const DVM_GLOBAL char *>(k_base + static_cast<uint64_t>(key0) * D * 2);
+    const DVM_GLOBAL char *vsrc = reinterpret_cast<const DVM_GLOBAL char *>(v_base + static_cast<uint64_t>(key0) * D * 2);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const uint32_t c = tid + 256u * i;  // chunk: key = c / 16, d chunk = c % 16
-      ks[i] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(k_base + (static_cast<uint64_t>(key0 + (c >> 4)) * D + ((c & 15u) << 3)) * 2);
-    }
-    if (tid < 128) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j)
-        vs[j] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(v_base + (static_cast<uint64_t>(key0 + v_kb * 8 + j) * D + v_db * 8) * 2);
-    }
-  };
-  auto store_kv = [&](uint32_t buf) {
-    uint16_t *base = lds + buf * kBuf;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t c = tid + 256u * i;
-      const uint32_t key = c >> 4, dc = c & 15u;
-      *reinterpret_cast<vu4 *>(base + (dc >> 3) * kKTile + tile_off(key, dc & 7u)) = ks[i];
-    }
-    if (tid < 128) {
-      // vs[j] holds key v_kb*8 + j, d = v_db*8 .. +7; row d of V^T wants keys v_kb*8 .. +7
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        vu4 o;
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj) {
-          const uint32_t lo = vs[2 * jj][i >> 1], hi = vs[2 * jj + 1][i >> 1];
-          o[jj] = __builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
-        }
-        *reinterpret_cast<vu4 *>(base + kVOff + tile_off(v_db * 8 + i, v_kb)) = o;
-      }
+      const uint32_t src_off = (i & 1) * 32u * D * 2u + (i >> 1) * 64u * 2u + ld_off[i & 1];  // keys 32.. for odd i, d 64.. for i >= 2
+      const uint32_t dst_off = (static_cast<uint32_t>(i) * 256u + wave_first) * 8u;
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(ksrc + src_off), (__attribute__((address_space(3))) void *)(kdst + dst_off), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(vsrc + src_off), (__attribute__((address_space(3))) void *)(vdst + dst_off), 16, 0, 0);
     }
   };
 
@@ -153,15 +148,24 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
   const uint32_t swz0 = (lj ^ (lj >> 3)) & 7u;
   const uint32_t lane_row = lj * ROW;
   const uint32_t k_x = (lh ^ swz0) << 3;  // K fragment: chunk 2*(kk&3) + h
-  const uint32_t v_x = swz0 << 3;         // V^T fragment: whole chunks, the half-wave picks 4 elements inside
+  // V^T fragments through ds_read_b64_tr_b16. Within a group of 16 lanes, lane r = 4*j + q supplies the
+  // address of 4 consecutive d of key K_j, and lane i of the group receives d0 + i of K_0..K_3. Groups
+  // 0/1 take d0 = 0/16 of a 32-wide d tile for the keys of half-wave 0, groups 2/3 the same for half-wave
+  // 1 (the half-waves' keys differ by 4, as in the score registers).
+  const uint32_t tr_j = (lane & 15u) >> 2, tr_q = lane & 3u, tr_g = lane >> 4;
+  const uint32_t tr_key = 4u * (tr_g >> 1) + tr_j;                 // key inside its group of 8 (low 3 bits)
+  const uint32_t tr_chunk = 2u * (tr_g & 1u) + (tr_q >> 1);          // 16-byte chunk inside the half d tile
+  const uint32_t tr_base = tr_key * ROW + 4u * (tr_q & 1u);          // row part + the half of the chunk
+  const uint32_t tr_x = (tr_chunk ^ tr_key) << 3;
   const uint32_t n_blocks = skv / BKV;
-  load_kv(0);
-  store_kv(0);
-  if (n_blocks > 1) load_kv(BKV);
+  fetch_kv(0, 0);
+  __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): the barrier does not wait for direct loads by itself
   __syncthreads();
   for (uint32_t kb = 0; kb < n_blocks; ++kb) {
     const uint32_t cur = kb & 1u;
     const uint16_t *kbuf = lds + cur * kBuf, *vbuf = lds + cur * kBuf + kVOff;
+    // the other buffer was read for the last time before the barrier that ended the previous block
+    if (kb + 1 < n_blocks) fetch_kv((kb + 1) * BKV, cur ^ 1u);
     // stage 1: S^T[key][query] for 2 key tiles x 2 query tiles
     vf16 s[2][2];
 #pragma unroll
@@ -180,8 +184,6 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
         for (int qt = 0; qt < 2; ++qt) s[kt][qt] = mfma<IS_BF16>(kf[kt], qf[qt][kk], s[kt][qt]);
       if (kk & 1) __builtin_amdgcn_sched_barrier(0);  // keep the fragment reads near their use: registers are scarce
     }
-    // the next block goes to the other buffer while the softmax runs
-    if (kb + 1 < n_blocks) store_kv(cur ^ 1u);
     __builtin_amdgcn_sched_barrier(0);
     // softmax of this block, per query (= per lane, both half-waves share a query)
     vu4 pf[2][2][2];  // [key tile][16-key step][query tile]: B operand of stage 2
@@ -194,14 +196,14 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
         for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kt][qt][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float m_new = fmaxf(m_run[qt], mx * c_log2);
-      const float alpha = exp2f(m_run[qt] - m_new);
+      const float alpha = exp2_neg(m_run[qt] - m_new);
       m_run[qt] = m_new;
       float sum = 0.0f;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-          const float pv = exp2f(s[kt][qt][r] * c_log2 - m_new);
+          const float pv = exp2_neg(s[kt][qt][r] * c_log2 - m_new);
           s[kt][qt][r] = pv;
           sum += pv;
         }
@@ -211,8 +213,11 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
           for (int e = 0; e < 4; ++e) pf[kt][st][qt][e] = pack2<IS_BF16>(s[kt][qt][8 * st + 2 * e], s[kt][qt][8 * st + 2 * e + 1]);
       }
       l_run[qt] = l_run[qt] * alpha + sum;
+      // after the first blocks the running maximum rarely moves: skip the rescale when no lane needs it
+      if (!wave_all(alpha == 1.0f)) {
 #pragma unroll
-      for (int dt = 0; dt < D / 32; ++dt) o_acc[dt][qt] = o_acc[dt][qt] * alpha;
+        for (int dt = 0; dt < D / 32; ++dt) o_acc[dt][qt] = o_acc[dt][qt] * alpha;
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
     // stage 2: O^T[d][query] += V^T[d][key] P^T[key][query]. Step (kt, st) contracts the 16 keys the
@@ -224,11 +229,16 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
         vu4 vf[D / 32];
 #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt) {
-          const int c0 = kt * 4 + st * 2;  // chunk of keys 32*kt + 16*st .. +7, the next chunk holds +8 .. +15
-          const uint16_t *rowp = vbuf + dt * 32 * ROW + lane_row + 4 * lh;
-          const vu2 a = *reinterpret_cast<const vu2 *>(rowp + (v_x ^ static_cast<uint32_t>((c0 ^ (4 * (dt & 1))) << 3)));
-          const vu2 bq = *reinterpret_cast<const vu2 *>(rowp + (v_x ^ static_cast<uint32_t>(((c0 + 1) ^ (4 * (dt & 1))) << 3)));
-          vf[dt] = vu4{a[0], a[1], bq[0], bq[1]};
+          // keys C + tr_key and C + 8 + tr_key, C = 32*kt + 16*st; swizzle(key) = (key & 7) ^ ((key >> 3) & 7), chunk =
+          // 4*(dt & 1) | tr_chunk: every address is a lane base plus (tr_x ^ constant) plus a constant
+          vu2 part[2];
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            const int c = kt * 32 + st * 16 + w * 8;
+            const uint16_t *ptr = vbuf + (dt >> 1) * kKTile + c * ROW + tr_base + (tr_x ^ static_cast<uint32_t>(((4 * (dt & 1)) ^ ((c >> 3) & 7)) << 3));
+            part[w] = __builtin_bit_cast(vu2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(ptr)));
+          }
+          vf[dt] = vu4{part[0][0], part[0][1], part[1][0], part[1][1]};
         }
 #pragma unroll
         for (int dt = 0; dt < D / 32; ++dt)
@@ -237,8 +247,8 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
         __builtin_amdgcn_sched_barrier(0);
       }
     }
+    __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): the next block has landed
     __syncthreads();
-    if (kb + 2 < n_blocks) load_kv((kb + 2) * BKV);
   }
 
   // O[query][d] = O^T / l, rounded once to the operand type. Lane (j, h) holds, per d tile and register
