@@ -91,7 +91,12 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
   const float scale = hp->scale;
   const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
   const uint32_t lj = lane & 31u, lh = lane >> 5;
-  const uint32_t b = blockIdx.x / q_blocks, qb = blockIdx.x % q_blocks;
+  // Workgroups are dealt to the 8 XCDs round robin and each XCD has its own L2: workgroup w takes position
+  // (w % 8) * (grid / 8) + w / 8 of the (head, query block) order, so the query blocks of one head, which
+  // all read the same K and V, run on one XCD at the same time and share them in its L2.
+  uint32_t pos = blockIdx.x;
+  if ((gridDim.x & 7u) == 0) pos = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const uint32_t b = pos / q_blocks, qb = pos % q_blocks;
   const uint64_t q_base = hp->q_addr + static_cast<uint64_t>(b) * sq * D * 2;
   const uint64_t k_base = hp->k_addr + static_cast<uint64_t>(b) * skv * D * 2;
   const uint64_t v_base = hp->v_addr + static_cast<uint64_t>(b) * skv * D * 2;
@@ -166,23 +171,38 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
     const uint16_t *kbuf = lds + cur * kBuf, *vbuf = lds + cur * kBuf + kVOff;
     // the other buffer was read for the last time before the barrier that ended the previous block
     if (kb + 1 < n_blocks) fetch_kv((kb + 1) * BKV, cur ^ 1u);
-    // stage 1: S^T[key][query] for 2 key tiles x 2 query tiles
+    // stage 1: S^T[key][query] for 2 key tiles x 2 query tiles. The fragments of step kk+1 are read while the
+    // MFMAs of step kk run (pinned: one wave per SIMD, nothing else would hide the local-memory latency).
     vf16 s[2][2];
+    vu4 kf[2][2];
+    auto read_k = [&](int fb, int kk) {
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-      for (int qt = 0; qt < 2; ++qt) s[kt][qt] = 0.0f;
+      for (int kt = 0; kt < 2; ++kt)
+        kf[fb][kt] = *reinterpret_cast<const vu4 *>(kbuf + (kk >> 2) * kKTile + kt * 32 * ROW + lane_row + (k_x ^ static_cast<uint32_t>((((kk & 3) * 2) ^ (4 * kt)) << 3)));
+    };
+    read_k(0, 0);
 #pragma unroll
     for (int kk = 0; kk < D / 16; ++kk) {
-      vu4 kf[2];
+      __builtin_amdgcn_sched_barrier(0);
+      if (kk + 1 < D / 16) read_k((kk + 1) & 1, kk + 1);
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
-        kf[kt] = *reinterpret_cast<const vu4 *>(kbuf + (kk >> 2) * kKTile + kt * 32 * ROW + lane_row + (k_x ^ static_cast<uint32_t>((((kk & 3) * 2) ^ (4 * kt)) << 3)));
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) s[kt][qt] = mfma<IS_BF16>(kf[kt], qf[qt][kk], s[kt][qt]);
-      if (kk & 1) __builtin_amdgcn_sched_barrier(0);  // keep the fragment reads near their use: registers are scarce
+        for (int qt = 0; qt < 2; ++qt) {
+          if (kk == 0) {
+            const vf16 zero = 0.0f;
+            s[kt][qt] = mfma<IS_BF16>(kf[0][kt], qf[qt][0], zero);
+          } else {
+            s[kt][qt] = mfma<IS_BF16>(kf[kk & 1][kt], qf[qt][kk], s[kt][qt]);
+          }
+        }
+      if (kk + 1 < D / 16) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
     // softmax of this block, per query (= per lane, both half-waves share a query)
@@ -221,32 +241,43 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
     }
     __builtin_amdgcn_sched_barrier(0);
     // stage 2: O^T[d][query] += V^T[d][key] P^T[key][query]. Step (kt, st) contracts the 16 keys the
-    // lane's registers 8*st .. 8*st+7 of tile kt hold: keys 32*kt + 16*st + {0..3, 8..11} + 4*h.
+    // lane's registers 8*st .. 8*st+7 of tile kt hold: keys 32*kt + 16*st + {0..3, 8..11} + 4*h. Fragments
+    // of the next step are read under the MFMAs of the current one.
+    vu4 vf[2][D / 32];
+    auto read_v = [&](int fb, int step) {
+      const int kt = step >> 1, st = step & 1;
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
+      for (int dt = 0; dt < D / 32; ++dt) {
+        // keys C + tr_key and C + 8 + tr_key, C = 32*kt + 16*st; swizzle(key) = (key & 7) ^ ((key >> 3) & 7), chunk =
+        // 4*(dt & 1) | tr_chunk: every address is a lane base plus (tr_x ^ constant) plus a constant
+        vu2 part[2];
 #pragma unroll
-      for (int st = 0; st < 2; ++st) {
-        vu4 vf[D / 32];
-#pragma unroll
-        for (int dt = 0; dt < D / 32; ++dt) {
-          // keys C + tr_key and C + 8 + tr_key, C = 32*kt + 16*st; swizzle(key) = (key & 7) ^ ((key >> 3) & 7), chunk =
-          // 4*(dt & 1) | tr_chunk: every address is a lane base plus (tr_x ^ constant) plus a constant
-          vu2 part[2];
-#pragma unroll
-          for (int w = 0; w < 2; ++w) {
-            const int c = kt * 32 + st * 16 + w * 8;
-            const uint16_t *ptr = vbuf + (dt >> 1) * kKTile + c * ROW + tr_base + (tr_x ^ static_cast<uint32_t>(((4 * (dt & 1)) ^ ((c >> 3) & 7)) << 3));
-            part[w] = __builtin_bit_cast(vu2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(ptr)));
-          }
-          vf[dt] = vu4{part[0][0], part[0][1], part[1][0], part[1][1]};
+        for (int w = 0; w < 2; ++w) {
+          const int c = kt * 32 + st * 16 + w * 8;
+          const uint16_t *ptr = vbuf + (dt >> 1) * kKTile + c * ROW + tr_base + (tr_x ^ static_cast<uint32_t>(((4 * (dt & 1)) ^ ((c >> 3) & 7)) << 3));
+          part[w] = __builtin_bit_cast(vu2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s *)(ptr)));
         }
+        vf[fb][dt] = vu4{part[0][0], part[0][1], part[1][0], part[1][1]};
+      }
+    };
+    read_v(0, 0);
 #pragma unroll
-        for (int dt = 0; dt < D / 32; ++dt)
+    for (int step = 0; step < 4; ++step) {
+      __builtin_amdgcn_sched_barrier(0);
+      if (step + 1 < 4) read_v((step + 1) & 1, step + 1);
 #pragma unroll
-          for (int qt = 0; qt < 2; ++qt) o_acc[dt][qt] = mfma<IS_BF16>(vf[dt], pf[kt][st][qt], o_acc[dt][qt]);
-        __builtin_amdgcn_sched_barrier(0);
+      for (int dt = 0; dt < D / 32; ++dt)
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) o_acc[dt][qt] = mfma<IS_BF16>(vf[step & 1][dt], pf[step >> 1][step & 1][qt], o_acc[dt][qt]);
+      if (step + 1 < 4) {
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
       }
     }
+    __builtin_amdgcn_sched_barrier(0);
     __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): the next block has landed
     __syncthreads();
   }
