@@ -63,6 +63,12 @@ def build(force=False, verbose=False):
         dev_objs.append(obj)
         if force or _stale(obj, [src] + deps):
             jobs.append(["hipcc"] + HIP_FLAGS + ["-c", src, "-o", obj])
+        if os.path.basename(src) == "vm_vector.hip":
+            # second build of the vector VM: four slabs per lane per instruction (kernels dvm_vm_vec_*_u4)
+            obj4 = os.path.join(OBJ, "vm_vector_u4.hip.o")
+            dev_objs.append(obj4)
+            if force or _stale(obj4, [src] + deps):
+                jobs.append(["hipcc"] + HIP_FLAGS + ["-DDVM_VEC_U=4", "-c", src, "-o", obj4])
     for src in _sources("host", ".cc"):
         obj = os.path.join(OBJ, os.path.basename(src) + ".o")
         host_objs.append(obj)

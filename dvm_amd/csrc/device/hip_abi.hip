@@ -13,6 +13,9 @@
 extern "C" __global__ void dvm_vm_vec_pw(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_rx(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_ry(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_pw_u4(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_rx_u4(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_ry_u4(const VmParam p);
 #define DVM_CUBE_DECL(prefix)                                \
   extern "C" __global__ void prefix##_nn(const VmParam p); \
   extern "C" __global__ void prefix##_nt(const VmParam p); \
@@ -53,11 +56,13 @@ __global__ void dvm_fill_u32_kernel(uint32_t *dst, uint32_t value, size_t n) {
   for (; i < n; i += stride) dst[i] = value;
 }
 
-// waves per SIMD each interpreter kernel fits at (from its VGPR count)
+// waves per SIMD each interpreter kernel fits at (from its VGPR count, allocated in blocks of 8: 92, 102 and 127
+// registers). The grid is a multiple of what is resident: one workgroup too many per CU costs a whole extra pass.
 uint32_t kernel_waves_per_simd(uint64_t kind) {
-  switch (kind) {
+  if (kind & VS_WIDE) return 2;
+  switch (kind & VS_KIND_MASK) {
     case VS_POINTWISE: return 5;
-    case VS_REDX: return 5;
+    case VS_REDX: return 4;
     case VS_REDY: return 4;
     default: return 2;
   }
@@ -84,7 +89,9 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
   g_dev.lds_per_wg = static_cast<uint32_t>(prop.sharedMemPerBlock);
   // gfx950 lets one workgroup use the CU's whole 160 KB; the kernels must opt in.
   std::vector<const void *> kernels = {reinterpret_cast<const void *>(dvm_vm_vec_pw), reinterpret_cast<const void *>(dvm_vm_vec_rx),
-                                       reinterpret_cast<const void *>(dvm_vm_vec_ry)};
+                                       reinterpret_cast<const void *>(dvm_vm_vec_ry),
+                                       reinterpret_cast<const void *>(dvm_vm_vec_pw_u4), reinterpret_cast<const void *>(dvm_vm_vec_rx_u4),
+                                       reinterpret_cast<const void *>(dvm_vm_vec_ry_u4)};
   for (const auto &tile : kCubeKernels)
     for (const auto &dt : tile)
       for (CubeKernel k : dt) kernels.push_back(reinterpret_cast<const void *>(k));
@@ -142,15 +149,17 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
         VI_OP(p.w[code_end - 1]) != VOP_END || h->n_kdim > DVM_VEC_MAXR || h->n_rdim > DVM_VEC_MAXR) {
       return static_cast<int>(hipErrorInvalidValue);
     }
-    switch (h->sched) {
+    const bool wide = (h->sched & VS_WIDE) != 0;
+    if (wide && threads > 512) return static_cast<int>(hipErrorInvalidValue);
+    switch (h->sched & VS_KIND_MASK) {
       case VS_POINTWISE:
-        hipLaunchKernelGGL(dvm_vm_vec_pw, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        hipLaunchKernelGGL(wide ? dvm_vm_vec_pw_u4 : dvm_vm_vec_pw, dim3(block_dim), dim3(threads), lds_bytes, s, p);
         break;
       case VS_REDX:
-        hipLaunchKernelGGL(dvm_vm_vec_rx, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        hipLaunchKernelGGL(wide ? dvm_vm_vec_rx_u4 : dvm_vm_vec_rx, dim3(block_dim), dim3(threads), lds_bytes, s, p);
         break;
       case VS_REDY:
-        hipLaunchKernelGGL(dvm_vm_vec_ry, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        hipLaunchKernelGGL(wide ? dvm_vm_vec_ry_u4 : dvm_vm_vec_ry, dim3(block_dim), dim3(threads), lds_bytes, s, p);
         break;
       default:
         return static_cast<int>(hipErrorInvalidValue);

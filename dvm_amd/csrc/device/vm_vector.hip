@@ -1017,6 +1017,13 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
 
 }  // namespace
 
+#if DVM_VEC_U == DVM_VEC_U_WIDE
+// the wide build: more registers per lane, so at most 512 lanes per workgroup
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_vec_pw_u4(const VmParam p) { vm_vector<VS_POINTWISE>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_vec_rx_u4(const VmParam p) { vm_vector<VS_REDX>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_vec_ry_u4(const VmParam p) { vm_vector<VS_REDY>(p); }
+#else
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_pw(const VmParam p) { vm_vector<VS_POINTWISE>(p); }
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_rx(const VmParam p) { vm_vector<VS_REDX>(p); }
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_ry(const VmParam p) { vm_vector<VS_REDY>(p); }
+#endif

@@ -183,7 +183,6 @@ namespace {
 constexpr int kMaxNodes = 160;     // nodes of one sub-kernel
 constexpr int kMaxAxes = 24;       // domain axes before merging
 constexpr int E = DVM_VEC_E;
-constexpr int U = DVM_VEC_U;
 
 enum AKind : uint8_t { AK_MEM, AK_SCALAR, AK_OP, AK_ALIAS, AK_REDUCE, AK_OUT };
 
@@ -690,6 +689,7 @@ class Compiler {
     code_.push_back(w);
   }
   int last_mem_ = -1;         // memory operand of the last memory instruction emitted in this round, or -1
+  int u_ = 2;                 // slabs per lane per instruction of the program being compiled
   bool uniform_emit_ = false; // the value being computed is the same in every element of a lane's accumulator
   int Resolve(int v) const {
     while (nodes_[v].kind == AK_ALIAS) v = nodes_[v].in[0];
@@ -1017,6 +1017,16 @@ void Compiler::ChooseSchedule() {
   hdr_.n_ridx = static_cast<uint32_t>(n_r);
   uint32_t threads = 256;
   single_round_ = true;
+  // Slabs per lane per instruction: the wide build of the VM halves the dispatches per element at the price
+  // of registers (at most 512 lanes per workgroup, two waves per SIMD). It pays where the instruction stream,
+  // not memory, sets the pace: reduces along the innermost axis with long rows.
+  // Measured on MI355X it does not pay (batch-norm 98 us against 76, RMSNorm 118 us against 104): two waves per
+  // SIMD hide too little latency. Kept as a tuning switch, off by default.
+  bool wide = false;
+  if (const char *e = std::getenv("DVM_VEC_WIDE")) wide = e[0] == '1' && !(nr_ > 0 && !inner_red);
+  u_ = wide ? DVM_VEC_U_WIDE : 2;
+  const uint32_t U = static_cast<uint32_t>(u_);
+  const uint32_t max_threads = wide ? 512u : 1024u;
   if (nr_ == 0) {
     hdr_.sched = VS_POINTWISE;
     if (n_k <= 64 * U) threads = 64;
@@ -1027,7 +1037,7 @@ void Compiler::ChooseSchedule() {
     hdr_.sched = VS_REDX;
     // lanes that share one output: enough to cover the reduce space in one round if possible
     uint32_t team = Pow2Ceil((n_r + U - 1) / U);
-    if (team > 1024) team = 1024;
+    if (team > max_threads) team = max_threads;
     if (team > 64) {
       hdr_.team_is_block = 1;
       threads = team;
@@ -1046,7 +1056,7 @@ void Compiler::ChooseSchedule() {
     uint32_t tx = n_k >= 64 ? 64 : Pow2Ceil(n_k);
     uint32_t ty = 256 / tx;
     const uint64_t items = (n_k + tx - 1) / tx;
-    if (items < 128 && n_r > 256) ty = 1024 / tx;  // few outputs: give each more lanes along the reduce space
+    if (items < 128 && n_r > 256) ty = max_threads / tx;  // few outputs: give each more lanes along the reduce space
     while (ty > 1 && static_cast<uint64_t>(ty) * U > 2 * n_r) ty >>= 1;
     threads = std::max<uint32_t>(64, tx * ty);
     ty = threads / tx;
@@ -1054,6 +1064,7 @@ void Compiler::ChooseSchedule() {
     hdr_.n_items = static_cast<uint32_t>(items);
     single_round_ = n_r <= static_cast<uint64_t>(ty) * U;
   }
+  if (wide) hdr_.sched |= VS_WIDE;
   prog_->threads = threads;
 }
 
@@ -1604,7 +1615,7 @@ void Compiler::EmitProgram() {
     }
   }
   // local memory budget for V registers
-  const uint32_t per_slot = static_cast<uint32_t>(U) * 16u * prog_->threads;
+  const uint32_t per_slot = static_cast<uint32_t>(u_) * 16u * prog_->threads;
   const uint32_t budget = g_system.lds_per_wg > 80 * 1024 ? 72 * 1024 : g_system.lds_per_wg - 8 * 1024;
   vslot_limit_ = std::min<int>(DVM_VEC_NREG, static_cast<int>(budget / per_slot));
   sreg_used_ = vslot_used_ = 0;
@@ -1627,7 +1638,7 @@ void Compiler::FinishProgram() {
   std::memcpy(prog_->blob.w, &hdr_, sizeof(hdr_));
   std::memcpy(prog_->blob.w + hdr_.mem_off, mems_, sizeof(VMemDesc) * n_mem_);
   std::memcpy(prog_->blob.w + hdr_.code_off, code_.data(), 8 * code_.size());
-  prog_->lds_bytes = prog_->threads * 8 + static_cast<uint32_t>(max_vslot_) * U * 16 * prog_->threads;
+  prog_->lds_bytes = prog_->threads * 8 + static_cast<uint32_t>(max_vslot_) * u_ * 16 * prog_->threads;
   uint64_t gt = (static_cast<uint64_t>(std::min<uint32_t>(hdr_.n_items, g_system.core_num * 4)) << 32) | prog_->threads;
   if (g_system.HasDevice()) {
     gt = g_system.Api().select_block_thread(hdr_.sched, hdr_.n_items, prog_->threads, prog_->lds_bytes);

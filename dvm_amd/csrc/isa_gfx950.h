@@ -15,7 +15,13 @@
 #define DVM_PARAM_BYTES 4096          // program blob travels as a kernel argument
 #define DVM_PARAM_WORDS (DVM_PARAM_BYTES / 8)
 #define DVM_VEC_E 8                   // consecutive elements per lane per slab (one or two 128-bit accesses)
-#define DVM_VEC_U 2                   // slabs per lane per instruction
+// Slabs per lane per instruction. The vector VM is built twice: with 2 (kernels dvm_vm_vec_*: up to 1024
+// lanes per workgroup) and with 4 (dvm_vm_vec_*_u4: half the instruction dispatches per element, more
+// registers per lane, up to 512 lanes per workgroup); VS_WIDE in the header's schedule word selects the latter.
+#ifndef DVM_VEC_U
+#define DVM_VEC_U 2
+#endif
+#define DVM_VEC_U_WIDE 4
 #define DVM_VEC_NREG 16               // V register slots per lane (local memory, sized per program)
 #define DVM_VEC_NSREG 8               // one-float S registers per lane (VGPRs)
 #define DVM_VEC_NSLOT 2               // concurrent reduce accumulators per sweep
@@ -43,6 +49,8 @@ enum {
   VS_POINTWISE = 0,  // lanes enumerate the whole (kept) index space, no reduce
   VS_REDX = 1,       // innermost axis is reduced: a team of lanes strides the reduce space of one output
   VS_REDY = 2,       // innermost axis is kept: lanes own output groups, wave rows partition the reduce space
+  VS_KIND_MASK = 0xf,
+  VS_WIDE = 0x10,    // flag: the program is laid out for DVM_VEC_U_WIDE slabs per lane (the *_u4 kernels)
 };
 
 // ---- opcodes ---------------------------------------------------------------
@@ -144,7 +152,7 @@ enum { VMF_VEC = 1 /* innermost stride 1 */, VMF_ALIGNED = 2 /* every E-group st
 
 typedef struct {
   uint32_t entry;        // VE_VECTOR
-  uint32_t sched;        // VS_*
+  uint32_t sched;        // VS_* | VS_WIDE
   uint32_t n_mem;
   uint32_t n_code;       // instruction words
   uint32_t n_kdim;
