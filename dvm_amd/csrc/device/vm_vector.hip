@@ -350,8 +350,36 @@ __device__ __forceinline__ void red_accumulate_k(RedAcc<SCHED> &r, const Acc &x,
   }
 }
 
+// Every slab of every lane of the wave is full (the common round): no per-element guards.
+template <int SCHED, int KIND>
+__device__ __forceinline__ void red_accumulate_full(RedAcc<SCHED> &r, const Acc &x) {
+  FOR_U {
+    if constexpr (SCHED == VS_REDY) {
+      FOR_E r.v[e] = red_op<KIND>(r.v[e], static_cast<double>(x.v[u][e]));
+    } else {
+      float d[E];
+      FOR_E d[e] = x.v[u][e];
+#pragma unroll
+      for (int w = 1; w < E; w <<= 1)
+#pragma unroll
+        for (int e = 0; e + w < E; e += 2 * w) d[e] = red_op<KIND>(d[e], d[e + w]);
+      r.v[0] = red_op<KIND>(r.v[0], static_cast<double>(d[0]));
+    }
+  }
+}
+
 template <int SCHED>
 __device__ __forceinline__ void red_accumulate(RedAcc<SCHED> &r, uint32_t kind, const Acc &x, uint32_t nvp) {
+  if (wave_all(nvp == kAllFull)) {
+    if (kind == VR_SUM) {
+      red_accumulate_full<SCHED, VR_SUM>(r, x);
+    } else if (kind == VR_MAX) {
+      red_accumulate_full<SCHED, VR_MAX>(r, x);
+    } else {
+      red_accumulate_full<SCHED, VR_MIN>(r, x);
+    }
+    return;
+  }
   if (kind == VR_SUM) {
     red_accumulate_k<SCHED, VR_SUM>(r, x, nvp);
   } else if (kind == VR_MAX) {

@@ -688,6 +688,7 @@ class Compiler {
     }
     code_.push_back(w);
   }
+  void DropCastBeforeStore(const uint32_t *mem_dtypes);
   int last_mem_ = -1;         // memory operand of the last memory instruction emitted in this round, or -1
   int u_ = 2;                 // slabs per lane per instruction of the program being compiled
   bool uniform_emit_ = false; // the value being computed is the same in every element of a lane's accumulator
@@ -1627,7 +1628,36 @@ void Compiler::EmitProgram() {
   Emit(VOP_END, 0, 0, 0, 0, 0);
 }
 
+
+// A rounding cast to fp16 / bf16 whose only reader is the store right behind it does nothing the store's own
+// conversion does not do (same round to nearest even): the cast instruction is dropped. `mem_dtypes[i]` is the
+// element type of memory operand i.
+void Compiler::DropCastBeforeStore(const uint32_t *mem_dtypes) {
+  std::vector<uint64_t> out;
+  out.reserve(code_.size());
+  for (size_t i = 0; i < code_.size(); ++i) {
+    const uint64_t w = code_[i];
+    if (VI_OP(w) == VOP_CAST && VI_SUB(w) == VC_RND && !(static_cast<uint32_t>(w) & VI_UNIFORM) && i + 2 < code_.size() + 1 && i + 1 < code_.size()) {
+      const uint64_t st = code_[i + 1];
+      const uint32_t next = i + 2 < code_.size() ? VI_OP(code_[i + 2]) : static_cast<uint32_t>(VOP_END);
+      const bool acc_dead = next == VOP_END || next == VOP_ENDSWEEP || next == VOP_SWEEP || next == VOP_LD || next == VOP_LDR ||
+                            next == VOP_LDS || next == VOP_LDI || next == VOP_FIN;
+      if (VI_OP(st) == VOP_ST && acc_dead) {
+        const uint32_t dt = mem_dtypes[VI_A(st)];
+        if ((VI_RND(w) == VRND_F16 && dt == VDT_F16) || (VI_RND(w) == VRND_BF16 && dt == VDT_BF16)) continue;
+      }
+    }
+    out.push_back(w);
+  }
+  code_.swap(out);
+}
+
 void Compiler::FinishProgram() {
+  {
+    uint32_t dts[DVM_VEC_MAXMEM];
+    for (int i = 0; i < n_mem_; ++i) dts[i] = mems_[i].dtype;
+    DropCastBeforeStore(dts);
+  }
   hdr_.n_mem = n_mem_;
   hdr_.n_code = static_cast<uint32_t>(code_.size());
   hdr_.mem_off = sizeof(VVecHeader) / 8;
@@ -1876,6 +1906,11 @@ void Compiler::CompileCube(int a) {
     ConsumeUse(x);
   }
   Emit(VOP_END, 0, 0, 0, 0, 0);
+  {
+    uint32_t dts[DVM_CUBE_MAXMEM];
+    for (int i = 0; i < n_mem_; ++i) dts[i] = cmems_[i].dtype;
+    DropCastBeforeStore(dts);
+  }
   h.n_mem = n_mem_;
   h.n_code = static_cast<uint32_t>(code_.size());
   h.mem_off = sizeof(VCubeHeader) / 8;
