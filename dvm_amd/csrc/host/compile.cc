@@ -181,6 +181,7 @@ void VKernel::Normalize() {
 namespace {
 
 constexpr int kMaxNodes = 160;     // nodes of one sub-kernel
+constexpr int kMaxAreaOps = 100;   // operators the partitioner puts into one sub-kernel
 constexpr int kMaxAxes = 24;       // domain axes before merging
 constexpr int E = DVM_VEC_E;
 
@@ -351,6 +352,7 @@ class Compiler {
     int64_t dom[kMaxRank];
     const NDObject *cube_op = nullptr;
     int attn = -1;  // index into attn_groups_ when the sub-kernel is one fused attention
+    int n_ops = 0;  // operators joined so far (a program has room for about 500 instruction words and 160 nodes)
   };
   std::vector<AreaInfo> areas_;
 
@@ -433,6 +435,7 @@ class Compiler {
     if (a >= static_cast<int>(areas_.size())) return true;  // a fresh sub-kernel
     const AreaInfo &ai = areas_[a];
     if (o->kind == kObjMatMul) return false;
+    if (ai.n_ops >= kMaxAreaOps && o->kind != kObjStore) return false;  // long graphs are cut into several launches
     if (ai.attn >= 0) return o->kind == kObjStore && o->in[0] == attn_groups_[ai.attn].m2;
     if (ai.cube) {
       if (!IsPointwiseKind(o->kind)) return false;
@@ -454,6 +457,7 @@ class Compiler {
   void Join(int a, const NDObject *o) {
     while (a >= static_cast<int>(areas_.size())) areas_.push_back(AreaInfo());
     AreaInfo &ai = areas_[a];
+    ++ai.n_ops;
     if (o->kind == kObjMatMul) {
       ai.cube = true;
       ai.cube_op = o;

@@ -236,3 +236,21 @@ def test_composite_gelu_tanh():  # tests/ut/test_composite_ops.py:22-71
         inner = (x + x * x * x * dt(0.044715)) * dt(0.7978845608)
         g = x * dt(0.5) * (np_tanh(inner) + dt(1.0))
         run_parity(lambda k, a: [gelu(k, a), tanh(k, a)], [x], eps=eps, golden=[g, np_tanh(x)], golden_eps=eps * 2)
+
+
+def test_graph_longer_than_one_program():  # tests/ut/test_eager_fusion.py:551-800 (bytecode beyond 4 KB): cut into several launches
+    x = np.random.default_rng(9).normal(0, 1, [64, 48]).astype(np.float32)
+
+    def build(k, a):
+        y = a
+        for i in range(700):
+            y = k.add(y, 0.5) if i % 2 else k.mul(y, 1.001)
+        return y
+    want = x.copy()
+    for i in range(700):
+        want = want + np.float32(0.5) if i % 2 else want * np.float32(1.001)
+    t = Tester("split")
+    out = t.store(build(t, t.load(x)))
+    t.run()
+    assert 2 <= t.num_launches() <= 10
+    assert np.array_equal(t.output(out), want)

@@ -216,3 +216,22 @@ def test_zero_size():  # tests/ut/test_codegen.py:116-164
     t.run()
     assert np.array_equal(t.output(s), np.zeros([16], np.float32))
     assert t.output(e).shape == (0, 16)
+
+
+def test_wide_build_matches(monkeypatch):
+    # the optional four-slabs-per-lane build of the VM (DVM_VEC_WIDE=1) computes the same results
+    monkeypatch.setenv("DVM_VEC_WIDE", "1")
+    rng = np.random.default_rng(77)
+    x = rng.normal(0, 1, [6, 5, 700]).astype(np.float32)
+    g = rng.normal(0, 1, [5, 1]).astype(np.float32)
+
+    def build(k, a, b):
+        m = k.mul(k.sum(a, (0, 2), True), 1.0 / 4200)
+        d = k.sub(a, m)
+        return [k.mul(d, b), k.max(a, (2,), False), k.add(a, 1.0)]
+    outs = run_parity(build, [x, g], golden=[(x - x.mean((0, 2), keepdims=True)) * g, x.max(2), x + 1], eps=1e-5)
+    assert outs[0].shape == x.shape
+    t = Tester("split", run_mode="das")
+    t.store(t.sum(t.load(x), (2,), False))
+    t.codegen()
+    assert " wide " in t.das()
