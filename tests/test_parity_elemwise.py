@@ -6,6 +6,7 @@ and bools exact); the graph additionally runs on the CPU oracle and both results
 import numpy as np
 import pytest
 
+from dvm_amd.tester import Tester
 from tests.util import run_parity
 
 pytestmark = pytest.mark.gpu
