@@ -24,6 +24,9 @@ def _load():
         raise ImportError(
             "dvm_amd native library missing (%s): run `python -m dvm_amd.build` first" % _LIB_PATH)
     lib = ctypes.CDLL(_LIB_PATH)
+    if not hasattr(lib, "dvm_rt_seq_add"):
+        raise ImportError("dvm_amd native library (%s) is older than the package: run `python -m dvm_amd.build`"
+                          % _LIB_PATH)
     vp, ci, cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
     i64p = ctypes.POINTER(ctypes.c_int64)
     opp = ctypes.POINTER(_Operand)
@@ -50,6 +53,8 @@ def _load():
         "dvm_rt_copy": (vp, [vp, vp]),
         "dvm_rt_matmul": (vp, [vp, vp, vp, ci, ci, vp]),
         "dvm_rt_set_store_inplace": (ci, [vp, vp]),
+        "dvm_rt_seq_add": (ci, [vp, ci, ctypes.c_uint]),
+        "dvm_rt_parallel_add": (ci, [vp, ci, ctypes.c_uint, cs]),
         "dvm_obj_rank": (ci, [vp]),
         "dvm_obj_shape": (ci, [vp, i64p, cs]),
         "dvm_obj_dtype": (ci, [vp]),
@@ -79,7 +84,20 @@ def _load():
     return lib
 
 
-_lib = _load()
+class _LazyLib:
+    """Loads libdvm.so at the first call, so that importing the package (the build step does) needs no
+    built library; any use of the backend without one raises ImportError."""
+
+    def __getattr__(self, name):
+        lib = self.__dict__.get("_real")
+        if lib is None:
+            lib = self.__dict__["_real"] = _load()
+            global _lib
+            _lib = lib
+        return getattr(lib, name)
+
+
+_lib = _LazyLib()
 
 
 def _check(ret):
@@ -226,6 +244,13 @@ class Kernel:
 
     def set_store_inplace(self, store):
         _check(_lib.dvm_rt_set_store_inplace(self._rt, store._h))
+
+    # -- sub-kernel groups of "seq" / "parallel" kernels (include/dvm_py.h:369-371) --
+    def seq_add(self, ktype, flags=0):
+        _check(_lib.dvm_rt_seq_add(self._rt, int(ktype), int(flags)))
+
+    def parallel_add(self, ktype, flags=0, core_limit=0):
+        _check(_lib.dvm_rt_parallel_add(self._rt, int(ktype), int(flags), int(core_limit)))
 
     # -- operators --
     def cast(self, input, type):

@@ -137,6 +137,10 @@ void ParseKernelType(const std::string &s, KernelType *type, uint32_t *flags) {
     *type = kMix;
   } else if (name == "cube") {
     *type = kCube;
+  } else if (name == "parallel") {
+    *type = kParallel;
+  } else if (name == "seq") {
+    *type = kSequence;
   } else {
     throw std::runtime_error("DVM EXCEPTION. reason: kernel type '" + name + "' is not supported by the gfx950 backend");
   }
@@ -387,6 +391,24 @@ dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int 
   return Guard(
       [&]() { return Handle(rt->kernel.MatMul(Obj(lhs), Obj(rhs), trans_a != 0, trans_b != 0, Obj(bias))); },
       static_cast<dvm_obj *>(nullptr));
+}
+
+int dvm_rt_seq_add(dvm_rt *rt, int ktype, unsigned flags) {
+  return Guard(
+      [&]() {
+        rt->kernel.SequenceAdd(static_cast<KernelType>(ktype), flags);
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_parallel_add(dvm_rt *rt, int ktype, unsigned flags, size_t core_limit) {
+  return Guard(
+      [&]() {
+        rt->kernel.ParallelAdd(static_cast<KernelType>(ktype), flags, core_limit);
+        return 0;
+      },
+      -1);
 }
 
 int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store) {

@@ -36,6 +36,7 @@ VKernel::~VKernel() {
 
 NDObject *VKernel::Append(NDObject *op) {
   op->id = static_cast<int>(ops_.size());
+  op->stage = cur_stage_;
   ops_.push_back(op);
   normalized_ = false;
   compiled_ = false;
@@ -352,6 +353,7 @@ class Compiler {
     int64_t dom[kMaxRank];
     const NDObject *cube_op = nullptr;
     int attn = -1;  // index into attn_groups_ when the sub-kernel is one fused attention
+    int stage = 0;  // the caller's group (parallel / sequence kernels); operators of different groups never share a launch
     int n_ops = 0;  // operators joined so far (a program has room for about 500 instruction words and 160 nodes)
   };
   std::vector<AreaInfo> areas_;
@@ -434,6 +436,7 @@ class Compiler {
   bool CanJoin(int a, const NDObject *o) {
     if (a >= static_cast<int>(areas_.size())) return true;  // a fresh sub-kernel
     const AreaInfo &ai = areas_[a];
+    if (ai.stage != o->stage) return false;
     if (o->kind == kObjMatMul) return false;
     if (ai.n_ops >= kMaxAreaOps && o->kind != kObjStore) return false;  // long graphs are cut into several launches
     if (ai.attn >= 0) return o->kind == kObjStore && o->in[0] == attn_groups_[ai.attn].m2;
@@ -457,6 +460,7 @@ class Compiler {
   void Join(int a, const NDObject *o) {
     while (a >= static_cast<int>(areas_.size())) areas_.push_back(AreaInfo());
     AreaInfo &ai = areas_[a];
+    if (ai.n_ops == 0) ai.stage = o->stage;
     ++ai.n_ops;
     if (o->kind == kObjMatMul) {
       ai.cube = true;
@@ -506,6 +510,8 @@ class Compiler {
           g.area = static_cast<int>(areas_.size());
           areas_.push_back(AreaInfo());
           areas_.back().attn = attn_of_[i];
+          areas_.back().stage = o->stage;
+          areas_.back().n_ops = 1;
         }
         area_[i] = g.area;
         continue;

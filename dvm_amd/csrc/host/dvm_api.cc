@@ -189,9 +189,12 @@ class Builder {
 
   NDObject *New(ObjKind kind, DataType t, NDObject *a = nullptr, NDObject *b = nullptr, NDObject *c = nullptr) {
     NDObject *o = new NDObject(kind, t);
-    o->in[0] = a;
-    o->in[1] = b;
-    o->in[2] = c;
+    // A Store handed on as an operand (a later stage of a sequence kernel reading an earlier stage's
+    // output, tests/ut/test_sequence_fusion.py:190-197) stands for the value it stores.
+    auto value_of = [](NDObject *x) { return x != nullptr && x->kind == kObjStore ? x->in[0] : x; };
+    o->in[0] = value_of(a);
+    o->in[1] = value_of(b);
+    o->in[2] = value_of(c);
     o->nin = c != nullptr ? 3 : (b != nullptr ? 2 : (a != nullptr ? 1 : 0));
     return k_->Append(o);
   }
@@ -462,6 +465,8 @@ void Kernel::Reset(KernelType type, uint32_t flags) {
     case kCube:
     case kMix:
     case kSplit:
+    case kParallel:
+    case kSequence:
       break;
     default:
       kernel_ = nullptr;
@@ -490,6 +495,7 @@ void Kernel::Clone(const Kernel &base, CloneHelper &helper) {
     c->aux_ref = o->aux_ref != nullptr ? helper.GetClone(o->aux_ref) : nullptr;
     c->addr = o->addr;
     if (o->kind == kObjLoad) c->shape_ref_ = c->aux_ref;
+    kernel_->SetStage(o->stage);
     kernel_->Append(c);
     helper.SetClone(o, c);
   }
@@ -677,8 +683,21 @@ NDObject *Kernel::AllGatherV2(NDObject *, const Comm *) { Unsupported("AllGather
 NDObject *Kernel::ReduceScatter(NDObject *, const Comm *) { Unsupported("ReduceScatter (single-GPU backend)"); }
 NDObject *Kernel::ExtOut(NDObject *, int) { Unsupported("ExtOut"); }
 void Kernel::SpecNext() { Unsupported("speculative kernels"); }
-void Kernel::ParallelAdd(KernelType, uint32_t, size_t) { Unsupported("parallel kernels"); }
-void Kernel::SequenceAdd(KernelType, uint32_t) { Unsupported("sequence kernels"); }
+
+// Parallel and sequence kernels (src/xkernel.h, include/dvm.h:248-251 of the reference): the caller
+// names the groups, every group becomes one or more launches of its own. The sub-kernel type and the
+// core limit are advice for the reference's tile model; here the partitioner's own rules decide what
+// a launch holds, and launches of one kernel run in stream order, which is a valid schedule for both.
+void Kernel::ParallelAdd(KernelType type, uint32_t, size_t) {
+  if (kernel_ == nullptr || kernel_->KType() != kParallel) Throw("ParallelAdd needs a kernel reset as kParallel");
+  if (type != kVector && type != kCube && type != kMix) Unsupported("this sub-kernel type");
+  kernel_->NextStage();
+}
+void Kernel::SequenceAdd(KernelType type, uint32_t) {
+  if (kernel_ == nullptr || kernel_->KType() != kSequence) Throw("SequenceAdd needs a kernel reset as kSequence");
+  if (type != kVector && type != kCube && type != kMix) Unsupported("this sub-kernel type");
+  kernel_->NextStage();
+}
 void Kernel::Clear() {}
 
 void Kernel::Normalize() { kernel_->Normalize(); }

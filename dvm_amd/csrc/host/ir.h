@@ -67,6 +67,7 @@ class NDObject {
   IntArrayRef *aux_ref = nullptr;  // reduce axes / broadcast target / reshape target / user shape of a load
   void *addr = nullptr;            // load / store address (may arrive later through a RelocEntry)
   int id = -1;                     // position in the kernel's operator list
+  int stage = 0;                   // sub-kernel group opened by Kernel::ParallelAdd / SequenceAdd
 
   // Shape as the API sees it, outermost first. Loads point at the caller's
   // IntArrayRef (dynamic shapes), every other node at its own storage.
@@ -150,6 +151,11 @@ class VKernel {
   bool IsDynamic() const { return (flags_ & kDynamic) != 0; }
 
   NDObject *Append(NDObject *op);
+  // Opens the next group of a parallel / sequence kernel: operators appended from now on never share
+  // a launch with earlier ones (src/xkernel.h: SeqKernel / ParallelKernel stages).
+  void NextStage() { ++cur_stage_; }
+  int Stage() const { return cur_stage_; }
+  void SetStage(int s) { cur_stage_ = s; }
   void Normalize();
   // Compiles every sub-kernel. With `pre` set no addresses are needed yet; returns the workspace size.
   size_t CodeGen(bool pre);
@@ -175,6 +181,7 @@ class VKernel {
   uint32_t flags_;
   bool normalized_ = false;
   bool compiled_ = false;
+  int cur_stage_ = 0;
   std::string dump_str_;
   friend class Compiler;
 };

@@ -61,6 +61,10 @@ dvm_obj *dvm_rt_reduce(dvm_rt *rt, int reduce_type, dvm_obj *x, dvm_shape *dims,
 dvm_obj *dvm_rt_copy(dvm_rt *rt, dvm_obj *x);
 dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int trans_b, dvm_obj *bias);
 int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store);
+// Group markers of "seq" and "parallel" kernels (KernelPy::SequenceAdd / ParallelAdd, include/dvm_py.h:369-371; Kernel::SequenceAdd /
+// ParallelAdd, include/dvm.h:250-251): operators built after the call belong to the next sub-kernel group.
+int dvm_rt_seq_add(dvm_rt *rt, int ktype, unsigned flags);
+int dvm_rt_parallel_add(dvm_rt *rt, int ktype, unsigned flags, size_t core_limit);
 
 int dvm_obj_rank(const dvm_obj *o);
 int dvm_obj_shape(const dvm_obj *o, int64_t *dims, size_t cap);

@@ -230,8 +230,18 @@ def _tid(dtype):
 
 
 class OracleKernel:
+    K_VEC, K_CUBE, K_MIX = 0, 1, 2
+
     def __init__(self):
         self.stores = []
+
+    # Group markers of sequence / parallel kernels (include/dvm.h:250-251 of the reference) say where
+    # launches end, not what is computed: the restatement evaluates operator by operator either way.
+    def seq_add(self, ktype, flags=0):
+        pass
+
+    def parallel_add(self, ktype, flags=0, core_limit=0):
+        pass
 
     # -- leaves --
     def load(self, array, dtype=None):

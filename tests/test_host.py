@@ -195,7 +195,7 @@ def test_zero_size_shapes_are_idle():
 
 def test_errors_are_runtime_errors_with_the_reference_prefix():
     with pytest.raises(RuntimeError, match="DVM EXCEPTION"):
-        Tester("parallel", run_mode="das")
+        Tester("eager", run_mode="das")
     t = Tester("vector", run_mode="das")
     a = t.load(np.zeros([4, 3], np.float32))
     b = t.load(np.zeros([4, 5], np.float32))
@@ -260,3 +260,49 @@ def test_attention_graph_is_recognised():
     for sq, skv, d in ((300, 192, 64), (300, 100, 128)):
         das = _attention(Tester("mix", run_mode="das"), sq, skv, d)
         assert das.count("== sub-kernel") == 3 and das.count("entry cube") == 2 and "entry attention" not in das, das
+
+
+def test_sequence_groups_are_launch_boundaries():
+    # tests/ut/test_sequence_fusion.py:22-33: two groups joined by a value; without the marker one launch would do
+    def build(kind, marker):
+        t = Tester(kind, run_mode="das")
+        if marker:
+            t.seq_add(Tester.K_VEC)
+        a = t.load(np.zeros([1024, 128], np.float32))
+        c = t.mul(a, t.add(a, 0.2))
+        if marker:
+            t.seq_add(Tester.K_VEC)
+        t.store_expect(t.mul(c, 0.7), 0)
+        t.codegen()
+        return t
+    assert build("split", False).num_launches() == 1
+    t = build("seq", True)
+    assert t.num_launches() == 2
+    assert t.workspace_bytes() >= 1024 * 128 * 4  # the value crossing the boundary lives in the workspace
+    with pytest.raises(RuntimeError, match="kSequence"):
+        Tester("split", run_mode="das").seq_add(Tester.K_VEC)
+    with pytest.raises(RuntimeError, match="kParallel"):
+        Tester("seq", run_mode="das").parallel_add(Tester.K_VEC)
+
+
+def test_parallel_groups_never_share_a_launch():
+    # tests/ut/test_parallel_fusion.py:26-48: three independent sub-kernels
+    t = Tester("parallel", run_mode="das")
+    for n in (256, 256, 1024):
+        t.parallel_add(Tester.K_VEC)
+        t.store_expect(t.add(t.load(np.zeros([n], np.float32)), 0.3), 0)
+    t.codegen()
+    assert t.num_launches() == 3
+
+
+def test_store_as_operand_reads_the_stored_value():
+    # tests/ut/test_sequence_fusion.py:190-197: a later group multiplies two earlier outputs
+    t = Tester("seq", run_mode="das")
+    t.seq_add(Tester.K_VEC)
+    a = t.load(np.zeros([8, 64], np.float32))
+    o0 = t.store_expect(t.add(a, 1.0), 0)
+    t.seq_add(Tester.K_VEC)
+    t.store_expect(t.mul(o0, o0), 0)
+    t.codegen()
+    assert t.num_launches() == 2
+    assert t.workspace_bytes() == 0  # the second group reads the first group's output buffer
