@@ -151,6 +151,13 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
     }
     const bool wide = (h->sched & VS_WIDE) != 0;
     if (wide && threads > 512) return static_cast<int>(hipErrorInvalidValue);
+    {
+      // local memory the interpreter will touch: reduce scratch and V registers
+      const uint64_t u = wide ? DVM_VEC_U_WIDE : 2;
+      if (lds_bytes < static_cast<uint64_t>(threads) * 8 + static_cast<uint64_t>(h->n_vslot) * u * 16 * threads) {
+        return static_cast<int>(hipErrorInvalidValue);
+      }
+    }
     switch (h->sched & VS_KIND_MASK) {
       case VS_POINTWISE:
         hipLaunchKernelGGL(wide ? dvm_vm_vec_pw_u4 : dvm_vm_vec_pw, dim3(block_dim), dim3(threads), lds_bytes, s, p);

@@ -47,6 +47,11 @@ constexpr uint32_t kAllOnes = U == 4 ? 0x1111u : (U == 2 ? 0x11u : 0x1u);
 constexpr uint32_t kAllFull = kAllOnes * 8u;
 
 __device__ __forceinline__ uint32_t uni(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+// Arguments of an out-of-line function arrive in vector registers even when every lane holds the same value;
+// reading them back through the first lane lets the function branch on them with scalar branches.
+__device__ __forceinline__ uint64_t uni64(uint64_t v) {
+  return (static_cast<uint64_t>(uni(static_cast<uint32_t>(v >> 32))) << 32) | uni(static_cast<uint32_t>(v));
+}
 
 __device__ __forceinline__ uint32_t fast_div(uint32_t n, const VDim &d) { return (__umulhi(n, d.magic) + n) >> d.shift; }
 
@@ -161,6 +166,9 @@ struct Offs {
 };
 
 __device__ __attribute__((noinline)) Acc mem_load_slow(uint64_t addr, uint32_t dtype, uint32_t flags, Offs off, uint32_t nvp) {
+  addr = uni64(addr);
+  dtype = uni(dtype);
+  flags = uni(flags);
   VMemDesc m;
   m.addr = addr;
   m.dtype = dtype;
@@ -188,6 +196,9 @@ __device__ __attribute__((noinline)) Acc mem_load_slow(uint64_t addr, uint32_t d
 }
 
 __device__ __attribute__((noinline)) void mem_store_slow(uint64_t addr, uint32_t dtype, uint32_t flags, Offs off, uint32_t nvp, Acc in) {
+  addr = uni64(addr);
+  dtype = uni(dtype);
+  flags = uni(flags);
   VMemDesc m;
   m.addr = addr;
   m.dtype = dtype;
@@ -395,6 +406,10 @@ template <int SCHED>
 __device__ __attribute__((noinline)) RedAcc<SCHED> red_finalize(RedAcc<SCHED> r, uint32_t rk, uint32_t tlog, bool team_is_block,
                                                                 uint32_t tid, uint32_t nthreads, uint32_t k_local,
                                                                 uint32_t r_local, double *scratch) {
+  rk = uni(rk);
+  tlog = uni(tlog);
+  team_is_block = uni(team_is_block ? 1u : 0u) != 0u;
+  nthreads = uni(nthreads);
   if constexpr (SCHED == VS_REDX) {
     double t = r.v[0];
     const uint32_t span = team_is_block ? 64u : (1u << tlog);
@@ -555,9 +570,11 @@ __device__ __forceinline__ uint32_t group_valid(uint32_t n, const VDim (&dims)[D
   return left < static_cast<uint32_t>(E) ? left : static_cast<uint32_t>(E);
 }
 
-// Arithmetic on one value per lane, for instructions flagged VI_UNIFORM. Out of line: these run once per
-// output (the scalar section between sweeps), never per element.
-__device__ __attribute__((noinline)) float uniform_binary(uint32_t op, uint32_t sub, float x, float y) {
+// Arithmetic on one value per lane, for instructions flagged VI_UNIFORM. Inlined, so that the opcode stays
+// in scalar registers and the selection below is a scalar branch (as arguments of an out-of-line function
+// the opcodes travel in vector registers and every case is walked under an execution mask); the library
+// functions with internal per-lane branches go through the out-of-line slab helpers.
+__device__ __forceinline__ float uniform_binary(uint32_t op, uint32_t sub, float x, float y) {
   if (op == VOP_BINF) {
     switch (sub & 0x3fu) {
       case VB_ADD: return x + y;
@@ -570,8 +587,8 @@ __device__ __attribute__((noinline)) float uniform_binary(uint32_t op, uint32_t 
       case VB_MAX: return x > y ? x : y;
       case VB_AND: return (x != 0.0f && y != 0.0f) ? 1.0f : 0.0f;
       case VB_OR: return (x != 0.0f || y != 0.0f) ? 1.0f : 0.0f;
-      case VB_POW: return powf(x, y);
-      default: return powf(y, x);
+      case VB_POW: return slab_pow(vf8(x), vf8(y))[0];
+      default: return slab_pow(vf8(y), vf8(x))[0];
     }
   }
   const uint32_t xi = __float_as_uint(x), yi = __float_as_uint(y);
@@ -595,12 +612,12 @@ __device__ __attribute__((noinline)) float uniform_binary(uint32_t op, uint32_t 
   return c ? 1.0f : 0.0f;
 }
 
-__device__ __attribute__((noinline)) float uniform_unary(uint32_t sub, float x) {
+__device__ __forceinline__ float uniform_unary(uint32_t sub, float x) {
   switch (sub) {
-    case VU_SQRT: return sqrtf(x);
+    case VU_SQRT: return slab_sqrt(vf8(x))[0];
     case VU_ABS: return fabsf(x);
-    case VU_LOG: return logf(x);
-    case VU_EXP: return expf(x);
+    case VU_LOG: return slab_log(vf8(x))[0];
+    case VU_EXP: return slab_exp(vf8(x))[0];
     case VU_ISFINITE: return isfinite(x) ? 1.0f : 0.0f;
     case VU_ROUND: return rintf(x);
     case VU_FLOOR: return floorf(x);
@@ -655,6 +672,8 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   const uint32_t nthreads = blockDim.x;
   const uint32_t tlog = h.team_log2;
   const bool team_is_block = h.team_is_block != 0;
+  // per-team runs (VOP_UNI_BEGIN .. VOP_UNI_END) are computed by the first wave when the team is the workgroup
+  const uint32_t skips_runs = (SCHED == VS_REDX && team_is_block && uni(tid >> 6) != 0u) ? 1u : 0u;
   vf4 *planes = reinterpret_cast<vf4 *>(lds + nthreads);  // first nthreads doubles: reduce scratch
 
   // lane -> (kept local index, reduce local index)
@@ -709,14 +728,24 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     Offs last_off;            // element offsets of the last memory instruction (VI_SAME_OFFS reuses them)
     FOR_U last_off.v[u] = 0;
 
+    // The instruction word is read from local memory one instruction ahead: the read of the next word is
+    // in flight while the current instruction executes. The next pc is known at decode time, because only
+    // the end of a round (VOP_ENDSWEEP, or an instruction flagged to close the round) ever jumps.
+    const vu2 *code64 = reinterpret_cast<const vu2 *>(code32);
     uint32_t pc = 0;
+    vu2 fetched = code64[0];
     while (true) {
-      const uint32_t w0 = uni(code32[2 * pc]);
-      const uint32_t imm = uni(code32[2 * pc + 1]);
-      ++pc;
-      const uint32_t op = w0 & 0xffu;
+      const uint32_t w0 = uni(fetched[0]);
+      const uint32_t imm = uni(fetched[1]);
+      const uint32_t op = w0 & 0x7fu;
       if (op == VOP_END) break;
       const uint32_t sub = (w0 >> 8) & 0xffu, a = w0 >> 24;
+      // branch-free: the round-closing bit and, for the waves that skip per-team runs, the jump to their end
+      const bool ends = SCHED != VS_POINTWISE && (w0 & VI_ENDS) != 0;
+      const uint32_t back = (ends ? 1u : 0u) & (round + 1 < n_rounds ? 1u : 0u);
+      pc = back ? sweep_pc : pc + 1;
+      pc += ((op == VOP_UNI_BEGIN ? 1u : 0u) & skips_runs) * (imm - 1u);
+      fetched = code64[pc];
 
       // ---- one value per lane (VI_UNIFORM): compute element 0 and copy it ----
       if (w0 & VI_UNIFORM) {
@@ -739,24 +768,32 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       if (op >= VOP_SRC_BASE) {
         const uint32_t kind = (w0 >> 16) & 0xfu;
         // ---- scalar source (immediate or S register): no need to widen it to U*E values ----
-        if ((kind == VK_IMM || kind == VK_SREG) && (op == VOP_BINF || op == VOP_BINI || op == VOP_CMP)) {
-          const float sv = kind == VK_IMM ? __uint_as_float(imm) : sreg_read(sr, a);
+        if ((kind == VK_IMM || kind == VK_SREG || kind == VK_SREG2) && (op == VOP_BINF || op == VOP_BINI || op == VOP_CMP)) {
+          float sv = kind == VK_IMM ? __uint_as_float(imm) : sreg_read(sr, a);
           if (op == VOP_BINF) {
-            switch (sub & 0x3fu) {
-              case VB_ADD: FOR_U acc.v[u] = acc.v[u] + sv; break;
-              case VB_SUB: FOR_U acc.v[u] = acc.v[u] - sv; break;
-              case VB_RSUB: FOR_U acc.v[u] = sv - acc.v[u]; break;
-              case VB_MUL: FOR_U acc.v[u] = acc.v[u] * sv; break;
-              case VB_DIV: FOR_U acc.v[u] = acc.v[u] / sv; break;
-              case VB_RDIV: FOR_U acc.v[u] = sv / acc.v[u]; break;
-              case VB_MIN: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] < sv ? acc.v[u][e] : sv; break;
-              case VB_MAX: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] > sv ? acc.v[u][e] : sv; break;
-              case VB_AND: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f && sv != 0.0f) ? 1.0f : 0.0f; break;
-              case VB_OR: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f || sv != 0.0f) ? 1.0f : 0.0f; break;
-              case VB_POW: FOR_U acc.v[u] = slab_pow(acc.v[u], vf8(sv)); break;
-              default: FOR_U acc.v[u] = slab_pow(vf8(sv), acc.v[u]); break;
+            // one operation, or two chained ones (VK_SREG2: the second sits in the immediate)
+            uint32_t bsub = sub & 0x3fu, brnd = (w0 >> 20) & 0x3u;
+            for (uint32_t left = kind == VK_SREG2 ? 2u : 1u;;) {
+              switch (bsub) {
+                case VB_ADD: FOR_U acc.v[u] = acc.v[u] + sv; break;
+                case VB_SUB: FOR_U acc.v[u] = acc.v[u] - sv; break;
+                case VB_RSUB: FOR_U acc.v[u] = sv - acc.v[u]; break;
+                case VB_MUL: FOR_U acc.v[u] = acc.v[u] * sv; break;
+                case VB_DIV: FOR_U acc.v[u] = acc.v[u] / sv; break;
+                case VB_RDIV: FOR_U acc.v[u] = sv / acc.v[u]; break;
+                case VB_MIN: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] < sv ? acc.v[u][e] : sv; break;
+                case VB_MAX: FOR_U FOR_E acc.v[u][e] = acc.v[u][e] > sv ? acc.v[u][e] : sv; break;
+                case VB_AND: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f && sv != 0.0f) ? 1.0f : 0.0f; break;
+                case VB_OR: FOR_U FOR_E acc.v[u][e] = (acc.v[u][e] != 0.0f || sv != 0.0f) ? 1.0f : 0.0f; break;
+                case VB_POW: FOR_U acc.v[u] = slab_pow(acc.v[u], vf8(sv)); break;
+                default: FOR_U acc.v[u] = slab_pow(vf8(sv), acc.v[u]); break;
+              }
+              apply_rnd(acc, brnd);
+              if (--left == 0u) break;
+              bsub = imm & 0x3fu;
+              brnd = (imm >> 16) & 0x3u;
+              sv = sreg_read(sr, (imm >> 8) & 0xffu);
             }
-            apply_rnd(acc, (w0 >> 20) & 0x3u);
           } else if (op == VOP_BINI) {
             const uint32_t si = __float_as_uint(sv);
             switch (sub & 0x3fu) {
@@ -907,6 +944,27 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
         case VOP_STS:
           sreg_write(sr, a, acc.v[0][0]);
           break;
+        case VOP_UNI_END: {
+          if constexpr (SCHED == VS_REDX) {
+            if (team_is_block) {
+              // what the run produced lives in the first wave's S registers and accumulator: pass it on
+              float *box = reinterpret_cast<float *>(lds);  // the reduce scratch is idle between sweeps
+              __syncthreads();
+              if (tid == 0) {
+                *reinterpret_cast<vf4 *>(box) = vf4{sr.s0, sr.s1, sr.s2, sr.s3};
+                *reinterpret_cast<vf4 *>(box + 4) = vf4{sr.s4, sr.s5, sr.s6, sr.s7};
+                box[8] = acc.v[0][0];
+              }
+              __syncthreads();
+              const vf4 lo = *reinterpret_cast<const vf4 *>(box), hi = *reinterpret_cast<const vf4 *>(box + 4);
+              const float av = box[8];
+              sr.s0 = lo[0]; sr.s1 = lo[1]; sr.s2 = lo[2]; sr.s3 = lo[3];
+              sr.s4 = hi[0]; sr.s5 = hi[1]; sr.s6 = hi[2]; sr.s7 = hi[3];
+              FOR_U acc.v[u] = av;  // (the next user of the scratch starts with a barrier of its own)
+            }
+          }
+          break;
+        }
         case VOP_ST: {
           const VMemDesc m = load_desc(prog32, mem_off, a);
           Offs off;
@@ -978,10 +1036,11 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       if constexpr (SCHED != VS_POINTWISE) {
         switch (op) {
           case VOP_RED: {
+            if (sub & VRF_SQUARE) FOR_U acc.v[u] = acc.v[u] * acc.v[u];  // the emitter fuses only where acc is dead afterwards
             if (a == 0) {
-              red_accumulate<SCHED>(racc0, sub, acc, nvp);
+              red_accumulate<SCHED>(racc0, sub & 0xfu, acc, nvp);
             } else {
-              red_accumulate<SCHED>(racc1, sub, acc, nvp);
+              red_accumulate<SCHED>(racc1, sub & 0xfu, acc, nvp);
             }
             break;
           }
@@ -993,19 +1052,6 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             red_init<SCHED>(racc0, slot_kinds & 0xfu);
             red_init<SCHED>(racc1, (slot_kinds >> 4) & 0xfu);
             ridx = r_local;
-            break;
-          }
-          case VOP_ENDSWEEP: {
-            ++round;
-            if (round < n_rounds) {
-              ridx += r_step * U;
-              pc = sweep_pc;
-            } else {
-              in_sweep = false;
-              const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
-              if (k0 <= VR_MIN) racc0 = red_finalize<SCHED>(racc0, k0, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
-              if (k1 <= VR_MIN) racc1 = red_finalize<SCHED>(racc1, k1, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
-            }
             break;
           }
           case VOP_FIN: {
@@ -1023,8 +1069,22 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             break;
         }
 
+        // end of a round: the next one (the decode above has already turned the pc back), or the end of
+        // the sweep, where the slots' partials are combined across lanes
+        if (ends) {
+          ++round;
+          if (round < n_rounds) {
+            ridx += r_step * U;
+          } else {
+            in_sweep = false;
+            const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
+            if (k0 <= VR_MIN) racc0 = red_finalize<SCHED>(racc0, k0, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
+            if (k1 <= VR_MIN) racc1 = red_finalize<SCHED>(racc1, k1, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
+          }
+        }
+
         // valid counts of the round's slabs
-        if (op == VOP_SWEEP || op == VOP_ENDSWEEP) {
+        if (op == VOP_SWEEP || ends) {
           if (in_sweep) {
             nvp = 0;
             FOR_U {

@@ -680,6 +680,7 @@ class Compiler {
   // emission helpers
   void Emit(uint32_t op, uint32_t sub, uint32_t kind, uint32_t rnd, uint32_t a, uint32_t imm) {
     uint64_t w = VI_MAKE(op, sub, kind, rnd, a, imm);
+    if (op == VOP_ENDSWEEP) w |= VI_ENDS;
     if (!cube_mode_) {
       const bool mem = op == VOP_ST || (op >= VOP_SRC_BASE && kind == VK_MEM);
       if (mem) {
@@ -699,6 +700,8 @@ class Compiler {
     code_.push_back(w);
   }
   void DropCastBeforeStore(const uint32_t *mem_dtypes);
+  void FuseSweepInstructions();
+  void MarkUniformRuns();
   int last_mem_ = -1;         // memory operand of the last memory instruction emitted in this round, or -1
   int u_ = 2;                 // slabs per lane per instruction of the program being compiled
   bool uniform_emit_ = false; // the value being computed is the same in every element of a lane's accumulator
@@ -1662,12 +1665,126 @@ void Compiler::DropCastBeforeStore(const uint32_t *mem_dtypes) {
   code_.swap(out);
 }
 
+// The interpreter pays a fixed price per instruction, so the short bodies of sweeps are tightened:
+//  * sum(x) and sum(x * x) of one value (mean and variance in one pass): the multiply joins the second reduce;
+//  * two float binaries in a row with S-register operands (x * scale + shift) become one chained instruction;
+//  * the VOP_ENDSWEEP behind a store or a reduce becomes a flag of that instruction.
+// Every fused form computes what the separate instructions compute, rounding by rounding.
+void Compiler::FuseSweepInstructions() {
+  auto defines_acc = [](uint32_t op) {
+    return op == VOP_LD || op == VOP_LDR || op == VOP_LDS || op == VOP_LDI || op == VOP_FIN || op == VOP_END;
+  };
+  std::vector<uint64_t> out;
+  out.reserve(code_.size());
+  size_t sweep_first = 0;  // index in code_ of the first instruction of the sweep being copied
+  for (size_t i = 0; i < code_.size(); ++i) {
+    const uint64_t w = code_[i];
+    const uint32_t lo = static_cast<uint32_t>(w);
+    if (VI_OP(w) == VOP_SWEEP) sweep_first = i + 1;
+    // Mul acc, acc ; reduce_sum rB, acc ; endsweep   (acc dead afterwards)  ->  reduce_sum.square rB, acc
+    if (VI_OP(w) == VOP_BINF && (VI_SUB(w) & 0x3fu) == VB_MUL && VI_KIND(w) == VK_ACC && VI_RND(w) == VRND_NONE &&
+        !(lo & VI_UNIFORM) && i + 2 < code_.size() && VI_OP(code_[i + 1]) == VOP_RED && VI_SUB(code_[i + 1]) == VR_SUM &&
+        VI_OP(code_[i + 2]) == VOP_ENDSWEEP && i + 3 < code_.size() && defines_acc(VI_OP(code_[i + 3])) &&
+        sweep_first < code_.size() && defines_acc(VI_OP(code_[sweep_first])) && sweep_first <= i) {
+      out.push_back(code_[i + 1] | (static_cast<uint64_t>(VRF_SQUARE) << 8));
+      ++i;
+      continue;
+    }
+    // two S-register float binaries in a row
+    if (VI_OP(w) == VOP_BINF && VI_KIND(w) == VK_SREG && !(lo & VI_UNIFORM) && i + 1 < code_.size()) {
+      const uint64_t n = code_[i + 1];
+      if (VI_OP(n) == VOP_BINF && VI_KIND(n) == VK_SREG && !(static_cast<uint32_t>(n) & VI_UNIFORM)) {
+        const uint32_t second = (VI_SUB(n) & 0x3fu) | (VI_A(n) << 8) | (VI_RND(n) << 16);
+        out.push_back(VI_MAKE(VOP_BINF, VI_SUB(w), VK_SREG2, VI_RND(w), VI_A(w), second));
+        ++i;
+        continue;
+      }
+    }
+    out.push_back(w);
+  }
+  // store / reduce ; endsweep  ->  one instruction that also closes the round; a sweep with nothing in it goes
+  code_.clear();
+  for (size_t i = 0; i < out.size(); ++i) {
+    uint64_t w = out[i];
+    if (VI_OP(w) == VOP_SWEEP && (VI_IMM(w) & 0xffu) == (VR_NONE | (VR_NONE << 4)) && i + 1 < out.size() &&
+        VI_OP(out[i + 1]) == VOP_ENDSWEEP) {
+      ++i;
+      continue;
+    }
+    if (i + 1 < out.size() && VI_OP(out[i + 1]) == VOP_ENDSWEEP) {
+      if (VI_OP(w) == VOP_ST) {
+        code_.push_back(w | VI_ENDS);
+        ++i;
+        continue;
+      }
+      if (VI_OP(w) == VOP_RED) {
+        code_.push_back(w | VI_ENDS);
+        ++i;
+        continue;
+      }
+    }
+    code_.push_back(w);
+  }
+}
+
+// Between sweeps a program computes per-output values (a mean, a scale): the same in every lane of the team
+// that owns the output. When the team is the whole workgroup, such a run is executed by one wave, which hands
+// the S registers and the accumulator to the others (VOP_UNI_BEGIN / VOP_UNI_END); sixteen waves interpreting
+// the same twenty scalar instructions cost more than the two barriers.
+void Compiler::MarkUniformRuns() {
+  if ((hdr_.sched & VS_KIND_MASK) != VS_REDX || !hdr_.team_is_block) return;
+  auto bcast_load = [&](uint64_t w) {
+    return VI_OP(w) == VOP_LD && VI_KIND(w) == VK_MEM && !(mems_[VI_A(w)].flags & VMF_VEC);
+  };
+  auto starts = [&](uint64_t w) {
+    const uint32_t op = VI_OP(w);
+    return op == VOP_FIN || op == VOP_LDS || op == VOP_LDI || bcast_load(w);
+  };
+  auto inside = [&](uint64_t w) {
+    const uint32_t op = VI_OP(w);
+    if (starts(w) || op == VOP_STS) return true;
+    const bool arith = op == VOP_UN || op == VOP_CAST || op == VOP_BINF || op == VOP_BINI || op == VOP_CMP;
+    return arith && (static_cast<uint32_t>(w) & VI_UNIFORM) != 0;
+  };
+  std::vector<uint64_t> out;
+  out.reserve(code_.size() + 8);
+  bool in_sweep = false;
+  for (size_t i = 0; i < code_.size();) {
+    const uint64_t w = code_[i];
+    const uint32_t op = VI_OP(w);
+    if (op == VOP_SWEEP) in_sweep = true;
+    if (static_cast<uint32_t>(w) & VI_ENDS) {
+      in_sweep = false;
+    }
+    if (!in_sweep && starts(w)) {
+      size_t j = i;
+      while (j < code_.size() && inside(code_[j])) ++j;
+      if (j - i >= 4) {
+        out.push_back(VI_MAKE(VOP_UNI_BEGIN, 0, 0, 0, 0, static_cast<uint32_t>(j - i + 1)));
+        out.insert(out.end(), code_.begin() + i, code_.begin() + j);
+        out.push_back(VI_MAKE(VOP_UNI_END, 0, 0, 0, 0, 0));
+        i = j;
+        continue;
+      }
+    }
+    out.push_back(w);
+    ++i;
+  }
+  code_.swap(out);
+}
+
 void Compiler::FinishProgram() {
   {
     uint32_t dts[DVM_VEC_MAXMEM];
     for (int i = 0; i < n_mem_; ++i) dts[i] = mems_[i].dtype;
     DropCastBeforeStore(dts);
   }
+  // tuning switches: DVM_VEC_FUSE=0 keeps the instruction stream as emitted, DVM_VEC_UNIRUN=0 lets every wave
+  // execute the per-team runs
+  static const bool fuse = !(std::getenv("DVM_VEC_FUSE") != nullptr && std::getenv("DVM_VEC_FUSE")[0] == '0');
+  static const bool unirun = !(std::getenv("DVM_VEC_UNIRUN") != nullptr && std::getenv("DVM_VEC_UNIRUN")[0] == '0');
+  if (fuse && (hdr_.sched & VS_KIND_MASK) != VS_POINTWISE) FuseSweepInstructions();
+  if (unirun) MarkUniformRuns();
   hdr_.n_mem = n_mem_;
   hdr_.n_code = static_cast<uint32_t>(code_.size());
   hdr_.mem_off = sizeof(VVecHeader) / 8;

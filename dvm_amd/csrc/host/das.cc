@@ -126,20 +126,37 @@ std::string &VKernel::DisAssemble() {
           }
           case VOP_STR: os << "mov v" << VI_A(w) << "." << kFmt[sub & 3] << ", acc"; break;
           case VOP_STS: os << "mov s" << VI_A(w) << ", acc"; break;
-          case VOP_ST: os << "store." << kMemTypes[mem_dtype(VI_A(w))] << " m" << VI_A(w) << ", acc"; break;
+          case VOP_ST:
+            os << "store." << kMemTypes[mem_dtype(VI_A(w))] << " m" << VI_A(w) << ", acc";
+            if (static_cast<uint32_t>(w) & VI_ENDS) os << "  ; endsweep";
+            break;
           case VOP_UN: os << kUn[sub] << "." << (sub == VU_IABS ? "int32" : kRnd[VI_RND(w)]) << " acc"; break;
           case VOP_CAST: {
             static const char *names[] = {"cast.f2i", "cast.i2f", "cast.round", "cast.f2b"};
             os << names[sub] << "." << kRnd[VI_RND(w)] << " acc";
             break;
           }
-          case VOP_RED: os << "reduce_" << kRed[sub] << " r" << VI_A(w) << ", acc"; break;
+          case VOP_RED:
+            os << "reduce_" << kRed[sub & 0xf] << ((sub & VRF_SQUARE) ? ".square" : "") << " r" << VI_A(w) << ", acc";
+            if (static_cast<uint32_t>(w) & VI_ENDS) os << "  ; endsweep";
+            break;
           case VOP_SWEEP: os << "sweep slots=" << kRed[(VI_IMM(w) & 0xf) < 3 ? (VI_IMM(w) & 0xf) : 0]
                              << ((VI_IMM(w) & 0xf) < 3 ? "" : "(none)"); break;
           case VOP_ENDSWEEP: os << "endsweep"; break;
           case VOP_FIN: os << "mov acc, r" << VI_A(w); break;
+          case VOP_UNI_BEGIN: os << "uniform run, " << (VI_IMM(w) - 1) << " instructions: first wave only when the team is the workgroup"; break;
+          case VOP_UNI_END: os << "end of uniform run"; break;
           case VOP_LD: os << "load." << kMemTypes[mem_dtype(VI_A(w))] << " acc, m" << VI_A(w); break;
-          case VOP_BINF: os << kBinF[sub & 0x3f] << "." << kRnd[VI_RND(w)] << " acc, "; PrintSrc(os, w); break;
+          case VOP_BINF:
+            if (VI_KIND(w) == VK_SREG2) {  // two chained operations
+              const uint32_t second = VI_IMM(w);
+              os << kBinF[sub & 0x3f] << "." << kRnd[VI_RND(w)] << " acc, s" << VI_A(w) << "  ; then " << kBinF[second & 0x3f] << "."
+                 << kRnd[(second >> 16) & 3] << " acc, s" << ((second >> 8) & 0xff);
+              break;
+            }
+            os << kBinF[sub & 0x3f] << "." << kRnd[VI_RND(w)] << " acc, ";
+            PrintSrc(os, w);
+            break;
           case VOP_BINI: os << kBinI[sub & 0x3f] << ".int32 acc, "; PrintSrc(os, w); break;
           case VOP_CMP: os << "Cmp" << kCmp[sub & 7] << "." << ((sub & VCMP_INT) ? "int32" : "fp32") << " acc, "; PrintSrc(os, w); break;
           case VOP_MSK: os << "mask "; PrintSrc(os, w); break;

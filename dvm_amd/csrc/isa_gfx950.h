@@ -71,6 +71,11 @@ enum {
   VOP_SWEEP = 10,    // start of a loop over the reduce index space; imm = slot kinds, 4 bits each
   VOP_ENDSWEEP = 11, // next round, or fall through and combine the slots across lanes
   VOP_FIN = 12,      // acc = combined slot[a]
+  VOP_UNI_BEGIN = 13,// start of a run whose values are the same in every lane of a team; imm = distance in
+                     // instructions to the matching VOP_UNI_END. When the team is the whole workgroup only its
+                     // first wave executes the run, the others jump to the end
+  VOP_UNI_END = 14,  // end of the run: the first wave's S registers and accumulator value are handed to the
+                     // other waves through local memory
   VOP_SRC_BASE = 16,
   VOP_LD = 16,       // acc = mem[a]             (kind is always VK_MEM)
   VOP_BINF = 17,     // acc = acc (sub = VB_*) src, float class
@@ -80,8 +85,10 @@ enum {
   VOP_MOVM = 21,     // acc = mask ? src : acc
 };
 
-// source kinds (bits 16..19)
-enum { VK_REG = 0, VK_IMM = 1, VK_MEM = 2, VK_ACC = 3, VK_SREG = 4 };
+// source kinds (bits 16..19). VK_SREG2 (VOP_BINF only) chains two float binaries with S-register operands in
+// one instruction: acc = (acc (sub) sreg[a]) (sub2) sreg[a2], each result rounded by its own rnd field; the
+// second operation sits in the immediate: [7:0] sub2, [15:8] a2, [17:16] rnd2.
+enum { VK_REG = 0, VK_IMM = 1, VK_MEM = 2, VK_ACC = 3, VK_SREG = 4, VK_SREG2 = 5 };
 // result rounding (bits 20..21): value is rounded to that format and widened back
 enum { VRND_NONE = 0, VRND_F16 = 1, VRND_BF16 = 2 };
 // V register storage formats
@@ -106,22 +113,27 @@ enum {
   VC_RND = 2,    // float -> float rounded per rnd field (f32->f16, f32->bf16)
   VC_F2B = 3,    // float -> bool container (x != 0 ? 1.0 : 0.0)
 };
-// reduce kinds
+// reduce kinds (low 4 bits of VOP_RED's sub field), and two modifiers of VOP_RED
 enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
+#define VRF_SQUARE 0x10u  // acc = acc * acc (the fp32 product) first; the multiply of a sum of squares rides in the reduce
 
 // instruction word:
-//   [7:0] opcode  [15:8] sub  [19:16] src kind  [21:20] rnd  [22] VI_UNIFORM  [23] VI_SAME_OFFS
+//   [6:0] opcode  [7] VI_ENDS  [15:8] sub  [19:16] src kind  [21:20] rnd  [22] VI_UNIFORM  [23] VI_SAME_OFFS
 //   [31:24] a (register / memory operand / slot index)   [63:32] imm32
 // VI_UNIFORM (vector VM, arithmetic without a memory or V-register operand): every element of the lane's
 // accumulator holds the same value, the instruction may compute one and copy it.
 // VI_SAME_OFFS (vector VM, memory instructions): the operand has the strides of the previous memory
 // instruction of the same round, whose element offsets are reused.
+// VI_ENDS (top bit of the opcode byte; set on every VOP_ENDSWEEP, and on a store or reduce that took over the
+// VOP_ENDSWEEP behind it): the instruction closes the round of its sweep. One bit, so that the decoder finds the
+// next pc without comparing opcodes.
+#define VI_ENDS 0x80u
 #define VI_UNIFORM (1u << 22)
 #define VI_SAME_OFFS (1u << 23)
 #define VI_MAKE(op, sub, kind, rnd, a, imm)                                                     \
   ((uint64_t)(op) | ((uint64_t)(sub) << 8) | ((uint64_t)(kind) << 16) | ((uint64_t)(rnd) << 20) | \
    ((uint64_t)(a) << 24) | ((uint64_t)(uint32_t)(imm) << 32))
-#define VI_OP(w) ((uint32_t)(w) & 0xffu)
+#define VI_OP(w) ((uint32_t)(w) & 0x7fu)
 #define VI_SUB(w) (((uint32_t)(w) >> 8) & 0xffu)
 #define VI_KIND(w) (((uint32_t)(w) >> 16) & 0xfu)
 #define VI_RND(w) (((uint32_t)(w) >> 20) & 0x3u)
