@@ -2,6 +2,7 @@
 // runtime wrappers the host emitter needs (see include/dvm_hip.h for the
 // reference interfaces each entry point replaces).
 #include <hip/hip_runtime.h>
+#include <algorithm>
 #include <stdint.h>
 #include <string.h>
 
@@ -152,11 +153,18 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
     const bool wide = (h->sched & VS_WIDE) != 0;
     if (wide && threads > 512) return static_cast<int>(hipErrorInvalidValue);
     {
-      // local memory the interpreter will touch: reduce scratch and V registers
+      // local memory the interpreter will touch: reduce scratch, V registers, rounds parked by a load
       const uint64_t u = wide ? DVM_VEC_U_WIDE : 2;
-      if (lds_bytes < static_cast<uint64_t>(threads) * 8 + static_cast<uint64_t>(h->n_vslot) * u * 16 * threads) {
-        return static_cast<int>(hipErrorInvalidValue);
+      uint64_t need = static_cast<uint64_t>(threads) * 8 + static_cast<uint64_t>(h->n_vslot) * u * 16 * threads;
+      uint64_t parked = 0;
+      for (uint64_t i = h->code_off; i < code_end; ++i) {
+        if (VI_OP(p.w[i]) == VOP_LD && (static_cast<uint32_t>(p.w[i]) & (VI_LD_KEEP_WR | VI_LD_KEEP_RD))) {
+          if (wide) return static_cast<int>(hipErrorInvalidValue);
+          parked = std::max<uint64_t>(parked, VI_IMM(p.w[i]));
+        }
       }
+      need += parked * threads * u * 32;
+      if (lds_bytes < need) return static_cast<int>(hipErrorInvalidValue);
     }
     switch (h->sched & VS_KIND_MASK) {
       case VS_POINTWISE:

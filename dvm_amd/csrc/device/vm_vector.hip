@@ -279,6 +279,15 @@ __device__ __forceinline__ void mem_load(const VMemDesc &m, const Offs &off, uin
   const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
   if (fast && wave_all(nvp == kAllFull)) {
     mem_load_wide(m, off, out);
+  } else if (!(m.flags & VMF_VEC) && (m.dtype == VDT_F32 || m.dtype == VDT_I32)) {
+    // one 32-bit element per slab, replicated (an operand broadcast along the innermost axis: a per-channel
+    // scale, a per-row statistic); lanes without a valid slab read the base element and get zero, like the
+    // guarded path. Inline: the out-of-line path saves registers to scratch memory around the call.
+    FOR_U {
+      const bool ok = ((nvp >> (4 * u)) & 0xfu) != 0u;
+      const float v = reinterpret_cast<const DVM_GLOBAL float *>(m.addr)[ok ? off.v[u] : 0u];
+      out.v[u] = ok ? v : 0.0f;
+    }
   } else {
     out = mem_load_slow(m.addr, m.dtype, m.flags, off, nvp);
   }
@@ -403,7 +412,7 @@ __device__ __forceinline__ void red_accumulate(RedAcc<SCHED> &r, uint32_t kind, 
 // Combines one slot's partials across the lanes that share an output; every
 // one of those lanes ends up with the result.
 template <int SCHED>
-__device__ __attribute__((noinline)) RedAcc<SCHED> red_finalize(RedAcc<SCHED> r, uint32_t rk, uint32_t tlog, bool team_is_block,
+__device__ __forceinline__ RedAcc<SCHED> red_finalize(RedAcc<SCHED> r, uint32_t rk, uint32_t tlog, bool team_is_block,
                                                                 uint32_t tid, uint32_t nthreads, uint32_t k_local,
                                                                 uint32_t r_local, double *scratch) {
   rk = uni(rk);
@@ -417,7 +426,7 @@ __device__ __attribute__((noinline)) RedAcc<SCHED> red_finalize(RedAcc<SCHED> r,
     if (team_is_block) {
       const uint32_t nw = (nthreads + 63u) >> 6;
       __syncthreads();
-      if ((tid & 63u) == 0) scratch[tid >> 6] = t;
+      scratch[tid >> 6] = t;  // every lane of a wave holds the wave's value: identical writes, no per-lane branch
       __syncthreads();
       t = scratch[0];
       for (uint32_t j = 1; j < nw; ++j) t = red_combine(rk, t, scratch[j]);
@@ -675,6 +684,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   // per-team runs (VOP_UNI_BEGIN .. VOP_UNI_END) are computed by the first wave when the team is the workgroup
   const uint32_t skips_runs = (SCHED == VS_REDX && team_is_block && uni(tid >> 6) != 0u) ? 1u : 0u;
   vf4 *planes = reinterpret_cast<vf4 *>(lds + nthreads);  // first nthreads doubles: reduce scratch
+  vf4 *keep_lds = planes + h.n_vslot * U * nthreads;      // behind the V registers: rounds parked by VI_LD_KEEP_WR
 
   // lane -> (kept local index, reduce local index)
   uint32_t k_local, r_local, k_per_wg, r_step;
@@ -724,6 +734,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     bool in_sweep = false;
     uint32_t nvp = nvp_out;
     uint32_t round = 0, sweep_pc = 0, slot_kinds = 0;
+    bool sweep_rev = false;   // the sweep walks its rounds last to first (VSW_REVERSE)
     uint32_t ridx = r_local;  // reduce-space index of slab 0 in the current round
     Offs last_off;            // element offsets of the last memory instruction (VI_SAME_OFFS reuses them)
     FOR_U last_off.v[u] = 0;
@@ -847,6 +858,26 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             last_off = off;
           }
           if (op == VOP_LD) {
+            if constexpr (SCHED == VS_REDX) {
+              // rounds parked in local memory by the load that opened an earlier sweep over this operand
+              const uint32_t lr = sweep_rev ? n_rounds - 1u - round : round;
+              const bool parked = in_sweep && lr < imm;
+              if (parked && (w0 & VI_LD_KEEP_RD)) {
+                FOR_U {
+                  const vf4 lo = keep_lds[((lr * U + u) * 2u) * nthreads + tid], hi = keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid];
+                  acc.v[u] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+                }
+                continue;
+              }
+              mem_load(m, off, nvp, acc);
+              if (parked && (w0 & VI_LD_KEEP_WR)) {
+                FOR_U {
+                  keep_lds[((lr * U + u) * 2u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 0, 1, 2, 3);
+                  keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 4, 5, 6, 7);
+                }
+              }
+              continue;
+            }
             mem_load(m, off, nvp, acc);
             continue;
           }
@@ -950,7 +981,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               // what the run produced lives in the first wave's S registers and accumulator: pass it on
               float *box = reinterpret_cast<float *>(lds);  // the reduce scratch is idle between sweeps
               __syncthreads();
-              if (tid == 0) {
+              if (skips_runs == 0u) {  // the first wave; its lanes hold identical values
                 *reinterpret_cast<vf4 *>(box) = vf4{sr.s0, sr.s1, sr.s2, sr.s3};
                 *reinterpret_cast<vf4 *>(box + 4) = vf4{sr.s4, sr.s5, sr.s6, sr.s7};
                 box[8] = acc.v[0][0];
@@ -1051,7 +1082,8 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             slot_kinds = imm;
             red_init<SCHED>(racc0, slot_kinds & 0xfu);
             red_init<SCHED>(racc1, (slot_kinds >> 4) & 0xfu);
-            ridx = r_local;
+            sweep_rev = SCHED == VS_REDX && (sub & VSW_REVERSE) != 0;
+            ridx = r_local + (sweep_rev ? (n_rounds - 1u) * r_step * U : 0u);
             break;
           }
           case VOP_FIN: {
@@ -1074,7 +1106,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
         if (ends) {
           ++round;
           if (round < n_rounds) {
-            ridx += r_step * U;
+            ridx = sweep_rev ? ridx - r_step * U : ridx + r_step * U;
           } else {
             in_sweep = false;
             const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;

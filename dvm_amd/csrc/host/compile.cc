@@ -702,6 +702,7 @@ class Compiler {
   void DropCastBeforeStore(const uint32_t *mem_dtypes);
   void FuseSweepInstructions();
   void MarkUniformRuns();
+  void PlanRereads();
   int last_mem_ = -1;         // memory operand of the last memory instruction emitted in this round, or -1
   int u_ = 2;                 // slabs per lane per instruction of the program being compiled
   bool uniform_emit_ = false; // the value being computed is the same in every element of a lane's accumulator
@@ -1773,6 +1774,58 @@ void Compiler::MarkUniformRuns() {
   code_.swap(out);
 }
 
+// A reduce with consumers reads its input twice: once for the statistics, once to apply them. What the
+// second sweep does not have to fetch again from HBM:
+//  * the first rounds of the first sweep stay in the workgroup's spare local memory (VI_LD_KEEP_WR/RD);
+//  * a later sweep without reduces of its own runs last round first (VSW_REVERSE), starting with the data the
+//    L2 cache still holds from the end of the sweep before, and ending with the parked rounds.
+// Called with the blob filled in and lds_bytes set; edits the instruction words in the blob.
+void Compiler::PlanRereads() {
+  // tuning switch DVM_VEC_REREAD: 0 off, 2 parked rounds only, 3 reversed sweeps only (default: both)
+  static const char mode = std::getenv("DVM_VEC_REREAD") != nullptr ? std::getenv("DVM_VEC_REREAD")[0] : '1';
+  const bool on = mode != '0', park = mode != '3', reverse = mode != '2';
+  if (!on || (hdr_.sched & VS_KIND_MASK) != VS_REDX || (hdr_.sched & VS_WIDE)) return;
+  uint64_t *cw = prog_->blob.w + hdr_.code_off;
+  const size_t n = code_.size();
+  const uint32_t team = hdr_.team_is_block ? prog_->threads : (1u << hdr_.team_log2);
+  const uint32_t per_round = team * u_;
+  const uint32_t n_rounds = (hdr_.n_ridx + per_round - 1) / per_round;
+  if (n_rounds < 2) return;
+  // sweeps: position of the VOP_SWEEP word and of the load that opens it (or -1)
+  struct Sw { size_t at; int ld; bool reduces; };
+  std::vector<Sw> sweeps;
+  for (size_t i = 0; i < n; ++i) {
+    if (VI_OP(cw[i]) != VOP_SWEEP) continue;
+    Sw sw{i, -1, (VI_IMM(cw[i]) & 0xffu) != (VR_NONE | (VR_NONE << 4))};
+    if (i + 1 < n && VI_OP(cw[i + 1]) == VOP_LD && VI_KIND(cw[i + 1]) == VK_MEM && (mems_[VI_A(cw[i + 1])].flags & VMF_VEC)) {
+      sw.ld = static_cast<int>(i + 1);
+    }
+    sweeps.push_back(sw);
+  }
+  for (size_t k = 1; k < sweeps.size(); ++k) {
+    if (reverse && !sweeps[k].reduces) cw[sweeps[k].at] |= static_cast<uint64_t>(VSW_REVERSE) << 8;
+  }
+  // park rounds of the first pair of sweeps that open with a load of the same operand
+  if (!park) return;
+  for (size_t a = 0; a + 1 < sweeps.size(); ++a) {
+    if (sweeps[a].ld < 0) continue;
+    for (size_t b = a + 1; b < sweeps.size(); ++b) {
+      if (sweeps[b].ld < 0 || VI_A(cw[sweeps[b].ld]) != VI_A(cw[sweeps[a].ld])) continue;
+      // local memory left to this workgroup when as many workgroups as the registers allow share the CU
+      const uint32_t per_cu = 1024 / std::max<uint32_t>(prog_->threads, 64);
+      const uint32_t budget = std::min<uint32_t>(160 * 1024, g_system.lds_per_wg) / per_cu;
+      const uint32_t fixed = prog_->lds_bytes + DVM_PARAM_BYTES + 1024;
+      const uint32_t per_keep = prog_->threads * u_ * 32;
+      if (budget <= fixed + per_keep) return;
+      const uint32_t rounds = std::min<uint32_t>(n_rounds, (budget - fixed) / per_keep);
+      cw[sweeps[a].ld] |= VI_LD_KEEP_WR | (static_cast<uint64_t>(rounds) << 32);
+      cw[sweeps[b].ld] |= VI_LD_KEEP_RD | (static_cast<uint64_t>(rounds) << 32);
+      prog_->lds_bytes += rounds * per_keep;
+      return;
+    }
+  }
+}
+
 void Compiler::FinishProgram() {
   {
     uint32_t dts[DVM_VEC_MAXMEM];
@@ -1796,6 +1849,7 @@ void Compiler::FinishProgram() {
   std::memcpy(prog_->blob.w + hdr_.mem_off, mems_, sizeof(VMemDesc) * n_mem_);
   std::memcpy(prog_->blob.w + hdr_.code_off, code_.data(), 8 * code_.size());
   prog_->lds_bytes = prog_->threads * 8 + static_cast<uint32_t>(max_vslot_) * u_ * 16 * prog_->threads;
+  PlanRereads();
   uint64_t gt = (static_cast<uint64_t>(std::min<uint32_t>(hdr_.n_items, g_system.core_num * 4)) << 32) | prog_->threads;
   if (g_system.HasDevice()) {
     gt = g_system.Api().select_block_thread(hdr_.sched, hdr_.n_items, prog_->threads, prog_->lds_bytes);

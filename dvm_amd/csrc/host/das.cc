@@ -140,13 +140,17 @@ std::string &VKernel::DisAssemble() {
             os << "reduce_" << kRed[sub & 0xf] << ((sub & VRF_SQUARE) ? ".square" : "") << " r" << VI_A(w) << ", acc";
             if (static_cast<uint32_t>(w) & VI_ENDS) os << "  ; endsweep";
             break;
-          case VOP_SWEEP: os << "sweep slots=" << kRed[(VI_IMM(w) & 0xf) < 3 ? (VI_IMM(w) & 0xf) : 0]
+          case VOP_SWEEP: os << ((sub & VSW_REVERSE) ? "sweep (last round first) slots=" : "sweep slots=") << kRed[(VI_IMM(w) & 0xf) < 3 ? (VI_IMM(w) & 0xf) : 0]
                              << ((VI_IMM(w) & 0xf) < 3 ? "" : "(none)"); break;
           case VOP_ENDSWEEP: os << "endsweep"; break;
           case VOP_FIN: os << "mov acc, r" << VI_A(w); break;
           case VOP_UNI_BEGIN: os << "uniform run, " << (VI_IMM(w) - 1) << " instructions: first wave only when the team is the workgroup"; break;
           case VOP_UNI_END: os << "end of uniform run"; break;
-          case VOP_LD: os << "load." << kMemTypes[mem_dtype(VI_A(w))] << " acc, m" << VI_A(w); break;
+          case VOP_LD:
+            os << "load." << kMemTypes[mem_dtype(VI_A(w))] << " acc, m" << VI_A(w);
+            if (static_cast<uint32_t>(w) & VI_LD_KEEP_WR) os << "  ; parks its first " << VI_IMM(w) << " rounds in local memory";
+            if (static_cast<uint32_t>(w) & VI_LD_KEEP_RD) os << "  ; takes its first " << VI_IMM(w) << " rounds from local memory";
+            break;
           case VOP_BINF:
             if (VI_KIND(w) == VK_SREG2) {  // two chained operations
               const uint32_t second = VI_IMM(w);

@@ -124,6 +124,15 @@ enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 // accumulator holds the same value, the instruction may compute one and copy it.
 // VI_SAME_OFFS (vector VM, memory instructions): the operand has the strides of the previous memory
 // instruction of the same round, whose element offsets are reused.
+// Re-reading less in the second sweep over a tensor (vector VM, schedule that reduces the innermost axis):
+//  VI_LD_KEEP_WR / VI_LD_KEEP_RD (VOP_LD that opens a sweep; the rnd field is free there, imm = number of rounds):
+//    the first load parks the slabs of its first imm rounds in local memory, the load that opens a later sweep
+//    over the same operand takes those rounds from there instead of from memory;
+//  VSW_REVERSE (sub field of VOP_SWEEP): the sweep walks its rounds last to first, so that it starts with
+//    what the sweep before it read last (still in the L2 cache) and ends with the parked rounds.
+#define VI_LD_KEEP_WR (1u << 20)
+#define VI_LD_KEEP_RD (1u << 21)
+#define VSW_REVERSE 1u
 // VI_ENDS (top bit of the opcode byte; set on every VOP_ENDSWEEP, and on a store or reduce that took over the
 // VOP_ENDSWEEP behind it): the instruction closes the round of its sweep. One bit, so that the decoder finds the
 // next pc without comparing opcodes.
