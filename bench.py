@@ -21,9 +21,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 # HBM bytes one launch of the headline kernel moves, from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of
 # `bench.py --traffic-probe`, each scaled by the same counter's reading for a plain copy of known size
-# (207.2 MB fetched + 118.4 MB written). A counter cannot be read from inside this script: the figure is
+# (170.4 MB fetched + 118.6 MB written). A counter cannot be read from inside this script: the figure is
 # re-measured and updated whenever the kernel's schedule changes.
-HEADLINE_TRAFFIC_BYTES = 325.7e6
+HEADLINE_TRAFFIC_BYTES = 289.0e6
 METRIC = "fused-op HBM GB/s (% roofline) + matmul TFLOPS (% MFMA peak); JIT us/shape"
 
 
