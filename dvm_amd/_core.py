@@ -425,6 +425,13 @@ class PyKernel(Kernel):
 
     @staticmethod
     def set_deterministic(enable):
+        """Config::SetDeterm of the reference picks ordered reduces over atomics. Reduces here never use atomics
+        (one team of lanes owns an output and combines in a fixed order), so both settings give the same bits."""
+        pass
+
+    def tile(self, start, end, num, factor=0):
+        """Manual tiling of the reference's tile model (RtKernelPy::Tile, src/pybind_api.cc:1093). The gfx950
+        schedules have no user-visible tiles; the hint is accepted and ignored."""
         pass
 
 

@@ -316,6 +316,7 @@ class Compiler {
     mode_ = mode;
     conservative_ = mode >= 2;
     area_.assign(n_, -1);
+    level_.assign(n_, 0);
     live_.assign(n_, 0);
     mat_.assign(n_, 0);
     ws_slot_.assign(n_, -1);
@@ -342,7 +343,7 @@ class Compiler {
  private:
   VKernel *k_;
   int n_;
-  std::vector<int> area_, ws_slot_, store_of_;
+  std::vector<int> area_, ws_slot_, store_of_, level_;
   std::vector<char> live_, mat_;
   int n_areas_ = 0;
   struct AreaInfo {
@@ -353,6 +354,7 @@ class Compiler {
     int64_t dom[kMaxRank];
     const NDObject *cube_op = nullptr;
     int attn = -1;  // index into attn_groups_ when the sub-kernel is one fused attention
+    int red_at_level[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // reduces per sweep: the interpreter has two reduce slots per sweep
     int stage = 0;  // the caller's group (parallel / sequence kernels); operators of different groups never share a launch
     int n_ops = 0;  // operators joined so far (a program has room for about 500 instruction words and 160 nodes)
   };
@@ -433,10 +435,25 @@ class Compiler {
     return true;
   }
 
+  // Sweep an operator would run in if it joined sub-kernel a: one more than the deepest reduce among the
+  // operators of a it depends on.
+  int LevelIn(int a, const NDObject *o) const {
+    int lvl = 0;
+    for (int j = 0; j < o->nin; ++j) {
+      const NDObject *v = o->in[j];
+      if (v == nullptr || area_[v->id] != a) continue;
+      lvl = std::max(lvl, level_[v->id] + (v->kind == kObjReduce ? 1 : 0));
+    }
+    return lvl;
+  }
+
   bool CanJoin(int a, const NDObject *o) {
     if (a >= static_cast<int>(areas_.size())) return true;  // a fresh sub-kernel
     const AreaInfo &ai = areas_[a];
     if (ai.stage != o->stage) return false;
+    // a store goes where the value it stores is computed (an operator's own output is never a reason to cut)
+    if (o->kind == kObjStore && ai.attn < 0 && !ai.cube && area_[o->in[0]->id] == a) return true;
+    if (o->kind == kObjReduce && LevelIn(a, o) < 8 && ai.red_at_level[LevelIn(a, o)] >= 2) return false;
     if (o->kind == kObjMatMul) return false;
     if (ai.n_ops >= kMaxAreaOps && o->kind != kObjStore) return false;  // long graphs are cut into several launches
     if (ai.attn >= 0) return o->kind == kObjStore && o->in[0] == attn_groups_[ai.attn].m2;
@@ -462,6 +479,8 @@ class Compiler {
     AreaInfo &ai = areas_[a];
     if (ai.n_ops == 0) ai.stage = o->stage;
     ++ai.n_ops;
+    level_[o->id] = LevelIn(a, o);
+    if (o->kind == kObjReduce && level_[o->id] < 8) ++ai.red_at_level[level_[o->id]];
     if (o->kind == kObjMatMul) {
       ai.cube = true;
       ai.cube_op = o;
@@ -750,7 +769,18 @@ void Compiler::BuildNodes(int a) {
     }
     AKind kind = AK_OP;
     if (o->kind == kObjCopy || o->kind == kObjBroadcast || o->kind == kObjReshape) kind = AK_ALIAS;
-    if (o->kind == kObjReduce) kind = AK_REDUCE;
+    if (o->kind == kObjReduce) {
+      // a reduce over axes of extent 1 only (tests/ut/test_reduce.py:91: [120,20,1] over axis 2) computes
+      // nothing: sum, max and min of one element are the element; it is a squeeze of its input
+      const NDObject *x = o->in[0];
+      bool nothing = true;
+      for (size_t j = 0; j < o->aux_ref->size; ++j) {
+        int64_t d = o->aux_ref->data[j];
+        if (d < 0) d += x->rank();
+        if (x->dim(static_cast<int>(d)) != 1) nothing = false;
+      }
+      kind = nothing ? AK_ALIAS : AK_REDUCE;
+    }
     if (o->kind == kObjStore) kind = AK_OUT;
     if (o->kind == kObjCast) {
       // widening conversions do not change the register value
@@ -820,7 +850,7 @@ void Compiler::UnifyAxes() {
         break;
       }
       case AK_ALIAS:
-        if (n.op->kind == kObjReshape) {
+        if (n.op->kind == kObjReshape || n.op->kind == kObjReduce) {  // dims of extent 1 come and go, the rest keep their order
           const ANode &x = nodes_[n.in[0]];
           int a = 0, b = 0;
           while (true) {

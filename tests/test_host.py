@@ -306,3 +306,26 @@ def test_store_as_operand_reads_the_stored_value():
     t.codegen()
     assert t.num_launches() == 2
     assert t.workspace_bytes() == 0  # the second group reads the first group's output buffer
+
+
+def test_three_sibling_reduces_take_two_launches():
+    # tests/ut/test_reduce.py:261-276: sum, max and min of one tensor; a sweep has two reduce slots
+    t = Tester("vector", run_mode="das")
+    x = t.load(np.zeros([128, 9, 257], np.float32))
+    outs = [t.sum(x, (0, 2), False), t.max(x, (0, 2), False), t.min(x, (0, 2), False)]
+    for o in outs:
+        t.store_expect(o, 0)
+    t.codegen()
+    assert t.num_launches() == 2
+    assert t.workspace_bytes() == 0  # every store sits in the launch that computes its value
+
+
+def test_reduce_over_axes_of_extent_one_is_a_squeeze():
+    # tests/ut/test_reduce.py:91: [120,20,1] over axis 2
+    t = Tester("vector", run_mode="das")
+    x = t.load(np.zeros([120, 20, 1], np.float32))
+    t.store_expect(t.max(x, (2,), True), 0)
+    t.store_expect(t.sum(x, (2,), False), 0)
+    t.codegen()
+    assert t.num_launches() == 1
+    assert "pointwise" in t.das()
