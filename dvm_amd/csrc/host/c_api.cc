@@ -141,6 +141,8 @@ void ParseKernelType(const std::string &s, KernelType *type, uint32_t *flags) {
     *type = kParallel;
   } else if (name == "seq") {
     *type = kSequence;
+  } else if (name == "eager") {
+    *type = kEager;
   } else {
     throw std::runtime_error("DVM EXCEPTION. reason: kernel type '" + name + "' is not supported by the gfx950 backend");
   }
@@ -152,8 +154,10 @@ void ParseKernelType(const std::string &s, KernelType *type, uint32_t *flags) {
     const std::string f = opts.substr(start, end - start);
     if (f == "dyn") {
       *flags |= kDynamic;
-    } else if (f == "uws") {
+    } else if (f == "uws" || f == "unify_ws") {
       *flags |= kUnifyWS;
+    } else if (f == "lazy") {
+      *flags |= kLazyCodeGen;
     } else if (!f.empty()) {
       throw std::runtime_error("DVM EXCEPTION. reason: kernel flag '" + f + "' is not supported by the gfx950 backend");
     }

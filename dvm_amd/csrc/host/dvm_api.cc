@@ -467,6 +467,9 @@ void Kernel::Reset(KernelType type, uint32_t flags) {
     case kSplit:
     case kParallel:
     case kSequence:
+    case kEager:  // operators are appended freely and cut into launches at code generation, exactly like kSplit:
+                  // the reference's incremental cutting (src/xkernel.cc EagerKernel) and lazy code generation
+                  // change when the work happens, not what is computed
       break;
     default:
       kernel_ = nullptr;

@@ -195,7 +195,7 @@ def test_zero_size_shapes_are_idle():
 
 def test_errors_are_runtime_errors_with_the_reference_prefix():
     with pytest.raises(RuntimeError, match="DVM EXCEPTION"):
-        Tester("eager", run_mode="das")
+        Tester("cluster", run_mode="das")
     t = Tester("vector", run_mode="das")
     a = t.load(np.zeros([4, 3], np.float32))
     b = t.load(np.zeros([4, 5], np.float32))

@@ -60,3 +60,40 @@ def run_parity(build, arrays, dtypes=None, ker="vector", eps=None, golden=None, 
             assert np.allclose(out, gi, rtol=e, atol=e, equal_nan=True), (
                 "output %d differs from the NumPy golden beyond %g\n%s" % (i, e, t.das()))
     return outs
+
+
+def run_graph(ker, build, oracle=True, oracle_eps=None, min_launches=None):
+    """build(k) builds a graph on k (the HIP Tester or the CPU oracle, same method names) and returns a list of
+    (store, golden, eps) with golden a NumPy array / scalar or None. Checks the HIP outputs against the oracle's
+    (usual tolerances, or oracle_eps) and against the goldens (eps, or the usual tolerance when None).
+    Returns the Tester."""
+    t = Tester(ker)
+    specs = build(t)
+    refs = None
+    if oracle:
+        o = OracleKernel()
+        refs = [o.output(s[0]) for s in build(o)]
+    t.run()
+    if min_launches is not None:
+        assert t.num_launches() >= min_launches, t.das()
+    for i, (st, gold, eps) in enumerate(specs):
+        out = t.output(st)
+        dt = int(st.dtype())
+        if dt == int(DataType.bfloat16):
+            out = Tester.convert_from_bf16(out)
+        exact = dt in (int(DataType.int32), int(DataType.bool))
+        if refs is not None:
+            ref = refs[i]
+            assert out.shape == ref.shape, "output %d: shape %s vs oracle %s" % (i, out.shape, ref.shape)
+            if exact:
+                assert np.array_equal(out, ref), "output %d differs from the oracle (bit-exact required)\n%s" % (i, t.das())
+            else:
+                e = oracle_eps if oracle_eps is not None else DEFAULT_EPS[dt]
+                assert np.allclose(out.astype(np.float32), ref.astype(np.float32), rtol=e, atol=e, equal_nan=True), (
+                    "output %d differs from the oracle beyond %g\n%s" % (i, e, t.das()))
+        if gold is not None:
+            e = eps if eps is not None else DEFAULT_EPS.get(dt, 0)
+            assert np.allclose(out, gold, rtol=e, atol=e, equal_nan=True), (
+                "output %d differs from the NumPy golden beyond %g: max abs diff %g\n%s"
+                % (i, e, np.nanmax(np.abs(np.asarray(out, np.float64) - np.asarray(gold, np.float64))), t.das()))
+    return t
