@@ -1,0 +1,67 @@
+"""GPU parity: broadcasts, restating the gpu-marked cases of tests/ut/test_broadcast.py of the reference with
+their exact shapes (some of them were regressions of its tiling: very long repeats, unaligned rows, bool and
+bf16 operands). NumPy expectations as there, the CPU oracle as second opinion; integers and bools exact."""
+import numpy as np
+import pytest
+
+from tests.util import run_graph
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dt", [np.float16, np.float32, np.int32])
+def test_broadcast_x_y(dt):  # tests/ut/test_broadcast.py:22-60
+    rng = np.random.default_rng(1)
+    a, b = rng.normal(0, 1, [16, 1]).astype(dt), rng.normal(0, 1, [16, 64]).astype(dt)
+    run_graph("", lambda k: [(k.store(k.broadcast(k.load(a), [16, 2])), np.broadcast_to(a, [16, 2]), 0)])
+    run_graph("", lambda k: [(k.store(k.add(k.broadcast(k.load(a), [16, 64]), k.load(b))), a + b, None)])
+    c = rng.normal(0, 1, [1, 32]).astype(dt)
+    run_graph("", lambda k: [(k.store(k.broadcast(k.load(c), [8, 32])), np.broadcast_to(c, [8, 32]), 0)])
+
+
+@pytest.mark.parametrize("dt", [np.float16, np.float32])
+def test_broadcast_multi(dt):  # :63-77
+    rng = np.random.default_rng(2)
+    a, b = rng.normal(0, 1, [10, 33, 64]).astype(dt), rng.normal(0, 1, [10, 1, 1]).astype(dt)
+
+    def g(k):
+        z = k.broadcast(k.add(k.broadcast(k.load(b), [10, 33, 1]), 0.1), [10, 33, 64])
+        return [(k.store(k.add(k.load(a), z)), a + (b + dt(0.1)), None)]
+    run_graph("", g)
+
+
+def test_broadcast_large_shape():  # :80-91
+    a = np.random.default_rng(3).random([20, 30, 1, 50]).astype(np.float32)
+    run_graph("", lambda k: [(k.store(k.broadcast(k.load(a), [20, 30, 40, 50])), np.broadcast_to(a, [20, 30, 40, 50]), 0)])
+
+
+def test_long_repeats_and_unaligned_rows():  # :109-132, :268-276
+    rng = np.random.default_rng(4)
+    a0 = rng.normal(0, 1, [1, 1]).astype(np.float32)
+    run_graph("", lambda k: [(k.store(k.broadcast(k.load(a0), [184965, 1])), np.broadcast_to(a0, (184965, 1)), 0)])
+    a1 = rng.normal(0, 1, [3, 4, 1]).astype(np.float32)
+    run_graph("", lambda k: [(k.store(k.broadcast(k.load(a1), [3, 4, 5])), np.broadcast_to(a1, (3, 4, 5)), 0)])
+    a2 = rng.normal(0, 1, [555555, 1]).astype(np.float16)
+    run_graph("", lambda k: [(k.store(k.broadcast(k.load(a2), [555555, 16])), np.broadcast_to(a2, [555555, 16]), 0)])
+
+
+def test_broadcast_bf16():  # :135-145
+    a0 = np.random.default_rng(5).normal(0, 1, [30, 40, 1]).astype(np.float32)
+    run_graph("", lambda k: [(k.store(k.broadcast(k.load(a0, "bfloat16"), [30, 40, 5])), np.broadcast_to(a0, (30, 40, 5)), 5e-3)])
+
+
+@pytest.mark.parametrize("scalar", [0.0, 0.2, True])
+def test_fill(scalar):  # :148-164
+    run_graph("", lambda k: [(k.store(k.full(0.2, [2, 64], "float32")), np.float32(0.2), None)])
+    run_graph("", lambda k: [(k.store(k.full(scalar, [2, 64], "bool")), np.full([2, 64], scalar, dtype=np.bool_), 0)])
+
+
+def test_broadcast_bool():  # :257-265
+    a0 = np.array([[True]]).astype(bool)
+    run_graph("", lambda k: [(k.store(k.broadcast(k.load(a0), [2, 3])), np.full([2, 3], True), 0)])
+
+
+def test_broadcast_then_reduce():  # :279-288 (the tile hint there is advice for the reference's tile model)
+    a = np.random.default_rng(6).normal(0, 0.1, [40, 20, 17, 1]).astype(np.float32)
+    run_graph("", lambda k: [(k.store(k.sum(k.broadcast(k.load(a), [40, 20, 17, 32]), (1,), True)),
+                              np.sum(np.broadcast_to(a, [40, 20, 17, 32]), (1,), keepdims=True), 1e-5)])
