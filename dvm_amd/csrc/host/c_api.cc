@@ -232,6 +232,7 @@ int dvm_rt_reset(dvm_rt *rt) {
   return Guard(
       [&]() {
         rt->FreeAll();
+        rt->fake_addr = 0x1000;  // dry runs hand out the same placeholder addresses after every reset
         rt->loads.clear();
         rt->stores.clear();
         rt->kernel.Reset(rt->ktype, rt->flags);

@@ -329,3 +329,39 @@ def test_reduce_over_axes_of_extent_one_is_a_squeeze():
     t.codegen()
     assert t.num_launches() == 1
     assert "pointwise" in t.das()
+
+
+def test_rebuilt_graphs_compile_to_the_same_program():
+    # tests/fuzz/test_eager_consistent.py: graphs rebuilt at random on one reused kernel object disassemble
+    # identically every time (no state leaks from one graph into the next)
+    def g0(t):
+        t.store(t.add(t.load(np.zeros([128], np.float32)), t.load(np.zeros([128], np.float32))))
+
+    def g1(t):
+        x1 = t.load(np.zeros([1, 32, 100, 44, 80], np.float32))
+        t.store(t.sum(t.mul(t.load(np.zeros([1, 32, 1, 44, 80], np.float32)), x1), (1,), False))
+        t.store(t.sum(t.mul(t.load(np.zeros([1, 1, 100, 44, 80], np.float32)), x1), (2,), False))
+
+    def g2(t):
+        x2 = t.matmul(t.load(np.zeros([2, 4, 512, 1024], np.float16)), t.load(np.zeros([1024, 512], np.float16)), False, False)
+        t.store(t.add(x2, 0.04))
+        t.store(t.mul(x2, 0.04))
+
+    def g3(t):
+        x0 = t.load(np.zeros([60, 288, 112], np.float32))
+        t.store(t.cast(t.cast(t.cast(t.cast(t.less(x0, 1), "float16"), "bool"), "float16"), "float32"))
+    graphs = [g0, g1, g2, g3]
+    t = Tester("eager", run_mode="das")
+    want = []
+    for g in graphs:
+        g(t)
+        t.codegen()
+        want.append(t.das())
+        t.reset()
+    rng = np.random.default_rng(0)
+    for _ in range(200):
+        i = int(rng.integers(0, len(graphs)))
+        graphs[i](t)
+        t.codegen()
+        assert t.das() == want[i]
+        t.reset()
