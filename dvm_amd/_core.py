@@ -429,6 +429,16 @@ class PyKernel(Kernel):
         (one team of lanes owns an output and combines in a fixed order), so both settings give the same bits."""
         pass
 
+    @staticmethod
+    def set_online_tuning(enable):
+        """The reference searches matmul tilings at run time (src/tuner.cc); tile choice here is a closed-form rule
+        of the problem size, so the switch is accepted and changes nothing."""
+        pass
+
+    @staticmethod
+    def set_lazy_tuning(enable):
+        pass
+
     def tile(self, start, end, num, factor=0):
         """Manual tiling of the reference's tile model (RtKernelPy::Tile, src/pybind_api.cc:1093). The gfx950
         schedules have no user-visible tiles; the hint is accepted and ignored."""
