@@ -53,6 +53,7 @@ def _load():
         "dvm_rt_copy": (vp, [vp, vp]),
         "dvm_rt_matmul": (vp, [vp, vp, vp, ci, ci, vp]),
         "dvm_rt_set_store_inplace": (ci, [vp, vp]),
+        "dvm_rt_clone": (ci, [vp, vp, ctypes.POINTER(ci), ctypes.POINTER(vp), cs, ctypes.POINTER(vp)]),
         "dvm_rt_seq_add": (ci, [vp, ci, ctypes.c_uint]),
         "dvm_rt_parallel_add": (ci, [vp, ci, ctypes.c_uint, cs]),
         "dvm_obj_rank": (ci, [vp]),
@@ -154,9 +155,12 @@ class NDObject:
 class IntArrayRef:
     """A shape (or axis list) whose values can change between codegen calls."""
 
-    def __init__(self, rt, shape=()):
-        arr, n = _i64(shape)
-        self._h = _ptr(_lib.dvm_rt_new_shape(rt, arr, n))
+    def __init__(self, rt, shape=(), handle=None):
+        if handle is not None:  # an existing reference of a cloned kernel
+            self._h = handle
+        else:
+            arr, n = _i64(shape)
+            self._h = _ptr(_lib.dvm_rt_new_shape(rt, arr, n))
         self._shape = tuple(int(v) for v in shape)
 
     def shape(self):
@@ -171,8 +175,8 @@ class IntArrayRef:
 class ScalarRef:
     """A scalar whose value is read again at every codegen."""
 
-    def __init__(self, rt, dtype):
-        self._h = _ptr(_lib.dvm_rt_new_scalar(rt, int(dtype)))
+    def __init__(self, rt, dtype, handle=None):
+        self._h = handle if handle is not None else _ptr(_lib.dvm_rt_new_scalar(rt, int(dtype)))
 
     def update(self, value):
         if isinstance(value, (int, np.integer)) and not isinstance(value, bool):
@@ -344,6 +348,41 @@ class PyKernel(Kernel):
         op = Kernel.load(self, ref, type)
         self._load_shape[op._h] = ref
         return op
+
+    def clone(self, base, remap):
+        """Copies `base`'s graph into this kernel (RtKernelPy::Clone, src/pybind_api.cc:923-993). `remap` lists
+        operators, shape / axis references and scalar references of `base`; their counterparts here are returned."""
+        items = list(remap)
+        base_loads = list(base._load_shape.items())  # (load handle, IntArrayRef)
+        kinds, handles = [], []
+        for it in items:
+            kinds.append(1 if isinstance(it, IntArrayRef) else (2 if isinstance(it, ScalarRef) else 0))
+            handles.append(it._h)
+        for h, ref in base_loads:
+            kinds += [0, 1]
+            handles += [h, ref._h]
+        n = len(kinds)
+        ck = (ctypes.c_int * n)(*kinds)
+        ch = (ctypes.c_void_p * n)(*handles)
+        co = (ctypes.c_void_p * n)()
+        _check(_lib.dvm_rt_clone(self._rt, base._rt, ck, ch, n, co))
+        self._keep, self._load_shape, self._inputs = [], {}, {}
+        out = []
+        for i, it in enumerate(items):
+            if kinds[i] == 1:
+                w = IntArrayRef(self._rt, it.shape(), handle=co[i])
+            elif kinds[i] == 2:
+                w = ScalarRef(self._rt, None, handle=co[i])
+            else:
+                w = self._wrap(co[i])
+            self._keep.append(w)
+            out.append(w)
+        for j, (h, ref) in enumerate(base_loads):
+            i = len(items) + 2 * j
+            sref = IntArrayRef(self._rt, ref.shape(), handle=co[i + 1])
+            self._keep.append(sref)
+            self._load_shape[co[i]] = sref
+        return tuple(out)
 
     def reset(self):
         _check(_lib.dvm_rt_reset(self._rt))

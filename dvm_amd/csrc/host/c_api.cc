@@ -398,6 +398,66 @@ dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int 
       static_cast<dvm_obj *>(nullptr));
 }
 
+// RtKernelPy::Clone (src/pybind_api.cc:923-993): rebuilds `base`'s graph in `rt`, with shapes, axis lists and
+// scalars of its own, and translates the n handles in `items` (kinds: 0 operator, 1 shape, 2 scalar) to the
+// clone's handles in `out`.
+int dvm_rt_clone(dvm_rt *rt, dvm_rt *base, const int *kinds, void *const *items, size_t n, void **out) {
+  return Guard(
+      [&]() {
+        struct Helper : public CloneHelper {
+          IntArrayRef *GetClone(IntArrayRef *shape) override {
+            auto it = shapes.find(shape);
+            return it != shapes.end() ? it->second : shape;
+          }
+          ScalarRef *GetClone(ScalarRef *scalar) override {
+            auto it = scalars.find(scalar);
+            return it != scalars.end() ? it->second : scalar;
+          }
+          NDObject *GetClone(NDObject *op) override {
+            auto it = ops.find(op);
+            return it != ops.end() ? it->second : nullptr;
+          }
+          void SetClone(NDObject *op, NDObject *clone) override { ops[op] = clone; }
+          std::map<IntArrayRef *, IntArrayRef *> shapes;
+          std::map<ScalarRef *, ScalarRef *> scalars;
+          std::map<NDObject *, NDObject *> ops;
+        } helper;
+        rt->FreeAll();
+        rt->loads.clear();
+        rt->stores.clear();
+        std::map<const dvm_shape *, dvm_shape *> shape_of;
+        std::map<const dvm_scalar *, dvm_scalar *> scalar_of;
+        for (const auto &sh : base->shapes) {
+          rt->shapes.emplace_back(new dvm_shape());
+          rt->shapes.back()->dims.reserve(kMaxRank);
+          rt->shapes.back()->Set(sh->dims.data(), sh->dims.size());
+          helper.shapes[&sh->ref] = &rt->shapes.back()->ref;
+          shape_of[sh.get()] = rt->shapes.back().get();
+        }
+        for (const auto &sc : base->scalars) {
+          rt->scalars.emplace_back(new dvm_scalar());
+          rt->scalars.back()->ref = sc->ref;
+          helper.scalars[&sc->ref] = &rt->scalars.back()->ref;
+          scalar_of[sc.get()] = rt->scalars.back().get();
+        }
+        rt->kernel.Clone(base->kernel, helper);
+        for (NDObject *o : base->loads) rt->loads.push_back(helper.GetClone(o));
+        for (NDObject *o : base->stores) rt->stores.push_back(helper.GetClone(o));
+        for (size_t i = 0; i < n; ++i) {
+          if (kinds[i] == 0) {
+            out[i] = helper.GetClone(static_cast<NDObject *>(items[i]));
+          } else if (kinds[i] == 1) {
+            out[i] = shape_of[static_cast<const dvm_shape *>(items[i])];
+          } else {
+            out[i] = scalar_of[static_cast<const dvm_scalar *>(items[i])];
+          }
+          if (out[i] == nullptr) throw std::runtime_error("DVM EXCEPTION. reason: clone of a handle that does not belong to the base kernel");
+        }
+        return 0;
+      },
+      -1);
+}
+
 int dvm_rt_seq_add(dvm_rt *rt, int ktype, unsigned flags) {
   return Guard(
       [&]() {

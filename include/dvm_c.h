@@ -64,6 +64,10 @@ int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store);
 // Group markers of "seq" and "parallel" kernels (KernelPy::SequenceAdd / ParallelAdd, include/dvm_py.h:369-371; Kernel::SequenceAdd /
 // ParallelAdd, include/dvm.h:250-251): operators built after the call belong to the next sub-kernel group.
 int dvm_rt_seq_add(dvm_rt *rt, int ktype, unsigned flags);
+// RtKernelPy::Clone (src/pybind_api.cc:923-993; Kernel::Clone, include/dvm.h:188): `rt` becomes a copy of `base`'s
+// graph with shapes, axis lists and scalars of its own. items[i] (kinds[i]: 0 dvm_obj*, 1 dvm_shape*, 2 dvm_scalar*)
+// are handles of `base`; out[i] receives the corresponding handle of `rt`.
+int dvm_rt_clone(dvm_rt *rt, dvm_rt *base, const int *kinds, void *const *items, size_t n, void **out);
 int dvm_rt_parallel_add(dvm_rt *rt, int ktype, unsigned flags, size_t core_limit);
 
 int dvm_obj_rank(const dvm_obj *o);

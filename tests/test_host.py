@@ -365,3 +365,21 @@ def test_rebuilt_graphs_compile_to_the_same_program():
         t.codegen()
         assert t.das() == want[i]
         t.reset()
+
+
+def test_clone_is_independent_of_its_base():
+    # tests/ut/test_clone.py:36-56: the clone has its own shape and axis references
+    t = Tester("vector:dyn", run_mode="das")
+    ax = t.load([], "float32")
+    dims = t.int_array()
+    out = t.store(t.sum(t.add(ax, 0.01), dims, True))
+    t.input(ax, np.zeros([10, 512], np.float32))
+    dims.update([0])
+    t.codegen()
+    t2 = Tester("vector:dyn", run_mode="das")
+    ax2, out2, dims2 = t2.clone(t, [ax, out, dims])
+    t2.input(ax2, np.zeros([64, 800], np.float32))
+    dims2.update([1])
+    t2.codegen()
+    assert out2.shape() == (64, 1) and out.shape() == (1, 512)
+    assert "reduce-x" in t2.das() and "reduce-y" in t.das()
