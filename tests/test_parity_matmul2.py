@@ -1,0 +1,119 @@
+"""GPU parity: the matmul cases of the reference's tests/ut/test_matmul.py beyond those in test_parity_matmul.py:
+very wide N, folded batches (a unit axis between batch and k), one operand used twice, a single-row product
+with a long k, the product + epilogue graphs written for other store paths (same mathematics here), dynamic
+shapes run repeatedly. NumPy expectations and tolerances as in the reference; the oracle where it takes seconds."""
+import numpy as np
+import pytest
+
+from dvm_amd.tester import Tester
+from tests.util import run_graph
+
+pytestmark = pytest.mark.gpu
+
+
+def _close(out, want, eps):
+    return np.allclose(out, want, rtol=eps, atol=eps)
+
+
+def test_matmul_n_big():  # tests/ut/test_matmul.py:455-472
+    np.random.seed(1)
+    ax, bx = Tester.fast_random_normal(0, 0.1, [256, 256]).astype(np.float16), Tester.fast_random_normal(0, 0.1, [81960, 256]).astype(np.float16)
+    np_c = np.matmul(ax.astype(np.float32), bx.astype(np.float32).T).astype(np.float16)
+    zx = Tester.fast_random_normal(0, 0.1, np_c.shape).astype(np.float16)
+    run_graph("mix", lambda k: [(k.store(k.add(k.matmul(k.load(ax), k.load(bx), False, True), k.load(zx))), np_c + zx, 2e-3)], oracle=False)
+
+
+@pytest.mark.parametrize("shape_a,shape_b,shape_bias", [([256, 1, 1000], [1000, 256], None), ([256, 1, 1000], [1000, 256], [256, 1, 256]),
+                                                        ([256, 1, 1000], [1000, 256], [1, 256]), ([520, 1, 40960], [40960, 256], [520, 1, 256]),
+                                                        ([520, 1, 40960], [40960, 256], [1, 256])])
+def test_batch_fold(shape_a, shape_b, shape_bias):  # :537-561
+    np.random.seed(2)
+    a, b = Tester.fast_random_normal(0, 0.1, shape_a).astype(np.float16), Tester.fast_random_normal(0, 0.1, shape_b).astype(np.float16)
+    expect = np.matmul(a.astype(np.float32), b.astype(np.float32)).astype(np.float16)
+    bias = Tester.fast_random_normal(0, 0.1, shape_bias).astype(np.float16) if shape_bias else None
+
+    def g(k):
+        out = k.matmul(k.load(a), k.load(b), False, False)
+        if bias is not None:
+            out = k.add(out, k.load(bias))
+        return [(k.store(out), expect + bias if bias is not None else expect, 2e-3)]
+    run_graph("mix", g, oracle=shape_a[-1] <= 1000, oracle_eps=2e-3)
+
+
+def test_batch_fold_broadcast():  # :562-583
+    np.random.seed(3)
+    a0 = Tester.fast_random_normal(0, 0.1, [632, 1, 3584]).astype(np.float16)
+    a1 = Tester.fast_random_normal(0, 0.1, [4608, 3584]).astype(np.float16)
+    a4 = np.random.normal(0, 0.1, [4608]).astype(np.float16)
+    e2 = np.matmul(a0.astype(np.float32), a1.swapaxes(-1, -2).astype(np.float32)).astype(np.float16)
+
+    def g(k):
+        x3 = k.cast(k.matmul(k.load(a0), k.load(a1), False, True), "float32")
+        return [(k.store(k.cast(k.add(x3, k.cast(k.load(a4), "float32")), "float16")), (e2.astype(np.float32) + a4.astype(np.float32)).astype(np.float16), 1e-3)]
+    run_graph("mix", g, oracle=False)
+
+
+@pytest.mark.parametrize("shape_a,shape_b", [([256, 256], [256, 256]), ([1024, 128], [128, 1024]), ([301, 256], [256, 401]),
+                                             ([300, 6400], [6400, 10240])])
+@pytest.mark.parametrize("z32", [False, True])
+def test_product_plus_tensor_abs(shape_a, shape_b, z32):  # :584-668 (three store paths there, one here)
+    rng = np.random.default_rng(shape_a[0])
+    ax, bx = rng.normal(0, 0.1, shape_a).astype(np.float16), rng.normal(0, 0.1, shape_b).astype(np.float16)
+    np_c = np.matmul(ax.astype(np.float32), bx.astype(np.float32))
+    zx = rng.normal(0, 0.1, np_c.shape).astype(np.float32 if z32 else np.float16)
+
+    def g(k):
+        c = k.matmul(k.load(ax), k.load(bx), False, False)
+        if z32:
+            c = k.cast(c, "float32")
+        return [(k.store(k.abs(k.add(c, k.load(zx)))), np.abs(np_c + zx), 2e-3 * max(1.0, float(np.abs(np_c).max())))]
+    run_graph("mix", g, oracle=shape_a[1] <= 256, oracle_eps=2e-3)
+
+
+@pytest.mark.parametrize("mode,shape", [("mix", [1024, 2048]), ("mix:dyn", [1000, 2000])])
+def test_same_matmul_input(mode, shape):  # :669-679
+    g0 = np.random.default_rng(4).normal(0, 0.1, shape).astype(np.float16)
+    expect = np.matmul(g0.astype(np.float32), g0.T.astype(np.float32)).astype(np.float16)
+    run_graph(mode, lambda k: (lambda a: [(k.store(k.matmul(a, a, False, True)), expect, 2e-3)])(k.load(g0)), oracle_eps=2e-3)
+
+
+@pytest.mark.parametrize("mode", ["mix", "mix:dyn"])
+def test_operand_also_in_epilogue(mode):  # :680-694
+    rng = np.random.default_rng(5)
+    g0, g1 = rng.normal(0, 0.1, [1024, 1024]).astype(np.float16), rng.normal(0, 0.1, [1024, 1536]).astype(np.float16)
+    expect = np.matmul(g0.astype(np.float32), g1.astype(np.float32)).astype(np.float16) + g1
+
+    def g(k):
+        b = k.load(g1)
+        return [(k.store(k.add(k.matmul(k.load(g0), b, False, False), b)), expect, 2e-3)]
+    run_graph(mode, g, oracle_eps=2e-3)
+
+
+@pytest.mark.parametrize("mix", [False, True])
+def test_dynamic_matmul_run_three_times(mix):  # :695-719
+    rng = np.random.default_rng(6)
+    a, b = rng.normal(0, 0.01, [4096, 4096]).astype(np.float16), rng.normal(0, 0.01, [4096, 4096]).astype(np.float16)
+    expect = np.matmul(a.astype(np.float32), b.astype(np.float32))
+    Tester.set_lazy_tuning(True)
+    try:
+        t = Tester("mix:dyn")
+        x0, x1 = t.load([], "float16"), t.load([], "float16")
+        x2 = t.matmul(x0, x1, False, False)
+        if mix:
+            x2 = t.add(x2, 0.1)
+            expect = expect + 0.1
+        x3 = t.store(x2)
+        for _ in range(3):
+            t.input(x0, a)
+            t.input(x1, b)
+            t.run()
+            assert t.check(x3, expect, 2e-3)
+    finally:
+        Tester.set_lazy_tuning(False)
+
+
+def test_single_row_long_k():  # :720-735
+    rng = np.random.default_rng(17)
+    np_a, np_b = rng.normal(0, 0.1, (1, 80000)).astype(np.float16), rng.normal(0, 0.1, (80000, 256)).astype(np.float16)
+    run_graph("mix", lambda k: [(k.store(k.matmul(k.load(np_a), k.load(np_b), False, False)),
+                                 np_a.astype(np.float32) @ np_b.astype(np.float32), 2e-3 * 30)], oracle_eps=2e-3 * 30)
