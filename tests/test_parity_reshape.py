@@ -97,7 +97,7 @@ def test_matmul_then_reshape():  # :296-311
     bx = Tester.fast_random_normal(0, 0.01, [3072, 3072]).astype(np.float16)
     e = np.matmul(ax.astype(np.float32), bx.astype(np.float32)).astype(np.float16)
     run_graph("mix", lambda k: [(k.store(k.reshape(k.matmul(k.load(ax), k.load(bx), False, False), (2, 510, 48, 64))),
-                                 np.reshape(e, (2, 510, 48, 64)), 2e-3)], oracle_eps=2e-3)
+                                 np.reshape(e, (2, 510, 48, 64)), 2e-3)], oracle=False)  # 9.6 GFLOP: NumPy golden only
 
 
 @pytest.mark.parametrize("shape_a,shape_b,shape_c", [([1, 8, 2048, 512], [1, 8, 512, 128], [8, 2048, 128]), ([2048, 512], [512, 512], [2048, 1, 512]),

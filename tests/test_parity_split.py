@@ -52,7 +52,7 @@ def test_static_matmul_with_bias(mode):  # :60-77
         rng.normal(0, 0.1, [1024]).astype(np.float16)
     res = np.matmul((xd * np.float16(0.5)).astype(np.float32), yd.astype(np.float32)).astype(np.float16) + bd + np.float16(0.1)
     run_graph(mode, lambda k: [(k.store(k.add(k.matmul(k.mul(k.load(xd), 0.5), k.load(yd), False, False, k.load(bd)), 0.1)), res, 2e-3)],
-              oracle_eps=2e-3)
+              oracle=mode == "split", oracle_eps=2e-3)
 
 
 @pytest.mark.parametrize("mode", ["split:dyn", "split:dyn,unify_ws"])
@@ -110,7 +110,7 @@ def test_matmul_stored_and_used(x_shape, y_shape, mode):  # :144-165
         s0 = k.store(x)
         return [(s0, res, 2e-3), (k.store(k.add(x, 0.1)), res + np.float16(0.1), 2e-3)]
     # rows of fast_random_normal are equal, sums over k = 40960 reach hundreds: tolerance relative to that, as np.allclose's rtol does
-    run_graph(mode, g, oracle=x_shape[1] <= 4096, oracle_eps=2e-3)
+    run_graph(mode, g, oracle=mode == "split:dyn", oracle_eps=2e-3)  # the scalar oracle takes 18 s on this size: once is enough
 
 
 @pytest.mark.parametrize("mode", ["split:unify_ws", "split:dyn,unify_ws"])
