@@ -53,6 +53,11 @@ def _load():
         "dvm_rt_copy": (vp, [vp, vp]),
         "dvm_rt_matmul": (vp, [vp, vp, vp, ci, ci, vp]),
         "dvm_rt_set_store_inplace": (ci, [vp, vp]),
+        "dvm_rt_view_load": (vp, [vp, vp, vp, ci]),
+        "dvm_rt_slice_load": (vp, [vp, vp, vp, vp, ci]),
+        "dvm_rt_stridedslice_load": (vp, [vp, vp, vp, vp, vp, ci]),
+        "dvm_rt_view_store": (vp, [vp, vp, vp, cs]),
+        "dvm_obj_set_view_offset": (ci, [vp, ctypes.c_longlong]),
         "dvm_rt_clone": (ci, [vp, vp, ctypes.POINTER(ci), ctypes.POINTER(vp), cs, ctypes.POINTER(vp)]),
         "dvm_rt_seq_add": (ci, [vp, ci, ctypes.c_uint]),
         "dvm_rt_parallel_add": (ci, [vp, ci, ctypes.c_uint, cs]),
@@ -249,6 +254,22 @@ class Kernel:
     def set_store_inplace(self, store):
         _check(_lib.dvm_rt_set_store_inplace(self._rt, store._h))
 
+    # -- strided views (include/dvm_py.h view_load / slice_load / stridedslice_load); innermost stride 1 --
+    def view_load(self, shape, stride, type):
+        return self._wrap(_lib.dvm_rt_view_load(self._rt, self._shape_ref(shape)._h, self._shape_ref(stride)._h, int(type)))
+
+    def slice_load(self, shape, start, size, type):
+        return self._wrap(_lib.dvm_rt_slice_load(self._rt, self._shape_ref(shape)._h, self._shape_ref(start)._h,
+                                                 self._shape_ref(size)._h, int(type)))
+
+    def stridedslice_load(self, shape, start, end, step, type):
+        return self._wrap(_lib.dvm_rt_stridedslice_load(self._rt, self._shape_ref(shape)._h, self._shape_ref(start)._h,
+                                                        self._shape_ref(end)._h, self._shape_ref(step)._h, int(type)))
+
+    def view_store(self, obj, stride, extent):
+        """Stores obj through element strides into a zero-initialised buffer of `extent` elements."""
+        return self._wrap(_lib.dvm_rt_view_store(self._rt, obj._h, self._shape_ref(stride)._h, int(extent)))
+
     # -- sub-kernel groups of "seq" / "parallel" kernels (include/dvm_py.h:369-371) --
     def seq_add(self, ktype, flags=0):
         _check(_lib.dvm_rt_seq_add(self._rt, int(ktype), int(flags)))
@@ -404,7 +425,7 @@ class PyKernel(Kernel):
         _lib.dvm_c_bf16_to_f32(src.ctypes.data, dst.ctypes.data, src.size)
         return dst
 
-    def input(self, load, array):
+    def input(self, load, array, offset=0):
         """Binds a numpy array (copied to the device), a scalar value, or a shape to a placeholder."""
         if isinstance(load, ScalarRef):
             load.update(array)
@@ -413,6 +434,8 @@ class PyKernel(Kernel):
             load.update(list(array))
             return
         arr = np.ascontiguousarray(array)
+        if offset:
+            _check(_lib.dvm_obj_set_view_offset(load._h, int(offset)))
         ref = self._load_shape.get(load._h)
         if ref is not None and tuple(ref.shape()) != tuple(arr.shape):
             ref.update(list(arr.shape))
@@ -437,8 +460,9 @@ class PyKernel(Kernel):
     def run(self, stream=None, sync=True):
         _check(_lib.dvm_rt_run(self._rt, ctypes.c_void_p(stream) if stream else None, int(sync)))
 
-    def output(self, store):
-        shape = store.shape()
+    def output(self, store, shape=None):
+        """The stored tensor; `shape` (strided stores) reads back the whole buffer the store wrote into."""
+        shape = store.shape() if shape is None else tuple(shape)
         dt = int(store.dtype())
         out = np.empty(shape, dtype=_NP_OF[dt])
         _check(_lib.dvm_rt_output(self._rt, store._h, out.ctypes.data, out.nbytes))

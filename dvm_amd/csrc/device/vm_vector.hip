@@ -134,6 +134,13 @@ __device__ __forceinline__ void elem_store(uint64_t base, uint32_t dtype, uint64
 // Slow path of a slab: scalar per-element accesses (ragged tail, unaligned rows, stride-0 operand).
 __device__ __forceinline__ vf8 slab_load_slow(const VMemDesc &m, uint64_t off, int nv) {
   vf8 out = 0.0f;
+  if (m.flags & VMF_GATHER) {
+    const uint64_t step = m.flags >> 8;
+    FOR_E {
+      if (e < nv) out[e] = elem_load(m.addr, m.dtype, off + e * step);
+    }
+    return out;
+  }
   if (!(m.flags & VMF_VEC)) {
     out = elem_load(m.addr, m.dtype, off);
     return out;
@@ -145,6 +152,13 @@ __device__ __forceinline__ vf8 slab_load_slow(const VMemDesc &m, uint64_t off, i
 }
 
 __device__ __forceinline__ void slab_store_slow(const VMemDesc &m, uint64_t off, int nv, vf8 in) {
+  if (m.flags & VMF_GATHER) {
+    const uint64_t step = m.flags >> 8;
+    FOR_E {
+      if (e < nv) elem_store(m.addr, m.dtype, off + e * step, in[e]);
+    }
+    return;
+  }
   if (!(m.flags & VMF_VEC)) {
     elem_store(m.addr, m.dtype, off, in[0]);
     return;
@@ -279,7 +293,7 @@ __device__ __forceinline__ void mem_load(const VMemDesc &m, const Offs &off, uin
   const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
   if (fast && wave_all(nvp == kAllFull)) {
     mem_load_wide(m, off, out);
-  } else if (!(m.flags & VMF_VEC) && (m.dtype == VDT_F32 || m.dtype == VDT_I32)) {
+  } else if (!(m.flags & (VMF_VEC | VMF_GATHER)) && (m.dtype == VDT_F32 || m.dtype == VDT_I32)) {
     // one 32-bit element per slab, replicated (an operand broadcast along the innermost axis: a per-channel
     // scale, a per-row statistic); lanes without a valid slab read the base element and get zero, like the
     // guarded path. Inline: the out-of-line path saves registers to scratch memory around the call.

@@ -55,6 +55,7 @@ struct dvm_rt {
   std::vector<std::unique_ptr<dvm_shape>> shapes;
   std::vector<std::unique_ptr<dvm_scalar>> scalars;
   std::vector<NDObject *> loads, stores;
+  std::map<NDObject *, size_t> store_extent;  // strided stores: elements of the whole buffer they write into
   std::map<NDObject *, Buffer> buffers;
   Buffer workspace;
   uint64_t fake_addr = 0x1000;
@@ -233,6 +234,7 @@ int dvm_rt_reset(dvm_rt *rt) {
       [&]() {
         rt->FreeAll();
         rt->fake_addr = 0x1000;  // dry runs hand out the same placeholder addresses after every reset
+        rt->store_extent.clear();
         rt->loads.clear();
         rt->stores.clear();
         rt->kernel.Reset(rt->ktype, rt->flags);
@@ -476,6 +478,52 @@ int dvm_rt_parallel_add(dvm_rt *rt, int ktype, unsigned flags, size_t core_limit
       -1);
 }
 
+dvm_obj *dvm_rt_view_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *stride, int dtype) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.Load(nullptr, &shape->ref, &stride->ref, static_cast<DataType>(dtype));
+        rt->loads.push_back(o);
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_slice_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *start, dvm_shape *size, int dtype) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.SliceLoad(nullptr, &shape->ref, &start->ref, &size->ref, static_cast<DataType>(dtype));
+        rt->loads.push_back(o);
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_stridedslice_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *start, dvm_shape *end, dvm_shape *step, int dtype) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.StridedSliceLoad(nullptr, &shape->ref, &start->ref, &end->ref, &step->ref, static_cast<DataType>(dtype));
+        rt->loads.push_back(o);
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_view_store(dvm_rt *rt, dvm_obj *x, dvm_shape *stride, size_t extent_elems) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.Store(nullptr, Obj(x), &stride->ref);
+        rt->stores.push_back(o);
+        rt->store_extent[o] = extent_elems;
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+int dvm_obj_set_view_offset(dvm_obj *io, long long elems) {
+  Obj(io)->view_offset = elems;
+  return 0;
+}
+
 int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store) {
   return Guard(
       [&]() {
@@ -531,6 +579,19 @@ int dvm_rt_codegen(dvm_rt *rt) {
         const auto t1 = std::chrono::steady_clock::now();
         // outputs take their size from the inferred shapes
         for (NDObject *s : rt->stores) {
+          auto ext = rt->store_extent.find(s);
+          if (ext != rt->store_extent.end()) {
+            // a strided store writes part of a larger buffer, which starts out as zeros
+            const size_t bytes = ext->second * DTypeSize(s->type_id_);
+            const bool fresh = rt->buffers.find(s) == rt->buffers.end() || rt->buffers[s].ptr == nullptr;
+            rt->Ensure(s, bytes);
+            if (fresh && !rt->das_mode && bytes > 0) {
+              std::vector<char> zeros(bytes, 0);
+              int rc = rt->Api().mem_to_dev(rt->buffers[s].ptr, zeros.data(), bytes);
+              if (rc != 0) throw std::runtime_error(std::string("host to device copy failed: ") + rt->Api().error_string(rc));
+            }
+            continue;
+          }
           const size_t bytes = static_cast<size_t>(s->numel()) * DTypeSize(s->type_id_);
           rt->Ensure(s, bytes);
         }

@@ -62,12 +62,59 @@ void BroadcastShapes(const NDObject *a, const NDObject *b, int64_t *out, size_t 
 }  // namespace
 
 void VKernel::Normalize() {
+  // a slice bound below zero counts from the end of its axis; bounds past either end stop there
+  // (src/dvm.cc:770-773,826-831 of the reference, which clips the end; NumPy's rule for both)
+  auto bound = [](int64_t v, int64_t extent) {
+    if (v < 0) v += extent;
+    return std::min(std::max<int64_t>(v, 0), extent);
+  };
   for (NDObject *o : ops_) {
     switch (o->kind) {
       case kObjLoad:
+        if (o->strided) {
+          if (o->slice_end != nullptr) {  // strided slice: the value's shape comes from start / end / step
+            const size_t r = o->full_shape_ref->size;
+            if (o->slice_start->size != r || o->slice_end->size != r || o->slice_step->size != r) Throw("slice lists do not match the tensor rank");
+            for (size_t i = 0; i < r; ++i) {
+              const int64_t st = o->slice_step->data[i];
+              if (st <= 0) Throw("slice step has to be positive");
+              const int64_t len = bound(o->slice_end->data[i], o->full_shape_ref->data[i]) -
+                                  bound(o->slice_start->data[i], o->full_shape_ref->data[i]);
+              o->shape_[i] = len > 0 ? (len + st - 1) / st : 0;
+            }
+            o->own_ref_.size = r;
+          }
+          const size_t r = o->shape_ref_->size;
+          if (r > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
+          o->view_base_ = o->view_offset;
+          if (o->stride_ref != nullptr) {
+            if (o->stride_ref->size != r) Throw("stride list does not match the tensor rank");
+            for (size_t i = 0; i < r; ++i) o->vstride_[i] = o->stride_ref->data[i];
+          } else {
+            if (o->full_shape_ref->size != r || o->slice_start->size != r) Throw("slice lists do not match the tensor rank");
+            int64_t dense = 1;
+            for (size_t i = r; i-- > 0;) {
+              const int64_t st = o->slice_step != nullptr ? o->slice_step->data[i] : 1;
+              const int64_t first = bound(o->slice_start->data[i], o->full_shape_ref->data[i]);
+              if (first + (o->shape_ref_->data[i] - 1) * st >= o->full_shape_ref->data[i]) {
+                if (o->shape_ref_->data[i] > 0) Throw("slice reaches outside the tensor");
+              }
+              o->vstride_[i] = dense * st;
+              o->view_base_ += first * dense;
+              dense *= o->full_shape_ref->data[i];
+            }
+          }
+        }
         if (o->shape_ref_->size > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
         break;
       case kObjStore:
+        o->SetShape(o->in[0]->shape_ref_->data, o->in[0]->shape_ref_->size);
+        if (o->strided) {
+          if (o->stride_ref->size != o->in[0]->shape_ref_->size) Throw("stride list does not match the tensor rank");
+          for (size_t i = 0; i < o->stride_ref->size; ++i) o->vstride_[i] = o->stride_ref->data[i];
+          o->view_base_ = o->view_offset;
+        }
+        break;
       case kObjUnary:
       case kObjBinaryS:
       case kObjCompareS:
@@ -201,6 +248,7 @@ struct ANode {
   int addr_op;          // load/store operator supplying the address, or -1
   int ws_slot;          // workspace slot, or -1
   int mem_idx;          // descriptor index in the program
+  const NDObject *view; // load / store that walks its buffer with strides of its own, or nullptr (dense)
   // emission state
   bool has_inner;       // varies along the innermost domain axis
   bool fd;              // has a reduced axis
@@ -562,7 +610,9 @@ class Compiler {
     for (int i = 0; i < n_; ++i) {
       NDObject *o = k_->ops_[i];
       if (!live_[i]) continue;
-      if (o->kind == kObjStore) store_of_[o->in[0]->id] = i;
+      // a value stored through a stride list is not read back from there by later launches: they expect
+      // the dense layout, so such a value also goes to the workspace when it crosses launches
+      if (o->kind == kObjStore && !o->strided) store_of_[o->in[0]->id] = i;
     }
     for (int i = 0; i < n_; ++i) {
       NDObject *o = k_->ops_[i];
@@ -598,6 +648,12 @@ class Compiler {
   int dim_of_axis_[kMaxAxes]; // ordered position -> merged dim
   // kept / reduced lists, innermost first (indices into dims_)
   int klist_[DVM_VEC_MAXR], rlist_[DVM_VEC_MAXR];
+  // Kept dims beyond the VM's DVM_VEC_MAXR (the outermost ones) are peeled: the program covers one index of
+  // them and is launched once per index, every operand address moved by that index times its stride.
+  static constexpr int kMaxPeel = 4;
+  int n_peel_ = 0;
+  int peel_dim_[kMaxPeel];
+  int64_t peel_stride_[DVM_VEC_MAXMEM][kMaxPeel];
   int nk_ = 0, nr_ = 0;
   // program under construction
   Program *prog_ = nullptr;
@@ -643,6 +699,10 @@ class Compiler {
       const NDObject *root = ViewRoot(v);
       if (root->kind == kObjLoad) {
         nodes_[idx].addr_op = root->id;
+        if (root->strided) {
+          if (root != v) Throw("DVM EXCEPTION. reason: a reshape of a strided load is not supported by the gfx950 backend");
+          nodes_[idx].view = root;
+        }
       } else if (ws_slot_[root->id] >= 0) {
         nodes_[idx].ws_slot = ws_slot_[root->id];
       } else {
@@ -678,6 +738,7 @@ class Compiler {
   void ChooseSchedule();
   void EmitProgram();
   void FinishProgram();
+  void ReplicatePeeled();
 
   // union-find over (node, dim) variables
   std::vector<int> uf_;
@@ -722,6 +783,7 @@ class Compiler {
   void FuseSweepInstructions();
   void MarkUniformRuns();
   void PlanRereads();
+  bool mem_is_view_[DVM_VEC_MAXMEM] = {false};  // memory operand i is a strided view
   int last_mem_ = -1;         // memory operand of the last memory instruction emitted in this round, or -1
   int u_ = 2;                 // slabs per lane per instruction of the program being compiled
   bool uniform_emit_ = false; // the value being computed is the same in every element of a lane's accumulator
@@ -792,7 +854,10 @@ void Compiler::BuildNodes(int a) {
     ANode &n = nodes_[idx];
     n.nin = o->nin;
     for (int j = 0; j < 3; ++j) n.in[j] = in_idx[j];
-    if (kind == AK_OUT) n.addr_op = i;
+    if (kind == AK_OUT) {
+      n.addr_op = i;
+      if (o->strided) n.view = o;
+    }
     node_of_[i] = idx;
     // a value later sub-kernels read and that the user does not store: write it to workspace
     if (mat_[i] && ws_slot_[i] >= 0) {
@@ -985,6 +1050,8 @@ void Compiler::OrderAndMerge() {
           // contiguous only if nothing of extent > 1 lies between them
           for (int d = d0 + 1; d < d1; ++d)
             if (n.dims[d] != 1) merge = false;
+          // and, for a strided view, if the outer stride is what a dense walk would have
+          if (n.view != nullptr && n.view->vstride_[d0] != n.view->vstride_[d1] * n.dims[d1]) merge = false;
         }
       }
     }
@@ -1005,14 +1072,16 @@ void Compiler::OrderAndMerge() {
     dims_[0].first_axis = dims_[0].last_axis = -1;
     n_dims_ = 1;
   }
-  nk_ = nr_ = 0;
+  nk_ = nr_ = n_peel_ = 0;
   for (int d = n_dims_ - 1; d >= 0; --d) {
     if (dims_[d].reduced) {
       if (nr_ >= DVM_VEC_MAXR) Fail("too many reduced dims");
       rlist_[nr_++] = d;
-    } else {
-      if (nk_ >= DVM_VEC_MAXR) Fail("too many kept dims");
+    } else if (nk_ < DVM_VEC_MAXR) {
       klist_[nk_++] = d;
+    } else {
+      if (n_peel_ >= kMaxPeel) Fail("too many kept dims");
+      peel_dim_[n_peel_++] = d;
     }
   }
 }
@@ -1132,7 +1201,8 @@ int Compiler::MemIndex(int v) {
       const int p = pos_[n.axis[d]];
       const int md = dim_of_axis_[p];
       dim_has[md] = true;
-      if (p == dims_[md].last_axis) dim_stride[md] = stride;  // the innermost axis of a merged dim carries its stride
+      // the innermost axis of a merged dim carries its stride; a strided view brings its own
+      if (p == dims_[md].last_axis) dim_stride[md] = n.view != nullptr ? n.view->vstride_[d] : stride;
     }
     stride *= n.dims[d];
   }
@@ -1154,15 +1224,29 @@ int Compiler::MemIndex(int v) {
     m.rstride[i] = static_cast<uint32_t>(dim_stride[md]);
     if (md != inner && (dim_stride[md] * isz) % need != 0) aligned = false;
   }
+  for (int i = 0; i < n_peel_; ++i) {
+    const int md = peel_dim_[i];
+    peel_stride_[n_mem_][i] = dim_has[md] ? dim_stride[md] * isz : 0;  // in bytes
+    if (peel_stride_[n_mem_][i] % need != 0) aligned = false;
+  }
   if (dim_has[inner] && dims_[inner].first_axis >= 0) {
-    if (dim_stride[inner] != 1) Fail("innermost axis is not contiguous");
-    m.flags |= VMF_VEC;
-    if (aligned) m.flags |= VMF_ALIGNED;
+    if (dim_stride[inner] == 1) {
+      m.flags |= VMF_VEC;
+      if (aligned) m.flags |= VMF_ALIGNED;
+    } else if (n.view != nullptr && dim_stride[inner] != 0) {
+      // a transposing or element-skipping view: element by element (correct, not fast)
+      if (dim_stride[inner] >= (1ll << 24) || dim_stride[inner] < 0) Fail("innermost stride above 2^24");
+      m.flags |= VMF_GATHER | (static_cast<uint32_t>(dim_stride[inner]) << 8);
+    } else if (dim_stride[inner] != 0) {
+      Fail("innermost axis is not contiguous");
+    }
   }
   Program::Patch p;
   p.word = static_cast<uint32_t>(sizeof(VVecHeader) / 8 + n_mem_ * (sizeof(VMemDesc) / 8));
   p.op_id = n.addr_op;
   p.ws_slot = n.ws_slot;
+  p.byte_offset = n.view != nullptr ? n.view->view_base_ * isz : 0;
+  mem_is_view_[n_mem_] = n.view != nullptr;
   p.role = Program::kPatchVecMem;
   prog_->patches.push_back(p);
   n.mem_idx = n_mem_++;
@@ -1765,7 +1849,7 @@ void Compiler::FuseSweepInstructions() {
 void Compiler::MarkUniformRuns() {
   if ((hdr_.sched & VS_KIND_MASK) != VS_REDX || !hdr_.team_is_block) return;
   auto bcast_load = [&](uint64_t w) {
-    return VI_OP(w) == VOP_LD && VI_KIND(w) == VK_MEM && !(mems_[VI_A(w)].flags & VMF_VEC);
+    return VI_OP(w) == VOP_LD && VI_KIND(w) == VK_MEM && !(mems_[VI_A(w)].flags & (VMF_VEC | VMF_GATHER)) && !mem_is_view_[VI_A(w)];
   };
   auto starts = [&](uint64_t w) {
     const uint32_t op = VI_OP(w);
@@ -1947,6 +2031,31 @@ void Compiler::CompileArea(int a) {
   }
   EmitProgram();
   FinishProgram();
+  if (n_peel_ > 0) ReplicatePeeled();
+}
+
+// One copy of the finished program per index of the peeled dims; patches are in operand order, one per VMemDesc.
+void Compiler::ReplicatePeeled() {
+  int64_t count = 1;
+  for (int i = 0; i < n_peel_; ++i) count *= dims_[peel_dim_[i]].extent;
+  if (count > 4096) Fail("too many kept dims");
+  const Program base = *prog_;
+  k_->programs_.pop_back();
+  for (int64_t c = 0; c < count; ++c) {
+    k_->programs_.push_back(base);
+    Program &p = k_->programs_.back();
+    if (c > 0) p.fills.clear();
+    int64_t rest = c;
+    for (int i = 0; i < n_peel_; ++i) {
+      const int64_t ext = dims_[peel_dim_[i]].extent;
+      const int64_t idx = rest % ext;
+      rest /= ext;
+      for (size_t m = 0; m < p.patches.size(); ++m) {
+        p.patches[m].byte_offset += idx * peel_stride_[m][i];
+      }
+    }
+  }
+  prog_ = &k_->programs_.back();
 }
 
 
@@ -1968,8 +2077,10 @@ int Compiler::CubeMemIndex(int v) {
     const int od = d + R - n.rank;
     if (n.dims[d] != 1) {
       if (od < 0 || n.dims[d] != cube_out_->dim(od)) Fail("epilogue operand does not broadcast to the matmul result");
-      if (stride >= (1ll << 32)) Fail("stride above 2^32");
-      const uint32_t st = static_cast<uint32_t>(stride);
+      const int64_t walk = n.view != nullptr ? n.view->vstride_[d] : stride;
+      if (walk >= (1ll << 32) || walk < 0) Fail("stride above 2^32");
+      const uint32_t st = static_cast<uint32_t>(walk);
+      if (od == R - 1 && st != 1) Throw("DVM EXCEPTION. reason: a strided view whose innermost stride is not 1 is not supported by the gfx950 backend");
       if (od == R - 1) m.stride_n = st;
       else if (od == R - 2) m.stride_m = st;
       else if (od == R - 3) m.stride_b1 = st;
@@ -1981,6 +2092,7 @@ int Compiler::CubeMemIndex(int v) {
   p.word = static_cast<uint32_t>(sizeof(VCubeHeader) / 8 + n_mem_ * (sizeof(VCubeMem) / 8));
   p.op_id = n.addr_op;
   p.ws_slot = n.ws_slot;
+  p.byte_offset = n.view != nullptr ? n.view->view_base_ * static_cast<int64_t>(DTypeSize(n.dtype)) : 0;
   p.role = Program::kPatchPlain;
   prog_->patches.push_back(p);
   n.mem_idx = n_mem_++;
@@ -2069,6 +2181,7 @@ void Compiler::CompileCube(int a) {
   // operand addresses
   for (int which = 0; which < 2; ++which) {
     const ANode &x = which == 0 ? an : bn;
+    if (x.view != nullptr) Throw("DVM EXCEPTION. reason: a strided view as a matmul operand is not supported by the gfx950 backend");
     Program::Patch p;
     p.word = static_cast<uint32_t>((which == 0 ? offsetof(VCubeHeader, a_addr) : offsetof(VCubeHeader, b_addr)) / 8);
     p.op_id = x.addr_op;
@@ -2182,7 +2295,7 @@ void Compiler::DetectAttention() {
     if (m1->kind != kObjMatMul || m1->trans_a || !m1->trans_b || m1->in[2] != nullptr || uses[m1->id] != 1) continue;
     if (m1->type_id_ != m2->type_id_) continue;
     NDObject *q = m1->in[0], *kk = m1->in[1];
-    if (q->kind != kObjLoad || kk->kind != kObjLoad || v->kind != kObjLoad) continue;
+    if (q->kind != kObjLoad || kk->kind != kObjLoad || v->kind != kObjLoad || q->strided || kk->strided || v->strided) continue;
     const int r = q->rank();
     if (kk->rank() != r || v->rank() != r || r < 2) continue;
     bool ok = q->dim(r - 1) == DVM_ATTN_D && kk->dim(r - 1) == DVM_ATTN_D && v->dim(r - 1) == DVM_ATTN_D && kk->dim(r - 2) == v->dim(r - 2) &&
@@ -2267,8 +2380,9 @@ void VKernel::BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *all
       uint64_t addr = 0;
       if (pt.op_id >= 0) {
         addr = reinterpret_cast<uint64_t>(ops_[pt.op_id]->addr);
+        if (addr != 0) addr += static_cast<uint64_t>(pt.byte_offset);
       } else if (pt.ws_slot >= 0) {
-        addr = reinterpret_cast<uint64_t>(ws_base_) + ws_offsets_[pt.ws_slot];
+        addr = reinterpret_cast<uint64_t>(ws_base_) + ws_offsets_[pt.ws_slot] + static_cast<uint64_t>(pt.byte_offset);
       }
       if (addr == 0) Throw("a tensor address is missing at launch");
       p.blob.w[pt.word] = addr;

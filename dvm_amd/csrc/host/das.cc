@@ -186,7 +186,7 @@ std::string &VKernel::DisAssemble() {
       for (uint32_t i = 0; i < h->n_mem; ++i) {
         char buf[32];
         std::snprintf(buf, sizeof(buf), "0x%llx", static_cast<unsigned long long>(mems[i].addr));
-        os << "  m" << i << ": " << kMemTypes[mems[i].dtype] << " @" << buf << ((mems[i].flags & VMF_VEC) ? " vec" : " bcast")
+        os << "  m" << i << ": " << kMemTypes[mems[i].dtype] << " @" << buf << ((mems[i].flags & VMF_VEC) ? " vec" : (mems[i].flags & VMF_GATHER) ? " gather" : " bcast")
            << ((mems[i].flags & VMF_ALIGNED) ? " aligned" : "") << " k[";
         for (uint32_t j = 0; j < h->n_kdim; ++j) os << (j ? "," : "") << mems[i].kstride[j];
         os << "] r[";

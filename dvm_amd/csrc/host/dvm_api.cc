@@ -497,7 +497,14 @@ void Kernel::Clone(const Kernel &base, CloneHelper &helper) {
     c->scalar.ref = o->scalar.ref != nullptr ? helper.GetClone(o->scalar.ref) : nullptr;
     c->aux_ref = o->aux_ref != nullptr ? helper.GetClone(o->aux_ref) : nullptr;
     c->addr = o->addr;
-    if (o->kind == kObjLoad) c->shape_ref_ = c->aux_ref;
+    c->strided = o->strided;
+    c->view_offset = o->view_offset;
+    c->stride_ref = o->stride_ref != nullptr ? helper.GetClone(o->stride_ref) : nullptr;
+    c->full_shape_ref = o->full_shape_ref != nullptr ? helper.GetClone(o->full_shape_ref) : nullptr;
+    c->slice_start = o->slice_start != nullptr ? helper.GetClone(o->slice_start) : nullptr;
+    c->slice_end = o->slice_end != nullptr ? helper.GetClone(o->slice_end) : nullptr;
+    c->slice_step = o->slice_step != nullptr ? helper.GetClone(o->slice_step) : nullptr;
+    if (o->kind == kObjLoad && c->aux_ref != nullptr) c->shape_ref_ = c->aux_ref;
     kernel_->SetStage(o->stage);
     kernel_->Append(c);
     helper.SetClone(o, c);
@@ -518,16 +525,38 @@ NDObject *Kernel::Load(void *addr, IntArrayRef *shape, DataType type) {
   return kernel_->Append(o);
 }
 
+// Strided views (include/dvm.h:195-201 of the reference: Load with a stride list, SliceLoad, StridedSliceLoad,
+// Store with a stride list). The innermost stride has to be 1: the VM reads and writes runs of consecutive
+// elements; transposing views are rejected when the kernel is compiled.
 NDObject *Kernel::Load(void *addr, IntArrayRef *shape, IntArrayRef *stride, DataType type) {
-  if (stride != nullptr) Unsupported("a strided load");
-  return Load(addr, shape, type);
+  NDObject *o = Load(addr, shape, type);
+  if (stride != nullptr) {
+    o->strided = true;
+    o->stride_ref = stride;
+  }
+  return o;
 }
 
 NDObject *Kernel::GlobalAccess(void *, IntArrayRef *, DataType) { Unsupported("GlobalAccess"); }
 NDObject *Kernel::GatherLoad(void *, IntArrayRef *, NDObject *, int, DataType, GatherMode) { Unsupported("GatherLoad"); }
-NDObject *Kernel::SliceLoad(void *, IntArrayRef *, IntArrayRef *, IntArrayRef *, DataType) { Unsupported("SliceLoad"); }
-NDObject *Kernel::StridedSliceLoad(void *, IntArrayRef *, IntArrayRef *, IntArrayRef *, IntArrayRef *, DataType) {
-  Unsupported("StridedSliceLoad");
+NDObject *Kernel::SliceLoad(void *addr, IntArrayRef *shape, IntArrayRef *start, IntArrayRef *size, DataType type) {
+  NDObject *o = Load(addr, size, type);  // the value has the slice's shape
+  o->strided = true;
+  o->full_shape_ref = shape;
+  o->slice_start = start;
+  return o;
+}
+NDObject *Kernel::StridedSliceLoad(void *addr, IntArrayRef *shape, IntArrayRef *start, IntArrayRef *end, IntArrayRef *step,
+                                   DataType type) {
+  NDObject *o = Load(addr, shape, type);
+  o->strided = true;
+  o->full_shape_ref = shape;
+  o->slice_start = start;
+  o->slice_end = end;
+  o->slice_step = step;
+  o->aux_ref = nullptr;
+  o->shape_ref_ = &o->own_ref_;  // the value's shape is computed from start / end / step
+  return o;
 }
 NDObject *Kernel::MultiLoad(void *, IntArrayRef *, DataType, const Comm *) { Unsupported("MultiLoad"); }
 
@@ -540,8 +569,12 @@ NDObject *Kernel::Store(void *addr, NDObject *input) {
 }
 
 NDObject *Kernel::Store(void *addr, NDObject *input, IntArrayRef *stride) {
-  if (stride != nullptr) Unsupported("a strided store");
-  return Store(addr, input);
+  NDObject *o = Store(addr, input);
+  if (stride != nullptr) {
+    o->strided = true;
+    o->stride_ref = stride;
+  }
+  return o;
 }
 
 NDObject *Kernel::PadStore(void *, NDObject *, int64_t) { Unsupported("PadStore"); }

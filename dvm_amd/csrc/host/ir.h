@@ -66,6 +66,16 @@ class NDObject {
   ScalarOperand scalar;
   IntArrayRef *aux_ref = nullptr;  // reduce axes / broadcast target / reshape target / user shape of a load
   void *addr = nullptr;            // load / store address (may arrive later through a RelocEntry)
+  // A load or store that walks its buffer with strides of its own (Kernel::Load / Store with a stride list,
+  // SliceLoad, StridedSliceLoad; src/ops.h ViewLoad family): element strides per dim and the element offset of
+  // the first element, refreshed from the references below at every Normalize().
+  bool strided = false;
+  int64_t vstride_[10] = {0};
+  int64_t view_offset = 0;         // fixed part of the offset (set by the runner for views into a larger array)
+  int64_t view_base_ = 0;          // view_offset plus what a slice's start adds
+  IntArrayRef *stride_ref = nullptr;                 // explicit strides
+  IntArrayRef *full_shape_ref = nullptr;             // slices: shape of the whole tensor
+  IntArrayRef *slice_start = nullptr, *slice_end = nullptr, *slice_step = nullptr;  // end/step only for strided slices
   int id = -1;                     // position in the kernel's operator list
   int stage = 0;                   // sub-kernel group opened by Kernel::ParallelAdd / SequenceAdd
 
@@ -111,6 +121,7 @@ struct Program {
     uint32_t word;   // 64-bit word of the blob that receives the address
     int op_id;       // load/store node whose address goes there, or -1
     int ws_slot;     // or the workspace slot
+    int64_t byte_offset = 0;  // added to the operator's address (strided views start inside their buffer)
     uint8_t role;    // kPatchVecMem: a VMemDesc (alignment flag follows the address); kPatchCubeOperand:
                      // a matmul operand (the fast path needs 16-byte alignment); kPatchPlain: nothing else;
                      // kPatchAligned16: an operand of the fused attention kernel, which only has 128-bit accesses

@@ -161,7 +161,7 @@ typedef struct {
 // A memory operand: base address plus element strides against the kept list
 // and the reduced list (position 0 = fastest varying). The stride of the
 // innermost domain axis is 0 (operand broadcast along it: one element is
-// loaded and replicated) or 1 (E consecutive elements).
+// loaded and replicated), 1 (E consecutive elements) or, with VMF_GATHER, any.
 typedef struct {
   uint64_t addr;
   uint32_t dtype;                  // VDT_*
@@ -169,7 +169,9 @@ typedef struct {
   uint32_t kstride[DVM_VEC_MAXR];
   uint32_t rstride[DVM_VEC_MAXR];
 } VMemDesc;
-enum { VMF_VEC = 1 /* innermost stride 1 */, VMF_ALIGNED = 2 /* every E-group starts 16-byte aligned */ };
+// VMF_GATHER: the innermost stride is neither 0 nor 1 (a transposing or element-skipping view); it sits in
+// flags[31:8] and in the stride entry of the innermost axis, and the operand is accessed element by element.
+enum { VMF_VEC = 1 /* innermost stride 1 */, VMF_ALIGNED = 2 /* every E-group starts 16-byte aligned */, VMF_GATHER = 4 };
 
 typedef struct {
   uint32_t entry;        // VE_VECTOR

@@ -79,6 +79,45 @@ class Tester(PyKernel):
         self.input(op, shape_arr)
         return op
 
+    # views: the array bound to the load is the whole buffer, the load reads part of it
+    def view_load(self, shape, stride, arr_dtype, offset=0, real_dtype=None):
+        if not isinstance(arr_dtype, np.ndarray):
+            return PyKernel.view_load(self, shape, stride, _normalize_dtype(arr_dtype))  # dynamic shape
+        arr, dtype_id, _ = self._prepare_array_input(arr_dtype, real_dtype)
+        op = PyKernel.view_load(self, shape, stride, dtype_id)
+        self.input(op, arr, offset)
+        return op
+
+    def slice_load(self, shape_arr, start, size, dtype=None):
+        if not isinstance(shape_arr, np.ndarray):
+            return PyKernel.slice_load(self, shape_arr, start, size, _normalize_dtype(dtype))
+        arr, dtype_id, shape = self._prepare_array_input(shape_arr, dtype)
+        op = PyKernel.slice_load(self, shape, start, size, dtype_id)
+        self.input(op, arr)
+        return op
+
+    def stridedslice_load(self, shape_arr, start, end, step, dtype=None):
+        if not isinstance(shape_arr, np.ndarray):
+            return PyKernel.stridedslice_load(self, shape_arr, start, end, step, _normalize_dtype(dtype))
+        arr, dtype_id, shape = self._prepare_array_input(shape_arr, dtype)
+        op = PyKernel.stridedslice_load(self, shape, start, end, step, dtype_id)
+        self.input(op, arr)
+        return op
+
+    def view_store_expect(self, x, stride, e, eps=None):
+        """Stores x through `stride` into a buffer shaped like e (zeros where nothing is written) and expects e."""
+        e = np.asarray(e)
+        op = PyKernel.view_store(self, x, stride, e.size)
+        self._view_shape = getattr(self, "_view_shape", {})
+        self._view_shape[op._h] = tuple(e.shape)
+        self.expects.append([op, e, eps])
+        return op
+
+    def output(self, store, shape=None):
+        if shape is None:
+            shape = getattr(self, "_view_shape", {}).get(store._h)
+        return PyKernel.output(self, store, shape)
+
     def cast(self, x, dtype):
         return PyKernel.cast(self, x, _normalize_dtype(dtype))
 

@@ -61,6 +61,15 @@ dvm_obj *dvm_rt_reduce(dvm_rt *rt, int reduce_type, dvm_obj *x, dvm_shape *dims,
 dvm_obj *dvm_rt_copy(dvm_rt *rt, dvm_obj *x);
 dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int trans_b, dvm_obj *bias);
 int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store);
+// Strided views (Kernel::Load / Store with a stride list, SliceLoad, StridedSliceLoad: include/dvm.h:195-201, 214 of the
+// reference; KernelPy view_load / slice_load / stridedslice_load, include/dvm_py.h). Strides are in elements, the
+// innermost one has to be 1. A view store writes into a zero-initialised buffer of extent_elems elements;
+// dvm_obj_set_view_offset moves the first element of a view that many elements into its buffer.
+dvm_obj *dvm_rt_view_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *stride, int dtype);
+dvm_obj *dvm_rt_slice_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *start, dvm_shape *size, int dtype);
+dvm_obj *dvm_rt_stridedslice_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *start, dvm_shape *end, dvm_shape *step, int dtype);
+dvm_obj *dvm_rt_view_store(dvm_rt *rt, dvm_obj *x, dvm_shape *stride, size_t extent_elems);
+int dvm_obj_set_view_offset(dvm_obj *io, long long elems);
 // Group markers of "seq" and "parallel" kernels (KernelPy::SequenceAdd / ParallelAdd, include/dvm_py.h:369-371; Kernel::SequenceAdd /
 // ParallelAdd, include/dvm.h:250-251): operators built after the call belong to the next sub-kernel group.
 int dvm_rt_seq_add(dvm_rt *rt, int ktype, unsigned flags);

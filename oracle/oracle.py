@@ -259,6 +259,40 @@ class OracleKernel:
             v = a.astype(np.float32)
         return OVal(v, t, is_load=True)
 
+    # Views (include/dvm.h:294,312,317,339 of the reference): a load reads element i0..in of its shape at
+    # offset + sum(i_d * stride_d) of the flat buffer; slice loads are the NumPy basic slices of the same
+    # bounds (negative bounds count from the end, bounds past the end are clipped); a strided store writes
+    # element i0..in of its value at sum(i_d * stride_d) of a zero-filled flat buffer.
+    def view_load(self, shape, stride, array, offset=0, real_dtype=None):
+        flat = np.ascontiguousarray(array).reshape(-1)
+        idx = np.full(tuple(shape), int(offset), np.int64)
+        for d, (n, st) in enumerate(zip(shape, stride)):
+            ext = [1] * len(shape)
+            ext[d] = n
+            idx = idx + (np.arange(n, dtype=np.int64) * int(st)).reshape(ext)
+        return self.load(flat[idx], real_dtype)
+
+    def slice_load(self, array, start, size, dtype=None):
+        a = np.asarray(array)
+        return self.load(a[tuple(slice(s, s + n) for s, n in zip(start, size))], dtype)
+
+    def stridedslice_load(self, array, start, end, step, dtype=None):
+        a = np.asarray(array)
+        return self.load(a[tuple(slice(s, e, p) for s, e, p in zip(start, end, step))], dtype)
+
+    def view_store_expect(self, x, stride, e, eps=None):
+        e = np.asarray(e)
+        out = np.zeros(e.size, x.a.dtype)
+        idx = np.zeros(x.a.shape, np.int64)
+        for d, (n, st) in enumerate(zip(x.a.shape, stride)):
+            ext = [1] * x.a.ndim
+            ext[d] = n
+            idx = idx + (np.arange(n, dtype=np.int64) * int(st)).reshape(ext)
+        out[idx.reshape(-1)] = x.a.reshape(-1)
+        v = OVal(out.reshape(e.shape), x.t)
+        self.stores.append(v)
+        return v
+
     def full(self, scalar, shape, dtype):
         t = _tid(dtype)
         if t == BOOL:

@@ -383,3 +383,49 @@ def test_clone_is_independent_of_its_base():
     t2.codegen()
     assert out2.shape() == (64, 1) and out.shape() == (1, 512)
     assert "reduce-x" in t2.das() and "reduce-y" in t.das()
+
+
+def test_strided_views_in_das_mode():
+    # include/dvm.h:294,312,317,339 of the reference: loads and stores through stride lists, slice loads
+    def dense(shape):
+        st = [1] * len(shape)
+        for i in range(len(shape) - 1, 0, -1):
+            st[i - 1] = st[i] * shape[i]
+        return st
+    a = np.zeros([30, 1000], np.float32)
+    # a row-major slice keeps the vector path; the operand strides are the buffer's, not the value's
+    t, das = _das(lambda t: t.store(t.add(t.view_load([20, 500], [1000, 1], a), 0.1)))
+    assert das.count("== sub-kernel") == 1 and "k[1,1000]" in das and " gather" not in das
+    # neighbouring axes the view holds densely still merge: [4, 2, 64, 64] out of [4, 2, 64, 96] is two dims
+    b = np.zeros([4, 2, 64, 96], np.float32)
+    t, das = _das(lambda t: t.store(t.add(t.view_load([4, 2, 64, 64], dense([4, 2, 64, 96]), b), 0.1)))
+    assert "kdims: 8 512 " in das
+    # an element-skipping innermost stride goes element by element
+    c = np.zeros([100, 2048], np.float32)
+    t, das = _das(lambda t: t.store(t.add(t.view_load([100, 200], [2048, 10], c), 0.1)))
+    assert " gather" in das
+    # six dims that cannot merge: four run inside the program, the two outermost become launches
+    d = np.zeros([4, 4, 4, 5, 6, 16], np.float32)
+    t, das = _das(lambda t: t.store(t.add(t.view_load([3, 2, 3, 4, 5, 12], dense(list(d.shape)), d), 0.1)))
+    assert das.count("== sub-kernel") == 6
+    # slices: negative bounds count from the end, an end past the axis stops at the axis
+    e = np.zeros([32, 7, 7], np.float32)
+    t = Tester("vector", run_mode="das")
+    x = t.stridedslice_load(e, (-30, 0, 0), (100, 7, 7), (1, 1, 1))
+    s = t.store(x)
+    t.codegen()
+    assert s.shape() == (30, 7, 7)
+    t = Tester("vector", run_mode="das")
+    t.store(t.slice_load(e, (3, 0, 0), (30, 7, 7)))
+    with pytest.raises(RuntimeError, match="slice reaches outside"):
+        t.codegen()
+    # a value stored through strides and used by a later launch is not read back through them
+    f = np.zeros([4, 1, 512], np.float32)
+    g = np.zeros([4, 8, 512], np.float32)
+
+    def two(t):
+        x0 = t.add(t.load(f), 0.1)
+        t.view_store_expect(x0, [1024, 512, 1], np.zeros([6, 2, 512], np.float32))
+        t.store(t.add(x0, t.load(g)))
+    t, das = _das(two, "split")
+    assert t.workspace_bytes() >= f.nbytes or das.count("== sub-kernel") == 1
