@@ -462,7 +462,7 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
   typedef typename SlabVec<SL>::type Slabs;
   const uint32_t *code32 = prog32 + 2 * h.code_off;
   static_assert(NTEMP == 4, "temporaries are named registers");
-  Slabs t0 = 0.0f, t1 = 0.0f, t2 = 0.0f, t3 = 0.0f;
+  Slabs t0, t1, t2, t3;  // never read before written (the emitter parks a value before it names the register)
   uint32_t mask = 0;
   uint32_t pc = 0;
   while (true) {

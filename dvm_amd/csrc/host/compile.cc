@@ -1549,8 +1549,14 @@ void Compiler::ComputeInto(int v) {
         reversed = true;
       } else {
         EmitValue(b);
-        SaveAcc(b);
-        EmitValue(a);
+        if (SimpleOperand(a)) {
+          // a was computed and parked on the way to b (b is a function of a, as in x / (exp(-x) + 1))
+          std::swap(a, b);
+          reversed = true;
+        } else {
+          SaveAcc(b);
+          EmitValue(a);
+        }
       }
       ConsumeUse(a);
       BeforeOverwrite();
