@@ -58,6 +58,11 @@ def _load():
         "dvm_rt_stridedslice_load": (vp, [vp, vp, vp, vp, vp, ci]),
         "dvm_rt_view_store": (vp, [vp, vp, vp, cs]),
         "dvm_obj_set_view_offset": (ci, [vp, ctypes.c_longlong]),
+        "dvm_rt_permute": (vp, [vp, vp, vp]),
+        "dvm_rt_slice": (vp, [vp, vp, vp, vp]),
+        "dvm_rt_slice_dim": (vp, [vp, vp, ci, vp, vp]),
+        "dvm_rt_split": (ci, [vp, vp, ci, ctypes.c_longlong, cs, ctypes.POINTER(vp)]),
+        "dvm_rt_concat": (vp, [vp, ctypes.POINTER(vp), cs, ci]),
         "dvm_rt_clone": (ci, [vp, vp, ctypes.POINTER(ci), ctypes.POINTER(vp), cs, ctypes.POINTER(vp)]),
         "dvm_rt_seq_add": (ci, [vp, ci, ctypes.c_uint]),
         "dvm_rt_parallel_add": (ci, [vp, ci, ctypes.c_uint, cs]),
@@ -269,6 +274,32 @@ class Kernel:
     def view_store(self, obj, stride, extent):
         """Stores obj through element strides into a zero-initialised buffer of `extent` elements."""
         return self._wrap(_lib.dvm_rt_view_store(self._rt, obj._h, self._shape_ref(stride)._h, int(extent)))
+
+    # -- views of values (include/dvm_py.h:163-189 of the reference): nothing is copied --
+    def permute(self, input, dims):
+        return self._wrap(_lib.dvm_rt_permute(self._rt, input._h, self._shape_ref(dims)._h))
+
+    def slice(self, input, start, size):
+        return self._wrap(_lib.dvm_rt_slice(self._rt, input._h, self._shape_ref(start)._h, self._shape_ref(size)._h))
+
+    def _int_scalar(self, v):
+        if isinstance(v, ScalarRef):
+            return v
+        ref = self.scalar(DataType.int32)
+        ref.update(int(v))
+        return ref
+
+    def slice_dim(self, input, dim, begin, end):
+        return self._wrap(_lib.dvm_rt_slice_dim(self._rt, input._h, int(dim), self._int_scalar(begin)._h, self._int_scalar(end)._h))
+
+    def concat(self, inputs, dim):
+        arr = (ctypes.c_void_p * len(inputs))(*[x._h for x in inputs])
+        return self._wrap(_lib.dvm_rt_concat(self._rt, arr, len(inputs), int(dim)))
+
+    def split(self, input, dim, split_size, split_num):
+        out = (ctypes.c_void_p * int(split_num))()
+        _check(_lib.dvm_rt_split(self._rt, input._h, int(dim), int(split_size), int(split_num), out))
+        return tuple(self._wrap(out[i]) for i in range(int(split_num)))
 
     # -- sub-kernel groups of "seq" / "parallel" kernels (include/dvm_py.h:369-371) --
     def seq_add(self, ktype, flags=0):

@@ -519,6 +519,38 @@ dvm_obj *dvm_rt_view_store(dvm_rt *rt, dvm_obj *x, dvm_shape *stride, size_t ext
       static_cast<dvm_obj *>(nullptr));
 }
 
+dvm_obj *dvm_rt_permute(dvm_rt *rt, dvm_obj *x, dvm_shape *dims) {
+  return Guard([&]() { return Handle(rt->kernel.Permute(Obj(x), &dims->ref)); }, static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_slice(dvm_rt *rt, dvm_obj *x, dvm_shape *start, dvm_shape *size) {
+  return Guard([&]() { return Handle(rt->kernel.Slice(Obj(x), &start->ref, &size->ref)); }, static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_slice_dim(dvm_rt *rt, dvm_obj *x, int dim, dvm_scalar *begin, dvm_scalar *end) {
+  return Guard([&]() { return Handle(rt->kernel.Slice(Obj(x), dim, &begin->ref, &end->ref)); }, static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_concat(dvm_rt *rt, dvm_obj **inputs, size_t n, int dim) {
+  return Guard(
+      [&]() {
+        std::vector<NDObject *> objs;
+        for (size_t i = 0; i < n; ++i) objs.push_back(Obj(inputs[i]));
+        return Handle(rt->kernel.Concat(objs.data(), objs.size(), dim));
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+int dvm_rt_split(dvm_rt *rt, dvm_obj *x, int dim, long long chunk, size_t num, dvm_obj **out) {
+  return Guard(
+      [&]() {
+        NDObject **parts = rt->kernel.Split(Obj(x), dim, chunk, num);
+        for (size_t i = 0; i < num; ++i) out[i] = Handle(parts[i]);
+        return 0;
+      },
+      -1);
+}
+
 int dvm_obj_set_view_offset(dvm_obj *io, long long elems) {
   Obj(io)->view_offset = elems;
   return 0;

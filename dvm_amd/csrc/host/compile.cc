@@ -178,7 +178,110 @@ void VKernel::Normalize() {
         o->own_ref_.size = n;
         break;
       }
+      case kObjConcatPart:
+        o->SetShape(o->in[0]->shape_ref_->data, o->in[0]->shape_ref_->size);
+        break;
+      case kObjConcat: {
+        const NDObject *first = o->parts[0];
+        const size_t r = first->shape_ref_->size;
+        int64_t dim = o->slice_dim;
+        if (dim < 0) dim += static_cast<int64_t>(r);
+        if (dim < 0 || dim >= static_cast<int64_t>(r)) Throw("concat dim out of range");
+        for (size_t i = 0; i < r; ++i) o->shape_[i] = first->shape_ref_->data[i];
+        o->shape_[dim] = 0;
+        for (const NDObject *p : o->parts) {
+          if (p->shape_ref_->size != r) Throw("concat inputs differ in rank");
+          for (size_t i = 0; i < r; ++i)
+            if (static_cast<int64_t>(i) != dim && p->shape_ref_->data[i] != first->shape_ref_->data[i]) Throw("concat inputs differ outside the concat dim");
+          o->shape_[dim] += p->shape_ref_->data[dim];
+        }
+        o->own_ref_.size = r;
+        int64_t dense[kMaxRank], acc = 1;
+        for (size_t i = r; i-- > 0;) {
+          dense[i] = acc;
+          acc *= o->shape_[i];
+        }
+        int64_t at = 0;
+        for (NDObject *p : o->parts) {  // where each part lands: the buffer's strides, its offset along the dim
+          p->strided = true;
+          for (size_t i = 0; i < r; ++i) p->vstride_[i] = dense[i];
+          p->view_base_ = at * dense[dim];
+          at += p->shape_ref_->data[dim];
+        }
+        break;
+      }
+      case kObjPermute:
+      case kObjSlice: {
+        // A view of the input's memory: element strides and offset of the input (its own when it is a view or a
+        // strided load, those of a dense row-major tensor otherwise), reordered or moved by the slice's start.
+        const NDObject *x = o->in[0];
+        const size_t r = x->shape_ref_->size;
+        int64_t xs[kMaxRank];
+        if (x->strided && x->kind != kObjStore) {
+          for (size_t i = 0; i < r; ++i) xs[i] = x->vstride_[i];
+          o->view_base_ = x->view_base_;
+        } else {
+          int64_t dense = 1;
+          for (size_t i = r; i-- > 0;) {
+            xs[i] = dense;
+            dense *= x->shape_ref_->data[i];
+          }
+          o->view_base_ = 0;
+        }
+        o->strided = true;
+        if (o->kind == kObjPermute) {
+          if (o->aux_ref->size != r) Throw("permutation does not match the tensor rank");
+          bool seen[kMaxRank] = {false};
+          for (size_t i = 0; i < r; ++i) {
+            int64_t d = o->aux_ref->data[i];
+            if (d < 0) d += static_cast<int64_t>(r);
+            if (d < 0 || d >= static_cast<int64_t>(r) || seen[d]) Throw("permutation names a dim twice or out of range");
+            seen[d] = true;
+            o->shape_[i] = x->shape_ref_->data[d];
+            o->vstride_[i] = xs[d];
+          }
+        } else if (o->slice_dim < 0 && o->slice_start != nullptr) {
+          if (o->slice_start->size != r || o->aux_ref->size != r) Throw("slice lists do not match the tensor rank");
+          for (size_t i = 0; i < r; ++i) {
+            const int64_t ext = x->shape_ref_->data[i];
+            int64_t st = o->slice_start->data[i];
+            if (st < 0) st += ext;
+            const int64_t n = o->aux_ref->data[i];
+            if (st < 0 || n < 0 || st + n > ext) Throw("slice reaches outside the tensor");
+            o->shape_[i] = n;
+            o->vstride_[i] = xs[i];
+            o->view_base_ += st * xs[i];
+          }
+        } else {
+          int64_t dim = o->slice_dim;
+          if (dim < 0) dim += static_cast<int64_t>(r);
+          if (dim < 0 || dim >= static_cast<int64_t>(r)) Throw("slice dim out of range");
+          auto as_int = [](const ScalarRef *s) -> int64_t {
+            switch (s->type) {
+              case kInt32: return s->i32;
+              case kInt64: return s->i64;
+              case kFloat32: return static_cast<int64_t>(s->f32);
+              default: Throw("slice bounds have to be integers");
+            }
+            return 0;
+          };
+          const int64_t ext = x->shape_ref_->data[dim];
+          const int64_t b = bound(o->dim_begin_ref != nullptr ? as_int(o->dim_begin_ref) : o->dim_begin, ext);
+          const int64_t e = bound(o->dim_end_ref != nullptr ? as_int(o->dim_end_ref) : o->dim_end, ext);
+          for (size_t i = 0; i < r; ++i) {
+            o->shape_[i] = x->shape_ref_->data[i];
+            o->vstride_[i] = xs[i];
+          }
+          o->shape_[dim] = e > b ? e - b : 0;
+          o->view_base_ += b * xs[dim];
+        }
+        o->own_ref_.size = r;
+        break;
+      }
       case kObjReshape: {
+        if (o->in[0]->strided && o->in[0]->kind != kObjStore && o->in[0]->kind != kObjLoad) {
+          Throw("DVM EXCEPTION. reason: a reshape of a permuted or sliced value needs a Copy in between on the gfx950 backend");
+        }
         const size_t r = o->aux_ref->size;
         if (r > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
         int64_t known = 1;
@@ -315,6 +418,7 @@ bool IsPointwiseKind(ObjKind k) {
     case kObjCopy:
     case kObjBroadcast:
     case kObjStore:
+    case kObjConcatPart:
       return true;
     default:
       return false;
@@ -427,14 +531,18 @@ class Compiler {
       if (!live_[i]) continue;
       for (int j = 0; j < o->nin; ++j)
         if (o->in[j] != nullptr) live_[o->in[j]->id] = 1;
+      for (NDObject *p : o->parts) live_[p->id] = 1;
     }
   }
 
   // ---------- partition into sub-kernels ----------
   static bool IsLeaf(const NDObject *o) { return o->kind == kObjLoad || o->kind == kObjBroadcastS; }
+  static bool IsStoreLike(const NDObject *o) { return o->kind == kObjStore || o->kind == kObjConcatPart; }
 
   // A view: reshape of a materialised value (or of a load) that is read through its new shape.
-  bool IsView(const NDObject *o) const { return o->kind == kObjReshape && !IsSqueezeReshape(o); }
+  bool IsView(const NDObject *o) const {
+    return (o->kind == kObjReshape && !IsSqueezeReshape(o)) || o->kind == kObjPermute || o->kind == kObjSlice;
+  }
 
   // The operator whose buffer a view chain ends at.
   const NDObject *ViewRoot(const NDObject *o) const {
@@ -500,10 +608,10 @@ class Compiler {
     const AreaInfo &ai = areas_[a];
     if (ai.stage != o->stage) return false;
     // a store goes where the value it stores is computed (an operator's own output is never a reason to cut)
-    if (o->kind == kObjStore && ai.attn < 0 && !ai.cube && area_[o->in[0]->id] == a) return true;
+    if (IsStoreLike(o) && ai.attn < 0 && !ai.cube && area_[o->in[0]->id] == a) return true;
     if (o->kind == kObjReduce && LevelIn(a, o) < 8 && ai.red_at_level[LevelIn(a, o)] >= 2) return false;
     if (o->kind == kObjMatMul) return false;
-    if (ai.n_ops >= kMaxAreaOps && o->kind != kObjStore) return false;  // long graphs are cut into several launches
+    if (ai.n_ops >= kMaxAreaOps && !IsStoreLike(o)) return false;  // long graphs are cut into several launches
     if (ai.attn >= 0) return o->kind == kObjStore && o->in[0] == attn_groups_[ai.attn].m2;
     if (ai.cube) {
       if (!IsPointwiseKind(o->kind)) return false;
@@ -569,6 +677,12 @@ class Compiler {
       NDObject *o = k_->ops_[i];
       if (!live_[i] || IsLeaf(o)) continue;
       if (IsView(o)) continue;  // read through by its consumers
+      if (o->kind == kObjConcat) {  // complete once the last of its parts has run; never computed itself
+        int a = 0;
+        for (const NDObject *p : o->parts) a = std::max(a, area_[p->id]);
+        area_[i] = a;
+        continue;
+      }
       const int c = find(i);
       if (comp_base[c] < 0) comp_base[c] = static_cast<int>(areas_.size());
       if (attn_of_[i] >= 0) {
@@ -593,11 +707,11 @@ class Compiler {
           if (IsLeaf(v)) continue;
           cut = true;
         }
-        if (o->kind == kObjMatMul) cut = true;
-        if (!fuse && v->kind == kObjReduce && o->kind != kObjStore) cut = true;  // the reference's rule: a reduce ends its sub-kernel
+        if (o->kind == kObjMatMul || v->kind == kObjConcat) cut = true;
+        if (!fuse && v->kind == kObjReduce && !IsStoreLike(o)) cut = true;  // the reference's rule: a reduce ends its sub-kernel
         a = std::max(a, area_[v->id] + (cut ? 1 : 0));
       }
-      if (o->kind == kObjMatMul || (mode_ >= 3 && o->kind != kObjStore)) a = std::max(a, static_cast<int>(areas_.size()));
+      if (o->kind == kObjMatMul || (mode_ >= 3 && !IsStoreLike(o))) a = std::max(a, static_cast<int>(areas_.size()));
       while (!CanJoin(a, o)) ++a;
       area_[i] = a;
       Join(a, o);
@@ -626,6 +740,8 @@ class Compiler {
         if (IsView(v) || (user_area != -2 && area_[root->id] != user_area)) mat_[root->id] = 1;
       }
     }
+    for (int i = 0; i < n_; ++i)
+      if (live_[i] && k_->ops_[i]->kind == kObjConcat) mat_[i] = 1;  // its parts need the buffer whoever reads it
     for (int i = 0; i < n_; ++i) {
       if (!mat_[i]) continue;
       NDObject *o = k_->ops_[i];
@@ -697,9 +813,11 @@ class Compiler {
     } else {
       idx = AddNode(AK_MEM, v, v->type_id_, v->shape_ref_->data, v->rank());
       const NDObject *root = ViewRoot(v);
+      // a permuted or sliced value carries the strides of the whole chain down to the root's memory
+      if (v->kind == kObjPermute || v->kind == kObjSlice) nodes_[idx].view = v;
       if (root->kind == kObjLoad) {
         nodes_[idx].addr_op = root->id;
-        if (root->strided) {
+        if (root->strided && nodes_[idx].view == nullptr) {
           if (root != v) Throw("DVM EXCEPTION. reason: a reshape of a strided load is not supported by the gfx950 backend");
           nodes_[idx].view = root;
         }
@@ -819,6 +937,7 @@ void Compiler::BuildNodes(int a) {
   for (int i = 0; i < n_; ++i) {
     if (area_[i] != a) continue;
     NDObject *o = k_->ops_[i];
+    if (o->kind == kObjConcat) continue;  // a buffer its parts fill, nothing to compute
     int in_idx[3] = {-1, -1, -1};
     for (int j = 0; j < o->nin; ++j) {
       NDObject *v = o->in[j];
@@ -843,7 +962,7 @@ void Compiler::BuildNodes(int a) {
       }
       kind = nothing ? AK_ALIAS : AK_REDUCE;
     }
-    if (o->kind == kObjStore) kind = AK_OUT;
+    if (IsStoreLike(o)) kind = AK_OUT;
     if (o->kind == kObjCast) {
       // widening conversions do not change the register value
       const DataType s = o->in[0]->type_id_, d = o->type_id_;
@@ -855,8 +974,13 @@ void Compiler::BuildNodes(int a) {
     n.nin = o->nin;
     for (int j = 0; j < 3; ++j) n.in[j] = in_idx[j];
     if (kind == AK_OUT) {
-      n.addr_op = i;
-      if (o->strided) n.view = o;
+      if (o->kind == kObjConcatPart) {
+        n.ws_slot = ws_slot_[o->cat->id];
+        n.view = o;
+      } else {
+        n.addr_op = i;
+        if (o->strided) n.view = o;
+      }
     }
     node_of_[i] = idx;
     // a value later sub-kernels read and that the user does not store: write it to workspace
@@ -950,6 +1074,34 @@ void Compiler::UnifyAxes() {
       if (x.rank != f.rank) Fail("reduces of different rank in one sub-kernel");
       for (int d = 0; d < x.rank; ++d)
         if (x.dims[d] != 1 && x.dims[d] == f.dims[d]) Union(Var(nodes_[i].in[0], d), Var(first, d));
+    }
+  }
+  // Outputs that no operator relates to the first one (consumers of two different views of one buffer, each
+  // with its own store) walk the same index space too: unified with it dim by dim from the right.
+  {
+    std::vector<int> comp(nn_);
+    for (int i = 0; i < nn_; ++i) comp[i] = i;
+    auto find = [&](int v) {
+      while (comp[v] != v) v = comp[v] = comp[comp[v]];
+      return v;
+    };
+    for (int i = 0; i < nn_; ++i)
+      for (int j = 0; j < nodes_[i].nin; ++j)
+        if (nodes_[i].in[j] >= 0) comp[find(i)] = find(nodes_[i].in[j]);
+    int anchor = -1;
+    for (int i = 0; i < nn_; ++i) {
+      if (nodes_[i].kind != AK_OUT) continue;
+      if (anchor < 0) {
+        anchor = i;
+        continue;
+      }
+      if (find(i) == find(anchor)) continue;
+      const ANode &o = nodes_[i], &f = nodes_[anchor];
+      for (int d = 0; d < o.rank; ++d) {
+        const int fd = d + f.rank - o.rank;
+        if (fd >= 0 && o.dims[d] != 1 && o.dims[d] == f.dims[fd]) Union(Var(i, d), Var(anchor, fd));
+      }
+      comp[find(i)] = find(anchor);
     }
   }
   // classes with extent > 1 become domain axes

@@ -81,6 +81,10 @@ std::string &VKernel::DumpGraph(bool ref_shapes) {
       case kObjBroadcastS: os << "BroadcastS"; break;
       case kObjReduce: os << "Reduce" << kReduceNames[o->op] << (o->keepdims ? "(keepdims)" : ""); break;
       case kObjReshape: os << "Reshape"; break;
+      case kObjPermute: os << "Permute"; break;
+      case kObjSlice: os << "Slice"; break;
+      case kObjConcatPart: os << "ConcatPart"; break;
+      case kObjConcat: os << "Concat"; break;
       case kObjCopy: os << "Copy"; break;
       case kObjMatMul: os << "MatMul" << (o->trans_a ? "T" : "N") << (o->trans_b ? "T" : "N"); break;
     }

@@ -504,6 +504,16 @@ void Kernel::Clone(const Kernel &base, CloneHelper &helper) {
     c->slice_start = o->slice_start != nullptr ? helper.GetClone(o->slice_start) : nullptr;
     c->slice_end = o->slice_end != nullptr ? helper.GetClone(o->slice_end) : nullptr;
     c->slice_step = o->slice_step != nullptr ? helper.GetClone(o->slice_step) : nullptr;
+    c->slice_dim = o->slice_dim;
+    for (NDObject *p : o->parts) {  // parts precede their Concat, so their clones exist
+      NDObject *pc = helper.GetClone(p);
+      c->parts.push_back(pc);
+      pc->cat = c;
+    }
+    c->dim_begin_ref = o->dim_begin_ref != nullptr ? helper.GetClone(o->dim_begin_ref) : nullptr;
+    c->dim_end_ref = o->dim_end_ref != nullptr ? helper.GetClone(o->dim_end_ref) : nullptr;
+    c->dim_begin = o->dim_begin;
+    c->dim_end = o->dim_end;
     if (o->kind == kObjLoad && c->aux_ref != nullptr) c->shape_ref_ = c->aux_ref;
     kernel_->SetStage(o->stage);
     kernel_->Append(c);
@@ -696,11 +706,54 @@ NDObject *Kernel::MatMul(NDObject *lhs, NDObject *rhs, bool trans_a, bool trans_
   return o;
 }
 
-NDObject *Kernel::Permute(NDObject *, IntArrayRef *) { Unsupported("Permute"); }
-NDObject *Kernel::Slice(NDObject *, IntArrayRef *, IntArrayRef *) { Unsupported("Slice"); }
-NDObject *Kernel::Slice(NDObject *, int, ScalarRef *, ScalarRef *) { Unsupported("Slice"); }
-NDObject *Kernel::Concat(NDObject **, size_t, int) { Unsupported("Concat"); }
-NDObject **Kernel::Split(NDObject *, int, int64_t, size_t) { Unsupported("Split"); }
+// Permute, Slice and Split are views: the input is kept (or written) in memory in its own layout and the
+// consumers read it through the view's strides and offset; nothing is copied.
+NDObject *Kernel::Permute(NDObject *input, IntArrayRef *dims) {
+  NDObject *o = Builder(kernel_).New(kObjPermute, input->type_id_, input);
+  o->aux_ref = dims;
+  return o;
+}
+NDObject *Kernel::Slice(NDObject *input, IntArrayRef *start, IntArrayRef *size) {
+  NDObject *o = Builder(kernel_).New(kObjSlice, input->type_id_, input);
+  o->slice_start = start;
+  o->aux_ref = size;
+  return o;
+}
+NDObject *Kernel::Slice(NDObject *input, int dim, ScalarRef *begin, ScalarRef *end) {
+  NDObject *o = Builder(kernel_).New(kObjSlice, input->type_id_, input);
+  o->slice_dim = dim;
+  o->dim_begin_ref = begin;
+  o->dim_end_ref = end;
+  return o;
+}
+// Concat: every input is written into its place in one buffer by the launch that computes it, the consumers read
+// that buffer.
+NDObject *Kernel::Concat(NDObject **inputs, size_t input_num, int dim) {
+  if (input_num == 0) Throw("concat needs at least one input");
+  Builder b(kernel_);
+  std::vector<NDObject *> parts;
+  for (size_t i = 0; i < input_num; ++i) {
+    if (inputs[i]->type_id_ != inputs[0]->type_id_) Throw("concat inputs differ in type");
+    parts.push_back(b.New(kObjConcatPart, inputs[i]->type_id_, inputs[i]));
+  }
+  NDObject *o = b.New(kObjConcat, inputs[0]->type_id_);
+  o->slice_dim = dim;
+  o->parts = parts;
+  for (NDObject *p : parts) p->cat = o;
+  return o;
+}
+NDObject **Kernel::Split(NDObject *input, int dim, int64_t split_size, size_t split_num) {
+  if (split_size <= 0 || split_num == 0) Throw("split needs a positive chunk size and count");
+  NDObject **out = kernel_->NewObjectArray(split_num);
+  for (size_t j = 0; j < split_num; ++j) {
+    NDObject *o = Builder(kernel_).New(kObjSlice, input->type_id_, input);
+    o->slice_dim = dim;
+    o->dim_begin = static_cast<int64_t>(j) * split_size;
+    o->dim_end = static_cast<int64_t>(j + 1) * split_size;  // clipped to the extent: the last chunk may be smaller
+    out[j] = o;
+  }
+  return out;
+}
 template <typename T>
 NDObject *Kernel::OneHot(NDObject *, IntArrayRef *, int, T, T) {
   Unsupported("OneHot");

@@ -37,6 +37,10 @@ enum ObjKind : uint8_t {
   kObjReshape,
   kObjCopy,
   kObjMatMul,
+  kObjPermute,   // view: dims reordered (aux_ref = source dim of every result dim)
+  kObjSlice,     // view: a box of the input (slice_start + aux_ref sizes, or one dim with begin / end)
+  kObjConcatPart,  // writes its input into its place in the buffer of a Concat (a store through strides)
+  kObjConcat,      // the buffer the parts wrote, read by the consumers like any value kept in memory
 };
 
 // A scalar operand: an immediate fixed at build time or a ScalarRef re-read at every code generation.
@@ -76,6 +80,13 @@ class NDObject {
   IntArrayRef *stride_ref = nullptr;                 // explicit strides
   IntArrayRef *full_shape_ref = nullptr;             // slices: shape of the whole tensor
   IntArrayRef *slice_start = nullptr, *slice_end = nullptr, *slice_step = nullptr;  // end/step only for strided slices
+  // kObjSlice along one dim (Slice(input, dim, begin, end) and the chunks of Split): bounds from the
+  // references when set, else the fixed values; negative bounds count from the end, both are clipped
+  NDObject *cat = nullptr;          // kObjConcatPart: the Concat it belongs to
+  std::vector<NDObject *> parts;    // kObjConcat: its parts, in order along slice_dim
+  int slice_dim = -1;
+  ScalarRef *dim_begin_ref = nullptr, *dim_end_ref = nullptr;
+  int64_t dim_begin = 0, dim_end = 0;
   int id = -1;                     // position in the kernel's operator list
   int stage = 0;                   // sub-kernel group opened by Kernel::ParallelAdd / SequenceAdd
 
@@ -178,6 +189,12 @@ class VKernel {
   std::string &Inspect();
 
   std::vector<NDObject *> ops_;
+  // arrays handed to the caller (the chunks of a Split); they live as long as the kernel's operators
+  NDObject **NewObjectArray(size_t n) {
+    obj_arrays_.emplace_back(n, nullptr);
+    return obj_arrays_.back().data();
+  }
+  std::vector<std::vector<NDObject *>> obj_arrays_;
   std::vector<Program> programs_;
   size_t ws_bytes_ = 0;
   std::vector<size_t> ws_offsets_;  // per workspace slot

@@ -63,13 +63,24 @@ dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int 
 int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store);
 // Strided views (Kernel::Load / Store with a stride list, SliceLoad, StridedSliceLoad: include/dvm.h:195-201, 214 of the
 // reference; KernelPy view_load / slice_load / stridedslice_load, include/dvm_py.h). Strides are in elements, the
-// innermost one has to be 1. A view store writes into a zero-initialised buffer of extent_elems elements;
+// innermost one may be anything (0 broadcasts, 1 is the fast path, others go element by element). A view store writes into a zero-initialised buffer of extent_elems elements;
 // dvm_obj_set_view_offset moves the first element of a view that many elements into its buffer.
 dvm_obj *dvm_rt_view_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *stride, int dtype);
 dvm_obj *dvm_rt_slice_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *start, dvm_shape *size, int dtype);
 dvm_obj *dvm_rt_stridedslice_load(dvm_rt *rt, dvm_shape *shape, dvm_shape *start, dvm_shape *end, dvm_shape *step, int dtype);
 dvm_obj *dvm_rt_view_store(dvm_rt *rt, dvm_obj *x, dvm_shape *stride, size_t extent_elems);
 int dvm_obj_set_view_offset(dvm_obj *io, long long elems);
+// Views of values (Kernel::Permute / Slice / Split, include/dvm.h:434,443,453,479 of the reference; KernelPy permute /
+// slice / slice_dim / split, include/dvm_py.h:347-358): dims[i] names the input dim that becomes result dim i; a slice
+// keeps `size` elements from `start` in every dim, or [begin, end) of one dim (negative bounds count from the end,
+// both are clipped; the scalars are re-read at every code generation); split writes `num` handles to `out`, chunks
+// of `chunk` along `dim`, the last one possibly smaller.
+dvm_obj *dvm_rt_permute(dvm_rt *rt, dvm_obj *x, dvm_shape *dims);
+dvm_obj *dvm_rt_slice(dvm_rt *rt, dvm_obj *x, dvm_shape *start, dvm_shape *size);
+dvm_obj *dvm_rt_slice_dim(dvm_rt *rt, dvm_obj *x, int dim, dvm_scalar *begin, dvm_scalar *end);
+int dvm_rt_split(dvm_rt *rt, dvm_obj *x, int dim, long long chunk, size_t num, dvm_obj **out);
+// Kernel::Concat (include/dvm.h:470 of the reference; KernelPy concat, include/dvm_py.h:173-181): the n inputs joined along `dim`.
+dvm_obj *dvm_rt_concat(dvm_rt *rt, dvm_obj **inputs, size_t n, int dim);
 // Group markers of "seq" and "parallel" kernels (KernelPy::SequenceAdd / ParallelAdd, include/dvm_py.h:369-371; Kernel::SequenceAdd /
 // ParallelAdd, include/dvm.h:250-251): operators built after the call belong to the next sub-kernel group.
 int dvm_rt_seq_add(dvm_rt *rt, int ktype, unsigned flags);

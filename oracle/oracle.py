@@ -473,6 +473,25 @@ class OracleKernel:
     def reshape(self, x, shape):
         return OVal(x.a.reshape(tuple(shape)), x.t, x.bool_result)
 
+    # views of values (include/dvm.h:434,443,453,479 of the reference): NumPy's transpose and basic slicing
+    def permute(self, x, dims):
+        return OVal(np.ascontiguousarray(np.transpose(x.a, tuple(dims))), x.t, x.bool_result)
+
+    def slice(self, x, start, size):
+        idx = tuple(slice(s + (n if s < 0 else 0), s + (n if s < 0 else 0) + k) for s, k, n in zip(start, size, x.a.shape))
+        return OVal(np.ascontiguousarray(x.a[idx]), x.t, x.bool_result)
+
+    def slice_dim(self, x, dim, begin, end):
+        idx = [slice(None)] * x.a.ndim
+        idx[dim] = slice(begin, end)
+        return OVal(np.ascontiguousarray(x.a[tuple(idx)]), x.t, x.bool_result)
+
+    def concat(self, inputs, dim):
+        return OVal(np.concatenate([x.a for x in inputs], axis=dim), inputs[0].t, inputs[0].bool_result)
+
+    def split(self, x, dim, split_size, split_num):
+        return tuple(self.slice_dim(x, dim, j * split_size, (j + 1) * split_size) for j in range(split_num))
+
     def copy(self, x):
         return OVal(x.a.copy(), x.t, x.bool_result)
 

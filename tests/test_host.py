@@ -429,3 +429,37 @@ def test_strided_views_in_das_mode():
         t.store(t.add(x0, t.load(g)))
     t, das = _das(two, "split")
     assert t.workspace_bytes() >= f.nbytes or das.count("== sub-kernel") == 1
+
+
+def test_views_of_values_in_das_mode():
+    # include/dvm.h:434-479 of the reference: Permute / Slice / Split / Concat
+    a = np.zeros([10, 20, 32], np.float32)
+    # a permuted load is read in place: one launch, the operand strides are the permuted ones
+    t, das = _das(lambda t: t.store(t.permute(t.load(a), [1, 0, 2])))
+    assert das.count("== sub-kernel") == 1 and "k[1,640,32]" in das
+    # a permuted computed value is written once in its own layout and read through the permuted strides
+    t, das = _das(lambda t: t.store(t.add(t.permute(t.add(t.load(a), 1.0), [1, 0, 2]), 2.0)), "split")
+    assert das.count("== sub-kernel") == 2 and t.workspace_bytes() >= a.nbytes
+    # a box out of a computed value: the second launch starts inside the first one's buffer
+    b = np.zeros([1024, 500], np.float32)
+    t, das = _das(lambda t: t.store(t.add(t.slice(t.mul(t.load(b), 0.1), [100, 100], [600, 300]), 0.2)), "split")
+    assert das.count("== sub-kernel") == 2 and "k[1,500]" in das
+    # the chunks of a split share their input's buffer; the last one is what is left
+    t = Tester("split", run_mode="das")
+    parts = t.split(t.mul(t.load(np.zeros([3, 500, 32], np.float32)), 0.7), 1, 200, 3)
+    outs = [t.store(t.add(p, 1.0)) for p in parts]
+    t.codegen()
+    assert [o.shape() for o in outs] == [(3, 200, 32), (3, 200, 32), (3, 100, 32)]
+    # concat: every part is written into its place by the launch that computes it
+    c0, c1 = np.zeros([3, 100], np.float32), np.zeros([3, 50], np.float32)
+    t, das = _das(lambda t: t.store(t.add(t.concat([t.mul(t.load(c0), 2.0), t.add(t.load(c1), 1.0)], 1), 0.5)), "split")
+    assert das.count("== sub-kernel") == 3 and das.count("k[1,150]") == 2 and t.workspace_bytes() >= 3 * 150 * 4
+    # what is not supported says so
+    t = Tester("vector", run_mode="das")
+    t.store(t.reshape(t.permute(t.load(np.zeros([4, 8], np.float32)), [1, 0]), [32]))
+    with pytest.raises(RuntimeError, match="needs a Copy"):
+        t.codegen()
+    t = Tester("vector", run_mode="das")
+    t.store(t.slice(t.load(np.zeros([4, 8], np.float32)), [2, 0], [4, 8]))
+    with pytest.raises(RuntimeError, match="slice reaches outside"):
+        t.codegen()
