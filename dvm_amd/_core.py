@@ -71,6 +71,7 @@ def _load():
         "dvm_obj_dtype": (ci, [vp]),
         "dvm_rt_input": (ci, [vp, vp, vp, cs]),
         "dvm_rt_bind_device": (ci, [vp, vp, vp]),
+        "dvm_rt_normalize": (ci, [vp]),
         "dvm_rt_codegen": (ci, [vp]),
         "dvm_rt_jit_us": (ctypes.c_double, [vp]),
         "dvm_rt_run": (ci, [vp, vp, ci]),
@@ -481,6 +482,10 @@ class PyKernel(Kernel):
         if shape is not None and io._h in self._load_shape:
             self._load_shape[io._h].update(list(shape))
         _check(_lib.dvm_rt_bind_device(self._rt, io._h, ctypes.c_void_p(device_ptr)))
+
+    def normalize(self):
+        """Shape inference only: store.shape() is valid afterwards."""
+        _check(_lib.dvm_rt_normalize(self._rt))
 
     def codegen(self, pass_names=None):
         _check(_lib.dvm_rt_codegen(self._rt))

@@ -603,6 +603,15 @@ int dvm_rt_bind_device(dvm_rt *rt, dvm_obj *io, void *device_ptr) {
       -1);
 }
 
+int dvm_rt_normalize(dvm_rt *rt) {
+  return Guard(
+      [&]() {
+        rt->kernel.Normalize();
+        return 0;
+      },
+      -1);
+}
+
 int dvm_rt_codegen(dvm_rt *rt) {
   return Guard(
       [&]() {

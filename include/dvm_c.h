@@ -99,6 +99,9 @@ int dvm_rt_input(dvm_rt *rt, dvm_obj *load, const void *host, size_t bytes);
 /* Binds a caller-owned device buffer to a load or store (no copy, no ownership). */
 int dvm_rt_bind_device(dvm_rt *rt, dvm_obj *io, void *device_ptr);
 /* Normalize + allocate unbound outputs + CodeGen with relocations. */
+// Shape inference only (what dvm_rt_codegen does first): afterwards dvm_obj_shape of a store is what the bound
+// inputs imply, so a caller can allocate its own output memory and bind it before code generation.
+int dvm_rt_normalize(dvm_rt *rt);
 int dvm_rt_codegen(dvm_rt *rt);
 /* Host wall time of the last Normalize + CodeGen in microseconds. */
 double dvm_rt_jit_us(const dvm_rt *rt);
