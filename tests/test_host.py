@@ -463,3 +463,28 @@ def test_views_of_values_in_das_mode():
     t.store(t.slice(t.load(np.zeros([4, 8], np.float32)), [2, 0], [4, 8]))
     with pytest.raises(RuntimeError, match="slice reaches outside"):
         t.codegen()
+
+
+def test_clone_carries_views():
+    # Kernel::Clone (include/dvm.h:188 of the reference) over a graph with Permute / Slice / Split / Concat and a
+    # strided load: the clone compiles to the same programs as its base
+    a = np.zeros([6, 40], np.float32)
+
+    def build(t):
+        x = t.load(a)
+        v = t.view_load([6, 20], [40, 2], a)
+        p0, _ = t.split(t.add(x, 1.0), 1, 20, 2)
+        c = t.concat([t.mul(p0, 2.0), t.slice_dim(x, 1, 5, 25), v], 1)
+        out = t.store(t.permute(t.add(c, 0.5), [1, 0]))
+        return x, v, out
+    t = Tester("split", run_mode="das")
+    x, v, out = build(t)
+    t.codegen()
+    t2 = Tester("split", run_mode="das")
+    x2, v2, out2 = t2.clone(t, [x, v, out])
+    t2.input(x2, a)
+    t2.input(v2, a)
+    t2.codegen()
+    assert out2.shape() == out.shape() == (60, 6)
+    strip = lambda d: "\n".join(l for l in d.splitlines() if "@0x" not in l)  # addresses differ, programs do not
+    assert strip(t2.das()) == strip(t.das()) and t.das().count("== sub-kernel") >= 3
