@@ -471,6 +471,7 @@ class Compiler {
     level_.assign(n_, 0);
     live_.assign(n_, 0);
     mat_.assign(n_, 0);
+    absorbed_.assign(n_, 0);
     ws_slot_.assign(n_, -1);
     store_of_.assign(n_, -1);
     MarkLive();
@@ -497,6 +498,7 @@ class Compiler {
   int n_;
   std::vector<int> area_, ws_slot_, store_of_, level_;
   std::vector<char> live_, mat_;
+  std::vector<char> absorbed_;  // stores of a Concat whose parts write the user's buffer themselves
   int n_areas_ = 0;
   struct AreaInfo {
     bool cube = false;
@@ -746,6 +748,10 @@ class Compiler {
       if (!mat_[i]) continue;
       NDObject *o = k_->ops_[i];
       if (store_of_[i] >= 0 && area_[store_of_[i]] == area_[i]) continue;  // later kernels read the user's output
+      if (o->kind == kObjConcat && store_of_[i] >= 0) {  // the parts write straight into the stored output
+        absorbed_[store_of_[i]] = 1;
+        continue;
+      }
       ws_slot_[i] = static_cast<int>(k_->ws_sizes_.size());
       k_->ws_sizes_.push_back(static_cast<size_t>(std::max<int64_t>(o->numel(), 1)) * DTypeSize(o->type_id_));
     }
@@ -938,6 +944,7 @@ void Compiler::BuildNodes(int a) {
     if (area_[i] != a) continue;
     NDObject *o = k_->ops_[i];
     if (o->kind == kObjConcat) continue;  // a buffer its parts fill, nothing to compute
+    if (absorbed_[i]) continue;             // its value was written in place by the parts of a Concat
     int in_idx[3] = {-1, -1, -1};
     for (int j = 0; j < o->nin; ++j) {
       NDObject *v = o->in[j];
@@ -976,6 +983,7 @@ void Compiler::BuildNodes(int a) {
     if (kind == AK_OUT) {
       if (o->kind == kObjConcatPart) {
         n.ws_slot = ws_slot_[o->cat->id];
+        if (n.ws_slot < 0) n.addr_op = store_of_[o->cat->id];
         n.view = o;
       } else {
         n.addr_op = i;
@@ -2158,6 +2166,10 @@ void Compiler::CompileArea(int a) {
     return;
   }
   BuildNodes(a);
+  if (nn_ == 0) {  // only stores that other launches have already served
+    prog_->skip = true;
+    return;
+  }
   // an empty domain: nothing to run, outputs that still have elements are zero-filled
   bool empty = false;
   for (int i = 0; i < nn_; ++i) {

@@ -454,6 +454,9 @@ def test_views_of_values_in_das_mode():
     c0, c1 = np.zeros([3, 100], np.float32), np.zeros([3, 50], np.float32)
     t, das = _das(lambda t: t.store(t.add(t.concat([t.mul(t.load(c0), 2.0), t.add(t.load(c1), 1.0)], 1), 0.5)), "split")
     assert das.count("== sub-kernel") == 3 and das.count("k[1,150]") == 2 and t.workspace_bytes() >= 3 * 150 * 4
+    # a Concat that is stored is assembled in the stored output: two launches, no workspace, no copy
+    t, das = _das(lambda t: t.store(t.concat([t.mul(t.load(c0), 2.0), t.add(t.load(c1), 1.0)], 1)), "split")
+    assert das.count("entry vector") == 2 and t.workspace_bytes() == 0 and t.num_launches() == 2
     # what is not supported says so
     t = Tester("vector", run_mode="das")
     t.store(t.reshape(t.permute(t.load(np.zeros([4, 8], np.float32)), [1, 0]), [32]))
