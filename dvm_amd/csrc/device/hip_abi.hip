@@ -28,6 +28,8 @@ DVM_CUBE_DECL(dvm_vm_cube_bf16_mid)
 DVM_CUBE_DECL(dvm_vm_cube_f16_mid)
 DVM_CUBE_DECL(dvm_vm_cube_bf16_small)
 DVM_CUBE_DECL(dvm_vm_cube_f16_small)
+DVM_CUBE_DECL(dvm_vm_cube_bf16_big8)
+DVM_CUBE_DECL(dvm_vm_cube_f16_big8)
 
 extern "C" __global__ void dvm_vm_attn_f16(const VmParam p);
 extern "C" __global__ void dvm_vm_attn_bf16(const VmParam p);
@@ -35,10 +37,11 @@ extern "C" __global__ void dvm_vm_attn_bf16(const VmParam p);
 typedef void (*CubeKernel)(const VmParam);
 #define DVM_CUBE_ROW(prefix) {prefix##_nn, prefix##_nt, prefix##_tn, prefix##_tt}
 // [tile][bf16][trans_a * 2 + trans_b]
-static const CubeKernel kCubeKernels[3][2][4] = {
+static const CubeKernel kCubeKernels[4][2][4] = {
     {DVM_CUBE_ROW(dvm_vm_cube_f16_big), DVM_CUBE_ROW(dvm_vm_cube_bf16_big)},
     {DVM_CUBE_ROW(dvm_vm_cube_f16_mid), DVM_CUBE_ROW(dvm_vm_cube_bf16_mid)},
-    {DVM_CUBE_ROW(dvm_vm_cube_f16_small), DVM_CUBE_ROW(dvm_vm_cube_bf16_small)}};
+    {DVM_CUBE_ROW(dvm_vm_cube_f16_small), DVM_CUBE_ROW(dvm_vm_cube_bf16_small)},
+    {DVM_CUBE_ROW(dvm_vm_cube_f16_big8), DVM_CUBE_ROW(dvm_vm_cube_bf16_big8)}};
 
 namespace {
 
@@ -183,10 +186,11 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
     const VCubeHeader *c = reinterpret_cast<const VCubeHeader *>(p.w);
     const uint64_t mem_end = static_cast<uint64_t>(c->mem_off) + static_cast<uint64_t>(c->n_mem) * (sizeof(VCubeMem) / 8);
     const uint64_t code_end = static_cast<uint64_t>(c->code_off) + c->n_code;
-    const uint32_t bt = c->tile == 0 ? 256u : (c->tile == 1 ? 128u : 64u);
+    const uint32_t bt = (c->tile == 0 || c->tile == 3) ? 256u : (c->tile == 1 ? 128u : 64u);
+    const uint32_t want_threads = c->tile == 3 ? 512u : 256u;  // tile 3: the 256x256 tile on eight waves
     // The tile loop trusts the header: check it describes the launch it gets.
     if (mem_end > DVM_PARAM_WORDS || code_end > DVM_PARAM_WORDS || c->n_code == 0 || VI_OP(p.w[code_end - 1]) != VOP_END ||
-        c->tile > 2 || threads != 256 || c->m == 0 || c->n == 0 || c->nb0 == 0 || c->nb1 == 0 ||
+        c->tile > 3 || threads != want_threads || c->m == 0 || c->n == 0 || c->nb0 == 0 || c->nb1 == 0 ||
         c->tiles_m != (c->m + bt - 1) / bt || c->tiles_n != (c->n + bt - 1) / bt || lds_bytes < DVM_CUBE_LDS_BYTES(bt) ||
         c->a_addr == 0 || c->b_addr == 0 || (c->dtype != VDT_F16 && c->dtype != VDT_BF16)) {
       return static_cast<int>(hipErrorInvalidValue);
@@ -196,7 +200,7 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
       return static_cast<int>(hipErrorInvalidValue);
     }
     const CubeKernel kern = kCubeKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0][(c->trans_a ? 2 : 0) + (c->trans_b ? 1 : 0)];
-    hipLaunchKernelGGL(kern, dim3(block_dim), dim3(256), lds_bytes, s, p);
+    hipLaunchKernelGGL(kern, dim3(block_dim), dim3(want_threads), lds_bytes, s, p);
   } else if (h->entry == VE_ATTN) {
     const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.w);
     // the kernel has no guards of its own beyond the query tail: the header must fit it exactly

@@ -83,21 +83,23 @@ struct LaneOffsets {
   uint32_t v[2];
 };
 
-template <int ROWS, bool KC>
+template <int ROWS, bool KC, int NTHR>
 struct Stage;
 
-template <int ROWS>
-struct Stage<ROWS, true> {
-  static constexpr int N = ROWS * BK / 8 / 256;  // 16-byte chunks per thread
+template <int ROWS, int NTHR>
+struct Stage<ROWS, true, NTHR> {
+  static constexpr int N = ROWS * BK / 8 / NTHR;  // 16-byte chunks per thread
+  static constexpr uint32_t RPS = NTHR / 8;        // rows one step of all threads covers
   static constexpr int N_LOADS = N, N_WRITES = 0;
 
-  // Chunk position p = 256*i + tid of the tile holds row p/8, logical chunk (p%8) ^ swizzle(row): with
-  // row = 32*i + tid/8 the swizzle only depends on the parity of i, hence two byte offsets per lane.
+  // Chunk position p = NTHR*i + tid of the tile holds row p/8, logical chunk (p%8) ^ swizzle(row): with
+  // row = RPS*i + tid/8 the swizzle depends at most on the parity of i (RPS = 32; not at all for 64), hence
+  // two byte offsets per lane.
   static __device__ __forceinline__ LaneOffsets lane_offset(uint32_t ld, uint32_t tid) {
     LaneOffsets o;
 #pragma unroll
     for (int par = 0; par < 2; ++par) {
-      const uint32_t row = 32u * par + (tid >> 3);
+      const uint32_t row = RPS * par + (tid >> 3);
       const uint32_t logical = (tid & 7u) ^ ((row ^ (row >> 3)) & 7u);
       o.v[par] = ((tid >> 3) * ld + (logical << 3)) * 2u;
     }
@@ -110,44 +112,53 @@ struct Stage<ROWS, true> {
     const uint32_t wave_first = uni(tid >> 6) * 64u;
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const DVM_GLOBAL char *src = base + static_cast<uint64_t>(i) * 32u * ld * 2u + lane.v[i & 1];
-      uint16_t *dst = tile + (static_cast<uint32_t>(i) * 256u + wave_first) * 8u;
+      const DVM_GLOBAL char *src = base + static_cast<uint64_t>(i) * RPS * ld * 2u + lane.v[i & 1];
+      uint16_t *dst = tile + (static_cast<uint32_t>(i) * NTHR + wave_first) * 8u;
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(src), (__attribute__((address_space(3))) void *)(dst), 16, 0, 0);
     }
   }
   __device__ __forceinline__ void commit(uint16_t *, uint32_t) const {}
 };
 
-template <int ROWS>
-struct Stage<ROWS, false> {
-  static_assert(ROWS <= 256, "one 8x8 block per thread");
+template <int ROWS, int NTHR>
+struct Stage<ROWS, false, NTHR> {
+  static_assert(ROWS <= 256, "one 8x8 block per thread, the first ROWS threads");
+  // 8 (k) x 8 (rows) element blocks, ROWS of them per tile. With 256 lanes one lane takes a whole block; with 512
+  // lanes and 256 rows two lanes share one, each taking 4 of its rows (8-byte loads, half the registers).
+  static constexpr int TPB = (NTHR == 512 && ROWS == 256) ? 2 : 1;  // lanes per block
+  static constexpr int RPT = 8 / TPB;                               // rows of the block a lane owns
   static constexpr int N = 8;
-  static constexpr int N_LOADS = 8, N_WRITES = 8;
-  vu4 r[N];
+  static constexpr int N_LOADS = 8, N_WRITES = RPT;
+  typedef uint32_t Row __attribute__((ext_vector_type(RPT / 2)));   // RPT 16-bit elements of one k
+  Row r[N];
+
+  static __device__ __forceinline__ bool active(uint32_t tid) { return (ROWS * TPB == NTHR) || tid < ROWS * TPB; }
 
   static __device__ __forceinline__ LaneOffsets lane_offset(uint32_t ld, uint32_t tid) {
-    const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
+    const uint32_t blk = tid / TPB, part = tid % TPB;
+    const uint32_t kb = blk / (ROWS / 8), rb = blk % (ROWS / 8);
     LaneOffsets o;
-    o.v[0] = o.v[1] = (kb * 8u * ld + rb * 8u) * 2u;
+    o.v[0] = o.v[1] = (kb * 8u * ld + rb * 8u + part * RPT) * 2u;
     return o;
   }
 
   __device__ __forceinline__ void fetch(uint64_t origin, uint32_t ld, const LaneOffsets &lane, uint32_t tid, uint16_t *) {
     const DVM_GLOBAL char *base = reinterpret_cast<const DVM_GLOBAL char *>(origin);
-    if (ROWS == 256 || tid < ROWS) {
+    if (active(tid)) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        r[j] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(base + static_cast<uint64_t>(j) * ld * 2u + lane.v[0]);
+        r[j] = *reinterpret_cast<const DVM_GLOBAL Row *>(base + static_cast<uint64_t>(j) * ld * 2u + lane.v[0]);
       }
     }
   }
 
   __device__ __forceinline__ void commit(uint16_t *tile, uint32_t tid) const {
-    if (ROWS == 256 || tid < ROWS) {
-      const uint32_t kb = tid / (ROWS / 8), rb = tid % (ROWS / 8);
-      // r[j] holds k = kb*8 + j, rows rb*8 .. +7; the tile wants, per row, k = kb*8 .. +7
+    if (active(tid)) {
+      const uint32_t blk = tid / TPB, part = tid % TPB;
+      const uint32_t kb = blk / (ROWS / 8), rb = blk % (ROWS / 8);
+      // r[j] holds k = kb*8 + j, rows rb*8 + part*RPT .. +RPT-1; the tile wants, per row, k = kb*8 .. +7
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
+      for (int i = 0; i < RPT; ++i) {
         vu4 o;
 #pragma unroll
         for (int jj = 0; jj < 4; ++jj) {
@@ -155,7 +166,7 @@ struct Stage<ROWS, false> {
           // bytes of the result, least significant first: (i odd ? upper : lower) half of lo, then of hi
           o[jj] = __builtin_amdgcn_perm(hi, lo, (i & 1) ? 0x07060302u : 0x05040100u);
         }
-        *reinterpret_cast<vu4 *>(tile + tile_off(rb * 8 + i, kb)) = o;
+        *reinterpret_cast<vu4 *>(tile + tile_off(rb * 8 + part * RPT + i, kb)) = o;
       }
     }
   }
@@ -163,10 +174,10 @@ struct Stage<ROWS, false> {
 
 // Generic staging of one tile straight into local memory, element by element (edge tiles, odd
 // leading dimensions, unaligned operands). Slow, correct for every shape.
-template <int ROWS>
+template <int ROWS, int NTHR>
 __device__ __attribute__((noinline)) void stage_generic(uint16_t *tile, uint64_t base, uint32_t ld, uint32_t row0, uint32_t k0,
                                                         uint32_t rows, uint32_t kext, uint32_t k_contig, uint32_t tid) {
-  for (uint32_t e = tid; e < ROWS * BK; e += 256u) {
+  for (uint32_t e = tid; e < ROWS * BK; e += NTHR) {
     const uint32_t row = e / BK, kk = e % BK;
     const uint32_t gr = row0 + row, gk = k0 + kk;
     uint16_t v = 0;
@@ -603,18 +614,20 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
 
 // Second half of a pass: the half tile sits in local memory, row major with PITCH floats per row;
 // every lane takes slabs of 8 columns and walks the epilogue program over them.
-template <int ROWS, int BN, int TM>
+template <int ROWS, int BN, int TM, int WM>
 __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
                                                         uint32_t pass, uint32_t m, uint32_t n) {
+  constexpr int NTHR = WM * 2 * 64;
   constexpr int PITCH = BN + 4;
   constexpr int GROUPS = BN / 8;               // slabs per row
-  constexpr int PER_THREAD = ROWS * GROUPS / 256;  // slabs per thread
-  constexpr int SL = PER_THREAD % 4 == 0 ? 4 : 2;
+  constexpr int PER_THREAD = ROWS * GROUPS / NTHR;  // slabs per thread
+  // four slabs per walk of the program where a wave may use all 512 registers; with two waves per SIMD two slabs
+  constexpr int SL = (PER_THREAD % 4 == 0 && WM == 2) ? 4 : 2;
   static_assert(PER_THREAD % SL == 0, "slab count per thread");
-  constexpr int ROWS_PER_STEP = 256 / GROUPS;  // rows one step of all 256 threads covers
+  constexpr int ROWS_PER_STEP = NTHR / GROUPS;  // rows one step of all threads covers
   const uint32_t tid = threadIdx.x;
   const uint32_t g = tid % GROUPS, r0 = tid / GROUPS;
-  constexpr int HALF = ROWS / 2;  // local rows [0, HALF) belong to the upper pair of waves, the rest to the lower pair
+  constexpr int HALF = ROWS / WM;  // local rows [i * HALF, (i + 1) * HALF) belong to the i-th row of waves
   const uint32_t col = n0 + g * 8;
   const uint32_t ncol = col >= n ? 0u : (n - col < 8u ? n - col : 8u);
   for (int it = 0; it < PER_THREAD / SL; ++it) {
@@ -640,9 +653,10 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
 
 // TM x TN 32x32 MFMA tiles per wave, 2 x 2 waves per workgroup; A_KC / B_KC: the operand's k axis is
 // contiguous in memory.
-template <bool IS_BF16, int TM, int TN, bool A_KC, bool B_KC>
+template <bool IS_BF16, int TM, int TN, bool A_KC, bool B_KC, int WM>
 __device__ __forceinline__ void vm_cube(const VmParam &p) {
-  constexpr int BM = 2 * TM * 32, BN = 2 * TN * 32;
+  constexpr int NTHR = WM * 2 * 64;  // WM x 2 waves
+  constexpr int BM = WM * TM * 32, BN = 2 * TN * 32;
   constexpr int PASSES = TM >= 2 ? 2 : 1;
   constexpr int PROWS = BM / PASSES;  // rows of the tile one epilogue pass covers
   constexpr int PITCH = BN + 4;
@@ -654,9 +668,9 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
     const VCubeHeader *hp = reinterpret_cast<const VCubeHeader *>(p.w);
     uint32_t used = (hp->code_off + hp->n_code) * 2;
     used = used < DVM_PARAM_BYTES / 4 ? used : DVM_PARAM_BYTES / 4;
-    const uint32_t trips = (used + 255) / 256;
+    const uint32_t trips = (used + NTHR - 1) / NTHR;
     for (uint32_t t = 0; t < trips; ++t) {
-      uint32_t i = t * 256 + threadIdx.x;
+      uint32_t i = t * NTHR + threadIdx.x;
       i = i < used ? i : used - 1;
       prog32[i] = src[i];
     }
@@ -714,14 +728,14 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       for (int j = 0; j < TN; ++j) acc[i][j] = 0.0f;
 
     if (h.fast && m0 + BM <= h.m && n0 + BN <= h.n) {
-      Stage<BM, A_KC> sa;
-      Stage<BN, B_KC> sb;
+      Stage<BM, A_KC, NTHR> sa;
+      Stage<BN, B_KC, NTHR> sb;
       // address of element (row0, k) of each operand, k advancing by BK per step
       const uint64_t a_org = a_base + (A_KC ? static_cast<uint64_t>(m0) * h.lda : static_cast<uint64_t>(m0)) * 2;
       const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb : static_cast<uint64_t>(n0)) * 2;
       const uint64_t a_step = (A_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.lda) * 2;
       const uint64_t b_step = (B_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.ldb) * 2;
-      const LaneOffsets a_voff = Stage<BM, A_KC>::lane_offset(h.lda, tid), b_voff = Stage<BN, B_KC>::lane_offset(h.ldb, tid);
+      const LaneOffsets a_voff = Stage<BM, A_KC, NTHR>::lane_offset(h.lda, tid), b_voff = Stage<BN, B_KC, NTHR>::lane_offset(h.ldb, tid);
       sa.fetch(a_org, h.lda, a_voff, tid, lds);
       sb.fetch(b_org, h.ldb, b_voff, tid, lds + kBBase);
       sa.commit(lds, tid);
@@ -761,9 +775,9 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
         constexpr int NREST = NM - NF > 0 ? NM - NF : 1;  // MFMAs left in a step after the fragment reads
         // staging instructions per such MFMA: ds_write of a k-strided operand (step 1), its global loads
         // (step 2), direct-to-LDS loads of a k-contiguous operand (step 3)
-        constexpr int NW = ((A_KC ? 0 : 8) + (B_KC ? 0 : 8) + NREST - 1) / NREST;
+        constexpr int NW = ((A_KC ? 0 : Stage<BM, false, NTHR>::N_WRITES) + (B_KC ? 0 : Stage<BN, false, NTHR>::N_WRITES) + NREST - 1) / NREST;
         constexpr int NL = ((A_KC ? 0 : 8) + (B_KC ? 0 : 8) + NREST - 1) / NREST;
-        constexpr int ND = ((A_KC ? Stage<BM, true>::N : 0) + (B_KC ? Stage<BN, true>::N : 0) + NREST - 1) / NREST;
+        constexpr int ND = ((A_KC ? Stage<BM, true, NTHR>::N : 0) + (B_KC ? Stage<BN, true, NTHR>::N : 0) + NREST - 1) / NREST;
         // step 0
         __builtin_amdgcn_sched_barrier(0);
         read_frags(1, cur, 1);
@@ -857,8 +871,8 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       __syncthreads();
     } else {
       for (uint32_t kt = 0; kt < nk; ++kt) {
-        stage_generic<BM>(lds, a_base, h.lda, m0, kt * BK, h.m, h.k, A_KC ? 1u : 0u, tid);
-        stage_generic<BN>(lds + kBBase, b_base, h.ldb, n0, kt * BK, h.n, h.k, B_KC ? 1u : 0u, tid);
+        stage_generic<BM, NTHR>(lds, a_base, h.lda, m0, kt * BK, h.m, h.k, A_KC ? 1u : 0u, tid);
+        stage_generic<BN, NTHR>(lds + kBBase, b_base, h.ldb, n0, kt * BK, h.n, h.k, B_KC ? 1u : 0u, tid);
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
@@ -887,13 +901,13 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
         for (int j = 0; j < TN; ++j) {
           const vf16 &c = acc[ps * FR + fi][j];
           // lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4 of the fragment
-          float *dst = dump + (wm * (PROWS / 2) + fi * 32 + (lane >> 5) * 4) * PITCH + (wn * TN + j) * 32 + (lane & 31u);
+          float *dst = dump + (wm * (PROWS / WM) + fi * 32 + (lane >> 5) * 4) * PITCH + (wn * TN + j) * 32 + (lane & 31u);
 #pragma unroll
           for (int r = 0; r < 16; ++r) dst[(8 * (r / 4) + (r % 4)) * PITCH] = c[r];
         }
       }
       __syncthreads();
-      epilogue_pass<PROWS, BN, TM>(dump, prog32, ea, m0, n0, ps, h.m, h.n);
+      epilogue_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n);
       __syncthreads();
     }
   }
@@ -901,17 +915,20 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
 
 }  // namespace
 
-#define DVM_CUBE_KERNEL(name, bf, tm, akc, bkc) \
-  extern "C" __global__ void __launch_bounds__(256) name(const VmParam p) { vm_cube<bf, tm, tm, akc, bkc>(p); }
-#define DVM_CUBE_LAYOUTS(prefix, bf, tm)            \
-  DVM_CUBE_KERNEL(prefix##_nn, bf, tm, true, false) \
-  DVM_CUBE_KERNEL(prefix##_nt, bf, tm, true, true)  \
-  DVM_CUBE_KERNEL(prefix##_tn, bf, tm, false, false) \
-  DVM_CUBE_KERNEL(prefix##_tt, bf, tm, false, true)
+#define DVM_CUBE_KERNEL(name, bf, tm, tn, wm, akc, bkc) \
+  extern "C" __global__ void __launch_bounds__(wm * 128) name(const VmParam p) { vm_cube<bf, tm, tn, akc, bkc, wm>(p); }
+#define DVM_CUBE_LAYOUTS(prefix, bf, tm, tn, wm)            \
+  DVM_CUBE_KERNEL(prefix##_nn, bf, tm, tn, wm, true, false) \
+  DVM_CUBE_KERNEL(prefix##_nt, bf, tm, tn, wm, true, true)  \
+  DVM_CUBE_KERNEL(prefix##_tn, bf, tm, tn, wm, false, false) \
+  DVM_CUBE_KERNEL(prefix##_tt, bf, tm, tn, wm, false, true)
 
-DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_big, true, 4)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_big, false, 4)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_mid, true, 2)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_mid, false, 2)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_small, true, 1)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_small, false, 1)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_big, true, 4, 4, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_big, false, 4, 4, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_mid, true, 2, 2, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_mid, false, 2, 2, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_small, true, 1, 1, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_small, false, 1, 1, 2)
+// the 256x256 tile on eight waves (4 x 2, 64x128 accumulators each): two waves per SIMD
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_big8, true, 2, 4, 4)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_big8, false, 2, 4, 4)

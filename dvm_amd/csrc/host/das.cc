@@ -200,10 +200,10 @@ std::string &VKernel::DisAssemble() {
       print_code(p.blob.w + h->code_off, h->n_code, [&](uint32_t m) { return mems[m].dtype; });
     } else if (h->entry == VE_CUBE) {
       const VCubeHeader *c = reinterpret_cast<const VCubeHeader *>(p.blob.w);
-      static const int tile[] = {256, 128, 64};
+      static const int tile[] = {256, 128, 64, 256};
       os << "entry cube " << kMemTypes[c->dtype] << " m=" << c->m << " n=" << c->n << " k=" << c->k << " trans_a=" << c->trans_a
          << " trans_b=" << c->trans_b << " batch=" << c->nb0 << "x" << c->nb1 << " tile=" << tile[c->tile] << " blocks=" << p.grid
-         << " lds=" << p.lds_bytes << (c->fast ? " fast" : " guarded") << "\n";
+         << " lds=" << p.lds_bytes << (c->fast ? " fast" : " guarded") << (c->tile == 3 ? " eight-waves" : "") << "\n";
       const VCubeMem *cm = reinterpret_cast<const VCubeMem *>(p.blob.w + c->mem_off);
       for (uint32_t i = 0; i < c->n_mem; ++i) {
         char buf[32];

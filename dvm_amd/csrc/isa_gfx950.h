@@ -223,7 +223,7 @@ typedef struct {
   uint32_t lda, ldb;   // leading dimensions in elements
   uint32_t nb0, nb1;   // batch extents (outer, inner); 1 when absent
   uint32_t a_sb0, a_sb1, b_sb0, b_sb1;  // batch strides in elements (0 = broadcast)
-  uint32_t tile;       // block tile: 0 = 256x256, 1 = 128x128, 2 = 64x64
+  uint32_t tile;       // block tile: 0 = 256x256, 1 = 128x128, 2 = 64x64 (four waves), 3 = 256x256 on eight waves (512 lanes)
   uint32_t tiles_m, tiles_n;
   uint32_t n_mem, n_code;
   uint32_t mem_off, code_off;  // word offsets

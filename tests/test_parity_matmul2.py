@@ -117,3 +117,38 @@ def test_single_row_long_k():  # :720-735
     np_a, np_b = rng.normal(0, 0.1, (1, 80000)).astype(np.float16), rng.normal(0, 0.1, (80000, 256)).astype(np.float16)
     run_graph("mix", lambda k: [(k.store(k.matmul(k.load(np_a), k.load(np_b), False, False)),
                                  np_a.astype(np.float32) @ np_b.astype(np.float32), 2e-3 * 30)], oracle_eps=2e-3 * 30)
+
+
+@pytest.mark.parametrize("waves", ["4", "8"])
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False), (True, True)])
+def test_big_tile_on_four_and_on_eight_waves(monkeypatch, waves, dtype, ta, tb):
+    # The 256x256 tile exists on four and on eight waves (the default depends on the layout): both builds, every
+    # layout, full tiles with a tail tile in m and n, an epilogue with a bias row and a second operand.
+    monkeypatch.setenv("DVM_CUBE_WAVES", waves)
+    monkeypatch.setenv("DVM_CUBE_TILE", "256")  # this size would get the 128x128 tile by itself
+    m, n, k = 1024 + 40, 2048 + 24, 512
+    r = np.random.default_rng(11)
+    af = (r.standard_normal([k, m] if ta else [m, k]) / 8).astype(np.float32)
+    bf = (r.standard_normal([n, k] if tb else [k, n]) / 8).astype(np.float32)
+    bias = r.standard_normal([n]).astype(np.float32)
+    other = r.standard_normal([m, n]).astype(np.float32)
+    t = Tester("mix")
+    if dtype == "bfloat16":
+        a16, b16 = Tester.convert_to_bf16(af), Tester.convert_to_bf16(bf)
+        a_ref, b_ref = Tester.convert_from_bf16(a16).astype(np.float64), Tester.convert_from_bf16(b16).astype(np.float64)
+        x, y = t.load(a16.shape, "bfloat16"), t.load(b16.shape, "bfloat16")
+        t.input(x, a16)
+        t.input(y, b16)
+    else:
+        a16, b16 = af.astype(np.float16), bf.astype(np.float16)
+        a_ref, b_ref = a16.astype(np.float64), b16.astype(np.float64)
+        x, y = t.load(a16), t.load(b16)
+    c = t.cast(t.matmul(x, y, ta, tb), "float32")
+    out = t.store(t.mul(t.add(c, t.load(bias)), t.load(other)))
+    t.run()
+    assert ("eight-waves" in t.das()) == (waves == "8"), t.das()
+    prod = (a_ref.T if ta else a_ref) @ (b_ref.T if tb else b_ref)
+    want = (prod + bias) * other
+    got = t.output(out).astype(np.float64)
+    assert np.allclose(got, want, rtol=1e-2, atol=1e-2), float(np.abs(got - want).max())
