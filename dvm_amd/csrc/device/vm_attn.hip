@@ -42,7 +42,6 @@ typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
 constexpr int D = DVM_ATTN_D;      // head dimension
 constexpr int BKV = DVM_ATTN_BKV;  // keys per block
-constexpr int WQ = 64;             // query rows per wave
 constexpr int ROW = 64;            // elements per local-memory tile row (128 bytes)
 
 __device__ __forceinline__ uint32_t uni(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
@@ -82,8 +81,16 @@ constexpr uint32_t kKTile = BKV * ROW;  // elements of one half tile
 constexpr uint32_t kVOff = 2 * kKTile;  // V block after the K block
 constexpr uint32_t kBuf = 4 * kKTile;   // elements per buffer
 
-template <bool IS_BF16>
+// NQT: 32-query tiles per wave. 2: four waves of 64 queries, one per SIMD with all 512 registers; 1: eight waves of
+// 32 queries, two per SIMD, so that one wave's softmax (vector ALU) runs under the other's MFMAs.
+template <bool IS_BF16, int NQT>
 __device__ __forceinline__ void vm_attn(const VmParam &p) {
+  constexpr int WQ = 32 * NQT;             // query rows per wave
+#ifndef DVM_ATTN_PIN8
+#define DVM_ATTN_PIN8 1
+#endif
+  constexpr bool PIN = NQT == 2 || DVM_ATTN_PIN8;
+  constexpr uint32_t NTHR = 64u * (DVM_ATTN_BQ / WQ);
   extern __shared__ double lds_raw[];
   uint16_t *lds = reinterpret_cast<uint16_t *>(lds_raw);
   const VAttnHeader *hp = reinterpret_cast<const VAttnHeader *>(p.w);
@@ -105,9 +112,9 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
 
   // Q fragments (B operand of stage 1): lane (j, h) holds Q[q0 + 32*qt + j][16*kk + 8*h .. +7]; rows
   // past the end repeat the last row (their results are never stored)
-  vu4 qf[2][D / 16];
+  vu4 qf[NQT][D / 16];
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < NQT; ++qt) {
     uint32_t row = q0 + 32 * qt + lj;
     row = row < sq ? row : sq - 1;
 #pragma unroll
@@ -116,13 +123,16 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
   }
 
   // Staging. A block of K or V is 64 keys x 128 d = two half tiles (d < 64, d >= 64) of 64 rows x 8 chunks of
-  // 16 bytes. Chunk position p = 256*i + tid (i = 0..3) of a block is half tile i/2, key 32*(i&1) + tid/8,
-  // physical chunk tid%8; the lane fetches the logical chunk that belongs there (physical ^ swizzle(key)),
-  // and a wave's 64 chunks land in 1 KB of consecutive local memory.
-  uint32_t ld_off[2];  // byte offset of the lane's chunk inside a block, for even / odd i
+  // 16 bytes. Chunk position p = NTHR*i + tid of a block is half tile p/512, key (p%512)/8, physical chunk tid%8
+  // (with 256 lanes: half tile i/2, key 32*(i&1) + tid/8; with 512: half tile i, key tid/8); the lane fetches
+  // the logical chunk that belongs there (physical ^ swizzle(key)), and a wave's 64 chunks land in 1 KB of
+  // consecutive local memory.
+  constexpr uint32_t KPS = NTHR / 8;       // keys one step of all lanes covers
+  constexpr int STEPS = 64 / KPS;          // steps per half tile
+  uint32_t ld_off[2];  // byte offset of the lane's chunk inside a block, for even / odd steps
 #pragma unroll
   for (int par = 0; par < 2; ++par) {
-    const uint32_t key = 32u * par + (tid >> 3);
+    const uint32_t key = KPS * par + (tid >> 3);
     const uint32_t logical = (tid & 7u) ^ ((key ^ (key >> 3)) & 7u);
     ld_off[par] = ((tid >> 3) * D + (logical << 3)) * 2u;
   }
@@ -132,20 +142,26 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
     const DVM_GLOBAL char *ksrc = reinterpret_cast<const DVM_GLOBAL char *>(k_base + static_cast<uint64_t>(key0) * D * 2);
     const DVM_GLOBAL char *vsrc = reinterpret_cast<const DVM_GLOBAL char *>(v_base + static_cast<uint64_t>(key0) * D * 2);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t src_off = (i & 1) * 32u * D * 2u + (i >> 1) * 64u * 2u + ld_off[i & 1];  // keys 32.. for odd i, d 64.. for i >= 2
-      const uint32_t dst_off = (static_cast<uint32_t>(i) * 256u + wave_first) * 8u;
+    for (int i = 0; i < 2 * STEPS; ++i) {
+      // step i % STEPS of half tile i / STEPS: later keys, then d 64..
+      const uint32_t src_off = (i % STEPS) * KPS * D * 2u + (i / STEPS) * 64u * 2u + ld_off[(i % STEPS) & 1];
+      const uint32_t dst_off = (static_cast<uint32_t>(i) * NTHR + wave_first) * 8u;
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(ksrc + src_off), (__attribute__((address_space(3))) void *)(kdst + dst_off), 16, 0, 0);
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(vsrc + src_off), (__attribute__((address_space(3))) void *)(vdst + dst_off), 16, 0, 0);
     }
   };
 
-  vf16 o_acc[D / 32][2];
+  vf16 o_acc[D / 32][NQT];
 #pragma unroll
   for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) o_acc[dt][qt] = 0.0f;
-  float m_run[2] = {-1.0e30f, -1.0e30f}, l_run[2] = {0.0f, 0.0f};
+    for (int qt = 0; qt < NQT; ++qt) o_acc[dt][qt] = 0.0f;
+  float m_run[NQT], l_run[NQT];
+#pragma unroll
+  for (int qt = 0; qt < NQT; ++qt) {
+    m_run[qt] = -1.0e30f;
+    l_run[qt] = 0.0f;
+  }
   const float c_log2 = scale * 1.44269504088896340736f;  // scores are handled in the log2 domain
 
   // Fragment reads. For row = 32*t + j of a tile the swizzle is swz0 ^ 4*(t & 1) with swz0 = (j ^ j>>3) & 7,
@@ -166,14 +182,11 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
   fetch_kv(0, 0);
   __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): the barrier does not wait for direct loads by itself
   __syncthreads();
-  for (uint32_t kb = 0; kb < n_blocks; ++kb) {
-    const uint32_t cur = kb & 1u;
-    const uint16_t *kbuf = lds + cur * kBuf, *vbuf = lds + cur * kBuf + kVOff;
-    // the other buffer was read for the last time before the barrier that ended the previous block
-    if (kb + 1 < n_blocks) fetch_kv((kb + 1) * BKV, cur ^ 1u);
-    // stage 1: S^T[key][query] for 2 key tiles x 2 query tiles. The fragments of step kk+1 are read while the
-    // MFMAs of step kk run (pinned: one wave per SIMD, nothing else would hide the local-memory latency).
-    vf16 s[2][2];
+  vf16 s[2][NQT];
+  vu4 pf[2][2][NQT];  // [key tile][16-key step][query tile]: B operand of stage 2
+  // stage 1: S^T[key][query] for 2 key tiles x NQT query tiles. The fragments of step kk+1 are read while the
+  // MFMAs of step kk run (pinned: with one wave per SIMD nothing else would hide the local-memory latency).
+  auto stage1 = [&](const uint16_t *kbuf) {
     vu4 kf[2][2];
     auto read_k = [&](int fb, int kk) {
 #pragma unroll
@@ -188,7 +201,7 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
+        for (int qt = 0; qt < NQT; ++qt) {
           if (kk == 0) {
             const vf16 zero = 0.0f;
             s[kt][qt] = mfma<IS_BF16>(kf[0][kt], qf[qt][0], zero);
@@ -196,19 +209,20 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
             s[kt][qt] = mfma<IS_BF16>(kf[kk & 1][kt], qf[qt][kk], s[kt][qt]);
           }
         }
-      if (kk + 1 < D / 16) {
+      if (kk + 1 < D / 16 && PIN) {  // the two fragment reads of the next step between the 2 * NQT MFMAs of this one
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
         __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        if (NQT == 2) __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    // softmax of this block, per query (= per lane, both half-waves share a query)
-    vu4 pf[2][2][2];  // [key tile][16-key step][query tile]: B operand of stage 2
+  };
+  // softmax of a block, per query (= per lane, both half-waves share a query)
+  auto softmax = [&]() {
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
+    for (int qt = 0; qt < NQT; ++qt) {
       float mx = s[0][qt][0];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
@@ -240,9 +254,11 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
       }
     }
     __builtin_amdgcn_sched_barrier(0);
-    // stage 2: O^T[d][query] += V^T[d][key] P^T[key][query]. Step (kt, st) contracts the 16 keys the
-    // lane's registers 8*st .. 8*st+7 of tile kt hold: keys 32*kt + 16*st + {0..3, 8..11} + 4*h. Fragments
-    // of the next step are read under the MFMAs of the current one.
+  };
+  // stage 2: O^T[d][query] += V^T[d][key] P^T[key][query]. Step (kt, st) contracts the 16 keys the
+  // lane's registers 8*st .. 8*st+7 of tile kt hold: keys 32*kt + 16*st + {0..3, 8..11} + 4*h. Fragments
+  // of the next step are read under the MFMAs of the current one.
+  auto stage2 = [&](const uint16_t *vbuf) {
     vu4 vf[2][D / 32];
     auto read_v = [&](int fb, int step) {
       const int kt = step >> 1, st = step & 1;
@@ -268,16 +284,27 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
 #pragma unroll
       for (int dt = 0; dt < D / 32; ++dt)
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) o_acc[dt][qt] = mfma<IS_BF16>(vf[step & 1][dt], pf[step >> 1][step & 1][qt], o_acc[dt][qt]);
-      if (step + 1 < 4) {
+        for (int qt = 0; qt < NQT; ++qt) o_acc[dt][qt] = mfma<IS_BF16>(vf[step & 1][dt], pf[step >> 1][step & 1][qt], o_acc[dt][qt]);
+      if (step + 1 < 4 && PIN) {  // the eight transposing reads of the next step between the 4 * NQT MFMAs of this one
 #pragma unroll
-        for (int q = 0; q < 8; ++q) {
+        for (int q = 0; q < 4 * NQT; ++q) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 8 / (4 * NQT), 0);
         }
       }
     }
     __builtin_amdgcn_sched_barrier(0);
+  };
+  // Running the waves that share a SIMD one phase apart (softmax and stage 2 of block kb-1, then stage 1 of block
+  // kb, with a third K/V buffer) was measured with eight waves and is slower (819-835 us against 767-788 us): the
+  // hardware interleaves the two waves well enough, and the rotation costs 50 registers.
+  for (uint32_t kb = 0; kb < n_blocks; ++kb) {
+    const uint32_t cur = kb & 1u;
+    // the other buffer was read for the last time before the barrier that ended the previous block
+    if (kb + 1 < n_blocks) fetch_kv((kb + 1) * BKV, cur ^ 1u);
+    stage1(lds + cur * kBuf);
+    softmax();
+    stage2(lds + cur * kBuf + kVOff);
     __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): the next block has landed
     __syncthreads();
   }
@@ -285,7 +312,7 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
   // O[query][d] = O^T / l, rounded once to the operand type. Lane (j, h) holds, per d tile and register
   // group g, d = 32*dt + 8*g + 4*h + 0..3: four consecutive values = one 8-byte store.
 #pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
+  for (int qt = 0; qt < NQT; ++qt) {
     const float l = l_run[qt] + __shfl_xor(l_run[qt], 32);
     const float inv = 1.0f / l;
     const uint32_t row = q0 + 32 * qt + lj;
@@ -306,5 +333,7 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
 
 }  // namespace
 
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_f16(const VmParam p) { vm_attn<false>(p); }
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_bf16(const VmParam p) { vm_attn<true>(p); }
+extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_f16(const VmParam p) { vm_attn<false, 2>(p); }
+extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_bf16(const VmParam p) { vm_attn<true, 2>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_attn_f16_w8(const VmParam p) { vm_attn<false, 1>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_attn_bf16_w8(const VmParam p) { vm_attn<true, 1>(p); }

@@ -2546,7 +2546,12 @@ void Compiler::CompileAttn(int gi) {
   } else {
     Fail("attention result has no destination");
   }
-  prog_->threads = 256;
+  // eight waves of 32 queries (two per SIMD: one wave's softmax runs under the other's MFMAs) measured 767-788 us
+  // on fp16 [8,32,2048,128] against 920-940 us for four waves of 64 queries; DVM_ATTN_WAVES=4 selects the latter
+  prog_->threads = 512;
+  if (const char *e = std::getenv("DVM_ATTN_WAVES")) {
+    if (std::atoi(e) == 4) prog_->threads = 256;
+  }
   prog_->lds_bytes = DVM_ATTN_LDS_BYTES;
   prog_->grid = h.nb * h.q_blocks;
 }

@@ -51,9 +51,11 @@ def _fused(q, k, v, dt="float16"):
     return Tester.convert_from_bf16(o) if dt == "bfloat16" else o
 
 
+@pytest.mark.parametrize("waves", ["8", "4"])  # the kernel has a build on eight waves (the default) and one on four
 @pytest.mark.parametrize("shape", [((2, 3), 256, 192), ((1,), 64, 64), ((3,), 100, 128), ((2, 2), 300, 2048), ((), 513, 640)])
 @pytest.mark.parametrize("dt", ["float16", "bfloat16"])
-def test_attention_fused(shape, dt):
+def test_attention_fused(monkeypatch, shape, dt, waves):
+    monkeypatch.setenv("DVM_ATTN_WAVES", waves)
     batch, sq, skv = shape
     rng = np.random.default_rng(sq)
     conv = (lambda x: x.astype(np.float16)) if dt == "float16" else _bf16
