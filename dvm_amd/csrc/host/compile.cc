@@ -786,6 +786,7 @@ class Compiler {
   bool conservative_ = false;
   int mode_ = 0;
   bool single_round_ = false;
+  bool split_inner_ = false;  // pointwise programs with a gathered operand walk the innermost axis in tiles of 64
   int acc_node_ = -1;
   uint32_t sreg_used_ = 0;
   uint32_t vslot_used_ = 0;
@@ -1301,7 +1302,31 @@ void Compiler::ChooseSchedule() {
   u_ = wide ? DVM_VEC_U_WIDE : 2;
   const uint32_t U = static_cast<uint32_t>(u_);
   const uint32_t max_threads = wide ? 512u : 1024u;
+  split_inner_ = false;
   if (nr_ == 0) {
+    // A gathered operand (innermost stride neither 0 nor 1: a transposing view) is read element by element. In
+    // the plain order a workgroup's slabs run along the innermost axis, so of every cache line it fetches it
+    // uses 4 bytes, and the workgroups that use the rest run elsewhere, most of them behind another L2. With the
+    // innermost axis walked in tiles of 64 elements (8 slabs) and the next axis inside that, a workgroup covers
+    // 64 x 64 elements and uses every line it fetches in full:
+    // kept dims [8 slabs][the other dims ...][innermost extent / 64].
+    static const bool tile_gather = !(std::getenv("DVM_VEC_GATHER_TILE") != nullptr && std::getenv("DVM_VEC_GATHER_TILE")[0] == '0');
+    if (tile_gather && nk_ >= 2 && nk_ < DVM_VEC_MAXR && klist_[0] == inner && dims_[inner].extent % (8 * E) == 0) {
+      for (int i = 0; i < nn_ && !split_inner_; ++i) {
+        const ANode &n = nodes_[i];
+        if ((n.kind != AK_MEM && n.kind != AK_OUT) || n.view == nullptr) continue;
+        for (int d = 0; d < n.rank; ++d) {
+          if (n.axis[d] < 0 || pos_[n.axis[d]] != dims_[inner].last_axis) continue;
+          const int64_t st = n.view->vstride_[d];
+          if (st != 0 && st != 1) split_inner_ = true;
+        }
+      }
+    }
+    if (split_inner_) {
+      hdr_.kdims[0] = MakeVDim(8);  // the other dims keep their places, the tiles go behind them
+      hdr_.kdims[nk_] = MakeVDim(static_cast<uint32_t>(inner_groups / 8));
+      hdr_.n_kdim = nk_ + 1;
+    }
     hdr_.sched = VS_POINTWISE;
     if (n_k <= 64 * U) threads = 64;
     else if (n_k <= 128 * U) threads = 128;
@@ -1390,6 +1415,10 @@ int Compiler::MemIndex(int v) {
     if (dim_stride[md] >= (1ll << 32)) Fail("stride above 2^32");
     m.kstride[i] = static_cast<uint32_t>(dim_stride[md]);
     if (md != inner && (dim_stride[md] * isz) % need != 0) aligned = false;
+  }
+  if (split_inner_ && dim_has[inner]) {  // the tiles of 64 along the innermost axis are the outermost kept dim
+    if (dim_stride[inner] * 64 >= (1ll << 32)) Fail("stride above 2^32");
+    m.kstride[nk_] = static_cast<uint32_t>(dim_stride[inner] * 64);
   }
   for (int i = 0; i < nr_; ++i) {
     const int md = rlist_[i];

@@ -404,6 +404,10 @@ def test_strided_views_in_das_mode():
     c = np.zeros([100, 2048], np.float32)
     t, das = _das(lambda t: t.store(t.add(t.view_load([100, 200], [2048, 10], c), 0.1)))
     assert " gather" in das
+    # a transposing view in a pointwise program: the innermost axis is walked in tiles of 64 with the next axis inside
+    e2 = np.zeros([2048, 4096], np.float32)
+    t, das = _das(lambda t: t.store(t.add(t.view_load([4096, 2048], [1, 4096], e2), 0.0)))
+    assert "kdims: 8 4096 32 " in das and "k[4096,1,262144]" in das and "k[1,2048,64]" in das
     # six dims that cannot merge: four run inside the program, the two outermost become launches
     d = np.zeros([4, 4, 4, 5, 6, 16], np.float32)
     t, das = _das(lambda t: t.store(t.add(t.view_load([3, 2, 3, 4, 5, 12], dense(list(d.shape)), d), 0.1)))
