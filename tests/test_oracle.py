@@ -212,3 +212,46 @@ def test_batchnorm_restatement():
     want = (x64 - x64.mean((0, 2, 3), keepdims=True)) / np.sqrt(x64.var((0, 2, 3), keepdims=True) + 1e-5)
     want = want * g[None, :, None, None] + b[None, :, None, None]
     assert np.allclose(ora.batchnorm_nchw(x, g, b, 1e-5), want, rtol=1e-5, atol=1e-5)
+
+
+def test_view_ops_against_element_loops():
+    # The view operators of the oracle (strided loads and stores, slices, permute, split, concat) against plain
+    # element-by-element loops over the flat buffer and against the values the reference's own tests expect
+    # (tests/ut/test_view.py: every tenth column, a transpose, zero strides, an element offset; tests/ut/test_slice.py:
+    # negative and out-of-range bounds), on inputs whose elements are all different.
+    k = OracleKernel()
+    a = np.arange(6 * 40, dtype=np.float32).reshape(6, 40)
+    flat = a.reshape(-1)
+
+    def by_loops(shape, stride, offset=0):
+        out = np.zeros(shape, np.float32)
+        for idx in np.ndindex(*shape):
+            out[idx] = flat[offset + sum(i * s for i, s in zip(idx, stride))]
+        return out
+    for shape, stride, offset in [([6, 4], [40, 10], 0), ([40, 6], [1, 40], 0), ([3, 5, 8], [80, 0, 2], 7), ([2, 20], [40, 1], 60)]:
+        assert np.array_equal(k.output(k.view_load(shape, stride, a, offset)), by_loops(shape, stride, offset))
+    assert np.array_equal(k.output(k.view_load([6, 4], [40, 10], a)), a[:, 0:40:10])         # tests/ut/test_view.py:137-144
+    assert np.array_equal(k.output(k.view_load([40, 6], [1, 40], a)), a.T)                   # :183-201
+    assert np.array_equal(k.output(k.slice_load(a, (1, 3), (4, 20))), a[1:5, 3:23])
+    assert np.array_equal(k.output(k.stridedslice_load(a, (-5, 0), (100, 40), (1, 1))), a[-5:100])  # tests/ut/test_slice.py:76-89
+    assert np.array_equal(k.output(k.stridedslice_load(a, (1, 2), (-2, 38), (2, 3))), a[1:-2:2, 2:38:3])
+    # a strided store: element i, j of the value lands at i * 50 + j * 2 of a zero-filled buffer
+    v = k.load(a[:3, :10])
+    e = np.zeros([4, 50], np.float32)
+    got = k.output(k.view_store_expect(v, [50, 2], e))
+    want = np.zeros(200, np.float32)
+    for i in range(3):
+        for j in range(10):
+            want[i * 50 + j * 2] = a[i, j]
+    assert np.array_equal(got, want.reshape(4, 50))
+    # permute: result dim i is input dim dims[i] (include/dvm.h:428-434 of the reference)
+    b = np.arange(2 * 3 * 4, dtype=np.float32).reshape(2, 3, 4)
+    p = k.output(k.permute(k.load(b), [2, 0, 1]))
+    assert p.shape == (4, 2, 3) and all(p[z, x, y] == b[x, y, z] for x in range(2) for y in range(3) for z in range(4))
+    # slices of values, split with a smaller last chunk, concat
+    assert np.array_equal(k.output(k.slice(k.load(a), [1, 5], [2, 7])), a[1:3, 5:12])
+    assert np.array_equal(k.output(k.slice_dim(k.load(a), 1, 5, -2)), a[:, 5:38])
+    parts = k.split(k.load(a), 1, 16, 3)
+    assert [k.output(x).shape for x in parts] == [(6, 16), (6, 16), (6, 8)] and np.array_equal(k.output(parts[2]), a[:, 32:])
+    c = k.output(k.concat([parts[2], parts[0]], 1))
+    assert c.shape == (6, 24) and np.array_equal(c[:, :8], a[:, 32:]) and np.array_equal(c[:, 8:], a[:, :16])
