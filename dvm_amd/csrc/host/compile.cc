@@ -629,6 +629,20 @@ class Compiler {
       if (ai.has_reduce && !SameReduce(ai.reduce, o)) return false;
       return mode_ == 0 || DomCompatible(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
     }
+    // A store of a value from outside (a load, a view, another launch's result) is a copy nothing else in the
+    // sub-kernel relates to: it joins only one whose index space it fills, element for element.
+    if (IsStoreLike(o) && ai.n_ops > 0) {  // same extents in the same order, dims of extent 1 aside
+      int i = 0, j = 0;
+      while (true) {
+        while (i < ai.rank && ai.dom[i] == 1) ++i;
+        while (j < o->rank() && o->dim(j) == 1) ++j;
+        if (i == ai.rank || j == o->rank()) break;
+        if (ai.dom[i] != o->dim(j)) return false;
+        ++i;
+        ++j;
+      }
+      if (i != ai.rank || j != o->rank()) return false;
+    }
     return mode_ == 0 || DomCompatible(ai, o->shape_ref_->data, o->rank());
   }
 
@@ -1106,9 +1120,21 @@ void Compiler::UnifyAxes() {
       }
       if (find(i) == find(anchor)) continue;
       const ANode &o = nodes_[i], &f = nodes_[anchor];
-      for (int d = 0; d < o.rank; ++d) {
-        const int fd = d + f.rank - o.rank;
-        if (fd >= 0 && o.dims[d] != 1 && o.dims[d] == f.dims[fd]) Union(Var(i, d), Var(anchor, fd));
+      // the k-th dim of extent > 1 of the one is the k-th of the other when they list the same extents ...
+      int od[kMaxRank], fdm[kMaxRank], no = 0, nf = 0;
+      for (int d = 0; d < o.rank; ++d)
+        if (o.dims[d] != 1) od[no++] = d;
+      for (int d = 0; d < f.rank; ++d)
+        if (f.dims[d] != 1) fdm[nf++] = d;
+      bool same = no == nf;
+      for (int q = 0; q < no && same; ++q) same = o.dims[od[q]] == f.dims[fdm[q]];
+      if (same) {
+        for (int q = 0; q < no; ++q) Union(Var(i, od[q]), Var(anchor, fdm[q]));
+      } else {  // ... else dim by dim from the right, where the extents agree
+        for (int d = 0; d < o.rank; ++d) {
+          const int fd = d + f.rank - o.rank;
+          if (fd >= 0 && o.dims[d] != 1 && o.dims[d] == f.dims[fd]) Union(Var(i, d), Var(anchor, fd));
+        }
       }
       comp[find(i)] = find(anchor);
     }

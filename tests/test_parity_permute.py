@@ -475,3 +475,25 @@ def test_sch_diamonds_of_slices_and_concats():  # :698-760
     run_graph("", g2)
     run_graph("", g3)
     run_graph("", g4)
+
+
+def test_copies_of_views_with_other_shapes_do_not_share_a_launch_wrongly():
+    # found by random graphs: stores of views of one value whose shapes differ (a chunk and a single element; the same
+    # three elements as [1,3,1] and, permuted, as [3,1,1]) were put into one launch whose index space fitted neither
+    a = rng(90).normal(0, 1, [5, 3, 24]).astype(np.float32)
+    b = rng(91).normal(0, 1, [5, 3, 24]).astype(np.float32)
+
+    def g1(k):
+        x = k.add(k.load(a), k.load(b))
+        parts = k.split(x, 2, 8, 3)
+        return [(k.store(k.mul(parts[1], 2.0)), (a + b)[:, :, 8:16] * np.float32(2.0), None),
+                (k.store(k.slice(parts[0], [4, 2, 3], [1, 1, 1])), (a + b)[4:5, 2:3, 3:4], None)]
+    run_graph("", g1)
+    c = rng(92).normal(0, 1, [5, 5, 128]).astype(np.float32)
+
+    def g2(k):
+        s = k.slice(k.load(c), [3, 2, 108], [1, 3, 16])
+        parts = k.split(s, 2, 1, 16)
+        return [(k.store(k.mul(parts[5], 2.0)), c[3:4, 2:5, 113:114] * np.float32(2.0), None),
+                (k.store(k.permute(k.slice_dim(parts[7], 0, 0, 1), [1, 0, 2])), np.transpose(c[3:4, 2:5, 115:116], (1, 0, 2)), 0)]
+    run_graph("", g2)
