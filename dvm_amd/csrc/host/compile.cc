@@ -800,6 +800,8 @@ class Compiler {
   bool conservative_ = false;
   int mode_ = 0;
   bool single_round_ = false;
+  int held_[kMaxNodes];  // registers whose release waits for the end of the sweep
+  int n_held_ = 0;
   bool split_inner_ = false;  // pointwise programs with a gathered operand walk the innermost axis in tiles of 64
   int acc_node_ = -1;
   uint32_t sreg_used_ = 0;
@@ -1550,7 +1552,16 @@ void Compiler::ConsumeUse(int v) {
   ANode &n = nodes_[v];
   if (n.uses > 0) --n.uses;
   const bool needed_later = n.last_sec > cur_sec_ && (!n.fd || single_round_);
-  if (n.uses == 0 && !needed_later && n.reg >= 0) ReleaseReg(v);
+  if (n.uses != 0 || needed_later || n.reg < 0) return;
+  // A sweep of several rounds runs its instructions again: a value from an earlier section keeps its
+  // register until the sweep ends, or a temporary of round one would replace it before round two reads it.
+  if ((cur_sec_ & 1) && !single_round_ && n.sec < cur_sec_) {
+    bool listed = false;
+    for (int i = 0; i < n_held_; ++i) listed |= held_[i] == v;
+    if (!listed) held_[n_held_++] = v;
+    return;
+  }
+  ReleaseReg(v);
 }
 
 bool Compiler::SimpleOperand(int v) {
@@ -1899,6 +1910,9 @@ void Compiler::EmitSection(int sec) {
     Emit(VOP_ENDSWEEP, 0, 0, 0, 0, 0);
     if (!single_round_) acc_node_ = -1;
   }
+  for (int i = 0; i < n_held_; ++i)
+    if (nodes_[held_[i]].uses == 0) ReleaseReg(held_[i]);
+  n_held_ = 0;
 }
 
 void Compiler::EmitProgram() {

@@ -495,3 +495,23 @@ def test_clone_carries_views():
     assert out2.shape() == out.shape() == (60, 6)
     strip = lambda d: "\n".join(l for l in d.splitlines() if "@0x" not in l)  # addresses differ, programs do not
     assert strip(t2.das()) == strip(t.das()) and t.das().count("== sub-kernel") >= 3
+
+
+def test_values_of_earlier_sections_keep_their_registers_through_a_sweep():
+    # 33 rows on a team of 16 lanes with two slabs each: the second sweep runs twice, so the register that holds
+    # twice the column maximum may not be handed to a temporary inside that sweep
+    t = Tester("", run_mode="das")
+    x = t.load(np.ones((33, 100), np.float32))
+    m = t.max(x, (0,), True)
+    m2 = t.add(m, m)
+    t.store(t.select(t.greater(x, m2), x, m2))
+    second = t.select(t.greater(m, x), m, x)
+    t.store(t.sub(second, x))
+    t.codegen()
+    lines = [l.strip() for l in t.das().splitlines()]
+    sweep2 = lines[[i for i, l in enumerate(lines) if l.startswith("sweep")][1]:]
+    held = [l.split()[1].rstrip(",") for l in lines if l.startswith("mov v") and lines.index(l) < lines.index(sweep2[0])]
+    assert held, t.das()
+    for l in sweep2:
+        if l.startswith("mov v"):
+            assert l.split()[1].rstrip(",") not in held, t.das()

@@ -235,3 +235,19 @@ def test_wide_build_matches(monkeypatch):
     t.store(t.sum(t.load(x), (2,), False))
     t.codegen()
     assert " wide " in t.das()
+
+
+@pytest.mark.parametrize("shape,axis", [((33, 100), 0), ((70, 257), 0), ((5, 3000), 1), ((3, 5000, 8), 1)])
+def test_reduce_result_outlives_temporaries_of_later_rounds(shape, axis):
+    # a second sweep of several rounds reads the reduce result in every round: temporaries of the first round
+    # must not take its register (two outputs with a compare each make the emitter park a mask per output)
+    x = np.random.default_rng(1161).uniform(0.25, 2.0, shape).astype(np.float32)
+
+    def build(k, a):
+        m = k.max(a, (axis,), True)
+        m2 = k.add(m, m)
+        first = k.select(k.greater(a, m2), a, m2)
+        second = k.select(k.greater(m, a), m, a)
+        return [first, k.sub(second, a)]
+    mx = x.max(axis, keepdims=True)
+    run_parity(build, [x], golden=[np.broadcast_to(2 * mx, shape), np.broadcast_to(mx, shape) - x], eps=0)
