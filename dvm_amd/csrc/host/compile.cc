@@ -1101,8 +1101,8 @@ void Compiler::UnifyAxes() {
         if (x.dims[d] != 1 && x.dims[d] == f.dims[d]) Union(Var(nodes_[i].in[0], d), Var(first, d));
     }
   }
-  // Outputs that no operator relates to the first one (consumers of two different views of one buffer, each
-  // with its own store) walk the same index space too: unified with it dim by dim from the right.
+  // Parts of the sub-kernel that no operator relates to each other (consumers of two different views of one
+  // buffer, each with its own store; a copy beside a reduce) walk the same index space too.
   {
     std::vector<int> comp(nn_);
     for (int i = 0; i < nn_; ++i) comp[i] = i;
@@ -1113,14 +1113,26 @@ void Compiler::UnifyAxes() {
     for (int i = 0; i < nn_; ++i)
       for (int j = 0; j < nodes_[i].nin; ++j)
         if (nodes_[i].in[j] >= 0) comp[find(i)] = find(nodes_[i].in[j]);
-    int anchor = -1;
+    // Each component is matched through its node with the most dims of extent > 1 (an output of a reduce has
+    // fewer dims than the walk that produces it); the component of the widest output is the anchor.
+    auto wide = [&](int v) {
+      int c = 0;
+      for (int d = 0; d < nodes_[v].rank; ++d) c += nodes_[v].dims[d] != 1;
+      return c;
+    };
+    std::vector<int> rep(nn_, -1);
     for (int i = 0; i < nn_; ++i) {
-      if (nodes_[i].kind != AK_OUT) continue;
-      if (anchor < 0) {
-        anchor = i;
-        continue;
-      }
-      if (find(i) == find(anchor)) continue;
+      if (nodes_[i].kind == AK_SCALAR) continue;
+      int &r = rep[find(i)];
+      if (r < 0 || wide(i) > wide(r)) r = i;
+    }
+    int anchor_out = -1;
+    for (int i = 0; i < nn_; ++i)
+      if (nodes_[i].kind == AK_OUT && (anchor_out < 0 || wide(rep[find(i)]) > wide(rep[find(anchor_out)]))) anchor_out = i;
+    const int anchor = anchor_out < 0 ? -1 : rep[find(anchor_out)];
+    for (int c = 0; c < nn_ && anchor >= 0; ++c) {
+      if (find(c) != c || rep[c] < 0 || c == find(anchor)) continue;
+      const int i = rep[c];
       const ANode &o = nodes_[i], &f = nodes_[anchor];
       // the k-th dim of extent > 1 of the one is the k-th of the other when they list the same extents ...
       int od[kMaxRank], fdm[kMaxRank], no = 0, nf = 0;
@@ -1138,7 +1150,6 @@ void Compiler::UnifyAxes() {
           if (fd >= 0 && o.dims[d] != 1 && o.dims[d] == f.dims[fd]) Union(Var(i, d), Var(anchor, fd));
         }
       }
-      comp[find(i)] = find(anchor);
     }
   }
   // classes with extent > 1 become domain axes

@@ -251,3 +251,20 @@ def test_reduce_result_outlives_temporaries_of_later_rounds(shape, axis):
         return [first, k.sub(second, a)]
     mx = x.max(axis, keepdims=True)
     run_parity(build, [x], golden=[np.broadcast_to(2 * mx, shape), np.broadcast_to(mx, shape) - x], eps=0)
+
+
+@pytest.mark.parametrize("three", [False, True])
+def test_copy_beside_a_reduce_to_one_element(three):
+    # an output of one element relates to no other output; the copies next to it are matched through the
+    # reduce's input, which has the dims the launch walks
+    x = np.random.default_rng(18).uniform(0.25, 2.0, [1, 2, 3000]).astype(np.float16)
+
+    def build(k, a):
+        f = k.cast(a, "float32")
+        flat = k.reshape(f, [6000])
+        other = k.reshape(k.mul(f, f), [6000])
+        outs = [other, k.sum(flat, (0,), True)]
+        return outs + [k.add(flat, 0.0)] if three else outs
+    xf = x.astype(np.float32).reshape(6000)
+    golden = [xf * xf, xf.sum(keepdims=True)] + ([xf] if three else [])
+    run_parity(build, [x], golden=golden, eps=1e-5)
