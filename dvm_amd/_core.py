@@ -445,14 +445,14 @@ class PyKernel(Kernel):
 
     @staticmethod
     def convert_to_bf16(array):
-        src = np.ascontiguousarray(array, dtype=np.float32)
+        src = np.asarray(array, dtype=np.float32, order="C")  # keeps rank 0, which ascontiguousarray would not
         dst = np.empty(src.shape, dtype=np.uint16)
         _lib.dvm_c_f32_to_bf16(src.ctypes.data, dst.ctypes.data, src.size)
         return dst
 
     @staticmethod
     def convert_from_bf16(array):
-        src = np.ascontiguousarray(array, dtype=np.uint16)
+        src = np.asarray(array, dtype=np.uint16, order="C")
         dst = np.empty(src.shape, dtype=np.float32)
         _lib.dvm_c_bf16_to_f32(src.ctypes.data, dst.ctypes.data, src.size)
         return dst
@@ -465,7 +465,7 @@ class PyKernel(Kernel):
         if isinstance(load, IntArrayRef):
             load.update(list(array))
             return
-        arr = np.ascontiguousarray(array)
+        arr = np.asarray(array, order="C")
         if offset:
             _check(_lib.dvm_obj_set_view_offset(load._h, int(offset)))
         ref = self._load_shape.get(load._h)

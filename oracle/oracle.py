@@ -72,7 +72,7 @@ def _p(a):
 
 
 def _c(a, dt):
-    return np.ascontiguousarray(a, dtype=dt)
+    return np.asarray(a, dtype=dt, order="C")  # a value of rank 0 keeps its rank (src/ops.cc:3080-3117 reduces to rank 0)
 
 
 # ---- raw functors on arrays ---------------------------------------------------------

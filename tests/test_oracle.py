@@ -255,3 +255,15 @@ def test_view_ops_against_element_loops():
     assert [k.output(x).shape for x in parts] == [(6, 16), (6, 16), (6, 8)] and np.array_equal(k.output(parts[2]), a[:, 32:])
     c = k.output(k.concat([parts[2], parts[0]], 1))
     assert c.shape == (6, 24) and np.array_equal(c[:, :8], a[:, 32:]) and np.array_equal(c[:, 8:], a[:, :16])
+
+
+def test_values_of_rank_zero_keep_their_rank():
+    # a reduce over every dim without keepdims has rank 0 (src/ops.cc:3080-3117); operators on it keep that rank
+    from oracle.oracle import OracleKernel
+    k = OracleKernel()
+    x = k.load(np.arange(5, dtype=np.float32))
+    m = k.max(x, (0,), False)
+    y = k.floor(k.add(m, 0.5))
+    assert k.output(k.store(m)).shape == () and k.output(k.store(y)).shape == ()
+    assert float(k.output(k.store(y))) == 4.0
+    assert k.output(k.store(k.add(x, y))).shape == (5,)

@@ -268,3 +268,16 @@ def test_copy_beside_a_reduce_to_one_element(three):
     xf = x.astype(np.float32).reshape(6000)
     golden = [xf * xf, xf.sum(keepdims=True)] + ([xf] if three else [])
     run_parity(build, [x], golden=golden, eps=1e-5)
+
+
+def test_operators_on_a_value_of_rank_zero():  # src/ops.cc:3080-3117: a reduce over every dim without keepdims
+    x = np.random.default_rng(5).uniform(-2, 2, [257]).astype(np.float32)
+
+    def build(k, a):
+        m = k.min(a, (0,), False)
+        r = k.floor(k.add(m, 0.25))
+        return [m, r, k.mul(a, r)]
+    outs = run_parity(build, [x], golden=[x.min(), np.floor(x.min() + np.float32(0.25)), x * np.floor(x.min() + np.float32(0.25))], eps=0)
+    assert outs[0].shape == () and outs[1].shape == () and outs[2].shape == (257,)
+    bf = Tester.convert_from_bf16(Tester.convert_to_bf16(np.float32(1.5)))
+    assert bf.shape == () and float(bf) == 1.5
