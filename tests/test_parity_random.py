@@ -122,3 +122,29 @@ def test_random_graphs_compile_without_a_gpu():
                 assert any(s in str(e) for s in ("needs a Copy", "not supported", "too many")), "case %d: %s" % (case, e)
                 continue
             assert "== sub-kernel" in t.das() or t.das() == ""
+
+
+@gpu
+@pytest.mark.parametrize("first", range(0, 120, 30))
+def test_attention_shapes(first):
+    # examples/03_attention.py:20-50 at random sizes: head dim 128 takes the fused kernel (any number of queries and
+    # keys, ragged tiles included), other head dims the three-launch path; 1e-2 against NumPy as in the example
+    import math
+    from tests.test_parity_attention import attention_graph, np_attention, _bf16
+    for case in range(first, first + 30):
+        rng = np.random.default_rng(7000 + case)
+        batch = [(), (1,), (3,), (2, 2)][int(rng.integers(0, 4))]
+        d = 128 if rng.random() < 0.7 else int(rng.choice([8, 64, 72, 256]))
+        sq = int(rng.choice([1, 5, 31, 32, 33, 64, 100, 127, 129, 255, 256, 400, 700]))
+        skv = int(rng.choice([1, 7, 63, 64, 65, 128, 200, 511, 513, 1000, 3000]))
+        dt = "float16" if rng.random() < 0.5 else "bfloat16"
+        conv = (lambda x: x.astype(np.float16)) if dt == "float16" else _bf16
+        q, k, v = (conv(rng.standard_normal(batch + (n, d))) for n in (sq, skv, skv))
+        t = Tester("mix")
+        dts = dt if dt == "bfloat16" else None
+        out = t.store(attention_graph(t, t.load(q, dts), t.load(k, dts), t.load(v, dts), 1.0 / math.sqrt(d), q.ndim, dt))
+        t.run()
+        got = _read(t, out)
+        want = np_attention(q, k, v)
+        assert got.shape == want.shape, (case, got.shape, want.shape)
+        assert np.allclose(got, want, rtol=1e-2, atol=1e-2), (case, batch, sq, skv, d, dt, float(np.abs(got - want).max()))
