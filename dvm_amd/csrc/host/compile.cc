@@ -1255,6 +1255,8 @@ void Compiler::OrderAndMerge() {
         }
       }
     }
+    // device coordinates are 32 bits wide: a tensor of 2^32 elements or more keeps its outer dims apart
+    if (merge && dims_[n_dims_ - 1].extent * axes_[order_[k]].extent >= (1ll << 32)) merge = false;
     if (merge) {
       dims_[n_dims_ - 1].extent *= axes_[order_[k]].extent;
       dims_[n_dims_ - 1].last_axis = k;

@@ -255,3 +255,17 @@ def test_graph_longer_than_one_program():  # tests/ut/test_eager_fusion.py:551-8
     t.run()
     assert 2 <= t.num_launches() <= 10
     assert np.array_equal(t.output(out), want)
+
+
+def test_tensor_of_more_than_2_32_elements():
+    # 5 x 2^30 one-byte elements: device coordinates are 32 bits wide, so the two dims stay apart instead of being
+    # merged into one flat axis; the second operand varies along the outer dim only
+    pat = np.random.default_rng(0).random(1 << 20) < 0.5
+    x = np.tile(pat, 5 * 1024).reshape(5, 1 << 30)
+    col = np.array([[True], [False], [True], [True], [False]])
+    t = Tester("")
+    st = t.store(t.logical_and(t.logical_not(t.load(x)), t.load(col)))
+    t.run()
+    out = t.output(st)
+    assert out.shape == x.shape and out.dtype == np.bool_
+    assert np.array_equal(out, ~x & col)
