@@ -24,7 +24,7 @@ def _load():
         raise ImportError(
             "dvm_amd native library missing (%s): run `python -m dvm_amd.build` first" % _LIB_PATH)
     lib = ctypes.CDLL(_LIB_PATH)
-    if not hasattr(lib, "dvm_rt_seq_add"):
+    if not hasattr(lib, "dvm_rt_unbind_device"):
         raise ImportError("dvm_amd native library (%s) is older than the package: run `python -m dvm_amd.build`"
                           % _LIB_PATH)
     vp, ci, cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -71,6 +71,7 @@ def _load():
         "dvm_obj_dtype": (ci, [vp]),
         "dvm_rt_input": (ci, [vp, vp, vp, cs]),
         "dvm_rt_bind_device": (ci, [vp, vp, vp]),
+        "dvm_rt_unbind_device": (ci, [vp]),
         "dvm_rt_normalize": (ci, [vp]),
         "dvm_rt_codegen": (ci, [vp]),
         "dvm_rt_jit_us": (ctypes.c_double, [vp]),
@@ -80,6 +81,8 @@ def _load():
         "dvm_rt_perf": (ci, [vp, ci, ci, ctypes.POINTER(ctypes.c_double)]),
         "dvm_rt_num_launches": (ci, [vp]),
         "dvm_rt_workspace_bytes": (cs, [vp]),
+        "dvm_rt_program_count": (ci, [vp]),
+        "dvm_rt_program": (ci, [vp, ci, vp, ctypes.POINTER(ctypes.c_uint32), ctypes.POINTER(ctypes.c_uint32), cs]),
         "dvm_rt_das": (ctypes.c_char_p, [vp]),
         "dvm_rt_dump": (ctypes.c_char_p, [vp]),
         "dvm_rt_dump_r": (ctypes.c_char_p, [vp]),
@@ -487,14 +490,24 @@ class PyKernel(Kernel):
         """Shape inference only: store.shape() is valid afterwards."""
         _check(_lib.dvm_rt_normalize(self._rt))
 
+    def release_device_bindings(self):
+        """Forgets caller-owned device memory bound earlier; the next input() / codegen() use buffers of the runner."""
+        _check(_lib.dvm_rt_unbind_device(self._rt))
+
     def codegen(self, pass_names=None):
+        """Normalize + CodeGen. The gfx950 pipeline is fixed: naming passes is an error, not a silent no-op."""
+        if pass_names:
+            raise RuntimeError("DVM EXCEPTION. reason: passes are fixed on the gfx950 backend (asked for: %s)" % ", ".join(pass_names))
         _check(_lib.dvm_rt_codegen(self._rt))
 
     def jit_us(self):
         return _lib.dvm_rt_jit_us(self._rt)
 
-    def run(self, stream=None, sync=True):
-        _check(_lib.dvm_rt_run(self._rt, ctypes.c_void_p(stream) if stream else None, int(sync)))
+    def run(self, stream=None, sync=True, on_given_stream=False):
+        """Launches on the runner's own stream, or on `stream` (a hipStream_t as an integer). With on_given_stream
+        the handle is taken as it is, 0 naming the device's default stream (what torch's default stream is)."""
+        flags = (1 if sync else 0) | (2 if on_given_stream else 0)
+        _check(_lib.dvm_rt_run(self._rt, ctypes.c_void_p(stream) if stream else None, flags))
 
     def output(self, store, shape=None):
         """The stored tensor; `shape` (strided stores) reads back the whole buffer the store wrote into."""
@@ -511,6 +524,20 @@ class PyKernel(Kernel):
         out = (ctypes.c_double * 3)()
         _check(_lib.dvm_rt_perf(self._rt, warmup, iters, out))
         return (out[0], out[1], out[2])
+
+    def programs(self):
+        """The compiled launches as (blob bytes, (workgroups, threads, lds_bytes), [workspace word indices]); the
+        workspace words of a blob hold byte offsets into the workspace (include/dvm_c.h, dvm_rt_program)."""
+        out = []
+        for i in range(_lib.dvm_rt_program_count(self._rt)):
+            blob = (ctypes.c_uint8 * 4096)()
+            geo = (ctypes.c_uint32 * 3)()
+            words = (ctypes.c_uint32 * 64)()
+            n = _lib.dvm_rt_program(self._rt, i, blob, geo, words, 64)
+            if n < 0:
+                raise RuntimeError(_lib.dvm_c_last_error().decode())
+            out.append((bytes(blob), (geo[0], geo[1], geo[2]), [words[j] for j in range(n)]))
+        return out
 
     def num_launches(self):
         return _lib.dvm_rt_num_launches(self._rt)

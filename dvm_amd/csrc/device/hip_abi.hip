@@ -45,7 +45,33 @@ static const CubeKernel kCubeKernels[4][2][4] = {
     {DVM_CUBE_ROW(dvm_vm_cube_f16_small), DVM_CUBE_ROW(dvm_vm_cube_bf16_small)},
     {DVM_CUBE_ROW(dvm_vm_cube_f16_big8), DVM_CUBE_ROW(dvm_vm_cube_bf16_big8)}};
 
+// The workspace of dvm_hip_launch_vm_static_ws: device memory that belongs to the library's code object, one copy
+// per device. Host code never uses this name as an address: it asks the runtime for the array's address on the
+// current device (hipGetSymbolAddress) and passes that.
+static __device__ __align__(256) unsigned char dvm_static_ws[DVM_HIP_STATIC_WS_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+void *g_static_ws[kMaxDevices] = {nullptr};  // address of dvm_static_ws on each device, looked up once per device
+
+// Address of the static workspace on the current device (no allocation: the array exists since the code object
+// was loaded there).
+int static_ws_address(void **out) {
+  int dev = -1;
+  hipError_t err = hipGetDevice(&dev);
+  if (err != hipSuccess) return static_cast<int>(err);
+  if (dev < 0 || dev >= kMaxDevices) return static_cast<int>(hipErrorInvalidDevice);
+  if (g_static_ws[dev] == nullptr) {
+    void *p = nullptr;
+    err = hipGetSymbolAddress(&p, HIP_SYMBOL(dvm_static_ws));
+    if (err != hipSuccess) return static_cast<int>(err);
+    if (p == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+    g_static_ws[dev] = p;
+  }
+  *out = g_static_ws[dev];
+  return 0;
+}
 
 struct DeviceInfo {
   bool ready = false;
@@ -111,6 +137,12 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
       (void)hipGetLastError();
     }
   }
+  {
+    // the static workspace of dvm_hip_launch_vm_static_ws: its address on this device, looked up once, here
+    void *ws = nullptr;
+    const int rc = static_ws_address(&ws);
+    if (rc != 0) return rc;
+  }
   g_dev.ready = true;
   if (conf != nullptr) {
     conf->core_num = g_dev.cus;
@@ -138,13 +170,12 @@ uint64_t dvm_hip_select_block_thread(uint64_t kind, uint64_t item_num, uint64_t 
   return (blocks << 32) | threads;
 }
 
-int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, uint32_t lds_bytes, void *stream) {
-  if (param == nullptr || block_dim == 0 || threads == 0 || threads > 1024 || (threads & 63u) != 0) {
+// Checks one program blob against the launch it is to get and launches the interpreter kernel its entry type names.
+static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads, uint32_t lds_bytes, void *stream) {
+  if (block_dim == 0 || threads == 0 || threads > 1024 || (threads & 63u) != 0) {
     return static_cast<int>(hipErrorInvalidValue);
   }
   if (lds_bytes > g_dev.lds_per_wg) return static_cast<int>(hipErrorInvalidValue);
-  VmParam p;
-  memcpy(&p, param, sizeof(p));
   const VVecHeader *h = reinterpret_cast<const VVecHeader *>(p.w);
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (h->entry == VE_VECTOR) {
@@ -224,6 +255,37 @@ int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, u
   return static_cast<int>(hipGetLastError());
 }
 
+int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, uint32_t lds_bytes, void *stream) {
+  if (param == nullptr) return static_cast<int>(hipErrorInvalidValue);
+  VmParam p;
+  memcpy(&p, param, sizeof(p));
+  return launch_checked(p, block_dim, threads, lds_bytes, stream);
+}
+
+int dvm_hip_launch_vm_static_ws(const void *params, uint32_t n_programs, const uint32_t *geometry, const uint32_t *ws_words,
+                                uint32_t n_ws, size_t ws_bytes, void *stream) {
+  if (params == nullptr || geometry == nullptr || (n_ws > 0 && ws_words == nullptr)) return static_cast<int>(hipErrorInvalidValue);
+  if (ws_bytes > DVM_HIP_STATIC_WS_BYTES) return DVM_HIP_ERROR_WS_TOO_LARGE;
+  for (uint32_t i = 0; i < n_ws; ++i) {
+    if (ws_words[2 * i] >= n_programs || ws_words[2 * i + 1] >= DVM_PARAM_WORDS) return DVM_HIP_ERROR_BAD_WS_WORD;
+    const VmParam *src = static_cast<const VmParam *>(params) + ws_words[2 * i];
+    if (src->w[ws_words[2 * i + 1]] >= ws_bytes) return DVM_HIP_ERROR_BAD_WS_WORD;
+  }
+  void *ws = nullptr;
+  int rc = static_ws_address(&ws);
+  if (rc != 0) return rc;
+  for (uint32_t prog = 0; prog < n_programs; ++prog) {
+    VmParam p;  // the caller's blob stays as it is: the offsets become addresses in this copy
+    memcpy(&p, static_cast<const VmParam *>(params) + prog, sizeof(p));
+    for (uint32_t i = 0; i < n_ws; ++i) {
+      if (ws_words[2 * i] == prog) p.w[ws_words[2 * i + 1]] += reinterpret_cast<uint64_t>(ws);
+    }
+    rc = launch_checked(p, geometry[3 * prog], geometry[3 * prog + 1], geometry[3 * prog + 2], stream);
+    if (rc != 0) return rc;
+  }
+  return 0;
+}
+
 int dvm_hip_fill_u32(void *dst, uint32_t value, size_t bytes, void *stream) {
   if (bytes == 0) return 0;
   if (dst == nullptr || (bytes & 3u) != 0) return static_cast<int>(hipErrorInvalidValue);
@@ -277,6 +339,10 @@ int dvm_hip_synchronize_event(void *event) { return static_cast<int>(hipEventSyn
 int dvm_hip_event_elapsed_time(float *ms, void *start, void *end) {
   return static_cast<int>(hipEventElapsedTime(ms, reinterpret_cast<hipEvent_t>(start), reinterpret_cast<hipEvent_t>(end)));
 }
-const char *dvm_hip_error_string(int code) { return hipGetErrorString(static_cast<hipError_t>(code)); }
+const char *dvm_hip_error_string(int code) {
+  if (code == DVM_HIP_ERROR_WS_TOO_LARGE) return "the programs need more workspace than the static workspace holds (DVM_HIP_STATIC_WS_BYTES)";
+  if (code == DVM_HIP_ERROR_BAD_WS_WORD) return "a workspace word names no program, no word of its blob, or an offset outside the workspace";
+  return hipGetErrorString(static_cast<hipError_t>(code));
+}
 
 }  // extern "C"

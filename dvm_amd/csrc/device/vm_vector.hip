@@ -423,6 +423,33 @@ __device__ __forceinline__ void red_accumulate(RedAcc<SCHED> &r, uint32_t kind, 
   }
 }
 
+// max / min over int32 values (the accumulator holds their bit patterns): integer compares inside a slab, the
+// running partial as a double, which holds every int32 exactly, so the combine across lanes is the float one.
+template <int SCHED>
+__device__ __forceinline__ void red_accumulate_int(RedAcc<SCHED> &r, uint32_t kind, const Acc &x, uint32_t nvp) {
+  const bool is_max = kind == VR_MAX;
+  FOR_U {
+    const int nv = static_cast<int>((nvp >> (4 * u)) & 0xfu);
+    if constexpr (SCHED == VS_REDY) {
+      FOR_E {
+        const double v = static_cast<double>(__float_as_int(x.v[u][e]));
+        const double t = is_max ? (v > r.v[e] ? v : r.v[e]) : (v < r.v[e] ? v : r.v[e]);
+        r.v[e] = e < nv ? t : r.v[e];
+      }
+    } else {
+      int32_t best = is_max ? INT32_MIN : INT32_MAX;
+      FOR_E {
+        const int32_t v = __float_as_int(x.v[u][e]);
+        const int32_t t = is_max ? max(best, v) : min(best, v);
+        best = e < nv ? t : best;
+      }
+      const double v = static_cast<double>(best);
+      const double t = is_max ? (v > r.v[0] ? v : r.v[0]) : (v < r.v[0] ? v : r.v[0]);
+      r.v[0] = nv > 0 ? t : r.v[0];
+    }
+  }
+}
+
 // Combines one slot's partials across the lanes that share an output; every
 // one of those lanes ends up with the result.
 template <int SCHED>
@@ -1082,7 +1109,13 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
         switch (op) {
           case VOP_RED: {
             if (sub & VRF_SQUARE) FOR_U acc.v[u] = acc.v[u] * acc.v[u];  // the emitter fuses only where acc is dead afterwards
-            if (a == 0) {
+            if (sub & VRF_INT) {
+              if (a == 0) {
+                red_accumulate_int<SCHED>(racc0, sub & 0xfu, acc, nvp);
+              } else {
+                red_accumulate_int<SCHED>(racc1, sub & 0xfu, acc, nvp);
+              }
+            } else if (a == 0) {
               red_accumulate<SCHED>(racc0, sub & 0xfu, acc, nvp);
             } else {
               red_accumulate<SCHED>(racc1, sub & 0xfu, acc, nvp);
@@ -1101,12 +1134,17 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             break;
           }
           case VOP_FIN: {
+            const bool as_int = (sub & VRF_INT) != 0;  // the partial is an int32 value held exactly by the double
             if constexpr (SCHED == VS_REDY) {
               vf8 t;
-              FOR_E t[e] = static_cast<float>(a == 0 ? racc0.v[e] : racc1.v[e]);
+              FOR_E {
+                const double d = a == 0 ? racc0.v[e] : racc1.v[e];
+                t[e] = as_int ? __int_as_float(static_cast<int32_t>(d)) : static_cast<float>(d);
+              }
               FOR_U acc.v[u] = t;
             } else {
-              const float t = static_cast<float>(a == 0 ? racc0.v[0] : racc1.v[0]);
+              const double d = a == 0 ? racc0.v[0] : racc1.v[0];
+              const float t = as_int ? __int_as_float(static_cast<int32_t>(d)) : static_cast<float>(d);
               FOR_U acc.v[u] = t;
             }
             break;

@@ -208,11 +208,15 @@ dvm_rt *dvm_rt_new(const char *ker_type, const char *run_mode, int dev_id) {
         rt->das_mode = mode == "das";
         if (!rt->das_mode && mode != "dev") throw std::runtime_error("DVM EXCEPTION. reason: run mode '" + mode + "' is not supported");
         rt->ws_alloc.rt = rt.get();
-        (void)dev_id;
         rt->kernel.Reset(rt->ktype, rt->flags);
         if (!rt->das_mode) {
           if (!g_system.HasDevice()) {
             throw std::runtime_error(std::string("DVM EXCEPTION. reason: no MI355X device layer: ") + g_system.LoadError());
+          }
+          // one device per process: the VM kernels and their limits were set up for it at the first use
+          if (dev_id != g_system.device_id) {
+            throw std::runtime_error("DVM EXCEPTION. reason: device " + std::to_string(dev_id) + " asked for, the backend runs on device " +
+                                     std::to_string(g_system.device_id) + " (set DEVICE_ID before the first kernel)");
           }
           int rc = rt->Api().create_stream(&rt->stream);
           if (rc != 0) throw std::runtime_error(std::string("stream creation failed: ") + rt->Api().error_string(rc));
@@ -580,6 +584,9 @@ int dvm_rt_input(dvm_rt *rt, dvm_obj *load, const void *host, size_t bytes) {
   return Guard(
       [&]() {
         NDObject *o = Obj(load);
+        // memory the caller bound earlier (dvm_rt_bind_device) is the caller's: host data never goes there
+        auto bound = rt->buffers.find(o);
+        if (bound != rt->buffers.end() && !bound->second.owned) bound->second = Buffer();
         rt->Ensure(o, bytes);
         if (!rt->das_mode && bytes > 0) {
           int rc = rt->Api().mem_to_dev(rt->buffers[o].ptr, host, bytes);
@@ -598,6 +605,22 @@ int dvm_rt_bind_device(dvm_rt *rt, dvm_obj *io, void *device_ptr) {
         b.ptr = device_ptr;
         b.owned = false;
         b.bytes = 0;
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_unbind_device(dvm_rt *rt) {
+  return Guard(
+      [&]() {
+        for (auto it = rt->buffers.begin(); it != rt->buffers.end();) {
+          if (!it->second.owned) {
+            it->first->addr = nullptr;
+            it = rt->buffers.erase(it);
+          } else {
+            ++it;
+          }
+        }
         return 0;
       },
       -1);
@@ -653,14 +676,14 @@ int dvm_rt_codegen(dvm_rt *rt) {
 
 double dvm_rt_jit_us(const dvm_rt *rt) { return rt->jit_us; }
 
-int dvm_rt_run(dvm_rt *rt, void *stream, int sync) {
+int dvm_rt_run(dvm_rt *rt, void *stream, int flags) {
   return Guard(
       [&]() {
         if (rt->das_mode) return 0;
-        void *s = stream != nullptr ? stream : rt->stream;
+        void *s = (stream != nullptr || (flags & DVM_RUN_ON_GIVEN_STREAM) != 0) ? stream : rt->stream;
         int rc = rt->kernel.Launch(s);
         if (rc != 0) throw std::runtime_error(std::string("launch failed: ") + rt->Api().error_string(rc));
-        if (sync != 0) {
+        if ((flags & DVM_RUN_WAIT) != 0) {
           rc = rt->Api().synchronize_stream(s);
           if (rc != 0) throw std::runtime_error(std::string("kernel execution failed: ") + rt->Api().error_string(rc));
         }
@@ -740,6 +763,35 @@ int dvm_rt_num_launches(const dvm_rt *rt) {
 }
 
 size_t dvm_rt_workspace_bytes(const dvm_rt *rt) { return rt->kernel.GetImpl()->ws_bytes_; }
+
+int dvm_rt_program_count(const dvm_rt *rt) { return static_cast<int>(rt->kernel.GetImpl()->programs_.size()); }
+
+int dvm_rt_program(dvm_rt *rt, int i, void *blob, uint32_t geometry[3], uint32_t *ws_words, size_t cap) {
+  return Guard(
+      [&]() {
+        VKernel *k = rt->kernel.GetImpl();
+        if (i < 0 || i >= static_cast<int>(k->programs_.size())) throw std::runtime_error("DVM EXCEPTION. reason: no such launch");
+        const Program &p = k->programs_[i];
+        if (!p.fills.empty()) throw std::runtime_error("DVM EXCEPTION. reason: this launch needs a buffer cleared first and cannot be exported");
+        VmParam copy = p.blob;
+        int n = 0;
+        geometry[0] = geometry[1] = geometry[2] = 0;
+        if (!p.skip) {
+          geometry[0] = p.grid;
+          geometry[1] = p.threads;
+          geometry[2] = p.lds_bytes;
+          for (const Program::Patch &pt : p.patches) {
+            if (pt.op_id >= 0 || pt.ws_slot < 0) continue;
+            copy.w[pt.word] = k->ws_offsets_[pt.ws_slot] + static_cast<uint64_t>(pt.byte_offset);
+            if (static_cast<size_t>(n) < cap) ws_words[n] = pt.word;
+            ++n;
+          }
+        }
+        std::memcpy(blob, &copy, sizeof(copy));
+        return n;
+      },
+      -1);
+}
 
 const char *dvm_rt_das(dvm_rt *rt) {
   return Guard([&]() { return rt->kernel.Das(); }, static_cast<const char *>(nullptr));

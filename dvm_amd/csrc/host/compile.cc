@@ -1851,7 +1851,7 @@ void Compiler::EmitSection(int sec) {
       ANode &n = nodes_[i];
       if (n.kind != AK_REDUCE || n.sec != sec - 1) continue;
       BeforeOverwrite();
-      Emit(VOP_FIN, 0, 0, 0, n.reg_fmt, 0);
+      Emit(VOP_FIN, n.dtype == kInt32 ? VRF_INT : 0, 0, 0, n.reg_fmt, 0);
       acc_node_ = i;
       SaveAcc(i);
     }
@@ -1904,7 +1904,7 @@ void Compiler::EmitSection(int sec) {
     EmitValue(x);
     if (n.kind == AK_REDUCE) {
       const uint32_t rk = n.op->op == kSum ? VR_SUM : (n.op->op == kMax ? VR_MAX : VR_MIN);
-      Emit(VOP_RED, rk, 0, 0, n.reg_fmt, 0);
+      Emit(VOP_RED, rk | (n.dtype == kInt32 ? VRF_INT : 0), 0, 0, n.reg_fmt, 0);
     } else {
       Emit(VOP_ST, 0, 0, 0, MemIndex(sinks[i]), 0);
     }

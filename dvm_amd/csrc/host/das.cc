@@ -141,13 +141,13 @@ std::string &VKernel::DisAssemble() {
             break;
           }
           case VOP_RED:
-            os << "reduce_" << kRed[sub & 0xf] << ((sub & VRF_SQUARE) ? ".square" : "") << " r" << VI_A(w) << ", acc";
+            os << "reduce_" << kRed[sub & 0xf] << ((sub & VRF_SQUARE) ? ".square" : "") << ((sub & VRF_INT) ? ".int32" : "") << " r" << VI_A(w) << ", acc";
             if (static_cast<uint32_t>(w) & VI_ENDS) os << "  ; endsweep";
             break;
           case VOP_SWEEP: os << ((sub & VSW_REVERSE) ? "sweep (last round first) slots=" : "sweep slots=") << kRed[(VI_IMM(w) & 0xf) < 3 ? (VI_IMM(w) & 0xf) : 0]
                              << ((VI_IMM(w) & 0xf) < 3 ? "" : "(none)"); break;
           case VOP_ENDSWEEP: os << "endsweep"; break;
-          case VOP_FIN: os << "mov acc, r" << VI_A(w); break;
+          case VOP_FIN: os << "mov" << ((sub & VRF_INT) ? ".int32" : "") << " acc, r" << VI_A(w); break;
           case VOP_UNI_BEGIN: os << "uniform run, " << (VI_IMM(w) - 1) << " instructions: first wave only when the team is the workgroup"; break;
           case VOP_UNI_END: os << "end of uniform run"; break;
           case VOP_LD:

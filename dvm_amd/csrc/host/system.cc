@@ -93,6 +93,7 @@ void System::Init() {
     load_error_ = g_err_store.c_str();
     return;
   }
+  device_id = dev;
   core_num = static_cast<uint32_t>(conf.core_num);
   lds_per_wg = static_cast<uint32_t>(conf.local_mem_size);
   lds_per_cu = lds_per_wg;

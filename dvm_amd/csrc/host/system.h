@@ -62,6 +62,7 @@ class System : public Config {
   // Device limits the emitter plans against. Without a device they hold the
   // MI355X figures, so that code generation and disassembly are the same on a
   // CPU-only machine as on the GPU box.
+  int device_id = 0;  // the device the VM was initialised on
   uint32_t core_num = 256;
   uint32_t lds_per_wg = 160 * 1024;
   uint32_t lds_per_cu = 160 * 1024;

@@ -116,6 +116,7 @@ enum {
 // reduce kinds (low 4 bits of VOP_RED's sub field), and two modifiers of VOP_RED
 enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 #define VRF_SQUARE 0x10u  // acc = acc * acc (the fp32 product) first; the multiply of a sum of squares rides in the reduce
+#define VRF_INT 0x20u     // VOP_RED (max / min) and VOP_FIN: the values are int32 bit patterns, compared as integers
 
 // instruction word:
 //   [6:0] opcode  [7] VI_ENDS  [15:8] sub  [19:16] src kind  [21:20] rnd  [22] VI_UNIFORM  [23] VI_SAME_OFFS

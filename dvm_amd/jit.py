@@ -1,115 +1,139 @@
-"""`@kernel` decorator: trace a Python function into a DVM kernel once, call it with numpy arrays or with
-torch tensors that live on the GPU (those are used in place, see JitKernel._call_on_tensors).
+"""`@kernel`: trace a Python function into a DVM kernel once, then call it like a function.
 
-Same contract as the reference's python/dvm/jit.py:20-78: the decorated
-function receives the kernel object and one placeholder index per argument;
-`k.load(idx, dtype)`, `k.scalar(idx)` and `k.int_array(idx)` declare what each
-argument is; calling the result binds the arguments, (re)generates code for a
-dynamic kernel, runs it and returns the stored outputs as numpy arrays.
+Public contract of the reference's python/dvm/jit.py:20-78: the decorated function receives the kernel object
+and one placeholder per argument (its position); `k.load(idx, dtype)`, `k.scalar(idx)` and `k.int_array(idx)`
+say what the argument at that position is; a call binds the arguments, generates code again when the kernel
+is dynamic, runs, and returns the stored outputs (one array, or a list when the function returned several).
+
+Arguments may be numpy arrays (copied to the device and back) or torch tensors that live on the GPU (read and
+written in place, launched on torch's current stream; see `_DeviceCall`).
 """
+import inspect
 import os
 
 from ._core import PyKernel, DataType
 
 
+class _Slot:
+    """What one positional argument of the traced function turned out to be."""
+
+    __slots__ = ("role", "handle")
+
+    def __init__(self, role, handle):
+        self.role, self.handle = role, handle  # role: "tensor", "scalar" or "ints"
+
+
 class JitKernel(PyKernel):
     def __init__(self, ker_type, dynamic, run_type="dev"):
+        spec = ker_type
         if dynamic:
-            ker_type += ",dyn" if ":" in ker_type else ":dyn"
-        dev_conf = os.getenv("DEVICE_ID")
-        dev_id = int(dev_conf) if dev_conf else 0
-        PyKernel.__init__(self, ker_type, run_type, dev_id)
-        self.inputs = None
-        self.outputs = None
-        self.dynamic = dynamic
+            spec += (",dyn" if ":" in ker_type else ":dyn")
+        PyKernel.__init__(self, spec, run_type, int(os.getenv("DEVICE_ID") or 0))
+        self.dynamic = bool(dynamic)
+        self._slots = []      # one _Slot per argument, filled while tracing
+        self._results = None  # what the traced function returned: a store or a sequence of stores
 
+    # ---- tracing ----
     def build(self, func):
-        arg_cnt = func.__code__.co_argcount - 1
-        self.inputs = [None] * arg_cnt
-        self.outputs = func(self, *range(arg_cnt))
+        positional = [p for p in inspect.signature(func).parameters.values()
+                      if p.kind in (p.POSITIONAL_ONLY, p.POSITIONAL_OR_KEYWORD)]
+        self._slots = [None] * (len(positional) - 1)  # the first parameter is the kernel itself
+        self._results = func(self, *range(len(self._slots)))
+        missing = [i for i, s in enumerate(self._slots) if s is None]
+        if missing:
+            raise TypeError("%s never declared what argument(s) %s are (k.load / k.scalar / k.int_array)"
+                            % (getattr(func, "__name__", "kernel"), missing))
         if not self.dynamic:
-            self.codegen(None)
+            self.codegen()
+
+    def _declare(self, index, role, handle):
+        if not 0 <= index < len(self._slots):
+            raise IndexError("placeholder %d is not an argument of the traced function" % index)
+        self._slots[index] = _Slot(role, handle)
+        return handle
 
     def load(self, index, dtype, shape=()):
-        op = PyKernel.load(self, list(shape), dtype)
-        self.inputs[index] = op
-        return op
+        return self._declare(index, "tensor", PyKernel.load(self, list(shape), dtype))
 
     def scalar(self, index, dtype=DataType.float32):
-        ref = PyKernel.scalar(self, dtype)
-        self.inputs[index] = ref
-        return ref
+        return self._declare(index, "scalar", PyKernel.scalar(self, dtype))
 
     def int_array(self, index):
-        ref = PyKernel.int_array(self)
-        self.inputs[index] = ref
-        return ref
+        return self._declare(index, "ints", PyKernel.int_array(self))
+
+    # ---- calling ----
+    def _stores(self):
+        many = isinstance(self._results, (list, tuple))
+        return (list(self._results) if many else [self._results]), many
 
     def __call__(self, *args):
-        if any(_is_device_tensor(a) for a in args):
-            return self._call_on_tensors(args)
-        for inp, arg in zip(self.inputs, args):
-            PyKernel.input(self, inp, arg)
+        if len(args) != len(self._slots):
+            raise TypeError("kernel takes %d arguments, %d given" % (len(self._slots), len(args)))
+        if any(_on_gpu(a) for a in args):
+            return _DeviceCall(self, args).run()
+        self.release_device_bindings()  # a call on torch tensors before this one left their addresses behind
+        for slot, value in zip(self._slots, args):
+            self.input(slot.handle, value)
         if self.dynamic:
-            self.codegen(None)
+            self.codegen()
         self.run()
-        if isinstance(self.outputs, (list, tuple)):
-            return [self.output(x) for x in self.outputs]
-        return self.output(self.outputs)
+        stores, many = self._stores()
+        arrays = [self.output(s) for s in stores]
+        return arrays if many else arrays[0]
 
 
-    def _call_on_tensors(self, args):
-        """torch tensors on the GPU as arguments: nothing is copied. Inputs are read where they are, outputs are
-        new torch tensors, and the launches go to torch's current stream without waiting for them (the caller
-        orders later work like after any torch operator). Scalars and shape lists are passed as usual."""
+class _DeviceCall:
+    """One call of a JitKernel on torch tensors that live on the GPU. Nothing is copied: loads read the tensors'
+    memory, every store gets a fresh torch tensor of the inferred shape, and the launches go to torch's current
+    stream without a synchronisation, like any torch operator. Scalars and shape lists are bound as usual."""
+
+    def __init__(self, kern, args):
         import torch
-        dev = None
-        keep = []
-        for inp, arg in zip(self.inputs, args):
-            if not _is_device_tensor(arg):
-                if isinstance(arg, torch.Tensor):
+        self.torch, self.kern, self.args = torch, kern, args
+        self.types = {int(DataType.bool): torch.bool, int(DataType.float16): torch.float16,
+                      int(DataType.bfloat16): torch.bfloat16, int(DataType.float32): torch.float32,
+                      int(DataType.int32): torch.int32}
+
+    def run(self):
+        torch, k = self.torch, self.kern
+        held, device = [], None
+        for slot, value in zip(k._slots, self.args):
+            if slot.role != "tensor" or not _on_gpu(value):
+                if isinstance(value, torch.Tensor):
                     raise TypeError("tensor arguments have to live on the GPU, all of them")
-                PyKernel.input(self, inp, arg)
+                k.input(slot.handle, value)
                 continue
-            want = _TORCH_DTYPES()[int(inp.dtype())]
-            if arg.dtype != want:
-                raise TypeError("argument is %s, the kernel's load is %s" % (arg.dtype, want))
-            t = arg.contiguous()
-            keep.append(t)
-            dev = t.device
-            self.bind_device(inp, t.data_ptr(), tuple(t.shape))
-        self.normalize()
-        single = not isinstance(self.outputs, (list, tuple))
+            want = self.types[int(slot.handle.dtype())]
+            if value.dtype != want:
+                raise TypeError("argument is %s, the kernel's load is %s" % (value.dtype, want))
+            dense = value.contiguous()
+            held.append(dense)
+            device = dense.device
+            k.bind_device(slot.handle, dense.data_ptr(), tuple(dense.shape))
+        k.normalize()  # output shapes are known from here on
+        stores, many = k._stores()
         outs = []
-        for st in ([self.outputs] if single else self.outputs):
-            o = torch.empty(tuple(st.shape()), dtype=_TORCH_DTYPES()[int(st.dtype())], device=dev)
-            self.bind_device(st, o.data_ptr())
+        for st in stores:
+            o = torch.empty(tuple(st.shape()), dtype=self.types[int(st.dtype())], device=device)
+            k.bind_device(st, o.data_ptr())
             outs.append(o)
-        self.codegen(None)  # addresses are part of the programs, so also for a kernel of fixed shapes
-        self.run(stream=torch.cuda.current_stream(dev).cuda_stream, sync=False)
-        self._alive = keep + outs  # until the next call: the launches may still be running
-        return outs[0] if single else outs
+        k.codegen()  # addresses are part of the programs, so also for a kernel of fixed shapes
+        k.run(stream=torch.cuda.current_stream(device).cuda_stream, sync=False, on_given_stream=True)
+        k._alive = held + outs  # until the next call: the launches may still be running
+        return outs if many else outs[0]
 
 
-def _is_device_tensor(a):
-    return hasattr(a, "data_ptr") and getattr(a, "is_cuda", False)
-
-
-def _TORCH_DTYPES():
-    import torch
-    return {int(DataType.bool): torch.bool, int(DataType.float16): torch.float16, int(DataType.bfloat16): torch.bfloat16,
-            int(DataType.float32): torch.float32, int(DataType.int32): torch.int32}
+def _on_gpu(value):
+    return hasattr(value, "data_ptr") and bool(getattr(value, "is_cuda", False))
 
 
 def kernel(ktype="split", dynamic=True, run_type="dev"):
-    if callable(ktype):
-        kobj = JitKernel("split", True)
-        kobj.build(ktype)
-        return kobj
+    """`@kernel` or `@kernel(ktype=..., dynamic=..., run_type=...)`."""
+    def trace(func, *conf):
+        traced = JitKernel(*conf)
+        traced.build(func)
+        return traced
 
-    def decorate(func):
-        kobj = JitKernel(ktype, dynamic, run_type)
-        kobj.build(func)
-        return kobj
-
-    return decorate
+    if callable(ktype):  # used bare: the default split kernel with dynamic shapes
+        return trace(ktype, "split", True)
+    return lambda func: trace(func, ktype, dynamic, run_type)

@@ -98,6 +98,9 @@ int dvm_obj_dtype(const dvm_obj *o);
 int dvm_rt_input(dvm_rt *rt, dvm_obj *load, const void *host, size_t bytes);
 /* Binds a caller-owned device buffer to a load or store (no copy, no ownership). */
 int dvm_rt_bind_device(dvm_rt *rt, dvm_obj *io, void *device_ptr);
+/* Forgets every binding made by dvm_rt_bind_device (the memory stays the caller's); loads and stores get
+ * buffers of the runner again at the next dvm_rt_input / dvm_rt_codegen. */
+int dvm_rt_unbind_device(dvm_rt *rt);
 /* Normalize + allocate unbound outputs + CodeGen with relocations. */
 // Shape inference only (what dvm_rt_codegen does first): afterwards dvm_obj_shape of a store is what the bound
 // inputs imply, so a caller can allocate its own output memory and bind it before code generation.
@@ -105,8 +108,11 @@ int dvm_rt_normalize(dvm_rt *rt);
 int dvm_rt_codegen(dvm_rt *rt);
 /* Host wall time of the last Normalize + CodeGen in microseconds. */
 double dvm_rt_jit_us(const dvm_rt *rt);
-/* Launch on the runner's stream (or on `stream` if not NULL) and, with sync != 0, wait. */
-int dvm_rt_run(dvm_rt *rt, void *stream, int sync);
+/* Launch and, with DVM_RUN_WAIT, wait for the stream. The stream is `stream` when that is not NULL or when
+ * DVM_RUN_ON_GIVEN_STREAM is set (then NULL names the device's default stream), else the runner's own. */
+#define DVM_RUN_WAIT 1
+#define DVM_RUN_ON_GIVEN_STREAM 2
+int dvm_rt_run(dvm_rt *rt, void *stream, int flags);
 int dvm_rt_output(dvm_rt *rt, dvm_obj *store, void *host, size_t bytes);
 void *dvm_rt_device_ptr(dvm_rt *rt, dvm_obj *io);
 /* warmup + iters timed launches with events: out = {min, max, mean} microseconds (src/pybind_api.cc:751-767). */
@@ -114,6 +120,17 @@ int dvm_rt_perf(dvm_rt *rt, int warmup, int iters, double out[3]);
 /* Number of device launches one run() issues. */
 int dvm_rt_num_launches(const dvm_rt *rt);
 size_t dvm_rt_workspace_bytes(const dvm_rt *rt);
+
+/* The compiled launches of the kernel, for a caller that drives the device layer (include/dvm_hip.h) itself:
+ * after dvm_rt_codegen, launch i of dvm_rt_program_count() is copied out as its 4096-byte blob with the bound
+ * input / output addresses in place, its geometry {workgroups, threads, lds_bytes} (all zero for a launch that
+ * has nothing to do) and the indices of the blob's 64-bit words that address the kernel's workspace. Those words
+ * hold byte offsets into the workspace (of dvm_rt_workspace_bytes() bytes) instead of addresses, which is the
+ * form dvm_hip_launch_vm_static_ws takes; adding a workspace address to each gives what dvm_hip_launch_vm
+ * takes. Returns the number of workspace words (at most `cap` are written), or -1. Kernels whose launches need a
+ * buffer cleared first (an output of a reduce over no elements) are refused. */
+int dvm_rt_program_count(const dvm_rt *rt);
+int dvm_rt_program(dvm_rt *rt, int i, void *blob, uint32_t geometry[3], uint32_t *ws_words, size_t cap);
 
 const char *dvm_rt_das(dvm_rt *rt);
 const char *dvm_rt_dump(dvm_rt *rt);

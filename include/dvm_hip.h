@@ -46,6 +46,29 @@ uint64_t dvm_hip_select_block_thread(uint64_t kind, uint64_t item_num, uint64_t 
  * Replaces dvm::gpu::LaunchVM (src/vm_gpu.h:155). */
 int dvm_hip_launch_vm(const void *param, uint32_t block_dim, uint32_t threads, uint32_t lds_bytes, void *stream);
 
+/* Launches `n_programs` program blobs in order on `stream`, with the workspace they share (the values one launch
+ * hands to a later one) placed in a workspace the library owns, and allocates nothing: no hipMalloc, no hipFree,
+ * no allocating library routine. It has no counterpart in the reference; it is for callers that cannot allocate
+ * device memory where they launch: code under HIP graph capture, tight serving loops, harnesses that forbid it.
+ * The existing route is dvm_hip_launch_vm once per blob with workspace addresses the caller allocated.
+ *   params     n_programs consecutive blobs of 4096 bytes (host memory), each as dvm_hip_launch_vm takes it,
+ *              input and output addresses filled in by the caller;
+ *   geometry   n_programs triples {workgroups, threads, lds_bytes};
+ *   ws_words   n_ws pairs {program index, index of a 64-bit word of that blob}: the word holds a byte offset into
+ *              the workspace instead of an address (a multiple of 16 for the matmul and attention operands);
+ *   ws_bytes   size of the workspace the offsets were planned for.
+ * The workspace is one array of DVM_HIP_STATIC_WS_BYTES bytes per device, 256-byte aligned, that lives in the
+ * library's device code from load to process exit. A larger ws_bytes, or an offset outside ws_bytes, is refused
+ * with DVM_HIP_ERROR_WS_TOO_LARGE / DVM_HIP_ERROR_BAD_WS_WORD before anything is launched. Nothing in it has to
+ * start at zero: a launch writes all of a value before a later launch reads it. Every call on a device uses that
+ * device's one array, which keeps what the last call left there: two calls that overlap on one device (different
+ * streams, or two threads) race on it; calls on one stream are ordered and safe. */
+#define DVM_HIP_STATIC_WS_BYTES (32u * 1024u * 1024u)
+#define DVM_HIP_ERROR_WS_TOO_LARGE (-2)
+#define DVM_HIP_ERROR_BAD_WS_WORD (-3)
+int dvm_hip_launch_vm_static_ws(const void *params, uint32_t n_programs, const uint32_t *geometry, const uint32_t *ws_words,
+                                uint32_t n_ws, size_t ws_bytes, void *stream);
+
 /* Fills `bytes` bytes at device address `dst` with the 32-bit pattern `value`
  * on `stream` using a fill kernel (safe under graph capture, unlike a memset
  * node). Used where the reference launches its clean kernels

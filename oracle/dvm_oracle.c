@@ -109,7 +109,12 @@ uint16_t ora_f32_to_bf16_host(float f) {
   return ora_f32_to_bf16_dev(f);
 }
 
-/* Rounds a float to the value set of element type t (1 fp16, 2 bf16, others unchanged). */
+/* Rounds a float to the value set of element type t (1 fp16, 2 bf16, others unchanged).
+ * bf16 and NaN: the bit trick the reference's device code uses (src/vm_gpu.cu:155-160, ora_f32_to_bf16_dev
+ * above) has no NaN case; it keeps every NaN whose low mantissa half does not carry out (the default quiet NaN
+ * 0x7fc00000 among them, which is what arithmetic produces) but turns the payloads 0x7fff8000..0x7fffffff into
+ * -0.0 and the like. The gfx950 hardware conversion keeps every NaN a NaN. The oracle follows the hardware
+ * here: a NaN stays a NaN. For every input that is not a NaN the two agree bit for bit. */
 static float round_to(int t, float v) {
   if (t == 1) return ora_f16_to_f32(ora_f32_to_f16(v));
   if (t == 2) return isnan(v) ? v : ora_bf16_to_f32(ora_f32_to_bf16_dev(v));

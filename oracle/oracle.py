@@ -501,6 +501,10 @@ class OracleKernel:
             dims = (dims,)
         if kind == 0:
             assert x.t == F32, "sum needs fp32 input"
+        if x.t == I32:
+            # max / min of integers: order-independent and exact; fp32 would not hold values above 2^24
+            fn = np.max if kind == 1 else np.min
+            return OVal(fn(x.a, axis=tuple(d % x.a.ndim for d in dims), keepdims=keepdims).astype(np.int32), x.t)
         return OVal(reduce_f32(kind, x.a, list(dims), keepdims), x.t)
 
     def sum(self, x, dims, keepdims=False):

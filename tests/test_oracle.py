@@ -203,6 +203,59 @@ def test_matmul_against_numpy():
     assert np.array_equal(k.output(k.matmul(k.load(a), k.load(b), False, False)), (a.astype(np.float32) @ b.astype(np.float32)).astype(np.float16))
 
 
+def test_matmul_transposes_and_bias_against_numpy():
+    """All four storage layouts and the bias row, on shapes where m, n and k all differ (a transposed index or a
+    bias added along the wrong axis changes the result), exactly representable values, so no tolerance."""
+    rng = np.random.default_rng(77)
+    m, n, kk = 5, 7, 11
+    a = rng.integers(-4, 5, (m, kk)).astype(np.float16)
+    b = rng.integers(-4, 5, (kk, n)).astype(np.float16)
+    bias = rng.integers(-8, 9, (n,)).astype(np.float16)
+    want = a.astype(np.float32) @ b.astype(np.float32)
+    for ta in (False, True):
+        for tb in (False, True):
+            k = OracleKernel()
+            la = k.load(np.ascontiguousarray(a.T) if ta else a)
+            lb = k.load(np.ascontiguousarray(b.T) if tb else b)
+            assert np.array_equal(k.output(k.matmul(la, lb, ta, tb)), want.astype(np.float16)), (ta, tb)
+            got = k.output(k.matmul(la, lb, ta, tb, k.load(bias)))
+            assert np.array_equal(got, (want + bias.astype(np.float32)[None, :]).astype(np.float16)), (ta, tb)
+    # batches broadcast like np.matmul; the bias joins the fp32 sum before the one rounding
+    a3 = rng.normal(0, 1, (3, 1, m, kk)).astype(np.float16)
+    b3 = rng.normal(0, 1, (1, 2, kk, n)).astype(np.float16)
+    k = OracleKernel()
+    got = k.output(k.matmul(k.load(a3), k.load(b3), False, False, k.load(bias)))
+    ref = np.matmul(a3.astype(np.float32), b3.astype(np.float32)) + bias.astype(np.float32)
+    assert got.shape == (3, 2, m, n) and np.allclose(got.astype(np.float32), ref, rtol=2e-3, atol=2e-3)
+    tiny = np.float16(2.0 ** -12)  # 1 + 2^-12 + 2^-12 rounds to 1 + 2^-10 only if the bias is added before rounding
+    k = OracleKernel()
+    one = k.load(np.array([[1.0, tiny]], np.float16))
+    got = k.output(k.matmul(one, k.load(np.array([[1.0], [1.0]], np.float16)), False, False, k.load(np.array([tiny * 2], np.float16))))
+    assert got[0, 0] == np.float16(1.0 + 3 * 2.0 ** -12)  # = nearest fp16 to 1.000732, i.e. 1 + 2^-10
+
+
+def test_int32_min_compares_and_reduces():
+    """int32 minimum, every compare and max / min reduces against NumPy, with values fp32 cannot hold."""
+    rng = np.random.default_rng(5)
+    x = rng.integers(-2 ** 31, 2 ** 31 - 1, [16, 257], dtype=np.int64).astype(np.int32)
+    y = rng.integers(-2 ** 31, 2 ** 31 - 1, [16, 257], dtype=np.int64).astype(np.int32)
+    y[::2] = x[::2]                 # equal pairs, so that == / != / <= / >= see both outcomes
+    y[1, :] = x[1, :] + 1           # neighbours above 2^24, which fp32 would merge
+    k = OracleKernel()
+    a, b = k.load(x), k.load(y)
+    assert np.array_equal(k.output(k.minimum(a, b)), np.minimum(x, y))
+    assert np.array_equal(k.output(k.maximum(a, b)), np.maximum(x, y))
+    for name, fn in [("equal", np.equal), ("not_equal", np.not_equal), ("greater", np.greater), ("greater_equal", np.greater_equal),
+                     ("less", np.less), ("less_equal", np.less_equal)]:
+        got = k.output(getattr(k, name)(a, b))
+        assert np.array_equal(got.astype(bool), fn(x, y)), name
+        got = k.output(getattr(k, name)(a, 7))
+        assert np.array_equal(got.astype(bool), fn(x, np.int32(7))), name + " scalar"
+    for dims in [(0,), (1,), (0, 1)]:
+        assert np.array_equal(k.output(k.max(a, dims, True)), np.max(x, dims, keepdims=True))
+        assert np.array_equal(k.output(k.min(a, dims, False)), np.min(x, dims))
+
+
 def test_batchnorm_restatement():
     rng = np.random.default_rng(1002)
     x = rng.normal(0, 1, [4, 16, 7, 9]).astype(np.float32)

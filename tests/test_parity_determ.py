@@ -101,3 +101,27 @@ def test_sum_over_both_axes_of_broadcast_add():  # tests/ut/test_reduce.py:326-3
     a0, a1 = rng.standard_normal([8002, 2]).astype(np.float32), rng.standard_normal([8002, 1]).astype(np.float32)
     run_parity(lambda k, x0, x1: k.sum(k.add(x0, x1), [0, 1], False), [a0, a1],
                golden=np.sum((a0 + a1).astype(np.float64), axis=(0, 1)), eps=1e-4)
+
+
+# max / min over int32 tensors compare integers: values above 2^24 (no fp32 holds them), negative values (whose
+# bit patterns order backwards as floats) and -1 (the bit pattern of a NaN) come out exact, along the innermost
+# axis (one team per output), along an outer axis (lanes own outputs) and with a consumer in the same launch.
+INT_SHAPES = [([64, 1000], (1,)), ([1000, 64], (0,)), ([7, 33, 129], (0, 2)), ([3, 40000], (1,)), ([5, 9, 300], (1,)),
+              ([200000], (0,))]
+
+
+@pytest.mark.parametrize("shape,dims", INT_SHAPES)
+def test_max_min_int32(shape, dims):
+    rng = np.random.default_rng(sum(shape))
+    x = rng.integers(-2**31, 2**31 - 1, shape, dtype=np.int64).astype(np.int32)
+    x.flat[::97] = -1
+    x.flat[5::89] = rng.integers(-40, 40, x.flat[5::89].shape).astype(np.int32)
+    mx, mn = np.max(x, dims, keepdims=True), np.min(x, dims, keepdims=True)
+    run_parity(lambda k, a: [k.max(a, dims, True), k.min(a, dims, True), k.sub(a, k.max(a, dims, True))], [x],
+               golden=[mx, mn, x - mx], eps=0)  # the subtraction wraps in int32, as NumPy's does
+
+
+def test_max_min_int32_small_negative():
+    x = -np.arange(1, 4097, dtype=np.int32).reshape(4, 1024)
+    run_parity(lambda k, a: [k.max(a, (1,), False), k.min(a, (0,), False)], [x],
+               golden=[np.max(x, 1), np.min(x, 0)], eps=0)

@@ -2,6 +2,7 @@
 import numpy as np
 import pytest
 
+from dvm_amd import DataType
 from dvm_amd.tester import Tester
 from tests.util import run_parity
 
@@ -192,7 +193,7 @@ def test_scalar_ref_updates():  # tests/ut/test_elemwise.py:500-532
     t = Tester("vector:dyn")
     x = t.load([1024], "float32")
     sf = t.scalar()
-    si = t.scalar("int32" if False else t.cast.__self__ and 4)  # an int32 scalar reference
+    si = t.scalar(DataType.int32)
     xi = t.load([1024], "int32")
     o1 = t.store(t.mul(x, sf))
     o2 = t.store(t.add(xi, si))

@@ -5,10 +5,11 @@ given, with a NumPy golden."""
 import numpy as np
 
 from dvm_amd import DataType
-from dvm_amd.tester import Tester
+from dvm_amd.tester import Tester, default_tolerance
 from oracle.oracle import OracleKernel
 
-DEFAULT_EPS = {int(DataType.float32): 1e-5, int(DataType.float16): 1e-3, int(DataType.bfloat16): 1e-2}
+# one tolerance policy for the harness and the parity tests
+DEFAULT_EPS = {int(t): default_tolerance(t) for t in (DataType.float32, DataType.float16, DataType.bfloat16)}
 
 
 def run_parity(build, arrays, dtypes=None, ker="vector", eps=None, golden=None, golden_eps=None, use_oracle=True):
