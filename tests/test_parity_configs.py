@@ -89,7 +89,7 @@ def test_config2_dynamic_rmsnorm_one_kernel_object():
         assert np.allclose(got, want, rtol=1e-2, atol=1e-2), "R=%d vs NumPy" % R
         # the oracle applies the reference's lowering op by op (fp32 arithmetic, one bf16 rounding per bf16 value)
         o = OracleKernel()
-        ref = Tester.convert_from_bf16(o.output(o.store(_rmsnorm(o, o.load(xf[:R], "bfloat16"), o.load(rf[:R], "bfloat16"), o.load(wv)))))
+        ref = o.output(o.store(_rmsnorm(o, o.load(xf[:R], "bfloat16"), o.load(rf[:R], "bfloat16"), o.load(wv))))  # bf16 values as fp32
         assert np.allclose(got, ref, rtol=1e-2, atol=1e-2), "R=%d vs oracle" % R
         # all but the elements whose fp32 value sits within rounding noise of a bf16 tie agree bit for bit
         assert np.mean(got != ref) < 1e-3, "R=%d: %g of the elements differ from the oracle" % (R, np.mean(got != ref))
