@@ -1,0 +1,58 @@
+// The fused attention launch.
+#include <algorithm>
+#include <cstdlib>
+#include <cmath>
+#include <cstddef>
+#include <cstring>
+#include <stdexcept>
+
+#include "compiler.h"
+
+namespace dvm {
+
+void Compiler::CompileAttn(int gi) {
+  const AttnGroup &g = attn_groups_[gi];
+  const int r = g.q->rank();
+  VAttnHeader h;
+  std::memset(&h, 0, sizeof(h));
+  h.entry = VE_ATTN;
+  h.dtype = MemDType(g.m2->type_id_);
+  int64_t nb = 1;
+  for (int d = 0; d < r - 2; ++d) nb *= g.q->dim(d);
+  h.nb = static_cast<uint32_t>(nb);
+  h.sq = static_cast<uint32_t>(g.q->dim(r - 2));
+  h.skv = static_cast<uint32_t>(g.k->dim(r - 2));
+  h.d = DVM_ATTN_D;
+  h.scale = g.scale;
+  h.q_blocks = (h.sq + DVM_ATTN_BQ - 1) / DVM_ATTN_BQ;
+  if (static_cast<uint64_t>(h.nb) * h.q_blocks >= (1ull << 31)) Fail("too many attention blocks");
+  std::memset(&prog_->blob, 0, sizeof(VmParam));
+  std::memcpy(prog_->blob.w, &h, sizeof(h));
+  auto patch = [&](size_t byte_off, int op_id, int ws_slot) {
+    Program::Patch p;
+    p.word = static_cast<uint32_t>(byte_off / 8);
+    p.op_id = op_id;
+    p.ws_slot = ws_slot;
+    p.role = Program::kPatchAligned16;
+    prog_->patches.push_back(p);
+  };
+  patch(offsetof(VAttnHeader, q_addr), g.q->id, -1);
+  patch(offsetof(VAttnHeader, k_addr), g.k->id, -1);
+  patch(offsetof(VAttnHeader, v_addr), g.v->id, -1);
+  // the result goes to the user's store when there is one in this sub-kernel, else to workspace
+  const int m2 = g.m2->id;
+  if (store_of_[m2] >= 0 && area_[store_of_[m2]] == area_[m2]) {
+    patch(offsetof(VAttnHeader, o_addr), store_of_[m2], -1);
+  } else if (ws_slot_[m2] >= 0) {
+    patch(offsetof(VAttnHeader, o_addr), -1, ws_slot_[m2]);
+  } else {
+    Fail("attention result has no destination");
+  }
+  // eight waves of 32 queries (two per SIMD: one wave's softmax runs under the other's MFMAs) measured 767-788 us
+  // on fp16 [8,32,2048,128] against 920-940 us for four waves of 64 queries; DVM_ATTN_WAVES=4 selects the latter
+  prog_->threads = 512;
+  if (k_->tuning_.attn_waves == 4) prog_->threads = 256;
+  prog_->lds_bytes = DVM_ATTN_LDS_BYTES;
+  prog_->grid = h.nb * h.q_blocks;
+}
+}  // namespace dvm

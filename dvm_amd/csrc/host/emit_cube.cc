@@ -1,0 +1,214 @@
+// Matmul sub-kernels: tile choice, operand descriptors, the epilogue program.
+#include <algorithm>
+#include <cstdlib>
+#include <cmath>
+#include <cstddef>
+#include <cstring>
+#include <stdexcept>
+
+#include "compiler.h"
+
+namespace dvm {
+
+// ---------- matmul sub-kernels ----------
+//
+// The matmul's operands are read from memory by the MFMA tile loop; every other operator of the
+// sub-kernel has the matmul's output shape and becomes the epilogue program, emitted with the same
+// accumulator-machine rules as a pointwise kernel whose accumulator starts out holding the product.
+
+int Compiler::CubeMemIndex(int v) {
+  ANode &n = nodes_[v];
+  if (n_mem_ >= DVM_CUBE_MAXMEM) Fail("too many memory operands in a matmul epilogue");
+  VCubeMem &m = cmems_[n_mem_];
+  std::memset(&m, 0, sizeof(m));
+  m.dtype = MemDType(n.dtype);
+  const int R = cube_out_->rank();
+  int64_t stride = 1;
+  for (int d = n.rank - 1; d >= 0; --d) {
+    const int od = d + R - n.rank;
+    if (n.dims[d] != 1) {
+      if (od < 0 || n.dims[d] != cube_out_->dim(od)) Fail("epilogue operand does not broadcast to the matmul result");
+      const int64_t walk = n.view != nullptr ? n.view->vstride_[d] : stride;
+      if (walk >= (1ll << 32) || walk < 0) Fail("stride above 2^32");
+      const uint32_t st = static_cast<uint32_t>(walk);
+      if (od == R - 1 && st != 1) Throw("DVM EXCEPTION. reason: a strided view whose innermost stride is not 1 is not supported by the gfx950 backend");
+      if (od == R - 1) m.stride_n = st;
+      else if (od == R - 2) m.stride_m = st;
+      else if (od == R - 3) m.stride_b1 = st;
+      else m.stride_b0 = st;
+    }
+    stride *= n.dims[d];
+  }
+  Program::Patch p;
+  p.word = static_cast<uint32_t>(sizeof(VCubeHeader) / 8 + n_mem_ * (sizeof(VCubeMem) / 8));
+  p.op_id = n.addr_op;
+  p.ws_slot = n.ws_slot;
+  p.byte_offset = n.view != nullptr ? n.view->view_base_ * static_cast<int64_t>(DTypeSize(n.dtype)) : 0;
+  p.role = Program::kPatchPlain;
+  prog_->patches.push_back(p);
+  n.mem_idx = n_mem_++;
+  return n.mem_idx;
+}
+
+void Compiler::CompileCube(int a) {
+  cube_mode_ = true;
+  BuildNodes(a);
+  int c = -1;
+  for (int i = 0; i < nn_; ++i)
+    if (nodes_[i].kind == AK_OP && nodes_[i].op->kind == kObjMatMul) c = i;
+  if (c < 0) Fail("matmul sub-kernel without a matmul");
+  NDObject *mm = nodes_[c].op;
+  cube_out_ = mm;
+  const ANode &an = nodes_[nodes_[c].in[0]], &bn = nodes_[nodes_[c].in[1]];
+  if (an.kind != AK_MEM || bn.kind != AK_MEM) Fail("matmul operands must come from memory");
+  if (an.dtype != bn.dtype || (an.dtype != kFloat16 && an.dtype != kBFloat16)) Fail("matmul operands must both be fp16 or both bf16");
+  const int R = mm->rank();
+  const int br = R - 2;
+  if (br > 2) Fail("matmul with more than two batch dimensions");
+  VCubeHeader h;
+  std::memset(&h, 0, sizeof(h));
+  h.entry = VE_CUBE;
+  h.dtype = MemDType(an.dtype);
+  const int64_t M = mm->dim(R - 2), N = mm->dim(R - 1);
+  const int64_t K = mm->trans_a ? an.dims[an.rank - 2] : an.dims[an.rank - 1];
+  if (M >= (1ll << 31) || N >= (1ll << 31) || K >= (1ll << 31)) Fail("matmul extent above 2^31");
+  h.m = static_cast<uint32_t>(M);
+  h.n = static_cast<uint32_t>(N);
+  h.k = static_cast<uint32_t>(K);
+  h.trans_a = mm->trans_a ? 1 : 0;
+  h.trans_b = mm->trans_b ? 1 : 0;
+  h.lda = static_cast<uint32_t>(an.dims[an.rank - 1]);
+  h.ldb = static_cast<uint32_t>(bn.dims[bn.rank - 1]);
+  h.nb0 = br == 2 ? static_cast<uint32_t>(mm->dim(0)) : 1;
+  h.nb1 = br >= 1 ? static_cast<uint32_t>(mm->dim(br - 1)) : 1;
+  auto batch_strides = [&](const ANode &x, uint32_t *s0, uint32_t *s1) {
+    *s0 = *s1 = 0;
+    int64_t stride = x.dims[x.rank - 1] * x.dims[x.rank - 2];
+    for (int d = x.rank - 3; d >= 0; --d) {
+      const int od = d + R - x.rank;
+      if (x.dims[d] != 1) {
+        if (stride >= (1ll << 32)) Fail("stride above 2^32");
+        if (od == R - 3) *s1 = static_cast<uint32_t>(stride);
+        else *s0 = static_cast<uint32_t>(stride);
+      }
+      stride *= x.dims[d];
+    }
+  };
+  batch_strides(an, &h.a_sb0, &h.a_sb1);
+  batch_strides(bn, &h.b_sb0, &h.b_sb1);
+  if (M == 0 || N == 0 || h.nb0 == 0 || h.nb1 == 0) {
+    prog_->skip = true;
+    return;
+  }
+  // block tile: the largest that still gives most compute units a tile
+  const uint64_t batch = static_cast<uint64_t>(h.nb0) * h.nb1;
+  auto tiles = [&](int64_t t) { return static_cast<uint64_t>((M + t - 1) / t) * static_cast<uint64_t>((N + t - 1) / t) * batch; };
+  const uint64_t cus = g_system.core_num;
+  int64_t bt;
+  if (tiles(256) * 4 >= cus * 3) {
+    h.tile = 0;
+    bt = 256;
+  } else if (tiles(128) * 2 >= cus) {
+    h.tile = 1;
+    bt = 128;
+  } else {
+    h.tile = 2;
+    bt = 64;
+  }
+  {  // tuning override: 256, 128 or 64
+    const int v = k_->tuning_.cube_tile;
+    if (v == 256 || v == 128 || v == 64) {
+      bt = v;
+      h.tile = v == 256 ? 0 : (v == 128 ? 1 : 2);
+    }
+  }
+  // The 256x256 tile also exists on eight waves (two per SIMD, 64x128 accumulators each): the second wave hides
+  // most of the epilogue and of the fragment-read latency, at 1.5 times the local-memory traffic per flop.
+  // Measured on MI355X, 8192x4096x4096 bf16: both operands k-contiguous 289 -> 283 us (with bias + SiLU
+  // 369 -> 354 us, k = 512: 81 -> 70 us); with a k-strided operand, whose tiles pass through registers, the four
+  // waves stay ahead (286 us against 324 us). DVM_CUBE_WAVES=4 / 8 forces either.
+  if (h.tile == 0) {
+    bool eight = !h.trans_a && h.trans_b;
+    if (k_->tuning_.cube_waves == 8) eight = true;
+    if (k_->tuning_.cube_waves == 4) eight = false;
+    if (eight) h.tile = 3;
+  }
+  h.tiles_m = static_cast<uint32_t>((M + bt - 1) / bt);
+  h.tiles_n = static_cast<uint32_t>((N + bt - 1) / bt);
+  if (tiles(bt) >= (1ull << 31)) Fail("too many matmul tiles");
+  h.fast = (K % 64 == 0 && K > 0 && h.lda < (1u << 22) && h.ldb < (1u << 22) && h.lda % 8 == 0 && h.ldb % 8 == 0 && h.a_sb0 % 8 == 0 &&
+            h.a_sb1 % 8 == 0 && h.b_sb0 % 8 == 0 && h.b_sb1 % 8 == 0)
+               ? 1
+               : 0;
+  // operand addresses
+  for (int which = 0; which < 2; ++which) {
+    const ANode &x = which == 0 ? an : bn;
+    if (x.view != nullptr) Throw("DVM EXCEPTION. reason: a strided view as a matmul operand is not supported by the gfx950 backend");
+    Program::Patch p;
+    p.word = static_cast<uint32_t>((which == 0 ? offsetof(VCubeHeader, a_addr) : offsetof(VCubeHeader, b_addr)) / 8);
+    p.op_id = x.addr_op;
+    p.ws_slot = x.ws_slot;
+    p.role = Program::kPatchCubeOperand;
+    prog_->patches.push_back(p);
+  }
+  // the epilogue: one section over values that all live in fragments
+  for (int i = 0; i < nn_; ++i) {
+    ANode &n = nodes_[i];
+    n.has_inner = true;
+    n.fd = false;
+    n.sec = 0;
+    n.last_sec = 0;
+    n.level = 0;
+    n.uses = 0;
+    n.in_cone = false;
+  }
+  // the tile loop reads A and B itself: they are no values of the epilogue
+  const int bias = nodes_[c].nin > 2 ? nodes_[c].in[2] : -1;
+  if (bias >= 0 && nodes_[bias].kind != AK_MEM) Fail("matmul bias must come from memory");
+  nodes_[c].nin = 0;
+  nr_ = 0;
+  n_sec_ = 1;
+  cur_sec_ = 0;
+  single_round_ = true;
+  vslot_limit_ = DVM_CUBE_NTEMP;
+  sreg_used_ = vslot_used_ = 0;
+  max_vslot_ = 0;
+  n_held_ = 0;
+  code_.clear();
+  n_mem_ = 0;
+  // the bias row joins the fp32 accumulators, which are then rounded once to the operand type: that
+  // is the matmul's value (src/vm_aic.cce:34-470)
+  if (bias >= 0) Emit(VOP_BINF, VB_ADD, VK_MEM, 0, MemIndex(bias), 0);
+  Emit(VOP_CAST, VC_RND, 0, RndOf(mm->type_id_), 0, 0);
+  acc_node_ = c;
+  int sinks[kMaxNodes];
+  int ns = 0;
+  for (int i = 0; i < nn_; ++i)
+    if (nodes_[i].kind == AK_OUT) sinks[ns++] = i;
+  for (int i = 0; i < ns; ++i) CountCone(nodes_[sinks[i]].in[0]);
+  for (int i = 0; i < ns; ++i) {
+    const int x = Resolve(nodes_[sinks[i]].in[0]);
+    EmitValue(x);
+    Emit(VOP_ST, 0, 0, 0, MemIndex(sinks[i]), 0);
+    ConsumeUse(x);
+  }
+  Emit(VOP_END, 0, 0, 0, 0, 0);
+  {
+    uint32_t dts[DVM_CUBE_MAXMEM];
+    for (int i = 0; i < n_mem_; ++i) dts[i] = cmems_[i].dtype;
+    DropCastBeforeStore(dts);
+  }
+  h.n_mem = n_mem_;
+  h.n_code = static_cast<uint32_t>(code_.size());
+  h.mem_off = sizeof(VCubeHeader) / 8;
+  h.code_off = h.mem_off + n_mem_ * (sizeof(VCubeMem) / 8);
+  if (h.code_off + code_.size() > DVM_PARAM_WORDS) Fail("program larger than 4 KB");
+  std::memset(&prog_->blob, 0, sizeof(VmParam));
+  std::memcpy(prog_->blob.w, &h, sizeof(h));
+  std::memcpy(prog_->blob.w + h.mem_off, cmems_, sizeof(VCubeMem) * n_mem_);
+  std::memcpy(prog_->blob.w + h.code_off, code_.data(), 8 * code_.size());
+  prog_->threads = h.tile == 3 ? 512 : 256;
+  prog_->lds_bytes = DVM_CUBE_LDS_BYTES(static_cast<uint32_t>(bt));
+  prog_->grid = static_cast<uint32_t>(tiles(bt));
+}
+}  // namespace dvm

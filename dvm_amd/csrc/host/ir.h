@@ -162,11 +162,25 @@ float BF16BitsToF32(uint16_t h);
 uint32_t ScalarToContainer(const ScalarRef &s, DataType t);
 
 struct DeviceApi;  // bound C ABI of libdvm_hip.so (system.cc)
+class Compiler;    // compiler.h
+
+// Tuning switches from the environment, read once when a kernel object is made (code generation runs in
+// microseconds; a getenv per switch per compile is a measurable part of that). -1: not set.
+struct Tuning {
+  int vec_wide = -1;    // DVM_VEC_WIDE=1: four slabs per lane in the vector VM
+  int vec_team = -1;    // DVM_VEC_TEAM=n: at most n lanes per output in reduces along the innermost axis
+  int cube_tile = -1;   // DVM_CUBE_TILE=256|128|64
+  int cube_waves = -1;  // DVM_CUBE_WAVES=4|8
+  int attn_waves = -1;  // DVM_ATTN_WAVES=4
+  bool debug = false;   // DVM_DEBUG: node dump in compile errors
+  void Read();
+};
 
 class VKernel {
  public:
-  VKernel(KernelType t, uint32_t f) : ktype_(t), flags_(f) {}
+  VKernel(KernelType t, uint32_t f) : ktype_(t), flags_(f) { tuning_.Read(); }
   ~VKernel();
+  Tuning tuning_;
 
   KernelType KType() const { return ktype_; }
   uint32_t Flags() const { return flags_; }
@@ -210,6 +224,7 @@ class VKernel {
   bool normalized_ = false;
   bool compiled_ = false;
   int cur_stage_ = 0;
+  Compiler *compiler_ = nullptr;  // kept between code generations of a dynamic kernel: its tables keep their storage
   std::string dump_str_;
   friend class Compiler;
 };

@@ -1,0 +1,142 @@
+// VKernel::CodeGen / BindAddresses / Launch and the loop over partition modes.
+#include <algorithm>
+#include <cstdlib>
+#include <cmath>
+#include <cstddef>
+#include <cstring>
+#include <stdexcept>
+
+#include "compiler.h"
+
+namespace dvm {
+
+VKernel::~VKernel() {
+  delete compiler_;
+  for (NDObject *o : ops_) delete o;
+}
+
+void Tuning::Read() {
+  auto num = [](const char *name) {
+    const char *e = std::getenv(name);
+    return e != nullptr ? std::atoi(e) : -1;
+  };
+  vec_wide = num("DVM_VEC_WIDE");
+  vec_team = num("DVM_VEC_TEAM");
+  cube_tile = num("DVM_CUBE_TILE");
+  cube_waves = num("DVM_CUBE_WAVES");
+  attn_waves = num("DVM_ATTN_WAVES");
+  debug = std::getenv("DVM_DEBUG") != nullptr;
+}
+
+// Partition modes, tried in order until every sub-kernel compiles: 0 joins an operator to its
+// producers' sub-kernel whenever the hard rules allow, 1 also requires broadcast-compatible
+// shapes, 2 additionally ends a sub-kernel after every reduce (the reference's rule), 3 gives
+// every operator its own sub-kernel.
+size_t Compiler::Run() {
+  n_ = static_cast<int>(k_->ops_.size());
+  for (int mode = k_->part_mode_; mode < 3; ++mode) {
+    try {
+      const size_t ws = RunOnce(mode);
+      k_->part_mode_ = mode;
+      return ws;
+    } catch (const std::runtime_error &) {
+    }
+  }
+  k_->part_mode_ = 3;
+  return RunOnce(3);
+}
+
+size_t Compiler::RunOnce(int mode) {
+  mode_ = mode;
+  conservative_ = mode >= 2;
+  area_.assign(n_, -1);
+  level_.assign(n_, 0);
+  live_.assign(n_, 0);
+  mat_.assign(n_, 0);
+  absorbed_.assign(n_, 0);
+  ws_slot_.assign(n_, -1);
+  store_of_.assign(n_, -1);
+  MarkLive();
+  attn_groups_.clear();
+  attn_of_.assign(n_, -1);
+  if (mode_ == 0) DetectAttention();
+  Partition();
+  k_->programs_.clear();
+  k_->ws_sizes_.clear();
+  k_->ws_offsets_.clear();
+  PlanMaterialisation();
+  for (int a = 0; a < n_areas_; ++a) CompileArea(a);
+  size_t total = 0;
+  for (size_t i = 0; i < k_->ws_sizes_.size(); ++i) {
+    k_->ws_offsets_.push_back(total);
+    total += (k_->ws_sizes_[i] + 255) & ~static_cast<size_t>(255);
+  }
+  k_->ws_bytes_ = total;
+  return total;
+}
+
+size_t VKernel::CodeGen(bool /*pre*/) {
+  if (!normalized_) Normalize();
+  if (compiler_ == nullptr) compiler_ = new Compiler(this);
+  const size_t ws = compiler_->Run();
+  compiled_ = true;
+  return ws;
+}
+
+void VKernel::BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *alloc, void *workspace) {
+  for (size_t i = 0; i < n; ++i) {
+    if (relocs[i].io != nullptr) relocs[i].io->addr = relocs[i].addr;
+  }
+  if (ws_bytes_ > 0) {
+    if (workspace != nullptr) {
+      ws_base_ = workspace;
+    } else if (alloc != nullptr) {
+      ws_base_ = alloc->Alloc(ws_bytes_);
+    }
+    if (ws_base_ == nullptr) Throw("kernel needs workspace but none was provided");
+  }
+  for (Program &p : programs_) {
+    if (p.skip) continue;
+    for (const Program::Patch &pt : p.patches) {
+      uint64_t addr = 0;
+      if (pt.op_id >= 0) {
+        addr = reinterpret_cast<uint64_t>(ops_[pt.op_id]->addr);
+        if (addr != 0) addr += static_cast<uint64_t>(pt.byte_offset);
+      } else if (pt.ws_slot >= 0) {
+        addr = reinterpret_cast<uint64_t>(ws_base_) + ws_offsets_[pt.ws_slot] + static_cast<uint64_t>(pt.byte_offset);
+      }
+      if (addr == 0) Throw("a tensor address is missing at launch");
+      p.blob.w[pt.word] = addr;
+      if ((addr & 15u) != 0) {
+        if (pt.role == Program::kPatchVecMem) {
+          reinterpret_cast<VMemDesc *>(p.blob.w + pt.word)->flags &= ~static_cast<uint32_t>(VMF_ALIGNED);
+        } else if (pt.role == Program::kPatchCubeOperand) {
+          reinterpret_cast<VCubeHeader *>(p.blob.w)->fast = 0;
+        } else if (pt.role == Program::kPatchAligned16) {
+          Throw("fused attention needs 16-byte aligned tensors");
+        }
+      }
+    }
+  }
+}
+
+int VKernel::Launch(void *stream) {
+  if (!compiled_) Throw("Launch before CodeGen");
+  if (!g_system.HasDevice()) {
+    Throw(std::string("no MI355X device layer: ") + g_system.LoadError());
+  }
+  const DeviceApi &api = g_system.Api();
+  for (Program &p : programs_) {
+    for (const Program::Fill &f : p.fills) {
+      void *dst = f.op_id >= 0 ? ops_[f.op_id]->addr
+                               : static_cast<void *>(static_cast<char *>(ws_base_) + ws_offsets_[f.ws_slot]);
+      int rc = api.fill_u32(dst, f.value, f.bytes, stream);
+      if (rc != 0) return rc;
+    }
+    if (p.skip) continue;
+    int rc = api.launch_vm(&p.blob, p.grid, p.threads, p.lds_bytes, stream);
+    if (rc != 0) return rc;
+  }
+  return 0;
+}
+}  // namespace dvm

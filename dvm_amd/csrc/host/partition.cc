@@ -1,0 +1,307 @@
+// Which operators share a launch (sub-kernel), and which values cross launches through memory.
+#include <algorithm>
+#include <cstdlib>
+#include <cmath>
+#include <cstddef>
+#include <cstring>
+#include <stdexcept>
+
+#include "compiler.h"
+
+namespace dvm {
+
+// ---------- liveness ----------
+void Compiler::MarkLive() {
+  for (int i = n_ - 1; i >= 0; --i) {
+    NDObject *o = k_->ops_[i];
+    if (o->kind == kObjStore) live_[i] = 1;
+    if (!live_[i]) continue;
+    for (int j = 0; j < o->nin; ++j)
+      if (o->in[j] != nullptr) live_[o->in[j]->id] = 1;
+    for (NDObject *p : o->parts) live_[p->id] = 1;
+  }
+}
+
+bool Compiler::DomCompatible(const AreaInfo &ai, const int64_t *dims, int rank) const {
+  const int r = std::max(ai.rank, rank);
+  for (int i = 0; i < r; ++i) {
+    const int64_t da = i + ai.rank >= r ? ai.dom[i + ai.rank - r] : 1;
+    const int64_t db = i + rank >= r ? dims[i + rank - r] : 1;
+    if (da != db && da != 1 && db != 1) return false;
+  }
+  return true;
+}
+
+void Compiler::DomMerge(AreaInfo &ai, const int64_t *dims, int rank) {
+  const int r = std::max(ai.rank, rank);
+  int64_t out[kMaxRank];
+  for (int i = 0; i < r; ++i) {
+    const int64_t da = i + ai.rank >= r ? ai.dom[i + ai.rank - r] : 1;
+    const int64_t db = i + rank >= r ? dims[i + rank - r] : 1;
+    out[i] = da == 1 ? db : da;
+  }
+  std::memcpy(ai.dom, out, sizeof(int64_t) * r);
+  ai.rank = r;
+}
+
+bool Compiler::SameReduce(const NDObject *a, const NDObject *b) {
+  const NDObject *xa = a->in[0], *xb = b->in[0];
+  if (xa->rank() != xb->rank()) return false;
+  for (int i = 0; i < xa->rank(); ++i)
+    if (xa->dim(i) != xb->dim(i)) return false;
+  bool ra[kMaxRank] = {false}, rb[kMaxRank] = {false};
+  for (size_t i = 0; i < a->aux_ref->size; ++i) {
+    int64_t d = a->aux_ref->data[i];
+    ra[d < 0 ? d + xa->rank() : d] = true;
+  }
+  for (size_t i = 0; i < b->aux_ref->size; ++i) {
+    int64_t d = b->aux_ref->data[i];
+    rb[d < 0 ? d + xb->rank() : d] = true;
+  }
+  for (int i = 0; i < xa->rank(); ++i)
+    if (xa->dim(i) != 1 && ra[i] != rb[i]) return false;
+  return true;
+}
+
+// Sweep an operator would run in if it joined sub-kernel a: one more than the deepest reduce among the
+// operators of a it depends on.
+int Compiler::LevelIn(int a, const NDObject *o) const {
+  int lvl = 0;
+  for (int j = 0; j < o->nin; ++j) {
+    const NDObject *v = o->in[j];
+    if (v == nullptr || area_[v->id] != a) continue;
+    lvl = std::max(lvl, level_[v->id] + (v->kind == kObjReduce ? 1 : 0));
+  }
+  return lvl;
+}
+
+bool Compiler::CanJoin(int a, const NDObject *o) {
+  if (a >= static_cast<int>(areas_.size())) return true;  // a fresh sub-kernel
+  const AreaInfo &ai = areas_[a];
+  if (ai.stage != o->stage) return false;
+  // a store goes where the value it stores is computed (an operator's own output is never a reason to cut)
+  if (IsStoreLike(o) && ai.attn < 0 && !ai.cube && area_[o->in[0]->id] == a) return true;
+  if (o->kind == kObjReduce && LevelIn(a, o) < 8 && ai.red_at_level[LevelIn(a, o)] >= 2) return false;
+  if (o->kind == kObjMatMul) return false;
+  if (ai.n_ops >= kMaxAreaOps && !IsStoreLike(o)) return false;  // long graphs are cut into several launches
+  if (ai.attn >= 0) return o->kind == kObjStore && o->in[0] == attn_groups_[ai.attn].m2;
+  if (ai.cube) {
+    if (!IsPointwiseKind(o->kind)) return false;
+    if (mode_ >= 2 && !(o->kind == kObjStore && o->in[0] == ai.cube_op)) return false;  // plain matmul, epilogue on its own
+    // the epilogue works on the matmul's own output domain
+    const NDObject *c = ai.cube_op;
+    if (o->rank() != c->rank()) return false;
+    for (int i = 0; i < o->rank(); ++i)
+      if (o->dim(i) != c->dim(i)) return false;
+    return true;
+  }
+  if (o->kind == kObjReduce) {
+    if (ai.has_reduce && !SameReduce(ai.reduce, o)) return false;
+    return mode_ == 0 || DomCompatible(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
+  }
+  // A store of a value from outside (a load, a view, another launch's result) is a copy nothing else in the
+  // sub-kernel relates to: it joins only one whose index space it fills, element for element.
+  if (IsStoreLike(o) && ai.n_ops > 0) {  // same extents in the same order, dims of extent 1 aside
+    int i = 0, j = 0;
+    while (true) {
+      while (i < ai.rank && ai.dom[i] == 1) ++i;
+      while (j < o->rank() && o->dim(j) == 1) ++j;
+      if (i == ai.rank || j == o->rank()) break;
+      if (ai.dom[i] != o->dim(j)) return false;
+      ++i;
+      ++j;
+    }
+    if (i != ai.rank || j != o->rank()) return false;
+  }
+  return mode_ == 0 || DomCompatible(ai, o->shape_ref_->data, o->rank());
+}
+
+void Compiler::Join(int a, const NDObject *o) {
+  while (a >= static_cast<int>(areas_.size())) areas_.push_back(AreaInfo());
+  AreaInfo &ai = areas_[a];
+  if (ai.n_ops == 0) ai.stage = o->stage;
+  ++ai.n_ops;
+  level_[o->id] = LevelIn(a, o);
+  if (o->kind == kObjReduce && level_[o->id] < 8) ++ai.red_at_level[level_[o->id]];
+  if (o->kind == kObjMatMul) {
+    ai.cube = true;
+    ai.cube_op = o;
+    return;
+  }
+  if (ai.cube) return;
+  if (o->kind == kObjReduce) {
+    if (!ai.has_reduce) {
+      ai.has_reduce = true;
+      ai.reduce = o;
+    }
+    DomMerge(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
+  }
+  DomMerge(ai, o->shape_ref_->data, o->rank());
+}
+
+void Compiler::Partition() {
+  areas_.clear();
+  const bool fuse = !conservative_;
+  // Operators that share no tensor (directly or through other operators) never share a
+  // sub-kernel: connected components are numbered first, each gets its own range of areas.
+  std::vector<int> &comp = scratch_a_;
+  comp.resize(n_);
+  for (int i = 0; i < n_; ++i) comp[i] = i;
+  auto find = [&](int x) {
+    while (comp[x] != x) x = comp[x] = comp[comp[x]];
+    return x;
+  };
+  for (int i = 0; i < n_; ++i) {
+    NDObject *o = k_->ops_[i];
+    if (!live_[i]) continue;
+    for (int j = 0; j < o->nin; ++j) {
+      if (o->in[j] == nullptr || o->in[j]->kind == kObjBroadcastS) continue;
+      comp[find(i)] = find(o->in[j]->id);
+    }
+  }
+  std::vector<int> &comp_base = scratch_b_;
+  comp_base.assign(n_, -1);
+  for (int i = 0; i < n_; ++i) {
+    NDObject *o = k_->ops_[i];
+    if (!live_[i] || IsLeaf(o)) continue;
+    if (IsView(o)) continue;  // read through by its consumers
+    if (o->kind == kObjConcat) {  // complete once the last of its parts has run; never computed itself
+      int a = 0;
+      for (const NDObject *p : o->parts) a = std::max(a, area_[p->id]);
+      area_[i] = a;
+      continue;
+    }
+    const int c = find(i);
+    if (comp_base[c] < 0) comp_base[c] = static_cast<int>(areas_.size());
+    if (attn_of_[i] >= 0) {
+      AttnGroup &g = attn_groups_[attn_of_[i]];
+      if (g.area < 0) {
+        g.area = static_cast<int>(areas_.size());
+        areas_.push_back(AreaInfo());
+        areas_.back().attn = attn_of_[i];
+        areas_.back().stage = o->stage;
+        areas_.back().n_ops = 1;
+      }
+      area_[i] = g.area;
+      continue;
+    }
+    int a = comp_base[c];
+    for (int j = 0; j < o->nin; ++j) {
+      const NDObject *v = o->in[j];
+      if (v == nullptr || IsLeaf(v)) continue;
+      bool cut = false;
+      if (IsView(v)) {
+        v = ViewRoot(v);
+        if (IsLeaf(v)) continue;
+        cut = true;
+      }
+      if (o->kind == kObjMatMul || v->kind == kObjConcat) cut = true;
+      if (!fuse && v->kind == kObjReduce && !IsStoreLike(o)) cut = true;  // the reference's rule: a reduce ends its sub-kernel
+      a = std::max(a, area_[v->id] + (cut ? 1 : 0));
+    }
+    if (o->kind == kObjMatMul || (mode_ >= 3 && !IsStoreLike(o))) a = std::max(a, static_cast<int>(areas_.size()));
+    while (!CanJoin(a, o)) ++a;
+    area_[i] = a;
+    Join(a, o);
+  }
+  n_areas_ = static_cast<int>(areas_.size());
+}
+
+// ---------- which values cross sub-kernels ----------
+void Compiler::PlanMaterialisation() {
+  for (int i = 0; i < n_; ++i) {
+    NDObject *o = k_->ops_[i];
+    if (!live_[i]) continue;
+    // a value stored through a stride list is not read back from there by later launches: they expect
+    // the dense layout, so such a value also goes to the workspace when it crosses launches
+    if (o->kind == kObjStore && !o->strided) store_of_[o->in[0]->id] = i;
+  }
+  for (int i = 0; i < n_; ++i) {
+    NDObject *o = k_->ops_[i];
+    if (!live_[i] || IsLeaf(o)) continue;
+    for (int j = 0; j < o->nin; ++j) {
+      const NDObject *v = o->in[j];
+      if (v == nullptr) continue;
+      const NDObject *root = ViewRoot(v);
+      if (IsLeaf(root) || root->kind == kObjLoad) continue;
+      const int user_area = IsView(o) ? -2 : area_[i];
+      if (IsView(v) || (user_area != -2 && area_[root->id] != user_area)) mat_[root->id] = 1;
+    }
+  }
+  for (int i = 0; i < n_; ++i)
+    if (live_[i] && k_->ops_[i]->kind == kObjConcat) mat_[i] = 1;  // its parts need the buffer whoever reads it
+  for (int i = 0; i < n_; ++i) {
+    if (!mat_[i]) continue;
+    NDObject *o = k_->ops_[i];
+    if (store_of_[i] >= 0 && area_[store_of_[i]] == area_[i]) continue;  // later kernels read the user's output
+    if (o->kind == kObjConcat && store_of_[i] >= 0) {  // the parts write straight into the stored output
+      absorbed_[store_of_[i]] = 1;
+      continue;
+    }
+    ws_slot_[i] = static_cast<int>(k_->ws_sizes_.size());
+    k_->ws_sizes_.push_back(static_cast<size_t>(std::max<int64_t>(o->numel(), 1)) * DTypeSize(o->type_id_));
+  }
+}
+
+// ---------- fused attention ----------
+
+void Compiler::DetectAttention() {
+  std::vector<int> &uses = scratch_a_;
+  uses.assign(n_, 0);
+  for (int i = 0; i < n_; ++i) {
+    if (!live_[i]) continue;
+    const NDObject *o = k_->ops_[i];
+    for (int j = 0; j < o->nin; ++j)
+      if (o->in[j] != nullptr) ++uses[o->in[j]->id];
+  }
+  auto last_axis_keep = [](const NDObject *r) {
+    if (!r->keepdims || r->aux_ref == nullptr || r->aux_ref->size != 1) return false;
+    const int64_t ax = r->aux_ref->data[0];
+    return ax == -1 || ax == r->in[0]->rank() - 1;
+  };
+  for (int i = 0; i < n_; ++i) {
+    if (!live_[i]) continue;
+    NDObject *m2 = k_->ops_[i];
+    if (m2->kind != kObjMatMul || m2->trans_a || m2->trans_b || m2->in[2] != nullptr) continue;
+    if (m2->type_id_ != kFloat16 && m2->type_id_ != kBFloat16) continue;
+    NDObject *p = m2->in[0], *v = m2->in[1];
+    if (p->kind != kObjCast || p->in[0]->type_id_ != kFloat32 || uses[p->id] != 1) continue;
+    NDObject *dv = p->in[0];
+    if (dv->kind != kObjBinary || dv->op != kDiv || uses[dv->id] != 1) continue;
+    NDObject *e = dv->in[0], *sm = dv->in[1];
+    if (sm->kind != kObjReduce || sm->op != kSum || sm->in[0] != e || uses[sm->id] != 1 || !last_axis_keep(sm)) continue;
+    if (e->kind != kObjUnary || e->op != kExp || uses[e->id] != 2) continue;
+    NDObject *sb = e->in[0];
+    if (sb->kind != kObjBinary || sb->op != kSub || uses[sb->id] != 1) continue;
+    NDObject *x = sb->in[0], *mx = sb->in[1];
+    if (mx->kind != kObjReduce || mx->op != kMax || mx->in[0] != x || uses[mx->id] != 1 || !last_axis_keep(mx)) continue;
+    if (x->kind != kObjCast || x->type_id_ != kFloat32 || uses[x->id] != 2) continue;
+    NDObject *sc = x->in[0];
+    NDObject *m1 = sc;
+    float scale = 1.0f;
+    NDObject *mul = nullptr;
+    if (sc->kind == kObjBinaryS && sc->op == kMul && uses[sc->id] == 1) {
+      mul = sc;
+      m1 = sc->in[0];
+      const uint32_t bits = ScalarToContainer(sc->scalar.Get(), sc->in[0]->type_id_);
+      std::memcpy(&scale, &bits, 4);
+    }
+    if (m1->kind != kObjMatMul || m1->trans_a || !m1->trans_b || m1->in[2] != nullptr || uses[m1->id] != 1) continue;
+    if (m1->type_id_ != m2->type_id_) continue;
+    NDObject *q = m1->in[0], *kk = m1->in[1];
+    if (q->kind != kObjLoad || kk->kind != kObjLoad || v->kind != kObjLoad || q->strided || kk->strided || v->strided) continue;
+    const int r = q->rank();
+    if (kk->rank() != r || v->rank() != r || r < 2) continue;
+    bool ok = q->dim(r - 1) == DVM_ATTN_D && kk->dim(r - 1) == DVM_ATTN_D && v->dim(r - 1) == DVM_ATTN_D && kk->dim(r - 2) == v->dim(r - 2) &&
+              kk->dim(r - 2) % DVM_ATTN_BKV == 0 && kk->dim(r - 2) > 0 && q->dim(r - 2) > 0;
+    for (int d = 0; d < r - 2 && ok; ++d) ok = q->dim(d) == kk->dim(d) && q->dim(d) == v->dim(d) && q->dim(d) > 0;
+    if (!ok || q->numel() >= (1ll << 31) || kk->numel() >= (1ll << 31)) continue;
+    AttnGroup g = {m1, m2, q, kk, v, scale, -1};
+    const int gi = static_cast<int>(attn_groups_.size());
+    attn_groups_.push_back(g);
+    NDObject *members[] = {m1, mul, x, mx, sb, e, sm, dv, p, m2};
+    for (NDObject *mbr : members)
+      if (mbr != nullptr) attn_of_[mbr->id] = gi;
+  }
+}
+}  // namespace dvm

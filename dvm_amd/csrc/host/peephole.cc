@@ -1,0 +1,198 @@
+// Passes over the emitted instruction words of a vector program.
+#include <algorithm>
+#include <cstdlib>
+#include <cmath>
+#include <cstddef>
+#include <cstring>
+#include <stdexcept>
+
+#include "compiler.h"
+
+namespace dvm {
+
+// A rounding cast to fp16 / bf16 whose only reader is the store right behind it does nothing the store's own
+// conversion does not do (same round to nearest even): the cast instruction is dropped. `mem_dtypes[i]` is the
+// element type of memory operand i.
+void Compiler::DropCastBeforeStore(const uint32_t *mem_dtypes) {
+  std::vector<uint64_t> &out = scratch_code_;
+  out.clear();
+  out.reserve(code_.size());
+  for (size_t i = 0; i < code_.size(); ++i) {
+    const uint64_t w = code_[i];
+    if (VI_OP(w) == VOP_CAST && VI_SUB(w) == VC_RND && !(static_cast<uint32_t>(w) & VI_UNIFORM) && i + 2 < code_.size() + 1 && i + 1 < code_.size()) {
+      const uint64_t st = code_[i + 1];
+      const uint32_t next = i + 2 < code_.size() ? VI_OP(code_[i + 2]) : static_cast<uint32_t>(VOP_END);
+      const bool acc_dead = next == VOP_END || next == VOP_ENDSWEEP || next == VOP_SWEEP || next == VOP_LD || next == VOP_LDR ||
+                            next == VOP_LDS || next == VOP_LDI || next == VOP_FIN;
+      if (VI_OP(st) == VOP_ST && acc_dead) {
+        const uint32_t dt = mem_dtypes[VI_A(st)];
+        if ((VI_RND(w) == VRND_F16 && dt == VDT_F16) || (VI_RND(w) == VRND_BF16 && dt == VDT_BF16)) continue;
+      }
+    }
+    out.push_back(w);
+  }
+  code_.swap(out);
+}
+
+// The interpreter pays a fixed price per instruction, so the short bodies of sweeps are tightened:
+//  * sum(x) and sum(x * x) of one value (mean and variance in one pass): the multiply joins the second reduce;
+//  * two float binaries in a row with S-register operands (x * scale + shift) become one chained instruction;
+//  * the VOP_ENDSWEEP behind a store or a reduce becomes a flag of that instruction.
+// Every fused form computes what the separate instructions compute, rounding by rounding.
+void Compiler::FuseSweepInstructions() {
+  auto defines_acc = [](uint32_t op) {
+    return op == VOP_LD || op == VOP_LDR || op == VOP_LDS || op == VOP_LDI || op == VOP_FIN || op == VOP_END;
+  };
+  std::vector<uint64_t> &out = scratch_code_;
+  out.clear();
+  out.reserve(code_.size());
+  size_t sweep_first = 0;  // index in code_ of the first instruction of the sweep being copied
+  for (size_t i = 0; i < code_.size(); ++i) {
+    const uint64_t w = code_[i];
+    const uint32_t lo = static_cast<uint32_t>(w);
+    if (VI_OP(w) == VOP_SWEEP) sweep_first = i + 1;
+    // Mul acc, acc ; reduce_sum rB, acc ; endsweep   (acc dead afterwards)  ->  reduce_sum.square rB, acc
+    if (VI_OP(w) == VOP_BINF && (VI_SUB(w) & 0x3fu) == VB_MUL && VI_KIND(w) == VK_ACC && VI_RND(w) == VRND_NONE &&
+        !(lo & VI_UNIFORM) && i + 2 < code_.size() && VI_OP(code_[i + 1]) == VOP_RED && VI_SUB(code_[i + 1]) == VR_SUM &&
+        VI_OP(code_[i + 2]) == VOP_ENDSWEEP && i + 3 < code_.size() && defines_acc(VI_OP(code_[i + 3])) &&
+        sweep_first < code_.size() && defines_acc(VI_OP(code_[sweep_first])) && sweep_first <= i) {
+      out.push_back(code_[i + 1] | (static_cast<uint64_t>(VRF_SQUARE) << 8));
+      ++i;
+      continue;
+    }
+    // two S-register float binaries in a row
+    if (VI_OP(w) == VOP_BINF && VI_KIND(w) == VK_SREG && !(lo & VI_UNIFORM) && i + 1 < code_.size()) {
+      const uint64_t n = code_[i + 1];
+      if (VI_OP(n) == VOP_BINF && VI_KIND(n) == VK_SREG && !(static_cast<uint32_t>(n) & VI_UNIFORM)) {
+        const uint32_t second = (VI_SUB(n) & 0x3fu) | (VI_A(n) << 8) | (VI_RND(n) << 16);
+        out.push_back(VI_MAKE(VOP_BINF, VI_SUB(w), VK_SREG2, VI_RND(w), VI_A(w), second));
+        ++i;
+        continue;
+      }
+    }
+    out.push_back(w);
+  }
+  // store / reduce ; endsweep  ->  one instruction that also closes the round; a sweep with nothing in it goes
+  code_.clear();
+  for (size_t i = 0; i < out.size(); ++i) {
+    uint64_t w = out[i];
+    if (VI_OP(w) == VOP_SWEEP && (VI_IMM(w) & 0xffu) == (VR_NONE | (VR_NONE << 4)) && i + 1 < out.size() &&
+        VI_OP(out[i + 1]) == VOP_ENDSWEEP) {
+      ++i;
+      continue;
+    }
+    if (i + 1 < out.size() && VI_OP(out[i + 1]) == VOP_ENDSWEEP) {
+      if (VI_OP(w) == VOP_ST) {
+        code_.push_back(w | VI_ENDS);
+        ++i;
+        continue;
+      }
+      if (VI_OP(w) == VOP_RED) {
+        code_.push_back(w | VI_ENDS);
+        ++i;
+        continue;
+      }
+    }
+    code_.push_back(w);
+  }
+}
+
+// Between sweeps a program computes per-output values (a mean, a scale): the same in every lane of the team
+// that owns the output. When the team is the whole workgroup, such a run is executed by one wave, which hands
+// the S registers and the accumulator to the others (VOP_UNI_BEGIN / VOP_UNI_END); sixteen waves interpreting
+// the same twenty scalar instructions cost more than the two barriers.
+void Compiler::MarkUniformRuns() {
+  if ((hdr_.sched & VS_KIND_MASK) != VS_REDX || !hdr_.team_is_block) return;
+  auto bcast_load = [&](uint64_t w) {
+    return VI_OP(w) == VOP_LD && VI_KIND(w) == VK_MEM && !(mems_[VI_A(w)].flags & (VMF_VEC | VMF_GATHER)) && !mem_is_view_[VI_A(w)];
+  };
+  auto starts = [&](uint64_t w) {
+    const uint32_t op = VI_OP(w);
+    return op == VOP_FIN || op == VOP_LDS || op == VOP_LDI || bcast_load(w);
+  };
+  auto inside = [&](uint64_t w) {
+    const uint32_t op = VI_OP(w);
+    if (starts(w) || op == VOP_STS) return true;
+    const bool arith = op == VOP_UN || op == VOP_CAST || op == VOP_BINF || op == VOP_BINI || op == VOP_CMP;
+    return arith && (static_cast<uint32_t>(w) & VI_UNIFORM) != 0;
+  };
+  std::vector<uint64_t> &out = scratch_code_;
+  out.clear();
+  out.reserve(code_.size() + 8);
+  bool in_sweep = false;
+  for (size_t i = 0; i < code_.size();) {
+    const uint64_t w = code_[i];
+    const uint32_t op = VI_OP(w);
+    if (op == VOP_SWEEP) in_sweep = true;
+    if (static_cast<uint32_t>(w) & VI_ENDS) {
+      in_sweep = false;
+    }
+    if (!in_sweep && starts(w)) {
+      size_t j = i;
+      while (j < code_.size() && inside(code_[j])) ++j;
+      if (j - i >= 4) {
+        out.push_back(VI_MAKE(VOP_UNI_BEGIN, 0, 0, 0, 0, static_cast<uint32_t>(j - i + 1)));
+        out.insert(out.end(), code_.begin() + i, code_.begin() + j);
+        out.push_back(VI_MAKE(VOP_UNI_END, 0, 0, 0, 0, 0));
+        i = j;
+        continue;
+      }
+    }
+    out.push_back(w);
+    ++i;
+  }
+  code_.swap(out);
+}
+
+// A reduce with consumers reads its input twice: once for the statistics, once to apply them. What the
+// second sweep does not have to fetch again from HBM:
+//  * the first rounds of the first sweep stay in the workgroup's spare local memory (VI_LD_KEEP_WR/RD);
+//  * a later sweep without reduces of its own runs last round first (VSW_REVERSE), starting with the data the
+//    L2 cache still holds from the end of the sweep before, and ending with the parked rounds.
+// Called with the blob filled in and lds_bytes set; edits the instruction words in the blob.
+void Compiler::PlanRereads() {
+  // tuning switch DVM_VEC_REREAD: 0 off, 2 parked rounds only, 3 reversed sweeps only (default: both)
+  static const char mode = std::getenv("DVM_VEC_REREAD") != nullptr ? std::getenv("DVM_VEC_REREAD")[0] : '1';
+  const bool on = mode != '0', park = mode != '3', reverse = mode != '2';
+  if (!on || (hdr_.sched & VS_KIND_MASK) != VS_REDX || (hdr_.sched & VS_WIDE)) return;
+  uint64_t *cw = prog_->blob.w + hdr_.code_off;
+  const size_t n = code_.size();
+  const uint32_t team = hdr_.team_is_block ? prog_->threads : (1u << hdr_.team_log2);
+  const uint32_t per_round = team * u_;
+  const uint32_t n_rounds = (hdr_.n_ridx + per_round - 1) / per_round;
+  if (n_rounds < 2) return;
+  // sweeps: position of the VOP_SWEEP word and of the load that opens it (or -1)
+  struct Sw { size_t at; int ld; bool reduces; };
+  std::vector<Sw> sweeps;
+  for (size_t i = 0; i < n; ++i) {
+    if (VI_OP(cw[i]) != VOP_SWEEP) continue;
+    Sw sw{i, -1, (VI_IMM(cw[i]) & 0xffu) != (VR_NONE | (VR_NONE << 4))};
+    if (i + 1 < n && VI_OP(cw[i + 1]) == VOP_LD && VI_KIND(cw[i + 1]) == VK_MEM && (mems_[VI_A(cw[i + 1])].flags & VMF_VEC)) {
+      sw.ld = static_cast<int>(i + 1);
+    }
+    sweeps.push_back(sw);
+  }
+  for (size_t k = 1; k < sweeps.size(); ++k) {
+    if (reverse && !sweeps[k].reduces) cw[sweeps[k].at] |= static_cast<uint64_t>(VSW_REVERSE) << 8;
+  }
+  // park rounds of the first pair of sweeps that open with a load of the same operand
+  if (!park) return;
+  for (size_t a = 0; a + 1 < sweeps.size(); ++a) {
+    if (sweeps[a].ld < 0) continue;
+    for (size_t b = a + 1; b < sweeps.size(); ++b) {
+      if (sweeps[b].ld < 0 || VI_A(cw[sweeps[b].ld]) != VI_A(cw[sweeps[a].ld])) continue;
+      // local memory left to this workgroup when as many workgroups as the registers allow share the CU
+      const uint32_t per_cu = 1024 / std::max<uint32_t>(prog_->threads, 64);
+      const uint32_t budget = std::min<uint32_t>(160 * 1024, g_system.lds_per_wg) / per_cu;
+      const uint32_t fixed = prog_->lds_bytes + DVM_PARAM_BYTES + 1024;
+      const uint32_t per_keep = prog_->threads * u_ * 32;
+      if (budget <= fixed + per_keep) return;
+      const uint32_t rounds = std::min<uint32_t>(n_rounds, (budget - fixed) / per_keep);
+      cw[sweeps[a].ld] |= VI_LD_KEEP_WR | (static_cast<uint64_t>(rounds) << 32);
+      cw[sweeps[b].ld] |= VI_LD_KEEP_RD | (static_cast<uint64_t>(rounds) << 32);
+      prog_->lds_bytes += rounds * per_keep;
+      return;
+    }
+  }
+}
+}  // namespace dvm
