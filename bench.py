@@ -243,6 +243,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true", help="omit the other BASELINE configs")
+    ap.add_argument("--configs", default="add,rmsnorm,attention,matmul", help="which of the other BASELINE configs to run (comma separated)")
     ap.add_argument("--traffic-probe", action="store_true", help="launch the headline kernel and a plain copy only (for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -273,9 +274,10 @@ def main():
     if not args.skip_cpu:
         line["cpu_baseline"] = cpu_baseline_batchnorm(bn["x"], bn["g"], bn["b"], bn["alg_bytes"])
     if not args.only_headline:
-        line["configs"] = {"add_fp32_32x32": bench_add(), "residual_rmsnorm_bf16_dynamic": bench_rmsnorm(),
-                           "attention_fp16_b8_h32_s2048_d128": bench_attention(),
-                           "matmul_bias_silu_bf16_8192x4096x4096": bench_matmul()}
+        others = {"add": ("add_fp32_32x32", bench_add), "rmsnorm": ("residual_rmsnorm_bf16_dynamic", bench_rmsnorm),
+                  "attention": ("attention_fp16_b8_h32_s2048_d128", bench_attention),
+                  "matmul": ("matmul_bias_silu_bf16_8192x4096x4096", bench_matmul)}
+        line["configs"] = {others[c][0]: others[c][1]() for c in args.configs.split(",") if c in others}
     print(json.dumps(line))
 
 

@@ -194,9 +194,10 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
       uint64_t need = static_cast<uint64_t>(threads) * 8 + static_cast<uint64_t>(h->n_vslot) * u * 16 * threads;
       uint64_t parked = 0;
       for (uint64_t i = h->code_off; i < code_end; ++i) {
-        if (VI_OP(p.w[i]) == VOP_LD && (static_cast<uint32_t>(p.w[i]) & (VI_LD_KEEP_WR | VI_LD_KEEP_RD))) {
+        if (VI_OP(p.w[i]) != VOP_LD) continue;
+        if (static_cast<uint32_t>(p.w[i]) & (VI_LD_KEEP_WR | VI_LD_KEEP_RD)) {
           if (wide) return static_cast<int>(hipErrorInvalidValue);
-          parked = std::max<uint64_t>(parked, VI_IMM(p.w[i]));
+          parked = std::max<uint64_t>(parked, VI_IMM(p.w[i]) & 0xffffu);
         }
       }
       need += parked * threads * u * 32;

@@ -35,6 +35,11 @@ typedef uint32_t vu2 __attribute__((ext_vector_type(2)));
 typedef _Float16 vh8 __attribute__((ext_vector_type(8)));
 
 #define DVM_GLOBAL __attribute__((address_space(1)))
+
+// local memory of a workgroup: the program (copied from the kernel argument once) and the dynamic segment
+// (reduce partials and hand-over boxes, V registers, parked rounds; laid out by the host)
+__shared__ uint32_t prog32[DVM_PARAM_BYTES / 4];
+extern __shared__ double lds[];
 #define FOR_U _Pragma("unroll") for (int u = 0; u < U; ++u)
 #define FOR_E _Pragma("unroll") for (int e = 0; e < E; ++e)
 
@@ -224,20 +229,53 @@ __device__ __attribute__((noinline)) void mem_store_slow(uint64_t addr, uint32_t
   }
 }
 
-// Wide path of a load: every lane of the wave owns U full, aligned slabs. All loads are issued before any use.
-__device__ __forceinline__ void mem_load_wide(const VMemDesc &m, const Offs &off, Acc &out) {
+// Which slabs of a round the whole wave can treat alike. `full`: bit u is set when slab u is full in every lane;
+// `uniform`: every slab is either full in every lane or empty in every lane, so the wave takes the wide paths on
+// the slabs in `full` and skips the others (the last round of a sweep usually has some slabs past the end).
+struct Slabs {
+  uint32_t nvp;      // valid counts, 4 bits per slab
+  uint32_t full;
+  bool uniform;
+};
+
+__device__ __forceinline__ Slabs slab_state(uint32_t nvp) {
+  Slabs s;
+  s.nvp = nvp;
+  s.full = 0;
+  uint32_t mixed = 0;
+  FOR_U {
+    const uint32_t nv = (nvp >> (4 * u)) & 0xfu;
+    const bool all_full = wave_all(nv == static_cast<uint32_t>(E));
+    const bool all_empty = wave_all(nv == 0u);
+    s.full |= (all_full ? 1u : 0u) << u;
+    mixed |= (all_full || all_empty) ? 0u : 1u;
+  }
+  s.uniform = mixed == 0u;
+  return s;
+}
+
+// Wide path of a load: the slabs in `full` are full and aligned in every lane of the wave (the others are empty
+// in every lane and read as zero). All loads are issued before any use.
+__device__ __forceinline__ void mem_load_wide(const VMemDesc &m, const Offs &off, uint32_t full, Acc &out) {
   const uint32_t dtype = m.dtype;
   if (dtype == VDT_F32 || dtype == VDT_I32) {
     vf4 a[U], b[U];
     FOR_U {
-      const DVM_GLOBAL vf4 *p = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off.v[u] * 4);
-      a[u] = p[0];
-      b[u] = p[1];
+      a[u] = 0.0f;
+      b[u] = 0.0f;
+      if ((full >> u) & 1u) {
+        const DVM_GLOBAL vf4 *p = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off.v[u] * 4);
+        a[u] = p[0];
+        b[u] = p[1];
+      }
     }
     FOR_U out.v[u] = __builtin_shufflevector(a[u], b[u], 0, 1, 2, 3, 4, 5, 6, 7);
   } else if (dtype == VDT_BF16) {
     vu4 a[U];
-    FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(m.addr + off.v[u] * 2);
+    FOR_U {
+      a[u] = 0u;
+      if ((full >> u) & 1u) a[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(m.addr + off.v[u] * 2);
+    }
     FOR_U {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -247,11 +285,17 @@ __device__ __forceinline__ void mem_load_wide(const VMemDesc &m, const Offs &off
     }
   } else if (dtype == VDT_F16) {
     vh8 a[U];
-    FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off.v[u] * 2);
+    FOR_U {
+      a[u] = static_cast<_Float16>(0.0f);
+      if ((full >> u) & 1u) a[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off.v[u] * 2);
+    }
     FOR_U out.v[u] = __builtin_convertvector(a[u], vf8);
   } else {
     vu2 a[U];
-    FOR_U a[u] = *reinterpret_cast<const DVM_GLOBAL vu2 *>(m.addr + off.v[u]);
+    FOR_U {
+      a[u] = 0u;
+      if ((full >> u) & 1u) a[u] = *reinterpret_cast<const DVM_GLOBAL vu2 *>(m.addr + off.v[u]);
+    }
     FOR_U {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -262,9 +306,10 @@ __device__ __forceinline__ void mem_load_wide(const VMemDesc &m, const Offs &off
   }
 }
 
-__device__ __forceinline__ void mem_store_wide(const VMemDesc &m, const Offs &off, const Acc &in) {
+__device__ __forceinline__ void mem_store_wide(const VMemDesc &m, const Offs &off, uint32_t full, const Acc &in) {
   const uint32_t dtype = m.dtype;
   FOR_U {
+    if (!((full >> u) & 1u)) continue;
     if (dtype == VDT_F32 || dtype == VDT_I32) {
       DVM_GLOBAL vf4 *p = reinterpret_cast<DVM_GLOBAL vf4 *>(m.addr + off.v[u] * 4);
       p[0] = __builtin_shufflevector(in.v[u], in.v[u], 0, 1, 2, 3);
@@ -289,10 +334,11 @@ __device__ __forceinline__ void mem_store_wide(const VMemDesc &m, const Offs &of
   }
 }
 
-__device__ __forceinline__ void mem_load(const VMemDesc &m, const Offs &off, uint32_t nvp, Acc &out) {
+__device__ __forceinline__ void mem_load(const VMemDesc &m, const Offs &off, const Slabs &sl, Acc &out) {
+  const uint32_t nvp = sl.nvp;
   const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
-  if (fast && wave_all(nvp == kAllFull)) {
-    mem_load_wide(m, off, out);
+  if (fast && sl.uniform) {
+    mem_load_wide(m, off, sl.full, out);
   } else if (!(m.flags & (VMF_VEC | VMF_GATHER)) && (m.dtype == VDT_F32 || m.dtype == VDT_I32)) {
     // one 32-bit element per slab, replicated (an operand broadcast along the innermost axis: a per-channel
     // scale, a per-row statistic); lanes without a valid slab read the base element and get zero, like the
@@ -307,12 +353,12 @@ __device__ __forceinline__ void mem_load(const VMemDesc &m, const Offs &off, uin
   }
 }
 
-__device__ __forceinline__ void mem_store(const VMemDesc &m, const Offs &off, uint32_t nvp, const Acc &in) {
+__device__ __forceinline__ void mem_store(const VMemDesc &m, const Offs &off, const Slabs &sl, const Acc &in) {
   const bool fast = (m.flags & (VMF_VEC | VMF_ALIGNED)) == (VMF_VEC | VMF_ALIGNED);
-  if (fast && wave_all(nvp == kAllFull)) {
-    mem_store_wide(m, off, in);
+  if (fast && sl.uniform) {
+    mem_store_wide(m, off, sl.full, in);
   } else {
-    mem_store_slow(m.addr, m.dtype, m.flags, off, nvp, in);
+    mem_store_slow(m.addr, m.dtype, m.flags, off, sl.nvp, in);
   }
 }
 
@@ -384,10 +430,11 @@ __device__ __forceinline__ void red_accumulate_k(RedAcc<SCHED> &r, const Acc &x,
   }
 }
 
-// Every slab of every lane of the wave is full (the common round): no per-element guards.
+// The slabs in `full` are full in every lane of the wave, the others empty (the common rounds): no per-element guards.
 template <int SCHED, int KIND>
-__device__ __forceinline__ void red_accumulate_full(RedAcc<SCHED> &r, const Acc &x) {
+__device__ __forceinline__ void red_accumulate_full(RedAcc<SCHED> &r, const Acc &x, uint32_t full) {
   FOR_U {
+    if (!((full >> u) & 1u)) continue;
     if constexpr (SCHED == VS_REDY) {
       FOR_E r.v[e] = red_op<KIND>(r.v[e], static_cast<double>(x.v[u][e]));
     } else {
@@ -403,14 +450,15 @@ __device__ __forceinline__ void red_accumulate_full(RedAcc<SCHED> &r, const Acc 
 }
 
 template <int SCHED>
-__device__ __forceinline__ void red_accumulate(RedAcc<SCHED> &r, uint32_t kind, const Acc &x, uint32_t nvp) {
-  if (wave_all(nvp == kAllFull)) {
+__device__ __forceinline__ void red_accumulate(RedAcc<SCHED> &r, uint32_t kind, const Acc &x, const Slabs &sl) {
+  const uint32_t nvp = sl.nvp;
+  if (sl.uniform) {
     if (kind == VR_SUM) {
-      red_accumulate_full<SCHED, VR_SUM>(r, x);
+      red_accumulate_full<SCHED, VR_SUM>(r, x, sl.full);
     } else if (kind == VR_MAX) {
-      red_accumulate_full<SCHED, VR_MAX>(r, x);
+      red_accumulate_full<SCHED, VR_MAX>(r, x, sl.full);
     } else {
-      red_accumulate_full<SCHED, VR_MIN>(r, x);
+      red_accumulate_full<SCHED, VR_MIN>(r, x, sl.full);
     }
     return;
   }
@@ -450,30 +498,62 @@ __device__ __forceinline__ void red_accumulate_int(RedAcc<SCHED> &r, uint32_t ki
   }
 }
 
-// Combines one slot's partials across the lanes that share an output; every
-// one of those lanes ends up with the result.
-template <int SCHED>
-__device__ __forceinline__ RedAcc<SCHED> red_finalize(RedAcc<SCHED> r, uint32_t rk, uint32_t tlog, bool team_is_block,
-                                                                uint32_t tid, uint32_t nthreads, uint32_t k_local,
-                                                                uint32_t r_local, double *scratch) {
-  rk = uni(rk);
+// Local memory shared by the lanes of a workgroup, in doubles from the start of the dynamic segment:
+//   [0, 64)   partials of the waves at the end of a sweep: two buffers (used in turn) of two slots of 16 waves;
+//   [64, 80)  what the first wave hands to the others after a per-team run: two buffers (in turn) of 16 floats.
+// With the buffers used in turn a wave cannot overwrite what a slower wave still has to read: between two uses of
+// one buffer lies the barrier of the other one, which the slower wave only reaches once its reads are done.
+// VS_REDY uses [0, lanes) as one buffer with barriers on both sides.
+constexpr uint32_t kPartialsPerBuffer = 32;
+constexpr uint32_t kBoxAt = 64;
+
+// End of a sweep, innermost axis reduced: combines the partials of both slots across the lanes that share an
+// output (a team inside a wave by shuffles; a team that is the workgroup through local memory, one barrier for
+// both slots). Every one of those lanes ends up with the results. `flip` selects the buffer and is toggled.
+__device__ __forceinline__ void red_finish_x(double &r0, double &r1, uint32_t k0, uint32_t k1, uint32_t tlog, bool team_is_block,
+                                             uint32_t tid, uint32_t nthreads, uint32_t &flip, double *shared) {
+  k0 = uni(k0);
+  k1 = uni(k1);
   tlog = uni(tlog);
   team_is_block = uni(team_is_block ? 1u : 0u) != 0u;
   nthreads = uni(nthreads);
-  if constexpr (SCHED == VS_REDX) {
-    double t = r.v[0];
-    const uint32_t span = team_is_block ? 64u : (1u << tlog);
-    for (uint32_t msk = 1; msk < span; msk <<= 1) t = red_combine(rk, t, shfl_xor_f64(t, msk));
-    if (team_is_block) {
-      const uint32_t nw = (nthreads + 63u) >> 6;
-      __syncthreads();
-      scratch[tid >> 6] = t;  // every lane of a wave holds the wave's value: identical writes, no per-lane branch
-      __syncthreads();
-      t = scratch[0];
-      for (uint32_t j = 1; j < nw; ++j) t = red_combine(rk, t, scratch[j]);
+  const bool on0 = k0 <= VR_MIN, on1 = k1 <= VR_MIN;
+  double t0 = r0, t1 = r1;
+  const uint32_t span = team_is_block ? 64u : (1u << tlog);
+  for (uint32_t msk = 1; msk < span; msk <<= 1) {
+    if (on0) t0 = red_combine(k0, t0, shfl_xor_f64(t0, msk));
+    if (on1) t1 = red_combine(k1, t1, shfl_xor_f64(t1, msk));
+  }
+  if (team_is_block) {
+    double *buf = shared + flip * kPartialsPerBuffer;
+    flip ^= 1u;
+    const uint32_t wave = tid >> 6, nw = (nthreads + 63u) >> 6;
+    buf[wave] = t0;  // every lane of a wave holds the wave's value: identical writes, no per-lane branch
+    buf[16 + wave] = t1;
+    __syncthreads();
+    // lane j takes wave (j mod 16)'s partial; four shuffle steps leave the total in every lane
+    const uint32_t j = tid & 15u;
+    const double a0 = buf[j], a1 = buf[16 + j];
+    t0 = j < nw ? a0 : red_identity(k0);
+    t1 = j < nw ? a1 : red_identity(k1);
+    for (uint32_t msk = 1; msk < 16u; msk <<= 1) {
+      if (on0) t0 = red_combine(k0, t0, shfl_xor_f64(t0, msk));
+      if (on1) t1 = red_combine(k1, t1, shfl_xor_f64(t1, msk));
     }
-    r.v[0] = t;
-  } else if constexpr (SCHED == VS_REDY) {
+  }
+  r0 = t0;
+  r1 = t1;
+}
+
+// End of a sweep, innermost axis kept: the rows of the workgroup that share an output group combine their
+// partials through local memory, element by element.
+template <int SCHED>
+__device__ __forceinline__ RedAcc<SCHED> red_finish_y(RedAcc<SCHED> r, uint32_t rk, uint32_t tlog, uint32_t nthreads, uint32_t k_local,
+                                                      uint32_t r_local, double *scratch) {
+  rk = uni(rk);
+  tlog = uni(tlog);
+  nthreads = uni(nthreads);
+  if constexpr (SCHED == VS_REDY) {
     const uint32_t tx = 1u << tlog, ty = nthreads >> tlog;
     if (ty > 1) {
       FOR_E {
@@ -575,16 +655,20 @@ __device__ __forceinline__ void vreg_load(const vf4 *planes, uint32_t slot, uint
   }
 }
 
+// A memory operand's descriptor from the program in local memory. Only what the interpreter branches on (element
+// type, flags) is made wave-uniform; the address and the strides only ever enter per-lane arithmetic, where a copy
+// in every lane serves as well as a scalar register and costs no v_readfirstlane and no scalar registers.
 __device__ __forceinline__ VMemDesc load_desc(const uint32_t *prog32, uint32_t mem_off_words, uint32_t idx) {
-  const uint32_t *d = prog32 + 2 * mem_off_words + idx * (sizeof(VMemDesc) / 4);
+  const vu4 *d = reinterpret_cast<const vu4 *>(prog32 + 2 * mem_off_words + idx * (sizeof(VMemDesc) / 4));
+  const vu4 d0 = d[0], d1 = d[1], d2 = d[2];
   VMemDesc m;
-  m.addr = static_cast<uint64_t>(uni(d[0])) | (static_cast<uint64_t>(uni(d[1])) << 32);
-  m.dtype = uni(d[2]);
-  m.flags = uni(d[3]);
+  m.addr = static_cast<uint64_t>(d0[0]) | (static_cast<uint64_t>(d0[1]) << 32);
+  m.dtype = uni(d0[2]);
+  m.flags = uni(d0[3]);
 #pragma unroll
   for (int i = 0; i < DVM_VEC_MAXR; ++i) {
-    m.kstride[i] = uni(d[4 + i]);
-    m.rstride[i] = uni(d[4 + DVM_VEC_MAXR + i]);
+    m.kstride[i] = d1[i];
+    m.rstride[i] = d2[i];
   }
   return m;
 }
@@ -592,7 +676,9 @@ __device__ __forceinline__ VMemDesc load_desc(const uint32_t *prog32, uint32_t m
 // Splits a flat index of an index space into its coordinates and returns the
 // element offset sum(coord * stride). The innermost-axis coordinate counts
 // E-groups when `inner` is set and is converted to elements.
-__device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim (&dims)[DVM_VEC_MAXR], uint32_t ndim,
+// `dims` points at the axis table in local memory: its entries feed per-lane arithmetic only, so they are read
+// where they are needed (one 128-bit read per division) instead of living in scalar registers for the whole launch.
+__device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim *dims, uint32_t ndim,
                                                  const uint32_t (&stride)[DVM_VEC_MAXR], bool inner) {
   uint64_t off = 0;
 #pragma unroll
@@ -600,8 +686,9 @@ __device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim (&dims)[
     if (i < static_cast<int>(ndim)) {
       uint32_t c = n;
       if (i + 1 < static_cast<int>(ndim)) {
-        const uint32_t q = fast_div(n, dims[i]);
-        c = n - q * dims[i].extent;
+        const vu4 dv = *reinterpret_cast<const vu4 *>(dims + i);  // extent, magic, shift, pad
+        const uint32_t q = (__umulhi(n, dv[1]) + n) >> dv[2];
+        c = n - q * dv[0];
         n = q;
       }
       if (i == 0 && inner) c *= E;
@@ -612,10 +699,13 @@ __device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim (&dims)[
 }
 
 // Valid element count (0..E) of the E-group with flat index n in a space whose first axis counts groups.
-__device__ __forceinline__ uint32_t group_valid(uint32_t n, const VDim (&dims)[DVM_VEC_MAXR], uint32_t ndim,
+__device__ __forceinline__ uint32_t group_valid(uint32_t n, const VDim *dims, uint32_t ndim,
                                                 uint32_t inner_extent) {
   uint32_t c = n;
-  if (ndim > 1) c = n - fast_div(n, dims[0]) * dims[0].extent;
+  if (ndim > 1) {
+    const vu4 dv = *reinterpret_cast<const vu4 *>(dims);
+    c = n - ((__umulhi(n, dv[1]) + n) >> dv[2]) * dv[0];
+  }
   const uint32_t left = inner_extent - c * E;
   return left < static_cast<uint32_t>(E) ? left : static_cast<uint32_t>(E);
 }
@@ -689,8 +779,6 @@ __device__ __forceinline__ float uniform_cast(uint32_t sub, float x) {
 
 template <int SCHED>
 __device__ __forceinline__ void vm_vector(const VmParam &p) {
-  extern __shared__ double lds[];
-  __shared__ uint32_t prog32[DVM_PARAM_BYTES / 4];
   // The blob arrives as a kernel argument; decoding from there would cost a
   // dependent scalar-memory round trip per access, so each workgroup copies it
   // into local memory once and decodes from there.
@@ -709,11 +797,26 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     }
     __syncthreads();
   }
-  VVecHeader h;
+  // the scalar fields of the header live in scalar registers; the axis tables stay in local memory
+  struct {
+    uint32_t n_kdim, n_rdim, team_log2, team_is_block, n_kidx, n_ridx, inner_extent, n_items, mem_off, code_off, n_vslot;
+    const VDim *kdims, *rdims;
+  } h;
   {
-    uint32_t *hw = reinterpret_cast<uint32_t *>(&h);
-#pragma unroll
-    for (int i = 0; i < static_cast<int>(sizeof(VVecHeader) / 4); ++i) hw[i] = uni(prog32[i]);
+    const VVecHeader *hp = reinterpret_cast<const VVecHeader *>(prog32);
+    h.n_kdim = uni(hp->n_kdim);
+    h.n_rdim = uni(hp->n_rdim);
+    h.team_log2 = uni(hp->team_log2);
+    h.team_is_block = uni(hp->team_is_block);
+    h.n_kidx = uni(hp->n_kidx);
+    h.n_ridx = uni(hp->n_ridx);
+    h.inner_extent = uni(hp->inner_extent);
+    h.n_items = uni(hp->n_items);
+    h.mem_off = uni(hp->mem_off);
+    h.code_off = uni(hp->code_off);
+    h.n_vslot = uni(hp->n_vslot);
+    h.kdims = hp->kdims;
+    h.rdims = hp->rdims;
   }
   const uint32_t mem_off = h.mem_off;
   const uint32_t *code32 = prog32 + 2 * h.code_off;
@@ -751,6 +854,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   RedAcc<SCHED> racc0, racc1;
   red_init<SCHED>(racc0, VR_SUM);
   red_init<SCHED>(racc1, VR_SUM);
+  uint32_t red_flip = 0, box_flip = 0;  // which of the two shared buffers the next sweep end / hand-over uses
 
   for (uint32_t item = blockIdx.x; item < h.n_items; item += gridDim.x) {
     // position of the lane in the kept space (POINTWISE: of slab 0; slab u is nthreads further each)
@@ -772,8 +876,9 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       nvp_out = nv * kAllOnes;
     }
 
+    const Slabs sl_out = slab_state(nvp_out);
     bool in_sweep = false;
-    uint32_t nvp = nvp_out;
+    Slabs sl = sl_out;  // valid counts of the current round's slabs (outside sweeps: of the lane's output)
     uint32_t round = 0, sweep_pc = 0, slot_kinds = 0;
     bool sweep_rev = false;   // the sweep walks its rounds last to first (VSW_REVERSE)
     uint32_t ridx = r_local;  // reduce-space index of slab 0 in the current round
@@ -799,6 +904,66 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       pc += ((op == VOP_UNI_BEGIN ? 1u : 0u) & skips_runs) * (imm - 1u);
       fetched = code64[pc];
 
+      // ---- a run of per-output arithmetic (VOP_UNI_BEGIN .. VOP_UNI_END): every instruction in it works on one
+      // value per lane, so the run has a small loop of its own: one float instead of the accumulator's U*E, a
+      // switch over the few opcodes a run may hold. (The waves that skip the run are already past it.) ----
+      if constexpr (SCHED == VS_REDX) {
+        if (op == VOP_UNI_BEGIN && skips_runs == 0u) {
+          const uint32_t run_end = pc + imm - 1u;  // index of the VOP_UNI_END
+          float x = acc.v[0][0];
+          while (pc < run_end) {
+            const uint32_t r0 = uni(fetched[0]);
+            const uint32_t rimm = uni(fetched[1]);
+            ++pc;
+            fetched = code64[pc];
+            const uint32_t rop = r0 & 0x7fu, rsub = (r0 >> 8) & 0xffu, ra = r0 >> 24, rkind = (r0 >> 16) & 0xfu;
+            if (rop >= VOP_SRC_BASE && rop != VOP_LD) {
+              const float sv = rkind == VK_IMM ? __uint_as_float(rimm) : (rkind == VK_SREG ? sreg_read(sr, ra) : x);
+              x = uniform_binary(rop, rsub, x, sv);
+              if (rop == VOP_BINF) {
+                const uint32_t rnd = (r0 >> 20) & 0x3u;
+                x = rnd == VRND_F16 ? round_f16(x) : (rnd == VRND_BF16 ? round_bf16(x) : x);
+              }
+              continue;
+            }
+            switch (rop) {
+              case VOP_FIN: {
+                const double d = ra == 0 ? racc0.v[0] : racc1.v[0];
+                x = (rsub & VRF_INT) ? __int_as_float(static_cast<int32_t>(d)) : static_cast<float>(d);
+                break;
+              }
+              case VOP_LDS: x = sreg_read(sr, ra); break;
+              case VOP_LDI: x = __uint_as_float(rimm); break;
+              case VOP_STS: sreg_write(sr, ra, x); break;
+              case VOP_LD: {  // one element per output (an operand without the reduced axes), any type
+                const VMemDesc m = load_desc(prog32, mem_off, ra);
+                uint64_t koff = last_off.v[0];
+                if (!(r0 & VI_SAME_OFFS)) koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, false);
+                FOR_U last_off.v[u] = koff;
+                const float v = elem_load(m.addr, m.dtype, kvalid ? koff : 0u);
+                x = kvalid ? v : 0.0f;
+                break;
+              }
+              case VOP_UN: {
+                x = uniform_unary(rsub, x);
+                const uint32_t rnd = (r0 >> 20) & 0x3u;
+                x = rnd == VRND_F16 ? round_f16(x) : (rnd == VRND_BF16 ? round_bf16(x) : x);
+                break;
+              }
+              default: {  // VOP_CAST
+                x = uniform_cast(rsub, x);
+                if (rsub == VC_I2F || rsub == VC_RND) {
+                  const uint32_t rnd = (r0 >> 20) & 0x3u;
+                  x = rnd == VRND_F16 ? round_f16(x) : (rnd == VRND_BF16 ? round_bf16(x) : x);
+                }
+                break;
+              }
+            }
+          }
+          FOR_U acc.v[u] = x;
+          continue;  // `fetched` holds the VOP_UNI_END
+        }
+      }
       // ---- one value per lane (VI_UNIFORM): compute element 0 and copy it ----
       if (w0 & VI_UNIFORM) {
         const uint32_t kind = (w0 >> 16) & 0xfu;
@@ -902,7 +1067,8 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             if constexpr (SCHED == VS_REDX) {
               // rounds parked in local memory by the load that opened an earlier sweep over this operand
               const uint32_t lr = sweep_rev ? n_rounds - 1u - round : round;
-              const bool parked = in_sweep && lr < imm;
+              const uint32_t n_parked = imm & 0xffffu;
+              const bool parked = in_sweep && lr < n_parked;
               if (parked && (w0 & VI_LD_KEEP_RD)) {
                 FOR_U {
                   const vf4 lo = keep_lds[((lr * U + u) * 2u) * nthreads + tid], hi = keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid];
@@ -910,7 +1076,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                 }
                 continue;
               }
-              mem_load(m, off, nvp, acc);
+              mem_load(m, off, sl, acc);
               if (parked && (w0 & VI_LD_KEEP_WR)) {
                 FOR_U {
                   keep_lds[((lr * U + u) * 2u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 0, 1, 2, 3);
@@ -919,10 +1085,10 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               }
               continue;
             }
-            mem_load(m, off, nvp, acc);
+            mem_load(m, off, sl, acc);
             continue;
           }
-          mem_load(m, off, nvp, src);
+          mem_load(m, off, sl, src);
         } else if (kind == VK_SREG) {
           const float v = sreg_read(sr, a);
           FOR_U src.v[u] = v;
@@ -1020,8 +1186,8 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
           if constexpr (SCHED == VS_REDX) {
             if (team_is_block) {
               // what the run produced lives in the first wave's S registers and accumulator: pass it on
-              float *box = reinterpret_cast<float *>(lds);  // the reduce scratch is idle between sweeps
-              __syncthreads();
+              float *box = reinterpret_cast<float *>(lds + kBoxAt) + box_flip * 16u;
+              box_flip ^= 1u;
               if (skips_runs == 0u) {  // the first wave; its lanes hold identical values
                 *reinterpret_cast<vf4 *>(box) = vf4{sr.s0, sr.s1, sr.s2, sr.s3};
                 *reinterpret_cast<vf4 *>(box + 4) = vf4{sr.s4, sr.s5, sr.s6, sr.s7};
@@ -1032,7 +1198,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               const float av = box[8];
               sr.s0 = lo[0]; sr.s1 = lo[1]; sr.s2 = lo[2]; sr.s3 = lo[3];
               sr.s4 = hi[0]; sr.s5 = hi[1]; sr.s6 = hi[2]; sr.s7 = hi[3];
-              FOR_U acc.v[u] = av;  // (the next user of the scratch starts with a barrier of its own)
+              FOR_U acc.v[u] = av;
             }
           }
           break;
@@ -1040,7 +1206,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
         case VOP_ST: {
           const VMemDesc m = load_desc(prog32, mem_off, a);
           Offs off;
-          uint32_t nvs = nvp;
+          Slabs st = sl;
           if (w0 & VI_SAME_OFFS) {
             off = last_off;
           } else {
@@ -1062,9 +1228,12 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             last_off = off;
           }
           if constexpr (SCHED != VS_POINTWISE) {
-            if (!in_sweep) nvs = r_local == 0 ? (nvp & 0xfu) : 0u;  // one lane per output, one slab
+            if (!in_sweep) {  // one lane per output, one slab: never the wide path
+              st.nvp = r_local == 0 ? (sl.nvp & 0xfu) : 0u;
+              st.uniform = false;
+            }
           }
-          mem_store(m, off, nvs, acc);
+          mem_store(m, off, st, acc);
           break;
         }
         case VOP_UN: {
@@ -1111,14 +1280,18 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             if (sub & VRF_SQUARE) FOR_U acc.v[u] = acc.v[u] * acc.v[u];  // the emitter fuses only where acc is dead afterwards
             if (sub & VRF_INT) {
               if (a == 0) {
-                red_accumulate_int<SCHED>(racc0, sub & 0xfu, acc, nvp);
+                red_accumulate_int<SCHED>(racc0, sub & 0xfu, acc, sl.nvp);
               } else {
-                red_accumulate_int<SCHED>(racc1, sub & 0xfu, acc, nvp);
+                red_accumulate_int<SCHED>(racc1, sub & 0xfu, acc, sl.nvp);
               }
             } else if (a == 0) {
-              red_accumulate<SCHED>(racc0, sub & 0xfu, acc, nvp);
+              red_accumulate<SCHED>(racc0, sub & 0xfu, acc, sl);
+              if (sub & VRF_PAIR) {  // the emitter pairs only where acc is dead afterwards
+                FOR_U acc.v[u] = acc.v[u] * acc.v[u];
+                red_accumulate<SCHED>(racc1, sub & 0xfu, acc, sl);
+              }
             } else {
-              red_accumulate<SCHED>(racc1, sub & 0xfu, acc, nvp);
+              red_accumulate<SCHED>(racc1, sub & 0xfu, acc, sl);
             }
             break;
           }
@@ -1162,15 +1335,21 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
           } else {
             in_sweep = false;
             const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
-            if (k0 <= VR_MIN) racc0 = red_finalize<SCHED>(racc0, k0, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
-            if (k1 <= VR_MIN) racc1 = red_finalize<SCHED>(racc1, k1, tlog, team_is_block, tid, nthreads, k_local, r_local, lds);
+            if constexpr (SCHED == VS_REDX) {
+              if (k0 <= VR_MIN || k1 <= VR_MIN) {
+                red_finish_x(racc0.v[0], racc1.v[0], k0, k1, tlog, team_is_block, tid, nthreads, red_flip, lds);
+              }
+            } else {
+              if (k0 <= VR_MIN) racc0 = red_finish_y<SCHED>(racc0, k0, tlog, nthreads, k_local, r_local, lds);
+              if (k1 <= VR_MIN) racc1 = red_finish_y<SCHED>(racc1, k1, tlog, nthreads, k_local, r_local, lds);
+            }
           }
         }
 
         // valid counts of the round's slabs
         if (op == VOP_SWEEP || ends) {
           if (in_sweep) {
-            nvp = 0;
+            uint32_t nvp = 0;
             FOR_U {
               const uint32_t ru = ridx + u * r_step;
               const bool ok = kvalid && ru < h.n_ridx;
@@ -1178,8 +1357,9 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               nv &= ok ? 0xfu : 0u;
               nvp |= nv << (4 * u);
             }
+            sl = slab_state(nvp);
           } else {
-            nvp = nvp_out;
+            sl = sl_out;
           }
         }
       }

@@ -62,6 +62,8 @@ struct ANode {
   uint8_t reg_fmt;
   bool in_cone;
   int last_sec;         // last section with a consumer
+  int slot;             // AK_REDUCE: reduce slot of its sweep
+  bool slot_ready;      // AK_REDUCE: the combined result sits in its slot (from the end of its sweep to the next sweep)
 };
 
 struct Axis {

@@ -141,19 +141,20 @@ std::string &VKernel::DisAssemble() {
             break;
           }
           case VOP_RED:
-            os << "reduce_" << kRed[sub & 0xf] << ((sub & VRF_SQUARE) ? ".square" : "") << ((sub & VRF_INT) ? ".int32" : "") << " r" << VI_A(w) << ", acc";
+            os << "reduce_" << kRed[sub & 0xf] << ((sub & VRF_SQUARE) ? ".square" : "") << ((sub & VRF_PAIR) ? " (and its square into r1)" : "") << ((sub & VRF_INT) ? ".int32" : "") << " r" << VI_A(w) << ", acc";
             if (static_cast<uint32_t>(w) & VI_ENDS) os << "  ; endsweep";
             break;
           case VOP_SWEEP: os << ((sub & VSW_REVERSE) ? "sweep (last round first) slots=" : "sweep slots=") << kRed[(VI_IMM(w) & 0xf) < 3 ? (VI_IMM(w) & 0xf) : 0]
-                             << ((VI_IMM(w) & 0xf) < 3 ? "" : "(none)"); break;
+                             << ((VI_IMM(w) & 0xf) < 3 ? "" : "(none)");
+            break;
           case VOP_ENDSWEEP: os << "endsweep"; break;
           case VOP_FIN: os << "mov" << ((sub & VRF_INT) ? ".int32" : "") << " acc, r" << VI_A(w); break;
-          case VOP_UNI_BEGIN: os << "uniform run, " << (VI_IMM(w) - 1) << " instructions: first wave only when the team is the workgroup"; break;
-          case VOP_UNI_END: os << "end of uniform run"; break;
+          case VOP_UNI_BEGIN: os << "per-output run, " << (VI_IMM(w) - 1) << " instructions on one value per lane (first wave only when the team is the workgroup)"; break;
+          case VOP_UNI_END: os << "end of per-output run"; break;
           case VOP_LD:
             os << "load." << kMemTypes[mem_dtype(VI_A(w))] << " acc, m" << VI_A(w);
-            if (static_cast<uint32_t>(w) & VI_LD_KEEP_WR) os << "  ; parks its first " << VI_IMM(w) << " rounds in local memory";
-            if (static_cast<uint32_t>(w) & VI_LD_KEEP_RD) os << "  ; takes its first " << VI_IMM(w) << " rounds from local memory";
+            if (static_cast<uint32_t>(w) & VI_LD_KEEP_WR) os << "  ; parks its first " << (VI_IMM(w) & 0xffffu) << " rounds in local memory";
+            if (static_cast<uint32_t>(w) & VI_LD_KEEP_RD) os << "  ; takes its first " << (VI_IMM(w) & 0xffffu) << " rounds from local memory";
             break;
           case VOP_BINF:
             if (VI_KIND(w) == VK_SREG2) {  // two chained operations

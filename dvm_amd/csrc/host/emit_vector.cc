@@ -169,6 +169,7 @@ void Compiler::BeforeOverwrite() {
   ANode &n = nodes_[acc_node_];
   if (n.kind == AK_MEM || n.kind == AK_SCALAR) return;  // cheaper to fetch again than to park
   const bool needed_later = n.last_sec > cur_sec_ && (!n.fd || single_round_);
+  if (n.kind == AK_REDUCE && n.slot_ready && !needed_later) return;  // still in its slot
   if ((n.uses > 0 || needed_later) && n.reg < 0) SaveAcc(acc_node_);
 }
 
@@ -226,6 +227,12 @@ void Compiler::EmitValue(int v) {
     } else {
       Emit(VOP_LDR, n.reg_fmt, 0, 0, n.reg, 0);
     }
+    acc_node_ = v;
+    return;
+  }
+  if (n.kind == AK_REDUCE && n.slot_ready) {
+    BeforeOverwrite();
+    Emit(VOP_FIN, n.dtype == kInt32 ? VRF_INT : 0, 0, 0, n.slot, 0);
     acc_node_ = v;
     return;
   }
@@ -457,12 +464,15 @@ void Compiler::EmitSection(int sec) {
     nodes_[i].in_cone = false;
   }
   if (!sweep && sec > 0) {
-    // results of the previous sweep's reduces become register values
+    // The previous sweep's reduces have their results in the slots, where this section reads them as often as
+    // it likes; a result that a later section needs becomes a register value now (the next sweep reuses the slots).
     for (int i = 0; i < nn_; ++i) {
       ANode &n = nodes_[i];
       if (n.kind != AK_REDUCE || n.sec != sec - 1) continue;
+      n.slot_ready = true;
+      if (n.last_sec <= sec) continue;
       BeforeOverwrite();
-      Emit(VOP_FIN, n.dtype == kInt32 ? VRF_INT : 0, 0, 0, n.reg_fmt, 0);
+      Emit(VOP_FIN, n.dtype == kInt32 ? VRF_INT : 0, 0, 0, n.slot, 0);
       acc_node_ = i;
       SaveAcc(i);
     }
@@ -500,10 +510,11 @@ void Compiler::EmitSection(int sec) {
       if (slot >= DVM_VEC_NSLOT) Fail("more than two reduces in one sweep");
       const uint32_t rk = n.op->op == kSum ? VR_SUM : (n.op->op == kMax ? VR_MAX : VR_MIN);
       kinds = (kinds & ~(0xfu << (4 * slot))) | (rk << (4 * slot));
-      n.reg_fmt = static_cast<uint8_t>(slot);  // slot number until the result is fetched
+      n.slot = slot;
       ++slot;
     }
     BeforeOverwrite();
+    for (int i = 0; i < nn_; ++i) nodes_[i].slot_ready = false;  // the sweep starts its slots afresh
     Emit(VOP_SWEEP, 0, 0, 0, 0, kinds);
     if (!single_round_) acc_node_ = -1;
   }
@@ -515,7 +526,7 @@ void Compiler::EmitSection(int sec) {
     EmitValue(x);
     if (n.kind == AK_REDUCE) {
       const uint32_t rk = n.op->op == kSum ? VR_SUM : (n.op->op == kMax ? VR_MAX : VR_MIN);
-      Emit(VOP_RED, rk | (n.dtype == kInt32 ? VRF_INT : 0), 0, 0, n.reg_fmt, 0);
+      Emit(VOP_RED, rk | (n.dtype == kInt32 ? VRF_INT : 0), 0, 0, n.slot, 0);
     } else {
       Emit(VOP_ST, 0, 0, 0, MemIndex(sinks[i]), 0);
     }

@@ -22,6 +22,7 @@ void Tuning::Read() {
   };
   vec_wide = num("DVM_VEC_WIDE");
   vec_team = num("DVM_VEC_TEAM");
+  vec_runs = num("DVM_VEC_RUNS");
   cube_tile = num("DVM_CUBE_TILE");
   cube_waves = num("DVM_CUBE_WAVES");
   attn_waves = num("DVM_ATTN_WAVES");

@@ -81,6 +81,13 @@ void Compiler::FuseSweepInstructions() {
       ++i;
       continue;
     }
+    // reduce_sum r0 ; reduce_sum.square r1 ; endsweep  ->  one instruction for both slots
+    if (VI_OP(w) == VOP_RED && VI_SUB(w) == VR_SUM && VI_A(w) == 0 && i + 2 < out.size() && VI_OP(out[i + 1]) == VOP_RED &&
+        VI_SUB(out[i + 1]) == (VR_SUM | VRF_SQUARE) && VI_A(out[i + 1]) == 1 && VI_OP(out[i + 2]) == VOP_ENDSWEEP) {
+      code_.push_back(w | (static_cast<uint64_t>(VRF_PAIR) << 8) | VI_ENDS);
+      i += 2;
+      continue;
+    }
     if (i + 1 < out.size() && VI_OP(out[i + 1]) == VOP_ENDSWEEP) {
       if (VI_OP(w) == VOP_ST) {
         code_.push_back(w | VI_ENDS);
@@ -97,12 +104,15 @@ void Compiler::FuseSweepInstructions() {
   }
 }
 
-// Between sweeps a program computes per-output values (a mean, a scale): the same in every lane of the team
-// that owns the output. When the team is the whole workgroup, such a run is executed by one wave, which hands
-// the S registers and the accumulator to the others (VOP_UNI_BEGIN / VOP_UNI_END); sixteen waves interpreting
-// the same twenty scalar instructions cost more than the two barriers.
+// Between sweeps a program computes per-output values (a mean, a scale): one number per lane, the same in every
+// lane of the team that owns the output. A run of such instructions is bracketed (VOP_UNI_BEGIN / VOP_UNI_END) and
+// the interpreter executes it in a small loop of its own, on one float instead of the whole accumulator. When the
+// team is the whole workgroup, only its first wave executes the run and hands the S registers and the accumulator
+// to the others through local memory: sixteen waves interpreting the same twenty scalar instructions cost more
+// than the one barrier.
 void Compiler::MarkUniformRuns() {
-  if ((hdr_.sched & VS_KIND_MASK) != VS_REDX || !hdr_.team_is_block) return;
+  if ((hdr_.sched & VS_KIND_MASK) != VS_REDX) return;
+  if (k_->tuning_.vec_runs == 1 && !hdr_.team_is_block) return;  // tuning: runs only where one wave stands in for the others
   auto bcast_load = [&](uint64_t w) {
     return VI_OP(w) == VOP_LD && VI_KIND(w) == VK_MEM && !(mems_[VI_A(w)].flags & (VMF_VEC | VMF_GATHER)) && !mem_is_view_[VI_A(w)];
   };
@@ -175,24 +185,25 @@ void Compiler::PlanRereads() {
   for (size_t k = 1; k < sweeps.size(); ++k) {
     if (reverse && !sweeps[k].reduces) cw[sweeps[k].at] |= static_cast<uint64_t>(VSW_REVERSE) << 8;
   }
+  // local memory left to this workgroup when as many workgroups as the registers allow share the CU
+  const uint32_t per_cu = 1024 / std::max<uint32_t>(prog_->threads, 64);
+  const uint32_t budget = std::min<uint32_t>(160 * 1024, g_system.lds_per_wg) / per_cu;
+  uint32_t fixed = prog_->lds_bytes + DVM_PARAM_BYTES + 1024;
+  const uint32_t per_round_bytes = prog_->threads * u_ * 32;  // one round of one operand, as fp32
   // park rounds of the first pair of sweeps that open with a load of the same operand
   if (!park) return;
   for (size_t a = 0; a + 1 < sweeps.size(); ++a) {
     if (sweeps[a].ld < 0) continue;
     for (size_t b = a + 1; b < sweeps.size(); ++b) {
       if (sweeps[b].ld < 0 || VI_A(cw[sweeps[b].ld]) != VI_A(cw[sweeps[a].ld])) continue;
-      // local memory left to this workgroup when as many workgroups as the registers allow share the CU
-      const uint32_t per_cu = 1024 / std::max<uint32_t>(prog_->threads, 64);
-      const uint32_t budget = std::min<uint32_t>(160 * 1024, g_system.lds_per_wg) / per_cu;
-      const uint32_t fixed = prog_->lds_bytes + DVM_PARAM_BYTES + 1024;
-      const uint32_t per_keep = prog_->threads * u_ * 32;
-      if (budget <= fixed + per_keep) return;
-      const uint32_t rounds = std::min<uint32_t>(n_rounds, (budget - fixed) / per_keep);
+      if (budget <= fixed + per_round_bytes) return;
+      const uint32_t rounds = std::min<uint32_t>(n_rounds, (budget - fixed) / per_round_bytes);
       cw[sweeps[a].ld] |= VI_LD_KEEP_WR | (static_cast<uint64_t>(rounds) << 32);
       cw[sweeps[b].ld] |= VI_LD_KEEP_RD | (static_cast<uint64_t>(rounds) << 32);
-      prog_->lds_bytes += rounds * per_keep;
+      prog_->lds_bytes += rounds * per_round_bytes;
       return;
     }
   }
 }
+
 }  // namespace dvm

@@ -116,6 +116,7 @@ enum {
 // reduce kinds (low 4 bits of VOP_RED's sub field), and two modifiers of VOP_RED
 enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 #define VRF_SQUARE 0x10u  // acc = acc * acc (the fp32 product) first; the multiply of a sum of squares rides in the reduce
+#define VRF_PAIR 0x40u    // VOP_RED into slot 0: the same value, squared, also goes to slot 1 (sum and sum of squares in one instruction)
 #define VRF_INT 0x20u     // VOP_RED (max / min) and VOP_FIN: the values are int32 bit patterns, compared as integers
 
 // instruction word:
@@ -191,9 +192,10 @@ typedef struct {
   uint32_t mem_off;      // word offset of VMemDesc[n_mem]
   uint32_t code_off;     // word offset of the instruction words
   uint32_t n_vslot;      // V register slots in use (each U*16 bytes per lane of local memory)
+  uint32_t pad[4];       // (keeps the axis tables 16-byte aligned: the interpreter reads them as 128-bit words)
   VDim kdims[DVM_VEC_MAXR];
   VDim rdims[DVM_VEC_MAXR];
-} VVecHeader;            // 64 + 128 = 192 bytes
+} VVecHeader;            // 80 + 128 = 208 bytes
 
 // ---- matmul programs (VE_CUBE) ---------------------------------------------------
 // C[b][m][n] = sum_k A[b][m][k] * B[b][k][n], fp32 accumulation on MFMA, then an epilogue program
