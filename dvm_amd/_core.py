@@ -24,7 +24,7 @@ def _load():
         raise ImportError(
             "dvm_amd native library missing (%s): run `python -m dvm_amd.build` first" % _LIB_PATH)
     lib = ctypes.CDLL(_LIB_PATH)
-    if not hasattr(lib, "dvm_rt_unbind_device"):
+    if not hasattr(lib, "dvm_rt_perf_samples"):
         raise ImportError("dvm_amd native library (%s) is older than the package: run `python -m dvm_amd.build`"
                           % _LIB_PATH)
     vp, ci, cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_size_t
@@ -79,6 +79,7 @@ def _load():
         "dvm_rt_output": (ci, [vp, vp, vp, cs]),
         "dvm_rt_device_ptr": (vp, [vp, vp]),
         "dvm_rt_perf": (ci, [vp, ci, ci, ctypes.POINTER(ctypes.c_double)]),
+        "dvm_rt_perf_samples": (ci, [vp, ci, ci, ctypes.POINTER(ctypes.c_double)]),
         "dvm_rt_num_launches": (ci, [vp]),
         "dvm_rt_workspace_bytes": (cs, [vp]),
         "dvm_rt_program_count": (ci, [vp]),
@@ -405,6 +406,10 @@ class PyKernel(Kernel):
         self._load_shape[op._h] = ref
         return op
 
+    def load_shape(self, load):
+        """The updatable shape behind a load (update it and generate code again to change the extent)."""
+        return self._load_shape[load._h]
+
     def clone(self, base, remap):
         """Copies `base`'s graph into this kernel (RtKernelPy::Clone, src/pybind_api.cc:923-993). `remap` lists
         operators, shape / axis references and scalar references of `base`; their counterparts here are returned."""
@@ -538,6 +543,12 @@ class PyKernel(Kernel):
                 raise RuntimeError(_lib.dvm_c_last_error().decode())
             out.append((bytes(blob), (geo[0], geo[1], geo[2]), [words[j] for j in range(n)]))
         return out
+
+    def perf_samples(self, warmup=3, iters=20):
+        """Microseconds of each of `iters` launches (HIP events on the runner's stream), after `warmup` launches."""
+        out = (ctypes.c_double * iters)()
+        _check(_lib.dvm_rt_perf_samples(self._rt, warmup, iters, out))
+        return [out[i] for i in range(iters)]
 
     def num_launches(self):
         return _lib.dvm_rt_num_launches(self._rt)

@@ -1,6 +1,7 @@
 // Flat C ABI + runner over dvm::Kernel (see include/dvm_c.h).
 #include "../../../include/dvm_c.h"
 
+#include <algorithm>
 #include <chrono>
 #include <cstring>
 #include <map>
@@ -715,42 +716,64 @@ void *dvm_rt_device_ptr(dvm_rt *rt, dvm_obj *io) {
   return it == rt->buffers.end() ? nullptr : it->second.ptr;
 }
 
+namespace {
+// warmup launches, then `iters` launches each bracketed by a pair of events on the runner's stream: microseconds per launch
+std::vector<double> TimedLaunches(dvm_rt *rt, int warmup, int iters) {
+  const DeviceApi &api = rt->Api();
+  for (int i = 0; i < warmup; ++i) {
+    int rc = rt->kernel.Launch(rt->stream);
+    if (rc != 0) throw std::runtime_error(std::string("launch failed: ") + api.error_string(rc));
+  }
+  api.synchronize_stream(rt->stream);
+  std::vector<void *> ev(2 * static_cast<size_t>(iters), nullptr);
+  for (auto &e : ev) api.create_event(&e);
+  int rc = 0;
+  for (int i = 0; i < iters && rc == 0; ++i) {
+    api.record_event(ev[2 * i], rt->stream);
+    rc = rt->kernel.Launch(rt->stream);
+    api.record_event(ev[2 * i + 1], rt->stream);
+  }
+  const int rs = api.synchronize_stream(rt->stream);
+  std::vector<double> us(static_cast<size_t>(iters), 0.0);
+  for (int i = 0; i < iters && rc == 0 && rs == 0; ++i) {
+    float ms = 0.0f;
+    api.event_elapsed_time(&ms, ev[2 * i], ev[2 * i + 1]);
+    us[i] = ms * 1000.0;
+  }
+  for (auto &e : ev) api.destroy_event(e);
+  if (rc != 0) throw std::runtime_error(std::string("launch failed: ") + api.error_string(rc));
+  if (rs != 0) throw std::runtime_error(std::string("kernel execution failed: ") + api.error_string(rs));
+  return us;
+}
+}  // namespace
+
 int dvm_rt_perf(dvm_rt *rt, int warmup, int iters, double out[3]) {
   return Guard(
       [&]() {
-        if (rt->das_mode) {
-          out[0] = out[1] = out[2] = 0.0;
-          return 0;
-        }
-        const DeviceApi &api = rt->Api();
-        for (int i = 0; i < warmup; ++i) {
-          int rc = rt->kernel.Launch(rt->stream);
-          if (rc != 0) throw std::runtime_error(std::string("launch failed: ") + api.error_string(rc));
-        }
-        api.synchronize_stream(rt->stream);
-        std::vector<void *> ev(2 * static_cast<size_t>(iters), nullptr);
-        for (auto &e : ev) api.create_event(&e);
-        for (int i = 0; i < iters; ++i) {
-          api.record_event(ev[2 * i], rt->stream);
-          int rc = rt->kernel.Launch(rt->stream);
-          api.record_event(ev[2 * i + 1], rt->stream);
-          if (rc != 0) throw std::runtime_error(std::string("launch failed: ") + api.error_string(rc));
-        }
-        int rc = api.synchronize_stream(rt->stream);
-        if (rc != 0) throw std::runtime_error(std::string("kernel execution failed: ") + api.error_string(rc));
+        out[0] = out[1] = out[2] = 0.0;
+        if (rt->das_mode || iters <= 0) return 0;
+        const std::vector<double> us = TimedLaunches(rt, warmup, iters);
         double mn = 1e30, mx = 0.0, sum = 0.0;
-        for (int i = 0; i < iters; ++i) {
-          float ms = 0.0f;
-          api.event_elapsed_time(&ms, ev[2 * i], ev[2 * i + 1]);
-          const double us = ms * 1000.0;
-          mn = std::min(mn, us);
-          mx = std::max(mx, us);
-          sum += us;
+        for (double v : us) {
+          mn = std::min(mn, v);
+          mx = std::max(mx, v);
+          sum += v;
         }
-        for (auto &e : ev) api.destroy_event(e);
         out[0] = mn;
         out[1] = mx;
-        out[2] = iters > 0 ? sum / iters : 0.0;
+        out[2] = sum / iters;
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_perf_samples(dvm_rt *rt, int warmup, int iters, double *samples) {
+  return Guard(
+      [&]() {
+        for (int i = 0; i < iters; ++i) samples[i] = 0.0;
+        if (rt->das_mode || iters <= 0) return 0;
+        const std::vector<double> us = TimedLaunches(rt, warmup, iters);
+        for (int i = 0; i < iters; ++i) samples[i] = us[i];
         return 0;
       },
       -1);

@@ -117,6 +117,8 @@ int dvm_rt_output(dvm_rt *rt, dvm_obj *store, void *host, size_t bytes);
 void *dvm_rt_device_ptr(dvm_rt *rt, dvm_obj *io);
 /* warmup + iters timed launches with events: out = {min, max, mean} microseconds (src/pybind_api.cc:751-767). */
 int dvm_rt_perf(dvm_rt *rt, int warmup, int iters, double out[3]);
+/* The same measurement, every launch's microseconds written to samples[0..iters) (for medians). */
+int dvm_rt_perf_samples(dvm_rt *rt, int warmup, int iters, double *samples);
 /* Number of device launches one run() issues. */
 int dvm_rt_num_launches(const dvm_rt *rt);
 size_t dvm_rt_workspace_bytes(const dvm_rt *rt);

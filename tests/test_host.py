@@ -515,3 +515,13 @@ def test_values_of_earlier_sections_keep_their_registers_through_a_sweep():
     for l in sweep2:
         if l.startswith("mov v"):
             assert l.split()[1].rstrip(",") not in held, t.das()
+
+
+def test_traffic_summary_was_measured_on_the_current_schedule_sources():
+    """bench.py reports roofline.traffic from profiles/vec_rx_batchnorm_hbm_traffic.txt; the summary records a hash
+    of the sources that decide the headline kernel's schedule. A change to any of them without a new counter run
+    would leave a stale figure in the bench line: this fails until the summary is measured again."""
+    import bench
+    traffic, source = bench.headline_traffic()
+    assert traffic is not None and traffic > 205522944, source
+    assert "measured on these sources" in source, source
