@@ -5,16 +5,15 @@
 // accumulation, one rounding to the operand type on write-out) plus the mix kernel's post-fusion
 // vector program (src/xkernel.cc:304-360). The reference's CUDA backend has no matmul at all
 // (src/system.cc:290-294); this kernel is specific to CDNA4:
-//  * v_mfma_f32_32x32x16 (bf16 / f16), 64-wide waves, 2 x 2 waves per workgroup, each wave owning a
+//  * v_mfma_f32_32x32x16 (bf16 / f16), 64-wide waves, WM x 2 waves per workgroup, each wave owning a
 //    (TM*32) x (TN*32) block of fp32 accumulators that stays in registers for the whole k loop;
-//  * operand tiles are staged through local memory with k contiguous: rows of 64 elements (128
-//    bytes, no padding) whose eight 16-byte chunks are XOR-swizzled by the row number, so that the
-//    fragment reads (32 consecutive rows, one chunk), the straight tile copies (one row, eight
-//    chunks) and the transposing copies (rows 8 apart, one chunk) are all free of bank conflicts;
-//  * operands whose k axis is strided in memory (B of an NN product, A of a TN product) are read
-//    along their contiguous axis and transposed in registers, 8x8 elements per lane, on the way in;
-//  * local memory is double buffered and fragments are double buffered in registers: the global
-//    loads of tile t+1 and the fragment reads of step s+1 are in flight while the MFMAs of step s run;
+//  * the 256x256 tile (four or eight waves) walks k in stages of 32 through a ring of four stage buffers in
+//    local memory, every operand layout a straight direct-to-LDS copy (global_load_lds_dwordx4), the k-strided
+//    ones read back through ds_read_b64_tr_b16 (tile_loop_ring below);
+//  * the 128x128 and 64x64 tiles stage 64 k at a time, double buffered, k contiguous in local memory: rows of
+//    128 bytes whose eight 16-byte chunks are XOR-swizzled by the row number; operands whose k axis is strided in
+//    memory (B of an NN product, A of a TN product) are transposed in registers there, 8x8 elements per lane;
+//  * fragments are double buffered in registers: the reads of step s+1 are in flight while the MFMAs of step s run;
 //  * the epilogue runs in two passes over half tiles: accumulators go to local memory once, row
 //    major, and come back as slabs of 8 consecutive columns per lane, so every memory operand of the
 //    epilogue and every store is a coalesced 128-bit access; the epilogue program is the vector
@@ -187,6 +186,234 @@ __device__ __attribute__((noinline)) void stage_generic(uint16_t *tile, uint64_t
     }
     tile[tile_off(row, kk >> 3) + (kk & 7u)] = v;
   }
+}
+
+// ---- the 256x256 tile on four waves: stages of 32 k, four of them in local memory ---------------------
+// A stage holds 256 rows x 32 k of each operand (16 KB + 16 KB); four stage buffers make a ring. While
+// stage s is multiplied, the direct loads of stages s+1 and s+2 are in flight and those of stage s+3 are
+// issued, a few at a time between the MFMAs, into the buffer stage s-1 has just left: every load has two
+// full stages (64 MFMAs per wave) to arrive before anyone waits for it, and the four waves never send
+// their loads in one burst. Both operand layouts are straight copies:
+//  * k contiguous in memory (A, or B of a product with trans_b): rows of 32 k = 64 bytes = four 16-byte
+//    chunks, chunk c of row r stored at chunk c ^ ((r>>1 ^ r>>3) & 3); a fragment is one ds_read_b128 per lane;
+//  * k strided (B, or A of a product with trans_a): the tile is stored as it lies in memory, 32 k rows of
+//    256 elements (512 bytes, 32 chunks), chunk c of k row kr stored at chunk c ^ kswz(kr & 3); a fragment is
+//    two ds_read_b64_tr_b16 per lane, which transpose 4 k x 16 rows inside each group of 16 lanes.
+// kswz = {0, 10, 4, 14}: the four k rows one transposing read touches land in four different 32-byte
+// columns of a 128-byte window, and the two 16-lane groups of a half-wave in different halves of 256 bytes.
+constexpr int SK = 32;                           // k extent of a stage
+constexpr uint32_t kStageOperand = 256 * SK;     // elements of one operand in a stage buffer
+constexpr uint32_t kStageBuf = 2 * kStageOperand;
+
+__device__ __forceinline__ uint32_t kc_swz(uint32_t row) { return ((row >> 1) ^ (row >> 3)) & 3u; }
+__device__ __forceinline__ uint32_t ks_swz(uint32_t krow) { return (((krow & 3u) + 4u * (krow & 1u)) << 1); }
+
+template <bool KC, int NTHR>
+struct StageLoad {
+  static constexpr int N = 1024 / NTHR;  // 16-byte chunks per lane: 256 rows x 64 bytes over the workgroup
+  uint32_t lane_off;  // byte offset of the lane's first chunk from the tile's origin
+  uint32_t step;      // byte distance between the lane's chunks
+
+  __device__ __forceinline__ void init(uint32_t ld, uint32_t tid) {
+    if constexpr (KC) {
+      // chunk position p = NTHR*i + tid: row p/4, physical chunk p%4 (NTHR/4 rows further do not change the swizzle)
+      const uint32_t row = tid >> 2;
+      lane_off = row * ld * 2u + (((tid & 3u) ^ kc_swz(row)) << 4);
+      step = (NTHR / 4u) * ld * 2u;
+    } else {
+      // chunk position p = NTHR*i + tid: k row p/32, physical chunk p%32
+      const uint32_t kr = tid >> 5;
+      lane_off = kr * ld * 2u + (((tid & 31u) ^ ks_swz(kr)) << 4);
+      step = (NTHR / 32u) * ld * 2u;
+    }
+  }
+  // origin: address of element (row0, k0) of the operand; dst: the operand's part of a stage buffer
+  template <int I>
+  __device__ __forceinline__ void issue(uint64_t origin, uint32_t wave_first, uint16_t *dst) const {
+    const DVM_GLOBAL char *src = reinterpret_cast<const DVM_GLOBAL char *>(origin) + (lane_off + static_cast<uint32_t>(I) * step);
+    __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(src),
+                                     (__attribute__((address_space(3))) void *)(dst + (static_cast<uint32_t>(I) * NTHR + wave_first) * 8u), 16, 0, 0);
+  }
+};
+
+// Fragment reads of one operand for one wave (r0: first of its rows). The reads are written as assembly:
+// behind a read the compiler knows about, it waits for every direct load in flight (it cannot tell that the
+// load writes another stage buffer), which would drain the ring; the price is that the loop waits for its
+// reads by hand (once per step, lgkmcnt(0), with the fragment registers as operands of the wait so that no
+// MFMA can move above it).
+__device__ __forceinline__ uint32_t lds_byte_address(const void *ptr) {
+  return static_cast<uint32_t>(reinterpret_cast<size_t>((__attribute__((address_space(3))) const char *)(ptr)));
+}
+
+template <bool KC>
+struct FragAddr {
+  uint32_t x[4];  // byte offsets inside the operand's part of a stage buffer
+
+  __device__ __forceinline__ void init(uint32_t r0, uint32_t lane) {
+    if constexpr (KC) {
+      // fragment f, step kk: row r0 + 32f + lane%32, chunk (2kk + lane/32) ^ swz(row); x[kk] for f = 0
+      const uint32_t j = lane & 31u, hh = lane >> 5;
+      const uint32_t sw = kc_swz(j);  // r0 (a multiple of 64) and 32f do not change it
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk) x[kk] = ((r0 + j) * SK + (((2u * kk + hh) ^ sw) << 3)) * 2u;
+      x[2] = x[3] = 0;
+    } else {
+      // fragment f, step kk, half w: the lane supplies k row 16kk + 8*(g>>1) + 4w + jj and the four elements
+      // r0 + 32f + 16*(g&1) + 4q .. +3, with g = lane/16, jj = (lane%16)/4, q = lane%4; x[f] for kk = w = 0
+      const uint32_t g = lane >> 4, jj = (lane & 15u) >> 2, q = lane & 3u;
+      const uint32_t kr = 8u * (g >> 1) + jj;
+      const uint32_t sw = ks_swz(jj);
+#pragma unroll
+      for (int f = 0; f < 4; ++f) {
+        const uint32_t chunk = (r0 >> 3) + 4u * f + 2u * (g & 1u) + (q >> 1);
+        x[f] = (kr * 256u + ((chunk ^ sw) << 3) + 4u * (q & 1u)) * 2u;
+      }
+    }
+  }
+  // base: byte address in local memory of the operand's part of the stage buffer
+  template <int F, int KK>
+  __device__ __forceinline__ vu4 read(uint32_t base) const {
+    if constexpr (KC) {
+      vu4 r;
+      asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(base + x[KK]), "n"(F * 32 * SK * 2));
+      return r;
+    } else {
+      vu2 lo, hi;
+      const uint32_t addr = base + x[F];
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(addr), "n"(KK * 16 * 512));
+      asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(addr), "n"(KK * 16 * 512 + 4 * 512));
+      return vu4{lo[0], lo[1], hi[0], hi[1]};
+    }
+  }
+};
+
+// The tile loop for WM x 2 waves (WM = 2: 128x128 accumulators per wave, one wave per SIMD; WM = 4: 64x128,
+// two per SIMD). a_org / b_org: address of element (m0, 0) of A and (n0, 0) of B; nks: stages (k / 32 >= 2).
+template <bool IS_BF16, bool A_KC, bool B_KC, int WM>
+__device__ __forceinline__ void tile_loop_ring(vf16 (&acc)[8 / WM][4], uint16_t *lds, uint64_t a_org, uint64_t b_org, uint32_t lda,
+                                               uint32_t ldb, uint32_t nks, uint32_t tid) {
+  constexpr int NTHR = WM * 128, TM = 8 / WM, TN = 4;
+  constexpr int NL = StageLoad<true, NTHR>::N;  // loads per lane, operand and stage
+  constexpr int BPG = TN / TM;                  // B fragments a group reads
+  static_assert(NL == TM && (NL == 2 || NL == 4), "one A or B load pair per group");
+  const uint32_t wave = tid >> 6, lane = tid & 63u;
+  const uint32_t wm = wave >> 1, wn = wave & 1u;
+  const uint32_t wave_first = uni(wave) * 64u;
+  StageLoad<A_KC, NTHR> la;
+  StageLoad<B_KC, NTHR> lb;
+  la.init(lda, tid);
+  lb.init(ldb, tid);
+  FragAddr<A_KC> fa;
+  FragAddr<B_KC> fb;
+  fa.init(wm * (TM * 32u), lane);
+  fb.init(wn * 128u, lane);
+  const uint64_t a_adv = (A_KC ? static_cast<uint64_t>(SK) : static_cast<uint64_t>(SK) * lda) * 2;
+  const uint64_t b_adv = (B_KC ? static_cast<uint64_t>(SK) : static_cast<uint64_t>(SK) * ldb) * 2;
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+
+  // group g of a stage (TM groups) sends 2 * NL / TM = two of the lane's loads: the first half of the groups
+  // A's, the second half B's
+  auto issue_pair = [&](uint32_t st, auto group) {
+    constexpr int G = decltype(group)::value;
+    uint16_t *buf = lds + (st & 3u) * kStageBuf;
+    if constexpr (2 * G < TM) {
+      const uint64_t ao = a_org + st * a_adv;
+      la.template issue<2 * G>(ao, wave_first, buf);
+      la.template issue<2 * G + 1>(ao, wave_first, buf);
+    } else {
+      const uint64_t bo = b_org + st * b_adv;
+      lb.template issue<2 * G - TM>(bo, wave_first, buf + kStageOperand);
+      lb.template issue<2 * G - TM + 1>(bo, wave_first, buf + kStageOperand);
+    }
+  };
+  vu4 af[2][TM], bf[2][TN];
+  const uint32_t lds_base = lds_byte_address(lds);
+  auto read_group = [&](auto fbuf, uint32_t st, auto kk, auto group) {  // the fragments group g is in charge of
+    constexpr int FB = decltype(fbuf)::value, KK = decltype(kk)::value, G = decltype(group)::value;
+    const uint32_t buf = lds_base + (st & 3u) * (kStageBuf * 2u);
+    af[FB][G] = fa.template read<G, KK>(buf);
+    bf[FB][BPG * G] = fb.template read<BPG * G, KK>(buf + kStageOperand * 2u);
+    if constexpr (BPG == 2) bf[FB][2 * G + 1] = fb.template read<2 * G + 1, KK>(buf + kStageOperand * 2u);
+  };
+  // every read issued so far has returned; the fragments of buffer fbuf may be used from here on
+  auto reads_done = [&](int fbuf) {
+    if constexpr (TM == 4) {
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(af[fbuf][0]), "+v"(af[fbuf][1]), "+v"(af[fbuf][2]), "+v"(af[fbuf][3]), "+v"(bf[fbuf][0]), "+v"(bf[fbuf][1]),
+                     "+v"(bf[fbuf][2]), "+v"(bf[fbuf][3]));
+    } else {
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(af[fbuf][0]), "+v"(af[fbuf][1]), "+v"(bf[fbuf][0]), "+v"(bf[fbuf][1]), "+v"(bf[fbuf][2]), "+v"(bf[fbuf][3]));
+    }
+  };
+  auto mfma_row = [&](int fbuf, int i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = mfma<IS_BF16>(af[fbuf][i], bf[fbuf][j], acc[i][j]);
+  };
+  // Waits until at most `stages` stages of this wave's loads are outstanding and all its local-memory reads have
+  // returned, then meets the other waves. One piece of assembly on purpose: behind __syncthreads() the compiler
+  // waits for every outstanding load (the direct loads write local memory), which would drain the ring.
+  auto meet = [](auto stages) {
+    constexpr int N = decltype(stages)::value * 2 * NL;
+    static_assert(N == 0 || N == 4 || N == 8 || N == 16, "vmcnt values spelled out below");
+    if constexpr (N == 16) asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else if constexpr (N == 8) asm volatile("s_waitcnt vmcnt(8) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else if constexpr (N == 4) asm volatile("s_waitcnt vmcnt(4) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  };
+  auto for_groups = [&](auto f) {
+    f(I0{});
+    f(I1{});
+    if constexpr (TM == 4) {
+      f(std::integral_constant<int, 2>{});
+      f(std::integral_constant<int, 3>{});
+    }
+  };
+
+  for_groups([&](auto g) { issue_pair(0, g); });
+  for_groups([&](auto g) { issue_pair(1, g); });
+  if (nks > 2) {
+    for_groups([&](auto g) { issue_pair(2, g); });
+    meet(std::integral_constant<int, 2>{});
+  } else {
+    meet(I1{});
+  }
+  for_groups([&](auto g) { read_group(I0{}, 0, I0{}, g); });
+
+  // One stage = two steps of 16 k, each TM groups of four MFMAs (one row of accumulator tiles). Group g of
+  // step 0 also reads its fragments of step 1 and sends two of the loads of stage st+3; step 1 first meets the
+  // other waves (stage st+1 has landed for everybody, and nobody reads stage st any more, whose buffer the
+  // loads issued after the next meeting overwrite), then its group g reads its fragments of stage st+1. The
+  // scheduler may not move anything across a group.
+  auto stage = [&](uint32_t st, auto loads, auto next) {
+    constexpr bool LOADS = decltype(loads)::value, NEXT = decltype(next)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    reads_done(0);
+    __builtin_amdgcn_sched_barrier(0);
+    for_groups([&](auto g) {
+      read_group(I1{}, st, I1{}, g);
+      if constexpr (LOADS) issue_pair(st + 3, g);
+      mfma_row(0, decltype(g)::value);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+    if constexpr (NEXT) {
+      if constexpr (LOADS) meet(std::integral_constant<int, 2>{});  // younger: the loads of stages st+2 and st+3
+      else meet(I0{});
+    }
+    reads_done(1);
+    __builtin_amdgcn_sched_barrier(0);
+    for_groups([&](auto g) {
+      if constexpr (NEXT) read_group(I0{}, st + 1, I0{}, g);
+      mfma_row(1, decltype(g)::value);
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  uint32_t st = 0;
+  for (; st + 3 < nks; ++st) stage(st, std::true_type{}, std::true_type{});
+  for (; st + 1 < nks; ++st) stage(st, std::false_type{}, std::true_type{});
+  stage(st, std::false_type{}, std::false_type{});
+  __syncthreads();
 }
 
 // ---- epilogue ---------------------------------------------------------------------------------------
@@ -464,6 +691,8 @@ __device__ __forceinline__ void apply_rnd(Slabs &a, uint32_t rnd) {
 
 struct EpiArgs {
   uint32_t mem_off, code_off, batch0, batch1;
+  uint32_t flags;   // VCubeHeader::epi_flags
+  uint32_t w0v, immv;  // per lane: the two words of instruction `lane` of the epilogue program (the first 64)
 };
 
 // Runs the epilogue program on SL slabs whose accumulator values are in `acc`.
@@ -477,8 +706,15 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
   uint32_t mask = 0;
   uint32_t pc = 0;
   while (true) {
-    const uint32_t w0 = uni(code32[2 * pc]);
-    const uint32_t imm = uni(code32[2 * pc + 1]);
+    // the program sits in two registers, one instruction per lane: no memory access to fetch one
+    uint32_t w0, imm;
+    if (pc < 64u) {
+      w0 = __builtin_amdgcn_readlane(h.w0v, pc);
+      imm = __builtin_amdgcn_readlane(h.immv, pc);
+    } else {
+      w0 = uni(code32[2 * pc]);
+      imm = uni(code32[2 * pc + 1]);
+    }
     ++pc;
     const uint32_t op = w0 & 0xffu;
     if (op == VOP_END) break;
@@ -515,6 +751,8 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
             case VB_MUL: acc = acc * src; break;
             case VB_DIV: acc = acc / src; break;
             case VB_RDIV: acc = src / acc; break;
+            case VB_DIV_APPROX: FOR_SE acc[q] = __fdividef(acc[q], src[q]); break;
+            case VB_RDIV_APPROX: FOR_SE acc[q] = __fdividef(src[q], acc[q]); break;
             case VB_MIN: FOR_SE acc[q] = acc[q] < src[q] ? acc[q] : src[q]; break;
             case VB_MAX: FOR_SE acc[q] = acc[q] > src[q] ? acc[q] : src[q]; break;
             case VB_AND: FOR_SE acc[q] = (acc[q] != 0.0f && src[q] != 0.0f) ? 1.0f : 0.0f; break;
@@ -577,9 +815,27 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
       case VOP_UN:
         switch (sub) {
           case VU_SQRT: acc = by_halves<SL>(acc, math_sqrt); break;
+          case VU_SQRT_APPROX: FOR_SE acc[q] = __builtin_amdgcn_sqrtf(acc[q]); break;
           case VU_ABS: FOR_SE acc[q] = fabsf(acc[q]); break;
           case VU_LOG: acc = by_halves<SL>(acc, math_log); break;
+          case VU_LOG_APPROX: FOR_SE acc[q] = __logf(acc[q]); break;
           case VU_EXP: acc = by_halves<SL>(acc, math_exp); break;
+          case VU_EXP_SCALED:  // the product is a value of its own: rounded to fp32, never contracted into what follows
+            FOR_SE {
+              float y = acc[q] * __uint_as_float(imm);
+              asm volatile("" : "+v"(y));
+              acc[q] = y;
+            }
+            acc = by_halves<SL>(acc, math_exp);
+            break;
+          case VU_EXP_APPROX: FOR_SE acc[q] = __expf(acc[q]); break;
+          case VU_EXP_SCALED_APPROX:
+            FOR_SE {
+              float y = acc[q] * __uint_as_float(imm);
+              asm volatile("" : "+v"(y));
+              acc[q] = __expf(y);
+            }
+            break;
           case VU_ISFINITE: FOR_SE acc[q] = isfinite(acc[q]) ? 1.0f : 0.0f; break;
           case VU_ROUND: FOR_SE acc[q] = rintf(acc[q]); break;
           case VU_FLOOR: FOR_SE acc[q] = floorf(acc[q]); break;
@@ -630,6 +886,12 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
   constexpr int HALF = ROWS / WM;  // local rows [i * HALF, (i + 1) * HALF) belong to the i-th row of waves
   const uint32_t col = n0 + g * 8;
   const uint32_t ncol = col >= n ? 0u : (n - col < 8u ? n - col : 8u);
+  {
+    const uint32_t *code32 = prog32 + 2 * ea.code_off;
+    const uint32_t li = (tid & 63u) < ea.w0v ? (tid & 63u) : 0u;  // w0v arrives holding the instruction count
+    ea.w0v = code32[2 * li];
+    ea.immv = code32[2 * li + 1];
+  }
   for (int it = 0; it < PER_THREAD / SL; ++it) {
     typename SlabVec<SL>::type acc;
     SlabRows rows;
@@ -727,7 +989,13 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
 #pragma unroll
       for (int j = 0; j < TN; ++j) acc[i][j] = 0.0f;
 
+    constexpr bool RING = BM == 256 && BN == 256;  // the ring of 32-deep stages
     if (h.fast && m0 + BM <= h.m && n0 + BN <= h.n) {
+     if constexpr (RING) {
+      const uint64_t a_org = a_base + (A_KC ? static_cast<uint64_t>(m0) * h.lda : static_cast<uint64_t>(m0)) * 2;
+      const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb : static_cast<uint64_t>(n0)) * 2;
+      tile_loop_ring<IS_BF16, A_KC, B_KC, WM>(acc, lds, a_org, b_org, h.lda, h.ldb, h.k / SK, tid);
+     } else {
       Stage<BM, A_KC, NTHR> sa;
       Stage<BN, B_KC, NTHR> sb;
       // address of element (row0, k) of each operand, k advancing by BK per step
@@ -869,6 +1137,7 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       }
       k_tile(kt, std::false_type{}, std::false_type{});
       __syncthreads();
+     }
     } else {
       for (uint32_t kt = 0; kt < nk; ++kt) {
         stage_generic<BM, NTHR>(lds, a_base, h.lda, m0, kt * BK, h.m, h.k, A_KC ? 1u : 0u, tid);
@@ -891,7 +1160,7 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
     }
 
     // epilogue: accumulators -> local memory (row major), then slabs through the program
-    const EpiArgs ea = {h.mem_off, h.code_off, bi0, bi1};
+    const EpiArgs ea = {h.mem_off, h.code_off, bi0, bi1, h.epi_flags, h.n_code, 0};
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
       constexpr int FR = TM / PASSES;  // fragment rows of a wave per pass

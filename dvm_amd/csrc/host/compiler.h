@@ -274,6 +274,7 @@ class Compiler {
 
   void CompileArea(int a);
   void CompileCube(int a);
+  uint32_t FuseCubeEpilogue();
   void CompileAttn(int g);
   void BuildNodes(int a);
   void UnifyAxes();

@@ -37,9 +37,9 @@ void PrintShape(std::ostringstream &os, const NDObject *o) {
 }
 
 const char *kMemTypes[] = {"bool", "fp16", "bf16", "fp32", "int32"};
-const char *kBinF[] = {"Add", "Sub", "RSub", "Mul", "Div", "RDiv", "Min", "Max", "And", "Or", "Pow", "RPow"};
+const char *kBinF[] = {"Add", "Sub", "RSub", "Mul", "Div", "RDiv", "Min", "Max", "And", "Or", "Pow", "RPow", "Div~", "RDiv~"};
 const char *kBinI[] = {"Add", "Sub", "RSub", "Mul", "Min", "Max"};
-const char *kUn[] = {"Sqrt", "Abs", "Log", "Exp", "IsFinite", "Round", "Floor", "Ceil", "Trunc", "Abs"};
+const char *kUn[] = {"Sqrt", "Abs", "Log", "Exp", "IsFinite", "Round", "Floor", "Ceil", "Trunc", "Abs", "Exp", "Exp~", "Exp~", "Log~", "Sqrt~"};
 const char *kCmp[] = {"Eq", "Ne", "Gt", "Ge", "Lt", "Le"};
 const char *kRnd[] = {"fp32", "fp16", "bf16", "?"};
 const char *kRed[] = {"sum", "max", "min"};
@@ -134,7 +134,13 @@ std::string &VKernel::DisAssemble() {
             os << "store." << kMemTypes[mem_dtype(VI_A(w))] << " m" << VI_A(w) << ", acc";
             if (static_cast<uint32_t>(w) & VI_ENDS) os << "  ; endsweep";
             break;
-          case VOP_UN: os << kUn[sub] << "." << (sub == VU_IABS ? "int32" : kRnd[VI_RND(w)]) << " acc"; break;
+          case VOP_UN:
+            if (sub == VU_EXP_SCALED || sub == VU_EXP_SCALED_APPROX) {
+              os << kUn[sub] << "." << kRnd[VI_RND(w)] << " acc * #0x" << std::hex << VI_IMM(w) << std::dec;
+              break;
+            }
+            os << kUn[sub] << "." << (sub == VU_IABS ? "int32" : kRnd[VI_RND(w)]) << " acc";
+            break;
           case VOP_CAST: {
             static const char *names[] = {"cast.f2i", "cast.i2f", "cast.round", "cast.f2b"};
             os << names[sub] << "." << kRnd[VI_RND(w)] << " acc";

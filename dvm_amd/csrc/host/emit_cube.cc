@@ -50,6 +50,78 @@ int Compiler::CubeMemIndex(int v) {
   return n.mem_idx;
 }
 
+// The epilogue interpreter pays a fixed price per instruction and walk (decode, a serial chain of a few hundred
+// cycles with one wave per SIMD), so pairs that one arm can compute are joined: a multiply by a constant followed
+// by Exp becomes VU_EXP_SCALED (exp(-x), exp(x * c)); the product is still rounded to fp32 on its own.
+// Then, when every store writes a 16-bit float and every operator is continuous in its inputs (no compare,
+// select, rounding to an integer, conversion to int32, so that an error of one fp32 ulp cannot flip a decision),
+// exp, log, sqrt and the divisions are replaced by their hardware approximations and the header says so.
+uint32_t Compiler::FuseCubeEpilogue() {
+  std::vector<uint64_t> &out = scratch_code_;
+  out.clear();
+  out.reserve(code_.size());
+  for (size_t i = 0; i < code_.size(); ++i) {
+    const uint64_t w = code_[i];
+    if (i + 1 < code_.size() && VI_OP(w) == VOP_BINF && VI_SUB(w) == VB_MUL && VI_KIND(w) == VK_IMM && VI_RND(w) == 0) {
+      const uint64_t nx = code_[i + 1];
+      if (VI_OP(nx) == VOP_UN && VI_SUB(nx) == VU_EXP) {
+        out.push_back(VI_MAKE(VOP_UN, VU_EXP_SCALED, 0, VI_RND(nx), 0, VI_IMM(w)));
+        ++i;
+        continue;
+      }
+    }
+    out.push_back(w);
+  }
+  code_.swap(out);
+  if (k_->tuning_.cube_exact == 1) return 0;
+  bool any = false;
+  for (uint64_t w : code_) {
+    switch (VI_OP(w)) {
+      case VOP_END:
+      case VOP_LD:
+      case VOP_LDR:
+      case VOP_LDI:
+      case VOP_STR:
+        break;
+      case VOP_ST: {
+        const uint32_t dt = cmems_[VI_A(w)].dtype;
+        if (dt != VDT_F16 && dt != VDT_BF16) return 0;
+        break;
+      }
+      case VOP_CAST:
+        if (VI_SUB(w) != VC_RND) return 0;
+        break;
+      case VOP_UN: {
+        const uint32_t u = VI_SUB(w);
+        if (u != VU_SQRT && u != VU_ABS && u != VU_LOG && u != VU_EXP && u != VU_EXP_SCALED) return 0;
+        if (u != VU_ABS) any = true;
+        break;
+      }
+      case VOP_BINF: {
+        const uint32_t b = VI_SUB(w);
+        if (b != VB_ADD && b != VB_SUB && b != VB_RSUB && b != VB_MUL && b != VB_DIV && b != VB_RDIV && b != VB_MIN && b != VB_MAX) return 0;
+        if (b == VB_DIV || b == VB_RDIV) any = true;
+        break;
+      }
+      default:
+        return 0;
+    }
+  }
+  if (!any) return 0;
+  for (uint64_t &w : code_) {
+    uint32_t sub = VI_SUB(w);
+    if (VI_OP(w) == VOP_UN) {
+      sub = sub == VU_EXP ? VU_EXP_APPROX : sub == VU_EXP_SCALED ? VU_EXP_SCALED_APPROX : sub == VU_LOG ? VU_LOG_APPROX : sub == VU_SQRT ? VU_SQRT_APPROX : sub;
+    } else if (VI_OP(w) == VOP_BINF) {
+      sub = sub == VB_DIV ? VB_DIV_APPROX : sub == VB_RDIV ? VB_RDIV_APPROX : sub;
+    } else {
+      continue;
+    }
+    w = (w & ~0xff00ull) | (static_cast<uint64_t>(sub) << 8);
+  }
+  return VCF_APPROX_MATH;
+}
+
 void Compiler::CompileCube(int a) {
   cube_mode_ = true;
   BuildNodes(a);
@@ -122,17 +194,12 @@ void Compiler::CompileCube(int a) {
       h.tile = v == 256 ? 0 : (v == 128 ? 1 : 2);
     }
   }
-  // The 256x256 tile also exists on eight waves (two per SIMD, 64x128 accumulators each): the second wave hides
-  // most of the epilogue and of the fragment-read latency, at 1.5 times the local-memory traffic per flop.
-  // Measured on MI355X, 8192x4096x4096 bf16: both operands k-contiguous 289 -> 283 us (with bias + SiLU
-  // 369 -> 354 us, k = 512: 81 -> 70 us); with a k-strided operand, whose tiles pass through registers, the four
-  // waves stay ahead (286 us against 324 us). DVM_CUBE_WAVES=4 / 8 forces either.
-  if (h.tile == 0) {
-    bool eight = !h.trans_a && h.trans_b;
-    if (k_->tuning_.cube_waves == 8) eight = true;
-    if (k_->tuning_.cube_waves == 4) eight = false;
-    if (eight) h.tile = 3;
-  }
+  // The 256x256 tile runs on eight waves (two per SIMD, 64x128 accumulators each) unless DVM_CUBE_WAVES=4 asks for
+  // four (one per SIMD, 128x128): the second wave of a SIMD fills the stalls of the first in the prologue and in
+  // the interpreted epilogue. Measured on MI355X, bf16 8192x4096xk, row-major operands, four -> eight waves:
+  // k = 64: 60 -> 54 us (with bias + SiLU 106 -> 87 us), k = 512: 82 -> 76 us, k = 4096: 296-301 us either way for
+  // the plain product (the sustained rate is set by the power cap there), 338-342 -> 334-339 us with bias + SiLU.
+  if (h.tile == 0 && k_->tuning_.cube_waves != 4) h.tile = 3;
   h.tiles_m = static_cast<uint32_t>((M + bt - 1) / bt);
   h.tiles_n = static_cast<uint32_t>((N + bt - 1) / bt);
   if (tiles(bt) >= (1ull << 31)) Fail("too many matmul tiles");
@@ -198,6 +265,7 @@ void Compiler::CompileCube(int a) {
     for (int i = 0; i < n_mem_; ++i) dts[i] = cmems_[i].dtype;
     DropCastBeforeStore(dts);
   }
+  h.epi_flags = FuseCubeEpilogue();
   h.n_mem = n_mem_;
   h.n_code = static_cast<uint32_t>(code_.size());
   h.mem_off = sizeof(VCubeHeader) / 8;

@@ -172,6 +172,7 @@ struct Tuning {
   int vec_runs = -1;    // DVM_VEC_RUNS=1: per-output runs only when the team is the whole workgroup
   int cube_tile = -1;   // DVM_CUBE_TILE=256|128|64
   int cube_waves = -1;  // DVM_CUBE_WAVES=4|8
+  int cube_exact = -1;  // DVM_CUBE_EXACT=1: never the hardware approximations of exp, log, sqrt, division in a matmul epilogue
   int attn_waves = -1;  // DVM_ATTN_WAVES=4
   bool debug = false;   // DVM_DEBUG: node dump in compile errors
   void Read();

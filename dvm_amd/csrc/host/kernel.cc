@@ -25,6 +25,7 @@ void Tuning::Read() {
   vec_runs = num("DVM_VEC_RUNS");
   cube_tile = num("DVM_CUBE_TILE");
   cube_waves = num("DVM_CUBE_WAVES");
+  cube_exact = num("DVM_CUBE_EXACT");
   attn_waves = num("DVM_ATTN_WAVES");
   debug = std::getenv("DVM_DEBUG") != nullptr;
 }

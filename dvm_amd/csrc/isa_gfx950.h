@@ -97,12 +97,17 @@ enum { VF_F32 = 0, VF_F16 = 1, VF_BF16 = 2 };
 // float binary sub-ops (R* = operands reversed: src op acc)
 enum {
   VB_ADD = 0, VB_SUB, VB_RSUB, VB_MUL, VB_DIV, VB_RDIV, VB_MIN, VB_MAX, VB_AND, VB_OR, VB_POW, VB_RPOW,
+  VB_DIV_APPROX, VB_RDIV_APPROX,  // matmul epilogues only: acc * rcp(src), src * rcp(acc) with v_rcp_f32
 };
 // int32 binary sub-ops
 enum { VBI_ADD = 0, VBI_SUB, VBI_RSUB, VBI_MUL, VBI_MIN, VBI_MAX };
 // unary sub-ops
 enum {
   VU_SQRT = 0, VU_ABS, VU_LOG, VU_EXP, VU_ISFINITE, VU_ROUND, VU_FLOOR, VU_CEIL, VU_TRUNC, VU_IABS,
+  // matmul epilogues only. VU_EXP_SCALED: acc = exp(acc * imm), the product rounded to fp32 first (the fused form
+  // of a multiply by a constant followed by Exp). The _APPROX forms use the hardware approximations (v_exp_f32,
+  // v_log_f32, v_sqrt_f32: one ulp of fp32); the host picks them under VCF_APPROX_MATH.
+  VU_EXP_SCALED, VU_EXP_APPROX, VU_EXP_SCALED_APPROX, VU_LOG_APPROX, VU_SQRT_APPROX,
 };
 // compare sub-ops (same order as dvm::BinaryType kEqual..kLessEqual); +VCMP_INT for int32 operands
 enum { VCMP_EQ = 0, VCMP_NE, VCMP_GT, VCMP_GE, VCMP_LT, VCMP_LE, VCMP_INT = 8 };
@@ -231,9 +236,15 @@ typedef struct {
   uint32_t n_mem, n_code;
   uint32_t mem_off, code_off;  // word offsets
   uint32_t fast;       // k is a multiple of 64 and every 8-element operand chunk is 16-byte aligned: full tiles take the vector path
-  uint32_t pad;
+  uint32_t epi_flags;  // VCF_*
   uint64_t a_addr, b_addr;
 } VCubeHeader;
+
+// VCubeHeader::epi_flags
+// Every store of the epilogue writes fp16 or bf16 and the program holds only operators that are continuous in
+// their inputs (no compare, select, rounding to integers, conversion to int32): the host has replaced exp, log,
+// sqrt and division by their _APPROX forms (one ulp of fp32; the 16-bit rounding is four orders coarser).
+#define VCF_APPROX_MATH 1u
 
 // Dynamic local memory a VE_CUBE launch needs for block tile `bt` (256, 128 or 64): the double-buffered
 // operand tiles of the k loop, or the half tile of fp32 accumulators the epilogue reads back.

@@ -152,3 +152,74 @@ def test_big_tile_on_four_and_on_eight_waves(monkeypatch, waves, dtype, ta, tb):
     want = (prod + bias) * other
     got = t.output(out).astype(np.float64)
     assert np.allclose(got, want, rtol=1e-2, atol=1e-2), float(np.abs(got - want).max())
+
+
+@pytest.mark.parametrize("exact", [False, True])
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16"])
+def test_epilogue_with_hardware_approximations(monkeypatch, exact, dtype):
+    # An epilogue whose stores are all 16-bit and whose operators are all continuous uses the hardware's exp, log,
+    # sqrt and reciprocal (one ulp of fp32); DVM_CUBE_EXACT=1 keeps the library routines. Both must sit within
+    # the 16-bit tolerance of the float64 closed form, and a multiply by a constant in front of Exp becomes one
+    # instruction with it.
+    if exact:
+        monkeypatch.setenv("DVM_CUBE_EXACT", "1")
+    m, n, k = 300, 520, 192
+    r = np.random.default_rng(21)
+    af, bf = (r.standard_normal([m, k]) / 8).astype(np.float32), (r.standard_normal([k, n]) / 8).astype(np.float32)
+    bias = r.standard_normal([n]).astype(np.float32)
+    t = Tester("mix")
+    if dtype == "bfloat16":
+        a16, b16 = Tester.convert_to_bf16(af), Tester.convert_to_bf16(bf)
+        a_ref, b_ref = Tester.convert_from_bf16(a16).astype(np.float64), Tester.convert_from_bf16(b16).astype(np.float64)
+        x, y = t.load(a16.shape, "bfloat16"), t.load(b16.shape, "bfloat16")
+        t.input(x, a16)
+        t.input(y, b16)
+        rnd = lambda v: Tester.convert_from_bf16(Tester.convert_to_bf16(v.astype(np.float32))).astype(np.float64)
+        eps = 1e-2
+    else:
+        a16, b16 = af.astype(np.float16), bf.astype(np.float16)
+        a_ref, b_ref = a16.astype(np.float64), b16.astype(np.float64)
+        x, y = t.load(a16), t.load(b16)
+        rnd = lambda v: v.astype(np.float16).astype(np.float64)
+        eps = 1e-3
+    h = t.add(t.cast(t.matmul(x, y, False, False), "float32"), t.load(bias))
+    silu = t.store(t.cast(t.div(h, t.add(t.exp(t.mul(h, -1.0)), 1.0)), dtype))
+    other = t.store(t.cast(t.div(t.log(t.add(t.sqrt(t.abs(h)), 1.5)), t.add(t.exp(h), 2.0)), dtype))
+    t.run()
+    das = t.das()
+    assert t.num_launches() == 1, das
+    assert ("Exp~" in das and "RDiv~" in das and "Log~" in das and "Sqrt~" in das) == (not exact), das
+    assert "acc * #0xbf800000" in das, das  # exp(-h) is one instruction
+    hh = rnd(a_ref @ b_ref) + bias
+    got = t.output(silu)
+    got = Tester.convert_from_bf16(got) if dtype == "bfloat16" else got.astype(np.float32)
+    assert np.allclose(got, hh / (1.0 + np.exp(-hh)), rtol=eps, atol=eps)
+    got = t.output(other)
+    got = Tester.convert_from_bf16(got) if dtype == "bfloat16" else got.astype(np.float32)
+    assert np.allclose(got, np.log(np.sqrt(np.abs(hh)) + 1.5) / (np.exp(hh) + 2.0), rtol=eps, atol=eps)
+
+
+def test_epilogue_with_an_fp32_store_or_a_decision_stays_exact():
+    m, n, k = 128, 256, 64
+    r = np.random.default_rng(22)
+    a16, b16 = (r.standard_normal([m, k]) / 8).astype(np.float16), (r.standard_normal([k, n]) / 8).astype(np.float16)
+    prod = a16.astype(np.float64) @ b16.astype(np.float64)
+    p16 = prod.astype(np.float16).astype(np.float64)
+    # an fp32 store next to the fp16 one
+    t = Tester("mix")
+    h = t.cast(t.matmul(t.load(a16), t.load(b16), False, False), "float32")
+    e = t.exp(h)
+    o16, o32 = t.store(t.cast(e, "float16")), t.store(e)
+    t.run()
+    assert "~" not in t.das(), t.das()
+    # the fp16 rounding of the product is the device's (fp32 accumulation): a few elements sit on the other side of a tie
+    d32 = np.abs(t.output(o32) - np.exp(p16))
+    assert np.mean(d32 > 1e-5 * (1 + np.exp(p16))) < 2e-3 and np.all(d32 < 1e-3)
+    assert np.allclose(t.output(o16).astype(np.float64), np.exp(p16), rtol=1e-3, atol=1e-3)
+    # a comparison on a value that went through exp
+    t = Tester("mix")
+    h = t.cast(t.matmul(t.load(a16), t.load(b16), False, False), "float32")
+    o = t.store(t.cast(t.select(t.greater(t.exp(h), 1.0), h, t.mul(h, 0.5)), "float16"))
+    t.run()
+    assert "~" not in t.das(), t.das()
+    assert np.allclose(t.output(o).astype(np.float64), np.where(np.exp(p16) > 1.0, p16, p16 * 0.5), rtol=1e-3, atol=1e-3)
