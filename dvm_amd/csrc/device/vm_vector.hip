@@ -306,6 +306,65 @@ __device__ __forceinline__ void mem_load_wide(const VMemDesc &m, const Offs &off
   }
 }
 
+// Two operands that walk memory identically (same element offsets), both on the wide path: every load of both is
+// issued before anything is used, so the pair costs one trip to memory instead of two.
+__device__ __forceinline__ void mem_load2_wide(const VMemDesc &m, const VMemDesc &mb, const Offs &off, uint32_t full, Acc &x, Acc &y) {
+  if (m.dtype == VDT_BF16 && mb.dtype == VDT_BF16) {
+    vu4 a[U], b[U];
+    FOR_U {
+      a[u] = 0u;
+      b[u] = 0u;
+      if ((full >> u) & 1u) {
+        a[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(m.addr + off.v[u] * 2);
+        b[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(mb.addr + off.v[u] * 2);
+      }
+    }
+    FOR_U {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        x.v[u][2 * i] = __uint_as_float(a[u][i] << 16);
+        x.v[u][2 * i + 1] = __uint_as_float(a[u][i] & 0xffff0000u);
+        y.v[u][2 * i] = __uint_as_float(b[u][i] << 16);
+        y.v[u][2 * i + 1] = __uint_as_float(b[u][i] & 0xffff0000u);
+      }
+    }
+  } else if (m.dtype == VDT_F16 && mb.dtype == VDT_F16) {
+    vh8 a[U], b[U];
+    FOR_U {
+      a[u] = static_cast<_Float16>(0.0f);
+      b[u] = static_cast<_Float16>(0.0f);
+      if ((full >> u) & 1u) {
+        a[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off.v[u] * 2);
+        b[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(mb.addr + off.v[u] * 2);
+      }
+    }
+    FOR_U {
+      x.v[u] = __builtin_convertvector(a[u], vf8);
+      y.v[u] = __builtin_convertvector(b[u], vf8);
+    }
+  } else if ((m.dtype == VDT_F32 || m.dtype == VDT_I32) && (mb.dtype == VDT_F32 || mb.dtype == VDT_I32)) {
+    vf4 a0[U], a1[U], b0[U], b1[U];
+    FOR_U {
+      a0[u] = a1[u] = b0[u] = b1[u] = 0.0f;
+      if ((full >> u) & 1u) {
+        const DVM_GLOBAL vf4 *pa = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off.v[u] * 4);
+        const DVM_GLOBAL vf4 *pb = reinterpret_cast<const DVM_GLOBAL vf4 *>(mb.addr + off.v[u] * 4);
+        a0[u] = pa[0];
+        a1[u] = pa[1];
+        b0[u] = pb[0];
+        b1[u] = pb[1];
+      }
+    }
+    FOR_U {
+      x.v[u] = __builtin_shufflevector(a0[u], a1[u], 0, 1, 2, 3, 4, 5, 6, 7);
+      y.v[u] = __builtin_shufflevector(b0[u], b1[u], 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  } else {  // operands of different widths: one after the other
+    mem_load_wide(m, off, full, x);
+    mem_load_wide(mb, off, full, y);
+  }
+}
+
 __device__ __forceinline__ void mem_store_wide(const VMemDesc &m, const Offs &off, uint32_t full, const Acc &in) {
   const uint32_t dtype = m.dtype;
   FOR_U {
@@ -892,17 +951,39 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     uint32_t pc = 0;
     vu2 fetched = code64[0];
     while (true) {
-      const uint32_t w0 = uni(fetched[0]);
+      uint32_t w0 = uni(fetched[0]);
       const uint32_t imm = uni(fetched[1]);
-      const uint32_t op = w0 & 0x7fu;
+      uint32_t op = w0 & 0x7fu;
       if (op == VOP_END) break;
-      const uint32_t sub = (w0 >> 8) & 0xffu, a = w0 >> 24;
+      uint32_t sub = (w0 >> 8) & 0xffu;  // (w0, op and sub change when a load takes the instruction behind it along)
+      const uint32_t a = w0 >> 24;
       // branch-free: the round-closing bit and, for the waves that skip per-team runs, the jump to their end
       const bool ends = SCHED != VS_POINTWISE && (w0 & VI_ENDS) != 0;
       const uint32_t back = (ends ? 1u : 0u) & (round + 1 < n_rounds ? 1u : 0u);
       pc = back ? sweep_pc : pc + 1;
       pc += ((op == VOP_UNI_BEGIN ? 1u : 0u) & skips_runs) * (imm - 1u);
       fetched = code64[pc];
+      // VOP_LD flagged VI_LD_PAIR: the next instruction is a float binary whose memory operand has the load's
+      // element offsets. When both take the wide path the load fetches both operands in one trip to memory and
+      // the binary is finished in the same dispatch (true: src holds its operand; w0, op, sub are the binary's).
+      auto take_next_along = [&](const VMemDesc &m, const Offs &off, const Slabs &s2, Acc &x, Acc &y) -> bool {
+        constexpr uint32_t kFast = VMF_VEC | VMF_ALIGNED;
+        if ((w0 & VI_LD_PAIR) != 0 && (m.flags & kFast) == kFast && s2.uniform) {
+          const uint32_t wb = uni(fetched[0]);
+          const VMemDesc mb = load_desc(prog32, mem_off, wb >> 24);
+          if ((mb.flags & kFast) == kFast) {
+            mem_load2_wide(m, mb, off, s2.full, x, y);
+            w0 = wb;
+            op = wb & 0x7fu;
+            sub = (wb >> 8) & 0xffu;
+            ++pc;
+            fetched = code64[pc];
+            return true;
+          }
+        }
+        mem_load(m, off, s2, x);
+        return false;
+      };
 
       // ---- a run of per-output arithmetic (VOP_UNI_BEGIN .. VOP_UNI_END): every instruction in it works on one
       // value per lane, so the run has a small loop of its own: one float instead of the accumulator's U*E, a
@@ -1076,19 +1157,22 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                 }
                 continue;
               }
-              mem_load(m, off, sl, acc);
-              if (parked && (w0 & VI_LD_KEEP_WR)) {
+              const bool keep = parked && (w0 & VI_LD_KEEP_WR) != 0;
+              const bool pair = take_next_along(m, off, sl, acc, src);
+              if (keep) {
                 FOR_U {
                   keep_lds[((lr * U + u) * 2u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 0, 1, 2, 3);
                   keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 4, 5, 6, 7);
                 }
               }
-              continue;
+              if (!pair) continue;
+            } else {
+              if (!take_next_along(m, off, sl, acc, src)) continue;
             }
-            mem_load(m, off, sl, acc);
-            continue;
+            // the binary instruction behind the load: its operand is in src, the switch below finishes it
+          } else {
+            mem_load(m, off, sl, src);
           }
-          mem_load(m, off, sl, src);
         } else if (kind == VK_SREG) {
           const float v = sreg_read(sr, a);
           FOR_U src.v[u] = v;

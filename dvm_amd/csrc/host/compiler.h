@@ -310,6 +310,7 @@ class Compiler {
   void DropCastBeforeStore(const uint32_t *mem_dtypes);
   void FuseSweepInstructions();
   void MarkUniformRuns();
+  void PairLoads();
   void PlanRereads();
   bool mem_is_view_[DVM_VEC_MAXMEM] = {false};  // memory operand i is a strided view
   int last_mem_ = -1;         // memory operand of the last memory instruction emitted in this round, or -1

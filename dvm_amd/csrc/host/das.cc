@@ -161,6 +161,7 @@ std::string &VKernel::DisAssemble() {
             os << "load." << kMemTypes[mem_dtype(VI_A(w))] << " acc, m" << VI_A(w);
             if (static_cast<uint32_t>(w) & VI_LD_KEEP_WR) os << "  ; parks its first " << (VI_IMM(w) & 0xffffu) << " rounds in local memory";
             if (static_cast<uint32_t>(w) & VI_LD_KEEP_RD) os << "  ; takes its first " << (VI_IMM(w) & 0xffffu) << " rounds from local memory";
+            if (static_cast<uint32_t>(w) & VI_LD_PAIR) os << "  ; fetches the next instruction's operand in the same trip";
             break;
           case VOP_BINF:
             if (VI_KIND(w) == VK_SREG2) {  // two chained operations

@@ -652,6 +652,7 @@ void Compiler::FinishProgram() {
   static const bool unirun = !(std::getenv("DVM_VEC_UNIRUN") != nullptr && std::getenv("DVM_VEC_UNIRUN")[0] == '0');
   if (fuse && (hdr_.sched & VS_KIND_MASK) != VS_POINTWISE) FuseSweepInstructions();
   if (unirun) MarkUniformRuns();
+  if (k_->tuning_.vec_pair != 0) PairLoads();
   hdr_.n_mem = n_mem_;
   hdr_.n_code = static_cast<uint32_t>(code_.size());
   hdr_.mem_off = sizeof(VVecHeader) / 8;

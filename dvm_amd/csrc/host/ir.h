@@ -170,6 +170,7 @@ struct Tuning {
   int vec_wide = -1;    // DVM_VEC_WIDE=1: four slabs per lane in the vector VM
   int vec_team = -1;    // DVM_VEC_TEAM=n: at most n lanes per output in reduces along the innermost axis
   int vec_runs = -1;    // DVM_VEC_RUNS=1: per-output runs only when the team is the whole workgroup
+  int vec_pair = -1;   // DVM_VEC_PAIR=0: a load never takes the binary instruction behind it along
   int cube_tile = -1;   // DVM_CUBE_TILE=256|128|64
   int cube_waves = -1;  // DVM_CUBE_WAVES=4|8
   int cube_exact = -1;  // DVM_CUBE_EXACT=1: never the hardware approximations of exp, log, sqrt, division in a matmul epilogue

@@ -23,6 +23,7 @@ void Tuning::Read() {
   vec_wide = num("DVM_VEC_WIDE");
   vec_team = num("DVM_VEC_TEAM");
   vec_runs = num("DVM_VEC_RUNS");
+  vec_pair = num("DVM_VEC_PAIR");
   cube_tile = num("DVM_CUBE_TILE");
   cube_waves = num("DVM_CUBE_WAVES");
   cube_exact = num("DVM_CUBE_EXACT");

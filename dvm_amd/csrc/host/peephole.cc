@@ -34,6 +34,22 @@ void Compiler::DropCastBeforeStore(const uint32_t *mem_dtypes) {
   code_.swap(out);
 }
 
+// A load followed by a float binary whose memory operand walks memory identically (x + residual, x * mask): the
+// load is told that it may take the binary along. The device then has both operands in flight together, one trip
+// to memory for the pair instead of two in a row, which is what a wave with little else in flight waits for.
+void Compiler::PairLoads() {
+  bool in_run = false;
+  for (size_t i = 0; i + 1 < code_.size(); ++i) {
+    const uint64_t w = code_[i], nx = code_[i + 1];
+    if (VI_OP(w) == VOP_UNI_BEGIN) in_run = true;
+    if (VI_OP(w) == VOP_UNI_END) in_run = false;
+    if (in_run || VI_OP(w) != VOP_LD || (static_cast<uint32_t>(w) & VI_UNIFORM)) continue;
+    if (VI_OP(nx) != VOP_BINF || VI_KIND(nx) != VK_MEM) continue;
+    if (!(static_cast<uint32_t>(nx) & VI_SAME_OFFS) || (static_cast<uint32_t>(nx) & (VI_UNIFORM | VI_ENDS))) continue;
+    code_[i] = w | VI_LD_PAIR;
+  }
+}
+
 // The interpreter pays a fixed price per instruction, so the short bodies of sweeps are tightened:
 //  * sum(x) and sum(x * x) of one value (mean and variance in one pass): the multiply joins the second reduce;
 //  * two float binaries in a row with S-register operands (x * scale + shift) become one chained instruction;

@@ -140,6 +140,10 @@ enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 #define VI_LD_KEEP_WR (1u << 20)
 #define VI_LD_KEEP_RD (1u << 21)
 #define VSW_REVERSE 1u
+// VI_LD_PAIR (lowest bit of VOP_LD's sub field, vector VM): the next instruction is a VOP_BINF whose operand is a
+// memory operand with VI_SAME_OFFS. The load may fetch both operands at once (one trip to memory for the pair)
+// and finish the binary in the same dispatch; an interpreter that ignores the flag computes the same.
+#define VI_LD_PAIR (1u << 8)
 // VI_ENDS (top bit of the opcode byte; set on every VOP_ENDSWEEP, and on a store or reduce that took over the
 // VOP_ENDSWEEP behind it): the instruction closes the round of its sweep. One bit, so that the decoder finds the
 // next pc without comparing opcodes.
