@@ -84,7 +84,30 @@ def build(force=False, verbose=False):
         _run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC"] + dev_objs + ["-o", hip_so])
     if force or _stale(host_so, host_objs):
         _run(["g++", "-shared", "-fPIC"] + host_objs + ["-o", host_so, "-ldl", "-lpthread"])
+    build_consumer_tests(force)
     return hip_so, host_so
+
+
+CONSUMER_TESTS = {"muladd": ["-ldvm", "-ldvm_hip"], "device_blob": ["-ldvm_hip"]}
+
+
+def consumer_test_command(name):
+    """g++ line for tests/cc/<name>.cc: a program outside the package that sees only include/*.h (and the bytecode
+    header, for the blob test) and links the built libraries."""
+    repo = os.path.dirname(ROOT)
+    src = os.path.join(repo, "tests", "cc", name + ".cc")
+    out = os.path.join(LIB, "tests", name)
+    rocm_lib = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "lib")
+    return src, out, (["g++", "-std=c++17", "-O1", "-Wall", "-I" + os.path.join(repo, "include"), "-I" + CSRC, src, "-o", out,
+                       "-L" + LIB] + CONSUMER_TESTS[name] + ["-Wl,-rpath,$ORIGIN/..", "-Wl,-rpath-link," + rocm_lib])
+
+
+def build_consumer_tests(force=False):
+    os.makedirs(os.path.join(LIB, "tests"), exist_ok=True)
+    for name in CONSUMER_TESTS:
+        src, out, cmd = consumer_test_command(name)
+        if os.path.exists(src) and (force or _stale(out, [src, os.path.join(LIB, "libdvm.so"), os.path.join(LIB, "libdvm_hip.so")] + _deps())):
+            _run(cmd)
 
 
 if __name__ == "__main__":
