@@ -195,7 +195,8 @@ __device__ __attribute__((noinline)) void stage_generic(uint16_t *tile, uint64_t
 // full stages (64 MFMAs per wave) to arrive before anyone waits for it, and the four waves never send
 // their loads in one burst. Both operand layouts are straight copies:
 //  * k contiguous in memory (A, or B of a product with trans_b): rows of 32 k = 64 bytes = four 16-byte
-//    chunks, chunk c of row r stored at chunk c ^ ((r>>1 ^ r>>3) & 3); a fragment is one ds_read_b128 per lane;
+//    chunks, chunk c of row r stored at chunk c ^ ((r >> 2) & 3): the 16 rows that one quarter of a fragment read
+//    touches (16 lanes x 16 bytes = all 64 banks once) then sit in 16 different bank groups; one ds_read_b128 per lane;
 //  * k strided (B, or A of a product with trans_a): the tile is stored as it lies in memory, 32 k rows of
 //    256 elements (512 bytes, 32 chunks), chunk c of k row kr stored at chunk c ^ kswz(kr & 3); a fragment is
 //    two ds_read_b64_tr_b16 per lane, which transpose 4 k x 16 rows inside each group of 16 lanes.
@@ -205,7 +206,7 @@ constexpr int SK = 32;                           // k extent of a stage
 constexpr uint32_t kStageOperand = 256 * SK;     // elements of one operand in a stage buffer
 constexpr uint32_t kStageBuf = 2 * kStageOperand;
 
-__device__ __forceinline__ uint32_t kc_swz(uint32_t row) { return ((row >> 1) ^ (row >> 3)) & 3u; }
+__device__ __forceinline__ uint32_t kc_swz(uint32_t row) { return (row >> 2) & 3u; }
 __device__ __forceinline__ uint32_t ks_swz(uint32_t krow) { return (((krow & 3u) + 4u * (krow & 1u)) << 1); }
 
 template <bool KC, int NTHR>
@@ -216,7 +217,7 @@ struct StageLoad {
 
   __device__ __forceinline__ void init(uint32_t ld, uint32_t tid) {
     if constexpr (KC) {
-      // chunk position p = NTHR*i + tid: row p/4, physical chunk p%4 (NTHR/4 rows further do not change the swizzle)
+      // chunk position p = NTHR*i + tid: row p/4, physical chunk p%4 (NTHR/4 = 64 or 128 rows further do not change the swizzle)
       const uint32_t row = tid >> 2;
       lane_off = row * ld * 2u + (((tid & 3u) ^ kc_swz(row)) << 4);
       step = (NTHR / 4u) * ld * 2u;

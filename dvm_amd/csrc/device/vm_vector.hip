@@ -365,6 +365,64 @@ __device__ __forceinline__ void mem_load2_wide(const VMemDesc &m, const VMemDesc
   }
 }
 
+// One operand at the element offsets of two rounds, both on the wide path: again every load is issued before
+// anything is used.
+__device__ __forceinline__ void mem_load_wide_2rounds(const VMemDesc &m, const Offs &off, const Offs &off2, uint32_t full, uint32_t full2,
+                                                      Acc &x, Acc &y) {
+  if (m.dtype == VDT_F32 || m.dtype == VDT_I32) {
+    vf4 a0[U], a1[U], b0[U], b1[U];
+    FOR_U {
+      a0[u] = a1[u] = b0[u] = b1[u] = 0.0f;
+      if ((full >> u) & 1u) {
+        const DVM_GLOBAL vf4 *pa = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off.v[u] * 4);
+        a0[u] = pa[0];
+        a1[u] = pa[1];
+      }
+      if ((full2 >> u) & 1u) {
+        const DVM_GLOBAL vf4 *pb = reinterpret_cast<const DVM_GLOBAL vf4 *>(m.addr + off2.v[u] * 4);
+        b0[u] = pb[0];
+        b1[u] = pb[1];
+      }
+    }
+    FOR_U {
+      x.v[u] = __builtin_shufflevector(a0[u], a1[u], 0, 1, 2, 3, 4, 5, 6, 7);
+      y.v[u] = __builtin_shufflevector(b0[u], b1[u], 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  } else if (m.dtype == VDT_BF16) {
+    vu4 a[U], b[U];
+    FOR_U {
+      a[u] = 0u;
+      b[u] = 0u;
+      if ((full >> u) & 1u) a[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(m.addr + off.v[u] * 2);
+      if ((full2 >> u) & 1u) b[u] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(m.addr + off2.v[u] * 2);
+    }
+    FOR_U {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        x.v[u][2 * i] = __uint_as_float(a[u][i] << 16);
+        x.v[u][2 * i + 1] = __uint_as_float(a[u][i] & 0xffff0000u);
+        y.v[u][2 * i] = __uint_as_float(b[u][i] << 16);
+        y.v[u][2 * i + 1] = __uint_as_float(b[u][i] & 0xffff0000u);
+      }
+    }
+  } else if (m.dtype == VDT_F16) {
+    vh8 a[U], b[U];
+    FOR_U {
+      a[u] = static_cast<_Float16>(0.0f);
+      b[u] = static_cast<_Float16>(0.0f);
+      if ((full >> u) & 1u) a[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off.v[u] * 2);
+      if ((full2 >> u) & 1u) b[u] = *reinterpret_cast<const DVM_GLOBAL vh8 *>(m.addr + off2.v[u] * 2);
+    }
+    FOR_U {
+      x.v[u] = __builtin_convertvector(a[u], vf8);
+      y.v[u] = __builtin_convertvector(b[u], vf8);
+    }
+  } else {
+    mem_load_wide(m, off, full, x);
+    mem_load_wide(m, off2, full2, y);
+  }
+}
+
 __device__ __forceinline__ void mem_store_wide(const VMemDesc &m, const Offs &off, uint32_t full, const Acc &in) {
   const uint32_t dtype = m.dtype;
   FOR_U {
@@ -963,6 +1021,46 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       pc = back ? sweep_pc : pc + 1;
       pc += ((op == VOP_UNI_BEGIN ? 1u : 0u) & skips_runs) * (imm - 1u);
       fetched = code64[pc];
+      auto end_round = [&](bool round_done, bool recount) {
+        if constexpr (SCHED != VS_POINTWISE) {
+          // end of a round: the next one (the decode above has already turned the pc back), or the end of
+          // the sweep, where the slots' partials are combined across lanes
+          if (round_done) {
+            ++round;
+            if (round < n_rounds) {
+              ridx = sweep_rev ? ridx - r_step * U : ridx + r_step * U;
+            } else {
+              in_sweep = false;
+              const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
+              if constexpr (SCHED == VS_REDX) {
+                if (k0 <= VR_MIN || k1 <= VR_MIN) {
+                  red_finish_x(racc0.v[0], racc1.v[0], k0, k1, tlog, team_is_block, tid, nthreads, red_flip, lds);
+                }
+              } else {
+                if (k0 <= VR_MIN) racc0 = red_finish_y<SCHED>(racc0, k0, tlog, nthreads, k_local, r_local, lds);
+                if (k1 <= VR_MIN) racc1 = red_finish_y<SCHED>(racc1, k1, tlog, nthreads, k_local, r_local, lds);
+              }
+            }
+          }
+
+          // valid counts of the round's slabs
+          if (recount) {
+            if (in_sweep) {
+              uint32_t nvp = 0;
+              FOR_U {
+                const uint32_t ru = ridx + u * r_step;
+                const bool ok = kvalid && ru < h.n_ridx;
+                uint32_t nv = inner_red ? group_valid(ok ? ru : 0u, h.rdims, h.n_rdim, h.inner_extent) : (nvp_out & 0xfu);
+                nv &= ok ? 0xfu : 0u;
+                nvp |= nv << (4 * u);
+              }
+              sl = slab_state(nvp);
+            } else {
+              sl = sl_out;
+            }
+          }
+        }
+      };
       // VOP_LD flagged VI_LD_PAIR: the next instruction is a float binary whose memory operand has the load's
       // element offsets. When both take the wide path the load fetches both operands in one trip to memory and
       // the binary is finished in the same dispatch (true: src holds its operand; w0, op, sub are the binary's).
@@ -1155,6 +1253,74 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                   const vf4 lo = keep_lds[((lr * U + u) * 2u) * nthreads + tid], hi = keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid];
                   acc.v[u] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
                 }
+                continue;
+              }
+              if (in_sweep && (w0 & VI_LD_RED2)) {
+                // The round is this load and the float reduce behind it, which closes the round: fetch this round
+                // and the next in one trip to memory, reduce both, and go on two rounds further.
+                const uint32_t wr = uni(fetched[0]);
+                const uint32_t rsub = (wr >> 8) & 0xffu, rslot = wr >> 24;
+                const bool have2 = round + 1u < n_rounds;
+                const uint32_t ridx2 = sweep_rev ? ridx - r_step * U : ridx + r_step * U;
+                Offs off2 = off;
+                Slabs sl2 = sl;
+                if (have2) {
+                  const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, !inner_red);
+                  uint32_t nvp2 = 0;
+                  FOR_U {
+                    const uint32_t ru = ridx2 + u * r_step;
+                    const bool ok = kvalid && ru < h.n_ridx;
+                    off2.v[u] = koff + space_offset(ok ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+                    uint32_t nv = inner_red ? group_valid(ok ? ru : 0u, h.rdims, h.n_rdim, h.inner_extent) : (nvp_out & 0xfu);
+                    nv &= ok ? 0xfu : 0u;
+                    nvp2 |= nv << (4 * u);
+                  }
+                  sl2 = slab_state(nvp2);
+                }
+                constexpr uint32_t kFast = VMF_VEC | VMF_ALIGNED;
+                if (have2 && (m.flags & kFast) == kFast && sl.uniform && sl2.uniform) {
+                  mem_load_wide_2rounds(m, off, off2, sl.full, sl2.full, acc, src);
+                } else {
+                  mem_load(m, off, sl, acc);
+                  if (have2) mem_load(m, off2, sl2, src);
+                }
+                if (w0 & VI_LD_KEEP_WR) {
+                  const uint32_t lr2 = sweep_rev ? lr - 1u : lr + 1u;
+                  if (lr < n_parked) {
+                    FOR_U {
+                      keep_lds[((lr * U + u) * 2u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 0, 1, 2, 3);
+                      keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 4, 5, 6, 7);
+                    }
+                  }
+                  if (have2 && lr2 < n_parked) {
+                    FOR_U {
+                      keep_lds[((lr2 * U + u) * 2u) * nthreads + tid] = __builtin_shufflevector(src.v[u], src.v[u], 0, 1, 2, 3);
+                      keep_lds[((lr2 * U + u) * 2u + 1u) * nthreads + tid] = __builtin_shufflevector(src.v[u], src.v[u], 4, 5, 6, 7);
+                    }
+                  }
+                }
+                auto reduce_into_slots = [&](Acc &x, const Slabs &sx) {  // what VOP_RED does, for one round's values
+                  if (rsub & VRF_SQUARE) FOR_U x.v[u] = x.v[u] * x.v[u];
+                  if (rslot == 0) {
+                    red_accumulate<SCHED>(racc0, rsub & 0xfu, x, sx);
+                    if (rsub & VRF_PAIR) {
+                      FOR_U x.v[u] = x.v[u] * x.v[u];
+                      red_accumulate<SCHED>(racc1, rsub & 0xfu, x, sx);
+                    }
+                  } else {
+                    red_accumulate<SCHED>(racc1, rsub & 0xfu, x, sx);
+                  }
+                };
+                reduce_into_slots(acc, sl);
+                if (have2) {
+                  reduce_into_slots(src, sl2);
+                  ++round;
+                  ridx = ridx2;
+                }
+                // the reduce is done: the round ends here, and the next instruction is the load again or what follows the reduce
+                pc = round + 1u < n_rounds ? sweep_pc : pc + 1u;
+                fetched = code64[pc];
+                end_round(true, true);
                 continue;
               }
               const bool keep = parked && (w0 & VI_LD_KEEP_WR) != 0;
@@ -1410,42 +1576,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             break;
         }
 
-        // end of a round: the next one (the decode above has already turned the pc back), or the end of
-        // the sweep, where the slots' partials are combined across lanes
-        if (ends) {
-          ++round;
-          if (round < n_rounds) {
-            ridx = sweep_rev ? ridx - r_step * U : ridx + r_step * U;
-          } else {
-            in_sweep = false;
-            const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
-            if constexpr (SCHED == VS_REDX) {
-              if (k0 <= VR_MIN || k1 <= VR_MIN) {
-                red_finish_x(racc0.v[0], racc1.v[0], k0, k1, tlog, team_is_block, tid, nthreads, red_flip, lds);
-              }
-            } else {
-              if (k0 <= VR_MIN) racc0 = red_finish_y<SCHED>(racc0, k0, tlog, nthreads, k_local, r_local, lds);
-              if (k1 <= VR_MIN) racc1 = red_finish_y<SCHED>(racc1, k1, tlog, nthreads, k_local, r_local, lds);
-            }
-          }
-        }
-
-        // valid counts of the round's slabs
-        if (op == VOP_SWEEP || ends) {
-          if (in_sweep) {
-            uint32_t nvp = 0;
-            FOR_U {
-              const uint32_t ru = ridx + u * r_step;
-              const bool ok = kvalid && ru < h.n_ridx;
-              uint32_t nv = inner_red ? group_valid(ok ? ru : 0u, h.rdims, h.n_rdim, h.inner_extent) : (nvp_out & 0xfu);
-              nv &= ok ? 0xfu : 0u;
-              nvp |= nv << (4 * u);
-            }
-            sl = slab_state(nvp);
-          } else {
-            sl = sl_out;
-          }
-        }
+        end_round(ends, op == VOP_SWEEP || ends);
       }
     }
   }

@@ -162,6 +162,7 @@ std::string &VKernel::DisAssemble() {
             if (static_cast<uint32_t>(w) & VI_LD_KEEP_WR) os << "  ; parks its first " << (VI_IMM(w) & 0xffffu) << " rounds in local memory";
             if (static_cast<uint32_t>(w) & VI_LD_KEEP_RD) os << "  ; takes its first " << (VI_IMM(w) & 0xffffu) << " rounds from local memory";
             if (static_cast<uint32_t>(w) & VI_LD_PAIR) os << "  ; fetches the next instruction's operand in the same trip";
+            if (static_cast<uint32_t>(w) & VI_LD_RED2) os << "  ; fetches two rounds per trip and does the reduce behind it";
             break;
           case VOP_BINF:
             if (VI_KIND(w) == VK_SREG2) {  // two chained operations

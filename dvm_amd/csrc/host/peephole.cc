@@ -48,6 +48,16 @@ void Compiler::PairLoads() {
     if (!(static_cast<uint32_t>(nx) & VI_SAME_OFFS) || (static_cast<uint32_t>(nx) & (VI_UNIFORM | VI_ENDS))) continue;
     code_[i] = w | VI_LD_PAIR;
   }
+  // A sweep whose body is one load and one float reduce (the statistics sweep of a normalisation): the load may
+  // fetch two rounds per trip and do the reduce itself.
+  if ((hdr_.sched & VS_KIND_MASK) == VS_REDX) {
+    for (size_t i = 1; i + 1 < code_.size(); ++i) {
+      const uint64_t w = code_[i], nx = code_[i + 1];
+      if (VI_OP(code_[i - 1]) != VOP_SWEEP || VI_OP(w) != VOP_LD || (static_cast<uint32_t>(w) & (VI_UNIFORM | VI_LD_PAIR))) continue;
+      if (VI_OP(nx) != VOP_RED || !(static_cast<uint32_t>(nx) & VI_ENDS) || (VI_SUB(nx) & VRF_INT)) continue;
+      code_[i] = w | VI_LD_RED2;
+    }
+  }
 }
 
 // The interpreter pays a fixed price per instruction, so the short bodies of sweeps are tightened:

@@ -144,6 +144,12 @@ enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 // memory operand with VI_SAME_OFFS. The load may fetch both operands at once (one trip to memory for the pair)
 // and finish the binary in the same dispatch; an interpreter that ignores the flag computes the same.
 #define VI_LD_PAIR (1u << 8)
+// VI_LD_RED2 (second bit of VOP_LD's sub field; schedule that reduces the innermost axis): the body of the sweep
+// is this load and one float VOP_RED with VI_ENDS behind it (a statistics sweep). The load may fetch this round
+// and the next in one trip to memory, do the reduce for both and step two rounds; an interpreter that ignores
+// the flag computes the same, round by round. (The partials of the two orders are the same sums: the reduce
+// accumulates per lane in the order of the rounds either way.)
+#define VI_LD_RED2 (1u << 9)
 // VI_ENDS (top bit of the opcode byte; set on every VOP_ENDSWEEP, and on a store or reduce that took over the
 // VOP_ENDSWEEP behind it): the instruction closes the round of its sweep. One bit, so that the decoder finds the
 // next pc without comparing opcodes.
