@@ -197,10 +197,12 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
         if (VI_OP(p.w[i]) != VOP_LD) continue;
         if (static_cast<uint32_t>(p.w[i]) & (VI_LD_KEEP_WR | VI_LD_KEEP_RD)) {
           if (wide) return static_cast<int>(hipErrorInvalidValue);
-          parked = std::max<uint64_t>(parked, VI_IMM(p.w[i]) & 0xffffu);
+          // rounds x bytes per slab: two 16-byte planes for fp32 values, one for values parked as fp16 / bf16
+          const uint64_t planes = ((VI_IMM(p.w[i]) >> 20) & 3u) == VF_F32 ? 2 : 1;
+          parked = std::max<uint64_t>(parked, (VI_IMM(p.w[i]) & 0xffffu) * planes);
         }
       }
-      need += parked * threads * u * 32;
+      need += parked * threads * u * 16;
       if (lds_bytes < need) return static_cast<int>(hipErrorInvalidValue);
     }
     switch (h->sched & VS_KIND_MASK) {

@@ -968,6 +968,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   Acc acc;
   FOR_U acc.v[u] = 0.0f;
   uint32_t mask = 0;
+  uint32_t park_slot = 0, park_fmt = 0;  // a value waiting to be parked after the instruction behind its load (slot + 1; 0: none)
   RedAcc<SCHED> racc0, racc1;
   red_init<SCHED>(racc0, VR_SUM);
   red_init<SCHED>(racc1, VR_SUM);
@@ -1247,12 +1248,14 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               // rounds parked in local memory by the load that opened an earlier sweep over this operand
               const uint32_t lr = sweep_rev ? n_rounds - 1u - round : round;
               const uint32_t n_parked = imm & 0xffffu;
+              const uint32_t keep_prefix = (imm >> 16) & 0x3u, keep_fmt = (imm >> 20) & 0x3u;  // VI_LD_KEEP_*: see isa_gfx950.h
+              const uint32_t keep_at = keep_fmt == VF_F32 ? 2u * lr : lr;  // fp32 values take two planes per slab
               const bool parked = in_sweep && lr < n_parked;
               if (parked && (w0 & VI_LD_KEEP_RD)) {
-                FOR_U {
-                  const vf4 lo = keep_lds[((lr * U + u) * 2u) * nthreads + tid], hi = keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid];
-                  acc.v[u] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-                }
+                vreg_load(keep_lds, keep_at, keep_fmt, nthreads, tid, acc);
+                // what was parked is the value behind the next keep_prefix instructions: they are done already
+                pc += keep_prefix;
+                fetched = code64[pc];
                 continue;
               }
               if (in_sweep && (w0 & VI_LD_RED2)) {
@@ -1284,20 +1287,10 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                   mem_load(m, off, sl, acc);
                   if (have2) mem_load(m, off2, sl2, src);
                 }
-                if (w0 & VI_LD_KEEP_WR) {
+                if (w0 & VI_LD_KEEP_WR) {  // (a load with a reduce behind it parks what it loaded: no prefix, fp32)
                   const uint32_t lr2 = sweep_rev ? lr - 1u : lr + 1u;
-                  if (lr < n_parked) {
-                    FOR_U {
-                      keep_lds[((lr * U + u) * 2u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 0, 1, 2, 3);
-                      keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 4, 5, 6, 7);
-                    }
-                  }
-                  if (have2 && lr2 < n_parked) {
-                    FOR_U {
-                      keep_lds[((lr2 * U + u) * 2u) * nthreads + tid] = __builtin_shufflevector(src.v[u], src.v[u], 0, 1, 2, 3);
-                      keep_lds[((lr2 * U + u) * 2u + 1u) * nthreads + tid] = __builtin_shufflevector(src.v[u], src.v[u], 4, 5, 6, 7);
-                    }
-                  }
+                  if (lr < n_parked) vreg_store(keep_lds, 2u * lr, VF_F32, nthreads, tid, acc);
+                  if (have2 && lr2 < n_parked) vreg_store(keep_lds, 2u * lr2, VF_F32, nthreads, tid, src);
                 }
                 auto reduce_into_slots = [&](Acc &x, const Slabs &sx) {  // what VOP_RED does, for one round's values
                   if (rsub & VRF_SQUARE) FOR_U x.v[u] = x.v[u] * x.v[u];
@@ -1326,9 +1319,11 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               const bool keep = parked && (w0 & VI_LD_KEEP_WR) != 0;
               const bool pair = take_next_along(m, off, sl, acc, src);
               if (keep) {
-                FOR_U {
-                  keep_lds[((lr * U + u) * 2u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 0, 1, 2, 3);
-                  keep_lds[((lr * U + u) * 2u + 1u) * nthreads + tid] = __builtin_shufflevector(acc.v[u], acc.v[u], 4, 5, 6, 7);
+                if (keep_prefix == 0) {
+                  vreg_store(keep_lds, keep_at, keep_fmt, nthreads, tid, acc);
+                } else {  // the value to park is the result of the instruction behind this load
+                  park_slot = keep_at + 1u;
+                  park_fmt = keep_fmt;
                 }
               }
               if (!pair) continue;
@@ -1407,6 +1402,12 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
           default: {  // VOP_MOVM
             FOR_U FOR_E acc.v[u][e] = ((mask >> (u * E + e)) & 1u) ? src.v[u][e] : acc.v[u][e];
             break;
+          }
+        }
+        if constexpr (SCHED == VS_REDX) {
+          if (park_slot != 0u) {  // this was the instruction behind a load that parks its round
+            vreg_store(keep_lds, park_slot - 1u, park_fmt, nthreads, tid, acc);
+            park_slot = 0u;
           }
         }
         continue;

@@ -159,8 +159,11 @@ std::string &VKernel::DisAssemble() {
           case VOP_UNI_END: os << "end of per-output run"; break;
           case VOP_LD:
             os << "load." << kMemTypes[mem_dtype(VI_A(w))] << " acc, m" << VI_A(w);
-            if (static_cast<uint32_t>(w) & VI_LD_KEEP_WR) os << "  ; parks its first " << (VI_IMM(w) & 0xffffu) << " rounds in local memory";
-            if (static_cast<uint32_t>(w) & VI_LD_KEEP_RD) os << "  ; takes its first " << (VI_IMM(w) & 0xffffu) << " rounds from local memory";
+            if (static_cast<uint32_t>(w) & (VI_LD_KEEP_WR | VI_LD_KEEP_RD)) {
+              const bool wr = (static_cast<uint32_t>(w) & VI_LD_KEEP_WR) != 0;
+              os << (wr ? "  ; parks its first " : "  ; takes its first ") << (VI_IMM(w) & 0xffffu) << (wr ? " rounds in local memory" : " rounds from local memory");
+              if ((VI_IMM(w) >> 16) & 3u) os << " (the value behind the next instruction, as " << kFmt[(VI_IMM(w) >> 20) & 3u] << ")";
+            }
             if (static_cast<uint32_t>(w) & VI_LD_PAIR) os << "  ; fetches the next instruction's operand in the same trip";
             if (static_cast<uint32_t>(w) & VI_LD_RED2) os << "  ; fetches two rounds per trip and does the reduce behind it";
             break;

@@ -222,11 +222,28 @@ void Compiler::PlanRereads() {
     if (sweeps[a].ld < 0) continue;
     for (size_t b = a + 1; b < sweeps.size(); ++b) {
       if (sweeps[b].ld < 0 || VI_A(cw[sweeps[b].ld]) != VI_A(cw[sweeps[a].ld])) continue;
-      if (budget <= fixed + per_round_bytes) return;
-      const uint32_t rounds = std::min<uint32_t>(n_rounds, (budget - fixed) / per_round_bytes);
-      cw[sweeps[a].ld] |= VI_LD_KEEP_WR | (static_cast<uint64_t>(rounds) << 32);
-      cw[sweeps[b].ld] |= VI_LD_KEEP_RD | (static_cast<uint64_t>(rounds) << 32);
-      prog_->lds_bytes += rounds * per_round_bytes;
+      // When both sweeps go on with the same instruction behind the load (x + residual: a float binary on an
+      // immediate or on a memory operand with the load's offsets), its result is what gets parked, and the
+      // reading sweep skips it in parked rounds: neither operand is read twice. A result rounded to a 16-bit
+      // type is parked in that type, at half the local memory per round.
+      uint32_t prefix = 0, fmt = VF_F32;
+      const size_t la = static_cast<size_t>(sweeps[a].ld), lb = static_cast<size_t>(sweeps[b].ld);
+      if (la + 2 < n && lb + 2 < n && cw[la + 1] == cw[lb + 1]) {
+        const uint64_t w = cw[la + 1];
+        const uint32_t lo = static_cast<uint32_t>(w);
+        const bool operand_ok = VI_KIND(w) == VK_IMM || (VI_KIND(w) == VK_MEM && (lo & VI_SAME_OFFS));
+        if (VI_OP(w) == VOP_BINF && operand_ok && !(lo & (VI_UNIFORM | VI_ENDS))) {
+          prefix = 1;
+          fmt = VI_RND(w) == VRND_F16 ? VF_F16 : (VI_RND(w) == VRND_BF16 ? VF_BF16 : VF_F32);
+        }
+      }
+      const uint32_t round_bytes = fmt == VF_F32 ? per_round_bytes : per_round_bytes / 2;
+      if (budget <= fixed + round_bytes) return;
+      const uint32_t rounds = std::min<uint32_t>(n_rounds, (budget - fixed) / round_bytes);
+      const uint64_t imm = static_cast<uint64_t>(rounds | (prefix << 16) | (fmt << 20)) << 32;
+      cw[la] |= VI_LD_KEEP_WR | imm;
+      cw[lb] |= VI_LD_KEEP_RD | imm;
+      prog_->lds_bytes += rounds * round_bytes;
       return;
     }
   }

@@ -132,9 +132,13 @@ enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 // VI_SAME_OFFS (vector VM, memory instructions): the operand has the strides of the previous memory
 // instruction of the same round, whose element offsets are reused.
 // Re-reading less in the second sweep over a tensor (vector VM, schedule that reduces the innermost axis):
-//  VI_LD_KEEP_WR / VI_LD_KEEP_RD (VOP_LD that opens a sweep; the rnd field is free there, imm = number of rounds):
-//    the first load parks the slabs of its first imm rounds in local memory, the load that opens a later sweep
-//    over the same operand takes those rounds from there instead of from memory;
+//  VI_LD_KEEP_WR / VI_LD_KEEP_RD (VOP_LD that opens a sweep; the rnd field is free there; imm[15:0] = number of
+//    rounds): the first load parks the slabs of its first rounds in local memory, the load that opens a later
+//    sweep over the same operand takes those rounds from there instead of from memory. imm[17:16] = p (0 or 1):
+//    what is parked is the accumulator behind the p instructions that follow the load, which both sweeps have in
+//    common (x + residual), and the reading sweep skips those p instructions in a parked round, so their memory
+//    operands are not read again either. imm[21:20] = VF_*: how the value is parked (fp32: two 16-byte planes per
+//    slab; fp16 / bf16, when the last common instruction rounds to that type: one);
 //  VSW_REVERSE (sub field of VOP_SWEEP): the sweep walks its rounds last to first, so that it starts with
 //    what the sweep before it read last (still in the L2 cache) and ends with the parked rounds.
 #define VI_LD_KEEP_WR (1u << 20)
