@@ -260,8 +260,9 @@ typedef struct {
 // sqrt and division by their _APPROX forms (one ulp of fp32; the 16-bit rounding is four orders coarser).
 #define VCF_APPROX_MATH 1u
 
-// Dynamic local memory a VE_CUBE launch needs for block tile `bt` (256, 128 or 64): the double-buffered
-// operand tiles of the k loop, or the half tile of fp32 accumulators the epilogue reads back.
+// Dynamic local memory a VE_CUBE launch needs for block tile `bt` (256, 128 or 64): the operand tiles of the k
+// loop (two buffers of 64 k per operand; for the 256 tile the same bytes as four stage buffers of 32 k), or the
+// half tile of fp32 accumulators the epilogue reads back.
 #define DVM_CUBE_LDS_BYTES(bt) \
   ((2u * (2u * (bt)) * 64u * 2u) > (((bt) >= 128u ? (bt) / 2u : (bt)) * ((bt) + 4u) * 4u) \
        ? (2u * (2u * (bt)) * 64u * 2u) \
