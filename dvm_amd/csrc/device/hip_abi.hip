@@ -235,6 +235,15 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
                     (c->a_addr & 15u) != 0 || (c->b_addr & 15u) != 0)) {
       return static_cast<int>(hipErrorInvalidValue);
     }
+    const uint32_t split = c->epi_flags & (VCF_SPLITK_PARTIAL | VCF_SPLITK_COMBINE);
+    if (split != 0) {
+      const uint64_t tiles = static_cast<uint64_t>(c->tiles_m) * c->tiles_n * c->nb0 * c->nb1;
+      if (split == (VCF_SPLITK_PARTIAL | VCF_SPLITK_COMBINE) || c->k_split < 2 || c->k_chunk == 0 || c->k_chunk % 64 != 0 ||
+          static_cast<uint64_t>(c->k_chunk) * (c->k_split - 1) >= c->k || static_cast<uint64_t>(c->k_chunk) * c->k_split < c->k ||
+          c->part_addr == 0 || (c->part_addr & 15u) != 0 || tiles * c->k_split >= (1ull << 31)) {
+        return static_cast<int>(hipErrorInvalidValue);
+      }
+    }
     const CubeKernel kern = kCubeKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0][(c->trans_a ? 2 : 0) + (c->trans_b ? 1 : 0)];
     hipLaunchKernelGGL(kern, dim3(block_dim), dim3(want_threads), lds_bytes, s, p);
   } else if (h->entry == VE_ATTN) {

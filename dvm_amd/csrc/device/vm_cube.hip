@@ -873,7 +873,7 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
 // every lane takes slabs of 8 columns and walks the epilogue program over them.
 template <int ROWS, int BN, int TM, int WM>
 __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
-                                                        uint32_t pass, uint32_t m, uint32_t n) {
+                                                        uint32_t pass, uint32_t m, uint32_t n, uint32_t m_lo, uint32_t n_lo) {
   constexpr int NTHR = WM * 2 * 64;
   constexpr int PITCH = BN + 4;
   constexpr int GROUPS = BN / 8;               // slabs per row
@@ -886,7 +886,8 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
   const uint32_t g = tid % GROUPS, r0 = tid / GROUPS;
   constexpr int HALF = ROWS / WM;  // local rows [i * HALF, (i + 1) * HALF) belong to the i-th row of waves
   const uint32_t col = n0 + g * 8;
-  const uint32_t ncol = col >= n ? 0u : (n - col < 8u ? n - col : 8u);
+  // (a tile moved back from the edge starts its columns a whole number of slabs before n_lo)
+  const uint32_t ncol = (col >= n || col < n_lo) ? 0u : (n - col < 8u ? n - col : 8u);
   {
     const uint32_t *code32 = prog32 + 2 * ea.code_off;
     const uint32_t li = (tid & 63u) < ea.w0v ? (tid & 63u) : 0u;  // w0v arrives holding the instruction count
@@ -902,7 +903,7 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
       const uint32_t lr = (it * SL + s) * ROWS_PER_STEP + r0;  // local row of the dump
       const uint32_t wm = lr / HALF, rr = lr % HALF;
       rows.row[s] = m0 + wm * (TM * 32) + pass * HALF + rr;
-      rows.ok |= (rows.row[s] < m ? 1u : 0u) << s;
+      rows.ok |= ((rows.row[s] < m && rows.row[s] >= m_lo) ? 1u : 0u) << s;
       const vf4 lo = *reinterpret_cast<const vf4 *>(dump + lr * PITCH + g * 8), hi = *reinterpret_cast<const vf4 *>(dump + lr * PITCH + g * 8 + 4);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -910,6 +911,7 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
         acc[s * 8 + 4 + e] = hi[e];
       }
     }
+    if (wave_all(rows.ok == 0u || ncol == 0u)) continue;  // nothing of these slabs is inside the tile's part of the output
     run_epilogue<SL>(acc, prog32, ea, rows, col, ncol);
   }
 }
@@ -955,7 +957,12 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
   const uint32_t wm = wave >> 1, wn = wave & 1u;
   const uint32_t tiles_per_batch = h.tiles_m * h.tiles_n;
   const uint32_t n_tiles = tiles_per_batch * h.nb0 * h.nb1;
-  const uint32_t nk = (h.k + BK - 1) / BK;
+  // Split k (VCF_SPLITK_*): the first launch has k_split workgroups per tile, each walks k_chunk of the k axis and
+  // leaves its fp32 accumulators in the partials buffer, register by register as the lanes hold them; the second
+  // launch has one workgroup per tile, adds the partials in ascending k order and runs the epilogue.
+  const bool split_part = (h.epi_flags & VCF_SPLITK_PARTIAL) != 0u, split_comb = (h.epi_flags & VCF_SPLITK_COMBINE) != 0u;
+  const uint32_t n_work = split_part ? n_tiles * h.k_split : n_tiles;
+  constexpr uint32_t kPartVecs = TM * TN * 4;  // 16-byte vectors a lane holds of the tile
 
   // Fragment reads: fragment i of this wave is rows r0 + 32*i of the staged tile (r0 = the lane's row
   // in fragment 0), and step kk wants chunk 2*kk + lane/32 of that row. With the swizzle of tile_off
@@ -968,19 +975,34 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
     return row + static_cast<uint32_t>(f) * 32u * BK + (x ^ static_cast<uint32_t>((kk << 4) ^ ((f & 1) << 5)));
   };
 
-  for (uint32_t t0 = blockIdx.x; t0 < n_tiles; t0 += gridDim.x) {
+  for (uint32_t t0 = blockIdx.x; t0 < n_work; t0 += gridDim.x) {
     // Tile order. Workgroups are dealt to the 8 XCDs round robin, each XCD has its own L2: workgroup w
     // takes position (w % 8) * (n_tiles / 8) + w / 8, so an XCD works through one contiguous eighth of the
     // order; the order itself walks 8-tile-wide column bands row by row, which makes the 32 tiles an XCD has
     // in flight a 4 x 8 block (12 operand panels to fetch instead of 18 for two full rows of 16).
     uint32_t t = t0;
-    if ((n_tiles & 7u) == 0 && gridDim.x == n_tiles) t = (t0 & 7u) * (n_tiles >> 3) + (t0 >> 3);
+    if ((n_work & 7u) == 0 && gridDim.x == n_work) t = (t0 & 7u) * (n_work >> 3) + (t0 >> 3);
+    const uint32_t ksplit = t / n_tiles;  // which part of the k axis (0 unless the launch writes partials)
+    t -= ksplit * n_tiles;
+    const uint32_t tile_id = t;
+    const uint32_t k_lo = ksplit * h.k_chunk;
+    const uint32_t k_hi = split_part ? (k_lo + h.k_chunk < h.k ? k_lo + h.k_chunk : h.k) : h.k;
+    const uint32_t nk = (k_hi - k_lo + BK - 1) / BK;
     const uint32_t batch = t / tiles_per_batch, tt = t % tiles_per_batch;
     const uint32_t bi0 = batch / h.nb1, bi1 = batch % h.nb1;
     const uint32_t band = tt / (h.tiles_m * 8u), in_band = tt % (h.tiles_m * 8u);
     const uint32_t band_w = h.tiles_n - band * 8u < 8u ? h.tiles_n - band * 8u : 8u;
     const uint32_t tm = in_band / band_w, tn = band * 8u + in_band % band_w;
-    const uint32_t m0 = tm * BM, n0 = tn * BN;
+    // A ragged tile at the bottom or right edge is moved back inside the output (it overlaps its neighbour) so that
+    // it can take the vector path like any full tile; its epilogue covers only the rows from m_lo and the columns
+    // from n_lo on, the part no other tile writes. (Columns move in whole 8-element slabs only; an operand whose
+    // rows are the contiguous axis needs the new origin 16-byte aligned.)
+    uint32_t m0 = tm * BM, n0 = tn * BN;
+    const uint32_t m_lo = m0, n_lo = n0;
+    if (h.fast) {
+      if (m0 + BM > h.m && h.m >= BM && (A_KC || (h.m & 7u) == 0)) m0 = h.m - BM;
+      if (n0 + BN > h.n && h.n >= BN && (h.n & 7u) == 0) n0 = h.n - BN;
+    }
     const uint64_t a_base = h.a_addr + (static_cast<uint64_t>(bi0) * h.a_sb0 + static_cast<uint64_t>(bi1) * h.a_sb1) * 2;
     const uint64_t b_base = h.b_addr + (static_cast<uint64_t>(bi0) * h.b_sb0 + static_cast<uint64_t>(bi1) * h.b_sb1) * 2;
 
@@ -991,17 +1013,31 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       for (int j = 0; j < TN; ++j) acc[i][j] = 0.0f;
 
     constexpr bool RING = BM == 256 && BN == 256;  // the ring of 32-deep stages
-    if (h.fast && m0 + BM <= h.m && n0 + BN <= h.n) {
+    // address of element (row0, k_lo) of each operand
+    const uint64_t a_org = a_base + (A_KC ? static_cast<uint64_t>(m0) * h.lda + k_lo : static_cast<uint64_t>(k_lo) * h.lda + m0) * 2;
+    const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb + k_lo : static_cast<uint64_t>(k_lo) * h.ldb + n0) * 2;
+    if (split_comb) {
+      const DVM_GLOBAL vf4 *src = reinterpret_cast<const DVM_GLOBAL vf4 *>(h.part_addr) + static_cast<uint64_t>(tile_id) * kPartVecs * NTHR + tid;
+      const uint64_t split_stride = static_cast<uint64_t>(n_tiles) * kPartVecs * NTHR;
+      for (uint32_t sp = 0; sp < h.k_split; ++sp) {
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+          for (int j = 0; j < TN; ++j)
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const vf4 v = src[sp * split_stride + static_cast<uint32_t>((i * TN + j) * 4 + q) * NTHR];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[e];
+            }
+      }
+    } else if (h.fast && m0 + BM <= h.m && n0 + BN <= h.n) {
      if constexpr (RING) {
-      const uint64_t a_org = a_base + (A_KC ? static_cast<uint64_t>(m0) * h.lda : static_cast<uint64_t>(m0)) * 2;
-      const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb : static_cast<uint64_t>(n0)) * 2;
-      tile_loop_ring<IS_BF16, A_KC, B_KC, WM>(acc, lds, a_org, b_org, h.lda, h.ldb, h.k / SK, tid);
+      tile_loop_ring<IS_BF16, A_KC, B_KC, WM>(acc, lds, a_org, b_org, h.lda, h.ldb, (k_hi - k_lo) / SK, tid);
      } else {
       Stage<BM, A_KC, NTHR> sa;
       Stage<BN, B_KC, NTHR> sb;
-      // address of element (row0, k) of each operand, k advancing by BK per step
-      const uint64_t a_org = a_base + (A_KC ? static_cast<uint64_t>(m0) * h.lda : static_cast<uint64_t>(m0)) * 2;
-      const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb : static_cast<uint64_t>(n0)) * 2;
+      // k advances by BK per step
       const uint64_t a_step = (A_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.lda) * 2;
       const uint64_t b_step = (B_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.ldb) * 2;
       const LaneOffsets a_voff = Stage<BM, A_KC, NTHR>::lane_offset(h.lda, tid), b_voff = Stage<BN, B_KC, NTHR>::lane_offset(h.ldb, tid);
@@ -1141,8 +1177,8 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
      }
     } else {
       for (uint32_t kt = 0; kt < nk; ++kt) {
-        stage_generic<BM, NTHR>(lds, a_base, h.lda, m0, kt * BK, h.m, h.k, A_KC ? 1u : 0u, tid);
-        stage_generic<BN, NTHR>(lds + kBBase, b_base, h.ldb, n0, kt * BK, h.n, h.k, B_KC ? 1u : 0u, tid);
+        stage_generic<BM, NTHR>(lds, a_base, h.lda, m0, k_lo + kt * BK, h.m, k_hi, A_KC ? 1u : 0u, tid);
+        stage_generic<BN, NTHR>(lds + kBBase, b_base, h.ldb, n0, k_lo + kt * BK, h.n, k_hi, B_KC ? 1u : 0u, tid);
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {
@@ -1160,6 +1196,21 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       }
     }
 
+    if (split_part) {
+      DVM_GLOBAL vf4 *dst = reinterpret_cast<DVM_GLOBAL vf4 *>(h.part_addr) +
+                            (static_cast<uint64_t>(ksplit) * n_tiles + tile_id) * kPartVecs * NTHR + tid;
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const vf16 &c = acc[i][j];
+            const vf4 v = {c[4 * q], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3]};
+            dst[static_cast<uint32_t>((i * TN + j) * 4 + q) * NTHR] = v;
+          }
+      continue;
+    }
     // epilogue: accumulators -> local memory (row major), then slabs through the program
     const EpiArgs ea = {h.mem_off, h.code_off, bi0, bi1, h.epi_flags, h.n_code, 0};
 #pragma unroll
@@ -1177,7 +1228,7 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
         }
       }
       __syncthreads();
-      epilogue_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n);
+      epilogue_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
       __syncthreads();
     }
   }

@@ -215,7 +215,10 @@ std::string &VKernel::DisAssemble() {
       static const int tile[] = {256, 128, 64, 256};
       os << "entry cube " << kMemTypes[c->dtype] << " m=" << c->m << " n=" << c->n << " k=" << c->k << " trans_a=" << c->trans_a
          << " trans_b=" << c->trans_b << " batch=" << c->nb0 << "x" << c->nb1 << " tile=" << tile[c->tile] << " blocks=" << p.grid
-         << " lds=" << p.lds_bytes << (c->fast ? " fast" : " guarded") << (c->tile == 3 ? " eight-waves" : "") << "\n";
+         << " lds=" << p.lds_bytes << (c->fast ? " fast" : " guarded") << (c->tile == 3 ? " eight-waves" : "");
+      if (c->epi_flags & VCF_SPLITK_PARTIAL) os << " split-k partials " << c->k_split << " x " << c->k_chunk;
+      if (c->epi_flags & VCF_SPLITK_COMBINE) os << " split-k sum of " << c->k_split;
+      os << "\n";
       const VCubeMem *cm = reinterpret_cast<const VCubeMem *>(p.blob.w + c->mem_off);
       for (uint32_t i = 0; i < c->n_mem; ++i) {
         char buf[32];
@@ -223,7 +226,11 @@ std::string &VKernel::DisAssemble() {
         os << "  m" << i << ": " << kMemTypes[cm[i].dtype] << " @" << buf << " strides n=" << cm[i].stride_n << " m=" << cm[i].stride_m
            << " b=" << cm[i].stride_b0 << "," << cm[i].stride_b1 << "\n";
       }
-      os << "  mmad acc, A, B\n";
+      if (c->epi_flags & VCF_SPLITK_PARTIAL) {
+        os << "  mmad acc, A, B\n  store.fp32 partials, acc\n";
+        continue;
+      }
+      os << ((c->epi_flags & VCF_SPLITK_COMBINE) ? "  sum acc, partials\n" : "  mmad acc, A, B\n");
       print_code(p.blob.w + c->code_off, c->n_code, [&](uint32_t m) { return cm[m].dtype; });
     } else if (h->entry == VE_ATTN) {
       const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.blob.w);

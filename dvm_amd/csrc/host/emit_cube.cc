@@ -199,6 +199,72 @@ void Compiler::CompileCube(int a) {
   // the interpreted epilogue. Measured on MI355X, bf16 8192x4096xk, row-major operands, four -> eight waves:
   // k = 64: 60 -> 54 us (with bias + SiLU 106 -> 87 us), k = 512: 82 -> 76 us, k = 4096: 296-301 us either way for
   // the plain product (the sustained rate is set by the power cap there), 338-342 -> 334-339 us with bias + SiLU.
+  // Split k: with fewer tiles than compute units and a long k axis, k_split workgroups share a tile's k axis and a
+  // second launch adds their fp32 partial tiles in a fixed order and runs the epilogue (the reference splits k into
+  // consecutive matmuls accumulating in fp32 when the operands exceed its L2, src/ops_m.cc:240-264,
+  // src/xkernel.cc:1511-1547; here the reason is to fill the chip). Every candidate (tile, parts) gets an estimate
+  // from figures measured on MI355X (bf16, microseconds): a workgroup's time per 64 k (2.2 for the 256 tile, 1.3 for
+  // 128, 0.71 for 64 alone on its compute unit and 0.9 when two share one; the guarded path of ragged or unaligned
+  // tiles takes about six times as long), rounds of workgroups over the chip, and for a split the second launch plus
+  // the time its one workgroup per tile needs per partial tile (8.5 / 4.5 / 0.55: a single workgroup streams at
+  // some 30 GB/s), which is what keeps deep splits of big tiles from paying.
+  uint32_t k_split = 1, k_chunk = 0;
+  {
+    const int forced = k_->tuning_.cube_splitk;
+    const bool user_tile = k_->tuning_.cube_tile == 256 || k_->tuning_.cube_tile == 128 || k_->tuning_.cube_tile == 64;
+    auto parts_of = [&](uint32_t want, uint32_t *chunk) -> uint32_t {  // parts actually made when `want` are asked for
+      if (want < 2 || K < 128) return 1;
+      const int64_t c = ((K + want - 1) / want + 63) / 64 * 64;
+      *chunk = static_cast<uint32_t>(c);
+      return static_cast<uint32_t>((K + c - 1) / c);
+    };
+    if (forced >= 2) {
+      k_split = parts_of(static_cast<uint32_t>(forced), &k_chunk);
+    } else if (forced != 0 && forced != 1) {
+      static const int64_t kTiles[3] = {256, 128, 64};
+      static const double kStepUs[3] = {2.2, 1.3, 0.71}, kPartUs[3] = {8.5, 4.5, 0.55};
+      const bool aligned = K % 64 == 0 && h.lda % 8 == 0 && h.ldb % 8 == 0;
+      double best = 0.0;
+      int best_tile = -1;
+      uint32_t best_split = 1, best_chunk = 0;
+      for (int ti = 0; ti < 3; ++ti) {
+        const int64_t t = kTiles[ti];
+        if (user_tile && t != bt) continue;
+        const uint64_t nt = tiles(t);
+        const uint64_t slots = ti == 2 ? 2 * cus : cus;  // two 64x64 workgroups fit a compute unit
+        const uint32_t max_split = nt >= slots ? 1u : static_cast<uint32_t>(std::min<uint64_t>(slots / nt, 32));
+        // (ragged edge tiles of an aligned product are moved back inside the output and stay on the vector path)
+        const bool m_fast = M % t == 0 || (M >= t && (!mm->trans_a || M % 8 == 0));
+        const bool n_fast = N % t == 0 || (N >= t && N % 8 == 0);
+        const double slow = (aligned && m_fast && n_fast) ? 1.0 : 6.0;
+        for (uint32_t want = 1; want <= max_split; want = want < 2 ? 2 : want * 2) {
+          uint32_t chunk = 0;
+          const uint32_t parts = parts_of(want, &chunk);
+          if (want > 1 && (parts < 2 || chunk < 256)) break;
+          const double steps = (parts > 1 ? static_cast<double>(chunk) : static_cast<double>(K)) / 64.0;
+          const uint64_t wgs = nt * parts;
+          const double rounds = std::ceil(static_cast<double>(wgs) / static_cast<double>(slots));
+          const double step_us = (ti == 2 && wgs > cus) ? 0.9 : kStepUs[ti];
+          double us = rounds * steps * step_us * slow + 3.0;
+          if (parts > 1) us += 5.0 + parts * kPartUs[ti];
+          if (parts > 1 && static_cast<double>(wgs) * static_cast<double>(t * t) * 4.0 > 512.0 * 1024 * 1024) continue;
+          if (best_tile < 0 || us < best) {
+            best = us;
+            best_tile = ti;
+            best_split = parts;
+            best_chunk = chunk;
+          }
+        }
+      }
+      // without a split the tile stays the one chosen above
+      if (best_tile >= 0 && best_split > 1) {
+        bt = kTiles[best_tile];
+        h.tile = static_cast<uint32_t>(best_tile);
+        k_split = best_split;
+        k_chunk = best_chunk;
+      }
+    }
+  }
   if (h.tile == 0 && k_->tuning_.cube_waves != 4) h.tile = 3;
   h.tiles_m = static_cast<uint32_t>((M + bt - 1) / bt);
   h.tiles_n = static_cast<uint32_t>((N + bt - 1) / bt);
@@ -278,5 +344,28 @@ void Compiler::CompileCube(int a) {
   prog_->threads = h.tile == 3 ? 512 : 256;
   prog_->lds_bytes = DVM_CUBE_LDS_BYTES(static_cast<uint32_t>(bt));
   prog_->grid = static_cast<uint32_t>(tiles(bt));
+  if (k_split > 1) {
+    // two launches of the same program: partial products per part of the k axis, then their sum and the epilogue
+    const int slot = static_cast<int>(k_->ws_sizes_.size());
+    k_->ws_sizes_.push_back(static_cast<size_t>(k_split) * tiles(bt) * static_cast<size_t>(bt * bt) * 4);
+    Program::Patch pp;
+    pp.word = static_cast<uint32_t>(offsetof(VCubeHeader, part_addr) / 8);
+    pp.op_id = -1;
+    pp.ws_slot = slot;
+    pp.role = Program::kPatchPlain;
+    prog_->patches.push_back(pp);
+    VCubeHeader *ph = reinterpret_cast<VCubeHeader *>(prog_->blob.w);
+    ph->k_split = k_split;
+    ph->k_chunk = k_chunk;
+    const uint32_t flags = ph->epi_flags;
+    ph->epi_flags = flags | VCF_SPLITK_PARTIAL;
+    prog_->grid = static_cast<uint32_t>(tiles(bt) * k_split);
+    const Program first = *prog_;
+    k_->programs_.push_back(first);
+    prog_ = &k_->programs_.back();
+    reinterpret_cast<VCubeHeader *>(prog_->blob.w)->epi_flags = flags | VCF_SPLITK_COMBINE;
+    prog_->grid = static_cast<uint32_t>(tiles(bt));
+    prog_->fills.clear();
+  }
 }
 }  // namespace dvm

@@ -173,6 +173,7 @@ struct Tuning {
   int vec_pair = -1;   // DVM_VEC_PAIR=0: a load never takes the binary instruction behind it along
   int cube_tile = -1;   // DVM_CUBE_TILE=256|128|64
   int cube_waves = -1;  // DVM_CUBE_WAVES=4|8
+  int cube_splitk = -1;  // DVM_CUBE_SPLITK=0: never split the k axis; N >= 2: split it N ways whenever the shape allows
   int cube_exact = -1;  // DVM_CUBE_EXACT=1: never the hardware approximations of exp, log, sqrt, division in a matmul epilogue
   int attn_waves = -1;  // DVM_ATTN_WAVES=4
   bool debug = false;   // DVM_DEBUG: node dump in compile errors

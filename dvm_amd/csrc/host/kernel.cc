@@ -27,6 +27,7 @@ void Tuning::Read() {
   cube_tile = num("DVM_CUBE_TILE");
   cube_waves = num("DVM_CUBE_WAVES");
   cube_exact = num("DVM_CUBE_EXACT");
+  cube_splitk = num("DVM_CUBE_SPLITK");
   attn_waves = num("DVM_ATTN_WAVES");
   debug = std::getenv("DVM_DEBUG") != nullptr;
 }

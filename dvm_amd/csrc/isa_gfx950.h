@@ -252,6 +252,9 @@ typedef struct {
   uint32_t fast;       // k is a multiple of 64 and every 8-element operand chunk is 16-byte aligned: full tiles take the vector path
   uint32_t epi_flags;  // VCF_*
   uint64_t a_addr, b_addr;
+  uint32_t k_split;    // VCF_SPLITK_*: parts the k axis is cut into (>= 2), each k_chunk long (a multiple of 64; the last
+  uint32_t k_chunk;    // may be shorter), and the fp32 partial tiles: [k_split][tiles][tile vectors][lanes] of 16 bytes
+  uint64_t part_addr;
 } VCubeHeader;
 
 // VCubeHeader::epi_flags
@@ -259,6 +262,12 @@ typedef struct {
 // their inputs (no compare, select, rounding to integers, conversion to int32): the host has replaced exp, log,
 // sqrt and division by their _APPROX forms (one ulp of fp32; the 16-bit rounding is four orders coarser).
 #define VCF_APPROX_MATH 1u
+// Split k, for products with fewer tiles than compute units and a long k axis: two launches of the same program.
+// VCF_SPLITK_PARTIAL: tiles * k_split workgroups; each multiplies one part of the k axis and writes its accumulators
+// to part_addr as the lanes hold them, no epilogue. VCF_SPLITK_COMBINE: one workgroup per tile adds the k_split
+// partials in ascending k order (fp32, the same order on every run) and runs the epilogue on the sum.
+#define VCF_SPLITK_PARTIAL 2u
+#define VCF_SPLITK_COMBINE 4u
 
 // Dynamic local memory a VE_CUBE launch needs for block tile `bt` (256, 128 or 64): the operand tiles of the k
 // loop (two buffers of 64 k per operand; for the 256 tile the same bytes as four stage buffers of 32 k), or the

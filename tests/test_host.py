@@ -232,6 +232,33 @@ def test_matmul_epilogue_is_one_cube_program():
     assert das.index("cast.round.bf16") < das.index("Add.fp32"), das
 
 
+def test_matmul_with_few_tiles_and_a_long_k_axis_is_split(monkeypatch):
+    # 16 tiles of 256x256 on 256 compute units, k = 16384: the k axis is shared, two launches, fp32 partial tiles in
+    # the workspace; DVM_CUBE_SPLITK=0 keeps the single launch, =N forces N parts (rounded to whole 64-k steps)
+    def compile_one(m, n, k):
+        t = Tester("mix", run_mode="das")
+        t.store(t.matmul(t.load(np.zeros([m, k], np.float16)), t.load(np.zeros([k, n], np.float16)), False, False))
+        t.codegen()
+        return t, t.das()
+    t, das = compile_one(1024, 1024, 16384)
+    assert das.count("== sub-kernel") == 2 and "split-k partials" in das and "split-k sum of" in das, das
+    assert "store.fp32 partials, acc" in das and "sum acc, partials" in das, das
+    import re
+    parts, chunk = map(int, re.search(r"split-k partials (\d+) x (\d+)", das).groups())
+    tile = int(re.search(r"tile=(\d+)", das).group(1))
+    assert parts >= 2 and chunk % 64 == 0 and chunk * (parts - 1) < 16384 <= chunk * parts, das
+    assert t.workspace_bytes() == parts * (1024 // tile) ** 2 * tile * tile * 4
+    assert "blocks=%d " % (parts * (1024 // tile) ** 2) in das and "blocks=%d " % ((1024 // tile) ** 2) in das, das
+    _, das = compile_one(8192, 4096, 4096)
+    assert "split-k" not in das and das.count("== sub-kernel") == 1, das
+    monkeypatch.setenv("DVM_CUBE_SPLITK", "0")
+    _, das = compile_one(1024, 1024, 16384)
+    assert "split-k" not in das and das.count("== sub-kernel") == 1, das
+    monkeypatch.setenv("DVM_CUBE_SPLITK", "3")
+    t, das = compile_one(256, 256, 1000)
+    assert "split-k partials 3 x 384" in das and "split-k sum of 3" in das, das
+
+
 def test_matmul_tile_follows_problem_size():
     for (m, n), tile in (((8192, 4096), 256), ((2048, 2048), 128), ((256, 256), 64)):
         t = Tester("mix", run_mode="das")

@@ -223,3 +223,29 @@ def test_epilogue_with_an_fp32_store_or_a_decision_stays_exact():
     t.run()
     assert "~" not in t.das(), t.das()
     assert np.allclose(t.output(o).astype(np.float64), np.where(np.exp(p16) > 1.0, p16, p16 * 0.5), rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.parametrize("tile", ["256", "128", "64"])
+@pytest.mark.parametrize("m,n", [(256 + 8, 512 + 16), (300, 520), (256, 264), (100, 300), (260, 257), (513, 1024)])
+@pytest.mark.parametrize("ta,tb", [(False, False), (False, True), (True, False)])
+def test_ragged_edge_tiles(monkeypatch, tile, m, n, ta, tb):
+    # A ragged tile at the bottom or right edge of an aligned product is moved back inside the output and multiplied
+    # like a full tile; its epilogue covers only the part no other tile writes. Shapes with one or both edges ragged,
+    # an extent below the tile (guarded path), n not a multiple of 8 (columns cannot move), every tile size; the
+    # epilogue reads a second [m, n] operand, so a row or column off by the shift would show.
+    monkeypatch.setenv("DVM_CUBE_TILE", tile)
+    monkeypatch.setenv("DVM_CUBE_SPLITK", "0")
+    k = 192
+    r = np.random.default_rng(m * 3 + n)
+    a16 = (r.standard_normal([k, m] if ta else [m, k]) / 8).astype(np.float16)
+    b16 = (r.standard_normal([n, k] if tb else [k, n]) / 8).astype(np.float16)
+    other = r.standard_normal([m, n]).astype(np.float32)
+    t = Tester("mix")
+    c = t.cast(t.matmul(t.load(a16), t.load(b16), ta, tb), "float32")
+    out = t.store(t.add(c, t.load(other)))
+    t.run()
+    a64, b64 = a16.astype(np.float64), b16.astype(np.float64)
+    prod = (a64.T if ta else a64) @ (b64.T if tb else b64)
+    got = t.output(out).astype(np.float64)
+    bound = 1e-5 + 2.0 ** -11 * np.abs(prod) * 1.01
+    assert (np.abs(got - (prod + other)) <= bound).all(), float(np.abs(got - (prod + other)).max())
