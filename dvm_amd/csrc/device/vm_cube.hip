@@ -171,20 +171,57 @@ struct Stage<ROWS, false, NTHR> {
   }
 };
 
-// Generic staging of one tile straight into local memory, element by element (edge tiles, odd
-// leading dimensions, unaligned operands). Slow, correct for every shape.
+// Generic staging of one tile straight into local memory (edge tiles, odd leading dimensions, unaligned
+// operands, a k axis that is no multiple of 64). The unit is a run of 8 elements that are consecutive in memory:
+// 8 k of one row (k contiguous) or 8 rows at one k (rows contiguous); a run that lies inside the operand and is
+// 16-byte aligned (vec_ok: leading dimension a multiple of 8 and an aligned base) is one 128-bit load, any other
+// run goes element by element and reads as zero outside the operand. Slow next to the tile loops, correct for
+// every shape.
 template <int ROWS, int NTHR>
 __device__ __attribute__((noinline)) void stage_generic(uint16_t *tile, uint64_t base, uint32_t ld, uint32_t row0, uint32_t k0,
-                                                        uint32_t rows, uint32_t kext, uint32_t k_contig, uint32_t tid) {
-  for (uint32_t e = tid; e < ROWS * BK; e += NTHR) {
-    const uint32_t row = e / BK, kk = e % BK;
-    const uint32_t gr = row0 + row, gk = k0 + kk;
-    uint16_t v = 0;
-    if (gr < rows && gk < kext) {
-      const uint64_t idx = k_contig ? static_cast<uint64_t>(gr) * ld + gk : static_cast<uint64_t>(gk) * ld + gr;
-      v = reinterpret_cast<const DVM_GLOBAL uint16_t *>(base)[idx];
+                                                        uint32_t rows, uint32_t kext, uint32_t k_contig, uint32_t vec_ok, uint32_t tid) {
+  const DVM_GLOBAL uint16_t *src = reinterpret_cast<const DVM_GLOBAL uint16_t *>(base);
+  if (k_contig) {
+    for (uint32_t c = tid; c < ROWS * (BK / 8); c += NTHR) {
+      const uint32_t row = c >> 3, kc = c & 7u;
+      const uint32_t gr = row0 + row, gk = k0 + kc * 8u;
+      vu4 v = {0u, 0u, 0u, 0u};
+      if (gr < rows && gk < kext) {
+        const uint64_t idx = static_cast<uint64_t>(gr) * ld + gk;
+        if (vec_ok != 0u && gk + 8u <= kext) {
+          v = *reinterpret_cast<const DVM_GLOBAL vu4 *>(src + idx);
+        } else {
+#pragma unroll
+          for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t e = gk + j < kext ? src[idx + j] : 0u;
+            v[j >> 1] |= e << (16u * (j & 1u));
+          }
+        }
+      }
+      *reinterpret_cast<vu4 *>(tile + tile_off(row, kc)) = v;
     }
-    tile[tile_off(row, kk >> 3) + (kk & 7u)] = v;
+  } else {
+    // consecutive lanes take consecutive runs of rows at one k: neighbouring 16 bytes of memory
+    const uint32_t row_vec = vec_ok != 0u && (row0 & 7u) == 0u ? 1u : 0u;
+    for (uint32_t c = tid; c < (ROWS / 8) * BK; c += NTHR) {
+      const uint32_t rb = c % (ROWS / 8), kk = c / (ROWS / 8);
+      const uint32_t gr = row0 + rb * 8u, gk = k0 + kk;
+      vu4 v = {0u, 0u, 0u, 0u};
+      if (gr < rows && gk < kext) {
+        const uint64_t idx = static_cast<uint64_t>(gk) * ld + gr;
+        if (row_vec != 0u && gr + 8u <= rows) {
+          v = *reinterpret_cast<const DVM_GLOBAL vu4 *>(src + idx);
+        } else {
+#pragma unroll
+          for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t e = gr + j < rows ? src[idx + j] : 0u;
+            v[j >> 1] |= e << (16u * (j & 1u));
+          }
+        }
+      }
+#pragma unroll
+      for (uint32_t j = 0; j < 8; ++j) tile[tile_off(rb * 8u + j, kk >> 3) + (kk & 7u)] = static_cast<uint16_t>(v[j >> 1] >> (16u * (j & 1u)));
+    }
   }
 }
 
@@ -1176,9 +1213,11 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       __syncthreads();
      }
     } else {
+      const uint32_t a_vec = ((h.lda & 7u) == 0u && (a_base & 15u) == 0u) ? 1u : 0u;
+      const uint32_t b_vec = ((h.ldb & 7u) == 0u && (b_base & 15u) == 0u) ? 1u : 0u;
       for (uint32_t kt = 0; kt < nk; ++kt) {
-        stage_generic<BM, NTHR>(lds, a_base, h.lda, m0, k_lo + kt * BK, h.m, k_hi, A_KC ? 1u : 0u, tid);
-        stage_generic<BN, NTHR>(lds + kBBase, b_base, h.ldb, n0, k_lo + kt * BK, h.n, k_hi, B_KC ? 1u : 0u, tid);
+        stage_generic<BM, NTHR>(lds, a_base, h.lda, m0, k_lo + kt * BK, h.m, k_hi, A_KC ? 1u : 0u, a_vec, tid);
+        stage_generic<BN, NTHR>(lds + kBBase, b_base, h.ldb, n0, k_lo + kt * BK, h.n, k_hi, B_KC ? 1u : 0u, b_vec, tid);
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < BK / 16; ++kk) {

@@ -205,7 +205,7 @@ void Compiler::CompileCube(int a) {
   // src/xkernel.cc:1511-1547; here the reason is to fill the chip). Every candidate (tile, parts) gets an estimate
   // from figures measured on MI355X (bf16, microseconds): a workgroup's time per 64 k (2.2 for the 256 tile, 1.3 for
   // 128, 0.71 for 64 alone on its compute unit and 0.9 when two share one; the guarded path of ragged or unaligned
-  // tiles takes about six times as long), rounds of workgroups over the chip, and for a split the second launch plus
+  // tiles takes about two and a half times as long), rounds of workgroups over the chip, and for a split the second launch plus
   // the time its one workgroup per tile needs per partial tile (8.5 / 4.5 / 0.55: a single workgroup streams at
   // some 30 GB/s), which is what keeps deep splits of big tiles from paying.
   uint32_t k_split = 1, k_chunk = 0;
@@ -236,7 +236,7 @@ void Compiler::CompileCube(int a) {
         // (ragged edge tiles of an aligned product are moved back inside the output and stay on the vector path)
         const bool m_fast = M % t == 0 || (M >= t && (!mm->trans_a || M % 8 == 0));
         const bool n_fast = N % t == 0 || (N >= t && N % 8 == 0);
-        const double slow = (aligned && m_fast && n_fast) ? 1.0 : 6.0;
+        const double slow = (aligned && m_fast && n_fast) ? 1.0 : 2.5;
         for (uint32_t want = 1; want <= max_split; want = want < 2 ? 2 : want * 2) {
           uint32_t chunk = 0;
           const uint32_t parts = parts_of(want, &chunk);
