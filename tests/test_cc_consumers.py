@@ -46,6 +46,25 @@ def test_blob_fixture_is_what_the_host_compiler_emits_today():
     assert blob == committed, "the bytecode changed: run python tests/golden/make_blob_fixture.py"
 
 
+def test_makefile_runs_the_commands_of_the_python_build():
+    # the make-style entry (DVM_ARCH=hip) compiles every source dvm_amd.build compiles, with the same flags, into the
+    # same objects: compare the command lines of a dry run from scratch
+    repo = os.path.dirname(HERE)
+    r = subprocess.run(["make", "-n", "-B", "all", "consumers"], cwd=repo, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    lines = [l for l in r.stdout.splitlines() if l.startswith(("hipcc", "g++"))]
+    compiled = sorted(l.split(" -c ")[1].split(" -o ")[0] + (" u4" if "-DDVM_VEC_U=4" in l else "") for l in lines if " -c " in l)
+    want = sorted(os.path.relpath(s, repo) for s in dvm_build._sources("device", ".hip") + dvm_build._sources("host", ".cc"))
+    want = sorted(want + ["dvm_amd/csrc/device/vm_vector.hip u4"])
+    assert compiled == want
+    for flag in dvm_build.HIP_FLAGS:
+        assert all(flag in l for l in lines if l.startswith("hipcc") and " -c " in l), flag
+    for flag in dvm_build.HOST_FLAGS:
+        assert all(flag in l for l in lines if l.startswith("g++") and " -c " in l), flag
+    r = subprocess.run(["make", "-n", "DVM_ARCH=gpu"], cwd=repo, capture_output=True, text=True)
+    assert r.returncode != 0 and "hip" in r.stderr
+
+
 @pytest.mark.gpu
 def test_cpp_consumer_of_dvm_h():
     r = subprocess.run([_binary("muladd")], capture_output=True, text=True, timeout=100)

@@ -474,3 +474,32 @@ def test_lazy_unified_workspace():  # :906-917
                                                      np.sum(a * np.float32(1.5), (0,), keepdims=True) + 0.1, None)])
     finally:
         Tester.set_deterministic(False)
+
+
+def test_product_plus_a_strided_view():  # :793-806: the epilogue reads a [1024, 512] window of a [1024, 1000] buffer
+    rng = np.random.default_rng(793)
+    a = rng.normal(0, 0.01, [1024, 1024]).astype(np.float16)
+    b = rng.normal(0, 0.01, [1024, 512]).astype(np.float16)
+    c = rng.normal(0, 1, [1024, 1000]).astype(np.float16)
+    t = Tester("eager")
+    x2 = t.matmul(t.load(a), t.load(b), False, False)
+    x4 = t.add(x2, t.view_load([1024, 512], [1000, 1], c))
+    t.store_expect(x4, np.matmul(a.astype(np.float32), b.astype(np.float32)).astype(np.float16) + c[:, :512])
+    assert t.run_check()
+    assert t.num_launches() == 1, t.das()
+
+
+def test_lazy_tuning_switch_is_accepted():  # :371-385: the same product three times on one kernel object, tuner on
+    rng = np.random.default_rng(371)
+    a = rng.normal(0, 0.01, [4096, 4096]).astype(np.float16)
+    b = rng.normal(0, 0.01, [4096, 4096]).astype(np.float16)
+    expect = np.matmul(a.astype(np.float32), b.astype(np.float32))
+    t = Tester("eager")
+    Tester.set_lazy_tuning(True)
+    try:
+        for _ in range(3):
+            t.store_expect(t.matmul(t.load(a), t.load(b), False, False), expect, 1e-3)
+            assert t.run_check()
+            t.reset()
+    finally:
+        Tester.set_lazy_tuning(False)

@@ -249,3 +249,27 @@ def test_ragged_edge_tiles(monkeypatch, tile, m, n, ta, tb):
     got = t.output(out).astype(np.float64)
     bound = 1e-5 + 2.0 ** -11 * np.abs(prod) * 1.01
     assert (np.abs(got - (prod + other)) <= bound).all(), float(np.abs(got - (prod + other)).max())
+
+
+@pytest.mark.parametrize("mix", [False, True])
+def test_dyn_shape_tuning(mix):  # tests/ut/test_matmul.py:697-718: a dynamic kernel run three times with the tuner switched on
+    Tester.set_lazy_tuning(True)
+    try:
+        t = Tester("mix:dyn")
+        x0, x1 = t.load([], "float16"), t.load([], "float16")
+        x2 = t.matmul(x0, x1, False, False)
+        rng = np.random.default_rng(697)
+        a = rng.normal(0, 0.01, [4096, 4096]).astype(np.float16)
+        b = rng.normal(0, 0.01, [4096, 4096]).astype(np.float16)
+        expect = np.matmul(a.astype(np.float32), b.astype(np.float32))
+        if mix:
+            x2 = t.add(x2, 0.1)
+            expect = expect + 0.1
+        x3 = t.store(x2)
+        for _ in range(3):
+            t.input(x0, a)
+            t.input(x1, b)
+            t.run()
+            assert t.check(x3, expect, 2e-3)
+    finally:
+        Tester.set_lazy_tuning(False)
