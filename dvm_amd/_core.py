@@ -53,6 +53,9 @@ def _load():
         "dvm_rt_copy": (vp, [vp, vp]),
         "dvm_rt_matmul": (vp, [vp, vp, vp, ci, ci, vp]),
         "dvm_rt_set_store_inplace": (ci, [vp, vp]),
+        "dvm_rt_set_store_temp": (ci, [vp, vp]),
+        "dvm_rt_set_load_bind": (ci, [vp, vp, vp]),
+        "dvm_rt_spec_next": (ci, [vp]),
         "dvm_rt_view_load": (vp, [vp, vp, vp, ci]),
         "dvm_rt_slice_load": (vp, [vp, vp, vp, vp, ci]),
         "dvm_rt_stridedslice_load": (vp, [vp, vp, vp, vp, vp, ci]),
@@ -263,6 +266,18 @@ class Kernel:
 
     def set_store_inplace(self, store):
         _check(_lib.dvm_rt_set_store_inplace(self._rt, store._h))
+
+    def set_store_temp(self, store):
+        """The store is no output of the kernel, only what loads bound to it read (KernelPy.set_store_temp)."""
+        _check(_lib.dvm_rt_set_store_temp(self._rt, store._h))
+
+    def set_load_bind(self, load, store):
+        """The load reads what `store` (a store of this kernel) writes; call it before the load's first use."""
+        _check(_lib.dvm_rt_set_load_bind(self._rt, load._h, store._h))
+
+    def spec_next(self):
+        """Stage marker of a kernel created as "vector:spec" (RtKernelPy.spec_next)."""
+        _check(_lib.dvm_rt_spec_next(self._rt))
 
     # -- strided views (include/dvm_py.h view_load / slice_load / stridedslice_load); innermost stride 1 --
     def view_load(self, shape, stride, type):

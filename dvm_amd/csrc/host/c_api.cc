@@ -160,6 +160,10 @@ void ParseKernelType(const std::string &s, KernelType *type, uint32_t *flags) {
       *flags |= kUnifyWS;
     } else if (f == "lazy") {
       *flags |= kLazyCodeGen;
+    } else if (f == "spec" && *type == kVector) {
+      *flags |= kSpeculate;
+    } else if (f == "priv1" && *type == kVector) {  // with "spec": the stages are found automatically (no SpecNext calls)
+      *flags |= kPrivate1;
     } else if (!f.empty()) {
       throw std::runtime_error("DVM EXCEPTION. reason: kernel flag '" + f + "' is not supported by the gfx950 backend");
     }
@@ -570,6 +574,33 @@ int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store) {
       -1);
 }
 
+int dvm_rt_set_store_temp(dvm_rt *rt, dvm_obj *store) {
+  return Guard(
+      [&]() {
+        rt->kernel.SetStoreTemp(Obj(store));
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_set_load_bind(dvm_rt *rt, dvm_obj *load, dvm_obj *store) {
+  return Guard(
+      [&]() {
+        rt->kernel.SetLoadBind(Obj(load), Obj(store));
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_spec_next(dvm_rt *rt) {
+  return Guard(
+      [&]() {
+        rt->kernel.SpecNext();
+        return 0;
+      },
+      -1);
+}
+
 int dvm_obj_rank(const dvm_obj *o) { return reinterpret_cast<const NDObject *>(o)->rank(); }
 
 int dvm_obj_shape(const dvm_obj *o, int64_t *dims, size_t cap) {
@@ -644,6 +675,7 @@ int dvm_rt_codegen(dvm_rt *rt) {
         const auto t1 = std::chrono::steady_clock::now();
         // outputs take their size from the inferred shapes
         for (NDObject *s : rt->stores) {
+          if (s->temp) continue;  // SetStoreTemp: no output of the kernel
           auto ext = rt->store_extent.find(s);
           if (ext != rt->store_extent.end()) {
             // a strided store writes part of a larger buffer, which starts out as zeros
@@ -664,6 +696,7 @@ int dvm_rt_codegen(dvm_rt *rt) {
         relocs.reserve(rt->buffers.size());
         for (auto &kv : rt->buffers) relocs.emplace_back(kv.first, kv.second.ptr);
         for (NDObject *l : rt->loads) {
+          if (l->bound != nullptr) continue;  // SetLoadBind: reads a value of the kernel, not memory of the caller
           if (rt->buffers.find(l) == rt->buffers.end()) throw std::runtime_error("DVM EXCEPTION. reason: a load has no input bound");
         }
         const auto t2 = std::chrono::steady_clock::now();

@@ -191,7 +191,11 @@ class Builder {
     NDObject *o = new NDObject(kind, t);
     // A Store handed on as an operand (a later stage of a sequence kernel reading an earlier stage's
     // output, tests/ut/test_sequence_fusion.py:190-197) stands for the value it stores.
-    auto value_of = [](NDObject *x) { return x != nullptr && x->kind == kObjStore ? x->in[0] : x; };
+    // A Load bound to a Store by SetLoadBind reads what that Store writes: inside one kernel that is the value itself.
+    auto value_of = [](NDObject *x) {
+      if (x != nullptr && x->kind == kObjLoad && x->bound != nullptr) x = x->bound;
+      return x != nullptr && x->kind == kObjStore ? x->in[0] : x;
+    };
     o->in[0] = value_of(a);
     o->in[1] = value_of(b);
     o->in[2] = value_of(c);
@@ -490,6 +494,8 @@ void Kernel::Clone(const Kernel &base, CloneHelper &helper) {
     c->trans_a = o->trans_a;
     c->trans_b = o->trans_b;
     c->inplace = o->inplace;
+    c->temp = o->temp;
+    c->bound = o->bound != nullptr ? helper.GetClone(o->bound) : nullptr;
     c->noloss_cast = o->noloss_cast;
     c->nin = o->nin;
     for (int i = 0; i < o->nin; ++i) c->in[i] = helper.GetClone(o->in[i]);
@@ -589,8 +595,23 @@ NDObject *Kernel::Store(void *addr, NDObject *input, IntArrayRef *stride) {
 
 NDObject *Kernel::PadStore(void *, NDObject *, int64_t) { Unsupported("PadStore"); }
 void Kernel::SetStoreInplace(NDObject *store) { store->inplace = true; }
-void Kernel::SetStoreTemp(NDObject *) { Unsupported("SetStoreTemp"); }
-void Kernel::SetLoadBind(NDObject *, NDObject *) { Unsupported("SetLoadBind"); }
+// A temporary Store and a Load bound to it hand a value from one part of a kernel to a later one through memory in
+// the reference (src/dvm.cc:1583-1588). Here operators read the value directly (the launches are cut at code
+// generation, and a value that crosses a cut gets its workspace there), so the bound Load stands for the stored value
+// in every operator built after the binding, and a temporary Store that nothing else needs is dropped as dead code.
+void Kernel::SetStoreTemp(NDObject *store) {
+  if (store == nullptr || store->kind != kObjStore) Throw("SetStoreTemp needs a Store");
+  store->temp = true;
+}
+void Kernel::SetLoadBind(NDObject *load, NDObject *access) {
+  if (load == nullptr || load->kind != kObjLoad || load->strided) Throw("SetLoadBind needs a plain Load");
+  if (access == nullptr || access->kind != kObjStore) Throw("SetLoadBind binds a Load to a Store of the same kernel");
+  if (load->type_id_ != access->type_id_) Throw("SetLoadBind: the Load and the Store differ in type");
+  for (NDObject *o : kernel_->ops_)
+    for (int i = 0; i < o->nin; ++i)
+      if (o->in[i] == load) Throw("SetLoadBind must come before the first use of the Load");
+  load->bound = access;
+}
 
 NDObject *Kernel::_Unary(int op_type, NDObject *input) {
   if (op_type < 0 || op_type >= kUnaryTypeEnd) return nullptr;
@@ -771,7 +792,14 @@ NDObject *Kernel::AllGather(NDObject *, const Comm *) { Unsupported("AllGather (
 NDObject *Kernel::AllGatherV2(NDObject *, const Comm *) { Unsupported("AllGatherV2 (single-GPU backend)"); }
 NDObject *Kernel::ReduceScatter(NDObject *, const Comm *) { Unsupported("ReduceScatter (single-GPU backend)"); }
 NDObject *Kernel::ExtOut(NDObject *, int) { Unsupported("ExtOut"); }
-void Kernel::SpecNext() { Unsupported("speculative kernels"); }
+// Stage boundary of a speculative vector kernel (kVector with kSpeculate). The reference tries to keep a reduce and its
+// consumers in one kernel and falls back to a cut one when the reduced extent does not fit a tile
+// (src/kernel.cc:2265-2578); the stage marker tells it where the cut would be. Here every vector kernel is compiled
+// that way (a reduce and its consumers are consecutive sweeps of one launch whenever the schedule allows, separate
+// launches otherwise), so the marker carries no information.
+void Kernel::SpecNext() {
+  if (!(kernel_->Flags() & kSpeculate)) Throw("SpecNext needs a kernel created with kSpeculate");
+}
 
 // Parallel and sequence kernels (src/xkernel.h, include/dvm.h:248-251 of the reference): the caller
 // names the groups, every group becomes one or more launches of its own. The sub-kernel type and the

@@ -64,6 +64,8 @@ class NDObject {
   bool keepdims = false;
   bool trans_a = false, trans_b = false;
   bool inplace = false;
+  bool temp = false;            // a Store marked by SetStoreTemp: no output of the kernel, only what bound loads read
+  NDObject *bound = nullptr;    // a Load bound to a Store of the same kernel by SetLoadBind: it reads the stored value
   bool noloss_cast = false;
   int nin = 0;
   NDObject *in[3] = {nullptr, nullptr, nullptr};

@@ -14,7 +14,7 @@ namespace dvm {
 void Compiler::MarkLive() {
   for (int i = n_ - 1; i >= 0; --i) {
     NDObject *o = k_->ops_[i];
-    if (o->kind == kObjStore) live_[i] = 1;
+    if (o->kind == kObjStore && !o->temp) live_[i] = 1;
     if (!live_[i]) continue;
     for (int j = 0; j < o->nin; ++j)
       if (o->in[j] != nullptr) live_[o->in[j]->id] = 1;

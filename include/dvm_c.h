@@ -61,6 +61,13 @@ dvm_obj *dvm_rt_reduce(dvm_rt *rt, int reduce_type, dvm_obj *x, dvm_shape *dims,
 dvm_obj *dvm_rt_copy(dvm_rt *rt, dvm_obj *x);
 dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int trans_b, dvm_obj *bias);
 int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store);
+// Kernel::SetStoreTemp / SetLoadBind / SpecNext (include/dvm.h:352-353, 544 of the reference; KernelPy set_store_temp /
+// set_load_bind, include/dvm_py.h:207-208, RtKernelPy spec_next): a Store that is no output of the kernel, a Load that
+// reads what a Store of the same kernel writes (bind before the Load's first use), the stage marker of a kernel
+// created as "vector:spec".
+int dvm_rt_set_store_temp(dvm_rt *rt, dvm_obj *store);
+int dvm_rt_set_load_bind(dvm_rt *rt, dvm_obj *load, dvm_obj *store);
+int dvm_rt_spec_next(dvm_rt *rt);
 // Strided views (Kernel::Load / Store with a stride list, SliceLoad, StridedSliceLoad: include/dvm.h:195-201, 214 of the
 // reference; KernelPy view_load / slice_load / stridedslice_load, include/dvm_py.h). Strides are in elements, the
 // innermost one may be anything (0 broadcasts, 1 is the fast path, others go element by element). A view store writes into a zero-initialised buffer of extent_elems elements;
