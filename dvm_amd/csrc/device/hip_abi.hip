@@ -14,6 +14,8 @@
 extern "C" __global__ void dvm_vm_vec_pw(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_rx(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_ry(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_rx_parts(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_ry_parts(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_pw_u4(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_rx_u4(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_ry_u4(const VmParam p);
@@ -121,7 +123,8 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
   g_dev.lds_per_wg = static_cast<uint32_t>(prop.sharedMemPerBlock);
   // gfx950 lets one workgroup use the CU's whole 160 KB; the kernels must opt in.
   std::vector<const void *> kernels = {reinterpret_cast<const void *>(dvm_vm_vec_pw), reinterpret_cast<const void *>(dvm_vm_vec_rx),
-                                       reinterpret_cast<const void *>(dvm_vm_vec_ry),
+                                       reinterpret_cast<const void *>(dvm_vm_vec_ry), reinterpret_cast<const void *>(dvm_vm_vec_rx_parts),
+                                       reinterpret_cast<const void *>(dvm_vm_vec_ry_parts),
                                        reinterpret_cast<const void *>(dvm_vm_vec_pw_u4), reinterpret_cast<const void *>(dvm_vm_vec_rx_u4),
                                        reinterpret_cast<const void *>(dvm_vm_vec_ry_u4)};
   for (const auto &tile : kCubeKernels)
@@ -188,6 +191,16 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
     }
     const bool wide = (h->sched & VS_WIDE) != 0;
     if (wide && threads > 512) return static_cast<int>(hipErrorInvalidValue);
+    // a reduce shared between workgroups: its parts are the outermost kept axis and cover the reduced index space
+    const bool parts = h->r_chunk != 0;
+    if (parts) {
+      const uint32_t kind = h->sched & VS_KIND_MASK;
+      if (wide || (kind != VS_REDX && kind != VS_REDY) || h->k_per_chunk == 0 || h->n_kidx % h->k_per_chunk != 0 || h->n_kdim == 0 ||
+          h->kdims[h->n_kdim - 1].extent != h->n_kidx / h->k_per_chunk ||
+          static_cast<uint64_t>(h->r_chunk) * (h->n_kidx / h->k_per_chunk) < h->n_ridx) {
+        return static_cast<int>(hipErrorInvalidValue);
+      }
+    }
     {
       // local memory the interpreter will touch: reduce scratch, V registers, rounds parked by a load
       const uint64_t u = wide ? DVM_VEC_U_WIDE : 2;
@@ -210,10 +223,10 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
         hipLaunchKernelGGL(wide ? dvm_vm_vec_pw_u4 : dvm_vm_vec_pw, dim3(block_dim), dim3(threads), lds_bytes, s, p);
         break;
       case VS_REDX:
-        hipLaunchKernelGGL(wide ? dvm_vm_vec_rx_u4 : dvm_vm_vec_rx, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        hipLaunchKernelGGL(parts ? dvm_vm_vec_rx_parts : (wide ? dvm_vm_vec_rx_u4 : dvm_vm_vec_rx), dim3(block_dim), dim3(threads), lds_bytes, s, p);
         break;
       case VS_REDY:
-        hipLaunchKernelGGL(wide ? dvm_vm_vec_ry_u4 : dvm_vm_vec_ry, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        hipLaunchKernelGGL(parts ? dvm_vm_vec_ry_parts : (wide ? dvm_vm_vec_ry_u4 : dvm_vm_vec_ry), dim3(block_dim), dim3(threads), lds_bytes, s, p);
         break;
       default:
         return static_cast<int>(hipErrorInvalidValue);

@@ -894,7 +894,9 @@ __device__ __forceinline__ float uniform_cast(uint32_t sub, float x) {
   return x != 0.0f ? 1.0f : 0.0f;
 }
 
-template <int SCHED>
+// PARTS: the program's reduce is shared between workgroups (VVecHeader::r_chunk); a build of its own, so that the
+// programs without one pay nothing for the part bounds.
+template <int SCHED, bool PARTS = false>
 __device__ __forceinline__ void vm_vector(const VmParam &p) {
   // The blob arrives as a kernel argument; decoding from there would cost a
   // dependent scalar-memory round trip per access, so each workgroup copies it
@@ -916,7 +918,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   }
   // the scalar fields of the header live in scalar registers; the axis tables stay in local memory
   struct {
-    uint32_t n_kdim, n_rdim, team_log2, team_is_block, n_kidx, n_ridx, inner_extent, n_items, mem_off, code_off, n_vslot;
+    uint32_t n_kdim, n_rdim, team_log2, team_is_block, n_kidx, n_ridx, inner_extent, n_items, mem_off, code_off, n_vslot, r_chunk, k_per_chunk;
     const VDim *kdims, *rdims;
   } h;
   {
@@ -932,6 +934,8 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     h.mem_off = uni(hp->mem_off);
     h.code_off = uni(hp->code_off);
     h.n_vslot = uni(hp->n_vslot);
+    h.r_chunk = uni(hp->r_chunk);
+    h.k_per_chunk = uni(hp->k_per_chunk);
     h.kdims = hp->kdims;
     h.rdims = hp->rdims;
   }
@@ -960,7 +964,9 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   } else {
     k_local = tid & ((1u << tlog) - 1u); r_local = tid >> tlog; k_per_wg = 1u << tlog; r_step = nthreads >> tlog;
   }
-  const uint32_t n_rounds = SCHED == VS_POINTWISE ? 1u : (h.n_ridx + r_step * U - 1) / (r_step * U);
+  // (a reduce shared between workgroups: a lane walks one part of the reduced index space, r_chunk indices long)
+  const uint32_t r_span = PARTS ? h.r_chunk : h.n_ridx;
+  const uint32_t n_rounds = SCHED == VS_POINTWISE ? 1u : (r_span + r_step * U - 1) / (r_step * U);
   constexpr bool inner_red = SCHED == VS_REDX;
 
   SRegs sr;
@@ -978,6 +984,12 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     // position of the lane in the kept space (POINTWISE: of slab 0; slab u is nthreads further each)
     const uint32_t kidx = item * k_per_wg + k_local;
     const bool kvalid = kidx < h.n_kidx;
+    // first index of the lane's part of the reduced index space, and the index behind its last
+    uint32_t r_base = 0, r_lim = h.n_ridx;
+    if constexpr (PARTS) {
+      r_base = (kidx / h.k_per_chunk) * h.r_chunk;
+      r_lim = (r_base + r_span < h.n_ridx) ? r_base + r_span : h.n_ridx;
+    }
     uint32_t nvp_out;  // valid counts outside sweeps
     if constexpr (SCHED == VS_POINTWISE) {
       nvp_out = 0;
@@ -999,7 +1011,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     Slabs sl = sl_out;  // valid counts of the current round's slabs (outside sweeps: of the lane's output)
     uint32_t round = 0, sweep_pc = 0, slot_kinds = 0;
     bool sweep_rev = false;   // the sweep walks its rounds last to first (VSW_REVERSE)
-    uint32_t ridx = r_local;  // reduce-space index of slab 0 in the current round
+    uint32_t ridx = r_base + r_local;  // reduce-space index of slab 0 in the current round
     Offs last_off;            // element offsets of the last memory instruction (VI_SAME_OFFS reuses them)
     FOR_U last_off.v[u] = 0;
 
@@ -1050,7 +1062,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               uint32_t nvp = 0;
               FOR_U {
                 const uint32_t ru = ridx + u * r_step;
-                const bool ok = kvalid && ru < h.n_ridx;
+                const bool ok = kvalid && ru < r_lim;
                 uint32_t nv = inner_red ? group_valid(ok ? ru : 0u, h.rdims, h.n_rdim, h.inner_extent) : (nvp_out & 0xfu);
                 nv &= ok ? 0xfu : 0u;
                 nvp |= nv << (4 * u);
@@ -1237,7 +1249,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                 off.v[u] = koff;
                 if (in_sweep) {
                   const uint32_t ru = ridx + u * r_step;
-                  off.v[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+                  off.v[u] += space_offset(ru < r_lim ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
                 }
               }
             }
@@ -1272,7 +1284,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                   uint32_t nvp2 = 0;
                   FOR_U {
                     const uint32_t ru = ridx2 + u * r_step;
-                    const bool ok = kvalid && ru < h.n_ridx;
+                    const bool ok = kvalid && ru < r_lim;
                     off2.v[u] = koff + space_offset(ok ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
                     uint32_t nv = inner_red ? group_valid(ok ? ru : 0u, h.rdims, h.n_rdim, h.inner_extent) : (nvp_out & 0xfu);
                     nv &= ok ? 0xfu : 0u;
@@ -1472,7 +1484,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                 off.v[u] = koff;
                 if (in_sweep) {
                   const uint32_t ru = ridx + u * r_step;
-                  off.v[u] += space_offset(ru < h.n_ridx ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
+                  off.v[u] += space_offset(ru < r_lim ? ru : 0u, h.rdims, h.n_rdim, m.rstride, inner_red);
                 }
               }
             }
@@ -1554,7 +1566,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             red_init<SCHED>(racc0, slot_kinds & 0xfu);
             red_init<SCHED>(racc1, (slot_kinds >> 4) & 0xfu);
             sweep_rev = SCHED == VS_REDX && (sub & VSW_REVERSE) != 0;
-            ridx = r_local + (sweep_rev ? (n_rounds - 1u) * r_step * U : 0u);
+            ridx = r_base + r_local + (sweep_rev ? (n_rounds - 1u) * r_step * U : 0u);
             break;
           }
           case VOP_FIN: {
@@ -1594,4 +1606,6 @@ extern "C" __global__ void __launch_bounds__(512) dvm_vm_vec_ry_u4(const VmParam
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_pw(const VmParam p) { vm_vector<VS_POINTWISE>(p); }
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_rx(const VmParam p) { vm_vector<VS_REDX>(p); }
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_ry(const VmParam p) { vm_vector<VS_REDY>(p); }
+extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_rx_parts(const VmParam p) { vm_vector<VS_REDX, true>(p); }
+extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_ry_parts(const VmParam p) { vm_vector<VS_REDY, true>(p); }
 #endif

@@ -157,6 +157,36 @@ class Compiler {
   size_t RunOnce(int mode);
 
  private:
+  size_t RunModes();
+
+  // ---------- reduces shared between workgroups ----------
+  // A reduce with few outputs gives the schedules few workgroups (one per output, or per 512 outputs along the
+  // innermost axis): a column sum of a [4096, 4096] tensor would run on 8 of 256 compute units, a sum of a whole
+  // tensor on one. The reference adds partial results across blocks with atomics (src/vm_gpu.cu:750-939); here, to
+  // keep results the same on every run, such a reduce R = reduce(x, dims) becomes, for the duration of one code
+  // generation, R' = the same reduce over each of S parts of the reduced index space (one more, outermost, dim of
+  // extent S on its result: a kept axis that no input has) and reduce(R', dim 0), which every consumer of R reads.
+  // Only reduces whose consumers work on the reduce's own output shape qualify (a consumer that walks x again would
+  // be as short of workgroups in the second launch). SplitLongReduces rewrites the operator list and returns true
+  // if it changed anything; UndoSplitReduces restores it and renumbers the operators the programs refer to.
+  bool SplitLongReduces();
+  void UndoSplitReduces(bool keep_programs);
+  struct SplitRecord {
+    NDObject *reduce;     // the user's reduce (holds part_split and the longer shape meanwhile)
+    NDObject *second;     // the synthetic reduce over the parts (owned here)
+    int64_t shape[kMaxRank];
+    size_t rank;
+    IntArrayRef axis0;    // {0}: what `second` reduces over
+    int64_t zero = 0;
+  };
+  std::vector<SplitRecord *> splits_;
+  struct Repoint {
+    NDObject *consumer;
+    int slot;
+    NDObject *was;
+  };
+  std::vector<Repoint> repoints_;
+  std::vector<NDObject *> saved_ops_;
   VKernel *k_;
   int n_;
   std::vector<int> area_, ws_slot_, store_of_, level_;
@@ -174,6 +204,7 @@ class Compiler {
     int red_at_level[8] = {0, 0, 0, 0, 0, 0, 0, 0};  // reduces per sweep: the interpreter has two reduce slots per sweep
     int stage = 0;  // the caller's group (parallel / sequence kernels); operators of different groups never share a launch
     int n_ops = 0;  // operators joined so far (a program has room for about 500 instruction words and 160 nodes)
+    bool has_part = false;  // holds a reduce shared between workgroups: only operators of its input's index space join
   };
   std::vector<AreaInfo> areas_;
 

@@ -192,7 +192,9 @@ std::string &VKernel::DisAssemble() {
       os << "entry vector sched=" << sched[h->sched & VS_KIND_MASK] << ((h->sched & VS_WIDE) ? " wide" : "") << " blocks=" << p.grid << " threads=" << p.threads
          << " lds=" << p.lds_bytes << " items=" << h->n_items << " kept=" << h->n_kidx << " red=" << h->n_ridx
          << " inner=" << h->inner_extent << " team=" << (h->team_is_block ? p.threads : (1u << h->team_log2))
-         << " vslots=" << h->n_vslot << "\n";
+         << " vslots=" << h->n_vslot;
+      if (h->r_chunk != 0 && h->k_per_chunk != 0) os << " shared-reduce parts=" << h->n_kidx / h->k_per_chunk << " x " << h->r_chunk;
+      os << "\n";
       os << "  kdims:";
       for (uint32_t i = 0; i < h->n_kdim; ++i) os << " " << h->kdims[i].extent;
       os << "  rdims:";

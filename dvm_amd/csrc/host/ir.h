@@ -66,6 +66,8 @@ class NDObject {
   bool inplace = false;
   bool temp = false;            // a Store marked by SetStoreTemp: no output of the kernel, only what bound loads read
   NDObject *bound = nullptr;    // a Load bound to a Store of the same kernel by SetLoadBind: it reads the stored value
+  int part_split = 0;           // kObjReduce, during code generation only: the reduce is shared between workgroups, its result
+                                // has one more (outermost) dim that numbers the parts (Compiler::SplitLongReduces)
   bool noloss_cast = false;
   int nin = 0;
   NDObject *in[3] = {nullptr, nullptr, nullptr};
@@ -175,6 +177,7 @@ struct Tuning {
   int vec_pair = -1;   // DVM_VEC_PAIR=0: a load never takes the binary instruction behind it along
   int cube_tile = -1;   // DVM_CUBE_TILE=256|128|64
   int cube_waves = -1;  // DVM_CUBE_WAVES=4|8
+  int red_split = -1;    // DVM_RED_SPLIT=0: never share a reduce between workgroups; N >= 2: N parts whenever the graph allows
   int cube_splitk = -1;  // DVM_CUBE_SPLITK=0: never split the k axis; N >= 2: split it N ways whenever the shape allows
   int cube_exact = -1;  // DVM_CUBE_EXACT=1: never the hardware approximations of exp, log, sqrt, division in a matmul epilogue
   int attn_waves = -1;  // DVM_ATTN_WAVES=4

@@ -28,6 +28,7 @@ void Tuning::Read() {
   cube_waves = num("DVM_CUBE_WAVES");
   cube_exact = num("DVM_CUBE_EXACT");
   cube_splitk = num("DVM_CUBE_SPLITK");
+  red_split = num("DVM_RED_SPLIT");
   attn_waves = num("DVM_ATTN_WAVES");
   debug = std::getenv("DVM_DEBUG") != nullptr;
 }
@@ -37,8 +38,27 @@ void Tuning::Read() {
 // shapes, 2 additionally ends a sub-kernel after every reduce (the reference's rule), 3 gives
 // every operator its own sub-kernel.
 size_t Compiler::Run() {
+  // Reduces with few outputs and a long reduced extent are rewritten, for this code generation only, into a reduce
+  // per part of the reduced index space and a reduce over the parts; should that graph not compile, the kernel
+  // is compiled as it was built.
+  if (SplitLongReduces()) {
+    bool done = false;
+    size_t ws = 0;
+    try {
+      ws = RunModes();
+      done = true;
+    } catch (const std::runtime_error &) {
+    }
+    UndoSplitReduces(done);
+    if (done) return ws;
+  }
+  return RunModes();
+}
+
+size_t Compiler::RunModes() {
   n_ = static_cast<int>(k_->ops_.size());
-  for (int mode = k_->part_mode_; mode < 3; ++mode) {
+  const int first_mode = k_->part_mode_;
+  for (int mode = first_mode; mode < 3; ++mode) {
     try {
       const size_t ws = RunOnce(mode);
       k_->part_mode_ = mode;
@@ -47,7 +67,12 @@ size_t Compiler::Run() {
     }
   }
   k_->part_mode_ = 3;
-  return RunOnce(3);
+  try {
+    return RunOnce(3);
+  } catch (const std::runtime_error &) {
+    k_->part_mode_ = first_mode;  // (what failed may be the rewritten graph: the next attempt starts where this one did)
+    throw;
+  }
 }
 
 size_t Compiler::RunOnce(int mode) {

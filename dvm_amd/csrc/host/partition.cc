@@ -81,6 +81,14 @@ bool Compiler::CanJoin(int a, const NDObject *o) {
   if (ai.stage != o->stage) return false;
   // a store goes where the value it stores is computed (an operator's own output is never a reason to cut)
   if (IsStoreLike(o) && ai.attn < 0 && !ai.cube && area_[o->in[0]->id] == a) return true;
+  if (ai.has_part || (o->kind == kObjReduce && o->part_split != 0 && ai.has_reduce)) {
+    // beside a reduce shared between workgroups only its like and operators on its input's index space
+    if (o->kind == kObjReduce) {
+      if (!ai.has_part || o->part_split != ai.reduce->part_split) return false;
+    } else if (o->numel() != ai.reduce->in[0]->numel()) {
+      return false;
+    }
+  }
   if (o->kind == kObjReduce && LevelIn(a, o) < 8 && ai.red_at_level[LevelIn(a, o)] >= 2) return false;
   if (o->kind == kObjMatMul) return false;
   if (ai.n_ops >= kMaxAreaOps && !IsStoreLike(o)) return false;  // long graphs are cut into several launches
@@ -133,6 +141,7 @@ void Compiler::Join(int a, const NDObject *o) {
     if (!ai.has_reduce) {
       ai.has_reduce = true;
       ai.reduce = o;
+      ai.has_part = o->part_split != 0;
     }
     DomMerge(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
   }
@@ -196,6 +205,7 @@ void Compiler::Partition() {
         cut = true;
       }
       if (o->kind == kObjMatMul || v->kind == kObjConcat) cut = true;
+      if (v->kind == kObjReduce && v->part_split != 0) cut = true;  // the reduce over the parts is a launch of its own
       if (!fuse && v->kind == kObjReduce && !IsStoreLike(o)) cut = true;  // the reference's rule: a reduce ends its sub-kernel
       a = std::max(a, area_[v->id] + (cut ? 1 : 0));
     }
@@ -205,6 +215,166 @@ void Compiler::Partition() {
     Join(a, o);
   }
   n_areas_ = static_cast<int>(areas_.size());
+}
+
+// ---------- reduces shared between workgroups ----------
+bool Compiler::SplitLongReduces() {
+  const int forced = k_->tuning_.red_split;
+  if (forced == 0 || forced == 1) return false;
+  std::vector<NDObject *> &ops = k_->ops_;
+  const uint64_t cus = std::max<uint64_t>(g_system.core_num, 1);
+  struct Cand {
+    NDObject *r;
+    int split;
+  };
+  std::vector<Cand> cands;
+  for (NDObject *r : ops) {
+    if (r->kind != kObjReduce || r->in[0] == nullptr || r->aux_ref == nullptr) continue;
+    const NDObject *x = r->in[0];
+    const int xr = x->rank();
+    if (xr == 0 || r->rank() + 1 > kMaxRank) continue;
+    bool red[kMaxRank] = {false};
+    for (size_t j = 0; j < r->aux_ref->size; ++j) {
+      int64_t d = r->aux_ref->data[j];
+      if (d < 0) d += xr;
+      if (d >= 0 && d < xr) red[d] = true;
+    }
+    uint64_t n_red = 1, n_out = 1;
+    int kept_dims = 0, last = -1;
+    bool empty = false;
+    for (int d = 0; d < xr; ++d) {
+      const int64_t e = x->dim(d);
+      if (e <= 0) empty = true;
+      if (e == 1) continue;
+      last = d;
+      if (red[d]) {
+        n_red *= static_cast<uint64_t>(e);
+      } else {
+        n_out *= static_cast<uint64_t>(e);
+        ++kept_dims;
+      }
+    }
+    if (empty || last < 0 || n_red < 2 || kept_dims > DVM_VEC_MAXR - 1) continue;
+    int split = 0;
+    if (forced >= 2) {
+      split = forced;
+    } else {
+      // workgroups the schedules would give it: one per output when the innermost axis is reduced, else one per
+      // 64 lanes of 8 outputs along the innermost axis
+      const uint64_t wgs = red[last] ? n_out : (n_out + 511) / 512;
+      if (wgs >= cus) continue;
+      // worth a second launch only when a workgroup would have a quarter of a million elements to itself (measured:
+      // [32, 65536] summed along its rows takes 18 us in one launch and 24-29 us in two)
+      const uint64_t outs_per_wg = red[last] ? 1 : std::min<uint64_t>(n_out, 512);
+      if (n_red * outs_per_wg < (1u << 18)) continue;
+      uint64_t want = 2 * cus / wgs;
+      split = 1;
+      while (static_cast<uint64_t>(split) * 2 <= want && split < 256) split *= 2;
+      // a part is worth a workgroup's while: 32k elements
+      while (split > 1 && n_red / static_cast<uint64_t>(split) * outs_per_wg < 32768) split /= 2;
+    }
+    if (split < 2 || n_red < 2ull * static_cast<uint64_t>(split)) continue;
+    // every consumer works on the reduce's own output
+    bool ok = false;
+    for (const NDObject *c : ops) {
+      for (int j = 0; j < c->nin; ++j) {
+        if (c->in[j] != r) continue;
+        ok = true;
+        if (c->numel() != r->numel() || c->kind == kObjReduce || c->kind == kObjMatMul || c->kind == kObjConcatPart) split = 0;
+      }
+      for (const NDObject *part : c->parts)
+        if (part == r) split = 0;
+    }
+    if (ok && split >= 2) cands.push_back({r, split});
+  }
+  // reduces that would share a launch are shared alike or not at all
+  for (size_t i = 0; i < cands.size(); ++i) {
+    for (const NDObject *q : ops) {
+      if (q->kind != kObjReduce || q == cands[i].r || q->in[0] == nullptr || q->aux_ref == nullptr) continue;
+      if (!SameReduce(cands[i].r, q)) continue;
+      bool also = false;
+      for (const Cand &c : cands)
+        if (c.r == q && c.split == cands[i].split) also = true;
+      if (!also) cands[i].split = 0;
+    }
+  }
+  bool any = false;
+  for (const Cand &c : cands) any = any || c.split >= 2;
+  if (!any) return false;
+  saved_ops_ = ops;
+  std::vector<NDObject *> next;
+  next.reserve(ops.size() + cands.size());
+  for (NDObject *o : saved_ops_) {
+    next.push_back(o);
+    for (const Cand &c : cands) {
+      if (c.r != o || c.split < 2) continue;
+      SplitRecord *rec = new SplitRecord();
+      rec->reduce = o;
+      rec->rank = static_cast<size_t>(o->rank());
+      for (size_t d = 0; d < rec->rank; ++d) rec->shape[d] = o->dim(static_cast<int>(d));
+      rec->axis0.data = &rec->zero;
+      rec->axis0.size = 1;
+      NDObject *second = new NDObject(kObjReduce, o->type_id_);
+      second->op = o->op;
+      second->in[0] = o;
+      second->nin = 1;
+      second->aux_ref = &rec->axis0;
+      second->keepdims = false;
+      second->stage = o->stage;
+      second->SetShape(rec->shape, rec->rank);
+      rec->second = second;
+      int64_t longer[kMaxRank];
+      longer[0] = c.split;
+      for (size_t d = 0; d < rec->rank; ++d) longer[d + 1] = rec->shape[d];
+      o->SetShape(longer, rec->rank + 1);
+      o->part_split = c.split;
+      splits_.push_back(rec);
+      next.push_back(second);
+    }
+  }
+  for (NDObject *c : saved_ops_) {
+    for (int j = 0; j < c->nin; ++j) {
+      for (SplitRecord *rec : splits_) {
+        if (c->in[j] != rec->reduce) continue;
+        repoints_.push_back({c, j, c->in[j]});
+        c->in[j] = rec->second;
+      }
+    }
+  }
+  ops.swap(next);
+  for (size_t i = 0; i < ops.size(); ++i) ops[i]->id = static_cast<int>(i);
+  return true;
+}
+
+void Compiler::UndoSplitReduces(bool keep_programs) {
+  std::vector<NDObject *> during = k_->ops_;  // operator numbers the programs refer to
+  for (const Repoint &rp : repoints_) rp.consumer->in[rp.slot] = rp.was;
+  repoints_.clear();
+  for (SplitRecord *rec : splits_) {
+    rec->reduce->part_split = 0;
+    rec->reduce->SetShape(rec->shape, rec->rank);
+  }
+  k_->ops_ = saved_ops_;
+  saved_ops_.clear();
+  for (size_t i = 0; i < k_->ops_.size(); ++i) k_->ops_[i]->id = static_cast<int>(i);
+  if (keep_programs) {
+    auto renumber = [&](int &op_id) {
+      if (op_id < 0) return;
+      NDObject *o = during[static_cast<size_t>(op_id)];
+      for (SplitRecord *rec : splits_)
+        if (rec->second == o) Throw("a program addresses memory through a reduce over parts");
+      op_id = o->id;
+    };
+    for (Program &p : k_->programs_) {
+      for (Program::Patch &pt : p.patches) renumber(pt.op_id);
+      for (Program::Fill &f : p.fills) renumber(f.op_id);
+    }
+  }
+  for (SplitRecord *rec : splits_) {
+    delete rec->second;
+    delete rec;
+  }
+  splits_.clear();
 }
 
 // ---------- which values cross sub-kernels ----------

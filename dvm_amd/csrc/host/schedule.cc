@@ -169,7 +169,7 @@ void Compiler::UnifyAxes() {
           int64_t d = n.op->aux_ref->data[j];
           red[d < 0 ? d + x.rank : d] = true;
         }
-        int od = 0;
+        int od = n.op->part_split != 0 ? 1 : 0;  // (a reduce shared between workgroups: dim 0 numbers the parts)
         for (int d = 0; d < x.rank; ++d) {
           if (red[d]) {
             if (x.dims[d] != 1) reduced_var[Var(n.in[0], d)] = 1;
@@ -206,15 +206,17 @@ void Compiler::UnifyAxes() {
   // Reduces that share a sub-kernel have the same input shape and axes: their inputs walk the
   // same index space even when no operator relates them, so their dims are unified by position.
   {
-    int first = -1;
+    int first = -1, first_red = -1;
     for (int i = 0; i < nn_; ++i) {
       if (nodes_[i].kind != AK_REDUCE) continue;
       if (first < 0) {
         first = nodes_[i].in[0];
+        first_red = i;
         continue;
       }
       const ANode &x = nodes_[nodes_[i].in[0]], &f = nodes_[first];
       if (x.rank != f.rank) Fail("reduces of different rank in one sub-kernel");
+      if (nodes_[i].op->part_split != 0 && first_red >= 0 && nodes_[first_red].op->part_split != 0) Union(Var(i, 0), Var(first_red, 0));
       for (int d = 0; d < x.rank; ++d)
         if (x.dims[d] != 1 && x.dims[d] == f.dims[d]) Union(Var(nodes_[i].in[0], d), Var(first, d));
     }
@@ -336,6 +338,13 @@ void Compiler::OrderAndMerge() {
       outer |= 1u << n.axis[d];
     }
   }
+  // the axis that numbers the parts of a shared reduce lies outside every other axis
+  for (int i = 0; i < nn_; ++i) {
+    const ANode &n = nodes_[i];
+    if (n.kind != AK_REDUCE || n.op->part_split == 0 || n.axis[0] < 0) continue;
+    for (int ax = 0; ax < n_axes_; ++ax)
+      if (ax != n.axis[0]) axes_[ax].before |= 1u << n.axis[0];
+  }
   uint32_t placed = 0;
   for (int k = 0; k < n_axes_; ++k) {
     int pick = -1;
@@ -448,6 +457,20 @@ void Compiler::ChooseSchedule() {
   hdr_.n_rdim = nr_;
   hdr_.n_kidx = static_cast<uint32_t>(n_k);
   hdr_.n_ridx = static_cast<uint32_t>(n_r);
+  // A reduce shared between workgroups: the axis that numbers its parts must be the outermost kept dim, by itself;
+  // the schedule is laid out for one part of the reduced index space.
+  uint32_t parts = 0;
+  for (int i = 0; i < nn_; ++i) {
+    const ANode &n = nodes_[i];
+    if (n.kind != AK_REDUCE || n.op->part_split == 0) continue;
+    parts = static_cast<uint32_t>(n.op->part_split);
+    const int ax = n.axis[0];
+    if (ax < 0 || nk_ == 0) Fail("no axis for the parts of a shared reduce");
+    const Dim &outer = dims_[klist_[nk_ - 1]];
+    if (outer.first_axis != pos_[ax] || outer.last_axis != pos_[ax] || n_peel_ > 0) Fail("the parts of a shared reduce are not the outermost kept dim");
+  }
+  const uint64_t n_r_whole = n_r;
+  if (parts != 0) n_r = (n_r + parts - 1) / parts;
   uint32_t threads = 256;
   single_round_ = true;
   // Slabs per lane per instruction: the wide build of the VM halves the dispatches per element at the price
@@ -456,7 +479,7 @@ void Compiler::ChooseSchedule() {
   // Measured on MI355X it does not pay (batch-norm 98 us against 76, RMSNorm 118 us against 104): two waves per
   // SIMD hide too little latency. Kept as a tuning switch, off by default.
   bool wide = false;
-  if (k_->tuning_.vec_wide == 1) wide = !(nr_ > 0 && !inner_red);
+  if (k_->tuning_.vec_wide == 1) wide = !(nr_ > 0 && !inner_red) && parts == 0;
   u_ = wide ? DVM_VEC_U_WIDE : 2;
   const uint32_t U = static_cast<uint32_t>(u_);
   const uint32_t max_threads = wide ? 512u : 1024u;
@@ -523,7 +546,10 @@ void Compiler::ChooseSchedule() {
     single_round_ = n_r <= static_cast<uint64_t>(team) * U;
   } else {
     hdr_.sched = VS_REDY;
-    uint32_t tx = n_k >= 64 ? 64 : Pow2Ceil(n_k);
+    // (a shared reduce: the lanes along the kept space stay inside one part where its outputs are few, so that the
+    // parts spread over workgroups)
+    const uint64_t n_k_part = parts != 0 ? std::max<uint64_t>(n_k / parts, 1) : n_k;
+    uint32_t tx = n_k_part >= 64 ? 64 : Pow2Ceil(n_k_part);
     uint32_t ty = 256 / tx;
     const uint64_t items = (n_k + tx - 1) / tx;
     if (items < 128 && n_r > 256) ty = max_threads / tx;  // few outputs: give each more lanes along the reduce space
@@ -535,6 +561,19 @@ void Compiler::ChooseSchedule() {
     single_round_ = n_r <= static_cast<uint64_t>(ty) * U;
   }
   if (wide) hdr_.sched |= VS_WIDE;
+  if (parts != 0) {
+    if (nr_ == 0) Fail("a shared reduce without a reduced dim");
+    // indices of the reduced space one round of a team covers; a part is whole rounds
+    const uint32_t team_lanes = inner_red ? (hdr_.team_is_block ? threads : (1u << hdr_.team_log2)) : threads >> hdr_.team_log2;
+    const uint64_t round = static_cast<uint64_t>(team_lanes) * U;
+    const uint64_t chunk = (n_r + round - 1) / round * round;
+    if (chunk >= (1ull << 31)) Fail("index space above 2^31 groups");
+    hdr_.r_chunk = static_cast<uint32_t>(chunk);
+    hdr_.k_per_chunk = static_cast<uint32_t>(n_k / parts);
+    if (hdr_.k_per_chunk == 0 || n_k % parts != 0) Fail("the parts of a shared reduce do not divide the kept index space");
+    single_round_ = chunk <= round;
+    (void)n_r_whole;
+  }
 
   prog_->threads = threads;
 }

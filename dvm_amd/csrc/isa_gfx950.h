@@ -211,7 +211,12 @@ typedef struct {
   uint32_t mem_off;      // word offset of VMemDesc[n_mem]
   uint32_t code_off;     // word offset of the instruction words
   uint32_t n_vslot;      // V register slots in use (each U*16 bytes per lane of local memory)
-  uint32_t pad[4];       // (keeps the axis tables 16-byte aligned: the interpreter reads them as 128-bit words)
+  // A reduce shared between workgroups (both 0 otherwise): the outermost kept axis numbers the parts of the reduced
+  // index space, r_chunk indices each (whole rounds; the last part may be short or empty); coordinate c of a lane along
+  // that axis is kidx / k_per_chunk, and the lane reduces the indices [c * r_chunk, min(n_ridx, (c + 1) * r_chunk)).
+  uint32_t r_chunk;
+  uint32_t k_per_chunk;
+  uint32_t pad[2];       // (keeps the axis tables 16-byte aligned: the interpreter reads them as 128-bit words)
   VDim kdims[DVM_VEC_MAXR];
   VDim rdims[DVM_VEC_MAXR];
 } VVecHeader;            // 80 + 128 = 208 bytes

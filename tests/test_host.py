@@ -232,6 +232,38 @@ def test_matmul_epilogue_is_one_cube_program():
     assert das.index("cast.round.bf16") < das.index("Add.fp32"), das
 
 
+def test_reduce_with_few_outputs_is_shared_between_workgroups(monkeypatch):
+    # a column sum of [4096, 4096] would run on 8 workgroups: for this code generation the reduce becomes one reduce per
+    # part of the rows (an outermost kept axis numbers the parts, no operand but the partial output has it) and a
+    # reduce over the parts, which also carries the arithmetic on the result; the operator list is as it was afterwards
+    def compile_one(shape, axes, graph=None):
+        t = Tester("split", run_mode="das")
+        x = t.load(np.zeros(shape, np.float32))
+        t.store(graph(t, x) if graph else t.mul(t.sum(x, axes, True), 0.5))
+        t.codegen()
+        return t, t.das()
+    t, das = compile_one([4096, 4096], (0,))
+    assert das.count("== sub-kernel") == 2 and "shared-reduce parts=64 x 64" in das, das
+    first, second = das.split("== sub-kernel 1 ==")
+    assert "kdims: 512 64  rdims: 4096" in first and "k[1,0] r[4096]" in first and "k[1,4096] r[0]" in first, das
+    assert "Mul.fp32 acc, #0x3f000000" in second and "Mul.fp32" not in first and "rdims: 64" in second, das
+    assert t.workspace_bytes() >= 64 * 4096 * 4
+    dump_before = t.dump()
+    t.codegen()
+    assert t.das() == das and t.dump() == dump_before
+    # rows that a workgroup each: nothing to share; a consumer that walks the input again: left alone
+    _, das = compile_one([8192, 4096], (1,))
+    assert "shared-reduce" not in das and das.count("== sub-kernel") == 1, das
+    _, das = compile_one([4, 1 << 20], (1,), lambda t, x: t.sub(x, t.max(x, (1,), True)))
+    assert "shared-reduce" not in das, das
+    monkeypatch.setenv("DVM_RED_SPLIT", "0")
+    _, das = compile_one([4096, 4096], (0,))
+    assert "shared-reduce" not in das and das.count("== sub-kernel") == 1, das
+    monkeypatch.setenv("DVM_RED_SPLIT", "3")
+    _, das = compile_one([1000], (0,))
+    assert "shared-reduce parts=3 x " in das, das
+
+
 def test_matmul_with_few_tiles_and_a_long_k_axis_is_split(monkeypatch):
     # 16 tiles of 256x256 on 256 compute units, k = 16384: the k axis is shared, two launches, fp32 partial tiles in
     # the workspace; DVM_CUBE_SPLITK=0 keeps the single launch, =N forces N parts (rounded to whole 64-k steps)
