@@ -740,6 +740,33 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
   typedef typename SlabVec<SL>::type Slabs;
   const uint32_t *code32 = prog32 + 2 * h.code_off;
   static_assert(NTEMP == 4, "temporaries are named registers");
+  auto mem_desc = [&](uint32_t a, uint64_t &addr, uint32_t &dtype, uint32_t &sn, uint32_t &sm, uint64_t &boff) {
+    const uint32_t *d = prog32 + 2 * h.mem_off + a * (sizeof(VCubeMem) / 4);
+    addr = static_cast<uint64_t>(uni(d[0])) | (static_cast<uint64_t>(uni(d[1])) << 32);
+    dtype = uni(d[2]);
+    sn = uni(d[4]);
+    sm = uni(d[5]);
+    boff = static_cast<uint64_t>(h.batch0) * uni(d[6]) + static_cast<uint64_t>(h.batch1) * uni(d[7]);
+  };
+  if (h.flags & VCF_PLAIN_STORE) {
+    // [Add mem] [cast.round] store: three instructions at most, done here without the dispatch loop
+    uint32_t at = 0;
+    uint32_t w0 = __builtin_amdgcn_readlane(h.w0v, 0);
+    uint64_t addr, boff;
+    uint32_t dtype, sn, sm;
+    if ((w0 & 0xffu) == VOP_BINF) {
+      mem_desc(w0 >> 24, addr, dtype, sn, sm, boff);
+      acc = acc + epi_load<SL>(addr, dtype, sn, sm, boff, rows, col, ncol);
+      w0 = __builtin_amdgcn_readlane(h.w0v, ++at);
+    }
+    if ((w0 & 0xffu) == VOP_CAST) {
+      apply_rnd<SL>(acc, (w0 >> 20) & 0x3u);
+      w0 = __builtin_amdgcn_readlane(h.w0v, ++at);
+    }
+    mem_desc(w0 >> 24, addr, dtype, sn, sm, boff);
+    epi_store<SL>(addr, dtype, sn, sm, boff, rows, col, ncol, acc);
+    return;
+  }
   Slabs t0, t1, t2, t3;  // never read before written (the emitter parks a value before it names the register)
   uint32_t mask = 0;
   uint32_t pc = 0;
@@ -904,6 +931,123 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
         break;
     }
   }
+}
+
+// The epilogue of a plain product, [Add mem] [cast.round] store (VCF_PLAIN_STORE), for one wave's slabs of a pass: when
+// they all lie inside the output and the operands take 128-bit accesses, every slab is read, finished and stored here
+// (the descriptors are decoded once, the bias row is fetched once: a lane's column does not change) and the function
+// returns true; otherwise the caller sends the slabs through epilogue_pass, which does the same with every guard.
+// A function of its own, and a small one: what a call costs is the registers the callee has to save (the interpreter's
+// pass saves and restores some hundred per lane through scratch memory, 12 us per tile and launch on MI355X).
+template <int ROWS, int BN, int TM, int WM>
+__device__ __attribute__((noinline)) bool epilogue_plain_pass(const float *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
+                                                              uint32_t pass, uint32_t m, uint32_t n, uint32_t m_lo, uint32_t n_lo) {
+  constexpr int NTHR = WM * 2 * 64;
+  constexpr int PITCH = BN + 4;
+  constexpr int GROUPS = BN / 8;
+  constexpr int PER_THREAD = ROWS * GROUPS / NTHR;
+  constexpr int ROWS_PER_STEP = NTHR / GROUPS;
+  constexpr int HALF = ROWS / WM;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t g = tid % GROUPS, r0 = tid / GROUPS;
+  const uint32_t col = n0 + g * 8;
+  const uint32_t ncol = (col >= n || col < n_lo) ? 0u : (n - col < 8u ? n - col : 8u);
+  // [Add mem] [cast.round] store, the epilogue of a plain product: when the wave's slabs are all inside the output and
+  // the operands take 128-bit accesses, every slab of the pass is read, finished and stored here in one go (the
+  // descriptors are decoded once, the bias row is fetched once: a lane's column does not change); otherwise the
+  // slabs go through run_epilogue below, which does the same three instructions with every guard.
+  const uint32_t *code32 = prog32 + 2 * ea.code_off;
+  auto desc = [&](uint32_t a, uint64_t &addr, uint32_t &dtype, uint32_t &sn, uint32_t &sm, uint64_t &boff) {
+    const uint32_t *d = prog32 + 2 * ea.mem_off + a * (sizeof(VCubeMem) / 4);
+    addr = static_cast<uint64_t>(uni(d[0])) | (static_cast<uint64_t>(uni(d[1])) << 32);
+    dtype = uni(d[2]);
+    sn = uni(d[4]);
+    sm = uni(d[5]);
+    boff = static_cast<uint64_t>(ea.batch0) * uni(d[6]) + static_cast<uint64_t>(ea.batch1) * uni(d[7]);
+  };
+  uint32_t at = 0, w0 = uni(code32[0]);
+  bool has_bias = false;
+  uint64_t b_addr = 0, b_boff = 0, s_addr, s_boff;
+  uint32_t b_dtype = 0, b_sn = 0, b_sm = 0, s_dtype, s_sn, s_sm, rnd = VRND_NONE;
+  if ((w0 & 0xffu) == VOP_BINF) {
+    has_bias = true;
+    desc(w0 >> 24, b_addr, b_dtype, b_sn, b_sm, b_boff);
+    w0 = uni(code32[2 * ++at]);
+  }
+  if ((w0 & 0xffu) == VOP_CAST) {
+    rnd = (w0 >> 20) & 0x3u;
+    w0 = uni(code32[2 * ++at]);
+  }
+  desc(w0 >> 24, s_addr, s_dtype, s_sn, s_sm, s_boff);
+  const uint32_t s_esz = elem_size(s_dtype);
+  bool fast = ncol == 8u && s_sn == 1u && s_esz != 1u && ((static_cast<uint64_t>(s_sm) * s_esz) & 15u) == 0u &&
+              ((s_addr + (s_boff + col) * s_esz) & 15u) == 0u;
+  if (has_bias) {  // a row of fp32 biases (the same for every row of the output), 128-bit loads
+    fast = fast && b_dtype == VDT_F32 && b_sn == 1u && b_sm == 0u && ((b_addr + (b_boff + col) * 4u) & 15u) == 0u;
+  }
+  auto row_of = [&](int q) -> uint32_t {
+    const uint32_t lr = q * ROWS_PER_STEP + r0;
+    return m0 + (lr / HALF) * (TM * 32) + pass * HALF + lr % HALF;
+  };
+  {  // the lane's rows grow with q: the first and the last bound them all
+    const uint32_t first = row_of(0), last = row_of(PER_THREAD - 1);
+    fast = fast && first >= m_lo && last < m && first <= last;
+  }
+  if (wave_all(fast)) {
+    vf4 blo = {0.0f, 0.0f, 0.0f, 0.0f}, bhi = blo;
+    if (has_bias) {
+      const DVM_GLOBAL vf4 *bp = reinterpret_cast<const DVM_GLOBAL vf4 *>(b_addr + (b_boff + col) * 4u);
+      blo = bp[0];
+      bhi = bp[1];
+    }
+    constexpr int CH = PER_THREAD < 4 ? PER_THREAD : 4;  // slabs in flight: few, so that the function stays small in registers
+#pragma unroll
+    for (int c0 = 0; c0 < PER_THREAD; c0 += CH) {
+      vf4 lo[CH], hi[CH];
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        const float *src = dump + ((c0 + q) * ROWS_PER_STEP + r0) * PITCH + g * 8;
+        lo[q] = *reinterpret_cast<const vf4 *>(src);
+        hi[q] = *reinterpret_cast<const vf4 *>(src + 4);
+      }
+#pragma unroll
+      for (int q = 0; q < CH; ++q) {
+        vf4 x = lo[q] + blo, y = hi[q] + bhi;
+        if (rnd == VRND_F16) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            x[e] = round_f16(x[e]);
+            y[e] = round_f16(y[e]);
+          }
+        } else if (rnd == VRND_BF16) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            x[e] = round_bf16(x[e]);
+            y[e] = round_bf16(y[e]);
+          }
+        }
+        const uint64_t o = (s_boff + col + static_cast<uint64_t>(row_of(c0 + q)) * s_sm) * s_esz;
+        if (s_esz == 4u) {
+          vu4 a, b;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            a[e] = __float_as_uint(x[e]);
+            b[e] = __float_as_uint(y[e]);
+          }
+          *reinterpret_cast<DVM_GLOBAL vu4 *>(s_addr + o) = a;
+          *reinterpret_cast<DVM_GLOBAL vu4 *>(s_addr + o + 16) = b;
+        } else if (s_dtype == VDT_F16) {
+          const vu4 a = {pack_f16(x[0], x[1]), pack_f16(x[2], x[3]), pack_f16(y[0], y[1]), pack_f16(y[2], y[3])};
+          *reinterpret_cast<DVM_GLOBAL vu4 *>(s_addr + o) = a;
+        } else {
+          const vu4 a = {pack_bf16(x[0], x[1]), pack_bf16(x[2], x[3]), pack_bf16(y[0], y[1]), pack_bf16(y[2], y[3])};
+          *reinterpret_cast<DVM_GLOBAL vu4 *>(s_addr + o) = a;
+        }
+      }
+    }
+    return true;
+  }
+  return false;
 }
 
 // Second half of a pass: the half tile sits in local memory, row major with PITCH floats per row;
@@ -1266,9 +1410,14 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
           for (int r = 0; r < 16; ++r) dst[(8 * (r / 4) + (r % 4)) * PITCH] = c[r];
         }
       }
-      __syncthreads();
-      epilogue_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
-      __syncthreads();
+      // The two meetings of a pass order local-memory accesses only (the dump before the slabs are read, the reads
+      // before the next dump): they wait for this wave's local-memory operations and not, as __syncthreads() would,
+      // for its stores to memory as well, which stay in flight under the next pass and the next tile's loop.
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo)) {
+        epilogue_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
   }
 }

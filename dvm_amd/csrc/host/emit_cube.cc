@@ -187,6 +187,15 @@ void Compiler::CompileCube(int a) {
     h.tile = 2;
     bt = 64;
   }
+  // ... unless most of such a tile would lie outside the output (batches of small matrices): a tile half the size
+  // that wastes less than half as much wins
+  {
+    auto padded = [&](int64_t t) { return static_cast<double>(tiles(t)) * static_cast<double>(t * t); };
+    while (bt > 64 && padded(bt) > 2.0 * padded(bt / 2)) {
+      bt /= 2;
+      ++h.tile;
+    }
+  }
   {  // tuning override: 256, 128 or 64
     const int v = k_->tuning_.cube_tile;
     if (v == 256 || v == 128 || v == 64) {
@@ -332,6 +341,12 @@ void Compiler::CompileCube(int a) {
     DropCastBeforeStore(dts);
   }
   h.epi_flags = FuseCubeEpilogue();
+  {  // [Add mem] [cast.round] store end: done natively by the kernel
+    size_t i = 0;
+    if (i < code_.size() && VI_OP(code_[i]) == VOP_BINF && VI_SUB(code_[i]) == VB_ADD && VI_KIND(code_[i]) == VK_MEM && VI_RND(code_[i]) == 0) ++i;
+    if (i < code_.size() && VI_OP(code_[i]) == VOP_CAST && VI_SUB(code_[i]) == VC_RND) ++i;
+    if (i + 2 == code_.size() && VI_OP(code_[i]) == VOP_ST && VI_OP(code_[i + 1]) == VOP_END && k_->tuning_.cube_exact != 2) h.epi_flags |= VCF_PLAIN_STORE;
+  }
   h.n_mem = n_mem_;
   h.n_code = static_cast<uint32_t>(code_.size());
   h.mem_off = sizeof(VCubeHeader) / 8;

@@ -271,6 +271,9 @@ typedef struct {
 // VCF_SPLITK_PARTIAL: tiles * k_split workgroups; each multiplies one part of the k axis and writes its accumulators
 // to part_addr as the lanes hold them, no epilogue. VCF_SPLITK_COMBINE: one workgroup per tile adds the k_split
 // partials in ascending k order (fp32, the same order on every run) and runs the epilogue on the sum.
+// The epilogue is [add of a memory operand (a bias row)] [rounding to a float type] store: the kernel does it in
+// place, without walking the program through the interpreter (a dispatch costs more than this whole epilogue).
+#define VCF_PLAIN_STORE 8u
 #define VCF_SPLITK_PARTIAL 2u
 #define VCF_SPLITK_COMBINE 4u
 
