@@ -734,7 +734,9 @@ struct EpiArgs {
 };
 
 // Runs the epilogue program on SL slabs whose accumulator values are in `acc`.
-template <int SL>
+// SLIM: the program holds only what VCF_SLIM lists (one temporary, float binaries, the hardware's exp / log / sqrt,
+// rounding, loads and stores): the arms of everything else are left out, and with them most of the registers.
+template <int SL, bool SLIM>
 __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, const uint32_t *prog32, const EpiArgs &h, const SlabRows &rows,
                                              uint32_t col, uint32_t ncol) {
   typedef typename SlabVec<SL>::type Slabs;
@@ -769,6 +771,10 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
   }
   Slabs t0, t1, t2, t3;  // never read before written (the emitter parks a value before it names the register)
   uint32_t mask = 0;
+  (void)t1;
+  (void)t2;
+  (void)t3;
+  (void)mask;
   uint32_t pc = 0;
   while (true) {
     // the program sits in two registers, one instruction per lane: no memory access to fetch one
@@ -800,7 +806,8 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
       } else if (kind == VK_IMM) {
         src = __uint_as_float(imm);
       } else if (kind == VK_REG) {
-        src = a == 0 ? t0 : (a == 1 ? t1 : (a == 2 ? t2 : t3));
+        if constexpr (SLIM) src = t0;
+        else src = a == 0 ? t0 : (a == 1 ? t1 : (a == 2 ? t2 : t3));
       } else {
         src = acc;
       }
@@ -820,15 +827,15 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
             case VB_RDIV_APPROX: FOR_SE acc[q] = __fdividef(src[q], acc[q]); break;
             case VB_MIN: FOR_SE acc[q] = acc[q] < src[q] ? acc[q] : src[q]; break;
             case VB_MAX: FOR_SE acc[q] = acc[q] > src[q] ? acc[q] : src[q]; break;
-            case VB_AND: FOR_SE acc[q] = (acc[q] != 0.0f && src[q] != 0.0f) ? 1.0f : 0.0f; break;
-            case VB_OR: FOR_SE acc[q] = (acc[q] != 0.0f || src[q] != 0.0f) ? 1.0f : 0.0f; break;
-            case VB_POW: acc = slab_pow<SL>(acc, src); break;
-            default: acc = slab_pow<SL>(src, acc); break;
+            case VB_AND: if constexpr (!SLIM) FOR_SE acc[q] = (acc[q] != 0.0f && src[q] != 0.0f) ? 1.0f : 0.0f; break;
+            case VB_OR: if constexpr (!SLIM) FOR_SE acc[q] = (acc[q] != 0.0f || src[q] != 0.0f) ? 1.0f : 0.0f; break;
+            case VB_POW: if constexpr (!SLIM) acc = slab_pow<SL>(acc, src); break;
+            default: if constexpr (!SLIM) acc = slab_pow<SL>(src, acc); break;
           }
           apply_rnd<SL>(acc, rnd);
           break;
         case VOP_BINI:
-          switch (sub & 0x3fu) {
+          if constexpr (!SLIM) switch (sub & 0x3fu) {
             case VBI_ADD: FOR_SE acc[q] = __uint_as_float(__float_as_uint(acc[q]) + __float_as_uint(src[q])); break;
             case VBI_SUB: FOR_SE acc[q] = __uint_as_float(__float_as_uint(acc[q]) - __float_as_uint(src[q])); break;
             case VBI_RSUB: FOR_SE acc[q] = __uint_as_float(__float_as_uint(src[q]) - __float_as_uint(acc[q])); break;
@@ -837,7 +844,7 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
             default: FOR_SE acc[q] = __int_as_float(max(__float_as_int(acc[q]), __float_as_int(src[q]))); break;
           }
           break;
-        case VOP_CMP: {
+        case VOP_CMP: if constexpr (!SLIM) {
           const uint32_t t = sub & 0x7u;
           if (sub & VCMP_INT) {
             FOR_SE {
@@ -852,46 +859,51 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
               acc[q] = c ? 1.0f : 0.0f;
             }
           }
-          break;
         }
+          break;
         case VOP_MSK:
-          mask = 0;
-          FOR_SE mask |= ((__float_as_uint(src[q]) << 1) != 0 ? 1u : 0u) << q;
+          if constexpr (!SLIM) {
+            mask = 0;
+            FOR_SE mask |= ((__float_as_uint(src[q]) << 1) != 0 ? 1u : 0u) << q;
+          }
           break;
         default:  // VOP_MOVM
-          FOR_SE acc[q] = ((mask >> q) & 1u) ? src[q] : acc[q];
+          if constexpr (!SLIM) FOR_SE acc[q] = ((mask >> q) & 1u) ? src[q] : acc[q];
           break;
       }
       continue;
     }
     switch (op) {
       case VOP_LDR:
-        acc = a == 0 ? t0 : (a == 1 ? t1 : (a == 2 ? t2 : t3));
+        if constexpr (SLIM) acc = t0;
+        else acc = a == 0 ? t0 : (a == 1 ? t1 : (a == 2 ? t2 : t3));
         break;
       case VOP_LDI:
         acc = __uint_as_float(imm);
         break;
       case VOP_STR:
-        if (a == 0) t0 = acc;
+        if (SLIM || a == 0) t0 = acc;
         else if (a == 1) t1 = acc;
         else if (a == 2) t2 = acc;
         else t3 = acc;
         break;
       case VOP_UN:
         switch (sub) {
-          case VU_SQRT: acc = by_halves<SL>(acc, math_sqrt); break;
+          case VU_SQRT: if constexpr (!SLIM) acc = by_halves<SL>(acc, math_sqrt); break;
           case VU_SQRT_APPROX: FOR_SE acc[q] = __builtin_amdgcn_sqrtf(acc[q]); break;
           case VU_ABS: FOR_SE acc[q] = fabsf(acc[q]); break;
-          case VU_LOG: acc = by_halves<SL>(acc, math_log); break;
+          case VU_LOG: if constexpr (!SLIM) acc = by_halves<SL>(acc, math_log); break;
           case VU_LOG_APPROX: FOR_SE acc[q] = __logf(acc[q]); break;
-          case VU_EXP: acc = by_halves<SL>(acc, math_exp); break;
+          case VU_EXP: if constexpr (!SLIM) acc = by_halves<SL>(acc, math_exp); break;
           case VU_EXP_SCALED:  // the product is a value of its own: rounded to fp32, never contracted into what follows
-            FOR_SE {
-              float y = acc[q] * __uint_as_float(imm);
-              asm volatile("" : "+v"(y));
-              acc[q] = y;
+            if constexpr (!SLIM) {
+              FOR_SE {
+                float y = acc[q] * __uint_as_float(imm);
+                asm volatile("" : "+v"(y));
+                acc[q] = y;
+              }
+              acc = by_halves<SL>(acc, math_exp);
             }
-            acc = by_halves<SL>(acc, math_exp);
             break;
           case VU_EXP_APPROX: FOR_SE acc[q] = __expf(acc[q]); break;
           case VU_EXP_SCALED_APPROX:
@@ -901,13 +913,13 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
               acc[q] = __expf(y);
             }
             break;
-          case VU_ISFINITE: FOR_SE acc[q] = isfinite(acc[q]) ? 1.0f : 0.0f; break;
-          case VU_ROUND: FOR_SE acc[q] = rintf(acc[q]); break;
-          case VU_FLOOR: FOR_SE acc[q] = floorf(acc[q]); break;
-          case VU_CEIL: FOR_SE acc[q] = ceilf(acc[q]); break;
-          case VU_TRUNC: FOR_SE acc[q] = truncf(acc[q]); break;
+          case VU_ISFINITE: if constexpr (!SLIM) FOR_SE acc[q] = isfinite(acc[q]) ? 1.0f : 0.0f; break;
+          case VU_ROUND: if constexpr (!SLIM) FOR_SE acc[q] = rintf(acc[q]); break;
+          case VU_FLOOR: if constexpr (!SLIM) FOR_SE acc[q] = floorf(acc[q]); break;
+          case VU_CEIL: if constexpr (!SLIM) FOR_SE acc[q] = ceilf(acc[q]); break;
+          case VU_TRUNC: if constexpr (!SLIM) FOR_SE acc[q] = truncf(acc[q]); break;
           default:
-            FOR_SE {
+            if constexpr (!SLIM) FOR_SE {
               const uint32_t x = __float_as_uint(acc[q]);
               acc[q] = __uint_as_float(static_cast<int32_t>(x) < 0 ? 0u - x : x);
             }
@@ -916,7 +928,9 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
         apply_rnd<SL>(acc, rnd);
         break;
       case VOP_CAST:
-        if (sub == VC_F2I) {
+        if (SLIM) {
+          apply_rnd<SL>(acc, rnd);
+        } else if (sub == VC_F2I) {
           FOR_SE acc[q] = __int_as_float(static_cast<int32_t>(acc[q]));
         } else if (sub == VC_I2F) {
           FOR_SE acc[q] = static_cast<float>(__float_as_int(acc[q]));
@@ -1052,7 +1066,7 @@ __device__ __attribute__((noinline)) bool epilogue_plain_pass(const float *dump,
 
 // Second half of a pass: the half tile sits in local memory, row major with PITCH floats per row;
 // every lane takes slabs of 8 columns and walks the epilogue program over them.
-template <int ROWS, int BN, int TM, int WM>
+template <int ROWS, int BN, int TM, int WM, bool SLIM>
 __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
                                                         uint32_t pass, uint32_t m, uint32_t n, uint32_t m_lo, uint32_t n_lo) {
   constexpr int NTHR = WM * 2 * 64;
@@ -1060,7 +1074,7 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
   constexpr int GROUPS = BN / 8;               // slabs per row
   constexpr int PER_THREAD = ROWS * GROUPS / NTHR;  // slabs per thread
   // four slabs per walk of the program where a wave may use all 512 registers; with two waves per SIMD two slabs
-  constexpr int SL = (PER_THREAD % 4 == 0 && WM == 2) ? 4 : 2;
+  constexpr int SL = (PER_THREAD % 4 == 0 && (WM == 2 || SLIM)) ? 4 : 2;
   static_assert(PER_THREAD % SL == 0, "slab count per thread");
   constexpr int ROWS_PER_STEP = NTHR / GROUPS;  // rows one step of all threads covers
   const uint32_t tid = threadIdx.x;
@@ -1093,7 +1107,7 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
       }
     }
     if (wave_all(rows.ok == 0u || ncol == 0u)) continue;  // nothing of these slabs is inside the tile's part of the output
-    run_epilogue<SL>(acc, prog32, ea, rows, col, ncol);
+    run_epilogue<SL, SLIM>(acc, prog32, ea, rows, col, ncol);
   }
 }
 
@@ -1415,7 +1429,8 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       // for its stores to memory as well, which stay in flight under the next pass and the next tile's loop.
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo)) {
-        epilogue_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
+        if (h.epi_flags & VCF_SLIM) epilogue_pass<PROWS, BN, TM, WM, true>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
+        else epilogue_pass<PROWS, BN, TM, WM, false>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
       }
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }

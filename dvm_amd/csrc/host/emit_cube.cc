@@ -341,6 +341,40 @@ void Compiler::CompileCube(int a) {
     DropCastBeforeStore(dts);
   }
   h.epi_flags = FuseCubeEpilogue();
+  {  // the slim pass takes programs of activation-like epilogues
+    bool slim = true;
+    for (uint64_t w : code_) {
+      const uint32_t sub = VI_SUB(w);
+      switch (VI_OP(w)) {
+        case VOP_END:
+        case VOP_LD:
+        case VOP_LDI:
+        case VOP_ST:
+          break;
+        case VOP_LDR:
+        case VOP_STR:
+          if (VI_A(w) != 0) slim = false;
+          break;
+        case VOP_CAST:
+          if (sub != VC_RND) slim = false;
+          break;
+        case VOP_UN:
+          if (sub != VU_ABS && sub != VU_EXP_APPROX && sub != VU_EXP_SCALED_APPROX && sub != VU_LOG_APPROX && sub != VU_SQRT_APPROX) slim = false;
+          break;
+        case VOP_BINF: {
+          const uint32_t b = sub & 0x3fu;
+          if (b != VB_ADD && b != VB_SUB && b != VB_RSUB && b != VB_MUL && b != VB_DIV && b != VB_RDIV && b != VB_DIV_APPROX &&
+              b != VB_RDIV_APPROX && b != VB_MIN && b != VB_MAX) slim = false;
+          if (VI_KIND(w) == VK_REG && VI_A(w) != 0) slim = false;
+          break;
+        }
+        default:
+          slim = false;
+          break;
+      }
+    }
+    if (slim && k_->tuning_.cube_exact != 2) h.epi_flags |= VCF_SLIM;
+  }
   {  // [Add mem] [cast.round] store end: done natively by the kernel
     size_t i = 0;
     if (i < code_.size() && VI_OP(code_[i]) == VOP_BINF && VI_SUB(code_[i]) == VB_ADD && VI_KIND(code_[i]) == VK_MEM && VI_RND(code_[i]) == 0) ++i;

@@ -274,6 +274,11 @@ typedef struct {
 // The epilogue is [add of a memory operand (a bias row)] [rounding to a float type] store: the kernel does it in
 // place, without walking the program through the interpreter (a dispatch costs more than this whole epilogue).
 #define VCF_PLAIN_STORE 8u
+// The epilogue holds only loads, stores, rounding, the temporary 0, float binaries (add, sub, rsub, mul, div, rdiv
+// and their hardware forms, min, max) and the unaries abs and the hardware's exp / scaled exp / log / sqrt: it runs
+// through a build of the interpreter's pass without the arms of everything else, which needs half the registers
+// (what calling the pass costs is the registers it saves).
+#define VCF_SLIM 16u
 #define VCF_SPLITK_PARTIAL 2u
 #define VCF_SPLITK_COMBINE 4u
 
