@@ -79,7 +79,7 @@ __device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk) {
 // KS source (k strided, the row index contiguous): 8x8 element blocks through registers, transposed on
 // the way (v_perm_b32), then written with ds_write_b128.
 struct LaneOffsets {
-  uint32_t v[2];
+  int32_t v[2];  // (signed: a row that is clamped back inside the operand lies before the row the loop would fetch)
 };
 
 template <int ROWS, bool KC, int NTHR>
@@ -94,13 +94,20 @@ struct Stage<ROWS, true, NTHR> {
   // Chunk position p = NTHR*i + tid of the tile holds row p/8, logical chunk (p%8) ^ swizzle(row): with
   // row = RPS*i + tid/8 the swizzle depends at most on the parity of i (RPS = 32; not at all for 64), hence
   // two byte offsets per lane.
-  static __device__ __forceinline__ LaneOffsets lane_offset(uint32_t ld, uint32_t tid) {
+  // rows_valid < ROWS (a tile of which only the first rows lie inside the operand; tiles of at most two chunks per
+  // lane only): the rows past the end fetch the last valid row instead, so that no load leaves the operand; what
+  // they feed are accumulator rows the epilogue never stores.
+  static constexpr bool kCanClamp = N <= 2;
+  static __device__ __forceinline__ LaneOffsets lane_offset(uint32_t ld, uint32_t tid, uint32_t rows_valid = ROWS) {
     LaneOffsets o;
 #pragma unroll
     for (int par = 0; par < 2; ++par) {
       const uint32_t row = RPS * par + (tid >> 3);
       const uint32_t logical = (tid & 7u) ^ ((row ^ (row >> 3)) & 7u);
-      o.v[par] = ((tid >> 3) * ld + (logical << 3)) * 2u;
+      uint32_t from = tid >> 3;  // row fetched, relative to the first row of chunk `par`
+      int32_t back = 0;
+      if (kCanClamp && row >= rows_valid) back = static_cast<int32_t>(rows_valid - 1u) - static_cast<int32_t>(row);
+      o.v[par] = (static_cast<int32_t>(from) + back) * static_cast<int32_t>(ld * 2u) + static_cast<int32_t>((logical << 3) * 2u);
     }
     return o;
   }
@@ -111,7 +118,7 @@ struct Stage<ROWS, true, NTHR> {
     const uint32_t wave_first = uni(tid >> 6) * 64u;
 #pragma unroll
     for (int i = 0; i < N; ++i) {
-      const DVM_GLOBAL char *src = base + static_cast<uint64_t>(i) * RPS * ld * 2u + lane.v[i & 1];
+      const DVM_GLOBAL char *src = base + (static_cast<int64_t>(static_cast<uint64_t>(i) * RPS * ld * 2u) + lane.v[i & 1]);
       uint16_t *dst = tile + (static_cast<uint32_t>(i) * NTHR + wave_first) * 8u;
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(src), (__attribute__((address_space(3))) void *)(dst), 16, 0, 0);
     }
@@ -137,7 +144,7 @@ struct Stage<ROWS, false, NTHR> {
     const uint32_t blk = tid / TPB, part = tid % TPB;
     const uint32_t kb = blk / (ROWS / 8), rb = blk % (ROWS / 8);
     LaneOffsets o;
-    o.v[0] = o.v[1] = (kb * 8u * ld + rb * 8u + part * RPT) * 2u;
+    o.v[0] = o.v[1] = static_cast<int32_t>((kb * 8u * ld + rb * 8u + part * RPT) * 2u);
     return o;
   }
 
@@ -1208,6 +1215,11 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       for (int j = 0; j < TN; ++j) acc[i][j] = 0.0f;
 
     constexpr bool RING = BM == 256 && BN == 256;  // the ring of 32-deep stages
+    // The smallest tile also takes the vector path when an operand with contiguous k has fewer rows than the tile
+    // (one to 63 rows of A against a weight matrix): the rows past the end fetch the last valid row.
+    constexpr bool a_clamps = !RING && A_KC && (BM * BK / 8 / NTHR) <= 2, b_clamps = !RING && B_KC && (BN * BK / 8 / NTHR) <= 2;
+    const uint32_t a_rows = h.m - m0 < static_cast<uint32_t>(BM) ? h.m - m0 : static_cast<uint32_t>(BM);
+    const uint32_t b_rows = h.n - n0 < static_cast<uint32_t>(BN) ? h.n - n0 : static_cast<uint32_t>(BN);
     // address of element (row0, k_lo) of each operand
     const uint64_t a_org = a_base + (A_KC ? static_cast<uint64_t>(m0) * h.lda + k_lo : static_cast<uint64_t>(k_lo) * h.lda + m0) * 2;
     const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb + k_lo : static_cast<uint64_t>(k_lo) * h.ldb + n0) * 2;
@@ -1226,7 +1238,7 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
               for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[e];
             }
       }
-    } else if (h.fast && m0 + BM <= h.m && n0 + BN <= h.n) {
+    } else if (h.fast && (m0 + BM <= h.m || a_clamps) && (n0 + BN <= h.n || b_clamps)) {
      if constexpr (RING) {
       tile_loop_ring<IS_BF16, A_KC, B_KC, WM>(acc, lds, a_org, b_org, h.lda, h.ldb, (k_hi - k_lo) / SK, tid);
      } else {
@@ -1235,7 +1247,11 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       // k advances by BK per step
       const uint64_t a_step = (A_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.lda) * 2;
       const uint64_t b_step = (B_KC ? static_cast<uint64_t>(BK) : static_cast<uint64_t>(BK) * h.ldb) * 2;
-      const LaneOffsets a_voff = Stage<BM, A_KC, NTHR>::lane_offset(h.lda, tid), b_voff = Stage<BN, B_KC, NTHR>::lane_offset(h.ldb, tid);
+      LaneOffsets a_voff, b_voff;
+      if constexpr (A_KC) a_voff = Stage<BM, A_KC, NTHR>::lane_offset(h.lda, tid, a_rows);
+      else a_voff = Stage<BM, A_KC, NTHR>::lane_offset(h.lda, tid);
+      if constexpr (B_KC) b_voff = Stage<BN, B_KC, NTHR>::lane_offset(h.ldb, tid, b_rows);
+      else b_voff = Stage<BN, B_KC, NTHR>::lane_offset(h.ldb, tid);
       sa.fetch(a_org, h.lda, a_voff, tid, lds);
       sb.fetch(b_org, h.ldb, b_voff, tid, lds + kBBase);
       sa.commit(lds, tid);

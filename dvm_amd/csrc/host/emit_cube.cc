@@ -243,8 +243,9 @@ void Compiler::CompileCube(int a) {
         const uint64_t slots = ti == 2 ? 2 * cus : cus;  // two 64x64 workgroups fit a compute unit
         const uint32_t max_split = nt >= slots ? 1u : static_cast<uint32_t>(std::min<uint64_t>(slots / nt, 32));
         // (ragged edge tiles of an aligned product are moved back inside the output and stay on the vector path)
-        const bool m_fast = M % t == 0 || (M >= t && (!mm->trans_a || M % 8 == 0));
-        const bool n_fast = N % t == 0 || (N >= t && N % 8 == 0);
+        // (and the 64 tile fetches the rows of a short operand with contiguous k through clamped addresses)
+        const bool m_fast = M % t == 0 || (M >= t && (!mm->trans_a || M % 8 == 0)) || (t == 64 && !mm->trans_a);
+        const bool n_fast = N % t == 0 || (N >= t && N % 8 == 0) || (t == 64 && mm->trans_b);
         const double slow = (aligned && m_fast && n_fast) ? 1.0 : 2.5;
         for (uint32_t want = 1; want <= max_split; want = want < 2 ? 2 : want * 2) {
           uint32_t chunk = 0;
