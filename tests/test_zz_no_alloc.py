@@ -90,3 +90,30 @@ def test_static_workspace_launch_matches_the_allocating_route():
     bad = (ctypes.c_uint32 * 2)(len(programs), 0)
     assert hip.dvm_hip_launch_vm_static_ws(blobs, len(programs), geo, bad, 1, t.workspace_bytes(), None) == ERR_BAD_WS_WORD
     assert hip.dvm_hip_launch_vm_static_ws(blobs, len(programs), geo, words, n_ws, 16, None) == ERR_BAD_WS_WORD  # offsets past ws_bytes
+
+
+def test_static_workspace_holds_the_partials_of_shared_reduces_and_split_products():
+    # two launches each, the first leaves fp32 partial results in the workspace: column sums of a [60000, 96] tensor
+    # (a reduce shared between workgroups) and a 256x256x8192 product with its k axis split
+    hip = _hip()
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal([60000, 96]).astype(np.float32)
+    a = (rng.standard_normal([256, 8192]) / 16).astype(np.float16)
+    b = (rng.standard_normal([8192, 256]) / 16).astype(np.float16)
+    kernels = []
+    t = Tester("split")
+    kernels.append((t, t.store(t.sum(t.load(x), (0,), True)), "shared-reduce parts="))
+    t = Tester("mix")
+    kernels.append((t, t.store(t.matmul(t.load(a), t.load(b), False, False)), "split-k partials"))
+    for t, out, marker in kernels:
+        t.run()
+        want = t.output(out).copy()
+        assert marker in t.das() and t.num_launches() == 2 and 0 < t.workspace_bytes() <= STATIC_WS_BYTES, t.das()
+        programs = t.programs()
+        blobs, geo, words, n_ws = _pack(programs)
+        assert n_ws >= 2  # the partials are written by the first launch and read by the second
+        assert hip.dvm_hip_memset(t.device_ptr(out), 0, want.nbytes) == 0
+        rc = hip.dvm_hip_launch_vm_static_ws(blobs, len(programs), geo, words, n_ws, t.workspace_bytes(), None)
+        assert rc == 0, hip.dvm_hip_error_string(rc)
+        assert hip.dvm_hip_synchronize_stream(None) == 0
+        assert np.array_equal(t.output(out).view(np.uint8), want.view(np.uint8)), marker
