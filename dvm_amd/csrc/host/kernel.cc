@@ -42,14 +42,16 @@ size_t Compiler::Run() {
   // per part of the reduced index space and a reduce over the parts; should that graph not compile, the kernel
   // is compiled as it was built.
   if (SplitLongReduces()) {
+    const int mode_before = k_->part_mode_;  // (the partition mode a kernel remembers is that of the graph as built)
     bool done = false;
     size_t ws = 0;
     try {
       ws = RunModes();
       done = true;
-    } catch (const std::runtime_error &) {
+    } catch (...) {  // whatever it was: the operator list must be restored, and the kernel as built gets its chance
     }
     UndoSplitReduces(done);
+    k_->part_mode_ = mode_before;
     if (done) return ws;
   }
   return RunModes();
