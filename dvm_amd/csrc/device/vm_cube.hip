@@ -1226,17 +1226,35 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
     if (split_comb) {
       const DVM_GLOBAL vf4 *src = reinterpret_cast<const DVM_GLOBAL vf4 *>(h.part_addr) + static_cast<uint64_t>(tile_id) * kPartVecs * NTHR + tid;
       const uint64_t split_stride = static_cast<uint64_t>(n_tiles) * kPartVecs * NTHR;
-      for (uint32_t sp = 0; sp < h.k_split; ++sp) {
+      // One fragment (16 registers) at a time, its vectors of four or eight parts in flight together: a trip to memory
+      // per fragment and group of parts instead of several per part (a single workgroup per tile is latency bound);
+      // the parts are still added in ascending order.
+      constexpr int PC = TM * TN == 4 ? 8 : 4;  // (fewer where the accumulators take half the registers, or two workgroups share a compute unit)
+      for (uint32_t sp0 = 0; sp0 < h.k_split; sp0 += PC) {
+        const uint32_t n_here = h.k_split - sp0 < static_cast<uint32_t>(PC) ? h.k_split - sp0 : static_cast<uint32_t>(PC);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
+          for (int j = 0; j < TN; ++j) {
+            vf4 v[PC][4];
+            const DVM_GLOBAL vf4 *frag = src + sp0 * split_stride + static_cast<uint32_t>((i * TN + j) * 4) * NTHR;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const vf4 v = src[sp * split_stride + static_cast<uint32_t>((i * TN + j) * 4 + q) * NTHR];
+            for (int pp = 0; pp < PC; ++pp) {
+              if (static_cast<uint32_t>(pp) < n_here) {
 #pragma unroll
-              for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[e];
+                for (int q = 0; q < 4; ++q) v[pp][q] = frag[pp * split_stride + static_cast<uint32_t>(q) * NTHR];
+              }
             }
+#pragma unroll
+            for (int pp = 0; pp < PC; ++pp) {
+              if (static_cast<uint32_t>(pp) < n_here) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+#pragma unroll
+                  for (int e = 0; e < 4; ++e) acc[i][j][4 * q + e] += v[pp][q][e];
+              }
+            }
+          }
       }
     } else if (h.fast && (m0 + BM <= h.m || a_clamps) && (n0 + BN <= h.n || b_clamps)) {
      if constexpr (RING) {
@@ -1455,20 +1473,22 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
 
 }  // namespace
 
-#define DVM_CUBE_KERNEL(name, bf, tm, tn, wm, akc, bkc) \
-  extern "C" __global__ void __launch_bounds__(wm * 128) name(const VmParam p) { vm_cube<bf, tm, tn, akc, bkc, wm>(p); }
-#define DVM_CUBE_LAYOUTS(prefix, bf, tm, tn, wm)            \
-  DVM_CUBE_KERNEL(prefix##_nn, bf, tm, tn, wm, true, false) \
-  DVM_CUBE_KERNEL(prefix##_nt, bf, tm, tn, wm, true, true)  \
-  DVM_CUBE_KERNEL(prefix##_tn, bf, tm, tn, wm, false, false) \
-  DVM_CUBE_KERNEL(prefix##_tt, bf, tm, tn, wm, false, true)
+// `occ` = waves per SIMD the register budget must leave room for (two workgroups of the 64x64 tile share a compute unit:
+// 256 registers a lane, vector and accumulation registers together)
+#define DVM_CUBE_KERNEL(name, bf, tm, tn, wm, occ, akc, bkc) \
+  extern "C" __global__ void __launch_bounds__(wm * 128, occ) name(const VmParam p) { vm_cube<bf, tm, tn, akc, bkc, wm>(p); }
+#define DVM_CUBE_LAYOUTS(prefix, bf, tm, tn, wm, occ)            \
+  DVM_CUBE_KERNEL(prefix##_nn, bf, tm, tn, wm, occ, true, false) \
+  DVM_CUBE_KERNEL(prefix##_nt, bf, tm, tn, wm, occ, true, true)  \
+  DVM_CUBE_KERNEL(prefix##_tn, bf, tm, tn, wm, occ, false, false) \
+  DVM_CUBE_KERNEL(prefix##_tt, bf, tm, tn, wm, occ, false, true)
 
-DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_big, true, 4, 4, 2)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_big, false, 4, 4, 2)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_mid, true, 2, 2, 2)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_mid, false, 2, 2, 2)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_small, true, 1, 1, 2)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_small, false, 1, 1, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_big, true, 4, 4, 2, 1)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_big, false, 4, 4, 2, 1)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_mid, true, 2, 2, 2, 1)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_mid, false, 2, 2, 2, 1)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_small, true, 1, 1, 2, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_small, false, 1, 1, 2, 2)
 // the 256x256 tile on eight waves (4 x 2, 64x128 accumulators each): two waves per SIMD
-DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_big8, true, 2, 4, 4)
-DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_big8, false, 2, 4, 4)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_bf16_big8, true, 2, 4, 4, 2)
+DVM_CUBE_LAYOUTS(dvm_vm_cube_f16_big8, false, 2, 4, 4, 2)

@@ -215,8 +215,9 @@ void Compiler::CompileCube(int a) {
   // from figures measured on MI355X (bf16, microseconds): a workgroup's time per 64 k (2.2 for the 256 tile, 1.3 for
   // 128, 0.71 for 64 alone on its compute unit and 0.9 when two share one; the guarded path of ragged or unaligned
   // tiles takes about two and a half times as long), rounds of workgroups over the chip, and for a split the second launch plus
-  // the time its one workgroup per tile needs per partial tile (8.5 / 4.5 / 0.55: a single workgroup streams at
-  // some 30 GB/s), which is what keeps deep splits of big tiles from paying.
+  // the time its one workgroup per tile needs per partial tile (3.2 / 0.8 / 0.2 with the vectors of several parts in
+  // flight together: a single workgroup streams at some 80 GB/s), which is what keeps deep splits of big tiles from
+  // paying, plus the time the first launch takes to write the partial tiles (some 4 TB/s over the whole chip).
   uint32_t k_split = 1, k_chunk = 0;
   {
     const int forced = k_->tuning_.cube_splitk;
@@ -231,7 +232,7 @@ void Compiler::CompileCube(int a) {
       k_split = parts_of(static_cast<uint32_t>(forced), &k_chunk);
     } else if (forced != 0 && forced != 1) {
       static const int64_t kTiles[3] = {256, 128, 64};
-      static const double kStepUs[3] = {2.2, 1.3, 0.71}, kPartUs[3] = {8.5, 4.5, 0.55};
+      static const double kStepUs[3] = {2.2, 1.3, 0.71}, kPartUs[3] = {3.2, 0.8, 0.2};
       const bool aligned = K % 64 == 0 && h.lda % 8 == 0 && h.ldb % 8 == 0;
       double best = 0.0;
       int best_tile = -1;
@@ -256,7 +257,7 @@ void Compiler::CompileCube(int a) {
           const double rounds = std::ceil(static_cast<double>(wgs) / static_cast<double>(slots));
           const double step_us = (ti == 2 && wgs > cus) ? 0.9 : kStepUs[ti];
           double us = rounds * steps * step_us * slow + 3.0;
-          if (parts > 1) us += 5.0 + parts * kPartUs[ti];
+          if (parts > 1) us += 5.0 + parts * kPartUs[ti] + static_cast<double>(wgs) * static_cast<double>(t * t) * 4.0 / 4.0e6;
           if (parts > 1 && static_cast<double>(wgs) * static_cast<double>(t * t) * 4.0 > 512.0 * 1024 * 1024) continue;
           if (best_tile < 0 || us < best) {
             best = us;
