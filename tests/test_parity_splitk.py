@@ -155,3 +155,23 @@ def test_split_against_the_unsplit_product(monkeypatch):
     differ = res["0"] != res["4"]
     assert differ.mean() < 0.02, float(differ.mean())
     assert np.allclose(res["0"], res["4"], rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.parametrize("tile", ["256", "128", "64"])
+@pytest.mark.parametrize("parts", [5, 7, 13])
+def test_part_counts_that_leave_the_last_group_of_partials_short(monkeypatch, tile, parts):
+    # the second launch reads the partial tiles in groups of four (tile 256, 64) or eight (tile 128): 5, 7 and 13 parts
+    # leave a last group of one, three, five or seven; the result must be the sum of exactly `parts` partials
+    monkeypatch.setenv("DVM_CUBE_TILE", tile)
+    monkeypatch.setenv("DVM_CUBE_SPLITK", str(parts))
+    m, n, k = 256 + 8, 320, parts * 128
+    rng = np.random.default_rng(parts * 1000 + int(tile))
+    a16, b16, a_ref, b_ref = _operands(rng, m, n, k, False, True, "float16", sigma=0.25)
+    t = Tester("mix")
+    out = t.store(t.cast(t.matmul(t.load(a16), t.load(b16), False, True), "float32"))
+    t.run()
+    assert ("split-k sum of %d" % parts) in t.das(), t.das()
+    want = _product(a_ref.astype(np.float64), b_ref.astype(np.float64), False, True)
+    got = t.output(out).astype(np.float64)
+    # fp32 accumulation, the product rounded to fp16 before the cast back
+    assert np.allclose(got, want, rtol=2e-3, atol=2e-3), float(np.abs(got - want).max())
