@@ -797,18 +797,29 @@ __device__ __forceinline__ VMemDesc load_desc(const uint32_t *prog32, uint32_t m
 // where they are needed (one 128-bit read per division) instead of living in scalar registers for the whole launch.
 __device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim *dims, uint32_t ndim,
                                                  const uint32_t (&stride)[DVM_VEC_MAXR], bool inner) {
-  uint64_t off = 0;
+  // a space of one axis (rows of a matrix, elements of a row): no division, and one uniform branch here instead of
+  // two per axis below (a dozen scalar branches per memory instruction otherwise: they, not the arithmetic, were
+  // most of what the offsets of an instruction cost)
+  if (ndim <= 1u) return (static_cast<uint64_t>(n) * stride[0]) * (inner ? static_cast<uint32_t>(E) : 1u);
+  // the first axis, then the second alone when there are two (one more uniform branch), else the rest
+  uint64_t off;
+  {
+    const vu4 dv = *reinterpret_cast<const vu4 *>(dims);  // extent, magic, shift, pad
+    const uint32_t q = (__umulhi(n, dv[1]) + n) >> dv[2];
+    off = (static_cast<uint64_t>(n - q * dv[0]) * stride[0]) * (inner ? static_cast<uint32_t>(E) : 1u);
+    n = q;
+  }
+  if (ndim == 2u) return off + static_cast<uint64_t>(n) * stride[1];
 #pragma unroll
-  for (int i = 0; i < DVM_VEC_MAXR; ++i) {
+  for (int i = 1; i < DVM_VEC_MAXR; ++i) {
     if (i < static_cast<int>(ndim)) {
       uint32_t c = n;
       if (i + 1 < static_cast<int>(ndim)) {
-        const vu4 dv = *reinterpret_cast<const vu4 *>(dims + i);  // extent, magic, shift, pad
+        const vu4 dv = *reinterpret_cast<const vu4 *>(dims + i);
         const uint32_t q = (__umulhi(n, dv[1]) + n) >> dv[2];
         c = n - q * dv[0];
         n = q;
       }
-      if (i == 0 && inner) c *= E;
       off += static_cast<uint64_t>(c) * stride[i];
     }
   }
@@ -1253,7 +1264,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                 }
               }
             }
-            last_off = off;
+            if (!(w0 & VI_OFFS_ASIDE)) last_off = off;
           }
           if (op == VOP_LD) {
             if constexpr (SCHED == VS_REDX) {

@@ -183,6 +183,7 @@ std::string &VKernel::DisAssemble() {
           case VOP_MOVM: os << "select acc, "; PrintSrc(os, w); break;
           default: os << "?"; break;
         }
+        if (VI_OP(w) > VOP_LD && VI_KIND(w) == VK_MEM && (static_cast<uint32_t>(w) & VI_OFFS_ASIDE)) os << "  ; offsets of its own (those before it stay current)";
         os << "\n";
       }
     };

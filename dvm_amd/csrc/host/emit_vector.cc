@@ -21,8 +21,12 @@ void Compiler::Emit(uint32_t op, uint32_t sub, uint32_t kind, uint32_t rnd, uint
       if (last_mem_ >= 0 && std::memcmp(mems_[last_mem_].kstride, mems_[a].kstride, sizeof(mems_[a].kstride)) == 0 &&
           std::memcmp(mems_[last_mem_].rstride, mems_[a].rstride, sizeof(mems_[a].rstride)) == 0) {
         w |= VI_SAME_OFFS;
+        last_mem_ = static_cast<int>(a);
+      } else if (last_mem_ >= 0 && op != VOP_ST && op != VOP_LD) {
+        w |= VI_OFFS_ASIDE;  // an operand on a path of its own: the offsets of the instruction before stay current
+      } else {
+        last_mem_ = static_cast<int>(a);
       }
-      last_mem_ = static_cast<int>(a);
     } else if (op == VOP_SWEEP || op == VOP_ENDSWEEP) {
       last_mem_ = -1;
     } else if (uniform_emit_ && (op == VOP_UN || op == VOP_CAST ||

@@ -160,6 +160,11 @@ enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 #define VI_ENDS 0x80u
 #define VI_UNIFORM (1u << 22)
 #define VI_SAME_OFFS (1u << 23)
+// VI_OFFS_ASIDE (top bit of the sub field; vector VM, a VOP_BINF / VOP_BINI / VOP_CMP / VOP_MSK / VOP_MOVM with a memory
+// operand): the operand walks memory differently from the memory instruction before it, and its offsets are not
+// what a later VI_SAME_OFFS refers to: that still means the instruction before this one (x * w stored where x came
+// from: the store reuses the load's offsets although the weight row was read in between).
+#define VI_OFFS_ASIDE (1u << 15)
 #define VI_MAKE(op, sub, kind, rnd, a, imm)                                                     \
   ((uint64_t)(op) | ((uint64_t)(sub) << 8) | ((uint64_t)(kind) << 16) | ((uint64_t)(rnd) << 20) | \
    ((uint64_t)(a) << 24) | ((uint64_t)(uint32_t)(imm) << 32))
