@@ -795,21 +795,12 @@ __device__ __forceinline__ VMemDesc load_desc(const uint32_t *prog32, uint32_t m
 // E-groups when `inner` is set and is converted to elements.
 // `dims` points at the axis table in local memory: its entries feed per-lane arithmetic only, so they are read
 // where they are needed (one 128-bit read per division) instead of living in scalar registers for the whole launch.
-__device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim *dims, uint32_t ndim,
-                                                 const uint32_t (&stride)[DVM_VEC_MAXR], bool inner) {
-  // a space of one axis (rows of a matrix, elements of a row): no division, and one uniform branch here instead of
-  // two per axis below (a dozen scalar branches per memory instruction otherwise: they, not the arithmetic, were
-  // most of what the offsets of an instruction cost)
-  if (ndim <= 1u) return (static_cast<uint64_t>(n) * stride[0]) * (inner ? static_cast<uint32_t>(E) : 1u);
-  // the first axis, then the second alone when there are two (one more uniform branch), else the rest
-  uint64_t off;
-  {
-    const vu4 dv = *reinterpret_cast<const vu4 *>(dims);  // extent, magic, shift, pad
-    const uint32_t q = (__umulhi(n, dv[1]) + n) >> dv[2];
-    off = (static_cast<uint64_t>(n - q * dv[0]) * stride[0]) * (inner ? static_cast<uint32_t>(E) : 1u);
-    n = q;
-  }
-  if (ndim == 2u) return off + static_cast<uint64_t>(n) * stride[1];
+// (three and four axes, out of line: rare, and inlined at every memory instruction their tests of the axis count sat
+// in scalar registers that the hot paths then had to spill)
+__device__ __attribute__((noinline)) uint64_t space_offset_rest(uint32_t n, const VDim *dims, uint32_t ndim, uint32_t s1, uint32_t s2,
+                                                                uint32_t s3) {
+  const uint32_t stride[DVM_VEC_MAXR] = {0u, s1, s2, s3};
+  uint64_t off = 0;
 #pragma unroll
   for (int i = 1; i < DVM_VEC_MAXR; ++i) {
     if (i < static_cast<int>(ndim)) {
@@ -824,6 +815,24 @@ __device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim *dims, u
     }
   }
   return off;
+}
+
+__device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim *dims, uint32_t ndim,
+                                                 const uint32_t (&stride)[DVM_VEC_MAXR], bool inner) {
+  // a space of one axis (rows of a matrix, elements of a row): no division, and one uniform branch here instead of
+  // two per axis (a dozen scalar branches per memory instruction otherwise: they, not the arithmetic, were most of
+  // what the offsets of an instruction cost)
+  if (ndim <= 1u) return (static_cast<uint64_t>(n) * stride[0]) * (inner ? static_cast<uint32_t>(E) : 1u);
+  // the first axis, then the second alone when there are two (one more uniform branch), else the rest
+  uint64_t off;
+  {
+    const vu4 dv = *reinterpret_cast<const vu4 *>(dims);  // extent, magic, shift, pad
+    const uint32_t q = (__umulhi(n, dv[1]) + n) >> dv[2];
+    off = (static_cast<uint64_t>(n - q * dv[0]) * stride[0]) * (inner ? static_cast<uint32_t>(E) : 1u);
+    n = q;
+  }
+  if (ndim == 2u) return off + static_cast<uint64_t>(n) * stride[1];
+  return off + space_offset_rest(n, dims, uni(ndim), stride[1], stride[2], stride[3]);
 }
 
 // Valid element count (0..E) of the E-group with flat index n in a space whose first axis counts groups.
