@@ -795,6 +795,15 @@ __device__ __forceinline__ VMemDesc load_desc(const uint32_t *prog32, uint32_t m
 // E-groups when `inner` is set and is converted to elements.
 // `dims` points at the axis table in local memory: its entries feed per-lane arithmetic only, so they are read
 // where they are needed (one 128-bit read per division) instead of living in scalar registers for the whole launch.
+// A uniform value as it is now, for a test that should be made where it stands: a test of a loop-invariant value is
+// otherwise hoisted out of the interpreter loop, and its result then occupies a pair of scalar registers for the
+// whole launch (enough of those and the kernel spills scalar registers into lanes of a vector register, which every
+// use reads back).
+__device__ __forceinline__ uint32_t fresh(uint32_t x) {
+  asm volatile("" : "+s"(x));
+  return x;
+}
+
 // (three and four axes, out of line: rare, and inlined at every memory instruction their tests of the axis count sat
 // in scalar registers that the hot paths then had to spill)
 __device__ __attribute__((noinline)) uint64_t space_offset_rest(uint32_t n, const VDim *dims, uint32_t ndim, uint32_t s1, uint32_t s2,
@@ -822,6 +831,7 @@ __device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim *dims, u
   // a space of one axis (rows of a matrix, elements of a row): no division, and one uniform branch here instead of
   // two per axis (a dozen scalar branches per memory instruction otherwise: they, not the arithmetic, were most of
   // what the offsets of an instruction cost)
+  ndim = fresh(ndim);
   if (ndim <= 1u) return (static_cast<uint64_t>(n) * stride[0]) * (inner ? static_cast<uint32_t>(E) : 1u);
   // the first axis, then the second alone when there are two (one more uniform branch), else the rest
   uint64_t off;
@@ -839,7 +849,7 @@ __device__ __forceinline__ uint64_t space_offset(uint32_t n, const VDim *dims, u
 __device__ __forceinline__ uint32_t group_valid(uint32_t n, const VDim *dims, uint32_t ndim,
                                                 uint32_t inner_extent) {
   uint32_t c = n;
-  if (ndim > 1) {
+  if (fresh(ndim) > 1u) {
     const vu4 dv = *reinterpret_cast<const vu4 *>(dims);
     c = n - ((__umulhi(n, dv[1]) + n) >> dv[2]) * dv[0];
   }
@@ -1067,7 +1077,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
               if constexpr (SCHED == VS_REDX) {
                 if (k0 <= VR_MIN || k1 <= VR_MIN) {
-                  red_finish_x(racc0.v[0], racc1.v[0], k0, k1, tlog, team_is_block, tid, nthreads, red_flip, lds);
+                  red_finish_x(racc0.v[0], racc1.v[0], k0, k1, tlog, fresh(h.team_is_block) != 0u, tid, nthreads, red_flip, lds);
                 }
               } else {
                 if (k0 <= VR_MIN) racc0 = red_finish_y<SCHED>(racc0, k0, tlog, nthreads, k_local, r_local, lds);
@@ -1467,7 +1477,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
           break;
         case VOP_UNI_END: {
           if constexpr (SCHED == VS_REDX) {
-            if (team_is_block) {
+            if (fresh(h.team_is_block) != 0u) {
               // what the run produced lives in the first wave's S registers and accumulator: pass it on
               float *box = reinterpret_cast<float *>(lds + kBoxAt) + box_flip * 16u;
               box_flip ^= 1u;
