@@ -205,6 +205,7 @@ class Compiler {
     int stage = 0;  // the caller's group (parallel / sequence kernels); operators of different groups never share a launch
     int n_ops = 0;  // operators joined so far (a program has room for about 500 instruction words and 160 nodes)
     bool has_part = false;  // holds a reduce shared between workgroups: only operators of its input's index space join
+    int64_t over_parts = 0;  // holds the reduce over the parts of a shared reduce: its output's elements (0: none); nothing larger joins
   };
   std::vector<AreaInfo> areas_;
 

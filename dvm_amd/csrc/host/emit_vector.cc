@@ -722,7 +722,12 @@ void Compiler::CompileArea(int a) {
   UnifyAxes();
   OrderAndMerge();
   ChooseSchedule();
-  // a stored value must span the index space it is stored from, or it would be written several times
+  // a stored value must span the index space it is stored from, or it would be written several times. (The axis
+  // that numbers the parts of a shared reduce is the exception: a value stored inside the sweep over the reduced space
+  // lies in exactly one part, as every element of the reduce's input does.)
+  int parts_axis = -1;
+  for (int i = 0; i < nn_; ++i)
+    if (nodes_[i].kind == AK_REDUCE && nodes_[i].op->part_split != 0 && nodes_[i].axis[0] >= 0) parts_axis = nodes_[i].axis[0];
   for (int i = 0; i < nn_; ++i) {
     const ANode &n = nodes_[i];
     if (n.kind != AK_OUT) continue;
@@ -733,8 +738,12 @@ void Compiler::CompileArea(int a) {
       have |= 1u << n.axis[d];
       if (axes_[n.axis[d]].reduced) fd = true;
     }
+    bool all_reduced = true;  // (does the value have every reduced axis? then it is stored once per element of the reduced space)
+    for (int ax = 0; ax < n_axes_; ++ax)
+      if (axes_[ax].reduced && !((have >> ax) & 1u)) all_reduced = false;
     for (int ax = 0; ax < n_axes_; ++ax) {
       if ((have >> ax) & 1u) continue;
+      if (ax == parts_axis && fd && all_reduced) continue;
       if (!axes_[ax].reduced || fd) Fail("output smaller than the kernel domain");
     }
   }

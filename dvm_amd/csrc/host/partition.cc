@@ -89,6 +89,10 @@ bool Compiler::CanJoin(int a, const NDObject *o) {
       return false;
     }
   }
+  // The launch that reduces over the parts of a shared reduce holds what works on the reduce's output (the mean, the
+  // variance, their stores). An operator on a larger index space (x - mean) would make that launch walk the larger
+  // space and reduce the parts again for every one of its elements: it reads the result from memory in a launch of its own.
+  if (ai.over_parts != 0 && o->numel() > ai.over_parts) return false;
   if (o->kind == kObjReduce && LevelIn(a, o) < 8 && ai.red_at_level[LevelIn(a, o)] >= 2) return false;
   if (o->kind == kObjMatMul) return false;
   if (ai.n_ops >= kMaxAreaOps && !IsStoreLike(o)) return false;  // long graphs are cut into several launches
@@ -143,6 +147,7 @@ void Compiler::Join(int a, const NDObject *o) {
       ai.reduce = o;
       ai.has_part = o->part_split != 0;
     }
+    if (o->in[0] != nullptr && o->in[0]->kind == kObjReduce && o->in[0]->part_split != 0) ai.over_parts = std::max<int64_t>(ai.over_parts, o->numel());
     DomMerge(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
   }
   DomMerge(ai, o->shape_ref_->data, o->rank());

@@ -553,6 +553,11 @@ void Compiler::ChooseSchedule() {
     uint32_t ty = 256 / tx;
     const uint64_t items = (n_k + tx - 1) / tx;
     if (items < 128 && n_r > 256) ty = max_threads / tx;  // few outputs: give each more lanes along the reduce space
+    else if (items < 128 && n_r >= 64) ty = 512 / tx;     // (the launch that reduces over the parts of a shared reduce, mostly)
+    // (the parts of a shared reduce: with fewer than two workgroups per compute unit, 512 lanes each put twice the
+    // loads in flight. Measured on MI355X, fp32 sums over axis 0: [8192,1024] 57 -> 47 us, [65536,768] 136 -> 97 us,
+    // [32,3136,256] over its first two axes 86 -> 70 us; 1024 lanes are slower again, 54 / 120 / 79 us)
+    if (parts != 0 && items < 2ull * g_system.core_num && n_r >= 32) ty = 512 / tx;
     while (ty > 1 && static_cast<uint64_t>(ty) * U > 2 * n_r) ty >>= 1;
     threads = std::max<uint32_t>(64, tx * ty);
     ty = threads / tx;

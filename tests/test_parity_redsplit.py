@@ -95,7 +95,8 @@ def test_a_pointwise_output_beside_a_shared_reduce():
     full = t.store(y)
     col = t.store(t.sum(y, (0,), False))
     t.run()
-    assert "shared-reduce parts=" in t.das(), t.das()
+    # (the pointwise output is stored by the launch that reduces the parts: every element of y lies in exactly one part)
+    assert "shared-reduce parts=" in t.das() and t.num_launches() == 2, t.das()
     assert np.array_equal(t.output(full), x + np.float32(1.0))
     assert _sum_close(t.output(col), (x + np.float32(1.0)).astype(np.float64), (0,))
 
@@ -143,3 +144,28 @@ def test_dynamic_shapes_shared_on_one_run_and_not_on_the_next():
         t.run()
         assert ("shared-reduce" in t.das()) == shared, (rows, cols, t.das())
         assert _sum_close(t.output(out), x.astype(np.float64), (0,)), (rows, cols)
+
+
+def test_consumers_larger_than_the_reduce_get_launches_of_their_own():
+    # (x - mean) / sqrt(var + eps) over axis 0 of [8192, 1024] (a batch-norm in channels-last layout): both sums are
+    # shared between workgroups; the launches that reduce over the parts hold the per-column arithmetic only, x - mean
+    # and the division read their results from memory (in one launch with them, every element of x would reduce the
+    # 128 partial sums of its column again)
+    rng = np.random.default_rng(16)
+    x = (rng.standard_normal([8192, 1024]) * 2 + 0.5).astype(np.float32)
+    t = Tester("split")
+    lx = t.load(x)
+    mean = t.mul(t.sum(lx, (0,), True), 1.0 / 8192)
+    d = t.sub(lx, mean)
+    var = t.mul(t.sum(t.mul(d, d), (0,), True), 1.0 / 8192)
+    out = t.store(t.div(d, t.sqrt(t.add(var, 1e-5))))
+    t.run()
+    das = t.das()
+    assert das.count("shared-reduce parts=") == 2 and t.num_launches() == 5, das
+    for entry in das.split("== sub-kernel")[1:]:
+        head = entry.splitlines()[1]
+        if "sched=reduce-y" in head and "shared-reduce" not in head:  # a launch that reduces over the parts
+            assert "kept=128 " in head, head
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean(0, keepdims=True)) / np.sqrt(x64.var(0, keepdims=True) + 1e-5)
+    assert np.allclose(t.output(out), want, rtol=1e-5, atol=1e-5), float(np.abs(t.output(out) - want).max())
