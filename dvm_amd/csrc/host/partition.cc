@@ -279,13 +279,14 @@ bool Compiler::SplitLongReduces() {
       while (split > 1 && n_red / static_cast<uint64_t>(split) * outs_per_wg < 32768) split /= 2;
     }
     if (split < 2 || n_red < 2ull * static_cast<uint64_t>(split)) continue;
-    // every consumer works on the reduce's own output
+    // every consumer works on the reduce's own output, or on a larger index space (x - max of a softmax: it then
+    // reads the result from memory in a launch of its own, see CanJoin)
     bool ok = false;
     for (const NDObject *c : ops) {
       for (int j = 0; j < c->nin; ++j) {
         if (c->in[j] != r) continue;
         ok = true;
-        if (c->numel() != r->numel() || c->kind == kObjReduce || c->kind == kObjMatMul || c->kind == kObjConcatPart) split = 0;
+        if (c->numel() < r->numel() || c->kind == kObjReduce || c->kind == kObjMatMul || c->kind == kObjConcatPart) split = 0;
       }
       for (const NDObject *part : c->parts)
         if (part == r) split = 0;

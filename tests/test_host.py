@@ -251,11 +251,15 @@ def test_reduce_with_few_outputs_is_shared_between_workgroups(monkeypatch):
     dump_before = t.dump()
     t.codegen()
     assert t.das() == das and t.dump() == dump_before
-    # rows that a workgroup each: nothing to share; a consumer that walks the input again: left alone
+    # rows that a workgroup each: nothing to share; a consumer that walks the input again (x - max) is shared too, and
+    # the launch that reduces over the parts holds nothing of the size of x: x - max reads the maxima from memory
     _, das = compile_one([8192, 4096], (1,))
     assert "shared-reduce" not in das and das.count("== sub-kernel") == 1, das
     _, das = compile_one([4, 1 << 20], (1,), lambda t, x: t.sub(x, t.max(x, (1,), True)))
-    assert "shared-reduce" not in das, das
+    assert "shared-reduce parts=" in das and das.count("== sub-kernel") == 3, das
+    over_parts = das.split("== sub-kernel")[2]
+    assert "kept=1 " in over_parts and "Sub.fp32" not in over_parts, das
+    assert "sched=pointwise" in das.split("== sub-kernel")[3] and "Sub.fp32" in das.split("== sub-kernel")[3], das
     monkeypatch.setenv("DVM_RED_SPLIT", "0")
     _, das = compile_one([4096, 4096], (0,))
     assert "shared-reduce" not in das and das.count("== sub-kernel") == 1, das

@@ -72,8 +72,10 @@ def test_two_reduces_of_one_input_and_what_follows_them():
     assert np.allclose(t.output(var), x64.var(0, keepdims=True), rtol=1e-4, atol=1e-4)
 
 
-def test_a_reduce_whose_consumer_walks_the_input_again_is_left_alone():
-    # softmax over rows of a million elements: the second sweep needs the whole row in one workgroup anyway
+def test_a_reduce_whose_consumer_walks_the_input_again():
+    # softmax over rows of 262144 elements, three rows: max and sum are both shared (three workgroups would walk a
+    # megabyte each three times: 180 us in one launch, 110 us in five); exp(x - max) reads the maxima from memory in the
+    # launch that sums its parts, and is stored there for the launch that divides
     rng = np.random.default_rng(12)
     x = rng.standard_normal([3, 1 << 18]).astype(np.float32)
     t = Tester("split")
@@ -81,10 +83,27 @@ def test_a_reduce_whose_consumer_walks_the_input_again_is_left_alone():
     e = t.exp(t.sub(lx, t.max(lx, (1,), True)))
     out = t.store(t.div(e, t.sum(e, (1,), True)))
     t.run()
-    assert "shared-reduce" not in t.das(), t.das()
+    das = t.das()
+    assert das.count("shared-reduce parts=") == 2 and t.num_launches() == 5, das
     x64 = x.astype(np.float64)
     e64 = np.exp(x64 - x64.max(1, keepdims=True))
     assert np.allclose(t.output(out), e64 / e64.sum(1, keepdims=True), rtol=1e-4, atol=1e-9)
+
+
+@pytest.mark.parametrize("shape", [(4096, 1024), (32000, 512)])
+def test_softmax_over_the_outer_axis(shape):
+    # max and sum over axis 0 with consumers on the whole tensor: two shared reduces, their results read from memory
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal(shape).astype(np.float32)
+    t = Tester("split")
+    lx = t.load(x)
+    e = t.exp(t.sub(lx, t.max(lx, (0,), True)))
+    out = t.store(t.div(e, t.sum(e, (0,), True)))
+    t.run()
+    assert t.das().count("shared-reduce parts=") == 2, t.das()
+    x64 = x.astype(np.float64)
+    e64 = np.exp(x64 - x64.max(0, keepdims=True))
+    assert np.allclose(t.output(out), e64 / e64.sum(0, keepdims=True), rtol=1e-4, atol=1e-9)
 
 
 def test_a_pointwise_output_beside_a_shared_reduce():
