@@ -451,12 +451,22 @@ void Compiler::DetectAttention() {
     if (sb->kind != kObjBinary || sb->op != kSub || uses[sb->id] != 1) continue;
     NDObject *x = sb->in[0], *mx = sb->in[1];
     if (mx->kind != kObjReduce || mx->op != kMax || mx->in[0] != x || uses[mx->id] != 1 || !last_axis_keep(mx)) continue;
-    if (x->kind != kObjCast || x->type_id_ != kFloat32 || uses[x->id] != 2) continue;
+    // the scale: on the 16-bit product in front of the cast (the example's order), or on the fp32 scores behind it
+    float scale = 1.0f;
+    NDObject *mul = nullptr, *mul32 = nullptr;
+    if (x->kind == kObjBinaryS && x->op == kMul && x->type_id_ == kFloat32 && uses[x->id] == 2 && x->in[0]->kind == kObjCast &&
+        uses[x->in[0]->id] == 1) {
+      mul32 = x;
+      const uint32_t bits = ScalarToContainer(x->scalar.Get(), kFloat32);
+      std::memcpy(&scale, &bits, 4);
+      x = x->in[0];
+    } else if (uses[x->id] != 2) {
+      continue;
+    }
+    if (x->kind != kObjCast || x->type_id_ != kFloat32) continue;
     NDObject *sc = x->in[0];
     NDObject *m1 = sc;
-    float scale = 1.0f;
-    NDObject *mul = nullptr;
-    if (sc->kind == kObjBinaryS && sc->op == kMul && uses[sc->id] == 1) {
+    if (mul32 == nullptr && sc->kind == kObjBinaryS && sc->op == kMul && uses[sc->id] == 1) {
       mul = sc;
       m1 = sc->in[0];
       const uint32_t bits = ScalarToContainer(sc->scalar.Get(), sc->in[0]->type_id_);
@@ -475,7 +485,7 @@ void Compiler::DetectAttention() {
     AttnGroup g = {m1, m2, q, kk, v, scale, -1};
     const int gi = static_cast<int>(attn_groups_.size());
     attn_groups_.push_back(g);
-    NDObject *members[] = {m1, mul, x, mx, sb, e, sm, dv, p, m2};
+    NDObject *members[] = {m1, mul, x, mul32, mx, sb, e, sm, dv, p, m2};
     for (NDObject *mbr : members)
       if (mbr != nullptr) attn_of_[mbr->id] = gi;
   }

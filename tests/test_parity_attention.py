@@ -87,3 +87,23 @@ def test_attention_full_size_heads():  # BASELINE config 4 shape, three sampled 
     for b, h in ((0, 0), (3, 17), (7, 31)):
         want = np_attention(q[b, h], k[b, h], v[b, h])
         assert np.allclose(got[b, h], want, rtol=1e-2, atol=1e-2), (b, h, np.abs(got[b, h] - want).max())
+
+
+@pytest.mark.parametrize("dt", ["float16", "bfloat16"])
+def test_attention_fused_with_the_scale_behind_the_cast(dt):
+    # the same graph with the scores scaled in fp32 (cast first, then the multiply): recognised as well
+    rng = np.random.default_rng(77)
+    conv = (lambda x: x.astype(np.float16)) if dt == "float16" else _bf16
+    q, k, v = (conv(rng.standard_normal((3, n, 128))) for n in (200, 320, 320))
+    t = Tester("mix")
+    dts = dt if dt == "bfloat16" else None
+    lq, lk, lv = t.load(q, dts), t.load(k, dts), t.load(v, dts)
+    x = t.mul(t.cast(t.matmul(lq, lk, False, True), "float32"), 1.0 / math.sqrt(128))
+    e = t.exp(t.sub(x, t.max(x, (2,), True)))
+    out = t.store(t.matmul(t.cast(t.div(e, t.sum(e, (2,), True)), dt), lv, False, False))
+    t.run()
+    assert "entry attention" in t.das() and t.num_launches() == 1, t.das()
+    got = t.output(out)
+    got = Tester.convert_from_bf16(got) if dt == "bfloat16" else got
+    want = np_attention(q, k, v)
+    assert np.allclose(got, want, rtol=1e-2, atol=1e-2), np.abs(got - want).max()
