@@ -493,6 +493,14 @@ __device__ __forceinline__ double red_identity(uint32_t kind) {
   return __builtin_huge_val();
 }
 
+template <int CTRL>
+__device__ __forceinline__ double dpp_f64(double v) {
+  int lo = __double2loint(v), hi = __double2hiint(v);
+  lo = __builtin_amdgcn_update_dpp(lo, lo, CTRL, 0xf, 0xf, false);
+  hi = __builtin_amdgcn_update_dpp(hi, hi, CTRL, 0xf, 0xf, false);
+  return __hiloint2double(hi, lo);
+}
+
 __device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
   int lo = __double2loint(v), hi = __double2hiint(v);
   lo = __shfl_xor(lo, mask, 64);
@@ -637,7 +645,27 @@ __device__ __forceinline__ void red_finish_x(double &r0, double &r1, uint32_t k0
   const bool on0 = k0 <= VR_MIN, on1 = k1 <= VR_MIN;
   double t0 = r0, t1 = r1;
   const uint32_t span = team_is_block ? 64u : (1u << tlog);
-  for (uint32_t msk = 1; msk < span; msk <<= 1) {
+  // Inside a row of 16 lanes the partner's value comes through the data-parallel-primitive path of the vector unit
+  // (neighbour, next pair, the mirror image within 8 and within 16: each step doubles the lanes whose partials a lane
+  // holds, and both partners compute the same sum), which costs an instruction instead of a trip through local
+  // memory; the rows of a wave are combined by shuffles.
+  if (span > 1u) {
+    if (on0) t0 = red_combine(k0, t0, dpp_f64<0xB1>(t0));  // quad_perm [1,0,3,2]
+    if (on1) t1 = red_combine(k1, t1, dpp_f64<0xB1>(t1));
+  }
+  if (span > 2u) {
+    if (on0) t0 = red_combine(k0, t0, dpp_f64<0x4E>(t0));  // quad_perm [2,3,0,1]
+    if (on1) t1 = red_combine(k1, t1, dpp_f64<0x4E>(t1));
+  }
+  if (span > 4u) {
+    if (on0) t0 = red_combine(k0, t0, dpp_f64<0x141>(t0));  // row_half_mirror
+    if (on1) t1 = red_combine(k1, t1, dpp_f64<0x141>(t1));
+  }
+  if (span > 8u) {
+    if (on0) t0 = red_combine(k0, t0, dpp_f64<0x140>(t0));  // row_mirror
+    if (on1) t1 = red_combine(k1, t1, dpp_f64<0x140>(t1));
+  }
+  for (uint32_t msk = 16; msk < span; msk <<= 1) {
     if (on0) t0 = red_combine(k0, t0, shfl_xor_f64(t0, msk));
     if (on1) t1 = red_combine(k1, t1, shfl_xor_f64(t1, msk));
   }
@@ -653,9 +681,17 @@ __device__ __forceinline__ void red_finish_x(double &r0, double &r1, uint32_t k0
     const double a0 = buf[j], a1 = buf[16 + j];
     t0 = j < nw ? a0 : red_identity(k0);
     t1 = j < nw ? a1 : red_identity(k1);
-    for (uint32_t msk = 1; msk < 16u; msk <<= 1) {
-      if (on0) t0 = red_combine(k0, t0, shfl_xor_f64(t0, msk));
-      if (on1) t1 = red_combine(k1, t1, shfl_xor_f64(t1, msk));
+    if (on0) {  // the 16 partials of a row of lanes: the same four steps
+      t0 = red_combine(k0, t0, dpp_f64<0xB1>(t0));
+      t0 = red_combine(k0, t0, dpp_f64<0x4E>(t0));
+      t0 = red_combine(k0, t0, dpp_f64<0x141>(t0));
+      t0 = red_combine(k0, t0, dpp_f64<0x140>(t0));
+    }
+    if (on1) {
+      t1 = red_combine(k1, t1, dpp_f64<0xB1>(t1));
+      t1 = red_combine(k1, t1, dpp_f64<0x4E>(t1));
+      t1 = red_combine(k1, t1, dpp_f64<0x141>(t1));
+      t1 = red_combine(k1, t1, dpp_f64<0x140>(t1));
     }
   }
   r0 = t0;
