@@ -340,6 +340,7 @@ class Compiler {
   // emission helpers
   void Emit(uint32_t op, uint32_t sub, uint32_t kind, uint32_t rnd, uint32_t a, uint32_t imm);
   void DropCastBeforeStore(const uint32_t *mem_dtypes);
+  void DropUnreadSRegStores();
   void FuseSweepInstructions();
   void MarkUniformRuns();
   void PairLoads();

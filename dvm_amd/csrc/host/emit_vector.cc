@@ -650,6 +650,7 @@ void Compiler::FinishProgram() {
     for (int i = 0; i < n_mem_; ++i) dts[i] = mems_[i].dtype;
     DropCastBeforeStore(dts);
   }
+  DropUnreadSRegStores();
   // tuning switches: DVM_VEC_FUSE=0 keeps the instruction stream as emitted, DVM_VEC_UNIRUN=0 lets every wave
   // execute the per-team runs
   static const bool fuse = !(std::getenv("DVM_VEC_FUSE") != nullptr && std::getenv("DVM_VEC_FUSE")[0] == '0');

@@ -10,6 +10,29 @@
 
 namespace dvm {
 
+// A value is copied into an S register wherever a later round of a sweep may need it again; when every row fits one
+// round nothing reads some of those registers (the maximum of a softmax row stays in the accumulator): the copies go.
+// A dispatch each, of the 18 a row of such a softmax takes.
+void Compiler::DropUnreadSRegStores() {
+  uint32_t read = 0;
+  for (uint64_t w : code_) {
+    const uint32_t op = VI_OP(w);
+    if (op == VOP_LDS) read |= 1u << VI_A(w);
+    if (op >= VOP_SRC_BASE && (VI_KIND(w) == VK_SREG || VI_KIND(w) == VK_SREG2)) {
+      read |= 1u << VI_A(w);
+      if (VI_KIND(w) == VK_SREG2) read |= 1u << ((VI_IMM(w) >> 8) & 0xffu);
+    }
+  }
+  std::vector<uint64_t> &out = scratch_code_;
+  out.clear();
+  out.reserve(code_.size());
+  for (uint64_t w : code_) {
+    if (VI_OP(w) == VOP_STS && VI_A(w) < 32 && !((read >> VI_A(w)) & 1u)) continue;
+    out.push_back(w);
+  }
+  code_.swap(out);
+}
+
 // A rounding cast to fp16 / bf16 whose only reader is the store right behind it does nothing the store's own
 // conversion does not do (same round to nearest even): the cast instruction is dropped. `mem_dtypes[i]` is the
 // element type of memory operand i.
@@ -111,6 +134,15 @@ void Compiler::FuseSweepInstructions() {
     if (VI_OP(w) == VOP_RED && VI_SUB(w) == VR_SUM && VI_A(w) == 0 && i + 2 < out.size() && VI_OP(out[i + 1]) == VOP_RED &&
         VI_SUB(out[i + 1]) == (VR_SUM | VRF_SQUARE) && VI_A(out[i + 1]) == 1 && VI_OP(out[i + 2]) == VOP_ENDSWEEP) {
       code_.push_back(w | (static_cast<uint64_t>(VRF_PAIR) << 8) | VI_ENDS);
+      i += 2;
+      continue;
+    }
+    // reduce ; copy to a V register ; endsweep  ->  the copy first (a plain reduce leaves the accumulator as it is), so
+    // that the reduce can close the round
+    if (VI_OP(w) == VOP_RED && !(VI_SUB(w) & (VRF_SQUARE | VRF_PAIR)) && i + 2 < out.size() && VI_OP(out[i + 1]) == VOP_STR &&
+        VI_OP(out[i + 2]) == VOP_ENDSWEEP) {
+      code_.push_back(out[i + 1]);
+      code_.push_back(w | VI_ENDS);
       i += 2;
       continue;
     }
@@ -243,6 +275,14 @@ void Compiler::PlanRereads() {
       const uint64_t imm = static_cast<uint64_t>(rounds | (prefix << 16) | (fmt << 20)) << 32;
       cw[la] |= VI_LD_KEEP_WR | imm;
       cw[lb] |= VI_LD_KEEP_RD | imm;
+      // a third sweep over the same operand (the division of a softmax) takes the parked rounds as well
+      for (size_t c = b + 1; c < sweeps.size(); ++c) {
+        if (sweeps[c].ld < 0 || VI_A(cw[sweeps[c].ld]) != VI_A(cw[la])) continue;
+        const size_t lc = static_cast<size_t>(sweeps[c].ld);
+        if (prefix != 0 && (lc + 1 >= n || cw[lc + 1] != cw[la + 1])) continue;
+        if (static_cast<uint32_t>(cw[lc]) & (VI_LD_KEEP_WR | VI_LD_KEEP_RD | VI_LD_RED2)) continue;
+        cw[lc] |= VI_LD_KEEP_RD | imm;
+      }
       prog_->lds_bytes += rounds * round_bytes;
       return;
     }
