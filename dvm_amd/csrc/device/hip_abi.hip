@@ -37,6 +37,10 @@ extern "C" __global__ void dvm_vm_attn_f16(const VmParam p);
 extern "C" __global__ void dvm_vm_attn_bf16(const VmParam p);
 extern "C" __global__ void dvm_vm_attn_f16_w8(const VmParam p);
 extern "C" __global__ void dvm_vm_attn_bf16_w8(const VmParam p);
+extern "C" __global__ void dvm_vm_attn_f16_d64(const VmParam p);
+extern "C" __global__ void dvm_vm_attn_bf16_d64(const VmParam p);
+extern "C" __global__ void dvm_vm_attn_f16_w8_d64(const VmParam p);
+extern "C" __global__ void dvm_vm_attn_bf16_w8_d64(const VmParam p);
 
 typedef void (*CubeKernel)(const VmParam);
 #define DVM_CUBE_ROW(prefix) {prefix##_nn, prefix##_nt, prefix##_tn, prefix##_tt}
@@ -262,17 +266,20 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
   } else if (h->entry == VE_ATTN) {
     const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.w);
     // the kernel has no guards of its own beyond the query tail: the header must fit it exactly
-    if (a->d != DVM_ATTN_D || a->skv == 0 || a->skv % DVM_ATTN_BKV != 0 || a->sq == 0 || a->nb == 0 ||
+    if (!DVM_ATTN_D_OK(a->d) || a->skv == 0 || a->skv % DVM_ATTN_BKV != 0 || a->sq == 0 || a->nb == 0 ||
         a->q_blocks != (a->sq + DVM_ATTN_BQ - 1) / DVM_ATTN_BQ || static_cast<uint64_t>(a->nb) * a->q_blocks != block_dim || (threads != 256 && threads != 512) ||
-        lds_bytes < DVM_ATTN_LDS_BYTES || a->q_addr == 0 || a->k_addr == 0 || a->v_addr == 0 || a->o_addr == 0 ||
+        lds_bytes < DVM_ATTN_LDS_BYTES_D(a->d) || a->q_addr == 0 || a->k_addr == 0 || a->v_addr == 0 || a->o_addr == 0 ||
         ((a->q_addr | a->k_addr | a->v_addr | a->o_addr) & 15u) != 0 || (a->dtype != VDT_F16 && a->dtype != VDT_BF16)) {
       return static_cast<int>(hipErrorInvalidValue);
     }
     // 256 lanes: four waves of 64 queries; 512 lanes: eight waves of 32 queries (same tile of 256 queries)
+    const bool bf = a->dtype == VDT_BF16, narrow = a->d != DVM_ATTN_D;
     if (threads == 512) {
-      hipLaunchKernelGGL(a->dtype == VDT_BF16 ? dvm_vm_attn_bf16_w8 : dvm_vm_attn_f16_w8, dim3(block_dim), dim3(512), lds_bytes, s, p);
+      hipLaunchKernelGGL(narrow ? (bf ? dvm_vm_attn_bf16_w8_d64 : dvm_vm_attn_f16_w8_d64) : (bf ? dvm_vm_attn_bf16_w8 : dvm_vm_attn_f16_w8),
+                         dim3(block_dim), dim3(512), lds_bytes, s, p);
     } else {
-      hipLaunchKernelGGL(a->dtype == VDT_BF16 ? dvm_vm_attn_bf16 : dvm_vm_attn_f16, dim3(block_dim), dim3(256), lds_bytes, s, p);
+      hipLaunchKernelGGL(narrow ? (bf ? dvm_vm_attn_bf16_d64 : dvm_vm_attn_f16_d64) : (bf ? dvm_vm_attn_bf16 : dvm_vm_attn_f16), dim3(block_dim),
+                         dim3(256), lds_bytes, s, p);
     }
   } else {
     return static_cast<int>(hipErrorInvalidValue);

@@ -40,7 +40,6 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 
-constexpr int D = DVM_ATTN_D;      // head dimension
 constexpr int BKV = DVM_ATTN_BKV;  // keys per block
 constexpr int ROW = 64;            // elements per local-memory tile row (128 bytes)
 
@@ -76,15 +75,18 @@ __device__ __forceinline__ uint32_t tile_off(uint32_t row, uint32_t chunk) {
   return row * ROW + ((chunk ^ ((row ^ (row >> 3)) & 7u)) << 3);
 }
 
-// Local memory per buffer: K block and V block, each as two tiles [64 keys][64 d] (d halves).
+// Local memory per buffer: K block and V block, each as D / 64 tiles [64 keys][64 d] (two d halves at D = 128).
 constexpr uint32_t kKTile = BKV * ROW;  // elements of one half tile
-constexpr uint32_t kVOff = 2 * kKTile;  // V block after the K block
-constexpr uint32_t kBuf = 4 * kKTile;   // elements per buffer
 
 // NQT: 32-query tiles per wave. 2: four waves of 64 queries, one per SIMD with all 512 registers; 1: eight waves of
 // 32 queries, two per SIMD, so that one wave's softmax (vector ALU) runs under the other's MFMAs.
-template <bool IS_BF16, int NQT>
+// D: head dimension, 64 or 128.
+template <bool IS_BF16, int NQT, int D>
 __device__ __forceinline__ void vm_attn(const VmParam &p) {
+  static_assert(D == 64 || D == 128, "head dimension");
+  constexpr int HT = D / 64;                  // half tiles per K or V block
+  constexpr uint32_t kVOff = HT * kKTile;     // V block after the K block
+  constexpr uint32_t kBuf = 2 * HT * kKTile;  // elements per buffer
   constexpr int WQ = 32 * NQT;             // query rows per wave
 #ifndef DVM_ATTN_PIN8
 #define DVM_ATTN_PIN8 1
@@ -142,7 +144,7 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
     const DVM_GLOBAL char *ksrc = reinterpret_cast<const DVM_GLOBAL char *>(k_base + static_cast<uint64_t>(key0) * D * 2);
     const DVM_GLOBAL char *vsrc = reinterpret_cast<const DVM_GLOBAL char *>(v_base + static_cast<uint64_t>(key0) * D * 2);
 #pragma unroll
-    for (int i = 0; i < 2 * STEPS; ++i) {
+    for (int i = 0; i < HT * STEPS; ++i) {
       // step i % STEPS of half tile i / STEPS: later keys, then d 64..
       const uint32_t src_off = (i % STEPS) * KPS * D * 2u + (i / STEPS) * 64u * 2u + ld_off[(i % STEPS) & 1];
       const uint32_t dst_off = (static_cast<uint32_t>(i) * NTHR + wave_first) * 8u;
@@ -287,9 +289,9 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
         for (int qt = 0; qt < NQT; ++qt) o_acc[dt][qt] = mfma<IS_BF16>(vf[step & 1][dt], pf[step >> 1][step & 1][qt], o_acc[dt][qt]);
       if (step + 1 < 4 && PIN) {  // the eight transposing reads of the next step between the 4 * NQT MFMAs of this one
 #pragma unroll
-        for (int q = 0; q < 4 * NQT; ++q) {
+        for (int q = 0; q < (D / 32) * NQT; ++q) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x100, 8 / (4 * NQT), 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 2 / NQT, 0);
         }
       }
     }
@@ -333,7 +335,12 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
 
 }  // namespace
 
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_f16(const VmParam p) { vm_attn<false, 2>(p); }
-extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_bf16(const VmParam p) { vm_attn<true, 2>(p); }
-extern "C" __global__ void __launch_bounds__(512) dvm_vm_attn_f16_w8(const VmParam p) { vm_attn<false, 1>(p); }
-extern "C" __global__ void __launch_bounds__(512) dvm_vm_attn_bf16_w8(const VmParam p) { vm_attn<true, 1>(p); }
+extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_f16(const VmParam p) { vm_attn<false, 2, 128>(p); }
+extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_bf16(const VmParam p) { vm_attn<true, 2, 128>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_attn_f16_w8(const VmParam p) { vm_attn<false, 1, 128>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_attn_bf16_w8(const VmParam p) { vm_attn<true, 1, 128>(p); }
+// head dimension 64
+extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_f16_d64(const VmParam p) { vm_attn<false, 2, 64>(p); }
+extern "C" __global__ void __launch_bounds__(256) dvm_vm_attn_bf16_d64(const VmParam p) { vm_attn<true, 2, 64>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_attn_f16_w8_d64(const VmParam p) { vm_attn<false, 1, 64>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_attn_bf16_w8_d64(const VmParam p) { vm_attn<true, 1, 64>(p); }

@@ -22,7 +22,7 @@ void Compiler::CompileAttn(int gi) {
   h.nb = static_cast<uint32_t>(nb);
   h.sq = static_cast<uint32_t>(g.q->dim(r - 2));
   h.skv = static_cast<uint32_t>(g.k->dim(r - 2));
-  h.d = DVM_ATTN_D;
+  h.d = static_cast<uint32_t>(g.q->dim(r - 1));
   h.scale = g.scale;
   h.q_blocks = (h.sq + DVM_ATTN_BQ - 1) / DVM_ATTN_BQ;
   if (static_cast<uint64_t>(h.nb) * h.q_blocks >= (1ull << 31)) Fail("too many attention blocks");
@@ -52,7 +52,7 @@ void Compiler::CompileAttn(int gi) {
   // on fp16 [8,32,2048,128] against 920-940 us for four waves of 64 queries; DVM_ATTN_WAVES=4 selects the latter
   prog_->threads = 512;
   if (k_->tuning_.attn_waves == 4) prog_->threads = 256;
-  prog_->lds_bytes = DVM_ATTN_LDS_BYTES;
+  prog_->lds_bytes = DVM_ATTN_LDS_BYTES_D(h.d);
   prog_->grid = h.nb * h.q_blocks;
 }
 }  // namespace dvm

@@ -478,7 +478,7 @@ void Compiler::DetectAttention() {
     if (q->kind != kObjLoad || kk->kind != kObjLoad || v->kind != kObjLoad || q->strided || kk->strided || v->strided) continue;
     const int r = q->rank();
     if (kk->rank() != r || v->rank() != r || r < 2) continue;
-    bool ok = q->dim(r - 1) == DVM_ATTN_D && kk->dim(r - 1) == DVM_ATTN_D && v->dim(r - 1) == DVM_ATTN_D && kk->dim(r - 2) == v->dim(r - 2) &&
+    bool ok = DVM_ATTN_D_OK(q->dim(r - 1)) && kk->dim(r - 1) == q->dim(r - 1) && v->dim(r - 1) == q->dim(r - 1) && kk->dim(r - 2) == v->dim(r - 2) &&
               kk->dim(r - 2) % DVM_ATTN_BKV == 0 && kk->dim(r - 2) > 0 && q->dim(r - 2) > 0;
     for (int d = 0; d < r - 2 && ok; ++d) ok = q->dim(d) == kk->dim(d) && q->dim(d) == v->dim(d) && q->dim(d) > 0;
     if (!ok || q->numel() >= (1ll << 31) || kk->numel() >= (1ll << 31)) continue;

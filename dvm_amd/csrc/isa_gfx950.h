@@ -302,15 +302,17 @@ typedef struct {
 // online softmax (running row max and sum), so the [sq][skv] score matrix never exists in memory.
 #define DVM_ATTN_BQ 256
 #define DVM_ATTN_BKV 64
-#define DVM_ATTN_D 128
-#define DVM_ATTN_LDS_BYTES (2u * 2u * DVM_ATTN_BKV * DVM_ATTN_D * 2u)
+#define DVM_ATTN_D 128                  // head dimension: this, or half of it
+#define DVM_ATTN_D_OK(d) ((d) == DVM_ATTN_D || (d) == DVM_ATTN_D / 2)
+#define DVM_ATTN_LDS_BYTES_D(d) (2u * 2u * DVM_ATTN_BKV * (d) * 2u)  // two buffers of a K block and a V block
+#define DVM_ATTN_LDS_BYTES DVM_ATTN_LDS_BYTES_D(DVM_ATTN_D)
 
 typedef struct {
   uint32_t entry;   // VE_ATTN
   uint32_t dtype;   // VDT_F16 or VDT_BF16
   uint32_t nb;      // batch * heads
   uint32_t sq, skv; // query rows, keys (skv a multiple of DVM_ATTN_BKV)
-  uint32_t d;       // head dimension (DVM_ATTN_D)
+  uint32_t d;       // head dimension: 128 or 64 (DVM_ATTN_D_OK)
   float scale;      // applied to Q K^T before the softmax
   uint32_t q_blocks;  // ceil(sq / DVM_ATTN_BQ)
   uint64_t q_addr, k_addr, v_addr, o_addr;

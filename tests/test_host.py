@@ -321,8 +321,10 @@ def _attention(t, sq, skv, d):
 def test_attention_graph_is_recognised():
     das = _attention(Tester("mix", run_mode="das"), 300, 192, 128)
     assert das.count("== sub-kernel") == 1 and "entry attention fp16 batch=2 sq=300 skv=192 d=128 scale=0.125" in das, das
+    das = _attention(Tester("mix", run_mode="das"), 300, 192, 64)
+    assert das.count("== sub-kernel") == 1 and "entry attention fp16 batch=2 sq=300 skv=192 d=64 " in das and "lds=32768" in das, das
     # other head sizes or ragged key counts run as matmul, softmax, matmul
-    for sq, skv, d in ((300, 192, 64), (300, 100, 128)):
+    for sq, skv, d in ((300, 192, 96), (300, 100, 128), (300, 100, 64)):
         das = _attention(Tester("mix", run_mode="das"), sq, skv, d)
         assert das.count("== sub-kernel") == 3 and das.count("entry cube") == 2 and "entry attention" not in das, das
 

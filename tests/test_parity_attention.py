@@ -107,3 +107,35 @@ def test_attention_fused_with_the_scale_behind_the_cast(dt):
     got = Tester.convert_from_bf16(got) if dt == "bfloat16" else got
     want = np_attention(q, k, v)
     assert np.allclose(got, want, rtol=1e-2, atol=1e-2), np.abs(got - want).max()
+
+
+@pytest.mark.parametrize("waves", ["8", "4"])
+@pytest.mark.parametrize("shape", [((2, 3), 256, 192), ((1,), 64, 64), ((3,), 100, 128), ((2,), 300, 1024), ((), 513, 640)])
+@pytest.mark.parametrize("dt", ["float16", "bfloat16"])
+def test_attention_fused_head_dimension_64(monkeypatch, shape, dt, waves):
+    # the same kernel built for a head dimension of 64 (one 64-wide tile per K and V block instead of two)
+    monkeypatch.setenv("DVM_ATTN_WAVES", waves)
+    batch, sq, skv = shape
+    rng = np.random.default_rng(sq + 1)
+    conv = (lambda x: x.astype(np.float16)) if dt == "float16" else _bf16
+    q, k, v = (conv(rng.standard_normal(batch + (n, 64))) for n in (sq, skv, skv))
+    got = _fused(q, k, v, dt)
+    want = np_attention(q, k, v)
+    assert got.shape == want.shape
+    assert np.allclose(got, want, rtol=1e-2, atol=1e-2), np.abs(got - want).max()
+
+
+def test_attention_head_dimension_64_constant_values():
+    # every row of V equal to c: the output rows are c whatever the scores; V = one-hot rows pick out softmax weights
+    rng = np.random.default_rng(5)
+    q, k = (rng.standard_normal((2, n, 64)).astype(np.float16) for n in (130, 192))
+    v = np.tile(np.linspace(-1, 1, 64, dtype=np.float16), (2, 192, 1))
+    got = _fused(q, k, v)
+    assert np.allclose(got, v[:, :1, :].astype(np.float32), atol=2e-3), np.abs(got - v[:, :1, :]).max()
+    v = np.zeros((2, 192, 64), np.float16)
+    v[:, np.arange(64) * 3, np.arange(64)] = 1.0  # output column d = weight of key 3 d
+    got = _fused(q, k, v).astype(np.float64)
+    s = np.matmul(q.astype(np.float64), np.swapaxes(k.astype(np.float64), -1, -2)) / 8.0
+    w = np.exp(s - s.max(-1, keepdims=True))
+    w /= w.sum(-1, keepdims=True)
+    assert np.allclose(got, w[:, :, ::3], rtol=1e-2, atol=1e-3), np.abs(got - w[:, :, ::3]).max()

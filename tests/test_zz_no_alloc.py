@@ -1,7 +1,7 @@
 """GPU test of dvm_hip_launch_vm_static_ws (include/dvm_hip.h): the launch entry point that allocates nothing and
 keeps the values one launch hands to the next in the library's own static workspace.
 
-The kernel is an attention graph at head dimension 64, which the fused kernel does not take: three launches
+The kernel is an attention graph at head dimension 96, which the fused kernel does not take: three launches
 (matmul, softmax with two chained reduces, matmul) and two values in the workspace. It runs through the existing
 route first (dvm_rt_run: dvm_hip_launch_vm per launch, workspace from hipMalloc), then its exported programs go
 through the new entry point via the C ABI of libdvm_hip.so; both results must agree bit for bit. Twice in a row on
@@ -56,8 +56,8 @@ def test_static_workspace_launch_matches_the_allocating_route():
     hip = _hip()
     rng = np.random.default_rng(7)
     t = Tester("mix:dyn")
-    lq, lk, lv = (t.load([1, 1, 64], "float16") for _ in range(3))
-    s = t.mul(t.matmul(lq, lk, False, True), 1.0 / math.sqrt(64))
+    lq, lk, lv = (t.load([1, 1, 96], "float16") for _ in range(3))  # (a head dimension the fused kernel does not take)
+    s = t.mul(t.matmul(lq, lk, False, True), 1.0 / math.sqrt(96))
     x = t.cast(s, "float32")
     x = t.sub(x, t.max(x, (2,), True))
     e = t.exp(x)
@@ -65,7 +65,7 @@ def test_static_workspace_launch_matches_the_allocating_route():
     out = t.store(t.matmul(p, lv, False, False))
 
     for heads, sq, skv in ((6, 384, 512), (2, 100, 192)):  # the second call is smaller than the first
-        q, k, v = (rng.standard_normal((heads, n, 64)).astype(np.float16) for n in (sq, skv, skv))
+        q, k, v = (rng.standard_normal((heads, n, 96)).astype(np.float16) for n in (sq, skv, skv))
         for load, arr in ((lq, q), (lk, k), (lv, v)):
             t.input(load, arr)
         t.run()  # the existing route
