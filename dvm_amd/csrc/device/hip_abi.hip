@@ -266,7 +266,7 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
   } else if (h->entry == VE_ATTN) {
     const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.w);
     // the kernel has no guards of its own beyond the query tail: the header must fit it exactly
-    if (!DVM_ATTN_D_OK(a->d) || a->skv == 0 || a->skv % DVM_ATTN_BKV != 0 || a->sq == 0 || a->nb == 0 ||
+    if (!DVM_ATTN_D_OK(a->d) || a->skv == 0 || !(a->scale > 0.0f) || a->sq == 0 || a->nb == 0 ||
         a->q_blocks != (a->sq + DVM_ATTN_BQ - 1) / DVM_ATTN_BQ || static_cast<uint64_t>(a->nb) * a->q_blocks != block_dim || (threads != 256 && threads != 512) ||
         lds_bytes < DVM_ATTN_LDS_BYTES_D(a->d) || a->q_addr == 0 || a->k_addr == 0 || a->v_addr == 0 || a->o_addr == 0 ||
         ((a->q_addr | a->k_addr | a->v_addr | a->o_addr) & 15u) != 0 || (a->dtype != VDT_F16 && a->dtype != VDT_BF16)) {

@@ -139,14 +139,20 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
     ld_off[par] = ((tid >> 3) * D + (logical << 3)) * 2u;
   }
   const uint32_t wave_first = uni(wave) * 64u;
+  // (a last block with fewer than BKV keys: the rows past the end fetch the last key again, their scores are masked)
   auto fetch_kv = [&](uint32_t key0, uint32_t buf) {
     uint16_t *kdst = lds + buf * kBuf, *vdst = lds + buf * kBuf + kVOff;
     const DVM_GLOBAL char *ksrc = reinterpret_cast<const DVM_GLOBAL char *>(k_base + static_cast<uint64_t>(key0) * D * 2);
     const DVM_GLOBAL char *vsrc = reinterpret_cast<const DVM_GLOBAL char *>(v_base + static_cast<uint64_t>(key0) * D * 2);
+    const uint32_t last_row = skv - 1u - key0;  // uniform; BKV - 1 or more in a full block
 #pragma unroll
     for (int i = 0; i < HT * STEPS; ++i) {
       // step i % STEPS of half tile i / STEPS: later keys, then d 64..
-      const uint32_t src_off = (i % STEPS) * KPS * D * 2u + (i / STEPS) * 64u * 2u + ld_off[(i % STEPS) & 1];
+      uint32_t src_off = (i % STEPS) * KPS * D * 2u + (i / STEPS) * 64u * 2u + ld_off[(i % STEPS) & 1];
+      if (last_row < static_cast<uint32_t>(BKV) - 1u) {
+        const uint32_t row = (i % STEPS) * KPS + (tid >> 3);
+        src_off -= (row > last_row ? row - last_row : 0u) * (D * 2u);
+      }
       const uint32_t dst_off = (static_cast<uint32_t>(i) * NTHR + wave_first) * 8u;
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(ksrc + src_off), (__attribute__((address_space(3))) void *)(kdst + dst_off), 16, 0, 0);
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(vsrc + src_off), (__attribute__((address_space(3))) void *)(vdst + dst_off), 16, 0, 0);
@@ -180,7 +186,7 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
   const uint32_t tr_chunk = 2u * (tr_g & 1u) + (tr_q >> 1);          // 16-byte chunk inside the half d tile
   const uint32_t tr_base = tr_key * ROW + 4u * (tr_q & 1u);          // row part + the half of the chunk
   const uint32_t tr_x = (tr_chunk ^ tr_key) << 3;
-  const uint32_t n_blocks = skv / BKV;
+  const uint32_t n_blocks = (skv + BKV - 1) / BKV;
   fetch_kv(0, 0);
   __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): the barrier does not wait for direct loads by itself
   __syncthreads();
@@ -305,6 +311,17 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
     // the other buffer was read for the last time before the barrier that ended the previous block
     if (kb + 1 < n_blocks) fetch_kv((kb + 1) * BKV, cur ^ 1u);
     stage1(lds + cur * kBuf);
+    if (kb * BKV + BKV > skv) {
+      // keys past the end: register r of key tile kt holds key 32*kt + 8*(r/4) + 4*h + r%4 of the block (scale > 0)
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const uint32_t key = kb * BKV + 32u * kt + 8u * (r >> 2) + 4u * lh + (r & 3);
+#pragma unroll
+          for (int qt = 0; qt < NQT; ++qt) s[kt][qt][r] = key < skv ? s[kt][qt][r] : -1.0e30f;
+        }
+    }
     softmax();
     stage2(lds + cur * kBuf + kVOff);
     __builtin_amdgcn_s_waitcnt((7 << 4) | (15 << 8));  // vmcnt(0): the next block has landed

@@ -479,7 +479,7 @@ void Compiler::DetectAttention() {
     const int r = q->rank();
     if (kk->rank() != r || v->rank() != r || r < 2) continue;
     bool ok = DVM_ATTN_D_OK(q->dim(r - 1)) && kk->dim(r - 1) == q->dim(r - 1) && v->dim(r - 1) == q->dim(r - 1) && kk->dim(r - 2) == v->dim(r - 2) &&
-              kk->dim(r - 2) % DVM_ATTN_BKV == 0 && kk->dim(r - 2) > 0 && q->dim(r - 2) > 0;
+              kk->dim(r - 2) > 0 && q->dim(r - 2) > 0 && scale > 0.0f;  // (the kernel takes maxima before it scales)
     for (int d = 0; d < r - 2 && ok; ++d) ok = q->dim(d) == kk->dim(d) && q->dim(d) == v->dim(d) && q->dim(d) > 0;
     if (!ok || q->numel() >= (1ll << 31) || kk->numel() >= (1ll << 31)) continue;
     AttnGroup g = {m1, m2, q, kk, v, scale, -1};

@@ -311,9 +311,9 @@ typedef struct {
   uint32_t entry;   // VE_ATTN
   uint32_t dtype;   // VDT_F16 or VDT_BF16
   uint32_t nb;      // batch * heads
-  uint32_t sq, skv; // query rows, keys (skv a multiple of DVM_ATTN_BKV)
+  uint32_t sq, skv; // query rows, keys (a last block of fewer than DVM_ATTN_BKV keys is masked)
   uint32_t d;       // head dimension: 128 or 64 (DVM_ATTN_D_OK)
-  float scale;      // applied to Q K^T before the softmax
+  float scale;      // applied to Q K^T before the softmax; positive
   uint32_t q_blocks;  // ceil(sq / DVM_ATTN_BQ)
   uint64_t q_addr, k_addr, v_addr, o_addr;
 } VAttnHeader;

@@ -323,8 +323,10 @@ def test_attention_graph_is_recognised():
     assert das.count("== sub-kernel") == 1 and "entry attention fp16 batch=2 sq=300 skv=192 d=128 scale=0.125" in das, das
     das = _attention(Tester("mix", run_mode="das"), 300, 192, 64)
     assert das.count("== sub-kernel") == 1 and "entry attention fp16 batch=2 sq=300 skv=192 d=64 " in das and "lds=32768" in das, das
-    # other head sizes or ragged key counts run as matmul, softmax, matmul
-    for sq, skv, d in ((300, 192, 96), (300, 100, 128), (300, 100, 64)):
+    das = _attention(Tester("mix", run_mode="das"), 300, 100, 128)  # a last block of 36 keys
+    assert das.count("== sub-kernel") == 1 and "entry attention fp16 batch=2 sq=300 skv=100 d=128 " in das, das
+    # other head sizes run as matmul, softmax, matmul
+    for sq, skv, d in ((300, 192, 96), (300, 100, 32)):
         das = _attention(Tester("mix", run_mode="das"), sq, skv, d)
         assert das.count("== sub-kernel") == 3 and das.count("entry cube") == 2 and "entry attention" not in das, das
 

@@ -139,3 +139,18 @@ def test_attention_head_dimension_64_constant_values():
     w = np.exp(s - s.max(-1, keepdims=True))
     w /= w.sum(-1, keepdims=True)
     assert np.allclose(got, w[:, :, ::3], rtol=1e-2, atol=1e-3), np.abs(got - w[:, :, ::3]).max()
+
+
+@pytest.mark.parametrize("waves", ["8", "4"])
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("sq,skv", [(100, 100), (197, 197), (64, 77), (300, 1), (33, 63), (256, 65), (40, 1000)])
+def test_attention_fused_with_a_short_last_block_of_keys(monkeypatch, waves, d, sq, skv):
+    # key counts that are no multiple of 64: the rows past the end are fetched from the last key and their scores masked.
+    # Large values in V would show a weight that leaked through the mask.
+    monkeypatch.setenv("DVM_ATTN_WAVES", waves)
+    rng = np.random.default_rng(sq * 1000 + skv)
+    q, k = (rng.standard_normal((2, n, d)).astype(np.float16) for n in (sq, skv))
+    v = (rng.standard_normal((2, skv, d)) * 4).astype(np.float16)
+    got = _fused(q, k, v)
+    want = np_attention(q, k, v)
+    assert np.allclose(got, want, rtol=1e-2, atol=2e-2), np.abs(got - want).max()
