@@ -32,6 +32,15 @@ DVM_CUBE_DECL(dvm_vm_cube_bf16_small)
 DVM_CUBE_DECL(dvm_vm_cube_f16_small)
 DVM_CUBE_DECL(dvm_vm_cube_bf16_big8)
 DVM_CUBE_DECL(dvm_vm_cube_f16_big8)
+// the builds that sum the partial tiles of a split k axis (second launch), [tile][bf16] below
+extern "C" __global__ void dvm_vm_cube_f16_big_comb(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_bf16_big_comb(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_f16_mid_comb(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_bf16_mid_comb(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_f16_small_comb(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_bf16_small_comb(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_f16_big8_comb(const VmParam p);
+extern "C" __global__ void dvm_vm_cube_bf16_big8_comb(const VmParam p);
 
 extern "C" __global__ void dvm_vm_attn_f16(const VmParam p);
 extern "C" __global__ void dvm_vm_attn_bf16(const VmParam p);
@@ -50,6 +59,10 @@ static const CubeKernel kCubeKernels[4][2][4] = {
     {DVM_CUBE_ROW(dvm_vm_cube_f16_mid), DVM_CUBE_ROW(dvm_vm_cube_bf16_mid)},
     {DVM_CUBE_ROW(dvm_vm_cube_f16_small), DVM_CUBE_ROW(dvm_vm_cube_bf16_small)},
     {DVM_CUBE_ROW(dvm_vm_cube_f16_big8), DVM_CUBE_ROW(dvm_vm_cube_bf16_big8)}};
+static const CubeKernel kCubeCombKernels[4][2] = {{dvm_vm_cube_f16_big_comb, dvm_vm_cube_bf16_big_comb},
+                                                  {dvm_vm_cube_f16_mid_comb, dvm_vm_cube_bf16_mid_comb},
+                                                  {dvm_vm_cube_f16_small_comb, dvm_vm_cube_bf16_small_comb},
+                                                  {dvm_vm_cube_f16_big8_comb, dvm_vm_cube_bf16_big8_comb}};
 
 // The workspace of dvm_hip_launch_vm_static_ws: device memory that belongs to the library's code object, one copy
 // per device. Host code never uses this name as an address: it asks the runtime for the array's address on the
@@ -134,6 +147,8 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
   for (const auto &tile : kCubeKernels)
     for (const auto &dt : tile)
       for (CubeKernel k : dt) kernels.push_back(reinterpret_cast<const void *>(k));
+  for (const auto &tile : kCubeCombKernels)
+    for (CubeKernel k : tile) kernels.push_back(reinterpret_cast<const void *>(k));
   kernels.push_back(reinterpret_cast<const void *>(dvm_vm_attn_f16));
   kernels.push_back(reinterpret_cast<const void *>(dvm_vm_attn_bf16));
   for (const void *k : kernels) {
@@ -261,7 +276,9 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
         return static_cast<int>(hipErrorInvalidValue);
       }
     }
-    const CubeKernel kern = kCubeKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0][(c->trans_a ? 2 : 0) + (c->trans_b ? 1 : 0)];
+    const CubeKernel kern = (c->epi_flags & VCF_SPLITK_COMBINE)
+                                ? kCubeCombKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0]
+                                : kCubeKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0][(c->trans_a ? 2 : 0) + (c->trans_b ? 1 : 0)];
     hipLaunchKernelGGL(kern, dim3(block_dim), dim3(want_threads), lds_bytes, s, p);
   } else if (h->entry == VE_ATTN) {
     const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.w);
