@@ -1424,6 +1424,16 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
             // the binary instruction behind the load: its operand is in src, the switch below finishes it
           } else {
             mem_load(m, off, sl, src);
+            if (op == VOP_BINF && (imm & VI_PRE_SREG)) {  // an S-register binary in front, while the operand is on its way
+              const float pv = sreg_read(sr, (imm >> 8) & 0xffu);
+              switch (imm & 0x3fu) {
+                case VB_ADD: FOR_U acc.v[u] = acc.v[u] + pv; break;
+                case VB_SUB: FOR_U acc.v[u] = acc.v[u] - pv; break;
+                case VB_RSUB: FOR_U acc.v[u] = pv - acc.v[u]; break;
+                default: FOR_U acc.v[u] = acc.v[u] * pv; break;
+              }
+              apply_rnd(acc, (imm >> 16) & 0x3u);
+            }
           }
         } else if (kind == VK_SREG) {
           const float v = sreg_read(sr, a);

@@ -174,6 +174,9 @@ std::string &VKernel::DisAssemble() {
                  << kRnd[(second >> 16) & 3] << " acc, s" << ((second >> 8) & 0xff);
               break;
             }
+            if (VI_KIND(w) == VK_MEM && (VI_IMM(w) & VI_PRE_SREG)) {
+              os << kBinF[VI_IMM(w) & 0x3f] << "." << kRnd[(VI_IMM(w) >> 16) & 3] << " acc, s" << ((VI_IMM(w) >> 8) & 0xff) << "  ; then ";
+            }
             os << kBinF[sub & 0x3f] << "." << kRnd[VI_RND(w)] << " acc, ";
             PrintSrc(os, w);
             break;

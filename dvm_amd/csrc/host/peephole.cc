@@ -67,7 +67,7 @@ void Compiler::PairLoads() {
     if (VI_OP(w) == VOP_UNI_BEGIN) in_run = true;
     if (VI_OP(w) == VOP_UNI_END) in_run = false;
     if (in_run || VI_OP(w) != VOP_LD || (static_cast<uint32_t>(w) & VI_UNIFORM)) continue;
-    if (VI_OP(nx) != VOP_BINF || VI_KIND(nx) != VK_MEM) continue;
+    if (VI_OP(nx) != VOP_BINF || VI_KIND(nx) != VK_MEM || (VI_IMM(nx) & VI_PRE_SREG)) continue;  // (the paired path runs the binary alone)
     if (!(static_cast<uint32_t>(nx) & VI_SAME_OFFS) || (static_cast<uint32_t>(nx) & (VI_UNIFORM | VI_ENDS))) continue;
     code_[i] = w | VI_LD_PAIR;
   }
@@ -115,6 +115,15 @@ void Compiler::FuseSweepInstructions() {
       if (VI_OP(n) == VOP_BINF && VI_KIND(n) == VK_SREG && !(static_cast<uint32_t>(n) & VI_UNIFORM)) {
         const uint32_t second = (VI_SUB(n) & 0x3fu) | (VI_A(n) << 8) | (VI_RND(n) << 16);
         out.push_back(VI_MAKE(VOP_BINF, VI_SUB(w), VK_SREG2, VI_RND(w), VI_A(w), second));
+        ++i;
+        continue;
+      }
+      // an S-register float binary in front of one on a memory operand: one instruction (VI_PRE_SREG)
+      const uint32_t sub1 = VI_SUB(w) & 0x3fu;
+      if (VI_OP(n) == VOP_BINF && VI_KIND(n) == VK_MEM && !(static_cast<uint32_t>(n) & VI_UNIFORM) && VI_IMM(n) == 0 &&
+          (sub1 == VB_ADD || sub1 == VB_SUB || sub1 == VB_RSUB || sub1 == VB_MUL)) {
+        const uint32_t pre = VI_PRE_SREG | sub1 | (VI_A(w) << 8) | (VI_RND(w) << 16);
+        out.push_back((n & 0xffffffffull) | (static_cast<uint64_t>(pre) << 32));
         ++i;
         continue;
       }

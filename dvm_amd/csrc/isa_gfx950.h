@@ -165,6 +165,11 @@ enum { VR_SUM = 0, VR_MAX = 1, VR_MIN = 2, VR_NONE = 15 };
 // what a later VI_SAME_OFFS refers to: that still means the instruction before this one (x * w stored where x came
 // from: the store reuses the load's offsets although the weight row was read in between).
 #define VI_OFFS_ASIDE (1u << 15)
+// VI_PRE_SREG (top bit of the immediate of a VOP_BINF with a memory operand, whose immediate is otherwise unused): an
+// S-register float binary runs in front of it, acc = acc (sub2) sreg[a2], rounded by rnd2, in the same dispatch (the
+// memory operand is on its way meanwhile): imm[7:0] sub2 (VB_ADD, VB_SUB, VB_RSUB or VB_MUL), imm[15:8] a2,
+// imm[17:16] rnd2. x * rstd * w of a normalisation is one instruction instead of two.
+#define VI_PRE_SREG (1u << 31)
 #define VI_MAKE(op, sub, kind, rnd, a, imm)                                                     \
   ((uint64_t)(op) | ((uint64_t)(sub) << 8) | ((uint64_t)(kind) << 16) | ((uint64_t)(rnd) << 20) | \
    ((uint64_t)(a) << 24) | ((uint64_t)(uint32_t)(imm) << 32))

@@ -98,3 +98,50 @@ def test_parked_sum_survives_a_mixed_type_pair(monkeypatch):
     assert np.array_equal(a, b)
     s64 = x.astype(np.float64) + y.astype(np.float64)
     assert np.allclose(a, s64 / np.abs(s64).sum(1, keepdims=True), rtol=1e-4, atol=1e-6)
+
+
+_PRE_SREG_SCRIPT = r"""
+import hashlib, sys
+import numpy as np
+from dvm_amd.tester import Tester
+rng = np.random.default_rng(21)
+rows, cols = 5000, 4096  # (one wave per row, four rounds: the statistic lives in an S register)
+x = Tester.convert_to_bf16(rng.standard_normal([rows, cols]).astype(np.float32))
+w = rng.uniform(0.5, 1.5, [cols]).astype(np.float32)
+digest = hashlib.sha256()
+fused = 0
+for first in ("mul", "add", "sub", "rsub"):
+    t = Tester("split")
+    lx = t.load(x.shape, "bfloat16"); t.input(lx, x)
+    h = t.cast(lx, "float32")
+    s = t.div(1.0, t.sqrt(t.add(t.mul(t.sum(t.mul(h, h), (1,), True), 1.0 / cols), 1e-6)))
+    y = {"mul": lambda: t.mul(h, s), "add": lambda: t.add(h, s), "sub": lambda: t.sub(h, s), "rsub": lambda: t.sub(s, h)}[first]()
+    out = t.store(t.cast(t.mul(y, t.load(w)), "bfloat16"))
+    t.run()
+    fused += t.das().count("  ; then Mul.fp32 acc, m")
+    got = t.output(out)
+    digest.update(got.tobytes())
+    h64 = Tester.convert_from_bf16(x).astype(np.float64)
+    s64 = 1.0 / np.sqrt((h64 * h64).mean(1, keepdims=True) + 1e-6)
+    y64 = {"mul": h64 * s64, "add": h64 + s64, "sub": h64 - s64, "rsub": s64 - h64}[first] * w
+    assert np.allclose(Tester.convert_from_bf16(got), y64, rtol=1e-2, atol=1e-2), first
+print(fused, digest.hexdigest())
+"""
+
+
+def test_an_s_register_binary_in_front_of_a_memory_binary_is_one_instruction():
+    # x * rstd * w: the multiply by the S register rides in the dispatch of the multiply by the weight row (VI_PRE_SREG).
+    # The same bits as with the instruction stream left as emitted (DVM_VEC_FUSE=0, read once per process: two processes).
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = {}
+    for fuse in ("1", "0"):
+        env = dict(os.environ, DVM_VEC_FUSE=fuse, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
+        p = subprocess.run([sys.executable, "-c", _PRE_SREG_SCRIPT], env=env, cwd=root, capture_output=True, text=True, timeout=100)
+        assert p.returncode == 0, p.stderr[-2000:]
+        n, digest = p.stdout.split()
+        res[fuse] = (int(n), digest)
+    assert res["1"][0] >= 3 and res["0"][0] == 0, res  # (one of the four forms may come out with its operands the other way round)
+    assert res["1"][1] == res["0"][1]
