@@ -26,7 +26,7 @@ HOST_FLAGS := -std=c++17 -O2 -fPIC -fvisibility=hidden -Wall
 
 DEV_SRC := $(sort $(wildcard $(CSRC)/device/*.hip))
 HOST_SRC := $(sort $(wildcard $(CSRC)/host/*.cc))
-HEADERS := $(CSRC)/isa_gfx950.h $(wildcard include/*.h) $(wildcard $(CSRC)/host/*.h)
+HEADERS := $(CSRC)/isa_gfx950.h $(wildcard include/*.h) $(wildcard $(CSRC)/host/*.h) $(wildcard $(CSRC)/device/*.h)
 DEV_OBJ := $(patsubst $(CSRC)/device/%.hip,$(OBJ)/%.hip.o,$(DEV_SRC)) $(OBJ)/vm_vector_u4.hip.o
 HOST_OBJ := $(patsubst $(CSRC)/host/%.cc,$(OBJ)/%.cc.o,$(HOST_SRC))
 

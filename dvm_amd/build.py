@@ -34,7 +34,7 @@ def _deps():
     out = [os.path.join(CSRC, "isa_gfx950.h")]
     inc = os.path.join(os.path.dirname(ROOT), "include")
     out += [os.path.join(inc, f) for f in os.listdir(inc)]
-    out += _sources("host", ".h")
+    out += _sources("host", ".h") + _sources("device", ".h")
     return out
 
 

@@ -16,6 +16,8 @@ extern "C" __global__ void dvm_vm_vec_rx(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_ry(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_rx_parts(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_ry_parts(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_rx_sw(const VmParam p);
+extern "C" __global__ void dvm_vm_vec_rx_sw_parts(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_pw_u4(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_rx_u4(const VmParam p);
 extern "C" __global__ void dvm_vm_vec_ry_u4(const VmParam p);
@@ -142,6 +144,7 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
   std::vector<const void *> kernels = {reinterpret_cast<const void *>(dvm_vm_vec_pw), reinterpret_cast<const void *>(dvm_vm_vec_rx),
                                        reinterpret_cast<const void *>(dvm_vm_vec_ry), reinterpret_cast<const void *>(dvm_vm_vec_rx_parts),
                                        reinterpret_cast<const void *>(dvm_vm_vec_ry_parts),
+                                       reinterpret_cast<const void *>(dvm_vm_vec_rx_sw), reinterpret_cast<const void *>(dvm_vm_vec_rx_sw_parts),
                                        reinterpret_cast<const void *>(dvm_vm_vec_pw_u4), reinterpret_cast<const void *>(dvm_vm_vec_rx_u4),
                                        reinterpret_cast<const void *>(dvm_vm_vec_ry_u4)};
   for (const auto &tile : kCubeKernels)
@@ -149,8 +152,11 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
       for (CubeKernel k : dt) kernels.push_back(reinterpret_cast<const void *>(k));
   for (const auto &tile : kCubeCombKernels)
     for (CubeKernel k : tile) kernels.push_back(reinterpret_cast<const void *>(k));
-  kernels.push_back(reinterpret_cast<const void *>(dvm_vm_attn_f16));
-  kernels.push_back(reinterpret_cast<const void *>(dvm_vm_attn_bf16));
+  for (const void *k : {reinterpret_cast<const void *>(dvm_vm_attn_f16), reinterpret_cast<const void *>(dvm_vm_attn_bf16),
+                        reinterpret_cast<const void *>(dvm_vm_attn_f16_w8), reinterpret_cast<const void *>(dvm_vm_attn_bf16_w8),
+                        reinterpret_cast<const void *>(dvm_vm_attn_f16_d64), reinterpret_cast<const void *>(dvm_vm_attn_bf16_d64),
+                        reinterpret_cast<const void *>(dvm_vm_attn_f16_w8_d64), reinterpret_cast<const void *>(dvm_vm_attn_bf16_w8_d64)})
+    kernels.push_back(k);
   for (const void *k : kernels) {
     if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(g_dev.lds_per_cu)) ==
         hipSuccess) {
@@ -192,8 +198,36 @@ uint64_t dvm_hip_select_block_thread(uint64_t kind, uint64_t item_num, uint64_t 
   return (blocks << 32) | threads;
 }
 
+// The sweep build decodes a sweep as [VOP_SWEEP] [VOP_LD] [body of at most DVM_VEC_SWEEP_BODY words, the last one
+// flagged VI_ENDS] without looking for anything else: a blob that carries VS_SWEEPS must have that shape. (The
+// table offsets have been checked by the caller.)
+static bool sweeps_flag_holds(const VmParam &p) {
+  const VVecHeader *h = reinterpret_cast<const VVecHeader *>(p.w);
+  const uint64_t *code = p.w + h->code_off;
+  for (uint32_t i = 0; i < h->n_code; ++i) {
+    const uint32_t op = VI_OP(code[i]);
+    if (op == VOP_LDR || op == VOP_STR || op == VOP_RED) return false;  // (outside a sweep)
+    if (op >= VOP_SRC_BASE || op == VOP_ST) {
+      if ((op >= VOP_SRC_BASE && VI_KIND(code[i]) == VK_REG) || ((VI_KIND(code[i]) == VK_MEM || op == VOP_ST) && VI_A(code[i]) >= h->n_mem)) return false;
+    }
+    if (op != VOP_SWEEP) continue;
+    if (i + 2 >= h->n_code || VI_OP(code[i + 1]) != VOP_LD || VI_A(code[i + 1]) >= h->n_mem) return false;
+    uint32_t j = i + 2;
+    for (;; ++j) {
+      if (j >= h->n_code || j - (i + 2) >= DVM_VEC_SWEEP_BODY) return false;
+      const uint32_t bop = VI_OP(code[j]);
+      if (bop != VOP_BINF && bop != VOP_RED && bop != VOP_ST && bop != VOP_UN && bop != VOP_CAST && bop != VOP_ENDSWEEP) return false;
+      if ((bop == VOP_ST || (bop == VOP_BINF && VI_KIND(code[j]) == VK_MEM)) && VI_A(code[j]) >= h->n_mem) return false;
+      if (bop == VOP_BINF && VI_KIND(code[j]) == VK_REG) return false;
+      if (static_cast<uint32_t>(code[j]) & VI_ENDS) break;
+    }
+    i = j;
+  }
+  return true;
+}
+
 // Checks one program blob against the launch it is to get and launches the interpreter kernel its entry type names.
-static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads, uint32_t lds_bytes, void *stream) {
+static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads, uint32_t lds_bytes, void *stream, bool check_only = false) {
   if (block_dim == 0 || threads == 0 || threads > 1024 || (threads & 63u) != 0) {
     return static_cast<int>(hipErrorInvalidValue);
   }
@@ -210,6 +244,9 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
     }
     const bool wide = (h->sched & VS_WIDE) != 0;
     if (wide && threads > 512) return static_cast<int>(hipErrorInvalidValue);
+    // the sweep build trusts the flag: it is only defined for programs that reduce the innermost axis, two slabs a lane
+    const bool sweeps = (h->sched & VS_SWEEPS) != 0;
+    if (sweeps && (wide || (h->sched & VS_KIND_MASK) != VS_REDX || !sweeps_flag_holds(p))) return static_cast<int>(hipErrorInvalidValue);
     // a reduce shared between workgroups: its parts are the outermost kept axis and cover the reduced index space
     const bool parts = h->r_chunk != 0;
     if (parts) {
@@ -237,12 +274,18 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
       need += parked * threads * u * 16;
       if (lds_bytes < need) return static_cast<int>(hipErrorInvalidValue);
     }
+    if ((h->sched & VS_KIND_MASK) > VS_REDY) return static_cast<int>(hipErrorInvalidValue);
+    if (check_only) return 0;
     switch (h->sched & VS_KIND_MASK) {
       case VS_POINTWISE:
         hipLaunchKernelGGL(wide ? dvm_vm_vec_pw_u4 : dvm_vm_vec_pw, dim3(block_dim), dim3(threads), lds_bytes, s, p);
         break;
       case VS_REDX:
-        hipLaunchKernelGGL(parts ? dvm_vm_vec_rx_parts : (wide ? dvm_vm_vec_rx_u4 : dvm_vm_vec_rx), dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        if (sweeps) {
+          hipLaunchKernelGGL(parts ? dvm_vm_vec_rx_sw_parts : dvm_vm_vec_rx_sw, dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        } else {
+          hipLaunchKernelGGL(parts ? dvm_vm_vec_rx_parts : (wide ? dvm_vm_vec_rx_u4 : dvm_vm_vec_rx), dim3(block_dim), dim3(threads), lds_bytes, s, p);
+        }
         break;
       case VS_REDY:
         hipLaunchKernelGGL(parts ? dvm_vm_vec_ry_parts : (wide ? dvm_vm_vec_ry_u4 : dvm_vm_vec_ry), dim3(block_dim), dim3(threads), lds_bytes, s, p);
@@ -279,6 +322,7 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
     const CubeKernel kern = (c->epi_flags & VCF_SPLITK_COMBINE)
                                 ? kCubeCombKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0]
                                 : kCubeKernels[c->tile][c->dtype == VDT_BF16 ? 1 : 0][(c->trans_a ? 2 : 0) + (c->trans_b ? 1 : 0)];
+    if (check_only) return 0;
     hipLaunchKernelGGL(kern, dim3(block_dim), dim3(want_threads), lds_bytes, s, p);
   } else if (h->entry == VE_ATTN) {
     const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.w);
@@ -291,6 +335,7 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
     }
     // 256 lanes: four waves of 64 queries; 512 lanes: eight waves of 32 queries (same tile of 256 queries)
     const bool bf = a->dtype == VDT_BF16, narrow = a->d != DVM_ATTN_D;
+    if (check_only) return 0;
     if (threads == 512) {
       hipLaunchKernelGGL(narrow ? (bf ? dvm_vm_attn_bf16_w8_d64 : dvm_vm_attn_f16_w8_d64) : (bf ? dvm_vm_attn_bf16_w8 : dvm_vm_attn_f16_w8),
                          dim3(block_dim), dim3(512), lds_bytes, s, p);
@@ -319,18 +364,27 @@ int dvm_hip_launch_vm_static_ws(const void *params, uint32_t n_programs, const u
     if (ws_words[2 * i] >= n_programs || ws_words[2 * i + 1] >= DVM_PARAM_WORDS) return DVM_HIP_ERROR_BAD_WS_WORD;
     const VmParam *src = static_cast<const VmParam *>(params) + ws_words[2 * i];
     if (src->w[ws_words[2 * i + 1]] >= ws_bytes) return DVM_HIP_ERROR_BAD_WS_WORD;
+    // a word listed twice would get the workspace address added twice
+    for (uint32_t j = 0; j < i; ++j)
+      if (ws_words[2 * j] == ws_words[2 * i] && ws_words[2 * j + 1] == ws_words[2 * i + 1]) return DVM_HIP_ERROR_BAD_WS_WORD;
   }
   void *ws = nullptr;
   int rc = static_ws_address(&ws);
   if (rc != 0) return rc;
-  for (uint32_t prog = 0; prog < n_programs; ++prog) {
-    VmParam p;  // the caller's blob stays as it is: the offsets become addresses in this copy
-    memcpy(&p, static_cast<const VmParam *>(params) + prog, sizeof(p));
-    for (uint32_t i = 0; i < n_ws; ++i) {
-      if (ws_words[2 * i] == prog) p.w[ws_words[2 * i + 1]] += reinterpret_cast<uint64_t>(ws);
+  // Two passes over the programs: every blob is checked against its geometry before the first one is launched.
+  // A program with nothing to do has the geometry {0, 0, 0} (the exporter's convention) and is passed over.
+  for (int pass = 0; pass < 2; ++pass) {
+    for (uint32_t prog = 0; prog < n_programs; ++prog) {
+      const uint32_t *g = geometry + 3 * prog;
+      if (g[0] == 0 && g[1] == 0 && g[2] == 0) continue;
+      VmParam p;  // the caller's blob stays as it is: the offsets become addresses in this copy
+      memcpy(&p, static_cast<const VmParam *>(params) + prog, sizeof(p));
+      for (uint32_t i = 0; i < n_ws; ++i) {
+        if (ws_words[2 * i] == prog) p.w[ws_words[2 * i + 1]] += reinterpret_cast<uint64_t>(ws);
+      }
+      rc = launch_checked(p, g[0], g[1], g[2], stream, pass == 0);
+      if (rc != 0) return rc;
     }
-    rc = launch_checked(p, geometry[3 * prog], geometry[3 * prog + 1], geometry[3 * prog + 2], stream);
-    if (rc != 0) return rc;
   }
   return 0;
 }

@@ -345,6 +345,7 @@ class Compiler {
   void MarkUniformRuns();
   void PairLoads();
   void PlanRereads();
+  bool FitsSweepBuild();
   bool mem_is_view_[DVM_VEC_MAXMEM] = {false};  // memory operand i is a strided view
   int last_mem_ = -1;         // memory operand of the last memory instruction emitted in this round, or -1
   int u_ = 2;                 // slabs per lane per instruction of the program being compiled

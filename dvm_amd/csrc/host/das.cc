@@ -193,7 +193,7 @@ std::string &VKernel::DisAssemble() {
     const VVecHeader *h = reinterpret_cast<const VVecHeader *>(p.blob.w);
     if (h->entry == VE_VECTOR) {
       static const char *sched[] = {"pointwise", "reduce-x", "reduce-y"};
-      os << "entry vector sched=" << sched[h->sched & VS_KIND_MASK] << ((h->sched & VS_WIDE) ? " wide" : "") << " blocks=" << p.grid << " threads=" << p.threads
+      os << "entry vector sched=" << sched[h->sched & VS_KIND_MASK] << ((h->sched & VS_WIDE) ? " wide" : "") << ((h->sched & VS_SWEEPS) ? " sweeps" : "") << " blocks=" << p.grid << " threads=" << p.threads
          << " lds=" << p.lds_bytes << " items=" << h->n_items << " kept=" << h->n_kidx << " red=" << h->n_ridx
          << " inner=" << h->inner_extent << " team=" << (h->team_is_block ? p.threads : (1u << h->team_log2))
          << " vslots=" << h->n_vslot;

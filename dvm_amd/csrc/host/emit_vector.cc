@@ -653,11 +653,10 @@ void Compiler::FinishProgram() {
   DropUnreadSRegStores();
   // tuning switches: DVM_VEC_FUSE=0 keeps the instruction stream as emitted, DVM_VEC_UNIRUN=0 lets every wave
   // execute the per-team runs
-  static const bool fuse = !(std::getenv("DVM_VEC_FUSE") != nullptr && std::getenv("DVM_VEC_FUSE")[0] == '0');
-  static const bool unirun = !(std::getenv("DVM_VEC_UNIRUN") != nullptr && std::getenv("DVM_VEC_UNIRUN")[0] == '0');
-  if (fuse && (hdr_.sched & VS_KIND_MASK) != VS_POINTWISE) FuseSweepInstructions();
-  if (unirun) MarkUniformRuns();
+  if (k_->tuning_.vec_fuse != 0 && (hdr_.sched & VS_KIND_MASK) != VS_POINTWISE) FuseSweepInstructions();
+  if (k_->tuning_.vec_unirun != 0) MarkUniformRuns();
   if (k_->tuning_.vec_pair != 0) PairLoads();
+  if (k_->tuning_.vec_sweeps != 0 && FitsSweepBuild()) hdr_.sched |= VS_SWEEPS;
   hdr_.n_mem = n_mem_;
   hdr_.n_code = static_cast<uint32_t>(code_.size());
   hdr_.mem_off = sizeof(VVecHeader) / 8;

@@ -175,6 +175,10 @@ struct Tuning {
   int vec_team = -1;    // DVM_VEC_TEAM=n: at most n lanes per output in reduces along the innermost axis
   int vec_runs = -1;    // DVM_VEC_RUNS=1: per-output runs only when the team is the whole workgroup
   int vec_pair = -1;   // DVM_VEC_PAIR=0: a load never takes the binary instruction behind it along
+  int vec_fuse = -1;    // DVM_VEC_FUSE=0: the instruction stream stays as emitted (no fused sweep instructions)
+  int vec_unirun = -1;  // DVM_VEC_UNIRUN=0: every wave executes the per-output runs
+  int vec_reread = -1;  // DVM_VEC_REREAD=0: nothing parked, no reversed sweeps; 2: parked rounds only; 3: reversed sweeps only
+  int vec_sweeps = -1;  // DVM_VEC_SWEEPS=0: never the sweep build of the vector VM
   int cube_tile = -1;   // DVM_CUBE_TILE=256|128|64
   int cube_waves = -1;  // DVM_CUBE_WAVES=4|8
   int red_split = -1;    // DVM_RED_SPLIT=0: never share a reduce between workgroups; N >= 2: N parts whenever the graph allows

@@ -24,6 +24,10 @@ void Tuning::Read() {
   vec_team = num("DVM_VEC_TEAM");
   vec_runs = num("DVM_VEC_RUNS");
   vec_pair = num("DVM_VEC_PAIR");
+  vec_fuse = num("DVM_VEC_FUSE");
+  vec_unirun = num("DVM_VEC_UNIRUN");
+  vec_reread = num("DVM_VEC_REREAD");
+  vec_sweeps = num("DVM_VEC_SWEEPS");
   cube_tile = num("DVM_CUBE_TILE");
   cube_waves = num("DVM_CUBE_WAVES");
   cube_exact = num("DVM_CUBE_EXACT");

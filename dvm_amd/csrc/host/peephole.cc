@@ -221,6 +221,91 @@ void Compiler::MarkUniformRuns() {
   code_.swap(out);
 }
 
+// Whether the finished instruction stream fits the sweep build of the device VM (VS_SWEEPS in isa_gfx950.h spells
+// out the vocabulary). Everything is decided from the instruction words and the operand descriptors: shapes,
+// alignment and ragged ends are the device's business on either build.
+bool Compiler::FitsSweepBuild() {
+  if ((hdr_.sched & VS_KIND_MASK) != VS_REDX || (hdr_.sched & VS_WIDE)) return false;
+  if (hdr_.n_kdim > 2 || hdr_.n_rdim > 2) return false;  // (the build walks index spaces of at most two axes)
+  auto plain_mem = [&](uint32_t a) { return (mems_[a].flags & (VMF_VEC | VMF_GATHER)) == 0; };
+  const size_t n = code_.size();
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t w = code_[i];
+    const uint32_t op = VI_OP(w), kind = VI_KIND(w);
+    if (op != VOP_SWEEP) {
+      // between the sweeps: one value per lane
+      switch (op) {
+        case VOP_END: case VOP_UNI_BEGIN: case VOP_UNI_END: case VOP_FIN: case VOP_LDS: case VOP_LDI: case VOP_STS:
+        case VOP_UN: case VOP_CAST: case VOP_ENDSWEEP:
+          break;
+        case VOP_ST:
+          if (!plain_mem(VI_A(w))) return false;
+          break;
+        case VOP_LD: case VOP_BINF: case VOP_BINI: case VOP_CMP: case VOP_MSK: case VOP_MOVM:
+          if (kind == VK_REG || (kind == VK_MEM && !plain_mem(VI_A(w)))) return false;
+          if (kind == VK_SREG2 && op != VOP_BINF) return false;
+          if (kind == VK_MEM && op == VOP_BINF && (VI_IMM(w) & VI_PRE_SREG)) return false;
+          break;
+        default:
+          return false;  // V registers
+      }
+      continue;
+    }
+    // a sweep: the load that opens it, then the body up to the instruction that closes the round
+    if (i + 2 >= n) return false;
+    const uint64_t ld = code_[i + 1];
+    if (VI_OP(ld) != VOP_LD || VI_KIND(ld) != VK_MEM || (static_cast<uint32_t>(ld) & (VI_UNIFORM | VI_ENDS))) return false;
+    const VMemDesc &ma = mems_[VI_A(ld)];
+    if ((ma.flags & (VMF_VEC | VMF_GATHER)) != VMF_VEC) return false;
+    auto walks_like_load = [&](uint32_t a) {
+      const VMemDesc &m = mems_[a];
+      if (m.flags & VMF_GATHER) return false;
+      bool none = true;
+      for (int d = 0; d < DVM_VEC_MAXR; ++d) none = none && m.rstride[d] == 0;
+      return none || std::memcmp(m.rstride, ma.rstride, sizeof(ma.rstride)) == 0;
+    };
+    size_t j = i + 2;
+    for (;; ++j) {
+      if (j >= n || j - (i + 2) >= DVM_VEC_SWEEP_BODY) return false;
+      const uint64_t b = code_[j];
+      const uint32_t bop = VI_OP(b), bk = VI_KIND(b), bsub = VI_SUB(b);
+      if (static_cast<uint32_t>(b) & VI_UNIFORM) return false;
+      switch (bop) {
+        case VOP_BINF:
+          if ((bsub & 0x3fu) > VB_MAX) return false;
+          if (bk == VK_MEM) {
+            if (!walks_like_load(VI_A(b))) return false;
+            if ((VI_IMM(b) & VI_PRE_SREG) && (VI_IMM(b) & 0x3fu) > VB_MAX) return false;
+          } else if (bk == VK_SREG2) {
+            if ((VI_IMM(b) & 0x3fu) > VB_MAX) return false;
+          } else if (bk != VK_IMM && bk != VK_SREG && bk != VK_ACC) {
+            return false;
+          }
+          break;
+        case VOP_RED:
+          if (bsub & VRF_INT) return false;
+          break;
+        case VOP_ST:
+          if (!walks_like_load(VI_A(b)) || !(mems_[VI_A(b)].flags & VMF_VEC)) return false;
+          break;
+        case VOP_UN:
+          if (bsub > VU_TRUNC) return false;
+          break;
+        case VOP_CAST:
+          if (bsub != VC_RND) return false;
+          break;
+        case VOP_ENDSWEEP:
+          break;
+        default:
+          return false;
+      }
+      if (static_cast<uint32_t>(b) & VI_ENDS) break;
+    }
+    i = j;
+  }
+  return true;
+}
+
 // A reduce with consumers reads its input twice: once for the statistics, once to apply them. What the
 // second sweep does not have to fetch again from HBM:
 //  * the first rounds of the first sweep stay in the workgroup's spare local memory (VI_LD_KEEP_WR/RD);
@@ -229,8 +314,8 @@ void Compiler::MarkUniformRuns() {
 // Called with the blob filled in and lds_bytes set; edits the instruction words in the blob.
 void Compiler::PlanRereads() {
   // tuning switch DVM_VEC_REREAD: 0 off, 2 parked rounds only, 3 reversed sweeps only (default: both)
-  static const char mode = std::getenv("DVM_VEC_REREAD") != nullptr ? std::getenv("DVM_VEC_REREAD")[0] : '1';
-  const bool on = mode != '0', park = mode != '3', reverse = mode != '2';
+  const int mode = k_->tuning_.vec_reread;
+  const bool on = mode != 0, park = mode != 3, reverse = mode != 2;
   if (!on || (hdr_.sched & VS_KIND_MASK) != VS_REDX || (hdr_.sched & VS_WIDE)) return;
   uint64_t *cw = prog_->blob.w + hdr_.code_off;
   const size_t n = code_.size();
