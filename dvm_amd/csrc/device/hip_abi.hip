@@ -204,6 +204,16 @@ uint64_t dvm_hip_select_block_thread(uint64_t kind, uint64_t item_num, uint64_t 
 static bool sweeps_flag_holds(const VmParam &p) {
   const VVecHeader *h = reinterpret_cast<const VVecHeader *>(p.w);
   const uint64_t *code = p.w + h->code_off;
+  const VMemDesc *mems = reinterpret_cast<const VMemDesc *>(p.w + h->mem_off);
+  if (h->n_kdim > 2 || h->n_rdim > 2) return false;
+  // an operand of a sweep is accessed without guards in the interior rounds: contiguous and 16-byte aligned, or one
+  // fp32 element per slab
+  auto unguarded_ok = [&](uint32_t a, bool must_be_wide) {
+    const VMemDesc &m = mems[a];
+    constexpr uint32_t kWide = VMF_VEC | VMF_ALIGNED;
+    if ((m.flags & (kWide | VMF_GATHER)) == kWide) return (m.addr & 15u) == 0;
+    return !must_be_wide && (m.flags & (VMF_VEC | VMF_GATHER)) == 0 && m.dtype == VDT_F32;
+  };
   for (uint32_t i = 0; i < h->n_code; ++i) {
     const uint32_t op = VI_OP(code[i]);
     if (op == VOP_LDR || op == VOP_STR || op == VOP_RED) return false;  // (outside a sweep)
@@ -211,13 +221,14 @@ static bool sweeps_flag_holds(const VmParam &p) {
       if ((op >= VOP_SRC_BASE && VI_KIND(code[i]) == VK_REG) || ((VI_KIND(code[i]) == VK_MEM || op == VOP_ST) && VI_A(code[i]) >= h->n_mem)) return false;
     }
     if (op != VOP_SWEEP) continue;
-    if (i + 2 >= h->n_code || VI_OP(code[i + 1]) != VOP_LD || VI_A(code[i + 1]) >= h->n_mem) return false;
+    if (i + 2 >= h->n_code || VI_OP(code[i + 1]) != VOP_LD || VI_A(code[i + 1]) >= h->n_mem || !unguarded_ok(VI_A(code[i + 1]), true)) return false;
     uint32_t j = i + 2;
     for (;; ++j) {
       if (j >= h->n_code || j - (i + 2) >= DVM_VEC_SWEEP_BODY) return false;
       const uint32_t bop = VI_OP(code[j]);
       if (bop != VOP_BINF && bop != VOP_RED && bop != VOP_ST && bop != VOP_UN && bop != VOP_CAST && bop != VOP_ENDSWEEP) return false;
-      if ((bop == VOP_ST || (bop == VOP_BINF && VI_KIND(code[j]) == VK_MEM)) && VI_A(code[j]) >= h->n_mem) return false;
+      if ((bop == VOP_ST || (bop == VOP_BINF && VI_KIND(code[j]) == VK_MEM)) &&
+          (VI_A(code[j]) >= h->n_mem || !unguarded_ok(VI_A(code[j]), bop == VOP_ST))) return false;
       if (bop == VOP_BINF && VI_KIND(code[j]) == VK_REG) return false;
       if (static_cast<uint32_t>(code[j]) & VI_ENDS) break;
     }

@@ -23,7 +23,8 @@
 
 namespace {
 
-
+// the program, copied from the kernel argument once per workgroup
+__shared__ uint32_t prog_lds[DVM_PARAM_BYTES / 4];
 
 // acc = acc (sub) s with one value s per lane
 __device__ __forceinline__ void lane_binary(Acc &acc, uint32_t sub, float s) {
@@ -94,19 +95,52 @@ __device__ __forceinline__ float round_to(float x, uint32_t rnd) {
   return rnd == VRND_F16 ? round_f16(x) : (rnd == VRND_BF16 ? round_bf16(x) : x);
 }
 
+// Builds with -DDVM_VEC_STAMPS write the memory clock (100 MHz) at the marks below, one row of sixteen stamps per
+// wave, to the address in the last word of the blob when that word is not zero: where a launch spends its time,
+// wave by wave. Nothing of it exists in a regular build.
+#ifdef DVM_VEC_STAMPS
+#define STAMP()                                                                                               \
+  do {                                                                                                        \
+    if (stamp_base != 0 && stamp_n < 32u) {                                                                   \
+      const uint64_t now = __builtin_amdgcn_s_memrealtime();                                                  \
+      if ((threadIdx.x & 63u) == 0u)                                                                          \
+        reinterpret_cast<DVM_GLOBAL uint64_t *>(stamp_base)[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 32u + stamp_n] = now; \
+      ++stamp_n;                                                                                              \
+    }                                                                                                         \
+  } while (0)
+#else
+#define STAMP() do {} while (0)
+#endif
+
 template <bool PARTS>
 __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
-  // Everything the kernel needs of the blob is read word by word from the kernel argument (scalar loads at uniform
-  // indices); no pointer into it is ever handed to a function that is not inlined.
+#ifdef DVM_VEC_STAMPS
+  const uint64_t stamp_base = p.w[DVM_PARAM_WORDS - 1];  // (a scalar load from the kernel argument)
+  uint32_t stamp_n = 0;
+#endif
+  // The blob arrives as a kernel argument, and that segment may live in host memory, uncached: every scalar load
+  // from it is then a trip over the bus (0.8 us measured per instruction word read that way). So the workgroup
+  // copies the words the program occupies into local memory once, in one trip, and decodes from there.
+  {
+    const uint32_t *src = reinterpret_cast<const uint32_t *>(p.w);
+    const VVecHeader *hp = reinterpret_cast<const VVecHeader *>(p.w);
+    uint32_t used = (hp->code_off + hp->n_code) * 2;
+    used = used < DVM_PARAM_BYTES / 4 ? used : DVM_PARAM_BYTES / 4;
+    const uint32_t trips = (used + blockDim.x - 1) / blockDim.x;
+    for (uint32_t t = 0; t < trips; ++t) {  // uniform trip count, clamped indices: no per-lane branch
+      uint32_t i = t * blockDim.x + threadIdx.x;
+      i = i < used ? i : used - 1;
+      prog_lds[i] = src[i];
+    }
+    __syncthreads();
+  }
+  STAMP();
   // (No index is clamped: the launch checks that the tables lie inside the blob, that every operand index names a
   // descriptor and that every sweep's body ends before the program does.)
-  auto word = [&](uint32_t i) -> uint64_t { return p.w[i]; };
-  auto word32 = [&](uint32_t i) -> uint32_t {  // 32-bit word i of the blob
-    const uint64_t w = word(i >> 1);
-    return static_cast<uint32_t>((i & 1u) ? (w >> 32) : w);
-  };
+  const vu2 *prog64 = reinterpret_cast<const vu2 *>(prog_lds);
+  auto word32 = [&](uint32_t i) -> uint32_t { return uni(prog_lds[i]); };  // 32-bit word i of the blob
   // Header fields the rounds of a sweep need stay in scalar registers; the others are read where they are used
-  // (HDR_NOW: the index passes through an empty assembly statement, so the compiler cannot move the load to the top
+  // (HDR_NOW: the index passes through an empty assembly statement, so the compiler cannot move the read to the top
   // of the kernel and keep its result alive through every loop: scalar registers are what this kernel runs out of).
 #define HDR(field) word32(static_cast<uint32_t>(offsetof(VVecHeader, field) / 4))
 #define HDR_NOW(field) word32(fresh_s(static_cast<uint32_t>(offsetof(VVecHeader, field) / 4)))
@@ -115,25 +149,26 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
   const uint32_t mem_off = HDR(mem_off), code_off = HDR(code_off);
   // the first axis of the reduced index space (the host gives this build programs of at most two kept and two reduced axes)
   const uint32_t rd_extent = HDR(rdims[0].extent), rd_magic = HDR(rdims[0].magic), rd_shift = HDR(rdims[0].shift);
-  auto code_at = [&](uint32_t pc) -> vu2 {
-    const uint64_t w = word(code_off + pc);
-    return vu2{static_cast<uint32_t>(w), static_cast<uint32_t>(w >> 32)};
+  auto code_at = [&](uint32_t pc) -> vu2 {  // (the caller makes the halves uniform where it branches on them)
+    return prog64[code_off + pc];
   };
+  // A memory operand's descriptor. Only what the kernel branches on (element type, flags) is made wave-uniform: the
+  // address and the strides only ever enter per-lane arithmetic, where a copy in every lane serves as well.
   struct Desc {
     uint64_t addr;
     uint32_t dtype, flags, ks0, ks1, rs0, rs1;
   };
   auto desc_at = [&](uint32_t idx) -> Desc {
-    const uint64_t *dw = p.w + (mem_off + idx * static_cast<uint32_t>(sizeof(VMemDesc) / 8));
-    const uint64_t w1 = dw[1], w2 = dw[2], w4 = dw[4];
+    const vu4 *dq = reinterpret_cast<const vu4 *>(prog_lds + 2u * (mem_off + idx * static_cast<uint32_t>(sizeof(VMemDesc) / 8)));
+    const vu4 q0 = dq[0], q1 = dq[1], q2 = dq[2];
     Desc d;
-    d.addr = dw[0];
-    d.dtype = static_cast<uint32_t>(w1);
-    d.flags = static_cast<uint32_t>(w1 >> 32);
-    d.ks0 = static_cast<uint32_t>(w2);
-    d.ks1 = static_cast<uint32_t>(w2 >> 32);
-    d.rs0 = static_cast<uint32_t>(w4);
-    d.rs1 = static_cast<uint32_t>(w4 >> 32);
+    d.addr = static_cast<uint64_t>(q0[0]) | (static_cast<uint64_t>(q0[1]) << 32);
+    d.dtype = uni(q0[2]);
+    d.flags = uni(q0[3]);
+    d.ks0 = q1[0];
+    d.ks1 = q1[1];
+    d.rs0 = q2[0];
+    d.rs1 = q2[1];
     return d;
   };
 
@@ -186,13 +221,16 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
     uint32_t pc = 0;
     vu2 fetched = code_at(0);
     while (true) {
-      const uint32_t w0 = fetched[0], imm = fetched[1];
+      const uint32_t w0 = uni(fetched[0]), imm = uni(fetched[1]);
       const uint32_t op = w0 & 0x7fu;
       if (op == VOP_END) break;
       const uint32_t sub = (w0 >> 8) & 0xffu, a = w0 >> 24, kind = (w0 >> 16) & 0xfu, rnd = (w0 >> 20) & 0x3u;
 
       if (op != VOP_SWEEP) {
         // ---- one value per lane ----
+#ifdef DVM_VEC_STAMPS_FINE
+        STAMP();
+#endif
         pc += (op == VOP_UNI_BEGIN && skips_runs != 0u) ? imm : 1u;  // (the waves that skip a run go on at its VOP_UNI_END)
         fetched = code_at(pc);
         if (op >= VOP_SRC_BASE) {
@@ -279,10 +317,13 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
       }
 
       // ---- a sweep: a native loop over its rounds ----
+      STAMP();
       const uint32_t slot_kinds = imm;
       const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
       const bool rev = (sub & VSW_REVERSE) != 0;
-      const vu2 ldw = code_at(pc + 1u);  // the VOP_LD that opens the body
+      vu2 ldw = code_at(pc + 1u);  // the VOP_LD that opens the body
+      ldw[0] = uni(ldw[0]);
+      ldw[1] = uni(ldw[1]);
       const uint32_t body_pc = pc + 2u;
       // the opening load's operand; every other operand of the body walks the reduced axes as it does, or not at all
       const Desc ma = desc_at(ldw[0] >> 24);
@@ -290,7 +331,9 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
       const uint32_t rs0 = ma.rs0, rs1 = ma.rs1;
       // the first instruction's operand rides with the opening load when both can take the wide path
       constexpr uint32_t kFast = VMF_VEC | VMF_ALIGNED;
-      const vu2 first_w = code_at(body_pc);
+      vu2 first_w = code_at(body_pc);
+      first_w[0] = uni(first_w[0]);
+      first_w[1] = uni(first_w[1]);
       uint32_t pair0 = ((first_w[0] & 0x7fu) == VOP_BINF && ((first_w[0] >> 16) & 0xfu) == VK_MEM && (first_w[0] & VI_SAME_OFFS) != 0 &&
                         !(first_w[1] & VI_PRE_SREG) && (ma.flags & kFast) == kFast) ? 1u : 0u;
       Desc mb = ma;
@@ -391,7 +434,7 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
 
         vu2 bfetched = code_at(bpc);
         while (true) {
-          const uint32_t w = bfetched[0], bimm = bfetched[1];
+          const uint32_t w = uni(bfetched[0]), bimm = uni(bfetched[1]);
           ++bpc;
           bfetched = code_at(bpc);
           const uint32_t bop = w & 0x7fu, bsub = (w >> 8) & 0xffu, bk = (w >> 16) & 0xfu, brnd = (w >> 20) & 0x3u, ba = w >> 24;
@@ -459,6 +502,57 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
         body_end = bpc;
       };
 
+      // A statistics sweep (the body is one float reduce) takes two interior rounds per trip to memory: the second
+      // round's slabs land in the registers an operand would use, and both rounds are reduced in their order.
+      const bool two_per_trip = (first_w[0] & 0x7fu) == VOP_RED && (first_w[0] & VI_ENDS) != 0u && (ldw[0] & VI_LD_KEEP_RD) == 0u &&
+                                (ma.flags & kFast) == kFast;
+      auto do_two_rounds = [&](uint32_t lr, uint32_t ridx, uint32_t lr2, uint32_t ridx2) {
+        auto walk = [&](uint32_t at) -> Offs {
+          Offs o;
+          FOR_U {
+            const uint32_t rc = at + u * r_step;
+            uint32_t c0 = rc, c1 = 0;
+            if (n_rdim > 1u) {
+              c1 = (__umulhi(rc, rd_magic) + rc) >> rd_shift;
+              c0 = rc - c1 * rd_extent;
+            }
+            o.v[u] = a_koff + (static_cast<uint64_t>(c0) * rs0) * static_cast<uint32_t>(E) + static_cast<uint64_t>(c1) * rs1;
+          }
+          return o;
+        };
+        Slabs sl;
+        sl.nvp = kAllFull;
+        sl.full = (1u << U) - 1u;
+        sl.uniform = true;
+        Desc da = ma;
+        da.dtype = fresh_s(ma.dtype);
+        Acc x0, x1;
+        mem_load_wide_2rounds(as_mem(da), walk(ridx), walk(ridx2), sl.full, sl.full, x0, x1);
+        const uint32_t l0 = fresh_s(ldw[0]), l1 = fresh_s(ldw[1]);
+        if (l0 & VI_LD_KEEP_WR) {  // (a load with a reduce behind it parks what it loaded: no prefix)
+          const uint32_t n_parked = l1 & 0xffffu, fmt = (l1 >> 20) & 0x3u;
+          if (lr < n_parked) vreg_store(keep_lds, fmt == VF_F32 ? 2u * lr : lr, fmt, nthreads, tid, x0);
+          if (lr2 < n_parked) vreg_store(keep_lds, fmt == VF_F32 ? 2u * lr2 : lr2, fmt, nthreads, tid, x1);
+        }
+        const uint32_t w = fresh_s(first_w[0]);
+        const uint32_t bsub = (w >> 8) & 0xffu;
+        auto reduce_into_slots = [&](Acc &x) {
+          if (bsub & VRF_SQUARE) FOR_U x.v[u] = x.v[u] * x.v[u];
+          if ((w >> 24) == 0u) {
+            reduce_round(racc0, bsub & 0xfu, x, sl);
+            if (bsub & VRF_PAIR) {
+              FOR_U x.v[u] = x.v[u] * x.v[u];
+              reduce_round(racc1, bsub & 0xfu, x, sl);
+            }
+          } else {
+            reduce_round(racc1, bsub & 0xfu, x, sl);
+          }
+        };
+        reduce_into_slots(x0);
+        reduce_into_slots(x1);
+        body_end = body_pc + 1u;
+      };
+
       const bool whole_groups = (inner_extent & (E - 1u)) == 0u;
       for (uint32_t round = 0; round < n_rounds; ++round) {
         const uint32_t lr = rev ? n_rounds - 1u - round : round;
@@ -466,6 +560,15 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
         // (the last slab of the lane decides: the indices of a lane's slabs ascend)
         const bool lane_full = kvalid && ridx + (U - 1u) * r_step < r_lim;
         if (whole_groups && wave_all(lane_full)) {
+          if (two_per_trip && round + 1u < n_rounds) {
+            const uint32_t lr2 = rev ? lr - 1u : lr + 1u;
+            const uint32_t ridx2 = r_base + r_local + lr2 * r_step * U;
+            if (wave_all(kvalid && ridx2 + (U - 1u) * r_step < r_lim)) {
+              do_two_rounds(lr, ridx, lr2, ridx2);
+              ++round;
+              continue;
+            }
+          }
           do_round(std::true_type{}, lr, ridx);
         } else {
           do_round(std::false_type{}, lr, ridx);
@@ -473,12 +576,16 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
       }
       pc = body_end;
       fetched = code_at(pc);
+      STAMP();
       if (k0 <= VR_MIN || k1 <= VR_MIN) {
         red_finish_x(racc0, racc1, k0, k1, HDR_NOW(team_log2), HDR_NOW(team_is_block) != 0u, tid, nthreads, red_flip, lds);
       }
+      STAMP();
     }
   }
+  STAMP();
 }
+#undef STAMP
 
 #undef HDR
 #undef HDR_NOW

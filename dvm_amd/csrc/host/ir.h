@@ -12,6 +12,7 @@
 #include <cstdint>
 #include <cstring>
 #include <string>
+#include <utility>
 #include <vector>
 
 #include "../../../include/dvm.h"
@@ -143,6 +144,23 @@ struct Program {
   };
   enum : uint8_t { kPatchVecMem = 0, kPatchCubeOperand = 1, kPatchPlain = 2, kPatchAligned16 = 3 };
   std::vector<Patch> patches;
+  // What binding an unaligned address takes away from the blob (the alignment flag of a memory operand, the sweep
+  // build of a vector program, the fast path of a matmul), as code generation left it: (32-bit word of the blob,
+  // value) pairs that every bind writes back first, so that a later bind of aligned addresses gets the fast paths back.
+  std::vector<std::pair<uint32_t, uint32_t>> bind_dependent;
+  void RememberBindDependent() {
+    bind_dependent.clear();
+    const uint32_t *w32 = reinterpret_cast<const uint32_t *>(blob.w);
+    auto keep = [&](size_t byte_offset) { bind_dependent.emplace_back(static_cast<uint32_t>(byte_offset / 4), w32[byte_offset / 4]); };
+    const uint32_t entry = w32[0];
+    if (entry == VE_VECTOR) {
+      keep(offsetof(VVecHeader, sched));
+      for (const Patch &pt : patches)
+        if (pt.role == kPatchVecMem) keep(static_cast<size_t>(pt.word) * 8 + offsetof(VMemDesc, flags));
+    } else if (entry == VE_CUBE) {
+      keep(offsetof(VCubeHeader, fast));
+    }
+  }
   // pre-launch fills (zero-size reduce identities, clean kernels)
   struct Fill {
     int op_id;

@@ -101,6 +101,8 @@ size_t Compiler::RunOnce(int mode) {
   k_->ws_offsets_.clear();
   PlanMaterialisation();
   for (int a = 0; a < n_areas_; ++a) CompileArea(a);
+  for (Program &p : k_->programs_)
+    if (!p.skip) p.RememberBindDependent();
   size_t total = 0;
   for (size_t i = 0; i < k_->ws_sizes_.size(); ++i) {
     k_->ws_offsets_.push_back(total);
@@ -132,6 +134,7 @@ void VKernel::BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *all
   }
   for (Program &p : programs_) {
     if (p.skip) continue;
+    for (const auto &orig : p.bind_dependent) reinterpret_cast<uint32_t *>(p.blob.w)[orig.first] = orig.second;
     for (const Program::Patch &pt : p.patches) {
       uint64_t addr = 0;
       if (pt.op_id >= 0) {
@@ -145,6 +148,8 @@ void VKernel::BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *all
       if ((addr & 15u) != 0) {
         if (pt.role == Program::kPatchVecMem) {
           reinterpret_cast<VMemDesc *>(p.blob.w + pt.word)->flags &= ~static_cast<uint32_t>(VMF_ALIGNED);
+          // (the sweep build accesses the operands of its interior rounds without guards: the generic kernel runs instead)
+          reinterpret_cast<VVecHeader *>(p.blob.w)->sched &= ~static_cast<uint32_t>(VS_SWEEPS);
         } else if (pt.role == Program::kPatchCubeOperand) {
           reinterpret_cast<VCubeHeader *>(p.blob.w)->fast = 0;
         } else if (pt.role == Program::kPatchAligned16) {

@@ -256,10 +256,12 @@ bool Compiler::FitsSweepBuild() {
     const uint64_t ld = code_[i + 1];
     if (VI_OP(ld) != VOP_LD || VI_KIND(ld) != VK_MEM || (static_cast<uint32_t>(ld) & (VI_UNIFORM | VI_ENDS))) return false;
     const VMemDesc &ma = mems_[VI_A(ld)];
-    if ((ma.flags & (VMF_VEC | VMF_GATHER)) != VMF_VEC) return false;
+    constexpr uint32_t kWide = VMF_VEC | VMF_ALIGNED;
+    if ((ma.flags & (kWide | VMF_GATHER)) != kWide) return false;
     auto walks_like_load = [&](uint32_t a) {
       const VMemDesc &m = mems_[a];
-      if (m.flags & VMF_GATHER) return false;
+      // contiguous and aligned, or one fp32 element per slab: what the build's interior rounds access without guards
+      if ((m.flags & (kWide | VMF_GATHER)) != kWide && !((m.flags & (VMF_VEC | VMF_GATHER)) == 0 && m.dtype == VDT_F32)) return false;
       bool none = true;
       for (int d = 0; d < DVM_VEC_MAXR; ++d) none = none && m.rstride[d] == 0;
       return none || std::memcmp(m.rstride, ma.rstride, sizeof(ma.rstride)) == 0;
