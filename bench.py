@@ -25,8 +25,9 @@ HBM_PEAK_GBS = 8000.0
 # also records a hash of the sources that decide the kernel's schedule (tests/test_host.py fails when they changed
 # since the measurement).
 TRAFFIC_SUMMARY = os.path.join("profiles", "vec_rx_batchnorm_hbm_traffic.txt")
-SCHEDULE_SOURCES = ["dvm_amd/csrc/device/vm_vector.hip", "dvm_amd/csrc/isa_gfx950.h", "dvm_amd/csrc/host/schedule.cc",
-                    "dvm_amd/csrc/host/emit_vector.cc", "dvm_amd/csrc/host/peephole.cc"]
+SCHEDULE_SOURCES = ["dvm_amd/csrc/device/vm_vector.hip", "dvm_amd/csrc/device/vm_vector_sweep.hip", "dvm_amd/csrc/device/vec_common.h",
+                    "dvm_amd/csrc/isa_gfx950.h", "dvm_amd/csrc/host/schedule.cc", "dvm_amd/csrc/host/emit_vector.cc",
+                    "dvm_amd/csrc/host/peephole.cc"]
 
 
 def schedule_sources_hash():
@@ -68,6 +69,47 @@ def bn_graph(t, x, g, b, n_red, eps):
     return t.add(t.mul(x, scale), shift)
 
 
+def bn_graph_two_pass(t, x, g, b, n_red, eps):
+    """The graph of the reference's own example (examples/02_batchnorm.py:27-42, with eps): the variance from the
+    centred values, i.e. a second statistics sweep over x - mean (robust where |mean| >> sigma; one more pass over x)."""
+    inv = 1.0 / n_red
+    mean = t.mul(t.sum(x, (0, 2, 3), True), inv)
+    xc = t.sub(x, mean)
+    var = t.mul(t.sum(t.mul(xc, xc), (0, 2, 3), True), inv)
+    return t.add(t.mul(t.div(xc, t.sqrt(t.add(var, eps))), g), b)
+
+
+def vector_kernel_name(das_text):
+    """Name of the vector VM kernel a one-launch program runs on, from its disassembly header."""
+    head = das_text.split("\n")[1]
+    if "sched=reduce-x" in head:
+        return "dvm_vm_vec_rx_sw" if " sweeps" in head else "dvm_vm_vec_rx"
+    return "dvm_vm_vec_ry" if "sched=reduce-y" in head else "dvm_vm_vec_pw"
+
+
+def bench_batchnorm_two_pass(x, g, b, iters=20):
+    """The two-pass form of the headline graph at the headline shape: time, launches, parity against float64."""
+    from dvm_amd.tester import Tester
+    n, c, h, w = x.shape
+    t = Tester("split:dyn")
+    lx, lg, lb = t.load(x), t.load(g), t.load(b)
+    out = t.store(bn_graph_two_pass(t, lx, lg, lb, n * h * w, 1e-5))
+    t.codegen()
+    t.run()
+    got = t.output(out)
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean((0, 2, 3), keepdims=True)) / np.sqrt(x64.var((0, 2, 3), keepdims=True) + 1e-5) * g + b
+    if not np.allclose(got, want, rtol=1e-5, atol=1e-5):
+        raise RuntimeError("two-pass batch-norm result differs from the NumPy golden")
+    smp = sorted(t.perf_samples(warmup=3, iters=iters))
+    med = smp[len(smp) // 2]
+    alg = 2 * x.nbytes + g.nbytes + b.nbytes
+    return {"graph": "sum(x) -> x - mean -> sum(sq) -> normalise (examples/02_batchnorm.py:27-42 with eps)", "launches": t.num_launches(),
+            "kernel": vector_kernel_name(t.das()), "kernel_us_median": round(med, 2), "kernel_us_min": round(smp[0], 2),
+            "kernel_us_mean": round(sum(smp) / len(smp), 2), "algorithmic_GBps": round(alg / med / 1e3, 1),
+            "frac_of_8TBps": round(alg / med / 1e3 / HBM_PEAK_GBS, 4), "parity_max_abs_err_vs_numpy_f64": float(np.max(np.abs(got - want)))}
+
+
 def bench_batchnorm(steps, warmup):
     from dvm_amd.tester import Tester
     n, c, h, w = 32, 256, 56, 56
@@ -79,6 +121,7 @@ def bench_batchnorm(steps, warmup):
     lx, lg, lb = t.load(x), t.load(g), t.load(b)
     out = t.store(bn_graph(t, lx, lg, lb, n * h * w, 1e-5))
     t.codegen()
+    kernel_name = vector_kernel_name(t.das())
     jit_cold = t.jit_us()
     t.codegen()
     jit_warm = t.jit_us()
@@ -106,6 +149,7 @@ def bench_batchnorm(steps, warmup):
     return {
         "x": x, "g": g, "b": b, "alg_bytes": alg_bytes, "ms_per_step": ms_per_step, "kernel_us_mean": ev_mean,
         "kernel_us_min": ev_min, "kernel_us_median": ev_median, "jit_us_cold": jit_cold, "jit_us_warm": jit_warm, "launches": launches, "max_rel_err": err,
+        "kernel": kernel_name,
     }
 
 
@@ -301,6 +345,48 @@ def bench_attention(b=8, h=32, s=2048, d=128, iters=10):
             "parity_heads_checked": 2}
 
 
+TORCH_ANCHOR = r"""
+import json, sys, torch
+dev = "cuda:0"
+def timeit(f, warm, iters):
+    for _ in range(warm): f()
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(iters):
+        a = torch.cuda.Event(enable_timing=True); b = torch.cuda.Event(enable_timing=True)
+        a.record(); f(); b.record(); b.synchronize(); ts.append(a.elapsed_time(b) * 1e3)
+    ts.sort(); return ts[0], ts[len(ts) // 2], sum(ts) / len(ts)
+g = torch.Generator(device=dev).manual_seed(1)
+out = {}
+if "matmul" in sys.argv:
+    A = (torch.randn(8192, 4096, device=dev, generator=g) / 8).bfloat16(); B = (torch.randn(4096, 4096, device=dev, generator=g) / 8).bfloat16()
+    mn, med, mean = timeit(lambda: torch.matmul(A, B), 10, 30)
+    out["matmul"] = {"op": "torch.matmul bf16 8192x4096x4096 (plain product, no epilogue)", "us_min": round(mn, 1), "us_median": round(med, 1),
+                     "us_mean": round(mean, 1), "TFLOPs_median": round(2 * 8192 * 4096 * 4096 / med / 1e6, 1)}
+if "attention" in sys.argv:
+    q, k, v = (torch.randn(8, 32, 2048, 128, device=dev, generator=g).half() for _ in range(3))
+    mn, med, mean = timeit(lambda: torch.nn.functional.scaled_dot_product_attention(q, k, v), 5, 20)
+    out["attention"] = {"op": "torch.nn.functional.scaled_dot_product_attention fp16 [8,32,2048,128]", "us_min": round(mn, 1), "us_median": round(med, 1),
+                        "us_mean": round(mean, 1), "TFLOPs_median": round(4 * 8 * 32 * 2048 * 2048 * 128 / med / 1e6, 1)}
+print("ANCHOR " + json.dumps(out))
+"""
+
+
+def torch_anchors(which):
+    """The vendor libraries on the same box, in a process of their own that imports torch first: torch.matmul
+    (hipBLASLt) and scaled_dot_product_attention at the shapes of configs[4] and configs[3], timed with events on
+    torch's stream. A stated ceiling of what this box sustains, not a target and never part of the product path."""
+    import subprocess
+    try:
+        r = subprocess.run([sys.executable, "-c", TORCH_ANCHOR] + list(which), capture_output=True, text=True, timeout=420)
+        for line in r.stdout.splitlines():
+            if line.startswith("ANCHOR "):
+                return json.loads(line[7:])
+        return {"error": (r.stderr or "no output").strip().splitlines()[-1][:200]}
+    except Exception as e:  # noqa: BLE001  (no torch, no time: the bench line goes out without the anchors)
+        return {"error": str(e)[:200]}
+
+
 def traffic_probe():
     """For the counter runs (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): five launches of the headline kernel
     and five launches of a plain copy of the same tensor through the pointwise VM kernel, whose traffic is
@@ -324,6 +410,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--skip-cpu", action="store_true", help="omit the CPU baseline leg")
     ap.add_argument("--only-headline", action="store_true", help="omit the other BASELINE configs")
+    ap.add_argument("--skip-torch-anchor", action="store_true", help="do not time torch.matmul / SDPA beside the two MFMA configs")
     ap.add_argument("--configs", default="add,rmsnorm,attention,matmul", help="which of the other BASELINE configs to run (comma separated)")
     ap.add_argument("--traffic-probe", action="store_true", help="launch the headline kernel and a plain copy only (for counter runs)")
     args = ap.parse_args()
@@ -351,7 +438,7 @@ def main():
                    "parity_max_rel_err_vs_numpy_f64": bn["max_rel_err"]},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "dvm_vm_vec_rx", "kernel_us_mean": round(bn["kernel_us_mean"], 2), "kernel_us_median": round(bn["kernel_us_median"], 2),
+                     "kernel": bn["kernel"], "kernel_us_mean": round(bn["kernel_us_mean"], 2), "kernel_us_median": round(bn["kernel_us_median"], 2),
                      "kernel_us_min": round(bn["kernel_us_min"], 2)},
     }
     if not args.skip_cpu:
@@ -361,6 +448,12 @@ def main():
                   "attention": ("attention_fp16_b8_h32_s2048_d128", bench_attention),
                   "matmul": ("matmul_bias_silu_bf16_8192x4096x4096", bench_matmul)}
         line["configs"] = {others[c][0]: others[c][1]() for c in args.configs.split(",") if c in others}
+        line["configs"]["batchnorm_two_pass_fp32_32x256x56x56"] = bench_batchnorm_two_pass(bn["x"], bn["g"], bn["b"])
+        wanted = [c for c in ("matmul", "attention") if c in args.configs.split(",")]
+        if wanted and not args.skip_torch_anchor:
+            anchors = torch_anchors(wanted)
+            for c in wanted:
+                line["configs"][others[c][0]]["same_box_vendor_library"] = anchors.get(c, anchors)
     print(json.dumps(line))
 
 

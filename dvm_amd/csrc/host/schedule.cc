@@ -523,8 +523,13 @@ void Compiler::ChooseSchedule() {
     // barrier separates the sweeps. Measured on MI355X, rows of 4096 bf16 (residual add + RMSNorm): 8192 rows
     // 98 us with 256 lanes per row, 83 us with 64; 2048 rows 30 / 28 (128 lanes) / 35 us; 1024 rows 18 / 22 / 30 us.
     // So: about 2^18 lanes in flight, at least one wave per output. DVM_VEC_TEAM caps the team by hand.
+    // (Rounded down to a power of two since the sweep build exists: rows of one wave or two then run as native loops.
+    // The same graph: 1536 rows 22.5 us with 256 lanes per row, 20.0 with 128; 3072 rows 28.5 with 128, 25.7 with 64.)
     {
-      uint32_t cap = std::max<uint32_t>(64, Pow2Ceil((1ull << 18) / std::max<uint64_t>(n_k, 1)));
+      const uint64_t lanes_per_output = (1ull << 18) / std::max<uint64_t>(n_k, 1);
+      uint32_t cap = Pow2Ceil(lanes_per_output);
+      if (cap > lanes_per_output) cap >>= 1;
+      cap = std::max<uint32_t>(64, cap);
       if (k_->tuning_.vec_team >= 1) {
         const uint32_t c = static_cast<uint32_t>(k_->tuning_.vec_team);
         if ((c & (c - 1)) == 0) cap = c;

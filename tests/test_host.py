@@ -594,3 +594,38 @@ def test_traffic_summary_was_measured_on_the_current_schedule_sources():
     traffic, source = bench.headline_traffic()
     assert traffic is not None and traffic > 205522944, source
     assert "measured on these sources" in source, source
+
+
+def _row_norm(t, rows, cols, dtype="float32", with_compare=False):
+    x = t.load(np.zeros((rows, cols), np.float32 if dtype == "float32" else np.float16))
+    xf = t.cast(x, "float32") if dtype != "float32" else x
+    mean = t.mul(t.sum(xf, (1,), True), 1.0 / cols)
+    xc = t.sub(xf, mean)
+    if with_compare:  # a select inside the second sweep: outside the sweep build's vocabulary
+        xc = t.select(t.greater(xc, 0.0), xc, t.mul(xc, 0.1))
+    var = t.mul(t.sum(t.mul(xc, xc), (1,), True), 1.0 / cols)
+    t.store(t.div(xc, t.sqrt(t.add(var, 1e-5))))
+    t.codegen()
+    return t.das()
+
+
+def test_sweep_build_is_chosen_from_the_instruction_words(monkeypatch):
+    """Which programs carry VS_SWEEPS (isa_gfx950.h): those that reduce the innermost axis in sweeps of several
+    rounds whose bodies are float chains behind one aligned, contiguous load."""
+    monkeypatch.delenv("DVM_VEC_SWEEPS", raising=False)
+    assert "reduce-x sweeps" in _row_norm(Tester("split", run_mode="das"), 8192, 4096)
+    assert "reduce-x sweeps" in _row_norm(Tester("split", run_mode="das"), 8192, 4096, "float16")
+    assert "reduce-x sweeps" in _row_norm(Tester("split", run_mode="das"), 3, 100000)
+    # a row that fits one round keeps its values in the accumulator between the sweeps: they do not start with a load
+    assert "reduce-x sweeps" not in _row_norm(Tester("split", run_mode="das"), 100, 512)
+    # compares and selects are not in the vocabulary
+    assert "reduce-x sweeps" not in _row_norm(Tester("split", run_mode="das"), 8192, 4096, with_compare=True)
+    # rows that do not start on 16 bytes
+    assert "reduce-x sweeps" not in _row_norm(Tester("split", run_mode="das"), 8192, 4100 + 1)
+    # int32 reduces
+    t = Tester("split", run_mode="das")
+    t.store(t.max(t.load(np.zeros((4096, 4096), np.int32)), (1,), True))
+    t.codegen()
+    assert "reduce-x" in t.das() and "sweeps" not in t.das(), t.das()
+    monkeypatch.setenv("DVM_VEC_SWEEPS", "0")
+    assert "reduce-x sweeps" not in _row_norm(Tester("split", run_mode="das"), 8192, 4096)
