@@ -147,27 +147,49 @@ void Compiler::CompileCube(int a) {
   h.m = static_cast<uint32_t>(M);
   h.n = static_cast<uint32_t>(N);
   h.k = static_cast<uint32_t>(K);
-  h.trans_a = mm->trans_a ? 1 : 0;
-  h.trans_b = mm->trans_b ? 1 : 0;
-  h.lda = static_cast<uint32_t>(an.dims[an.rank - 1]);
-  h.ldb = static_cast<uint32_t>(bn.dims[bn.rank - 1]);
   h.nb0 = br == 2 ? static_cast<uint32_t>(mm->dim(0)) : 1;
   h.nb1 = br >= 1 ? static_cast<uint32_t>(mm->dim(br - 1)) : 1;
-  auto batch_strides = [&](const ANode &x, uint32_t *s0, uint32_t *s1) {
+  // An operand is a matrix (or a batch of matrices) walked through a leading dimension and up to two batch strides.
+  // A dense tensor gives those from its shape; a strided view (a load with strides, a slice, a permute of a stored
+  // value: a sliced weight, the heads-first view of a [batch, seq, heads, dim] tensor, a transposed K) gives them
+  // from its element strides: with the innermost stride 1 the matrix is read as it lies, with the second-innermost
+  // stride 1 it is the transpose of what lies in memory and the operand's transpose flag flips. Nothing is copied.
+  // (The reference reads views into its cube unit as well: include/dvm.h:434-479, src/isa.h:1187-1452.)
+  auto operand_layout = [&](const ANode &x, bool *flip, uint32_t *ld, uint32_t *s0, uint32_t *s1) {
+    *flip = false;
     *s0 = *s1 = 0;
-    int64_t stride = x.dims[x.rank - 1] * x.dims[x.rank - 2];
-    for (int d = x.rank - 3; d >= 0; --d) {
-      const int od = d + R - x.rank;
-      if (x.dims[d] != 1) {
-        if (stride >= (1ll << 32)) Fail("stride above 2^32");
-        if (od == R - 3) *s1 = static_cast<uint32_t>(stride);
-        else *s0 = static_cast<uint32_t>(stride);
-      }
+    const int r = x.rank;
+    int64_t walk[kMaxAxes];
+    int64_t stride = 1;
+    for (int d = r - 1; d >= 0; --d) {
+      walk[d] = x.view != nullptr ? x.view->vstride_[d] : stride;
       stride *= x.dims[d];
     }
+    for (int d = 0; d < r; ++d)
+      if (x.dims[d] != 1 && (walk[d] < 0 || walk[d] >= (1ll << 32))) Fail("stride above 2^32");
+    const int64_t rows = x.dims[r - 2], cols = x.dims[r - 1];
+    if (cols == 1 || walk[r - 1] == 1) {
+      *ld = static_cast<uint32_t>(rows == 1 ? std::max<int64_t>(cols, 1) : walk[r - 2]);
+    } else if (rows == 1 || walk[r - 2] == 1) {
+      *flip = true;
+      *ld = static_cast<uint32_t>(cols == 1 ? std::max<int64_t>(rows, 1) : walk[r - 1]);
+    } else {
+      Throw("DVM EXCEPTION. reason: a matmul operand view with no contiguous axis is not supported by the gfx950 backend (Copy it first)");
+    }
+    if (*ld == 0) Throw("DVM EXCEPTION. reason: a matmul operand view that repeats its rows is not supported by the gfx950 backend (Copy it first)");
+    for (int d = r - 3; d >= 0; --d) {
+      const int od = d + R - r;
+      if (x.dims[d] == 1) continue;
+      if (od == R - 3) *s1 = static_cast<uint32_t>(walk[d]);
+      else *s0 = static_cast<uint32_t>(walk[d]);
+    }
   };
-  batch_strides(an, &h.a_sb0, &h.a_sb1);
-  batch_strides(bn, &h.b_sb0, &h.b_sb1);
+  bool flip_a = false, flip_b = false;
+  operand_layout(an, &flip_a, &h.lda, &h.a_sb0, &h.a_sb1);
+  operand_layout(bn, &flip_b, &h.ldb, &h.b_sb0, &h.b_sb1);
+  const bool trans_a = mm->trans_a != flip_a, trans_b = mm->trans_b != flip_b;  // as the operands lie in memory
+  h.trans_a = trans_a ? 1 : 0;
+  h.trans_b = trans_b ? 1 : 0;
   if (M == 0 || N == 0 || h.nb0 == 0 || h.nb1 == 0) {
     prog_->skip = true;
     return;
@@ -247,8 +269,8 @@ void Compiler::CompileCube(int a) {
         const uint32_t max_split = nt >= slots ? 1u : static_cast<uint32_t>(std::min<uint64_t>(slots / nt, 32));
         // (ragged edge tiles of an aligned product are moved back inside the output and stay on the vector path)
         // (and the 64 tile fetches the rows of a short operand with contiguous k through clamped addresses)
-        const bool m_fast = M % t == 0 || (M >= t && (!mm->trans_a || M % 8 == 0)) || (t == 64 && !mm->trans_a);
-        const bool n_fast = N % t == 0 || (N >= t && N % 8 == 0) || (t == 64 && mm->trans_b);
+        const bool m_fast = M % t == 0 || (M >= t && (!trans_a || M % 8 == 0)) || (t == 64 && !trans_a);
+        const bool n_fast = N % t == 0 || (N >= t && N % 8 == 0) || (t == 64 && trans_b);
         const double slow = (aligned && m_fast && n_fast) ? 1.0 : 2.5;
         for (uint32_t want = 1; want <= max_split; want = want < 2 ? 2 : want * 2) {
           uint32_t chunk = 0;
@@ -289,11 +311,11 @@ void Compiler::CompileCube(int a) {
   // operand addresses
   for (int which = 0; which < 2; ++which) {
     const ANode &x = which == 0 ? an : bn;
-    if (x.view != nullptr) Throw("DVM EXCEPTION. reason: a strided view as a matmul operand is not supported by the gfx950 backend");
     Program::Patch p;
     p.word = static_cast<uint32_t>((which == 0 ? offsetof(VCubeHeader, a_addr) : offsetof(VCubeHeader, b_addr)) / 8);
     p.op_id = x.addr_op;
     p.ws_slot = x.ws_slot;
+    p.byte_offset = x.view != nullptr ? x.view->view_base_ * static_cast<int64_t>(DTypeSize(x.dtype)) : 0;
     p.role = Program::kPatchCubeOperand;
     prog_->patches.push_back(p);
   }
