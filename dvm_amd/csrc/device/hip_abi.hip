@@ -341,8 +341,14 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
     if (!DVM_ATTN_D_OK(a->d) || a->skv == 0 || !(a->scale > 0.0f) || a->sq == 0 || a->nb == 0 ||
         a->q_blocks != (a->sq + DVM_ATTN_BQ - 1) / DVM_ATTN_BQ || static_cast<uint64_t>(a->nb) * a->q_blocks != block_dim || (threads != 256 && threads != 512) ||
         lds_bytes < DVM_ATTN_LDS_BYTES_D(a->d) || a->q_addr == 0 || a->k_addr == 0 || a->v_addr == 0 || a->o_addr == 0 ||
-        ((a->q_addr | a->k_addr | a->v_addr | a->o_addr) & 15u) != 0 || (a->dtype != VDT_F16 && a->dtype != VDT_BF16)) {
+        ((a->q_addr | a->k_addr | a->v_addr | a->o_addr) & 15u) != 0 || (a->dtype != VDT_F16 && a->dtype != VDT_BF16) ||
+        a->nb_inner == 0 || a->nb % a->nb_inner != 0) {
       return static_cast<int>(hipErrorInvalidValue);
+    }
+    for (int i = 0; i < 4; ++i) {  // rows of at least d elements, every stride on 16 bytes (the kernel has 128-bit accesses only)
+      if (a->row_stride[i] < a->d || a->row_stride[i] >= (1u << 22) || ((a->row_stride[i] | a->outer_stride[i] | a->inner_stride[i]) & 7u) != 0) {
+        return static_cast<int>(hipErrorInvalidValue);
+      }
     }
     // 256 lanes: four waves of 64 queries; 512 lanes: eight waves of 32 queries (same tile of 256 queries)
     const bool bf = a->dtype == VDT_BF16, narrow = a->d != DVM_ATTN_D;

@@ -106,10 +106,13 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
   uint32_t pos = blockIdx.x;
   if ((gridDim.x & 7u) == 0) pos = (blockIdx.x & 7u) * (gridDim.x >> 3) + (blockIdx.x >> 3);
   const uint32_t b = pos / q_blocks, qb = pos % q_blocks;
-  const uint64_t q_base = hp->q_addr + static_cast<uint64_t>(b) * sq * D * 2;
-  const uint64_t k_base = hp->k_addr + static_cast<uint64_t>(b) * skv * D * 2;
-  const uint64_t v_base = hp->v_addr + static_cast<uint64_t>(b) * skv * D * 2;
-  const uint64_t o_base = hp->o_addr + static_cast<uint64_t>(b) * sq * D * 2;
+  // the (batch, head) pair's matrices: strides in elements from the header (views are read in place)
+  const uint32_t b_out = b / hp->nb_inner, b_in = b % hp->nb_inner;
+  auto base_of = [&](uint64_t addr, int which) -> uint64_t {
+    return addr + (static_cast<uint64_t>(b_out) * hp->outer_stride[which] + static_cast<uint64_t>(b_in) * hp->inner_stride[which]) * 2;
+  };
+  const uint64_t q_base = base_of(hp->q_addr, 0), k_base = base_of(hp->k_addr, 1), v_base = base_of(hp->v_addr, 2), o_base = base_of(hp->o_addr, 3);
+  const uint32_t ldq = hp->row_stride[0], ldk = hp->row_stride[1], ldv = hp->row_stride[2], ldo = hp->row_stride[3];
   const uint32_t q0 = qb * DVM_ATTN_BQ + wave * WQ;
 
   // Q fragments (B operand of stage 1): lane (j, h) holds Q[q0 + 32*qt + j][16*kk + 8*h .. +7]; rows
@@ -121,7 +124,7 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
     row = row < sq ? row : sq - 1;
 #pragma unroll
     for (int kk = 0; kk < D / 16; ++kk)
-      qf[qt][kk] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(q_base + (static_cast<uint64_t>(row) * D + 16 * kk + 8 * lh) * 2);
+      qf[qt][kk] = *reinterpret_cast<const DVM_GLOBAL vu4 *>(q_base + (static_cast<uint64_t>(row) * ldq + 16 * kk + 8 * lh) * 2);
   }
 
   // Staging. A block of K or V is 64 keys x 128 d = two half tiles (d < 64, d >= 64) of 64 rows x 8 chunks of
@@ -131,31 +134,29 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
   // consecutive local memory.
   constexpr uint32_t KPS = NTHR / 8;       // keys one step of all lanes covers
   constexpr int STEPS = 64 / KPS;          // steps per half tile
-  uint32_t ld_off[2];  // byte offset of the lane's chunk inside a block, for even / odd steps
+  uint32_t col_off[2];  // byte offset of the lane's chunk inside its row, for even / odd steps
 #pragma unroll
   for (int par = 0; par < 2; ++par) {
     const uint32_t key = KPS * par + (tid >> 3);
     const uint32_t logical = (tid & 7u) ^ ((key ^ (key >> 3)) & 7u);
-    ld_off[par] = ((tid >> 3) * D + (logical << 3)) * 2u;
+    col_off[par] = (logical << 3) * 2u;
   }
   const uint32_t wave_first = uni(wave) * 64u;
   // (a last block with fewer than BKV keys: the rows past the end fetch the last key again, their scores are masked)
   auto fetch_kv = [&](uint32_t key0, uint32_t buf) {
     uint16_t *kdst = lds + buf * kBuf, *vdst = lds + buf * kBuf + kVOff;
-    const DVM_GLOBAL char *ksrc = reinterpret_cast<const DVM_GLOBAL char *>(k_base + static_cast<uint64_t>(key0) * D * 2);
-    const DVM_GLOBAL char *vsrc = reinterpret_cast<const DVM_GLOBAL char *>(v_base + static_cast<uint64_t>(key0) * D * 2);
+    const DVM_GLOBAL char *ksrc = reinterpret_cast<const DVM_GLOBAL char *>(k_base + static_cast<uint64_t>(key0) * ldk * 2);
+    const DVM_GLOBAL char *vsrc = reinterpret_cast<const DVM_GLOBAL char *>(v_base + static_cast<uint64_t>(key0) * ldv * 2);
     const uint32_t last_row = skv - 1u - key0;  // uniform; BKV - 1 or more in a full block
 #pragma unroll
     for (int i = 0; i < HT * STEPS; ++i) {
       // step i % STEPS of half tile i / STEPS: later keys, then d 64..
-      uint32_t src_off = (i % STEPS) * KPS * D * 2u + (i / STEPS) * 64u * 2u + ld_off[(i % STEPS) & 1];
-      if (last_row < static_cast<uint32_t>(BKV) - 1u) {
-        const uint32_t row = (i % STEPS) * KPS + (tid >> 3);
-        src_off -= (row > last_row ? row - last_row : 0u) * (D * 2u);
-      }
+      uint32_t row = (i % STEPS) * KPS + (tid >> 3);
+      if (last_row < static_cast<uint32_t>(BKV) - 1u) row = row > last_row ? last_row : row;
+      const uint32_t col = (i / STEPS) * 64u * 2u + col_off[(i % STEPS) & 1];
       const uint32_t dst_off = (static_cast<uint32_t>(i) * NTHR + wave_first) * 8u;
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(ksrc + src_off), (__attribute__((address_space(3))) void *)(kdst + dst_off), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(vsrc + src_off), (__attribute__((address_space(3))) void *)(vdst + dst_off), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(ksrc + (row * ldk * 2u + col)), (__attribute__((address_space(3))) void *)(kdst + dst_off), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const DVM_GLOBAL void *>(vsrc + (row * ldv * 2u + col)), (__attribute__((address_space(3))) void *)(vdst + dst_off), 16, 0, 0);
     }
   };
 
@@ -343,7 +344,7 @@ __device__ __forceinline__ void vm_attn(const VmParam &p) {
           vu2 w;
           w[0] = pack2<IS_BF16>(o_acc[dt][qt][4 * g] * inv, o_acc[dt][qt][4 * g + 1] * inv);
           w[1] = pack2<IS_BF16>(o_acc[dt][qt][4 * g + 2] * inv, o_acc[dt][qt][4 * g + 3] * inv);
-          *reinterpret_cast<DVM_GLOBAL vu2 *>(o_base + (static_cast<uint64_t>(row) * D + dt * 32 + 8 * g + 4 * lh) * 2) = w;
+          *reinterpret_cast<DVM_GLOBAL vu2 *>(o_base + (static_cast<uint64_t>(row) * ldo + dt * 32 + 8 * g + 4 * lh) * 2) = w;
         }
       }
     }

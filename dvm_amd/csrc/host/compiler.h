@@ -216,6 +216,16 @@ class Compiler {
     float scale;
     int area;
   };
+  // How an operand of a fused attention lies in memory (VAttnHeader: strides in elements). `ok`: the kernel can
+  // read it in place (a load, or a permute / slice of a load; head dimension contiguous; at most two batch axes
+  // unless it is dense; every stride a multiple of eight elements).
+  struct AttnLayout {
+    bool ok = false;
+    const NDObject *root = nullptr;  // the load whose address the operand starts from
+    int64_t base = 0;                // element offset of the view inside that buffer
+    uint32_t row = 0, outer = 0, inner = 0, nb_inner = 1;
+  };
+  AttnLayout AttnOperandLayout(const NDObject *x) const;
   std::vector<AttnGroup> attn_groups_;
   std::vector<int> attn_of_;
   void DetectAttention();

@@ -244,6 +244,16 @@ std::string &VKernel::DisAssemble() {
       const VAttnHeader *a = reinterpret_cast<const VAttnHeader *>(p.blob.w);
       os << "entry attention " << kMemTypes[a->dtype] << " batch=" << a->nb << " sq=" << a->sq << " skv=" << a->skv << " d=" << a->d
          << " scale=" << a->scale << " blocks=" << p.grid << " lds=" << p.lds_bytes << "\n";
+      {
+        static const char *names[4] = {"q", "k", "v", "o"};
+        const uint32_t rows[4] = {a->sq, a->skv, a->skv, a->sq};
+        for (int i = 0; i < 4; ++i) {  // operands that are not dense [batch][rows][d]
+          const bool dense = a->row_stride[i] == a->d && (a->nb_inner == 1 ? a->outer_stride[i] == rows[i] * a->d
+                                                                           : (a->inner_stride[i] == rows[i] * a->d && a->outer_stride[i] == rows[i] * a->d * a->nb_inner));
+          if (!dense) os << "  " << names[i] << ": view, strides row=" << a->row_stride[i] << " batch=" << a->outer_stride[i] << "," << a->inner_stride[i]
+                         << " (inner batch extent " << a->nb_inner << ")\n";
+        }
+      }
       os << "  mmad s, K, Q^T\n  online_softmax p, s\n  mmad o, V^T, p\n  store o\n";
     } else {
       os << "entry type " << h->entry << " blocks=" << p.grid << " threads=" << p.threads << "\n";

@@ -149,7 +149,11 @@ void VKernel::BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *all
         if (pt.role == Program::kPatchVecMem) {
           reinterpret_cast<VMemDesc *>(p.blob.w + pt.word)->flags &= ~static_cast<uint32_t>(VMF_ALIGNED);
           // (the sweep build accesses the operands of its interior rounds without guards: the generic kernel runs instead)
-          reinterpret_cast<VVecHeader *>(p.blob.w)->sched &= ~static_cast<uint32_t>(VS_SWEEPS);
+          uint32_t sched;
+          char *sched_at = reinterpret_cast<char *>(p.blob.w) + offsetof(VVecHeader, sched);
+          std::memcpy(&sched, sched_at, sizeof(sched));
+          sched &= ~static_cast<uint32_t>(VS_SWEEPS);
+          std::memcpy(sched_at, &sched, sizeof(sched));
         } else if (pt.role == Program::kPatchCubeOperand) {
           reinterpret_cast<VCubeHeader *>(p.blob.w)->fast = 0;
         } else if (pt.role == Program::kPatchAligned16) {

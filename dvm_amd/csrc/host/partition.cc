@@ -421,6 +421,49 @@ void Compiler::PlanMaterialisation() {
 
 // ---------- fused attention ----------
 
+Compiler::AttnLayout Compiler::AttnOperandLayout(const NDObject *x) const {
+  AttnLayout l;
+  const NDObject *root = ViewRoot(x);
+  if (root->kind != kObjLoad) return l;
+  const bool is_view = x != root ? (x->kind == kObjPermute || x->kind == kObjSlice) : root->strided;
+  if (x != root && !is_view) return l;      // (a reshape in the chain)
+  if (x != root && root->strided) return l; // (a view of a strided load: its strides are not composed)
+  const int r = x->rank();
+  if (r < 2) return l;
+  l.root = root;
+  const int64_t rows = x->dim(r - 2), d = x->dim(r - 1);
+  if (!is_view) {  // dense: any number of batch axes, they collapse into one
+    l.ok = true;
+    l.row = static_cast<uint32_t>(d);
+    l.outer = static_cast<uint32_t>(rows * d);
+    l.inner = 0;
+    l.nb_inner = 1;
+    return l;
+  }
+  if (r > 4) return l;
+  const int64_t *st = x->vstride_;
+  if (d != 1 && st[r - 1] != 1) return l;
+  auto fits = [](int64_t v) { return v >= 0 && v < (1ll << 24) * 64 && v % 8 == 0; };
+  const int64_t row = rows == 1 ? d : st[r - 2];
+  if (row < d || row >= (1ll << 22) || row % 8 != 0 || x->view_base_ % 8 != 0 || x->view_base_ < 0) return l;
+  int64_t outer = 0, inner = 0, nb_inner = 1;
+  if (r == 3) {
+    outer = x->dim(0) == 1 ? 0 : st[0];
+  } else if (r == 4) {
+    outer = x->dim(0) == 1 ? 0 : st[0];
+    inner = x->dim(1) == 1 ? 0 : st[1];
+    nb_inner = x->dim(1);
+  }
+  if (!fits(outer) || !fits(inner) || outer >= (1ll << 32) || inner >= (1ll << 32)) return l;
+  l.ok = true;
+  l.base = x->view_base_;
+  l.row = static_cast<uint32_t>(row);
+  l.outer = static_cast<uint32_t>(outer);
+  l.inner = static_cast<uint32_t>(inner);
+  l.nb_inner = static_cast<uint32_t>(nb_inner);
+  return l;
+}
+
 void Compiler::DetectAttention() {
   std::vector<int> &uses = scratch_a_;
   uses.assign(n_, 0);
@@ -475,7 +518,27 @@ void Compiler::DetectAttention() {
     if (m1->kind != kObjMatMul || m1->trans_a || !m1->trans_b || m1->in[2] != nullptr || uses[m1->id] != 1) continue;
     if (m1->type_id_ != m2->type_id_) continue;
     NDObject *q = m1->in[0], *kk = m1->in[1];
-    if (q->kind != kObjLoad || kk->kind != kObjLoad || v->kind != kObjLoad || q->strided || kk->strided || v->strided) continue;
+    // q, k, v: loads, or views of loads the kernel can walk in place (a heads-first view of a [batch, seq, heads, d]
+    // tensor, a slice of a longer cache); the three agree on how the batch axes split
+    const AttnLayout lq = AttnOperandLayout(q), lk = AttnOperandLayout(kk), lv = AttnOperandLayout(v);
+    if (!lq.ok || !lk.ok || !lv.ok) continue;
+    {
+      uint32_t nbi = 1;
+      bool same = true;
+      for (const AttnLayout *l : {&lq, &lk, &lv}) {
+        if (l->nb_inner == 1) continue;
+        if (nbi != 1 && nbi != l->nb_inner) same = false;
+        nbi = l->nb_inner;
+      }
+      // (a dense operand beside a view with two batch axes: its collapsed batch stride must split the same way,
+      // which holds when its own rank gives the same inner extent)
+      for (const AttnLayout *l : {&lq, &lk, &lv})
+        if (nbi != 1 && l->nb_inner == 1 && l->inner == 0 && l->root != nullptr) {
+          const NDObject *t = l == &lq ? q : (l == &lk ? kk : v);
+          if (t->rank() != 4 || static_cast<uint32_t>(t->dim(1)) != nbi) same = false;
+        }
+      if (!same) continue;
+    }
     const int r = q->rank();
     if (kk->rank() != r || v->rank() != r || r < 2) continue;
     bool ok = DVM_ATTN_D_OK(q->dim(r - 1)) && kk->dim(r - 1) == q->dim(r - 1) && v->dim(r - 1) == q->dim(r - 1) && kk->dim(r - 2) == v->dim(r - 2) &&

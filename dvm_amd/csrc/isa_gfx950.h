@@ -330,6 +330,14 @@ typedef struct {
   float scale;      // applied to Q K^T before the softmax; positive
   uint32_t q_blocks;  // ceil(sq / DVM_ATTN_BQ)
   uint64_t q_addr, k_addr, v_addr, o_addr;
+  // How Q, K, V, O (in this order) lie in memory: element stride from one row (query or key) to the next, and from
+  // one (batch, head) pair to the next along the outer and the inner of two batch axes; pair b has the indices
+  // (b / nb_inner, b % nb_inner). Every stride is a multiple of 8 elements (16 bytes). A dense [nb][rows][d] tensor
+  // has row = d, outer = rows * d with nb_inner = 1; the heads-first view of a [batch][seq][heads][d] tensor has
+  // row = heads * d, outer = seq * heads * d, inner = d with nb_inner = heads.
+  uint32_t nb_inner;
+  uint32_t row_stride[4], outer_stride[4], inner_stride[4];
+  uint32_t pad;
 } VAttnHeader;
 
 typedef struct {

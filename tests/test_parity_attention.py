@@ -154,3 +154,53 @@ def test_attention_fused_with_a_short_last_block_of_keys(monkeypatch, waves, d, 
     got = _fused(q, k, v)
     want = np_attention(q, k, v)
     assert np.allclose(got, want, rtol=1e-2, atol=2e-2), np.abs(got - want).max()
+
+
+# ---- views as operands of the fused kernel: read in place, one launch ----
+
+@pytest.mark.parametrize("b,s,h,d", [(2, 320, 4, 128), (1, 200, 3, 64), (2, 512, 2, 128)])
+@pytest.mark.parametrize("how", ["view_load", "permute"])
+def test_attention_on_sequence_major_tensors_read_heads_first(b, s, h, d, how):
+    # q, k, v stored [batch, seq, heads, d] and read as [batch, heads, seq, d]; the result is dense, heads first
+    rng = np.random.default_rng(b * 1000 + s + h)
+    q, k, v = (rng.standard_normal((b, s, h, d)).astype(np.float16) for _ in range(3))
+    t = Tester("mix")
+    if how == "view_load":
+        stride = [s * h * d, d, h * d, 1]
+        lq, lk, lv = (t.view_load([b, h, s, d], stride, x) for x in (q, k, v))
+    else:
+        lq, lk, lv = (t.permute(t.load(x), [0, 2, 1, 3]) for x in (q, k, v))
+    out = t.store(attention_graph(t, lq, lk, lv, 1.0 / math.sqrt(d), 4))
+    t.run()
+    assert "entry attention" in t.das() and "view, strides" in t.das() and t.num_launches() == 1, t.das()
+    want = np_attention(q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3))
+    assert np.allclose(t.output(out), want, rtol=1e-2, atol=1e-2)
+
+
+def test_attention_on_a_window_of_a_longer_key_value_cache():
+    # k, v are the first skv rows of a cache [heads, 1024, d]; q dense (a dense operand beside views)
+    rng = np.random.default_rng(77)
+    hds, sq, skv, d, cap = 6, 128, 333, 128, 1024
+    q = rng.standard_normal((hds, sq, d)).astype(np.float16)
+    kc, vc = (rng.standard_normal((hds, cap, d)).astype(np.float16) for _ in range(2))
+    t = Tester("mix")
+    lk = t.slice_load(kc, [0, 0, 0], [hds, skv, d])
+    lv = t.slice_load(vc, [0, 8, 0], [hds, skv, d])  # (a window that starts inside the cache)
+    out = t.store(attention_graph(t, t.load(q), lk, lv, 1.0 / math.sqrt(d), 3))
+    t.run()
+    assert "entry attention" in t.das() and t.num_launches() == 1, t.das()
+    assert np.allclose(t.output(out), np_attention(q, kc[:, :skv], vc[:, 8:8 + skv]), rtol=1e-2, atol=1e-2)
+
+
+def test_attention_views_the_kernel_cannot_walk_run_unfused():
+    # a head dimension that is not contiguous in memory: three launches, same result
+    rng = np.random.default_rng(78)
+    hds, s, d = 2, 128, 64
+    q, v = (rng.standard_normal((hds, s, d)).astype(np.float16) for _ in range(2))
+    kt = rng.standard_normal((hds, d, s)).astype(np.float16)  # K stored transposed
+    t = Tester("mix")
+    lk = t.view_load([hds, s, d], [d * s, 1, s], kt)
+    out = t.store(attention_graph(t, t.load(q), lk, t.load(v), 1.0 / math.sqrt(d), 3))
+    t.run()
+    assert "entry attention" not in t.das(), t.das()
+    assert np.allclose(t.output(out), np_attention(q, kt.transpose(0, 2, 1), v), rtol=1e-2, atol=1e-2)
