@@ -11,7 +11,8 @@ import os
 import numpy as np
 
 _LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
-_LIB_PATH = os.path.join(_LIB_DIR, "libdvm.so")
+# DVM_HOST_LIBRARY names another build of the host library (the sanitizer build of `make asan=1`)
+_LIB_PATH = os.environ.get("DVM_HOST_LIBRARY") or os.path.join(_LIB_DIR, "libdvm.so")
 
 
 class _Operand(ctypes.Structure):

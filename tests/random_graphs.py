@@ -370,3 +370,39 @@ def view_graph(case):
         return stores
     return build
 
+
+
+def compile_in_das_mode(seeds):
+    """The host compiler alone on `seeds` cases of every generator, in disassembly mode (no GPU): what `make
+    asan-check` runs against the sanitizer build. A compile error with one of the documented messages is a valid
+    outcome; anything else, or a sanitizer report, ends the run."""
+    from dvm_amd.tester import Tester
+    from oracle.oracle import OracleKernel
+    done = refused = 0
+    for case in range(seeds):
+        for gen, ker in ((lambda c: pointwise_reduce_graph(c, True), ""), (typed_graph, ""), (matmul_graph, "mix"), (view_graph, "")):
+            build = gen(case)
+            if gen is not matmul_graph:
+                try:  # (the plan of a graph is made on the oracle; a case it rejects is no case)
+                    build(OracleKernel())
+                except Exception:  # noqa: BLE001
+                    continue
+            t = Tester(ker, run_mode="das")
+            try:
+                build(t)
+                t.codegen()
+                t.das()
+                done += 1
+            except RuntimeError as e:
+                if not any(s in str(e) for s in ("needs a Copy", "not supported", "too many")):
+                    raise RuntimeError("case %d: %s" % (case, e)) from e
+                refused += 1
+    return done, refused
+
+
+if __name__ == "__main__":
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--das-seeds", type=int, default=200)
+    n_done, n_refused = compile_in_das_mode(ap.parse_args().das_seeds)
+    print("compiled %d random graphs in disassembly mode, %d refused with a documented error" % (n_done, n_refused))

@@ -181,8 +181,10 @@ def test_dynamic_shape_recodegen_is_consistent():
         fresh.codegen()
         strip = lambda s: re.sub(r"@0x[0-9a-f]+", "@", s)
         assert strip(reused.das()) == strip(fresh.das()), rows
-    # per-shape JIT stays far below the 50 us budget once the kernel exists (first call excluded)
-    assert sorted(jit[1:])[len(jit[1:]) // 2] < 50.0, jit
+    # per-shape JIT stays far below the 50 us budget once the kernel exists (first call excluded; not a statement
+    # about a sanitizer build of the host library, which DVM_HOST_LIBRARY names)
+    if not os.environ.get("DVM_HOST_LIBRARY"):
+        assert sorted(jit[1:])[len(jit[1:]) // 2] < 50.0, jit
 
 
 def test_zero_size_shapes_are_idle():
