@@ -75,6 +75,8 @@ def _load():
         "dvm_obj_dtype": (ci, [vp]),
         "dvm_rt_input": (ci, [vp, vp, vp, cs]),
         "dvm_rt_bind_device": (ci, [vp, vp, vp]),
+        "dvm_rt_bind_device_view": (ci, [vp, vp, vp, i64p, cs]),
+        "dvm_rt_set_workspace_allocator": (ci, [vp, vp, vp]),
         "dvm_rt_unbind_device": (ci, [vp]),
         "dvm_rt_normalize": (ci, [vp]),
         "dvm_rt_codegen": (ci, [vp]),
@@ -501,11 +503,30 @@ class PyKernel(Kernel):
         self._inputs[load._h] = arr
         _check(_lib.dvm_rt_input(self._rt, load._h, arr.ctypes.data, arr.nbytes))
 
-    def bind_device(self, io, device_ptr, shape=None):
-        """Binds caller-owned device memory (e.g. a torch tensor's data_ptr()) to a load or store."""
+    def bind_device(self, io, device_ptr, shape=None, strides=None):
+        """Binds caller-owned device memory (e.g. a torch tensor's data_ptr()) to a load or store. `strides`
+        (elements, one per dim) binds a load to memory that is not contiguous: it is then read through them."""
         if shape is not None and io._h in self._load_shape:
             self._load_shape[io._h].update(list(shape))
-        _check(_lib.dvm_rt_bind_device(self._rt, io._h, ctypes.c_void_p(device_ptr)))
+        if strides is not None:
+            arr, n = _i64(strides)
+            _check(_lib.dvm_rt_bind_device_view(self._rt, io._h, ctypes.c_void_p(device_ptr), arr, n))
+        elif io._h in self._load_shape:  # (a load that was strided at an earlier call is dense again)
+            _check(_lib.dvm_rt_bind_device_view(self._rt, io._h, ctypes.c_void_p(device_ptr), None, 0))
+        else:
+            _check(_lib.dvm_rt_bind_device(self._rt, io._h, ctypes.c_void_p(device_ptr)))
+
+    def set_workspace_allocator(self, alloc):
+        """`alloc(nbytes) -> device address` supplies the workspace of the launches from now on (a framework's
+        caching allocator); None gives it back to the runner. The memory has to stay valid until the launches of
+        the run that follows have finished."""
+        if alloc is None:
+            self._ws_callback = None
+            _check(_lib.dvm_rt_set_workspace_allocator(self._rt, None, None))
+            return
+        proto = ctypes.CFUNCTYPE(ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p)
+        self._ws_callback = proto(lambda nbytes, _user: int(alloc(int(nbytes))))  # kept alive with the kernel
+        _check(_lib.dvm_rt_set_workspace_allocator(self._rt, ctypes.cast(self._ws_callback, ctypes.c_void_p), None))
 
     def normalize(self):
         """Shape inference only: store.shape() is valid afterwards."""

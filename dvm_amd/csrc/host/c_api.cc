@@ -59,6 +59,9 @@ struct dvm_rt {
   std::map<NDObject *, size_t> store_extent;  // strided stores: elements of the whole buffer they write into
   std::map<NDObject *, Buffer> buffers;
   Buffer workspace;
+  dvm_ws_alloc_fn ws_fn = nullptr;  // the caller's workspace allocator (dvm_rt_set_workspace_allocator), or none
+  void *ws_user = nullptr;
+  std::map<NDObject *, std::unique_ptr<dvm_shape>> view_strides;  // loads bound through strides (dvm_rt_bind_device_view)
   uint64_t fake_addr = 0x1000;
   double jit_us = 0.0;
   WsAlloc ws_alloc;
@@ -102,7 +105,15 @@ namespace {
 
 void *WsAlloc::Alloc(size_t size) {
   Buffer &w = rt->workspace;
-  if (w.ptr == nullptr || w.bytes < size) {
+  if (rt->ws_fn != nullptr && !rt->das_mode) {  // the caller's allocator: asked at every code generation, never freed here
+    rt->Release(w);
+    w.ptr = rt->ws_fn(size, rt->ws_user);
+    if (w.ptr == nullptr) throw std::runtime_error("DVM EXCEPTION. reason: the workspace allocator returned no memory");
+    w.bytes = size;
+    w.owned = false;
+    return w.ptr;
+  }
+  if (w.ptr == nullptr || w.bytes < size || !w.owned) {
     rt->Release(w);
     w.ptr = rt->AllocDevice(size);
     w.bytes = size;
@@ -642,9 +653,54 @@ int dvm_rt_bind_device(dvm_rt *rt, dvm_obj *io, void *device_ptr) {
       -1);
 }
 
+int dvm_rt_bind_device_view(dvm_rt *rt, dvm_obj *load, void *device_ptr, const int64_t *strides, size_t rank) {
+  return Guard(
+      [&]() {
+        NDObject *o = Obj(load);
+        if (o->kind != kObjLoad || o->full_shape_ref != nullptr) throw std::runtime_error("DVM EXCEPTION. reason: only a plain load takes a strided binding");
+        if (strides == nullptr) {
+          if (rt->view_strides.erase(o) != 0) {
+            o->strided = false;
+            o->stride_ref = nullptr;
+          }
+        } else {
+          if (rank != static_cast<size_t>(o->shape_ref_->size)) throw std::runtime_error("DVM EXCEPTION. reason: one stride per dim of the load");
+          std::unique_ptr<dvm_shape> &st = rt->view_strides[o];
+          if (!st) st.reset(new dvm_shape());
+          st->Set(strides, rank);
+          o->strided = true;
+          o->stride_ref = &st->ref;
+          o->view_offset = 0;
+        }
+        Buffer &b = rt->buffers[o];
+        rt->Release(b);
+        b.ptr = device_ptr;
+        b.owned = false;
+        b.bytes = 0;
+        return 0;
+      },
+      -1);
+}
+
+int dvm_rt_set_workspace_allocator(dvm_rt *rt, dvm_ws_alloc_fn alloc, void *user) {
+  return Guard(
+      [&]() {
+        rt->ws_fn = alloc;
+        rt->ws_user = user;
+        if (!rt->workspace.owned) rt->workspace = Buffer();  // (memory of an earlier allocator is not ours to keep)
+        return 0;
+      },
+      -1);
+}
+
 int dvm_rt_unbind_device(dvm_rt *rt) {
   return Guard(
       [&]() {
+        for (auto &kv : rt->view_strides) {
+          kv.first->strided = false;
+          kv.first->stride_ref = nullptr;
+        }
+        rt->view_strides.clear();
         for (auto it = rt->buffers.begin(); it != rt->buffers.end();) {
           if (!it->second.owned) {
             it->first->addr = nullptr;

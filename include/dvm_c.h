@@ -105,6 +105,17 @@ int dvm_obj_dtype(const dvm_obj *o);
 int dvm_rt_input(dvm_rt *rt, dvm_obj *load, const void *host, size_t bytes);
 /* Binds a caller-owned device buffer to a load or store (no copy, no ownership). */
 int dvm_rt_bind_device(dvm_rt *rt, dvm_obj *io, void *device_ptr);
+/* Binds a caller-owned device buffer to a load that reads it through element strides (a tensor that is not
+ * contiguous: a transposed or sliced view), `strides[rank]` against the load's shape; NULL makes the load dense
+ * again. The reference takes such tensors through Load with a stride list (include/dvm.h:294); its torch adapter
+ * passes a tensor's strides the same way (docs/pytorch.md:209-262). */
+int dvm_rt_bind_device_view(dvm_rt *rt, dvm_obj *load, void *device_ptr, const int64_t *strides, size_t rank);
+/* The workspace of the kernel's launches comes from `alloc(bytes, user)` (device memory that stays valid until the
+ * launches of the next dvm_rt_run have finished) instead of the runner's own allocation: the counterpart of the
+ * WsAllocator argument of Kernel::CodeGen (include/dvm.h:208-210), so that a framework's caching allocator can
+ * own it. NULL restores the runner's allocation. */
+typedef void *(*dvm_ws_alloc_fn)(size_t bytes, void *user);
+int dvm_rt_set_workspace_allocator(dvm_rt *rt, dvm_ws_alloc_fn alloc, void *user);
 /* Forgets every binding made by dvm_rt_bind_device (the memory stays the caller's); loads and stores get
  * buffers of the runner again at the next dvm_rt_input / dvm_rt_codegen. */
 int dvm_rt_unbind_device(dvm_rt *rt);
