@@ -130,6 +130,9 @@ int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf) {
   hipError_t err = hipGetDeviceCount(&count);
   if (err != hipSuccess) return static_cast<int>(err);
   if (dev_id < 0 || dev_id >= count) return static_cast<int>(hipErrorInvalidDevice);
+  // The limits below (compute units, local memory) are one set per process: a second call has to name the same
+  // device. (One process drives one GPU; another device's limits would silently replace the first's otherwise.)
+  if (g_dev.ready && g_dev.dev != dev_id) return DVM_HIP_ERROR_OTHER_DEVICE;
   err = hipSetDevice(dev_id);
   if (err != hipSuccess) return static_cast<int>(err);
   hipDeviceProp_t prop;
@@ -461,6 +464,7 @@ int dvm_hip_event_elapsed_time(float *ms, void *start, void *end) {
 }
 const char *dvm_hip_error_string(int code) {
   if (code == DVM_HIP_ERROR_WS_TOO_LARGE) return "the programs need more workspace than the static workspace holds (DVM_HIP_STATIC_WS_BYTES)";
+  if (code == DVM_HIP_ERROR_OTHER_DEVICE) return "dvm_hip_init_vm was called for another device before: one process drives one device";
   if (code == DVM_HIP_ERROR_BAD_WS_WORD) return "a workspace word names no program, no word of its blob, or an offset outside the workspace";
   return hipGetErrorString(static_cast<hipError_t>(code));
 }

@@ -29,7 +29,10 @@ typedef struct {
 } dvm_hip_sysconfig;
 
 /* Queries device `dev_id`, loads the VM kernels and fills `conf`.
+ * The limits it finds are one set per process: a later call has to name the same device, another one gets
+ * DVM_HIP_ERROR_OTHER_DEVICE (one process drives one GPU, as the reference's runtime does after SetDevice).
  * Replaces dvm::gpu::InitVM (src/vm_gpu.h:153). */
+#define DVM_HIP_ERROR_OTHER_DEVICE (-4)
 int dvm_hip_init_vm(int dev_id, dvm_hip_sysconfig *conf);
 
 /* Launch geometry for a program of interpreter kind `kind` (the schedule id

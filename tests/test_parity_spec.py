@@ -102,32 +102,36 @@ def test_dyn_spec_fall_reduce():  # :113-130
         assert t.check(x5, np.sum(d1 + 0.02, axis=dims_shape, keepdims=True) * (d1 + 0.02), 1e-4)
 
 
-@pytest.mark.parametrize("fallback_first", [False, True])
-def test_dyn_spec_rmsnorm_reloc(fallback_first):  # :134-160: rows that fit a tile and rows of 65536 on one kernel object
-    t = Tester("vector:spec,dyn")
-    x = t.load([-1, -1], "float16")
-    gamma = t.load([-1], "float16")
-    width = t.scalar(dvm.int64)
-    x_fp32 = t.cast(x, "float32")
-    square_sum = t.sum(t.mul(x_fp32, x_fp32), [1], True)
-    t.spec_next()
-    rstd = t.div(1.0, t.sqrt(t.add(t.div(square_sum, width), 1e-6)))
-    normalized = t.cast(t.mul(x_fp32, rstd), "float16")
-    out = t.store(t.mul(normalized, gamma))
-    shapes = [(2, 8192), (3, 65536), (17, 129), (4, 32768)]
-    if fallback_first:
-        shapes = shapes[1:] + shapes[:1]
-    rng = np.random.default_rng(17)
-    for rows, cols in shapes * 2:
-        x_data = rng.normal(0, 1, (rows, cols)).astype(np.float16)
-        gamma_data = rng.normal(1, 0.1, (cols,)).astype(np.float16)
-        t.input(x, x_data)
-        t.input(gamma, gamma_data)
-        width.update(cols)
-        t.run()
-        x_ref = x_data.astype(np.float32)
-        rstd_ref = 1.0 / np.sqrt(np.mean(x_ref * x_ref, axis=1, keepdims=True) + 1e-6)
-        assert t.check(out, (x_ref * rstd_ref).astype(np.float16) * gamma_data, 3e-3)
+def _rmsnorm_fp16(x, gamma):
+    """RMSNorm in fp32 on fp16 data, the normalised value rounded to fp16 before the scale by gamma."""
+    xf = x.astype(np.float32)
+    return (xf / np.sqrt((xf * xf).mean(axis=1, keepdims=True) + 1e-6)).astype(np.float16) * gamma
+
+
+# The case of :134-160: ONE dynamic speculative kernel object serves rows that fit a tile of the reference's vector
+# core and rows that do not (65536 elements), in either order, and gets new addresses at every call. The row length
+# enters the graph as an int64 scalar that is updated per call.
+RELOC_SHAPES = [(2, 8192), (3, 65536), (17, 129), (4, 32768)]
+
+
+@pytest.mark.parametrize("order", [RELOC_SHAPES, RELOC_SHAPES[1:] + RELOC_SHAPES[:1]], ids=["tile_first", "long_rows_first"])
+def test_dyn_spec_rmsnorm_reloc(order):
+    k = Tester("vector:spec,dyn")
+    rows_in, scale_in, n_cols = k.load([-1, -1], "float16"), k.load([-1], "float16"), k.scalar(dvm.int64)
+    v = k.cast(rows_in, "float32")
+    sq = k.sum(k.mul(v, v), [1], True)
+    k.spec_next()
+    inv_rms = k.div(1.0, k.sqrt(k.add(k.div(sq, n_cols), 1e-6)))
+    result = k.store(k.mul(k.cast(k.mul(v, inv_rms), "float16"), scale_in))
+    gen = np.random.default_rng(17)
+    for n_rows, width in order + order:  # every shape twice: the second visit finds the kernel object used
+        data = gen.normal(0, 1, (n_rows, width)).astype(np.float16)
+        gamma = gen.normal(1, 0.1, (width,)).astype(np.float16)
+        k.input(rows_in, data)
+        k.input(scale_in, gamma)
+        n_cols.update(width)
+        k.run()
+        assert k.check(result, _rmsnorm_fp16(data, gamma), 3e-3), (n_rows, width)
 
 
 def test_spec_dead_code():  # :164-174: a load nobody uses
