@@ -363,6 +363,17 @@ void Compiler::UndoSplitReduces(bool keep_programs) {
   k_->ops_ = saved_ops_;
   saved_ops_.clear();
   for (size_t i = 0; i < k_->ops_.size(); ++i) k_->ops_[i]->id = static_cast<int>(i);
+  // (the records go whatever happens below: a later code generation must not find them again)
+  struct DropRecords {
+    std::vector<SplitRecord *> &v;
+    ~DropRecords() {
+      for (SplitRecord *rec : v) {
+        delete rec->second;
+        delete rec;
+      }
+      v.clear();
+    }
+  } drop{splits_};
   if (keep_programs) {
     auto renumber = [&](int &op_id) {
       if (op_id < 0) return;
@@ -376,11 +387,6 @@ void Compiler::UndoSplitReduces(bool keep_programs) {
       for (Program::Fill &f : p.fills) renumber(f.op_id);
     }
   }
-  for (SplitRecord *rec : splits_) {
-    delete rec->second;
-    delete rec;
-  }
-  splits_.clear();
 }
 
 // ---------- which values cross sub-kernels ----------

@@ -117,3 +117,32 @@ def test_static_workspace_holds_the_partials_of_shared_reduces_and_split_product
         assert rc == 0, hip.dvm_hip_error_string(rc)
         assert hip.dvm_hip_synchronize_stream(None) == 0
         assert np.array_equal(t.output(out).view(np.uint8), want.view(np.uint8)), marker
+
+
+def test_static_workspace_passes_over_launches_with_nothing_to_do_and_refuses_a_word_listed_twice():
+    # A kernel with a sub-kernel over an empty tensor: its exported program has the geometry {0, 0, 0}. The entry point
+    # passes over it, as the allocating route does; the other programs still run, and every program is checked
+    # against its geometry before the first one is launched.
+    hip = _hip()
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal([70000, 64]).astype(np.float32)
+    t = Tester("split")
+    out = t.store(t.sum(t.load(x), (0,), True))          # a shared reduce: two launches and a workspace
+    t.store(t.mul(t.load(np.zeros([0, 16], np.float32)), 2.0))  # nothing to do
+    t.run()
+    want = t.output(out).copy()
+    programs = t.programs()
+    assert any(tuple(p[1]) == (0, 0, 0) for p in programs) and sum(1 for p in programs if tuple(p[1]) != (0, 0, 0)) == 2, [p[1] for p in programs]
+    blobs, geo, words, n_ws = _pack(programs)
+    assert hip.dvm_hip_memset(t.device_ptr(out), 0, want.nbytes) == 0
+    rc = hip.dvm_hip_launch_vm_static_ws(blobs, len(programs), geo, words, n_ws, t.workspace_bytes(), None)
+    assert rc == 0, hip.dvm_hip_error_string(rc)
+    assert hip.dvm_hip_synchronize_stream(None) == 0
+    assert np.array_equal(t.output(out).view(np.uint8), want.view(np.uint8))
+    # the same workspace word listed twice would get the workspace address added twice: refused, nothing launched
+    pairs = [v for i, p in enumerate(programs) for w in p[2] for v in (i, w)]
+    twice = (ctypes.c_uint32 * (len(pairs) + 2))(*(pairs + pairs[:2]))
+    assert hip.dvm_hip_memset(t.device_ptr(out), 0, want.nbytes) == 0
+    assert hip.dvm_hip_launch_vm_static_ws(blobs, len(programs), geo, twice, n_ws + 1, t.workspace_bytes(), None) == ERR_BAD_WS_WORD
+    assert hip.dvm_hip_synchronize_stream(None) == 0
+    assert not t.output(out).any()
