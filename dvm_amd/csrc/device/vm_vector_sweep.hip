@@ -276,7 +276,9 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
           case VOP_LDS: x = sreg_get(a); break;
           case VOP_LDI: x = __uint_as_float(imm); break;
           case VOP_STS: sreg_write(sr, a, x); break;
-          case VOP_UN: x = round_to(uniform_unary(sub, x), rnd); break;
+          case VOP_UN:  // (square root and logarithm in line: the out-of-line forms save registers to scratch memory around the call)
+            x = round_to(sub == VU_SQRT ? sqrtf(x) : (sub == VU_LOG ? logf(x) : uniform_unary(sub, x)), rnd);
+            break;
           case VOP_CAST: {
             x = uniform_cast(sub, x);
             if (sub == VC_I2F || sub == VC_RND) x = round_to(x, rnd);
@@ -417,8 +419,17 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
         uint32_t bpc = body_pc;
         bool have_operand = false;  // the first instruction's operand is in `operand` already
         if (parked && keep_rd) {
-          vreg_load(keep_lds, keep_at, keep_fmt, nthreads, tid, acc);
           bpc += keep_prefix;  // what was parked is the value behind the first keep_prefix instructions
+          // The round starts from local memory; when the first instruction it executes fetches a memory operand (the
+          // weight row of a normalisation), that trip starts first and the parked slabs are unpacked under it.
+          const vu2 ahead = code_at(bpc);
+          const uint32_t aw = uni(ahead[0]);
+          if ((aw & 0x7fu) == VOP_BINF && ((aw >> 16) & 0xfu) == VK_MEM) {
+            const Desc d = desc_at(aw >> 24);
+            mem_load(as_mem(d), offsets_of(d), sl, operand);
+            have_operand = true;
+          }
+          vreg_load(keep_lds, keep_at, keep_fmt, nthreads, tid, acc);
         } else {
           Offs off;
           FOR_U off.v[u] = a_koff + roff.v[u];
