@@ -258,6 +258,8 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
     }
     const bool wide = (h->sched & VS_WIDE) != 0;
     if (wide && threads > 512) return static_cast<int>(hipErrorInvalidValue);
+    // (the kernels that keep the innermost axis are built for at most 512 lanes as well)
+    if ((h->sched & VS_KIND_MASK) == VS_REDY && threads > 512) return static_cast<int>(hipErrorInvalidValue);
     // the sweep build trusts the flag: it is only defined for programs that reduce the innermost axis, two slabs a lane
     const bool sweeps = (h->sched & VS_SWEEPS) != 0;
     if (sweeps && (wide || (h->sched & VS_KIND_MASK) != VS_REDX || !sweeps_flag_holds(p))) return static_cast<int>(hipErrorInvalidValue);
@@ -274,7 +276,7 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
     {
       // local memory the interpreter will touch: reduce scratch, V registers, rounds parked by a load
       const uint64_t u = wide ? DVM_VEC_U_WIDE : 2;
-      uint64_t need = static_cast<uint64_t>(threads) * 8 + static_cast<uint64_t>(h->n_vslot) * u * 16 * threads;
+      uint64_t need = static_cast<uint64_t>(DVM_VEC_RED_SCRATCH_DOUBLES(h->sched, threads)) * 8 + static_cast<uint64_t>(h->n_vslot) * u * 16 * threads;
       uint64_t parked = 0;
       for (uint64_t i = h->code_off; i < code_end; ++i) {
         if (VI_OP(p.w[i]) != VOP_LD) continue;

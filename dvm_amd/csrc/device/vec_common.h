@@ -624,7 +624,7 @@ __device__ __forceinline__ void red_accumulate_int(RedAcc<SCHED> &r, uint32_t ki
 //   [64, 80)  what the first wave hands to the others after a per-team run: two buffers (in turn) of 16 floats.
 // With the buffers used in turn a wave cannot overwrite what a slower wave still has to read: between two uses of
 // one buffer lies the barrier of the other one, which the slower wave only reaches once its reads are done.
-// VS_REDY uses [0, lanes) as one buffer with barriers on both sides.
+// VS_REDY uses [0, E * lanes) as one buffer with barriers on both sides.
 constexpr uint32_t kPartialsPerBuffer = 32;
 constexpr uint32_t kBoxAt = 64;
 
@@ -695,7 +695,10 @@ __device__ __forceinline__ void red_finish_x(double &r0, double &r1, uint32_t k0
 }
 
 // End of a sweep, innermost axis kept: the rows of the workgroup that share an output group combine their
-// partials through local memory, element by element.
+// partials through local memory (DVM_VEC_RED_SCRATCH_DOUBLES doubles: one per lane and element). Every lane writes
+// its E partials; the lane of row r then combines, for element r (and r + rows, ...) of its group, the partials of
+// all rows in row order and leaves the result where row 0's was; after a second barrier every lane reads the E
+// results of its group. Three barriers per slot, and each partial is read once.
 template <int SCHED>
 __device__ __forceinline__ RedAcc<SCHED> red_finish_y(RedAcc<SCHED> r, uint32_t rk, uint32_t tlog, uint32_t nthreads, uint32_t k_local,
                                                       uint32_t r_local, double *scratch) {
@@ -705,14 +708,25 @@ __device__ __forceinline__ RedAcc<SCHED> red_finish_y(RedAcc<SCHED> r, uint32_t 
   if constexpr (SCHED == VS_REDY) {
     const uint32_t tx = 1u << tlog, ty = nthreads >> tlog;
     if (ty > 1) {
-      FOR_E {
-        __syncthreads();
-        scratch[r_local * tx + k_local] = r.v[e];
-        __syncthreads();
-        double t = scratch[k_local];
-        for (uint32_t j = 1; j < ty; ++j) t = red_combine(rk, t, scratch[j * tx + k_local]);
-        r.v[e] = t;
+      __syncthreads();  // (what an earlier sweep left here has been read)
+      FOR_E scratch[(e * ty + r_local) * tx + k_local] = r.v[e];
+      __syncthreads();
+      for (uint32_t v = r_local; v < static_cast<uint32_t>(E); v += ty) {
+        const double *col = scratch + v * ty * tx + k_local;
+        double t = col[0];
+        uint32_t j = 1;
+        for (; j + 4 <= ty; j += 4) {  // four reads in flight, combined in row order
+          const double a0 = col[j * tx], a1 = col[(j + 1) * tx], a2 = col[(j + 2) * tx], a3 = col[(j + 3) * tx];
+          t = red_combine(rk, t, a0);
+          t = red_combine(rk, t, a1);
+          t = red_combine(rk, t, a2);
+          t = red_combine(rk, t, a3);
+        }
+        for (; j < ty; ++j) t = red_combine(rk, t, col[j * tx]);
+        scratch[v * ty * tx + k_local] = t;
       }
+      __syncthreads();
+      FOR_E r.v[e] = scratch[e * ty * tx + k_local];
     }
   }
   return r;

@@ -79,7 +79,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
   const bool team_is_block = h.team_is_block != 0;
   // per-team runs (VOP_UNI_BEGIN .. VOP_UNI_END) are computed by the first wave when the team is the workgroup
   const uint32_t skips_runs = (SCHED == VS_REDX && team_is_block && uni(tid >> 6) != 0u) ? 1u : 0u;
-  vf4 *planes = reinterpret_cast<vf4 *>(lds + nthreads);  // first nthreads doubles: reduce scratch
+  vf4 *planes = reinterpret_cast<vf4 *>(lds + DVM_VEC_RED_SCRATCH_DOUBLES(SCHED, nthreads));  // behind the reduce scratch
   vf4 *keep_lds = planes + h.n_vslot * U * nthreads;      // behind the V registers: rounds parked by VI_LD_KEEP_WR
 
   // lane -> (kept local index, reduce local index)
@@ -470,6 +470,67 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                 }
               }
               if (!pair) continue;
+            } else if constexpr (SCHED == VS_REDY) {
+              if (in_sweep && (w0 & VI_LD_RED2)) {
+                // The round is this load and the float reduce behind it, which closes the round. A lane's rounds are
+                // rows far apart in memory and nothing else of the wave is in flight meanwhile, so up to four rounds
+                // are fetched in one trip and reduced one after the other, in the order of the rounds.
+                constexpr int NR = 4;
+                const uint32_t wr = uni(fetched[0]);
+                const uint32_t rsub = (wr >> 8) & 0xffu, rslot = wr >> 24;
+                const uint32_t left = n_rounds - round;
+                const uint32_t take = left < static_cast<uint32_t>(NR) ? left : static_cast<uint32_t>(NR);
+                constexpr uint32_t kFast = VMF_VEC | VMF_ALIGNED;
+                Offs offs[NR];
+                Slabs sls[NR];
+                Acc xs[NR];
+                offs[0] = off;
+                sls[0] = sl;
+                bool wide_all = take == static_cast<uint32_t>(NR) && (m.flags & kFast) == kFast && sl.uniform;
+                const uint64_t koff = space_offset(kvalid ? kidx : 0u, h.kdims, h.n_kdim, m.kstride, true);
+#pragma unroll
+                for (int j = 1; j < NR; ++j) {
+                  uint32_t nvp_j = 0;
+                  FOR_U {
+                    const uint32_t ru = ridx + (static_cast<uint32_t>(j) * U + u) * r_step;
+                    const bool ok = kvalid && ru < r_lim;
+                    offs[j].v[u] = koff + space_offset(ok ? ru : 0u, h.rdims, h.n_rdim, m.rstride, false);
+                    nvp_j |= (ok ? (nvp_out & 0xfu) : 0u) << (4 * u);
+                  }
+                  sls[j] = slab_state(nvp_j);
+                  wide_all = wide_all && sls[j].uniform;
+                }
+                if (wide_all) {
+#pragma unroll
+                  for (int j = 0; j < NR; ++j) mem_load_wide(m, offs[j], sls[j].full, xs[j]);
+                } else {
+#pragma unroll
+                  for (int j = 0; j < NR; ++j)
+                    if (static_cast<uint32_t>(j) < take) mem_load(m, offs[j], sls[j], xs[j]);
+                }
+#pragma unroll
+                for (int j = 0; j < NR; ++j) {
+                  if (static_cast<uint32_t>(j) >= take) break;
+                  Acc &x = xs[j];
+                  if (rsub & VRF_SQUARE) FOR_U x.v[u] = x.v[u] * x.v[u];
+                  if (rslot == 0) {
+                    red_accumulate<SCHED>(racc0, rsub & 0xfu, x, sls[j]);
+                    if (rsub & VRF_PAIR) {
+                      FOR_U x.v[u] = x.v[u] * x.v[u];
+                      red_accumulate<SCHED>(racc1, rsub & 0xfu, x, sls[j]);
+                    }
+                  } else {
+                    red_accumulate<SCHED>(racc1, rsub & 0xfu, x, sls[j]);
+                  }
+                }
+                round += take - 1u;
+                ridx += (take - 1u) * r_step * U;
+                pc = round + 1u < n_rounds ? sweep_pc : pc + 1u;
+                fetched = code64[pc];
+                end_round(true, true);
+                continue;
+              }
+              if (!take_next_along(m, off, sl, acc, src)) continue;
             } else {
               if (!take_next_along(m, off, sl, acc, src)) continue;
             }
@@ -746,7 +807,9 @@ extern "C" __global__ void __launch_bounds__(512) dvm_vm_vec_ry_u4(const VmParam
 #else
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_pw(const VmParam p) { vm_vector<VS_POINTWISE>(p); }
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_rx(const VmParam p) { vm_vector<VS_REDX>(p); }
-extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_ry(const VmParam p) { vm_vector<VS_REDY>(p); }
+// (the schedule that keeps the innermost axis holds one fp64 partial per element and slot and fetches four rounds
+// per trip: it takes more registers than 1024 lanes leave, and the host gives it at most 512)
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_vec_ry(const VmParam p) { vm_vector<VS_REDY>(p); }
 extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_rx_parts(const VmParam p) { vm_vector<VS_REDX, true>(p); }
-extern "C" __global__ void __launch_bounds__(1024) dvm_vm_vec_ry_parts(const VmParam p) { vm_vector<VS_REDY, true>(p); }
+extern "C" __global__ void __launch_bounds__(512) dvm_vm_vec_ry_parts(const VmParam p) { vm_vector<VS_REDY, true>(p); }
 #endif

@@ -174,12 +174,23 @@ class Compiler {
   struct SplitRecord {
     NDObject *reduce;     // the user's reduce (holds part_split and the longer shape meanwhile)
     NDObject *second;     // the synthetic reduce over the parts (owned here)
+    NDObject *turned = nullptr;  // the partial results seen with the parts innermost: what `second` reads (owned here)
+    NDObject *layout = nullptr;  // strides the launch over the parts stores its results with: parts innermost (owned here)
     int64_t shape[kMaxRank];
     size_t rank;
-    IntArrayRef axis0;    // {0}: what `second` reduces over
+    IntArrayRef axis0;    // what `second` reduces over: {0}, or the last dim of `turned`
     int64_t zero = 0;
+    IntArrayRef turn_order;  // the permutation `turned` stands for
+    int64_t turn_dims[kMaxRank];
   };
   std::vector<SplitRecord *> splits_;
+  // The strides a shared reduce's partial results are stored with (nullptr: dense in their own shape).
+  const NDObject *PartsLayout(const NDObject *o) const {
+    if (o->kind != kObjReduce || o->part_split == 0) return nullptr;
+    for (const SplitRecord *rec : splits_)
+      if (rec->reduce == o) return rec->layout;
+    return nullptr;
+  }
   struct Repoint {
     NDObject *consumer;
     int slot;

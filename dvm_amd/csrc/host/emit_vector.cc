@@ -667,7 +667,7 @@ void Compiler::FinishProgram() {
   std::memcpy(prog_->blob.w, &hdr_, sizeof(hdr_));
   std::memcpy(prog_->blob.w + hdr_.mem_off, mems_, sizeof(VMemDesc) * n_mem_);
   std::memcpy(prog_->blob.w + hdr_.code_off, code_.data(), 8 * code_.size());
-  prog_->lds_bytes = prog_->threads * 8 + static_cast<uint32_t>(max_vslot_) * u_ * 16 * prog_->threads;
+  prog_->lds_bytes = DVM_VEC_RED_SCRATCH_DOUBLES(hdr_.sched, prog_->threads) * 8 + static_cast<uint32_t>(max_vslot_) * u_ * 16 * prog_->threads;
   PlanRereads();
   uint64_t gt = (static_cast<uint64_t>(std::min<uint32_t>(hdr_.n_items, g_system.core_num * 4)) << 32) | prog_->threads;
   if (g_system.HasDevice()) {

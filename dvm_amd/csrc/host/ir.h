@@ -199,6 +199,7 @@ struct Tuning {
   int vec_sweeps = -1;  // DVM_VEC_SWEEPS=0: never the sweep build of the vector VM
   int cube_tile = -1;   // DVM_CUBE_TILE=256|128|64
   int cube_waves = -1;  // DVM_CUBE_WAVES=4|8
+  int red_split_turn = -1;  // DVM_RED_SPLIT_TURN=0: the reduce over the parts of a shared reduce walks them outermost, as they lie in memory
   int red_split = -1;    // DVM_RED_SPLIT=0: never share a reduce between workgroups; N >= 2: N parts whenever the graph allows
   int cube_splitk = -1;  // DVM_CUBE_SPLITK=0: never split the k axis; N >= 2: split it N ways whenever the shape allows
   int cube_exact = -1;  // DVM_CUBE_EXACT=1: never the hardware approximations of exp, log, sqrt, division in a matmul epilogue

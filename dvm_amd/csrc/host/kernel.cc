@@ -33,6 +33,7 @@ void Tuning::Read() {
   cube_exact = num("DVM_CUBE_EXACT");
   cube_splitk = num("DVM_CUBE_SPLITK");
   red_split = num("DVM_RED_SPLIT");
+  red_split_turn = num("DVM_RED_SPLIT_TURN");
   attn_waves = num("DVM_ATTN_WAVES");
   debug = std::getenv("DVM_DEBUG") != nullptr;
 }

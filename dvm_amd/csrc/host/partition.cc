@@ -147,7 +147,10 @@ void Compiler::Join(int a, const NDObject *o) {
       ai.reduce = o;
       ai.has_part = o->part_split != 0;
     }
-    if (o->in[0] != nullptr && o->in[0]->kind == kObjReduce && o->in[0]->part_split != 0) ai.over_parts = std::max<int64_t>(ai.over_parts, o->numel());
+    if (o->in[0] != nullptr) {
+      const NDObject *src = ViewRoot(o->in[0]);
+      if (src->kind == kObjReduce && src->part_split != 0) ai.over_parts = std::max<int64_t>(ai.over_parts, o->numel());
+    }
     DomMerge(ai, o->in[0]->shape_ref_->data, o->in[0]->rank());
   }
   DomMerge(ai, o->shape_ref_->data, o->rank());
@@ -335,6 +338,43 @@ bool Compiler::SplitLongReduces() {
       o->SetShape(longer, rec->rank + 1);
       o->part_split = c.split;
       splits_.push_back(rec);
+      if (k_->tuning_.red_split_turn != 0) {
+        // The partial results are written with the parts innermost ([outputs][parts]: a scattered store of a few
+        // values per workgroup), and the second reduce reads them through a view of that shape: it reduces the
+        // innermost axis of a dense operand, a row per output, rows spread over workgroups, every element of a row
+        // fetched at once. Over the outermost axis the same reduce had one workgroup per 512 outputs and a round
+        // trip to memory per two parts.
+        NDObject *layout = new NDObject(kObjStore, o->type_id_);
+        layout->strided = true;
+        layout->view_base_ = 0;
+        layout->vstride_[0] = 1;
+        NDObject *turned = new NDObject(kObjPermute, o->type_id_);
+        turned->in[0] = o;
+        turned->nin = 1;
+        turned->stage = o->stage;
+        turned->strided = true;
+        turned->view_base_ = 0;
+        int64_t shape_t[kMaxRank], dense = c.split;
+        for (size_t d = rec->rank; d-- > 0;) {
+          shape_t[d] = rec->shape[d];
+          turned->vstride_[d] = dense;
+          layout->vstride_[d + 1] = dense;
+          dense *= rec->shape[d];
+          rec->turn_dims[d] = static_cast<int64_t>(d) + 1;
+        }
+        shape_t[rec->rank] = c.split;
+        turned->vstride_[rec->rank] = 1;
+        rec->turn_dims[rec->rank] = 0;
+        rec->turn_order.data = rec->turn_dims;
+        rec->turn_order.size = rec->rank + 1;
+        turned->aux_ref = &rec->turn_order;
+        turned->SetShape(shape_t, rec->rank + 1);
+        rec->layout = layout;
+        rec->turned = turned;
+        rec->zero = static_cast<int64_t>(rec->rank);
+        second->in[0] = turned;
+        next.push_back(turned);
+      }
       next.push_back(second);
     }
   }
@@ -369,6 +409,8 @@ void Compiler::UndoSplitReduces(bool keep_programs) {
     ~DropRecords() {
       for (SplitRecord *rec : v) {
         delete rec->second;
+        delete rec->turned;
+        delete rec->layout;
         delete rec;
       }
       v.clear();

@@ -72,8 +72,8 @@ void Compiler::PairLoads() {
     code_[i] = w | VI_LD_PAIR;
   }
   // A sweep whose body is one load and one float reduce (the statistics sweep of a normalisation): the load may
-  // fetch two rounds per trip and do the reduce itself.
-  if ((hdr_.sched & VS_KIND_MASK) == VS_REDX) {
+  // fetch several rounds per trip and do the reduce itself.
+  if ((hdr_.sched & VS_KIND_MASK) != VS_POINTWISE) {
     for (size_t i = 1; i + 1 < code_.size(); ++i) {
       const uint64_t w = code_[i], nx = code_[i + 1];
       if (VI_OP(code_[i - 1]) != VOP_SWEEP || VI_OP(w) != VOP_LD || (static_cast<uint32_t>(w) & (VI_UNIFORM | VI_LD_PAIR))) continue;

@@ -131,6 +131,7 @@ void Compiler::BuildNodes(int a) {
       nodes_[out].nin = 1;
       nodes_[out].in[0] = idx;
       nodes_[out].ws_slot = ws_slot_[i];
+      nodes_[out].view = PartsLayout(o);
     }
   }
 }
@@ -557,7 +558,7 @@ void Compiler::ChooseSchedule() {
     uint32_t tx = n_k_part >= 64 ? 64 : Pow2Ceil(n_k_part);
     uint32_t ty = 256 / tx;
     const uint64_t items = (n_k + tx - 1) / tx;
-    if (items < 128 && n_r > 256) ty = max_threads / tx;  // few outputs: give each more lanes along the reduce space
+    if (items < 128 && n_r > 256) ty = 512 / tx;  // few outputs: give each more lanes along the reduce space (the kernel's limit is 512)
     else if (items < 128 && n_r >= 64) ty = 512 / tx;     // (the launch that reduces over the parts of a shared reduce, mostly)
     // (the parts of a shared reduce: with fewer than two workgroups per compute unit, 512 lanes each put twice the
     // loads in flight. Measured on MI355X, fp32 sums over axis 0: [8192,1024] 57 -> 47 us, [65536,768] 136 -> 97 us,

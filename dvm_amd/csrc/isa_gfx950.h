@@ -61,6 +61,10 @@ enum {
   VS_SWEEPS = 0x20,
 };
 #define DVM_VEC_SWEEP_BODY 6
+// Local memory at the start of a vector program's segment, in doubles: what the lanes of a workgroup combine their
+// reduce partials through. One double per lane; eight (one per element of a lane's group) on the schedule that keeps
+// the innermost axis. The V registers lie behind it.
+#define DVM_VEC_RED_SCRATCH_DOUBLES(sched, threads) ((((sched) & 0xfu) == 2u ? 8u : 1u) * (threads))
 
 // ---- opcodes ---------------------------------------------------------------
 // The interpreter is an accumulator machine. Per lane, `acc` holds U slabs of E
