@@ -229,8 +229,9 @@ static bool sweeps_flag_holds(const VmParam &p) {
     for (;; ++j) {
       if (j >= h->n_code || j - (i + 2) >= DVM_VEC_SWEEP_BODY) return false;
       const uint32_t bop = VI_OP(code[j]);
-      if (bop != VOP_BINF && bop != VOP_RED && bop != VOP_ST && bop != VOP_UN && bop != VOP_CAST && bop != VOP_ENDSWEEP) return false;
-      if ((bop == VOP_ST || (bop == VOP_BINF && VI_KIND(code[j]) == VK_MEM)) &&
+      if (bop != VOP_BINF && bop != VOP_RED && bop != VOP_ST && bop != VOP_UN && bop != VOP_CAST && bop != VOP_ENDSWEEP && bop != VOP_LD) return false;
+      if (bop == VOP_LD && VI_KIND(code[j]) != VK_MEM) return false;
+      if ((bop == VOP_ST || bop == VOP_LD || (bop == VOP_BINF && VI_KIND(code[j]) == VK_MEM)) &&
           (VI_A(code[j]) >= h->n_mem || !unguarded_ok(VI_A(code[j]), bop == VOP_ST))) return false;
       if (bop == VOP_BINF && VI_KIND(code[j]) == VK_REG) return false;
       if (static_cast<uint32_t>(code[j]) & VI_ENDS) break;

@@ -970,6 +970,23 @@ __device__ __forceinline__ float uniform_cast(uint32_t sub, float x) {
   return x != 0.0f ? 1.0f : 0.0f;
 }
 
+// Builds with -DDVM_VEC_STAMPS write the memory clock (100 MHz) at the STAMP() marks of the interpreter kernels, one row of 32 stamps per
+// wave, to the address in the last word of the blob when that word is not zero: where a launch spends its time,
+// wave by wave. Nothing of it exists in a regular build.
+#ifdef DVM_VEC_STAMPS
+#define STAMP()                                                                                               \
+  do {                                                                                                        \
+    if (stamp_base != 0 && stamp_n < 32u) {                                                                   \
+      const uint64_t now = __builtin_amdgcn_s_memrealtime();                                                  \
+      if ((threadIdx.x & 63u) == 0u)                                                                          \
+        reinterpret_cast<DVM_GLOBAL uint64_t *>(stamp_base)[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 32u + stamp_n] = now; \
+      ++stamp_n;                                                                                              \
+    }                                                                                                         \
+  } while (0)
+#else
+#define STAMP() do {} while (0)
+#endif
+
 }  // namespace
 
 #endif  // DVM_DEVICE_VEC_COMMON_H_

@@ -29,6 +29,11 @@ __shared__ uint32_t prog32[DVM_PARAM_BYTES / 4];
 // programs without one pay nothing for the part bounds.
 template <int SCHED, bool PARTS = false>
 __device__ __forceinline__ void vm_vector(const VmParam &p) {
+#ifdef DVM_VEC_STAMPS
+  const uint64_t stamp_base = p.w[DVM_PARAM_WORDS - 1];
+  uint32_t stamp_n = 0;
+#endif
+  STAMP();
   // The blob arrives as a kernel argument; decoding from there would cost a
   // dependent scalar-memory round trip per access, so each workgroup copies it
   // into local memory once and decodes from there.
@@ -47,6 +52,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
     }
     __syncthreads();
   }
+  STAMP();
   // the scalar fields of the header live in scalar registers; the axis tables stay in local memory
   struct {
     uint32_t n_kdim, n_rdim, team_log2, team_is_block, n_kidx, n_ridx, inner_extent, n_items, mem_off, code_off, n_vslot, r_chunk, k_per_chunk;
@@ -175,6 +181,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               ridx = sweep_rev ? ridx - r_step * U : ridx + r_step * U;
             } else {
               in_sweep = false;
+              STAMP();
               const uint32_t k0 = slot_kinds & 0xfu, k1 = (slot_kinds >> 4) & 0xfu;
               if constexpr (SCHED == VS_REDX) {
                 if (k0 <= VR_MIN || k1 <= VR_MIN) {
@@ -184,6 +191,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                 if (k0 <= VR_MIN) racc0 = red_finish_y<SCHED>(racc0, k0, tlog, nthreads, k_local, r_local, lds);
                 if (k1 <= VR_MIN) racc1 = red_finish_y<SCHED>(racc1, k1, tlog, nthreads, k_local, r_local, lds);
               }
+              STAMP();
             }
           }
 
@@ -523,6 +531,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
                     red_accumulate<SCHED>(racc1, rsub & 0xfu, x, sls[j]);
                   }
                 }
+                STAMP();
                 round += take - 1u;
                 ridx += (take - 1u) * r_step * U;
                 pc = round + 1u < n_rounds ? sweep_pc : pc + 1u;
@@ -795,6 +804,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
       }
     }
   }
+  STAMP();
 }
 
 }  // namespace

@@ -95,22 +95,6 @@ __device__ __forceinline__ float round_to(float x, uint32_t rnd) {
   return rnd == VRND_F16 ? round_f16(x) : (rnd == VRND_BF16 ? round_bf16(x) : x);
 }
 
-// Builds with -DDVM_VEC_STAMPS write the memory clock (100 MHz) at the marks below, one row of sixteen stamps per
-// wave, to the address in the last word of the blob when that word is not zero: where a launch spends its time,
-// wave by wave. Nothing of it exists in a regular build.
-#ifdef DVM_VEC_STAMPS
-#define STAMP()                                                                                               \
-  do {                                                                                                        \
-    if (stamp_base != 0 && stamp_n < 32u) {                                                                   \
-      const uint64_t now = __builtin_amdgcn_s_memrealtime();                                                  \
-      if ((threadIdx.x & 63u) == 0u)                                                                          \
-        reinterpret_cast<DVM_GLOBAL uint64_t *>(stamp_base)[(blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6)) * 32u + stamp_n] = now; \
-      ++stamp_n;                                                                                              \
-    }                                                                                                         \
-  } while (0)
-#else
-#define STAMP() do {} while (0)
-#endif
 
 template <bool PARTS>
 __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
@@ -488,6 +472,9 @@ __device__ __forceinline__ void vm_vector_sweeps(const VmParam &p) {
           } else if (bop == VOP_ST) {
             const Desc d = desc_at(ba);
             mem_store(as_mem(d), offsets_of(d), sl, acc);
+          } else if (bop == VOP_LD) {  // another operand's round (two reduces of two inputs in one sweep)
+            const Desc d = desc_at(ba);
+            mem_load(as_mem(d), offsets_of(d), sl, acc);
           } else if (bop == VOP_UN) {
             switch (bsub) {
               case VU_EXP: FOR_U acc.v[u] = slab_exp(acc.v[u]); break;

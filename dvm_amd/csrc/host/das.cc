@@ -165,7 +165,7 @@ std::string &VKernel::DisAssemble() {
               if ((VI_IMM(w) >> 16) & 3u) os << " (the value behind the next instruction, as " << kFmt[(VI_IMM(w) >> 20) & 3u] << ")";
             }
             if (static_cast<uint32_t>(w) & VI_LD_PAIR) os << "  ; fetches the next instruction's operand in the same trip";
-            if (static_cast<uint32_t>(w) & VI_LD_RED2) os << "  ; fetches two rounds per trip and does the reduce behind it";
+            if (static_cast<uint32_t>(w) & VI_LD_RED2) os << "  ; fetches several rounds per trip and does the reduce behind it";
             break;
           case VOP_BINF:
             if (VI_KIND(w) == VK_SREG2) {  // two chained operations

@@ -287,6 +287,9 @@ bool Compiler::FitsSweepBuild() {
         case VOP_RED:
           if (bsub & VRF_INT) return false;
           break;
+        case VOP_LD:  // another input of the sweep
+          if (bk != VK_MEM || !walks_like_load(VI_A(b)) || (static_cast<uint32_t>(b) & (VI_LD_KEEP_WR | VI_LD_KEEP_RD | VI_LD_RED2))) return false;
+          break;
         case VOP_ST:
           if (!walks_like_load(VI_A(b)) || !(mems_[VI_A(b)].flags & VMF_VEC)) return false;
           break;

@@ -53,7 +53,8 @@ enum {
   VS_WIDE = 0x10,    // flag: the program is laid out for DVM_VEC_U_WIDE slabs per lane (the *_u4 kernels)
   // flag (VS_REDX only): every sweep is a load of a contiguous operand followed by at most DVM_VEC_SWEEP_BODY
   // instructions out of: float binaries (add .. max) on immediates, S registers, the accumulator or memory operands
-  // that walk the reduced index space like the load (or not at all), float unaries, roundings, float reduces, stores;
+  // that walk the reduced index space like the load (or not at all), float unaries, roundings, float reduces, stores,
+  // loads of further operands that walk like the first;
   // between the sweeps nothing touches a V register; the kept and the reduced index space have at most two axes
   // each. Such a program may run on the sweep build of the VM
   // (dvm_vm_vec_rx_sw), which decodes a sweep's body once per sweep instead of once per instruction and round; the

@@ -247,8 +247,10 @@ def test_reduce_with_few_outputs_is_shared_between_workgroups(monkeypatch):
     t, das = compile_one([4096, 4096], (0,))
     assert das.count("== sub-kernel") == 2 and "shared-reduce parts=64 x 64" in das, das
     first, second = das.split("== sub-kernel 1 ==")
-    assert "kdims: 512 64  rdims: 4096" in first and "k[1,0] r[4096]" in first and "k[1,4096] r[0]" in first, das
-    assert "Mul.fp32 acc, #0x3f000000" in second and "Mul.fp32" not in first and "rdims: 64" in second, das
+    # (the partial sums are stored with the parts innermost, 64 to a column: the second launch reduces along rows)
+    assert "kdims: 512 64  rdims: 4096" in first and "k[1,0] r[4096]" in first and "gather k[64,1] r[0]" in first, das
+    assert "Mul.fp32 acc, #0x3f000000" in second and "Mul.fp32" not in first, das
+    assert "sched=reduce-x sweeps" in second and "kdims: 4096  rdims: 8" in second and "vec aligned k[64] r[1]" in second, das
     assert t.workspace_bytes() >= 64 * 4096 * 4
     dump_before = t.dump()
     t.codegen()
@@ -260,7 +262,7 @@ def test_reduce_with_few_outputs_is_shared_between_workgroups(monkeypatch):
     _, das = compile_one([4, 1 << 20], (1,), lambda t, x: t.sub(x, t.max(x, (1,), True)))
     assert "shared-reduce parts=" in das and das.count("== sub-kernel") == 3, das
     over_parts = das.split("== sub-kernel")[2]
-    assert "kept=1 " in over_parts and "Sub.fp32" not in over_parts, das
+    assert "kept=4 " in over_parts and "Sub.fp32" not in over_parts, das
     assert "sched=pointwise" in das.split("== sub-kernel")[3] and "Sub.fp32" in das.split("== sub-kernel")[3], das
     monkeypatch.setenv("DVM_RED_SPLIT", "0")
     _, das = compile_one([4096, 4096], (0,))
@@ -268,6 +270,11 @@ def test_reduce_with_few_outputs_is_shared_between_workgroups(monkeypatch):
     monkeypatch.setenv("DVM_RED_SPLIT", "3")
     _, das = compile_one([1000], (0,))
     assert "shared-reduce parts=3 x " in das, das
+    # DVM_RED_SPLIT_TURN=0: the partial results dense in their own shape, parts outermost, and reduced that way
+    monkeypatch.setenv("DVM_RED_SPLIT", "-1")
+    monkeypatch.setenv("DVM_RED_SPLIT_TURN", "0")
+    _, das = compile_one([4096, 4096], (0,))
+    assert "k[1,4096] r[0]" in das and "gather" not in das and "rdims: 64" in das.split("== sub-kernel 1 ==")[1], das
 
 
 def test_matmul_with_few_tiles_and_a_long_k_axis_is_split(monkeypatch):

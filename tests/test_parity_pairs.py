@@ -38,7 +38,7 @@ def test_statistics_sweeps_two_rounds_per_trip(monkeypatch, shape, dtype):
 
     (a, am), das_on = _run(monkeypatch, True, build)
     (b, bm), das_off = _run(monkeypatch, False, build)
-    assert "two rounds per trip" in das_on and "two rounds per trip" not in das_off, das_on
+    assert "rounds per trip" in das_on and "rounds per trip" not in das_off, das_on
     assert np.array_equal(a, b) and np.array_equal(am, bm)
     x64 = x.astype(np.float64)
     want = (x64 - x64.mean(1, keepdims=True)) / np.sqrt(x64.var(1, keepdims=True) + 1e-5)

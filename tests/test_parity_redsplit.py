@@ -188,3 +188,74 @@ def test_consumers_larger_than_the_reduce_get_launches_of_their_own():
     x64 = x.astype(np.float64)
     want = (x64 - x64.mean(0, keepdims=True)) / np.sqrt(x64.var(0, keepdims=True) + 1e-5)
     assert np.allclose(t.output(out), want, rtol=1e-5, atol=1e-5), float(np.abs(t.output(out) - want).max())
+
+
+def _channels_last_batch_norm(t, x, g, b):
+    n = x.shape[0] * x.shape[1] * x.shape[2]
+    lx, lg, lb = t.load(x), t.load(g), t.load(b)
+    mean = t.mul(t.sum(lx, (0, 1, 2), True), 1.0 / n)
+    var = t.sub(t.mul(t.sum(t.mul(lx, lx), (0, 1, 2), True), 1.0 / n), t.mul(mean, mean))
+    scale = t.div(lg, t.sqrt(t.add(var, 1e-5)))
+    return t.store(t.add(t.mul(lx, scale), t.sub(lb, t.mul(mean, scale)))), t.store(mean)
+
+
+@pytest.mark.parametrize("shape", [(32, 56, 56, 256), (8, 28, 28, 96), (4, 57, 31, 40)])
+def test_batch_norm_channels_last(monkeypatch, shape):
+    # [N, H, W, C] with the statistics over N, H, W: the innermost axis is kept, the reduce is shared between workgroups.
+    # Its partial results are stored with the parts innermost, so the launch over the parts reduces along rows (the sweep
+    # build where the part count allows); with DVM_RED_SPLIT_TURN=0 it walks them outermost. Both against float64.
+    rng = np.random.default_rng(shape[3])
+    x = (rng.standard_normal(shape, dtype=np.float32) * 2.0 + 3.0).astype(np.float32)
+    g = rng.uniform(0.5, 1.5, [1, 1, 1, shape[3]]).astype(np.float32)
+    b = rng.normal(0, 0.1, [1, 1, 1, shape[3]]).astype(np.float32)
+    x64 = x.astype(np.float64)
+    want = (x64 - x64.mean((0, 1, 2), keepdims=True)) / np.sqrt(x64.var((0, 1, 2), keepdims=True) + 1e-5) * g + b
+    for turn in ("1", "0"):
+        monkeypatch.setenv("DVM_RED_SPLIT_TURN", turn)
+        monkeypatch.setenv("DVM_RED_SPLIT", "64" if shape[0] < 32 else "-1")
+        t = Tester("split")
+        y, mean = _channels_last_batch_norm(t, x, g, b)
+        t.run()
+        das = t.das()
+        assert "shared-reduce parts=" in das and t.num_launches() == 3, das
+        if turn == "1":
+            assert "sched=reduce-x" in das and "gather" in das, das  # rows of partial results, written scattered
+        else:
+            assert "sched=reduce-x" not in das, das
+        assert np.allclose(t.output(mean), x64.mean((0, 1, 2), keepdims=True), rtol=1e-5, atol=1e-5)
+        assert np.allclose(t.output(y), want, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("rows,cols,parts", [(4096, 512, 16), (4100, 520, 16), (1031, 64, 4), (30000, 8, 32), (257, 4096, 2)])
+@pytest.mark.parametrize("kind", ["sum", "sumsq", "max"])
+def test_column_reduces_fetch_several_rounds_per_trip(monkeypatch, rows, cols, parts, kind):
+    # a sweep that is one load and one reduce takes four rounds per trip to memory on the schedule that keeps the
+    # innermost axis: row counts that leave one, two and three rounds for the last trip, ragged columns, rows past the end
+    monkeypatch.setenv("DVM_RED_SPLIT", str(parts))
+    rng = np.random.default_rng(rows + cols)
+    x = rng.standard_normal([rows, cols], dtype=np.float32)
+    t = Tester("split")
+    lx = t.load(x)
+    if kind == "sum":
+        o = t.store(t.sum(lx, (0,), True))
+    elif kind == "sumsq":
+        o = t.store(t.sum(t.mul(lx, lx), (0,), True))
+    else:
+        o = t.store(t.max(lx, (0,), True))
+    t.run()
+    das = t.das()
+    assert "fetches several rounds per trip" in das, das
+    got = t.output(o)
+    x64 = x.astype(np.float64)
+    if kind == "max":
+        assert np.array_equal(got, x.max(0, keepdims=True))
+    elif kind == "sum":
+        assert _sum_close(got, x64, (0,))
+    else:
+        assert _sum_close(got, x64 * x64, (0,))
+    # no atomics anywhere: a second run gives the same bits
+    t2 = Tester("split")
+    l2 = t2.load(x)
+    o2 = t2.store(t2.sum(l2, (0,), True) if kind == "sum" else (t2.sum(t2.mul(l2, l2), (0,), True) if kind == "sumsq" else t2.max(l2, (0,), True)))
+    t2.run()
+    assert np.array_equal(got, t2.output(o2))
