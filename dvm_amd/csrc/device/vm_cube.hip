@@ -738,7 +738,29 @@ struct EpiArgs {
   uint32_t mem_off, code_off, batch0, batch1;
   uint32_t flags;   // VCubeHeader::epi_flags
   uint32_t w0v, immv;  // per lane: the two words of instruction `lane` of the epilogue program (the first 64)
+  uint32_t first;      // the instruction the epilogue starts at (VCF_DUMP16: the kernel has done the ones before it)
 };
+
+// What the epilogue reads the tile back from: fp32 accumulators (D16 = 0), or values already rounded to the operand
+// type and kept as their 16 bits (1: bf16, 2: fp16). One slab = 8 columns of local row `lr`.
+template <int D16, int BN>
+__device__ __forceinline__ void dump_read_slab(const void *dump, uint32_t lr, uint32_t g, vf4 &lo, vf4 &hi) {
+  if constexpr (D16 == 0) {
+    const float *src = reinterpret_cast<const float *>(dump) + lr * (BN + 4) + g * 8;
+    lo = *reinterpret_cast<const vf4 *>(src);
+    hi = *reinterpret_cast<const vf4 *>(src + 4);
+  } else {
+    const vu4 a = *reinterpret_cast<const vu4 *>(reinterpret_cast<const uint16_t *>(dump) + lr * (BN + 8) + g * 8);
+    if constexpr (D16 == 1) {
+      lo = vf4{__uint_as_float(a[0] << 16), __uint_as_float(a[0] & 0xffff0000u), __uint_as_float(a[1] << 16), __uint_as_float(a[1] & 0xffff0000u)};
+      hi = vf4{__uint_as_float(a[2] << 16), __uint_as_float(a[2] & 0xffff0000u), __uint_as_float(a[3] << 16), __uint_as_float(a[3] & 0xffff0000u)};
+    } else {
+      auto h2f = [](uint32_t bits) { return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(bits & 0xffffu))); };
+      lo = vf4{h2f(a[0]), h2f(a[0] >> 16), h2f(a[1]), h2f(a[1] >> 16)};
+      hi = vf4{h2f(a[2]), h2f(a[2] >> 16), h2f(a[3]), h2f(a[3] >> 16)};
+    }
+  }
+}
 
 // Runs the epilogue program on SL slabs whose accumulator values are in `acc`.
 // SLIM: the program holds only what VCF_SLIM lists (one temporary, float binaries, the hardware's exp / log / sqrt,
@@ -759,8 +781,8 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
   };
   if (h.flags & VCF_PLAIN_STORE) {
     // [Add mem] [cast.round] store: three instructions at most, done here without the dispatch loop
-    uint32_t at = 0;
-    uint32_t w0 = __builtin_amdgcn_readlane(h.w0v, 0);
+    uint32_t at = h.first;
+    uint32_t w0 = __builtin_amdgcn_readlane(h.w0v, at);
     uint64_t addr, boff;
     uint32_t dtype, sn, sm;
     if ((w0 & 0xffu) == VOP_BINF) {
@@ -782,7 +804,7 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
   (void)t2;
   (void)t3;
   (void)mask;
-  uint32_t pc = 0;
+  uint32_t pc = h.first;
   while (true) {
     // the program sits in two registers, one instruction per lane: no memory access to fetch one
     uint32_t w0, imm;
@@ -960,11 +982,10 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
 // returns true; otherwise the caller sends the slabs through epilogue_pass, which does the same with every guard.
 // A function of its own, and a small one: what a call costs is the registers the callee has to save (the interpreter's
 // pass saves and restores some hundred per lane through scratch memory, 12 us per tile and launch on MI355X).
-template <int ROWS, int BN, int TM, int WM>
-__device__ __attribute__((noinline)) bool epilogue_plain_pass(const float *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
+template <int ROWS, int BN, int TM, int WM, int D16>
+__device__ __attribute__((noinline)) bool epilogue_plain_pass(const void *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
                                                               uint32_t pass, uint32_t m, uint32_t n, uint32_t m_lo, uint32_t n_lo) {
   constexpr int NTHR = WM * 2 * 64;
-  constexpr int PITCH = BN + 4;
   constexpr int GROUPS = BN / 8;
   constexpr int PER_THREAD = ROWS * GROUPS / NTHR;
   constexpr int ROWS_PER_STEP = NTHR / GROUPS;
@@ -986,7 +1007,7 @@ __device__ __attribute__((noinline)) bool epilogue_plain_pass(const float *dump,
     sm = uni(d[5]);
     boff = static_cast<uint64_t>(ea.batch0) * uni(d[6]) + static_cast<uint64_t>(ea.batch1) * uni(d[7]);
   };
-  uint32_t at = 0, w0 = uni(code32[0]);
+  uint32_t at = ea.first, w0 = uni(code32[2 * at]);
   bool has_bias = false;
   uint64_t b_addr = 0, b_boff = 0, s_addr, s_boff;
   uint32_t b_dtype = 0, b_sn = 0, b_sm = 0, s_dtype, s_sn, s_sm, rnd = VRND_NONE;
@@ -1027,9 +1048,7 @@ __device__ __attribute__((noinline)) bool epilogue_plain_pass(const float *dump,
       vf4 lo[CH], hi[CH];
 #pragma unroll
       for (int q = 0; q < CH; ++q) {
-        const float *src = dump + ((c0 + q) * ROWS_PER_STEP + r0) * PITCH + g * 8;
-        lo[q] = *reinterpret_cast<const vf4 *>(src);
-        hi[q] = *reinterpret_cast<const vf4 *>(src + 4);
+        dump_read_slab<D16, BN>(dump, (c0 + q) * ROWS_PER_STEP + r0, g, lo[q], hi[q]);
       }
 #pragma unroll
       for (int q = 0; q < CH; ++q) {
@@ -1073,11 +1092,10 @@ __device__ __attribute__((noinline)) bool epilogue_plain_pass(const float *dump,
 
 // Second half of a pass: the half tile sits in local memory, row major with PITCH floats per row;
 // every lane takes slabs of 8 columns and walks the epilogue program over them.
-template <int ROWS, int BN, int TM, int WM, bool SLIM>
-__device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
+template <int ROWS, int BN, int TM, int WM, bool SLIM, int D16>
+__device__ __forceinline__ void epilogue_pass_body(const void *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
                                                         uint32_t pass, uint32_t m, uint32_t n, uint32_t m_lo, uint32_t n_lo) {
   constexpr int NTHR = WM * 2 * 64;
-  constexpr int PITCH = BN + 4;
   constexpr int GROUPS = BN / 8;               // slabs per row
   constexpr int PER_THREAD = ROWS * GROUPS / NTHR;  // slabs per thread
   // four slabs per walk of the program where a wave may use all 512 registers; with two waves per SIMD two slabs
@@ -1106,7 +1124,8 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
       const uint32_t wm = lr / HALF, rr = lr % HALF;
       rows.row[s] = m0 + wm * (TM * 32) + pass * HALF + rr;
       rows.ok |= ((rows.row[s] < m && rows.row[s] >= m_lo) ? 1u : 0u) << s;
-      const vf4 lo = *reinterpret_cast<const vf4 *>(dump + lr * PITCH + g * 8), hi = *reinterpret_cast<const vf4 *>(dump + lr * PITCH + g * 8 + 4);
+      vf4 lo, hi;
+      dump_read_slab<D16, BN>(dump, lr, g, lo, hi);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         acc[s * 8 + e] = lo[e];
@@ -1116,6 +1135,12 @@ __device__ __attribute__((noinline)) void epilogue_pass(const float *dump, const
     if (wave_all(rows.ok == 0u || ncol == 0u)) continue;  // nothing of these slabs is inside the tile's part of the output
     run_epilogue<SL, SLIM>(acc, prog32, ea, rows, col, ncol);
   }
+}
+
+template <int ROWS, int BN, int TM, int WM, bool SLIM, int D16>
+__device__ __attribute__((noinline)) void epilogue_pass(const void *dump, const uint32_t *prog32, EpiArgs ea, uint32_t m0, uint32_t n0,
+                                                        uint32_t pass, uint32_t m, uint32_t n, uint32_t m_lo, uint32_t n_lo) {
+  epilogue_pass_body<ROWS, BN, TM, WM, SLIM, D16>(dump, prog32, ea, m0, n0, pass, m, n, m_lo, n_lo);
 }
 
 // TM x TN 32x32 MFMA tiles per wave, 2 x 2 waves per workgroup; A_KC / B_KC: the operand's k axis is
@@ -1448,7 +1473,64 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       continue;
     }
     // epilogue: accumulators -> local memory (row major), then slabs through the program
-    const EpiArgs ea = {h.mem_off, h.code_off, bi0, bi1, h.epi_flags, h.n_code, 0};
+    if (h.epi_flags & VCF_DUMP16) {
+      // The program starts with [add of a bias row] [rounding to the operand type]: done here, where a lane's column
+      // is fixed (one bias value per fragment column). The rounded values are kept as their 16 bits, so the whole
+      // tile fits local memory and goes through the epilogue in one pass, with no accumulator left alive across it.
+      constexpr int D16K = IS_BF16 ? 1 : 2;
+      constexpr int P16 = BN + 8;
+      const uint32_t *code32 = prog32 + 2 * h.code_off;
+      const uint32_t w_first = uni(code32[0]);
+      uint32_t first = 0;
+      float bias[TN];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) bias[j] = 0.0f;
+      if ((w_first & 0xffu) == VOP_BINF) {
+        first = 1;
+        const uint32_t *d = prog32 + 2 * h.mem_off + (w_first >> 24) * (sizeof(VCubeMem) / 4);
+        const uint64_t addr = static_cast<uint64_t>(uni(d[0])) | (static_cast<uint64_t>(uni(d[1])) << 32);
+        const uint32_t dtype = uni(d[2]);
+        const uint64_t boff = static_cast<uint64_t>(bi0) * uni(d[6]) + static_cast<uint64_t>(bi1) * uni(d[7]);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const uint32_t col = n0 + (wn * TN + j) * 32 + (lane & 31u);
+          const uint64_t at = boff + (col < h.n ? col : 0u);  // (columns past the edge are never stored)
+          bias[j] = dtype == VDT_F32 ? reinterpret_cast<const DVM_GLOBAL float *>(addr)[at]
+                                     : cvt_in(dtype, reinterpret_cast<const DVM_GLOBAL uint16_t *>(addr)[at]);
+        }
+      }
+      // (the rounding is the next instruction, or what the program's one store does anyway)
+      if ((uni(code32[2 * first]) & 0xffu) == VOP_CAST) ++first;
+      const EpiArgs ea = {h.mem_off, h.code_off, bi0, bi1, h.epi_flags, h.n_code, 0, first};
+      uint16_t *tile16 = reinterpret_cast<uint16_t *>(lds_raw);
+#pragma unroll
+      for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+          const vf16 &c = acc[i][j];
+          // lane holds column lane%32, rows 8*(r/4) + 4*(lane/32) + r%4 of the fragment
+          uint16_t *dst = tile16 + (wm * (TM * 32) + i * 32 + (lane >> 5) * 4) * P16 + (wn * TN + j) * 32 + (lane & 31u);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float v = c[r] + bias[j];
+            uint16_t bits;
+            if constexpr (IS_BF16) bits = static_cast<uint16_t>(__float_as_uint(round_bf16(v)) >> 16);
+            else bits = __builtin_bit_cast(uint16_t, static_cast<_Float16>(v));
+            dst[(8 * (r / 4) + (r % 4)) * P16] = bits;
+          }
+        }
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<BM, BN, TM, WM, D16K>(tile16, prog32, ea, m0, n0, 0, h.m, h.n, m_lo, n_lo)) {
+        if (h.epi_flags & VCF_SLIM) {
+          epilogue_pass_body<BM, BN, TM, WM, true, D16K>(tile16, prog32, ea, m0, n0, 0, h.m, h.n, m_lo, n_lo);
+        }
+        else epilogue_pass<BM, BN, TM, WM, false, D16K>(tile16, prog32, ea, m0, n0, 0, h.m, h.n, m_lo, n_lo);
+      }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      continue;
+    }
+    const EpiArgs ea = {h.mem_off, h.code_off, bi0, bi1, h.epi_flags, h.n_code, 0, 0};
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps) {
       constexpr int FR = TM / PASSES;  // fragment rows of a wave per pass
@@ -1467,9 +1549,9 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       // before the next dump): they wait for this wave's local-memory operations and not, as __syncthreads() would,
       // for its stores to memory as well, which stay in flight under the next pass and the next tile's loop.
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<PROWS, BN, TM, WM>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo)) {
-        if (h.epi_flags & VCF_SLIM) epilogue_pass<PROWS, BN, TM, WM, true>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
-        else epilogue_pass<PROWS, BN, TM, WM, false>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
+      if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<PROWS, BN, TM, WM, 0>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo)) {
+        if (h.epi_flags & VCF_SLIM) epilogue_pass<PROWS, BN, TM, WM, true, 0>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
+        else epilogue_pass<PROWS, BN, TM, WM, false, 0>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
       }
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }

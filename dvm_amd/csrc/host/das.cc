@@ -224,6 +224,7 @@ std::string &VKernel::DisAssemble() {
          << " lds=" << p.lds_bytes << (c->fast ? " fast" : " guarded") << (c->tile == 3 ? " eight-waves" : "");
       if (c->epi_flags & VCF_PLAIN_STORE) os << " plain-store";
       else if (c->epi_flags & VCF_SLIM) os << " slim-epilogue";
+      if (c->epi_flags & VCF_DUMP16) os << " tile-as-16-bit";
       if (c->epi_flags & VCF_SPLITK_PARTIAL) os << " split-k partials " << c->k_split << " x " << c->k_chunk;
       if (c->epi_flags & VCF_SPLITK_COMBINE) os << " split-k sum of " << c->k_split;
       os << "\n";

@@ -407,6 +407,24 @@ void Compiler::CompileCube(int a) {
     if (i < code_.size() && VI_OP(code_[i]) == VOP_CAST && VI_SUB(code_[i]) == VC_RND) ++i;
     if (i + 2 == code_.size() && VI_OP(code_[i]) == VOP_ST && VI_OP(code_[i + 1]) == VOP_END && k_->tuning_.cube_exact != 2) h.epi_flags |= VCF_PLAIN_STORE;
   }
+  {  // [Add of a bias row] cast.round to the operand type in front: the kernel does them where the accumulators are
+    size_t i = 0;
+    bool ok = k_->tuning_.cube_dump16 != 0;
+    if (i < code_.size() && VI_OP(code_[i]) == VOP_BINF) {
+      const uint64_t w = code_[i];
+      ok = ok && VI_SUB(w) == VB_ADD && VI_KIND(w) == VK_MEM && VI_RND(w) == 0 && VI_A(w) < static_cast<uint32_t>(n_mem_);
+      if (ok) {
+        const VCubeMem &b = cmems_[VI_A(w)];
+        ok = b.stride_n == 1 && b.stride_m == 0 && (b.dtype == VDT_F32 || b.dtype == VDT_F16 || b.dtype == VDT_BF16);
+      }
+      ++i;
+    }
+    // (the rounding is an instruction, or what the one store of the program does: it writes the operand type)
+    const bool rounds = i < code_.size() && VI_OP(code_[i]) == VOP_CAST && VI_SUB(code_[i]) == VC_RND && VI_RND(code_[i]) == RndOf(mm->type_id_);
+    const bool store_rounds = i + 2 == code_.size() && VI_OP(code_[i]) == VOP_ST && VI_OP(code_[i + 1]) == VOP_END &&
+                              VI_A(code_[i]) < static_cast<uint32_t>(n_mem_) && cmems_[VI_A(code_[i])].dtype == MemDType(mm->type_id_);
+    if (ok && (rounds || store_rounds)) h.epi_flags |= VCF_DUMP16;
+  }
   h.n_mem = n_mem_;
   h.n_code = static_cast<uint32_t>(code_.size());
   h.mem_off = sizeof(VCubeHeader) / 8;

@@ -31,6 +31,7 @@ void Tuning::Read() {
   cube_tile = num("DVM_CUBE_TILE");
   cube_waves = num("DVM_CUBE_WAVES");
   cube_exact = num("DVM_CUBE_EXACT");
+  cube_dump16 = num("DVM_CUBE_DUMP16");
   cube_splitk = num("DVM_CUBE_SPLITK");
   red_split = num("DVM_RED_SPLIT");
   red_split_turn = num("DVM_RED_SPLIT_TURN");

@@ -303,16 +303,26 @@ typedef struct {
 // through a build of the interpreter's pass without the arms of everything else, which needs half the registers
 // (what calling the pass costs is the registers it saves).
 #define VCF_SLIM 16u
+// The program starts with [add of a bias row: one value per column, the same for every row] [rounding to the
+// operand type] (or, in place of the rounding, consists of nothing but one store of the operand type behind the
+// add), which is what every product's program starts with unless its bias walks memory some other way.
+// The kernel then does these two in the layout the accumulators have (a lane's column is fixed there: one bias value
+// per fragment), hands the epilogue the whole tile as 16-bit values in one pass, and the interpreter starts behind
+// them. (As fp32 only half a 256 x 256 tile fits local memory, and the second half's accumulators stayed live across
+// the first half's pass: registers saved to scratch memory around the call.)
+#define VCF_DUMP16 32u
 #define VCF_SPLITK_PARTIAL 2u
 #define VCF_SPLITK_COMBINE 4u
 
 // Dynamic local memory a VE_CUBE launch needs for block tile `bt` (256, 128 or 64): the operand tiles of the k
-// loop (two buffers of 64 k per operand; for the 256 tile the same bytes as four stage buffers of 32 k), or the
-// half tile of fp32 accumulators the epilogue reads back.
+// loop (two buffers of 64 k per operand; for the 256 tile the same bytes as four stage buffers of 32 k), or what
+// the epilogue reads back: half the tile as fp32 accumulators, or the whole tile as 16-bit values (VCF_DUMP16).
+#define DVM_CUBE_LDS_LOOP_BYTES(bt) (2u * (2u * (bt)) * 64u * 2u)
+#define DVM_CUBE_LDS_DUMP32_BYTES(bt) (((bt) >= 128u ? (bt) / 2u : (bt)) * ((bt) + 4u) * 4u)
+#define DVM_CUBE_LDS_DUMP16_BYTES(bt) ((bt) * ((bt) + 8u) * 2u)
+#define DVM_CUBE_MAX2(a, b) ((a) > (b) ? (a) : (b))
 #define DVM_CUBE_LDS_BYTES(bt) \
-  ((2u * (2u * (bt)) * 64u * 2u) > (((bt) >= 128u ? (bt) / 2u : (bt)) * ((bt) + 4u) * 4u) \
-       ? (2u * (2u * (bt)) * 64u * 2u) \
-       : (((bt) >= 128u ? (bt) / 2u : (bt)) * ((bt) + 4u) * 4u))
+  DVM_CUBE_MAX2(DVM_CUBE_LDS_LOOP_BYTES(bt), DVM_CUBE_MAX2(DVM_CUBE_LDS_DUMP32_BYTES(bt), DVM_CUBE_LDS_DUMP16_BYTES(bt)))
 
 // ---- fused attention programs (VE_ATTN) -------------------------------------------
 // O[b] = softmax(Q[b] K[b]^T * scale) V[b] for nb independent (batch, head) pairs, all operands row
