@@ -151,8 +151,8 @@ DataType.float32 = DataType(3)
 DataType.int32 = DataType(4)
 DataType.int64 = DataType(5)
 
-_NP_OF = {0: np.bool_, 1: np.float16, 2: np.uint16, 3: np.float32, 4: np.int32}
-_ITEMSIZE = {0: 1, 1: 2, 2: 2, 3: 4, 4: 4}
+_NP_OF = {0: np.bool_, 1: np.float16, 2: np.uint16, 3: np.float32, 4: np.int32, 5: np.int64}
+_ITEMSIZE = {0: 1, 1: 2, 2: 2, 3: 4, 4: 4, 5: 8}
 
 
 def _i64(seq):

@@ -195,13 +195,16 @@ NDObject *BinaryDispatch(Kernel &k, const dvm_operand *l, const dvm_operand *r) 
     switch (r->kind) {
       case 0: return k.Binary<kOp>(lhs, Obj(r->obj));
       case 1: return k.Binary<kOp>(lhs, static_cast<float>(r->f));
-      case 2: return k.Binary<kOp>(lhs, static_cast<int32_t>(r->i));
+      case 2:  // (an integer that does not fit 32 bits travels as int64: it only means something to an int64 tensor)
+        if (r->i != static_cast<int32_t>(r->i)) return k.Binary<kOp>(lhs, static_cast<int64_t>(r->i));
+        return k.Binary<kOp>(lhs, static_cast<int32_t>(r->i));
       case 3: return k.Binary<kOp>(lhs, &r->ref->ref);
       default: break;
     }
   } else if (l->kind == 1) {
     return with_rhs(static_cast<float>(l->f));
   } else if (l->kind == 2) {
+    if (l->i != static_cast<int32_t>(l->i)) return with_rhs(static_cast<int64_t>(l->i));
     return with_rhs(static_cast<int32_t>(l->i));
   } else if (l->kind == 3) {
     return with_rhs(&l->ref->ref);
@@ -286,6 +289,8 @@ dvm_scalar *dvm_rt_new_scalar(dvm_rt *rt, int dtype) {
         dvm_scalar *s = rt->scalars.back().get();
         if (dtype == kInt32) {
           s->ref = 0;
+        } else if (dtype == kInt64) {
+          s->ref = static_cast<int64_t>(0);
         } else {
           s->ref = 0.0f;
         }
@@ -297,6 +302,8 @@ dvm_scalar *dvm_rt_new_scalar(dvm_rt *rt, int dtype) {
 int dvm_scalar_update_f(dvm_scalar *s, double v) {
   if (s->ref.type == kInt32) {
     s->ref = static_cast<int32_t>(v);
+  } else if (s->ref.type == kInt64) {
+    s->ref = static_cast<int64_t>(v);
   } else {
     s->ref = static_cast<float>(v);
   }
@@ -306,6 +313,8 @@ int dvm_scalar_update_f(dvm_scalar *s, double v) {
 int dvm_scalar_update_i(dvm_scalar *s, int64_t v) {
   if (s->ref.type == kInt32) {
     s->ref = static_cast<int32_t>(v);
+  } else if (s->ref.type == kInt64) {
+    s->ref = v;
   } else {
     s->ref = static_cast<float>(v);
   }
@@ -388,7 +397,9 @@ dvm_obj *dvm_rt_full(dvm_rt *rt, const dvm_operand *value, dvm_shape *shape, int
         const DataType t = static_cast<DataType>(dtype);
         switch (value->kind) {
           case 1: return Handle(rt->kernel.Broadcast(static_cast<float>(value->f), &shape->ref, t));
-          case 2: return Handle(rt->kernel.Broadcast(static_cast<int32_t>(value->i), &shape->ref, t));
+          case 2:
+            if (value->i != static_cast<int32_t>(value->i)) return Handle(rt->kernel.Broadcast(static_cast<int64_t>(value->i), &shape->ref, t));
+            return Handle(rt->kernel.Broadcast(static_cast<int32_t>(value->i), &shape->ref, t));
           case 3: return Handle(rt->kernel.Broadcast(&value->ref->ref, &shape->ref, t));
           default: throw std::runtime_error("DVM EXCEPTION. reason: full needs a scalar value");
         }

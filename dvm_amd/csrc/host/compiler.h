@@ -250,7 +250,7 @@ class Compiler {
 
   // A view: reshape of a materialised value (or of a load) that is read through its new shape.
   bool IsView(const NDObject *o) const {
-    return (o->kind == kObjReshape && !IsSqueezeReshape(o)) || o->kind == kObjPermute || o->kind == kObjSlice;
+    return (o->kind == kObjReshape && !IsSqueezeReshape(o)) || o->kind == kObjPermute || o->kind == kObjSlice || o->kind == kObjHalf64;
   }
 
   // The operator whose buffer a view chain ends at.

@@ -87,6 +87,8 @@ std::string &VKernel::DumpGraph(bool ref_shapes) {
       case kObjConcat: os << "Concat"; break;
       case kObjCopy: os << "Copy"; break;
       case kObjMatMul: os << "MatMul" << (o->trans_a ? "T" : "N") << (o->trans_b ? "T" : "N"); break;
+      case kObjPack64: os << "Pack"; break;
+      case kObjHalf64: os << (o->op == 0 ? "ExtractLo" : "ExtractHi"); break;
     }
     os << "." << DTypeName(o->type_id_) << "(";
     for (int i = 0; i < o->nin; ++i) {

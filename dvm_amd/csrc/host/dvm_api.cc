@@ -106,7 +106,17 @@ uint32_t FloatBits(float f) {
 
 }  // namespace
 
-uint32_t ScalarToContainer(const ScalarRef &s, DataType t) {
+uint32_t ScalarToContainer(const ScalarRef &s, DataType t, int half64) {
+  if (half64 != 0) {  // one 32-bit word of an int64 scalar (whatever type it arrived as, converted like a C cast)
+    int64_t v;
+    switch (s.type) {
+      case kInt64: v = s.i64; break;
+      case kInt32: v = s.i32; break;
+      default: v = static_cast<int64_t>(ScalarAsFloat(s)); break;
+    }
+    const uint64_t u = static_cast<uint64_t>(v);
+    return static_cast<uint32_t>(half64 == 1 ? u : u >> 32);
+  }
   switch (t) {
     case kFloat16: {
       if (s.type == kFloat16) return FloatBits(F16BitsToF32(s.f16));
@@ -231,9 +241,120 @@ class Builder {
     return false;
   }
 
+  // ---- int64 tensors: pairs of int32 tensors (the reference's lowering, src/dvm.cc:478-760) ----
+  // The 32-bit words of an int64 value: part 0 the low words, 1 the high words.
+  NDObject *Half(NDObject *x, int part) {
+    if (x->kind == kObjLoad && x->bound != nullptr) x = x->bound;
+    if (x->kind == kObjStore) x = x->in[part];  // (a Store handed on as an operand stands for the value it stores)
+    if (x->type_id_ == kInt32) return x;        // (the word itself: the store case above)
+    if (x->kind == kObjPack64) return x->in[part];
+    if (x->kind != kObjLoad) Throw("an int64 operand that is neither a Load nor the result of an int64 operator");
+    for (auto it = k_->ops_.rbegin(); it != k_->ops_.rend(); ++it)  // one view per load and word, however often it is used
+      if ((*it)->kind == kObjHalf64 && (*it)->in[0] == x && (*it)->op == part && (*it)->stage == k_->Stage()) return *it;
+    NDObject *o = new NDObject(kObjHalf64, kInt32);
+    o->in[0] = x;
+    o->nin = 1;
+    o->op = static_cast<uint8_t>(part);
+    return k_->Append(o);
+  }
+  NDObject *Pack(NDObject *lo, NDObject *hi) { return New(kObjPack64, kInt64, lo, hi); }
+  static ScalarOperand Imm32(int32_t v) {
+    ScalarOperand s;
+    s.imm = v;
+    return s;
+  }
+  // (x <u y) on the bit patterns of two int32 tensors, as int32 0 / 1: both are moved by 2^31 first
+  NDObject *UnsignedLess32(NDObject *x, NDObject *y) {
+    NDObject *xb = NewBinaryS(kAdd, x, Imm32(INT32_MIN), false), *yb = NewBinaryS(kAdd, y, Imm32(INT32_MIN), false);
+    return NoLossCast(TensorBinary(kLess, xb, yb), kInt32);
+  }
+  NDObject *Add64(NDObject *l, NDObject *r) {  // src/dvm.cc:678-689
+    NDObject *llo = Half(l, 0), *rlo = Half(r, 0), *lhi = Half(l, 1), *rhi = Half(r, 1);
+    NDObject *lo = TensorBinary(kAdd, llo, rlo);
+    NDObject *carry = UnsignedLess32(lo, llo);
+    return Pack(lo, TensorBinary(kAdd, TensorBinary(kAdd, lhi, rhi), carry));
+  }
+  NDObject *Sub64(NDObject *l, NDObject *r) {  // src/dvm.cc:691-702
+    NDObject *llo = Half(l, 0), *rlo = Half(r, 0), *lhi = Half(l, 1), *rhi = Half(r, 1);
+    NDObject *lo = TensorBinary(kSub, llo, rlo);
+    NDObject *borrow = UnsignedLess32(llo, rlo);
+    return Pack(lo, TensorBinary(kSub, TensorBinary(kSub, lhi, rhi), borrow));
+  }
+  NDObject *Compare64(int op, NDObject *l, NDObject *r) {  // src/dvm.cc:717-760
+    NDObject *llo = Half(l, 0), *rlo = Half(r, 0), *lhi = Half(l, 1), *rhi = Half(r, 1);
+    if (op == kEqual) return TensorBinary(kLogicalAnd, TensorBinary(kEqual, lhi, rhi), TensorBinary(kEqual, llo, rlo));
+    if (op == kNotEqual) return TensorBinary(kLogicalOr, TensorBinary(kNotEqual, lhi, rhi), TensorBinary(kNotEqual, llo, rlo));
+    // the high words decide, as signed numbers; where they are equal, the low words, as unsigned ones
+    NDObject *lb = NewBinaryS(kAdd, llo, Imm32(INT32_MIN), false), *rb = NewBinaryS(kAdd, rlo, Imm32(INT32_MIN), false);
+    NDObject *hi_cmp = NoLossCast(TensorBinary(op, lhi, rhi), kInt32);
+    NDObject *hi_eq = NoLossCast(TensorBinary(kEqual, lhi, rhi), kInt32);
+    NDObject *lo_cmp = NoLossCast(TensorBinary(op, lb, rb), kInt32);
+    return NoLossCast(New(kObjSelect, kInt32, hi_eq, lo_cmp, hi_cmp), kBool);
+  }
+  // An int64 scalar as a tensor of the given shape (its two words as int32 fills; a ScalarRef is read again at
+  // every code generation).
+  NDObject *Fill64(const ScalarOperand &s, IntArrayRef *shape) {
+    NDObject *w[2];
+    for (int part = 0; part < 2; ++part) {
+      w[part] = New(kObjBroadcastS, kInt32);
+      w[part]->scalar = s;
+      w[part]->aux_ref = shape;
+      w[part]->half64 = static_cast<uint8_t>(part + 1);
+    }
+    return Pack(w[0], w[1]);
+  }
+  NDObject *ToInt64(NDObject *x) {
+    if (x->type_id_ == kInt32) {  // sign extension: the high word is 0 - (x < 0)
+      NDObject *neg = NoLossCast(ScalarBinary(kLess, Imm32(0), x, true), kInt32);
+      return Pack(x, NewBinaryS(kAdd, NewBinaryS(kMul, neg, Imm32(-1), false), Imm32(0), false));
+    }
+    if (x->type_id_ != kFloat32) return ToInt64(Cast(x, x->type_id_ == kBool ? kInt32 : kFloat32));
+    // fp32 -> int64 truncates toward zero (a C cast; magnitudes of 2^63 and above, infinities and NaN are undefined
+    // there as well). |x| is split into its part above 2^32 and the rest, both exact in fp32; the low word goes
+    // through the int32 conversion; a negative x negates the pair.
+    ScalarOperand two32, inv32, two31, zero;
+    two32.imm = 4294967296.0f;
+    inv32.imm = 1.0f / 4294967296.0f;
+    two31.imm = -2147483648.0f;
+    zero.imm = 0.0f;
+    NDObject *a = Unary(kAbs, Unary(kTrunc, x));
+    NDObject *hi_f = Unary(kFloor, NewBinaryS(kMul, a, inv32, false));
+    NDObject *lo_f = TensorBinary(kSub, a, NewBinaryS(kMul, hi_f, two32, false));
+    // (the low part, in [0, 2^32), to its 32-bit pattern: below 2^31 the int32 conversion itself; from 2^31 on the
+    // conversion of the value less 2^31, an exact subtraction there, moved back by an integer add)
+    ScalarOperand pos31;
+    pos31.imm = 2147483648.0f;
+    NDObject *top = NoLossCast(ScalarBinary(kGreaterEqual, pos31, lo_f, true), kInt32);
+    NDObject *lo_top = NewBinaryS(kAdd, Cast(NewBinaryS(kAdd, lo_f, two31, false), kInt32), Imm32(INT32_MIN), false);
+    NDObject *lo = New(kObjSelect, kInt32, top, lo_top, Cast(lo_f, kInt32));
+    NDObject *hi = Cast(hi_f, kInt32);
+    // -(hi:lo) = (0 - lo) : (0 - hi - (lo != 0))
+    NDObject *nlo = NewBinaryS(kAdd, NewBinaryS(kMul, lo, Imm32(-1), false), Imm32(0), false);
+    NDObject *lo_nz = NoLossCast(ScalarBinary(kNotEqual, Imm32(0), lo, true), kInt32);
+    NDObject *nhi = TensorBinary(kSub, NewBinaryS(kMul, hi, Imm32(-1), false), lo_nz);
+    NDObject *is_neg = NoLossCast(ScalarBinary(kLess, zero, x, true), kInt32);
+    return Pack(New(kObjSelect, kInt32, is_neg, nlo, lo), New(kObjSelect, kInt32, is_neg, nhi, hi));
+  }
+  NDObject *FromInt64(NDObject *x, DataType t) {
+    NDObject *lo = Half(x, 0), *hi = Half(x, 1);
+    if (t == kInt32) return lo;  // the low word: what a C cast keeps
+    if (t == kBool) return TensorBinary(kLogicalOr, ScalarBinary(kNotEqual, Imm32(0), hi, true), ScalarBinary(kNotEqual, Imm32(0), lo, true));
+    // to a float type, in fp32: the value is (high + [low < 0]) * 2^32 + low with the low word read as a signed
+    // number, so that small magnitudes of either sign have a zero first term and come out exact; beyond 24
+    // significant bits the two roundings of the sum can differ from one rounding of the value by a unit in the last
+    // place.
+    ScalarOperand two32;
+    two32.imm = 4294967296.0f;
+    NDObject *neg = Cast(NoLossCast(ScalarBinary(kLess, Imm32(0), lo, true), kInt32), kFloat32);
+    NDObject *hi_f = TensorBinary(kAdd, Cast(hi, kFloat32), neg);
+    NDObject *f = TensorBinary(kAdd, NewBinaryS(kMul, hi_f, two32, false), Cast(lo, kFloat32));
+    return Cast(f, t);
+  }
+
   NDObject *Cast(NDObject *x, DataType t) {
     if (x->type_id_ == t) return x;
-    if (t == kInt64 || x->type_id_ == kInt64) Unsupported("int64 tensors");
+    if (t == kInt64) return ToInt64(x);
+    if (x->type_id_ == kInt64) return FromInt64(x, t);
     if (t == kBool && !IsBoolResult(x)) {
       ScalarOperand zero;
       zero.imm = 0;
@@ -250,7 +371,7 @@ class Builder {
 
   NDObject *BroadcastScalar(const ScalarOperand &s, IntArrayRef *shape, DataType t) {
     if (t == kBool) return Cast(BroadcastScalar(s, shape, kFloat16), kBool);
-    if (t == kInt64) Unsupported("int64 tensors");
+    if (t == kInt64) return Fill64(s, shape);
     NDObject *o = New(kObjBroadcastS, t);
     o->scalar = s;
     o->aux_ref = shape;
@@ -269,7 +390,7 @@ class Builder {
         if (op >= kRound && op <= kTrunc) return Cast(Unary(op, Cast(x, kFloat32)), kFloat16);
         break;
       case kInt64:
-        Unsupported("int64 tensors");
+        Unsupported("a unary operator on int64 tensors");
       default:
         break;
     }
@@ -304,7 +425,11 @@ class Builder {
         if (op == kPow) return Cast(TensorBinary(op, Cast(l, kFloat32), Cast(r, kFloat32)), kFloat16);
         break;
       case kInt64:
-        Unsupported("int64 tensors");
+        if (r->type_id_ != kInt64) Throw("int64 operator with an operand of another type");
+        if (IsCompare(op)) return Compare64(op, l, r);
+        if (op == kAdd) return Add64(l, r);
+        if (op == kSub) return Sub64(l, r);
+        Unsupported("this binary operator on int64 tensors");  // (the reference has add, sub and the compares: src/dvm.cc:1351-1364)
       default:
         break;
     }
@@ -352,7 +477,10 @@ class Builder {
   // Tensor (op) scalar when the operation has a scalar form; null otherwise.
   // rhs_val: the scalar is the right operand.
   NDObject *ScalarBinary(int op, const ScalarOperand &s, NDObject *x, bool rhs_val) {
-    if (x->type_id_ == kInt64) Unsupported("int64 tensors");
+    if (x->type_id_ == kInt64) {  // the scalar as a tensor of its two words, then the tensor form
+      NDObject *b = Fill64(s, x->shape_ref_);
+      return rhs_val ? TensorBinary(op, x, b) : TensorBinary(op, b, x);
+    }
     const bool is_ref = s.ref != nullptr;
     switch (op) {
       case kAdd:
@@ -497,6 +625,11 @@ void Kernel::Clone(const Kernel &base, CloneHelper &helper) {
     c->temp = o->temp;
     c->bound = o->bound != nullptr ? helper.GetClone(o->bound) : nullptr;
     c->noloss_cast = o->noloss_cast;
+    c->half64 = o->half64;
+    if (o->hi_view != nullptr) {
+      c->hi_view = new NDObject(kObjStore, kInt32);
+      c->hi_view->strided = true;
+    }
     c->nin = o->nin;
     for (int i = 0; i < o->nin; ++i) c->in[i] = helper.GetClone(o->in[i]);
     c->scalar.imm = o->scalar.imm;
@@ -533,7 +666,6 @@ void Kernel::SetNameHint(const char *name, const char *fullname) {
 }
 
 NDObject *Kernel::Load(void *addr, IntArrayRef *shape, DataType type) {
-  if (type == kInt64) Unsupported("int64 tensors");
   NDObject *o = new NDObject(kObjLoad, type);
   o->addr = addr;
   o->aux_ref = shape;
@@ -578,6 +710,18 @@ NDObject *Kernel::MultiLoad(void *, IntArrayRef *, DataType, const Comm *) { Uns
 
 NDObject *Kernel::Store(void *addr, NDObject *input) {
   Builder b(kernel_);
+  if (input->type_id_ == kInt64) {
+    // the two words of every element are stored through strides into one buffer (kObjStore with two inputs)
+    NDObject *lo = b.Half(input, 0), *hi = b.Half(input, 1);
+    if (lo->kind == kObjHalf64) lo = b.New(kObjCopy, kInt32, lo);
+    if (hi->kind == kObjHalf64) hi = b.New(kObjCopy, kInt32, hi);
+    NDObject *o = b.New(kObjStore, kInt64, lo, hi);
+    o->addr = addr;
+    o->strided = true;  // (nothing reads a value back from this buffer as if it were dense)
+    o->hi_view = new NDObject(kObjStore, kInt32);
+    o->hi_view->strided = true;
+    return o;
+  }
   if (input->IsLoad()) input = b.New(kObjCopy, input->type_id_, input);
   NDObject *o = b.New(kObjStore, input->type_id_, input);
   o->addr = addr;
@@ -586,7 +730,9 @@ NDObject *Kernel::Store(void *addr, NDObject *input) {
 
 NDObject *Kernel::Store(void *addr, NDObject *input, IntArrayRef *stride) {
   NDObject *o = Store(addr, input);
-  if (stride != nullptr) {
+  if (stride != nullptr && o->type_id_ == kInt64) {
+    o->stride_ref = stride;  // (in int64 elements; Normalize doubles them)
+  } else if (stride != nullptr) {
     o->strided = true;
     o->stride_ref = stride;
   }
@@ -680,7 +826,11 @@ NDObject *Kernel::_Reduce(int op_type, NDObject *input, IntArrayRef *dims, bool 
 
 NDObject *Kernel::Select(NDObject *cond, NDObject *lhs, NDObject *rhs) {
   Builder b(kernel_);
-  if (lhs->type_id_ == kInt64) Unsupported("int64 tensors");
+  if (lhs->type_id_ == kInt64) {  // word by word (src/dvm.cc:704-715)
+    if (rhs->type_id_ != kInt64) Throw("select between an int64 tensor and one of another type");
+    NDObject *c = b.NoLossCast(cond, kInt32);
+    return b.Pack(b.New(kObjSelect, kInt32, c, b.Half(lhs, 0), b.Half(rhs, 0)), b.New(kObjSelect, kInt32, c, b.Half(lhs, 1), b.Half(rhs, 1)));
+  }
   if (cond->type_id_ != lhs->type_id_) cond = b.NoLossCast(cond, lhs->type_id_);
   return b.New(kObjSelect, lhs->type_id_, cond, lhs, rhs);
 }
@@ -693,6 +843,7 @@ NDObject *Kernel::Broadcast(NDObject *input, IntArrayRef *shape) {
     NDObject *r = Broadcast(b.NoLossCast(input, kFloat16), shape);
     return b.NoLossCast(r, kBool);
   }
+  if (input->type_id_ == kInt64) return b.Pack(Broadcast(b.Half(input, 0), shape), Broadcast(b.Half(input, 1), shape));
   NDObject *o = b.New(kObjBroadcast, input->type_id_, input);
   o->aux_ref = shape;
   return o;
@@ -710,12 +861,20 @@ template NDObject *Kernel::Broadcast<BFloat16>(BFloat16, IntArrayRef *, DataType
 template NDObject *Kernel::Broadcast<ScalarRef *>(ScalarRef *, IntArrayRef *, DataType);
 
 NDObject *Kernel::Reshape(NDObject *input, IntArrayRef *shape) {
+  if (input->type_id_ == kInt64) {
+    Builder b(kernel_);
+    return b.Pack(Reshape(b.Half(input, 0), shape), Reshape(b.Half(input, 1), shape));
+  }
   NDObject *o = Builder(kernel_).New(kObjReshape, input->type_id_, input);
   o->aux_ref = shape;
   return o;
 }
 
-NDObject *Kernel::Copy(NDObject *input) { return Builder(kernel_).New(kObjCopy, input->type_id_, input); }
+NDObject *Kernel::Copy(NDObject *input) {
+  Builder b(kernel_);
+  if (input->type_id_ == kInt64) return b.Pack(Copy(b.Half(input, 0)), Copy(b.Half(input, 1)));
+  return b.New(kObjCopy, input->type_id_, input);
+}
 
 NDObject *Kernel::MatMul(NDObject *lhs, NDObject *rhs, bool trans_a, bool trans_b, NDObject *bias) {
   if (lhs->type_id_ != rhs->type_id_ || (lhs->type_id_ != kFloat16 && lhs->type_id_ != kBFloat16)) {
@@ -730,17 +889,29 @@ NDObject *Kernel::MatMul(NDObject *lhs, NDObject *rhs, bool trans_a, bool trans_
 // Permute, Slice and Split are views: the input is kept (or written) in memory in its own layout and the
 // consumers read it through the view's strides and offset; nothing is copied.
 NDObject *Kernel::Permute(NDObject *input, IntArrayRef *dims) {
+  if (input->type_id_ == kInt64) {
+    Builder b(kernel_);
+    return b.Pack(Permute(b.Half(input, 0), dims), Permute(b.Half(input, 1), dims));
+  }
   NDObject *o = Builder(kernel_).New(kObjPermute, input->type_id_, input);
   o->aux_ref = dims;
   return o;
 }
 NDObject *Kernel::Slice(NDObject *input, IntArrayRef *start, IntArrayRef *size) {
+  if (input->type_id_ == kInt64) {
+    Builder b(kernel_);
+    return b.Pack(Slice(b.Half(input, 0), start, size), Slice(b.Half(input, 1), start, size));
+  }
   NDObject *o = Builder(kernel_).New(kObjSlice, input->type_id_, input);
   o->slice_start = start;
   o->aux_ref = size;
   return o;
 }
 NDObject *Kernel::Slice(NDObject *input, int dim, ScalarRef *begin, ScalarRef *end) {
+  if (input->type_id_ == kInt64) {
+    Builder b(kernel_);
+    return b.Pack(Slice(b.Half(input, 0), dim, begin, end), Slice(b.Half(input, 1), dim, begin, end));
+  }
   NDObject *o = Builder(kernel_).New(kObjSlice, input->type_id_, input);
   o->slice_dim = dim;
   o->dim_begin_ref = begin;
@@ -752,6 +923,15 @@ NDObject *Kernel::Slice(NDObject *input, int dim, ScalarRef *begin, ScalarRef *e
 NDObject *Kernel::Concat(NDObject **inputs, size_t input_num, int dim) {
   if (input_num == 0) Throw("concat needs at least one input");
   Builder b(kernel_);
+  if (inputs[0]->type_id_ == kInt64) {  // word by word
+    std::vector<NDObject *> lo, hi;
+    for (size_t i = 0; i < input_num; ++i) {
+      if (inputs[i]->type_id_ != kInt64) Throw("concat inputs differ in type");
+      lo.push_back(b.Half(inputs[i], 0));
+      hi.push_back(b.Half(inputs[i], 1));
+    }
+    return b.Pack(Concat(lo.data(), input_num, dim), Concat(hi.data(), input_num, dim));
+  }
   std::vector<NDObject *> parts;
   for (size_t i = 0; i < input_num; ++i) {
     if (inputs[i]->type_id_ != inputs[0]->type_id_) Throw("concat inputs differ in type");

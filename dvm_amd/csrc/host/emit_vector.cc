@@ -212,7 +212,7 @@ void Compiler::EmitOperandInsn(uint32_t op, uint32_t sub, uint32_t rnd, int v) {
   } else if (n.kind == AK_MEM) {
     Emit(op, sub, VK_MEM, rnd, MemIndex(v), 0);
   } else if (n.kind == AK_SCALAR) {
-    Emit(op, sub, VK_IMM, rnd, 0, ScalarToContainer(n.op->scalar.Get(), n.dtype));
+    Emit(op, sub, VK_IMM, rnd, 0, ScalarToContainer(n.op->scalar.Get(), n.dtype, n.op->half64));
   } else {
     Fail("operand is not addressable");
   }
@@ -295,7 +295,7 @@ void Compiler::ComputeInto(int v) {
       return;
     case AK_SCALAR:
       BeforeOverwrite();
-      Emit(VOP_LDI, 0, 0, 0, 0, ScalarToContainer(o->scalar.Get(), n.dtype));
+      Emit(VOP_LDI, 0, 0, 0, 0, ScalarToContainer(o->scalar.Get(), n.dtype, o->half64));
       return;
     case AK_REDUCE:
       Fail("reduce result used before it is complete");

@@ -42,6 +42,11 @@ enum ObjKind : uint8_t {
   kObjSlice,     // view: a box of the input (slice_start + aux_ref sizes, or one dim with begin / end)
   kObjConcatPart,  // writes its input into its place in the buffer of a Concat (a store through strides)
   kObjConcat,      // the buffer the parts wrote, read by the consumers like any value kept in memory
+  // int64 tensors are pairs of int32 tensors (the reference's lowering, src/dvm.cc:478-760): the low and the high
+  // words of every element. An int64 value the API hands out is a kObjPack64 (in[0] = low words, in[1] = high
+  // words; a handle only, nothing computes it), or a Load of that type, whose words are read through two views:
+  kObjPack64,
+  kObjHalf64,      // view of an int64 Load: every second 32-bit word of its memory (op = 0 low words, 1 high words)
 };
 
 // A scalar operand: an immediate fixed at build time or a ScalarRef re-read at every code generation.
@@ -70,6 +75,9 @@ class NDObject {
   int part_split = 0;           // kObjReduce, during code generation only: the reduce is shared between workgroups, its result
                                 // has one more (outermost) dim that numbers the parts (Compiler::SplitLongReduces)
   bool noloss_cast = false;
+  uint8_t half64 = 0;           // kObjBroadcastS of an int64 scalar as int32 words: 1 = its low word, 2 = its high word
+  NDObject *hi_view = nullptr;  // kObjStore of an int64 value (in[0] low, in[1] high words): where the high words go
+                                // (owned; the Store itself says where the low words go)
   int nin = 0;
   NDObject *in[3] = {nullptr, nullptr, nullptr};
   ScalarOperand scalar;
@@ -181,7 +189,7 @@ float BF16BitsToF32(uint16_t h);
 // type `t`: the value is first converted to `t` exactly like the reference's
 // EncodeScalar (src/dvm.cc:186-223), then widened to the VM's container
 // (fp32 bits for bool/f16/bf16/f32 tensors, two's complement for int32).
-uint32_t ScalarToContainer(const ScalarRef &s, DataType t);
+uint32_t ScalarToContainer(const ScalarRef &s, DataType t, int half64 = 0);
 
 struct DeviceApi;  // bound C ABI of libdvm_hip.so (system.cc)
 class Compiler;    // compiler.h

@@ -12,7 +12,10 @@ namespace dvm {
 
 VKernel::~VKernel() {
   delete compiler_;
-  for (NDObject *o : ops_) delete o;
+  for (NDObject *o : ops_) {
+    delete o->hi_view;
+    delete o;
+  }
 }
 
 void Tuning::Read() {

@@ -83,12 +83,46 @@ void VKernel::Normalize() {
         break;
       case kObjStore:
         o->SetShape(o->in[0]->shape_ref_->data, o->in[0]->shape_ref_->size);
+        if (o->type_id_ == kInt64) {
+          // the low words go to every second 32-bit word of the buffer, the high words (hi_view) to the ones between
+          const size_t r = o->in[0]->shape_ref_->size;
+          if (o->stride_ref != nullptr && o->stride_ref->size != r) Throw("stride list does not match the tensor rank");
+          int64_t dense = 1;
+          for (size_t i = r; i-- > 0;) {
+            o->vstride_[i] = 2 * (o->stride_ref != nullptr ? o->stride_ref->data[i] : dense);
+            dense *= o->shape_[i];
+          }
+          o->view_base_ = 2 * o->view_offset;
+          NDObject *hv = o->hi_view;
+          hv->SetShape(o->shape_, r);
+          for (size_t i = 0; i < r; ++i) hv->vstride_[i] = o->vstride_[i];
+          hv->view_base_ = o->view_base_ + 1;
+          break;
+        }
         if (o->strided) {
           if (o->stride_ref->size != o->in[0]->shape_ref_->size) Throw("stride list does not match the tensor rank");
           for (size_t i = 0; i < o->stride_ref->size; ++i) o->vstride_[i] = o->stride_ref->data[i];
           o->view_base_ = o->view_offset;
         }
         break;
+      case kObjPack64:
+        o->SetShape(o->in[0]->shape_ref_->data, o->in[0]->shape_ref_->size);
+        break;
+      case kObjHalf64: {
+        // the 32-bit words of an int64 Load: its strides (its own when it is a strided load, else those of a dense
+        // tensor) doubled, its offset doubled, plus one for the high words
+        const NDObject *x = o->in[0];
+        const size_t r = x->shape_ref_->size;
+        o->SetShape(x->shape_ref_->data, r);
+        int64_t dense = 1;
+        for (size_t i = r; i-- > 0;) {
+          o->vstride_[i] = 2 * (x->strided ? x->vstride_[i] : dense);
+          dense *= x->shape_ref_->data[i];
+        }
+        o->view_base_ = 2 * (x->strided ? x->view_base_ : 0) + o->op;
+        o->strided = true;
+        break;
+      }
       case kObjUnary:
       case kObjBinaryS:
       case kObjCompareS:

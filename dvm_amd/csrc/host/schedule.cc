@@ -37,7 +37,7 @@ int Compiler::LeafFor(NDObject *v) {
     idx = AddNode(AK_MEM, v, v->type_id_, v->shape_ref_->data, v->rank());
     const NDObject *root = ViewRoot(v);
     // a permuted or sliced value carries the strides of the whole chain down to the root's memory
-    if (v->kind == kObjPermute || v->kind == kObjSlice) nodes_[idx].view = v;
+    if (v->kind == kObjPermute || v->kind == kObjSlice || v->kind == kObjHalf64) nodes_[idx].view = v;
     if (root->kind == kObjLoad) {
       nodes_[idx].addr_op = root->id;
       if (root->strided && nodes_[idx].view == nullptr) {
@@ -109,6 +109,18 @@ void Compiler::BuildNodes(int a) {
       const DataType s = o->in[0]->type_id_, d = o->type_id_;
       const bool nop = (d == kFloat32 && (s == kFloat16 || s == kBFloat16)) || (s == kBool && d != kInt32);
       if (nop) kind = AK_ALIAS;
+    }
+    if (o->kind == kObjStore && o->type_id_ == kInt64) {
+      // an int64 value is two int32 values: each is stored through strides into its own words of the buffer
+      for (int part = 0; part < 2; ++part) {
+        const int out = AddNode(AK_OUT, o, kInt32, o->shape_ref_->data, o->rank());
+        nodes_[out].nin = 1;
+        nodes_[out].in[0] = in_idx[part];
+        nodes_[out].addr_op = i;
+        nodes_[out].view = part == 0 ? o : o->hi_view;
+        if (part == 0) node_of_[i] = out;
+      }
+      continue;
     }
     const int idx = AddNode(kind, o, o->type_id_, o->shape_ref_->data, o->rank());
     ANode &n = nodes_[idx];

@@ -100,7 +100,7 @@ class _DeviceCall:
         self.torch, self.kern, self.args, self.out = torch, kern, args, out
         self.types = {int(DataType.bool): torch.bool, int(DataType.float16): torch.float16,
                       int(DataType.bfloat16): torch.bfloat16, int(DataType.float32): torch.float32,
-                      int(DataType.int32): torch.int32}
+                      int(DataType.int32): torch.int32, int(DataType.int64): torch.int64}
 
     def _bind_inputs(self, in_place):
         """Binds the arguments; `in_place`: tensors that are not contiguous are read through their strides,

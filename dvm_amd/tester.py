@@ -199,7 +199,7 @@ class Tester(PyKernel):
 
     # The reference's graph passes by the names its tests select them with (src/pybind_api.cc:616-650). What each
     # one achieves either always happens here or has no counterpart on an accumulator machine:
-    _ALWAYS_DONE = ("DeadCodeEliminate", "EliminateReshape", "EliminateDiamondView")  # liveness, views read through
+    _ALWAYS_DONE = ("DeadCodeEliminate", "EliminateReshape", "EliminateDiamondView")  # liveness; reshapes are views
     _NO_COUNTERPART = ("PrintPeakLive", "ReorderStore", "ReorderLoad", "CompactPeakLiveness", "VectorDoubleBuffer",
                        "InsertRemovePad", "VfFusion")  # scheduling of tiles in a unified buffer
 
