@@ -638,3 +638,23 @@ def test_sweep_build_is_chosen_from_the_instruction_words(monkeypatch):
     assert "reduce-x" in t.das() and "sweeps" not in t.das(), t.das()
     monkeypatch.setenv("DVM_VEC_SWEEPS", "0")
     assert "reduce-x sweeps" not in _row_norm(Tester("split", run_mode="das"), 8192, 4096)
+
+
+def test_int64_graph_lowers_to_int32_words_without_a_gpu():
+    # an int64 value is its low and high 32-bit words (src/dvm.cc:478-760 of the reference): loads are read through two
+    # strided views of one buffer, operators work on the words, a store writes both through strides; one launch
+    t = Tester("split", run_mode="das")
+    a = np.zeros([13, 131], np.int64)
+    x, y = t.load(a), t.load(a)
+    s = t.add(x, y)
+    t.store(t.select(t.greater(s, 0x123456789), s, t.sub(y, 5)))
+    t.store(t.cast(t.load(np.zeros([13, 131], np.float32)), "int64"))
+    t.codegen()
+    dump, das = t.dump(), t.das()
+    assert "ExtractLo.int32" in dump and "ExtractHi.int32" in dump and "Pack.int64" in dump and "Store.int64" in dump, dump
+    assert t.num_launches() == 2 and "int64" not in das, das          # (one launch per independent graph) the device sees int32 words only
+    assert das.count("gather k[2,262]") + das.count("gather k[2]") >= 4, das   # every second word of the buffers
+    assert "#0x23456789" in das and "#0x00000001" in das, das          # the scalar's two words
+    for refuse in (lambda: t.mul(x, y), lambda: t.abs(x), lambda: t.sum(x, (0,), True)):
+        with pytest.raises(RuntimeError):
+            refuse()
