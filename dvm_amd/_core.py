@@ -86,6 +86,10 @@ def _load():
         "dvm_rt_device_ptr": (vp, [vp, vp]),
         "dvm_rt_perf": (ci, [vp, ci, ci, ctypes.POINTER(ctypes.c_double)]),
         "dvm_rt_perf_samples": (ci, [vp, ci, ci, ctypes.POINTER(ctypes.c_double)]),
+        "dvm_set_online_tuner": (None, [ci]),
+        "dvm_set_lazy_tuner": (None, [ci]),
+        "dvm_tuner_stats": (None, [ctypes.POINTER(ctypes.c_uint64), ctypes.POINTER(ctypes.c_uint64)]),
+        "dvm_tuner_clear": (None, []),
         "dvm_rt_num_launches": (ci, [vp]),
         "dvm_rt_workspace_bytes": (cs, [vp]),
         "dvm_rt_program_count": (ci, [vp]),
@@ -604,13 +608,28 @@ class PyKernel(Kernel):
 
     @staticmethod
     def set_online_tuning(enable):
-        """The reference searches matmul tilings at run time (src/tuner.cc); tile choice here is a closed-form rule
-        of the problem size, so the switch is accepted and changes nothing."""
-        pass
+        """Config::SetOnlineTuner of the reference (include/dvm.h:735): the first code generation of a matmul shape on
+        a machine with a device times every (block tile, parts of the k axis) candidate there and remembers the
+        fastest for the process; without it tile and split come from figures measured once on an MI355X."""
+        _lib.dvm_set_online_tuner(1 if enable else 0)
 
     @staticmethod
     def set_lazy_tuning(enable):
-        pass
+        """Config::SetLazyTuner (include/dvm.h:737). The reference's lazy tuner spreads its trials over the launches
+        of the application; a trial here costs microseconds to compile, so both switches tune at the first code
+        generation of a shape."""
+        _lib.dvm_set_lazy_tuner(1 if enable else 0)
+
+    @staticmethod
+    def tuner_stats():
+        """(product shapes measured so far, entries of the tuner's table)."""
+        a, b = ctypes.c_uint64(0), ctypes.c_uint64(0)
+        _lib.dvm_tuner_stats(ctypes.byref(a), ctypes.byref(b))
+        return int(a.value), int(b.value)
+
+    @staticmethod
+    def tuner_clear():
+        _lib.dvm_tuner_clear()
 
     def tile(self, start, end, num, factor=0):
         """Manual tiling of the reference's tile model (RtKernelPy::Tile, src/pybind_api.cc:1093). The gfx950

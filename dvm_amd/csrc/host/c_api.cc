@@ -11,6 +11,7 @@
 #include <vector>
 
 #include "ir.h"
+#include "compiler.h"
 #include "system.h"
 
 using namespace dvm;
@@ -866,6 +867,19 @@ int dvm_rt_perf(dvm_rt *rt, int warmup, int iters, double out[3]) {
       },
       -1);
 }
+
+void dvm_set_online_tuner(int enable) {
+  g_system.Init();
+  if (enable) g_system.SetOnlineTuner();
+  else g_system.UnsetOnlineTuner();
+}
+void dvm_set_lazy_tuner(int enable) {
+  g_system.Init();
+  if (enable) g_system.SetLazyTuner();
+  else g_system.UnsetLazyTuner();
+}
+void dvm_tuner_stats(uint64_t *shapes_measured, uint64_t *table_size) { CubeTunerStats(shapes_measured, table_size); }
+void dvm_tuner_clear(void) { CubeTunerClear(); }
 
 int dvm_rt_perf_samples(dvm_rt *rt, int warmup, int iters, double *samples) {
   return Guard(

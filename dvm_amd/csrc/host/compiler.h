@@ -144,6 +144,23 @@ inline bool IsSqueezeReshape(const NDObject *o) {
 }
 
 
+// ---------- online tuner of matmul launches (host/tuner.cc) ----------
+struct CubeProblem {
+  int64_t m = 0, n = 0, k = 0, nb0 = 1, nb1 = 1;
+  DataType dtype = kFloat16;
+  bool trans_a = false, trans_b = false;
+};
+struct CubeChoice {
+  int tile = 0;    // 256, 128 or 64; 0: nothing measured
+  int split = 1;   // parts of the k axis (1: one launch)
+  double us = 0.0;
+};
+// The measured choice for a product shape, measuring it first when the shape is new and a tuner is switched on
+// (Config::SetOnlineTuner / SetLazyTuner). False: no tuner, no device, or the shape could not be measured.
+bool CubeTunerLookup(const CubeProblem &q, CubeChoice *out);
+void CubeTunerStats(uint64_t *shapes_measured, uint64_t *table_size);
+void CubeTunerClear();
+
 class Compiler {
  public:
   explicit Compiler(VKernel *k) : k_(k), n_(static_cast<int>(k->ops_.size())) {}

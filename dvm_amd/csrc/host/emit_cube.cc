@@ -194,6 +194,32 @@ void Compiler::CompileCube(int a) {
     prog_->skip = true;
     return;
   }
+  // A measured choice of tile and split for this product shape (the online tuner, host/tuner.cc) stands in for the
+  // two tuning switches for the rest of this function; a switch the user has set wins.
+  struct RestoreTuning {
+    Tuning &t;
+    const int tile, split;
+    ~RestoreTuning() {
+      t.cube_tile = tile;
+      t.cube_splitk = split;
+    }
+  } restore_tuning{k_->tuning_, k_->tuning_.cube_tile, k_->tuning_.cube_splitk};
+  if (!k_->tuning_.in_tuner && k_->tuning_.cube_tile < 0 && k_->tuning_.cube_splitk < 0 && K > 0) {
+    CubeProblem q;
+    q.m = M;
+    q.n = N;
+    q.k = K;
+    q.nb0 = h.nb0;
+    q.nb1 = h.nb1;
+    q.dtype = mm->type_id_;
+    q.trans_a = trans_a;
+    q.trans_b = trans_b;
+    CubeChoice c;
+    if (CubeTunerLookup(q, &c)) {
+      k_->tuning_.cube_tile = c.tile;
+      k_->tuning_.cube_splitk = c.split <= 1 ? 0 : c.split;
+    }
+  }
   // block tile: the largest that still gives most compute units a tile
   const uint64_t batch = static_cast<uint64_t>(h.nb0) * h.nb1;
   auto tiles = [&](int64_t t) { return static_cast<uint64_t>((M + t - 1) / t) * static_cast<uint64_t>((N + t - 1) / t) * batch; };

@@ -214,6 +214,7 @@ struct Tuning {
   int cube_exact = -1;  // DVM_CUBE_EXACT=1: never the hardware approximations of exp, log, sqrt, division in a matmul epilogue
   int attn_waves = -1;  // DVM_ATTN_WAVES=4
   bool debug = false;   // DVM_DEBUG: node dump in compile errors
+  bool in_tuner = false;  // the kernel is a candidate the online tuner is timing: it is not tuned itself
   void Read();
 };
 

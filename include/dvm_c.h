@@ -137,6 +137,14 @@ void *dvm_rt_device_ptr(dvm_rt *rt, dvm_obj *io);
 int dvm_rt_perf(dvm_rt *rt, int warmup, int iters, double out[3]);
 /* The same measurement, every launch's microseconds written to samples[0..iters) (for medians). */
 int dvm_rt_perf_samples(dvm_rt *rt, int warmup, int iters, double *samples);
+/* The matmul tuner (Config::SetOnlineTuner / SetLazyTuner of include/dvm.h; the reference's table of tuned tile
+ * parameters, src/ops_m.h:174-263): with either switched on, the first code generation of a product shape on a
+ * machine with a device times every (block tile, parts of the k axis) candidate there and remembers the fastest for
+ * the process. dvm_tuner_stats: shapes measured so far and entries of the table; dvm_tuner_clear empties the table. */
+void dvm_set_online_tuner(int enable);
+void dvm_set_lazy_tuner(int enable);
+void dvm_tuner_stats(uint64_t *shapes_measured, uint64_t *table_size);
+void dvm_tuner_clear(void);
 /* Number of device launches one run() issues. */
 int dvm_rt_num_launches(const dvm_rt *rt);
 size_t dvm_rt_workspace_bytes(const dvm_rt *rt);
