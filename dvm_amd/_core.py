@@ -63,6 +63,11 @@ def _load():
         "dvm_rt_view_store": (vp, [vp, vp, vp, cs]),
         "dvm_obj_set_view_offset": (ci, [vp, ctypes.c_longlong]),
         "dvm_rt_permute": (vp, [vp, vp, vp]),
+        "dvm_rt_global_access": (vp, [vp, vp, ci]),
+        "dvm_rt_gather_load": (vp, [vp, vp, vp, ci, ci, ci]),
+        "dvm_rt_pad_store": (vp, [vp, vp, ctypes.c_longlong]),
+        "dvm_rt_one_hot": (vp, [vp, vp, vp, ci, ctypes.c_double, ctypes.c_double, ci]),
+        "dvm_rt_element_any": (vp, [vp, vp]),
         "dvm_rt_slice": (vp, [vp, vp, vp, vp]),
         "dvm_rt_slice_dim": (vp, [vp, vp, ci, vp, vp]),
         "dvm_rt_split": (ci, [vp, vp, ci, ctypes.c_longlong, cs, ctypes.POINTER(vp)]),
@@ -224,6 +229,7 @@ class Kernel:
     def __init__(self):
         self._rt = None
         self._keep = []
+        self._pad_of = {}  # pad_store handle -> pad size
 
     # -- references --
     def _shape_ref(self, shape):
@@ -301,6 +307,32 @@ class Kernel:
     def view_store(self, obj, stride, extent):
         """Stores obj through element strides into a zero-initialised buffer of `extent` elements."""
         return self._wrap(_lib.dvm_rt_view_store(self._rt, obj._h, self._shape_ref(stride)._h, int(extent)))
+
+    # -- gathers, one-hot, padded stores (include/dvm_py.h:302-327 of the reference) --
+    def global_access(self, shape, type):
+        """Names a tensor for another operator to read (the int32 index of gather_load); fed like a load."""
+        return self._wrap(_lib.dvm_rt_global_access(self._rt, self._shape_ref(shape)._h, int(type)))
+
+    def gather_load(self, shape, index, type, axis=0, gather_mode=0):
+        """The tensor of `shape` fed to the returned operator, read at `index` along `axis`: gather_mode 0 is NumPy's
+        take_along_axis, 1 its take. Negative indices count from the end; indices past either end are clipped."""
+        return self._wrap(_lib.dvm_rt_gather_load(self._rt, self._shape_ref(shape)._h, index._h, int(type), int(axis), int(gather_mode)))
+
+    def pad_store(self, obj, pad_size):
+        """Stores obj into a buffer whose innermost rows are pad_size elements longer (zeros there); output() gives
+        that whole buffer."""
+        op = self._wrap(_lib.dvm_rt_pad_store(self._rt, obj._h, int(pad_size)))
+        self._pad_of[op._h] = int(pad_size)
+        return op
+
+    def one_hot(self, indices, depth, axis, on_value, off_value, type):
+        """A dim of extent depth at position axis: on_value where the position equals the int32 index, else off_value."""
+        depth_ref = depth if isinstance(depth, IntArrayRef) else self._shape_ref([int(depth)])
+        return self._wrap(_lib.dvm_rt_one_hot(self._rt, indices._h, depth_ref._h, int(axis), float(on_value), float(off_value), int(type)))
+
+    def element_any(self, input):
+        """One fp32 value: the maximum over every element (1 when any element of a 0 / 1 mask is set)."""
+        return self._wrap(_lib.dvm_rt_element_any(self._rt, input._h))
 
     # -- views of values (include/dvm_py.h:163-189 of the reference): nothing is copied --
     def permute(self, input, dims):
@@ -428,6 +460,18 @@ class PyKernel(Kernel):
         self._load_shape[op._h] = ref
         return op
 
+    def global_access(self, shape, type):
+        ref = self._shape_ref(shape)
+        op = Kernel.global_access(self, ref, type)
+        self._load_shape[op._h] = ref
+        return op
+
+    def gather_load(self, shape, index, type, axis=0, gather_mode=0):
+        ref = self._shape_ref(shape)  # the source tensor's shape: input() on the returned operator updates it
+        op = Kernel.gather_load(self, ref, index, type, axis, gather_mode)
+        self._load_shape[op._h] = ref
+        return op
+
     def load_shape(self, load):
         """The updatable shape behind a load (update it and generate code again to change the extent)."""
         return self._load_shape[load._h]
@@ -470,6 +514,7 @@ class PyKernel(Kernel):
     def reset(self):
         _check(_lib.dvm_rt_reset(self._rt))
         self._keep = []
+        self._pad_of = {}
         self._load_shape = {}
         self._inputs = {}
 
@@ -557,6 +602,8 @@ class PyKernel(Kernel):
     def output(self, store, shape=None):
         """The stored tensor; `shape` (strided stores) reads back the whole buffer the store wrote into."""
         shape = store.shape() if shape is None else tuple(shape)
+        if store._h in self._pad_of and len(shape) > 0:
+            shape = tuple(shape[:-1]) + (shape[-1] + self._pad_of[store._h],)
         dt = int(store.dtype())
         out = np.empty(shape, dtype=_NP_OF[dt])
         _check(_lib.dvm_rt_output(self._rt, store._h, out.ctypes.data, out.nbytes))

@@ -219,7 +219,7 @@ static bool sweeps_flag_holds(const VmParam &p) {
   };
   for (uint32_t i = 0; i < h->n_code; ++i) {
     const uint32_t op = VI_OP(code[i]);
-    if (op == VOP_LDR || op == VOP_STR || op == VOP_RED) return false;  // (outside a sweep)
+    if (op == VOP_LDR || op == VOP_STR || op == VOP_RED || op == VOP_LDX) return false;  // (outside a sweep)
     if (op >= VOP_SRC_BASE || op == VOP_ST) {
       if ((op >= VOP_SRC_BASE && VI_KIND(code[i]) == VK_REG) || ((VI_KIND(code[i]) == VK_MEM || op == VOP_ST) && VI_A(code[i]) >= h->n_mem)) return false;
     }
@@ -256,6 +256,14 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
     if (mem_end > DVM_PARAM_WORDS || code_end > DVM_PARAM_WORDS || h->n_code == 0 ||
         VI_OP(p.w[code_end - 1]) != VOP_END || h->n_kdim > DVM_VEC_MAXR || h->n_rdim > DVM_VEC_MAXR) {
       return static_cast<int>(hipErrorInvalidValue);
+    }
+    {
+      // an operand without memory behind it (VDT_IOTA) is read element by element only, and never written
+      const VMemDesc *mems = reinterpret_cast<const VMemDesc *>(p.w + h->mem_off);
+      for (uint32_t i = 0; i < h->n_mem; ++i)
+        if (mems[i].dtype > VDT_IOTA || (mems[i].dtype == VDT_IOTA && (mems[i].flags & VMF_ALIGNED))) return static_cast<int>(hipErrorInvalidValue);
+      for (uint64_t i = h->code_off; i < code_end; ++i)
+        if (VI_OP(p.w[i]) == VOP_ST && (VI_A(p.w[i]) >= h->n_mem || mems[VI_A(p.w[i])].dtype == VDT_IOTA)) return static_cast<int>(hipErrorInvalidValue);
     }
     const bool wide = (h->sched & VS_WIDE) != 0;
     if (wide && threads > 512) return static_cast<int>(hipErrorInvalidValue);

@@ -107,6 +107,8 @@ __device__ __forceinline__ float elem_load(uint64_t base, uint32_t dtype, uint64
       return static_cast<float>(reinterpret_cast<const DVM_GLOBAL _Float16 *>(base)[off]);
     case VDT_BF16:
       return __uint_as_float(static_cast<uint32_t>(reinterpret_cast<const DVM_GLOBAL uint16_t *>(base)[off]) << 16);
+    case VDT_IOTA:  // no memory: the element is its own offset
+      return __int_as_float(static_cast<int32_t>(base + off));
     default:  // VDT_BOOL
       return reinterpret_cast<const DVM_GLOBAL uint8_t *>(base)[off] != 0 ? 1.0f : 0.0f;
   }
@@ -125,6 +127,8 @@ __device__ __forceinline__ void elem_store(uint64_t base, uint32_t dtype, uint64
       break;
     case VDT_BF16:
       reinterpret_cast<DVM_GLOBAL uint16_t *>(base)[off] = static_cast<uint16_t>(f32_to_bf16_bits(v));
+      break;
+    case VDT_IOTA:  // (nothing to write to; the launch refuses such programs)
       break;
     default:
       reinterpret_cast<DVM_GLOBAL uint8_t *>(base)[off] = v != 0.0f ? 1 : 0;
@@ -223,6 +227,27 @@ __device__ __attribute__((noinline)) void mem_store_slow(uint64_t addr, uint32_t
     if (nv == 0) continue;
     slab_store_slow(m, off.v[u], nv, in.v[u]);
   }
+}
+
+// VOP_LDX: element e of a slab comes from the operand's offset for that element plus the lane's own int32 value
+// (an offset in elements the program has computed from an index tensor).
+__device__ __attribute__((noinline)) Acc mem_gather(uint64_t addr, uint32_t dtype, uint32_t flags, Offs off, uint32_t nvp, Acc idx) {
+  addr = uni64(addr);
+  dtype = uni(dtype);
+  flags = uni(flags);
+  const uint64_t step = (flags & VMF_GATHER) ? (flags >> 8) : ((flags & VMF_VEC) ? 1u : 0u);
+  Acc out;
+  FOR_U {
+    const int nv = static_cast<int>((nvp >> (4 * u)) & 0xfu);
+    out.v[u] = 0.0f;
+    FOR_E {
+      if (e < nv) {
+        const int64_t at = static_cast<int64_t>(off.v[u] + e * step) + static_cast<int64_t>(__float_as_int(idx.v[u][e]));
+        out.v[u][e] = elem_load(addr, dtype, static_cast<uint64_t>(at));
+      }
+    }
+  }
+  return out;
 }
 
 // Which slabs of a round the whole wave can treat alike. `full`: bit u is set when slab u is full in every lane;
@@ -903,6 +928,13 @@ __device__ __forceinline__ uint32_t group_valid(uint32_t n, const VDim *dims, ui
   return left < static_cast<uint32_t>(E) ? left : static_cast<uint32_t>(E);
 }
 
+// VBI_WRAP: an index into an axis of extent n, negative values counting from the end, clipped into the axis
+__device__ __forceinline__ int32_t wrap_index(int32_t i, int32_t n) {
+  i = i < 0 ? i + n : i;
+  i = i < n - 1 ? i : n - 1;
+  return i > 0 ? i : 0;
+}
+
 // Arithmetic on one value per lane, for instructions flagged VI_UNIFORM. Inlined, so that the opcode stays
 // in scalar registers and the selection below is a scalar branch (as arguments of an out-of-line function
 // the opcodes travel in vector registers and every case is walked under an execution mask); the library
@@ -933,6 +965,7 @@ __device__ __forceinline__ float uniform_binary(uint32_t op, uint32_t sub, float
       case VBI_RSUB: return __uint_as_float(yi - xi);
       case VBI_MUL: return __uint_as_float(xi * yi);
       case VBI_MIN: return __int_as_float(min(xs, ys));
+      case VBI_WRAP: return __int_as_float(wrap_index(xs, ys));
       default: return __int_as_float(max(xs, ys));
     }
   }

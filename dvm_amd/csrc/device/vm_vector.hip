@@ -350,6 +350,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               case VBI_RSUB: FOR_U FOR_E acc.v[u][e] = __uint_as_float(si - __float_as_uint(acc.v[u][e])); break;
               case VBI_MUL: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(acc.v[u][e]) * si); break;
               case VBI_MIN: FOR_U FOR_E acc.v[u][e] = __int_as_float(min(__float_as_int(acc.v[u][e]), static_cast<int32_t>(si))); break;
+              case VBI_WRAP: FOR_U FOR_E acc.v[u][e] = __int_as_float(wrap_index(__float_as_int(acc.v[u][e]), static_cast<int32_t>(si))); break;
               default: FOR_U FOR_E acc.v[u][e] = __int_as_float(max(__float_as_int(acc.v[u][e]), static_cast<int32_t>(si))); break;
             }
           } else {
@@ -544,6 +545,9 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               if (!take_next_along(m, off, sl, acc, src)) continue;
             }
             // the binary instruction behind the load: its operand is in src, the switch below finishes it
+          } else if (op == VOP_LDX) {
+            acc = mem_gather(m.addr, m.dtype, m.flags, off, sl.nvp, acc);
+            continue;
           } else {
             mem_load(m, off, sl, src);
             if (op == VOP_BINF && (imm & VI_PRE_SREG)) {  // an S-register binary in front, while the operand is on its way
@@ -595,6 +599,7 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               case VBI_RSUB: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(src.v[u][e]) - __float_as_uint(acc.v[u][e])); break;
               case VBI_MUL: FOR_U FOR_E acc.v[u][e] = __uint_as_float(__float_as_uint(acc.v[u][e]) * __float_as_uint(src.v[u][e])); break;
               case VBI_MIN: FOR_U FOR_E acc.v[u][e] = __int_as_float(min(__float_as_int(acc.v[u][e]), __float_as_int(src.v[u][e]))); break;
+              case VBI_WRAP: FOR_U FOR_E acc.v[u][e] = __int_as_float(wrap_index(__float_as_int(acc.v[u][e]), __float_as_int(src.v[u][e]))); break;
               default: FOR_U FOR_E acc.v[u][e] = __int_as_float(max(__float_as_int(acc.v[u][e]), __float_as_int(src.v[u][e]))); break;
             }
             break;

@@ -551,6 +551,47 @@ dvm_obj *dvm_rt_view_store(dvm_rt *rt, dvm_obj *x, dvm_shape *stride, size_t ext
       static_cast<dvm_obj *>(nullptr));
 }
 
+dvm_obj *dvm_rt_global_access(dvm_rt *rt, dvm_shape *shape, int dtype) { return dvm_rt_load(rt, shape, dtype); }
+
+dvm_obj *dvm_rt_gather_load(dvm_rt *rt, dvm_shape *shape, dvm_obj *index, int dtype, int axis, int gather_mode) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.GatherLoad(nullptr, &shape->ref, Obj(index), axis, static_cast<DataType>(dtype),
+                                            gather_mode == 1 ? kSliceGather : kElementGather);
+        rt->loads.push_back(o);  // the source tensor is bound to the operator like a load's
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_pad_store(dvm_rt *rt, dvm_obj *x, long long pad_size) {
+  return Guard(
+      [&]() {
+        NDObject *o = rt->kernel.PadStore(nullptr, Obj(x), pad_size);
+        rt->stores.push_back(o);
+        return Handle(o);
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_one_hot(dvm_rt *rt, dvm_obj *indices, dvm_shape *depth, int axis, double on_value, double off_value, int dtype) {
+  return Guard(
+      [&]() {
+        switch (static_cast<DataType>(dtype)) {
+          case kFloat32: return Handle(rt->kernel.OneHot(Obj(indices), &depth->ref, axis, static_cast<float>(on_value), static_cast<float>(off_value)));
+          case kInt32: return Handle(rt->kernel.OneHot(Obj(indices), &depth->ref, axis, static_cast<int32_t>(on_value), static_cast<int32_t>(off_value)));
+          case kFloat16: return Handle(rt->kernel.OneHot(Obj(indices), &depth->ref, axis, Float16(static_cast<float>(on_value)), Float16(static_cast<float>(off_value))));
+          case kBFloat16: return Handle(rt->kernel.OneHot(Obj(indices), &depth->ref, axis, BFloat16(static_cast<float>(on_value)), BFloat16(static_cast<float>(off_value))));
+          default: throw std::runtime_error("DVM EXCEPTION. reason: one_hot makes fp32, int32, fp16 or bf16 tensors");
+        }
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
+dvm_obj *dvm_rt_element_any(dvm_rt *rt, dvm_obj *x) {
+  return Guard([&]() { return Handle(rt->kernel.ElemAny(Obj(x))); }, static_cast<dvm_obj *>(nullptr));
+}
+
 dvm_obj *dvm_rt_permute(dvm_rt *rt, dvm_obj *x, dvm_shape *dims) {
   return Guard([&]() { return Handle(rt->kernel.Permute(Obj(x), &dims->ref)); }, static_cast<dvm_obj *>(nullptr));
 }
@@ -745,9 +786,17 @@ int dvm_rt_codegen(dvm_rt *rt) {
         for (NDObject *s : rt->stores) {
           if (s->temp) continue;  // SetStoreTemp: no output of the kernel
           auto ext = rt->store_extent.find(s);
-          if (ext != rt->store_extent.end()) {
+          if (ext != rt->store_extent.end() || s->pad_size >= 0) {
             // a strided store writes part of a larger buffer, which starts out as zeros
-            const size_t bytes = ext->second * DTypeSize(s->type_id_);
+            size_t elems = 0;
+            if (s->pad_size >= 0) {  // PadStore: rows pad_size longer than the value's
+              elems = s->rank() > 0 ? 1 : 0;
+              for (int d = 0; d + 1 < s->rank(); ++d) elems *= static_cast<size_t>(s->dim(d));
+              if (s->rank() > 0) elems *= static_cast<size_t>(s->dim(s->rank() - 1) + s->pad_size);
+            } else {
+              elems = ext->second;
+            }
+            const size_t bytes = elems * DTypeSize(s->type_id_);
             const bool fresh = rt->buffers.find(s) == rt->buffers.end() || rt->buffers[s].ptr == nullptr;
             rt->Ensure(s, bytes);
             if (fresh && !rt->das_mode && bytes > 0) {

@@ -36,9 +36,9 @@ void PrintShape(std::ostringstream &os, const NDObject *o) {
   os << "]";
 }
 
-const char *kMemTypes[] = {"bool", "fp16", "bf16", "fp32", "int32"};
+const char *kMemTypes[] = {"bool", "fp16", "bf16", "fp32", "int32", "positions"};
 const char *kBinF[] = {"Add", "Sub", "RSub", "Mul", "Div", "RDiv", "Min", "Max", "And", "Or", "Pow", "RPow", "Div~", "RDiv~"};
-const char *kBinI[] = {"Add", "Sub", "RSub", "Mul", "Min", "Max"};
+const char *kBinI[] = {"Add", "Sub", "RSub", "Mul", "Min", "Max", "WrapIndex"};
 const char *kUn[] = {"Sqrt", "Abs", "Log", "Exp", "IsFinite", "Round", "Floor", "Ceil", "Trunc", "Abs", "Exp", "Exp~", "Exp~", "Log~", "Sqrt~"};
 const char *kCmp[] = {"Eq", "Ne", "Gt", "Ge", "Lt", "Le"};
 const char *kRnd[] = {"fp32", "fp16", "bf16", "?"};
@@ -88,6 +88,8 @@ std::string &VKernel::DumpGraph(bool ref_shapes) {
       case kObjCopy: os << "Copy"; break;
       case kObjMatMul: os << "MatMul" << (o->trans_a ? "T" : "N") << (o->trans_b ? "T" : "N"); break;
       case kObjPack64: os << "Pack"; break;
+      case kObjOneHot: os << "OneHot<" << o->slice_dim << ">"; break;
+      case kObjGather: os << "GatherLoad<" << o->slice_dim << ", gather_mode(" << static_cast<int>(o->op) << ")>"; break;
       case kObjHalf64: os << (o->op == 0 ? "ExtractLo" : "ExtractHi"); break;
     }
     os << "." << DTypeName(o->type_id_) << "(";
@@ -184,6 +186,7 @@ std::string &VKernel::DisAssemble() {
             break;
           case VOP_BINI: os << kBinI[sub & 0x3f] << ".int32 acc, "; PrintSrc(os, w); break;
           case VOP_CMP: os << "Cmp" << kCmp[sub & 7] << "." << ((sub & VCMP_INT) ? "int32" : "fp32") << " acc, "; PrintSrc(os, w); break;
+          case VOP_LDX: os << "gather_load." << kMemTypes[mem_dtype(VI_A(w))] << " acc, m" << VI_A(w) << " + acc"; break;
           case VOP_MSK: os << "mask "; PrintSrc(os, w); break;
           case VOP_MOVM: os << "select acc, "; PrintSrc(os, w); break;
           default: os << "?"; break;

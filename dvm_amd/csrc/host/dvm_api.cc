@@ -634,7 +634,18 @@ void Kernel::Clone(const Kernel &base, CloneHelper &helper) {
     for (int i = 0; i < o->nin; ++i) c->in[i] = helper.GetClone(o->in[i]);
     c->scalar.imm = o->scalar.imm;
     c->scalar.ref = o->scalar.ref != nullptr ? helper.GetClone(o->scalar.ref) : nullptr;
-    c->aux_ref = o->aux_ref != nullptr ? helper.GetClone(o->aux_ref) : nullptr;
+    if (o->aux_ref == &o->own_axes_ref_) {  // a list the operator made for itself
+      std::memcpy(c->own_axes_, o->own_axes_, sizeof(c->own_axes_));
+      c->own_axes_ref_.data = c->own_axes_;
+      c->own_axes_ref_.size = o->own_axes_ref_.size;
+      c->aux_ref = &c->own_axes_ref_;
+    } else {
+      c->aux_ref = o->aux_ref != nullptr ? helper.GetClone(o->aux_ref) : nullptr;
+    }
+    c->elem_any = o->elem_any;
+    c->pad_size = o->pad_size;
+    c->scalar2.imm = o->scalar2.imm;
+    c->scalar2.ref = o->scalar2.ref != nullptr ? helper.GetClone(o->scalar2.ref) : nullptr;
     c->addr = o->addr;
     c->strided = o->strided;
     c->view_offset = o->view_offset;
@@ -685,8 +696,23 @@ NDObject *Kernel::Load(void *addr, IntArrayRef *shape, IntArrayRef *stride, Data
   return o;
 }
 
-NDObject *Kernel::GlobalAccess(void *, IntArrayRef *, DataType) { Unsupported("GlobalAccess"); }
-NDObject *Kernel::GatherLoad(void *, IntArrayRef *, NDObject *, int, DataType, GatherMode) { Unsupported("GatherLoad"); }
+// GlobalAccess names a tensor in memory for another operator to read (the index of a GatherLoad,
+// include/dvm.h:284,297-307 of the reference). Here that is a Load: a load nothing reads costs nothing.
+NDObject *Kernel::GlobalAccess(void *addr, IntArrayRef *shape, DataType type) { return Load(addr, shape, type); }
+
+// GatherLoad (src/ops.h:632-657 of the reference; tests/ut/test_gather_load.py): the source tensor read at the
+// positions an int32 index tensor names along one axis. Negative indices count from the end of the axis; indices past
+// either end are clipped into it (the reference leaves them undefined).
+NDObject *Kernel::GatherLoad(void *addr, IntArrayRef *shape, NDObject *index, int axis, DataType type, GatherMode gather_mode) {
+  if (index == nullptr || index->type_id_ != kInt32) Throw("GatherLoad needs an int32 index tensor");
+  if (type == kInt64) Throw("GatherLoad of int64 tensors is not supported by the gfx950 backend");
+  NDObject *o = Builder(kernel_).New(kObjGather, type, index);
+  o->addr = addr;
+  o->full_shape_ref = shape;
+  o->slice_dim = axis;
+  o->op = gather_mode == kSliceGather ? 1 : 0;
+  return o;
+}
 NDObject *Kernel::SliceLoad(void *addr, IntArrayRef *shape, IntArrayRef *start, IntArrayRef *size, DataType type) {
   NDObject *o = Load(addr, size, type);  // the value has the slice's shape
   o->strided = true;
@@ -739,7 +765,16 @@ NDObject *Kernel::Store(void *addr, NDObject *input, IntArrayRef *stride) {
   return o;
 }
 
-NDObject *Kernel::PadStore(void *, NDObject *, int64_t) { Unsupported("PadStore"); }
+// PadStore (src/ops.h:713-731, src/ops.cc:1399-1412 of the reference): a store into a buffer whose innermost rows
+// are pad_size elements longer than the value's; the padding is not written.
+NDObject *Kernel::PadStore(void *addr, NDObject *input, int64_t pad_size) {
+  if (pad_size < 0) Throw("PadStore needs a pad size of zero or more");
+  if (input->type_id_ == kInt64) Throw("PadStore of int64 tensors is not supported by the gfx950 backend");
+  NDObject *o = Store(addr, input);
+  o->strided = true;
+  o->pad_size = pad_size;
+  return o;
+}
 void Kernel::SetStoreInplace(NDObject *store) { store->inplace = true; }
 // A temporary Store and a Load bound to it hand a value from one part of a kernel to a later one through memory in
 // the reference (src/dvm.cc:1583-1588). Here operators read the value directly (the launches are cut at code
@@ -955,15 +990,43 @@ NDObject **Kernel::Split(NDObject *input, int dim, int64_t split_size, size_t sp
   }
   return out;
 }
+// OneHot (include/dvm.h:482-491, src/ops.h:1333 of the reference; tests/ut/test_onehot.py): a dim of extent depth at
+// position axis, on_value where the position equals the index, off_value elsewhere (also for indices outside [0, depth)).
 template <typename T>
-NDObject *Kernel::OneHot(NDObject *, IntArrayRef *, int, T, T) {
-  Unsupported("OneHot");
+NDObject *Kernel::OneHot(NDObject *indices, IntArrayRef *depth, int axis, T on_value, T off_value) {
+  if (indices == nullptr || indices->type_id_ != kInt32) Throw("OneHot needs int32 indices");
+  DataType t = kFloat32;
+  if constexpr (std::is_same<T, int32_t>::value) t = kInt32;
+  if constexpr (std::is_same<T, Float16>::value) t = kFloat16;
+  if constexpr (std::is_same<T, BFloat16>::value) t = kBFloat16;
+  NDObject *o = Builder(kernel_).New(kObjOneHot, t, indices);
+  o->aux_ref = depth;
+  o->slice_dim = axis;
+  o->scalar = MakeOperand(on_value).sc;
+  o->scalar2 = MakeOperand(off_value).sc;
+  return o;
 }
 template NDObject *Kernel::OneHot<float>(NDObject *, IntArrayRef *, int, float, float);
 template NDObject *Kernel::OneHot<int32_t>(NDObject *, IntArrayRef *, int, int32_t, int32_t);
 template NDObject *Kernel::OneHot<Float16>(NDObject *, IntArrayRef *, int, Float16, Float16);
 template NDObject *Kernel::OneHot<BFloat16>(NDObject *, IntArrayRef *, int, BFloat16, BFloat16);
-NDObject *Kernel::ElemAny(NDObject *) { Unsupported("ElemAny"); }
+// ElemAny (src/ops.h:874-892, src/vm_aiv.cce:193-210 of the reference; tests/ut/test_element_any.py): one fp32 value,
+// the maximum over every element of the input, so 1 when any element of a 0 / 1 mask is set. (The reference stores it
+// only when it is not zero, into a buffer the caller has cleared; here it is always stored.)
+NDObject *Kernel::ElemAny(NDObject *input) {
+  if (input->type_id_ != kFloat32) Throw("ElemAny needs an fp32 input");
+  kernel_->Normalize();  // (the input's rank)
+  NDObject *o = Builder(kernel_).New(kObjReduce, kFloat32, input);
+  o->op = static_cast<uint8_t>(kMax);
+  const int r = o->in[0]->rank();
+  for (int i = 0; i < r; ++i) o->own_axes_[i] = i;
+  o->own_axes_ref_.data = o->own_axes_;
+  o->own_axes_ref_.size = static_cast<size_t>(r);
+  o->aux_ref = &o->own_axes_ref_;
+  o->keepdims = false;
+  o->elem_any = true;
+  return o;
+}
 NDObject *Kernel::GroupedMatMul(NDObject *, NDObject *, bool, bool, NDObject *, NDObject *, GmmSplitType, GmmListType) {
   Unsupported("GroupedMatMul");
 }

@@ -46,7 +46,9 @@ int Compiler::MemIndex(int v) {
   if (n_mem_ >= DVM_VEC_MAXMEM) Fail("too many memory operands");
   VMemDesc &m = mems_[n_mem_];
   std::memset(&m, 0, sizeof(m));
-  m.dtype = MemDType(n.dtype);
+  // (a OneHot's own operand: the positions along its new dim, no memory behind them)
+  const bool iota = n.kind == AK_OP && n.op->kind == kObjOneHot;
+  m.dtype = iota ? VDT_IOTA : MemDType(n.dtype);
   // element stride of every axis the operand has (row-major over its own shape)
   int64_t stride = 1;
   int64_t dim_stride[kMaxAxes];
@@ -63,7 +65,7 @@ int Compiler::MemIndex(int v) {
   }
   const int inner = n_dims_ - 1;
   bool aligned = true;
-  const int64_t isz = static_cast<int64_t>(DTypeSize(n.dtype));
+  const int64_t isz = iota ? 4 : static_cast<int64_t>(DTypeSize(n.dtype));
   const int64_t need = isz * E >= 16 ? 16 : isz * E;
   for (int i = 0; i < nk_; ++i) {
     const int md = klist_[i];
@@ -100,13 +102,14 @@ int Compiler::MemIndex(int v) {
       Fail("innermost axis is not contiguous");
     }
   }
+  if (iota) m.flags &= ~static_cast<uint32_t>(VMF_ALIGNED);  // element by element: the 128-bit paths would read memory
   Program::Patch p;
   p.word = static_cast<uint32_t>(sizeof(VVecHeader) / 8 + n_mem_ * (sizeof(VMemDesc) / 8));
   p.op_id = n.addr_op;
   p.ws_slot = n.ws_slot;
   p.byte_offset = n.view != nullptr ? n.view->view_base_ * isz : 0;
   mem_is_view_[n_mem_] = n.view != nullptr;
-  p.role = Program::kPatchVecMem;
+  p.role = iota ? Program::kPatchIota : Program::kPatchVecMem;
   prog_->patches.push_back(p);
   n.mem_idx = n_mem_++;
   return n.mem_idx;
@@ -440,6 +443,29 @@ void Compiler::ComputeInto(int v) {
       BeforeOverwrite();
       EmitOperandInsn(VOP_MSK, 0, 0, c);
       EmitOperandInsn(VOP_MOVM, 0, 0, x);
+      return;
+    }
+    case kObjOneHot: {
+      const int x = Resolve(n.in[0]);
+      EmitValue(x);
+      ConsumeUse(x);
+      BeforeOverwrite();
+      // index == position along the new dim ? on : off
+      Emit(VOP_CMP, VCMP_EQ + VCMP_INT, VK_MEM, 0, MemIndex(v), 0);
+      Emit(VOP_MSK, 0, VK_ACC, 0, 0, 0);
+      Emit(VOP_LDI, 0, 0, 0, 0, ScalarToContainer(o->scalar2.Get(), n.dtype));
+      Emit(VOP_MOVM, 0, VK_IMM, 0, 0, ScalarToContainer(o->scalar.Get(), n.dtype));
+      return;
+    }
+    case kObjGather: {
+      const int x = Resolve(n.in[0]);
+      EmitValue(x);
+      ConsumeUse(x);
+      BeforeOverwrite();
+      // the index becomes an offset in elements: wrapped into the gathered dim, times that dim's stride
+      Emit(VOP_BINI, VBI_WRAP, VK_IMM, 0, 0, static_cast<uint32_t>(o->gather_extent));
+      if (o->gather_stride != 1) Emit(VOP_BINI, VBI_MUL, VK_IMM, 0, 0, static_cast<uint32_t>(o->gather_stride));
+      Emit(VOP_LDX, 0, VK_MEM, 0, MemIndex(v), 0);
       return;
     }
     default:

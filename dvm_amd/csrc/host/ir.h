@@ -47,6 +47,16 @@ enum ObjKind : uint8_t {
   // words; a handle only, nothing computes it), or a Load of that type, whose words are read through two views:
   kObjPack64,
   kObjHalf64,      // view of an int64 Load: every second 32-bit word of its memory (op = 0 low words, 1 high words)
+  // OneHot (src/ops.h:1333 of the reference): in[0] = int32 indices; the result has one more dim, of extent aux_ref[0],
+  // at position slice_dim; scalar where the position along that dim equals the index, scalar2 elsewhere. The positions
+  // are a memory operand without memory (VDT_IOTA) that walks the result's index space with the strides in vstride_.
+  kObjOneHot,
+  // GatherLoad (src/ops.h:632): the node is the source tensor (addr; full_shape_ref = its shape) read at positions an
+  // int32 index tensor names along dim slice_dim. in[0] = the index values. op = 0: the index has the result's shape,
+  // result[i..] = source[i.. with the index value in place of the coordinate along the dim] (NumPy take_along_axis);
+  // op = 1: the index's dims replace the dim (NumPy take). vstride_ = the source's strides seen from the result's
+  // index space, 0 along the gathered dims.
+  kObjGather,
 };
 
 // A scalar operand: an immediate fixed at build time or a ScalarRef re-read at every code generation.
@@ -81,6 +91,13 @@ class NDObject {
   int nin = 0;
   NDObject *in[3] = {nullptr, nullptr, nullptr};
   ScalarOperand scalar;
+  ScalarOperand scalar2;           // kObjOneHot: the value where the index does not match
+  bool elem_any = false;           // kObjReduce made by ElemAny: a reduce to one element, result of shape [1]
+  int64_t pad_size = -1;           // kObjStore made by PadStore: rows of the buffer are this many elements longer than the value's
+  int64_t gather_extent = 0, gather_stride = 0;  // kObjGather: extent and element stride of the gathered dim of the source
+  // storage for a list of dims an operator made for itself (the reduce behind ElemAny): aux_ref points here then
+  int64_t own_axes_[10] = {0};
+  IntArrayRef own_axes_ref_;
   IntArrayRef *aux_ref = nullptr;  // reduce axes / broadcast target / reshape target / user shape of a load
   void *addr = nullptr;            // load / store address (may arrive later through a RelocEntry)
   // A load or store that walks its buffer with strides of its own (Kernel::Load / Store with a stride list,
@@ -146,11 +163,12 @@ struct Program {
     int op_id;       // load/store node whose address goes there, or -1
     int ws_slot;     // or the workspace slot
     int64_t byte_offset = 0;  // added to the operator's address (strided views start inside their buffer)
-    uint8_t role;    // kPatchVecMem: a VMemDesc (alignment flag follows the address); kPatchCubeOperand:
+    uint8_t role;    // kPatchVecMem: a VMemDesc (alignment flag follows the address); kPatchIota: a VMemDesc without
+                     // memory, whose address word is its first value (byte_offset / 4); kPatchCubeOperand:
                      // a matmul operand (the fast path needs 16-byte alignment); kPatchPlain: nothing else;
                      // kPatchAligned16: an operand of the fused attention kernel, which only has 128-bit accesses
   };
-  enum : uint8_t { kPatchVecMem = 0, kPatchCubeOperand = 1, kPatchPlain = 2, kPatchAligned16 = 3 };
+  enum : uint8_t { kPatchVecMem = 0, kPatchCubeOperand = 1, kPatchPlain = 2, kPatchAligned16 = 3, kPatchIota = 4 };
   std::vector<Patch> patches;
   // What binding an unaligned address takes away from the blob (the alignment flag of a memory operand, the sweep
   // build of a vector program, the fast path of a matmul), as code generation left it: (32-bit word of the blob,

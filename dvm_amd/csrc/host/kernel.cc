@@ -142,6 +142,10 @@ void VKernel::BindAddresses(const RelocEntry *relocs, size_t n, WsAllocator *all
     for (const auto &orig : p.bind_dependent) reinterpret_cast<uint32_t *>(p.blob.w)[orig.first] = orig.second;
     for (const Program::Patch &pt : p.patches) {
       uint64_t addr = 0;
+      if (pt.role == Program::kPatchIota) {  // positions along an axis: no memory, the word is the first value
+        p.blob.w[pt.word] = static_cast<uint64_t>(pt.byte_offset / 4);
+        continue;
+      }
       if (pt.op_id >= 0) {
         addr = reinterpret_cast<uint64_t>(ops_[pt.op_id]->addr);
         if (addr != 0) addr += static_cast<uint64_t>(pt.byte_offset);

@@ -99,6 +99,18 @@ void VKernel::Normalize() {
           hv->view_base_ = o->view_base_ + 1;
           break;
         }
+        if (o->pad_size >= 0) {
+          // PadStore (src/ops.cc:1399-1412): the buffer's rows are pad_size elements longer than the value's
+          const size_t r = o->in[0]->shape_ref_->size;
+          if (r == 0) Throw("PadStore of a value without dims");
+          int64_t dense = 1;
+          for (size_t i = r; i-- > 0;) {
+            o->vstride_[i] = dense;
+            dense *= o->shape_[i] + (i + 1 == r ? o->pad_size : 0);
+          }
+          o->view_base_ = o->view_offset;
+          break;
+        }
         if (o->strided) {
           if (o->stride_ref->size != o->in[0]->shape_ref_->size) Throw("stride list does not match the tensor rank");
           for (size_t i = 0; i < o->stride_ref->size; ++i) o->vstride_[i] = o->stride_ref->data[i];
@@ -108,6 +120,67 @@ void VKernel::Normalize() {
       case kObjPack64:
         o->SetShape(o->in[0]->shape_ref_->data, o->in[0]->shape_ref_->size);
         break;
+      case kObjOneHot: {
+        const NDObject *x = o->in[0];
+        const size_t r = x->shape_ref_->size;
+        if (r + 1 > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
+        if (o->aux_ref == nullptr || o->aux_ref->size != 1 || o->aux_ref->data[0] < 0) Throw("OneHot needs one depth");
+        int64_t axis = o->slice_dim;
+        if (axis < 0) axis += static_cast<int64_t>(r) + 1;
+        if (axis < 0 || axis > static_cast<int64_t>(r)) Throw("OneHot axis out of range");
+        for (size_t i = 0, j = 0; i <= r; ++i) {
+          o->shape_[i] = static_cast<int64_t>(i) == axis ? o->aux_ref->data[0] : x->shape_ref_->data[j++];
+          o->vstride_[i] = static_cast<int64_t>(i) == axis ? 1 : 0;
+        }
+        o->own_ref_.size = r + 1;
+        o->view_base_ = 0;  // (vstride_ describes the operator's own operand; the value itself is dense: strided stays false)
+        break;
+      }
+      case kObjGather: {
+        const NDObject *ix = o->in[0];
+        const IntArrayRef *src = o->full_shape_ref;
+        const size_t rs = src->size, ri = ix->shape_ref_->size;
+        int64_t axis = o->slice_dim;
+        if (axis < 0) axis += static_cast<int64_t>(rs);
+        if (rs == 0 || axis < 0 || axis >= static_cast<int64_t>(rs)) Throw("gather axis out of range");
+        int64_t dense[kMaxRank], acc = 1;
+        for (size_t i = rs; i-- > 0;) {
+          dense[i] = acc;
+          acc *= src->data[i];
+        }
+        o->gather_extent = src->data[axis];
+        o->gather_stride = dense[axis];
+        if (acc >= (1ll << 31)) Throw("GatherLoad from a tensor of 2^31 elements or more");  // (offsets are int32 arithmetic)
+        if (o->gather_extent == 0 && ix->numel() > 0) Throw("GatherLoad along an empty dim");
+        if (o->op == 0) {  // the index has the source's rank; the result takes its shape
+          if (ri != rs) Throw("the index of an element gather needs the rank of the source");
+          for (size_t i = 0; i < rs; ++i) {
+            if (static_cast<int64_t>(i) != axis && ix->shape_ref_->data[i] > src->data[i]) Throw("the index of an element gather reaches outside the source");
+            o->shape_[i] = ix->shape_ref_->data[i];
+            o->vstride_[i] = static_cast<int64_t>(i) == axis ? 0 : dense[i];
+          }
+          o->own_ref_.size = rs;
+        } else {  // the index's dims stand where the gathered dim was
+          const size_t r = rs - 1 + ri;
+          if (r > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
+          size_t n = 0;
+          for (size_t i = 0; i < static_cast<size_t>(axis); ++i, ++n) {
+            o->shape_[n] = src->data[i];
+            o->vstride_[n] = dense[i];
+          }
+          for (size_t i = 0; i < ri; ++i, ++n) {
+            o->shape_[n] = ix->shape_ref_->data[i];
+            o->vstride_[n] = 0;
+          }
+          for (size_t i = static_cast<size_t>(axis) + 1; i < rs; ++i, ++n) {
+            o->shape_[n] = src->data[i];
+            o->vstride_[n] = dense[i];
+          }
+          o->own_ref_.size = r;
+        }
+        o->view_base_ = 0;  // (vstride_ describes the operator's own operand; the value itself is dense: strided stays false)
+        break;
+      }
       case kObjHalf64: {
         // the 32-bit words of an int64 Load: its strides (its own when it is a strided load, else those of a dense
         // tensor) doubled, its offset doubled, plus one for the high words
@@ -183,6 +256,7 @@ void VKernel::Normalize() {
             o->shape_[n++] = x->shape_ref_->data[i];
           }
         }
+        if (n == 0 && o->elem_any) o->shape_[n++] = 1;  // (ElemAny's result has shape [1])
         o->own_ref_.size = n;
         break;
       }

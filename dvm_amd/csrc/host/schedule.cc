@@ -136,6 +136,10 @@ void Compiler::BuildNodes(int a) {
         if (o->strided) n.view = o;
       }
     }
+    if (o->kind == kObjOneHot || o->kind == kObjGather) {
+      n.view = o;  // the operator's own operand: positions along the new dim / the source tensor
+      if (o->kind == kObjGather) n.addr_op = i;
+    }
     node_of_[i] = idx;
     // a value later sub-kernels read and that the user does not store: write it to workspace
     if (mat_[i] && ws_slot_[i] >= 0) {
@@ -211,6 +215,24 @@ void Compiler::UnifyAxes() {
         }
         break;
       case AK_OP:
+        if (n.op->kind == kObjOneHot || (n.op->kind == kObjGather && n.op->op == 1)) {
+          // the input's dims stand in the result's in order, apart from the dim a OneHot adds / with the dims of a
+          // slice gather's index where the gathered dim was
+          const ANode &x = nodes_[n.in[0]];
+          int64_t at = n.op->slice_dim;
+          if (n.op->kind == kObjOneHot) {
+            if (at < 0) at += n.rank;
+            for (int d = 0; d < x.rank; ++d) {
+              const int od = d < at ? d : d + 1;
+              if (x.dims[d] != 1 && x.dims[d] == n.dims[od]) Union(Var(i, od), Var(n.in[0], d));
+            }
+          } else {
+            if (at < 0) at += n.rank - x.rank + 1;
+            for (int d = 0; d < x.rank; ++d)
+              if (x.dims[d] != 1 && x.dims[d] == n.dims[at + d]) Union(Var(i, static_cast<int>(at) + d), Var(n.in[0], d));
+          }
+          break;
+        }
         for (int j = 0; j < n.nin; ++j)
           if (n.in[j] >= 0) UnifyAligned(i, n.in[j]);
         break;
@@ -382,7 +404,7 @@ void Compiler::OrderAndMerge() {
       merge = axes_[a0].reduced == axes_[a1].reduced;
       for (int i = 0; i < nn_ && merge; ++i) {
         const ANode &n = nodes_[i];
-        if (n.kind != AK_MEM && n.kind != AK_OUT) continue;
+        if (n.kind != AK_MEM && n.kind != AK_OUT && !(n.kind == AK_OP && n.view != nullptr)) continue;
         int d0 = -1, d1 = -1;
         for (int d = 0; d < n.rank; ++d) {
           if (n.axis[d] == a0) d0 = d;
@@ -508,7 +530,7 @@ void Compiler::ChooseSchedule() {
     if (tile_gather && nk_ >= 2 && nk_ < DVM_VEC_MAXR && klist_[0] == inner && dims_[inner].extent % (8 * E) == 0) {
       for (int i = 0; i < nn_ && !split_inner_; ++i) {
         const ANode &n = nodes_[i];
-        if ((n.kind != AK_MEM && n.kind != AK_OUT) || n.view == nullptr) continue;
+        if ((n.kind != AK_MEM && n.kind != AK_OUT && n.kind != AK_OP) || n.view == nullptr) continue;
         for (int d = 0; d < n.rank; ++d) {
           if (n.axis[d] < 0 || pos_[n.axis[d]] != dims_[inner].last_axis) continue;
           const int64_t st = n.view->vstride_[d];

@@ -42,6 +42,10 @@ enum {
   VDT_BF16 = 2,
   VDT_F32 = 3,
   VDT_I32 = 4,
+  // No memory behind it: the element at offset i of the operand is the int32 value addr + i. With stride 1 along one
+  // axis and 0 along the others it is that axis's coordinate (the position a one-hot compares its indices with).
+  // Loads only, never with VMF_ALIGNED (the 128-bit paths would read memory).
+  VDT_IOTA = 5,
 };
 
 // ---- schedules -------------------------------------------------------------
@@ -97,6 +101,7 @@ enum {
   VOP_CMP = 19,      // acc = acc (sub = VCMP_*, +8 for int32) src ? 1 : 0 in the operand's container
   VOP_MSK = 20,      // mask = src != 0          (per element predicate)
   VOP_MOVM = 21,     // acc = mask ? src : acc
+  VOP_LDX = 22,      // acc = mem[a] at the operand's offsets plus acc (int32, in elements): a gather. kind is VK_MEM
 };
 
 // source kinds (bits 16..19). VK_SREG2 (VOP_BINF only) chains two float binaries with S-register operands in
@@ -114,7 +119,8 @@ enum {
   VB_DIV_APPROX, VB_RDIV_APPROX,  // matmul epilogues only: acc * rcp(src), src * rcp(acc) with v_rcp_f32
 };
 // int32 binary sub-ops
-enum { VBI_ADD = 0, VBI_SUB, VBI_RSUB, VBI_MUL, VBI_MIN, VBI_MAX };
+// VBI_WRAP: an index into an axis of extent src: acc + src where acc is negative, then clipped to [0, src - 1]
+enum { VBI_ADD = 0, VBI_SUB, VBI_RSUB, VBI_MUL, VBI_MIN, VBI_MAX, VBI_WRAP };
 // unary sub-ops
 enum {
   VU_SQRT = 0, VU_ABS, VU_LOG, VU_EXP, VU_ISFINITE, VU_ROUND, VU_FLOOR, VU_CEIL, VU_TRUNC, VU_IABS,

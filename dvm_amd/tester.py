@@ -120,6 +120,20 @@ class Tester(PyKernel):
             return PyKernel.view_load(self, shape, stride, as_datatype(arr_dtype))
         return self._bound(lambda h: PyKernel.view_load(self, shape, stride, h.dtype), arr_dtype, real_dtype, offset)
 
+    def global_access(self, shape_arr, dtype=None):
+        dtype = DataType.int32 if dtype is None else dtype
+        if not isinstance(shape_arr, np.ndarray):
+            return PyKernel.global_access(self, shape_arr, as_datatype(dtype))
+        return self._bound(lambda h: PyKernel.global_access(self, h.shape, h.dtype), shape_arr, dtype)
+
+    def gather_load(self, data_arr, index_op, axis=0, dtype=None, gather_mode=0):
+        if not isinstance(data_arr, np.ndarray):
+            return PyKernel.gather_load(self, data_arr, index_op, as_datatype(dtype), axis, gather_mode)
+        return self._bound(lambda h: PyKernel.gather_load(self, h.shape, index_op, h.dtype, axis, gather_mode), data_arr, dtype)
+
+    def one_hot(self, indices, depth, axis, on_value, off_value, dtype):
+        return PyKernel.one_hot(self, indices, depth, axis, on_value, off_value, as_datatype(dtype))
+
     def slice_load(self, shape_arr, start, size, dtype=None):
         if not isinstance(shape_arr, np.ndarray):
             return PyKernel.slice_load(self, shape_arr, start, size, as_datatype(dtype))
@@ -150,6 +164,12 @@ class Tester(PyKernel):
         self._buffer_shape[op._h] = tuple(e.shape)
         self._expectations.append(Expectation(op, e, eps, tuple(e.shape)))
         return op
+
+    def clear_store_memory(self, store):
+        """RtKernelPy.clear_store_memory (src/pybind_api.cc:874-877 of the reference) zeroes an output before the run, for
+        element_any, which there only stores a value that is not zero. Here element_any always stores its result, so
+        there is nothing to clear."""
+        del store
 
     def output(self, store, shape=None):
         return PyKernel.output(self, store, shape if shape is not None else self._buffer_shape.get(store._h))

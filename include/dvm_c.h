@@ -60,6 +60,17 @@ dvm_obj *dvm_rt_reshape(dvm_rt *rt, dvm_obj *x, dvm_shape *shape);
 dvm_obj *dvm_rt_reduce(dvm_rt *rt, int reduce_type, dvm_obj *x, dvm_shape *dims, int keepdims);
 dvm_obj *dvm_rt_copy(dvm_rt *rt, dvm_obj *x);
 dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int trans_b, dvm_obj *bias);
+// Kernel::GlobalAccess / GatherLoad / PadStore / OneHot / ElemAny (include/dvm.h:284, 297-307, 344, 482-496 of the
+// reference; KernelPy global_access / gather_load / pad_store / one_hot / element_any, include/dvm_py.h:302-327).
+// global_access names an int32 index tensor (bound like a load); gather_load reads the tensor bound to the returned
+// handle (like a load's input) at those indices along `axis` (gather_mode 0: NumPy take_along_axis, 1: NumPy take);
+// pad_store writes into a buffer whose innermost rows are pad_size elements longer than the value's (the output is
+// that larger buffer); one_hot's depth is a one-element shape; element_any gives one fp32 value, the maximum of x.
+dvm_obj *dvm_rt_global_access(dvm_rt *rt, dvm_shape *shape, int dtype);
+dvm_obj *dvm_rt_gather_load(dvm_rt *rt, dvm_shape *shape, dvm_obj *index, int dtype, int axis, int gather_mode);
+dvm_obj *dvm_rt_pad_store(dvm_rt *rt, dvm_obj *x, long long pad_size);
+dvm_obj *dvm_rt_one_hot(dvm_rt *rt, dvm_obj *indices, dvm_shape *depth, int axis, double on_value, double off_value, int dtype);
+dvm_obj *dvm_rt_element_any(dvm_rt *rt, dvm_obj *x);
 int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store);
 // Kernel::SetStoreTemp / SetLoadBind / SpecNext (include/dvm.h:352-353, 544 of the reference; KernelPy set_store_temp /
 // set_load_bind, include/dvm_py.h:207-208, RtKernelPy spec_next): a Store that is no output of the kernel, a Load that

@@ -293,6 +293,65 @@ class OracleKernel:
         self.stores.append(v)
         return v
 
+    # Gathers, one-hot, padded stores, element_any (include/dvm.h:284,297-307,344,482-496 of the reference; expected
+    # values of tests/ut/test_gather_load.py, test_onehot.py:22-38, test_pad.py, test_element_any.py):
+    #  * gather_mode 0: out[i0..in] = data[i0 .. index[i0..in] (at `axis`) .. in] (NumPy take_along_axis), gather_mode 1:
+    #    the index's dims replace `axis` (NumPy take); a negative index counts from the end of the axis. What an index
+    #    outside [-n, n) reads is not defined by the reference; the product clips it into the axis and so does this.
+    #  * one_hot: a dim of extent depth at position axis, on_value where the position equals the index, off_value
+    #    elsewhere (an index outside [0, depth) matches no position).
+    #  * pad_store: the value written into the first columns of a zero-filled buffer whose innermost rows are pad
+    #    elements longer.
+    #  * element_any: the maximum over every element, as one fp32 value of shape [1].
+    def global_access(self, array, dtype=None):
+        return self.load(array, "int32" if dtype is None else dtype)
+
+    def gather_load(self, data, index, axis=0, dtype=None, gather_mode=0):
+        src = self.load(data, dtype)
+        n = src.a.shape[axis]
+        ix = index.a.astype(np.int64)
+        ix = np.clip(np.where(ix < 0, ix + n, ix), 0, n - 1)
+        ax = axis % src.a.ndim
+        if gather_mode == 1:
+            out = np.empty(src.a.shape[:ax] + ix.shape + src.a.shape[ax + 1:], src.a.dtype)
+            for pos in np.ndindex(*ix.shape):
+                out[(slice(None),) * ax + pos] = src.a[(slice(None),) * ax + (int(ix[pos]),)]
+        else:
+            out = np.empty(ix.shape, src.a.dtype)
+            for pos in np.ndindex(*ix.shape):
+                at = list(pos)
+                at[ax] = int(ix[pos])
+                out[pos] = src.a[tuple(at)]
+        return OVal(out, src.t)
+
+    def one_hot(self, indices, depth, axis, on_value, off_value, dtype):
+        t = _tid(dtype)
+        ix = indices.a
+        ax = axis if axis >= 0 else ix.ndim + axis + 1
+        shape = ix.shape[:ax] + (int(depth),) + ix.shape[ax:]
+        np_t = np.int32 if t == I32 else np.float32
+        out = np.full(shape, self._enc(off_value, t), np_t)
+        on = self._enc(on_value, t)
+        for pos in np.ndindex(*ix.shape):
+            i = int(ix[pos])
+            if 0 <= i < depth:
+                out[pos[:ax] + (i,) + pos[ax:]] = on
+        return OVal(out, t)
+
+    def pad_store(self, x, pad):
+        out = np.zeros(x.a.shape[:-1] + (x.a.shape[-1] + int(pad),), x.a.dtype)
+        out[..., :x.a.shape[-1]] = x.a
+        v = OVal(out, x.t)
+        self.stores.append(v)
+        return v
+
+    def element_any(self, x):
+        assert x.t == F32, "element_any needs fp32 input"
+        return OVal(reduce_f32(1, x.a, list(range(x.a.ndim)), False).reshape(1), F32)
+
+    def clear_store_memory(self, store):
+        pass
+
     def full(self, scalar, shape, dtype):
         t = _tid(dtype)
         if t == BOOL:

@@ -658,3 +658,76 @@ def test_int64_graph_lowers_to_int32_words_without_a_gpu():
     for refuse in (lambda: t.mul(x, y), lambda: t.abs(x), lambda: t.sum(x, (0,), True)):
         with pytest.raises(RuntimeError):
             refuse()
+
+
+def test_gather_onehot_pad_any_compile_without_a_gpu():
+    # OneHot compares the indices with an operand that has no memory behind it (the positions along the new dim);
+    # GatherLoad turns the index into an element offset (wrapped into the axis, times its stride) added to the
+    # operand's own; PadStore is a store through the strides of the longer rows; ElemAny is a max over every dim
+    t = Tester("vector", run_mode="das")
+    ix = t.load(np.zeros([40, 16], np.int32))
+    t.store(t.mul(t.one_hot(ix, 20, 1, 2.0, 0.0, "float32"), t.load(np.zeros([40, 20, 16], np.float32))))
+    t.codegen()
+    dump, das = t.dump(), t.das()
+    assert "OneHot<1>.fp32" in dump and "[40,20,16]" in dump, dump
+    assert t.num_launches() == 1 and "positions @0x0 bcast k[0,1,0]" in das and "CmpEq.int32 acc, m1" in das, das
+    assert "broadcast_s acc, #0x00000000" in das and "select acc, #0x40000000" in das, das
+
+    t = Tester("vector", run_mode="das")
+    src = np.zeros([16, 128, 256], np.float16)
+    y = t.gather_load(src, t.global_access(np.zeros([9, 33], np.int32)), axis=1, gather_mode=1)
+    t.store(t.add(y, 0.25))
+    t.codegen()
+    dump, das = t.dump(), t.das()
+    assert "GatherLoad<1, gather_mode(1)>.fp16" in dump and "[16,9,33,256]" in dump, dump
+    assert "WrapIndex.int32 acc, #0x00000080" in das and "Mul.int32 acc, #0x00000100" in das and "gather_load.fp16 acc, m1 + acc" in das, das
+    assert "k[1,0,32768]" in das, das  # the source's strides seen from the result: nothing along the index's dims
+
+    t = Tester("vector", run_mode="das")
+    o = t.pad_store(t.abs(t.load(np.zeros([200, 111], np.float32))), 139)
+    t.codegen()
+    assert "k[1,250]" in t.das(), t.das()
+    assert t.output(o).shape == (200, 250)
+
+    t = Tester("vector", run_mode="das")
+    t.store(t.element_any(t.abs(t.load(np.zeros([127, 127], np.float32)))))
+    t.codegen()
+    assert "ReduceMax.fp32" in t.dump() and "[1]" in t.dump() and "reduce_max r0" in t.das()
+
+    # what is refused when the graph is built or its shapes are known
+    t = Tester("vector", run_mode="das")
+    with pytest.raises(RuntimeError):
+        t.one_hot(t.load(np.zeros([4], np.float32)), 3, 0, 1.0, 0.0, "float32")      # indices have to be int32
+    with pytest.raises(RuntimeError):
+        t.gather_load(np.zeros([4, 4], np.float32), t.load(np.zeros([4], np.float32)), axis=0, gather_mode=1)
+    with pytest.raises(RuntimeError):
+        t.element_any(t.load(np.zeros([4], np.float16)))
+    t = Tester("vector", run_mode="das")
+    t.store(t.gather_load(np.zeros([4, 4], np.float32), t.global_access(np.zeros([3, 9], np.int32)), axis=0))
+    with pytest.raises(RuntimeError):  # an element gather's index may not be wider than the source in the other dims
+        t.codegen()
+
+
+def test_clone_carries_gathers_onehots_padded_stores_and_element_any():
+    src, idx, lab = np.zeros([50, 24], np.float32), np.zeros([7], np.int32), np.zeros([7], np.int32)
+
+    def build(t):
+        i, l = t.global_access(idx), t.load(lab)
+        g = t.gather_load(src, i, axis=0, gather_mode=1)
+        oh = t.one_hot(l, 24, 1, 1.0, 0.0, "float32")
+        o1 = t.pad_store(t.mul(g, oh), 8)
+        o2 = t.store(t.element_any(t.abs(g)))
+        return i, l, g, o1, o2
+    t = Tester("split", run_mode="das")
+    i, l, g, o1, o2 = build(t)
+    t.codegen()
+    t2 = Tester("split", run_mode="das")
+    i2, l2, g2, p1, p2 = t2.clone(t, [i, l, g, o1, o2])
+    t2.input(i2, idx)
+    t2.input(l2, lab)
+    t2.input(g2, src)
+    t2.codegen()
+    assert p1.shape() == o1.shape() == (7, 24) and p2.shape() == (1,)
+    strip = lambda d: "\n".join(x for x in d.splitlines() if "@0x" not in x)
+    assert strip(t2.das()) == strip(t.das()), t2.das()
+    assert "r[1,32]" in t2.das() and "gather_load.fp32" in t2.das() and "positions" in t2.das(), t2.das()

@@ -320,3 +320,60 @@ def test_values_of_rank_zero_keep_their_rank():
     assert k.output(k.store(m)).shape == () and k.output(k.store(y)).shape == ()
     assert float(k.output(k.store(y))) == 4.0
     assert k.output(k.store(k.add(x, y))).shape == (5,)
+
+
+def _onehot_by_reference_rule(indices, depth, axis, on_value, off_value):
+    """The expectation the reference's own test builds (tests/ut/test_onehot.py:22-38): indices seen as [outer, inner]
+    around the new dim, out[x, indices[x, y], y] = on_value in a buffer filled with off_value."""
+    axis = axis if axis >= 0 else indices.ndim + axis + 1
+    outer = int(np.prod(indices.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(indices.shape[axis:], dtype=np.int64))
+    ix = indices.reshape(outer, inner)
+    out = np.full((outer, depth, inner), off_value, np.int32 if isinstance(on_value, int) else np.float32)
+    for x in range(outer):
+        for y in range(inner):
+            out[x, ix[x, y], y] = on_value
+    return out.reshape(indices.shape[:axis] + (depth,) + indices.shape[axis:])
+
+
+def test_gather_onehot_pad_any_against_numpy_and_the_reference_rule():
+    rng = np.random.default_rng(11)
+    k = OracleKernel()
+    # one_hot against the rule of the reference's test, every axis position, both value classes
+    for shape, depth in [((5,), 7), ((4, 6), 5), ((2, 3, 4), 3)]:
+        ix = rng.integers(0, depth, shape).astype(np.int32)
+        for axis in list(range(len(shape) + 1)) + [-1]:
+            got = k.output(k.one_hot(k.load(ix), depth, axis, 2.0, 0.5, "float32"))
+            assert np.array_equal(got, _onehot_by_reference_rule(ix, depth, axis, 2.0, 0.5))
+            got = k.output(k.one_hot(k.load(ix), depth, axis, 3, -1, "int32"))
+            assert got.dtype == np.int32 and np.array_equal(got, _onehot_by_reference_rule(ix, depth, axis, 3, -1))
+    # an index outside [0, depth) matches no position; on / off are rounded to the result type
+    got = k.output(k.one_hot(k.load(np.array([-1, 0, 9], np.int32)), 4, 1, 1.0, 0.0, "float32"))
+    assert np.array_equal(got, np.array([[0, 0, 0, 0], [1, 0, 0, 0], [0, 0, 0, 0]], np.float32))
+    got = k.output(k.one_hot(k.load(np.array([1], np.int32)), 2, 0, 0.1, 0.3, "float16"))
+    assert got.dtype == np.float16 and np.array_equal(got, np.array([[0.3], [0.1]], np.float16))
+    # gathers against NumPy's take / take_along_axis, negative indices included (tests/ut/test_gather_load.py:33-75)
+    for src_shape, ix_shape, axis in [((6, 5), (7,), 0), ((3, 8, 4), (2, 5), 1), ((2, 4, 6), (9,), -1), ((2, 3, 5, 4), (3, 2), 2)]:
+        x = rng.normal(0, 1, src_shape).astype(np.float32)
+        n = src_shape[axis]
+        ix = rng.integers(-n, n, ix_shape).astype(np.int32)
+        got = k.output(k.gather_load(x, k.global_access(ix), axis=axis, gather_mode=1))
+        assert np.array_equal(got, np.take(x, ix, axis=axis))
+        along_shape = list(src_shape)
+        along_shape[axis] = 3
+        ia = rng.integers(-n, n, along_shape).astype(np.int32)
+        got = k.output(k.gather_load(x, k.global_access(ia), axis=axis))
+        assert np.array_equal(got, np.take_along_axis(x, ia.astype(np.int64), axis=axis))
+    # indices past either end are clipped into the axis
+    x = np.arange(5, dtype=np.float32)
+    got = k.output(k.gather_load(x, k.global_access(np.array([7, -9, 4, -5], np.int32)), axis=0, gather_mode=1))
+    assert np.array_equal(got, np.array([4, 0, 4, 0], np.float32))
+    # pad_store (src/ops.cc:1399-1412): rows pad elements longer, zeros in the padding
+    v = rng.normal(0, 1, (3, 4)).astype(np.float32)
+    got = k.output(k.pad_store(k.load(v), 5))
+    assert got.shape == (3, 9) and np.array_equal(got[:, :4], v) and not got[:, 4:].any()
+    # element_any: 1 when any element of a 0 / 1 mask is set (tests/ut/test_element_any.py:22-50)
+    m = np.zeros((9, 9), np.float32)
+    assert k.output(k.element_any(k.load(m))).tolist() == [0.0]
+    m[3, 7] = 1
+    assert k.output(k.element_any(k.load(m))).tolist() == [1.0]
