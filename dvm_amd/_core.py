@@ -68,6 +68,7 @@ def _load():
         "dvm_rt_pad_store": (vp, [vp, vp, ctypes.c_longlong]),
         "dvm_rt_one_hot": (vp, [vp, vp, vp, ci, ctypes.c_double, ctypes.c_double, ci]),
         "dvm_rt_element_any": (vp, [vp, vp]),
+        "dvm_rt_grouped_matmul": (vp, [vp, vp, vp, ci, ci, vp, vp, ci, ci]),
         "dvm_rt_slice": (vp, [vp, vp, vp, vp]),
         "dvm_rt_slice_dim": (vp, [vp, vp, ci, vp, vp]),
         "dvm_rt_split": (ci, [vp, vp, ci, ctypes.c_longlong, cs, ctypes.POINTER(vp)]),
@@ -404,6 +405,14 @@ class Kernel:
     def matmul(self, lhs, rhs, trans_a, trans_b, bias=None):
         return self._wrap(_lib.dvm_rt_matmul(self._rt, lhs._h, rhs._h, int(bool(trans_a)), int(bool(trans_b)),
                                              bias._h if bias is not None else None))
+
+    def grouped_matmul(self, lhs, rhs, trans_a, trans_b, bias, group_list, group_type, group_list_type=0):
+        """One product per group (KernelPy.grouped_matmul). group_type 0: the groups are ranges of lhs's rows, rhs is
+        [groups, k, n], the result [m, n]; 2: ranges of the k axis, the result [groups, m, n]. group_list: a load of
+        int64 values, the ranges' upper bounds (group_list_type 0) or sizes (1), read on the device at every launch."""
+        return self._wrap(_lib.dvm_rt_grouped_matmul(self._rt, lhs._h, rhs._h, int(bool(trans_a)), int(bool(trans_b)),
+                                                     bias._h if bias is not None else None, group_list._h,
+                                                     int(group_type), int(group_list_type)))
 
     # -- introspection --
     def das(self):

@@ -331,7 +331,18 @@ static int launch_checked(const VmParam &p, uint32_t block_dim, uint32_t threads
         c->a_addr == 0 || c->b_addr == 0 || (c->dtype != VDT_F16 && c->dtype != VDT_BF16)) {
       return static_cast<int>(hipErrorInvalidValue);
     }
-    if (c->fast && (c->lda >= (1u << 22) || c->ldb >= (1u << 22) || c->k % 64 != 0 || c->k == 0 || c->lda % 8 != 0 || c->ldb % 8 != 0 ||
+    if (c->group_mode != VCG_NONE) {
+      // a grouped product: one inner batch axis (the groups), its list in memory, its table of bounds behind the tile
+      // buffers in local memory, and the whole k axis per workgroup
+      const bool rows = c->group_mode == VCG_M_BOUND || c->group_mode == VCG_M_SIZE;
+      if (c->group_mode > VCG_K_SIZE || c->group_addr == 0 || (c->group_addr & (c->group_i32 ? 3u : 7u)) != 0 || c->nb0 != 1 ||
+          c->nb1 > DVM_CUBE_MAX_GROUPS || (c->epi_flags & (VCF_SPLITK_PARTIAL | VCF_SPLITK_COMBINE)) != 0 ||
+          lds_bytes < DVM_CUBE_LDS_BYTES(bt) + 8u * c->nb1 || (rows && (c->a_sb0 != 0 || c->a_sb1 != 0))) {
+        return static_cast<int>(hipErrorInvalidValue);
+      }
+    }
+    const bool k_groups = c->group_mode == VCG_K_BOUND || c->group_mode == VCG_K_SIZE;
+    if (c->fast && (c->lda >= (1u << 22) || c->ldb >= (1u << 22) || (c->k % 64 != 0 && !k_groups) || c->k == 0 || c->lda % 8 != 0 || c->ldb % 8 != 0 ||
                     (c->a_addr & 15u) != 0 || (c->b_addr & 15u) != 0)) {
       return static_cast<int>(hipErrorInvalidValue);
     }

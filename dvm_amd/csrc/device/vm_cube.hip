@@ -195,7 +195,7 @@ __device__ __attribute__((noinline)) void stage_generic(uint16_t *tile, uint64_t
       vu4 v = {0u, 0u, 0u, 0u};
       if (gr < rows && gk < kext) {
         const uint64_t idx = static_cast<uint64_t>(gr) * ld + gk;
-        if (vec_ok != 0u && gk + 8u <= kext) {
+        if (vec_ok != 0u && (gk & 7u) == 0u && gk + 8u <= kext) {  // (a group's k range may start anywhere)
           v = *reinterpret_cast<const DVM_GLOBAL vu4 *>(src + idx);
         } else {
 #pragma unroll
@@ -1179,14 +1179,64 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
   }
   uint16_t *lds = reinterpret_cast<uint16_t *>(lds_raw);
   float *dump = reinterpret_cast<float *>(lds_raw);
+  // A grouped product (VCG_*): the upper bounds of the groups' ranges, read once from the list in memory (its sizes
+  // summed up, every value clipped into the axis the groups split), behind the tile buffers in local memory. Groups of
+  // rows get a second table behind the first: how many rows of tiles the groups up to and including g touch (a tile a
+  // bound runs through counts for both sides), so that the work items are exactly the tiles that have rows to store.
+  uint32_t *gtab = reinterpret_cast<uint32_t *>(reinterpret_cast<char *>(lds_raw) + DVM_CUBE_LDS_BYTES(static_cast<uint32_t>(BM)));
+  const uint32_t gmode = COMB ? static_cast<uint32_t>(VCG_NONE) : h.group_mode;
+  const bool g_rows = gmode == VCG_M_BOUND || gmode == VCG_M_SIZE;
+  uint32_t *gpre = gtab + h.nb1;
+  if (gmode != VCG_NONE) {
+    const bool sizes = gmode == VCG_M_SIZE || gmode == VCG_K_SIZE;
+    const uint32_t limit = g_rows ? h.m : h.k, groups = h.nb1;
+    auto entry = [&](uint32_t i) -> uint32_t {
+      long long v = h.group_i32 ? static_cast<long long>(reinterpret_cast<const DVM_GLOBAL int32_t *>(h.group_addr)[i])
+                                : reinterpret_cast<const DVM_GLOBAL long long *>(h.group_addr)[i];
+      v = v < 0 ? 0 : v;
+      return v > static_cast<long long>(limit) ? limit : static_cast<uint32_t>(v);
+    };
+    // the first wave sums values up, 64 at a time (an inclusive scan across its lanes, the total carried on), never past `cap`
+    auto running_sum = [&](uint32_t *table, auto value, uint32_t cap) {
+      if (threadIdx.x >= 64u) return;
+      uint32_t carry = 0;
+      for (uint32_t c0 = 0; c0 < groups; c0 += 64u) {
+        const uint32_t i = c0 + threadIdx.x;
+        uint32_t v = i < groups ? value(i) : 0u;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+          const uint32_t up = __shfl_up(v, d, 64);
+          if (static_cast<int>(threadIdx.x) >= d) v = v + up < cap ? v + up : cap;  // (both at most cap, cap below 2^31)
+        }
+        v = v + carry < cap ? v + carry : cap;
+        if (i < groups) table[i] = v;
+        carry = __shfl(v, 63, 64);
+      }
+    };
+    if (!sizes) {
+      for (uint32_t i = threadIdx.x; i < groups; i += NTHR) gtab[i] = entry(i);
+    } else {
+      running_sum(gtab, entry, limit);
+    }
+    __syncthreads();
+    if (g_rows) {
+      running_sum(gpre, [&](uint32_t g) -> uint32_t {
+        const uint32_t lo = g != 0u ? gtab[g - 1u] : 0u, hi = gtab[g];
+        return hi > lo ? (hi + BM - 1u) / BM - lo / BM : 0u;
+      }, 0x7fffffffu);
+      __syncthreads();
+    }
+  }
   // [A buffer 0 | A buffer 1 | B buffer 0 | B buffer 1], offsets in elements
   constexpr uint32_t kABuf = BM * BK, kBBuf = BN * BK, kBBase = 2 * kABuf;
 
   const uint32_t tid = threadIdx.x;
   const uint32_t wave = tid >> 6, lane = tid & 63u;
   const uint32_t wm = wave >> 1, wn = wave & 1u;
-  const uint32_t tiles_per_batch = h.tiles_m * h.tiles_n;
-  const uint32_t n_tiles = tiles_per_batch * h.nb0 * h.nb1;
+  // (groups of rows: the rows of tiles the groups touch, one after the other, stand in for the tile rows of one matrix)
+  const uint32_t tile_rows = g_rows ? uni(gpre[h.nb1 - 1u]) : h.tiles_m;
+  const uint32_t tiles_per_batch = tile_rows * h.tiles_n;
+  const uint32_t n_tiles = g_rows ? tiles_per_batch : tiles_per_batch * h.nb0 * h.nb1;
   // Split k (VCF_SPLITK_*): the first launch has k_split workgroups per tile, each walks k_chunk of the k axis and
   // leaves its fp32 accumulators in the partials buffer, register by register as the lanes hold them; the second
   // launch has one workgroup per tile, adds the partials in ascending k order and runs the epilogue.
@@ -1211,24 +1261,58 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
     // order; the order itself walks 8-tile-wide column bands row by row, which makes the 32 tiles an XCD has
     // in flight a 4 x 8 block (12 operand panels to fetch instead of 18 for two full rows of 16).
     uint32_t t = t0;
-    if ((n_work & 7u) == 0 && gridDim.x == n_work) t = (t0 & 7u) * (n_work >> 3) + (t0 >> 3);
+    if ((n_work & 7u) == 0 && gridDim.x >= n_work) t = (t0 & 7u) * (n_work >> 3) + (t0 >> 3);
     const uint32_t ksplit = t / n_tiles;  // which part of the k axis (0 unless the launch writes partials)
     t -= ksplit * n_tiles;
     const uint32_t tile_id = t;
-    const uint32_t k_lo = ksplit * h.k_chunk;
-    const uint32_t k_hi = split_part ? (k_lo + h.k_chunk < h.k ? k_lo + h.k_chunk : h.k) : h.k;
-    const uint32_t nk = (k_hi - k_lo + BK - 1) / BK;
+    uint32_t k_lo = ksplit * h.k_chunk;
+    uint32_t k_hi = split_part ? (k_lo + h.k_chunk < h.k ? k_lo + h.k_chunk : h.k) : h.k;
     const uint32_t batch = t / tiles_per_batch, tt = t % tiles_per_batch;
-    const uint32_t bi0 = batch / h.nb1, bi1 = batch % h.nb1;
-    const uint32_t band = tt / (h.tiles_m * 8u), in_band = tt % (h.tiles_m * 8u);
+    uint32_t bi0 = batch / h.nb1, bi1 = batch % h.nb1;
+    const uint32_t band = tt / (tile_rows * 8u), in_band = tt % (tile_rows * 8u);
     const uint32_t band_w = h.tiles_n - band * 8u < 8u ? h.tiles_n - band * 8u : 8u;
-    const uint32_t tm = in_band / band_w, tn = band * 8u + in_band % band_w;
+    uint32_t tm = in_band / band_w;
+    const uint32_t tn = band * 8u + in_band % band_w;
+    if (g_rows) {
+      // which group the row of tiles belongs to (the first whose running count exceeds its number), and which of the
+      // group's rows of tiles it is
+      uint32_t lo = 0, hi = h.nb1 - 1u;
+      while (lo < hi) {
+        const uint32_t mid = (lo + hi) >> 1;
+        if (uni(gpre[mid]) > tm) hi = mid;
+        else lo = mid + 1u;
+      }
+      bi0 = 0;
+      bi1 = lo;
+      const uint32_t first_row = lo != 0u ? uni(gtab[lo - 1u]) : 0u;
+      tm = first_row / BM + (tm - (lo != 0u ? uni(gpre[lo - 1u]) : 0u));
+    }
     // A ragged tile at the bottom or right edge is moved back inside the output (it overlaps its neighbour) so that
     // it can take the vector path like any full tile; its epilogue covers only the rows from m_lo and the columns
     // from n_lo on, the part no other tile writes. (Columns move in whole 8-element slabs only; an operand whose
     // rows are the contiguous axis needs the new origin 16-byte aligned.)
     uint32_t m0 = tm * BM, n0 = tn * BN;
-    const uint32_t m_lo = m0, n_lo = n0;
+    uint32_t m_lo = m0, m_end = h.m;  // the rows of the output this tile stores
+    const uint32_t n_lo = n0;
+    bool k_fast = true;
+    if (gmode != VCG_NONE) {
+      const uint32_t g_lo = bi1 != 0u ? uni(gtab[bi1 - 1u]) : 0u;
+      uint32_t g_hi = uni(gtab[bi1]);
+      g_hi = g_hi > g_lo ? g_hi : g_lo;
+      if (gmode == VCG_M_BOUND || gmode == VCG_M_SIZE) {
+        // the rows of the tile that belong to this group; none: the tile is another group's
+        const uint32_t t_hi = m0 + BM < h.m ? m0 + BM : h.m;
+        m_lo = m0 > g_lo ? m0 : g_lo;
+        m_end = t_hi < g_hi ? t_hi : g_hi;
+        if (m_lo >= m_end) continue;
+      } else {
+        // the group's part of the k axis; the vector path takes it when it is whole steps from an aligned start
+        k_lo = g_lo;
+        k_hi = g_hi;
+        k_fast = (k_lo & 7u) == 0u && k_hi > k_lo && ((k_hi - k_lo) & 63u) == 0u;
+      }
+    }
+    const uint32_t nk = (k_hi - k_lo + BK - 1) / BK;
     if (h.fast) {
       if (m0 + BM > h.m && h.m >= BM && (A_KC || (h.m & 7u) == 0)) m0 = h.m - BM;
       if (n0 + BN > h.n && h.n >= BN && (h.n & 7u) == 0) n0 = h.n - BN;
@@ -1285,7 +1369,7 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
           }
       }
     } else {
-    if (h.fast && (m0 + BM <= h.m || a_clamps) && (n0 + BN <= h.n || b_clamps)) {
+    if (h.fast && k_fast && (m0 + BM <= h.m || a_clamps) && (n0 + BN <= h.n || b_clamps)) {
      if constexpr (RING) {
       tile_loop_ring<IS_BF16, A_KC, B_KC, WM>(acc, lds, a_org, b_org, h.lda, h.ldb, (k_hi - k_lo) / SK, tid);
      } else {
@@ -1521,11 +1605,11 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
         }
       }
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<BM, BN, TM, WM, D16K>(tile16, prog32, ea, m0, n0, 0, h.m, h.n, m_lo, n_lo)) {
+      if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<BM, BN, TM, WM, D16K>(tile16, prog32, ea, m0, n0, 0, m_end, h.n, m_lo, n_lo)) {
         if (h.epi_flags & VCF_SLIM) {
-          epilogue_pass_body<BM, BN, TM, WM, true, D16K>(tile16, prog32, ea, m0, n0, 0, h.m, h.n, m_lo, n_lo);
+          epilogue_pass_body<BM, BN, TM, WM, true, D16K>(tile16, prog32, ea, m0, n0, 0, m_end, h.n, m_lo, n_lo);
         }
-        else epilogue_pass<BM, BN, TM, WM, false, D16K>(tile16, prog32, ea, m0, n0, 0, h.m, h.n, m_lo, n_lo);
+        else epilogue_pass<BM, BN, TM, WM, false, D16K>(tile16, prog32, ea, m0, n0, 0, m_end, h.n, m_lo, n_lo);
       }
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
       continue;
@@ -1549,9 +1633,9 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       // before the next dump): they wait for this wave's local-memory operations and not, as __syncthreads() would,
       // for its stores to memory as well, which stay in flight under the next pass and the next tile's loop.
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-      if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<PROWS, BN, TM, WM, 0>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo)) {
-        if (h.epi_flags & VCF_SLIM) epilogue_pass<PROWS, BN, TM, WM, true, 0>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
-        else epilogue_pass<PROWS, BN, TM, WM, false, 0>(dump, prog32, ea, m0, n0, ps, h.m, h.n, m_lo, n_lo);
+      if (!(h.epi_flags & VCF_PLAIN_STORE) || !epilogue_plain_pass<PROWS, BN, TM, WM, 0>(dump, prog32, ea, m0, n0, ps, m_end, h.n, m_lo, n_lo)) {
+        if (h.epi_flags & VCF_SLIM) epilogue_pass<PROWS, BN, TM, WM, true, 0>(dump, prog32, ea, m0, n0, ps, m_end, h.n, m_lo, n_lo);
+        else epilogue_pass<PROWS, BN, TM, WM, false, 0>(dump, prog32, ea, m0, n0, ps, m_end, h.n, m_lo, n_lo);
       }
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }

@@ -432,6 +432,19 @@ dvm_obj *dvm_rt_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int 
       static_cast<dvm_obj *>(nullptr));
 }
 
+dvm_obj *dvm_rt_grouped_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int trans_b, dvm_obj *bias, dvm_obj *group_list,
+                               int group_type, int group_list_type) {
+  return Guard(
+      [&]() {
+        if (group_type < 0 || group_type >= kGroupTypeEnd || group_list_type < 0 || group_list_type >= kEnd) {
+          throw std::runtime_error("DVM EXCEPTION. reason: grouped_matmul: no such group type or list type");
+        }
+        return Handle(rt->kernel.GroupedMatMul(Obj(lhs), Obj(rhs), trans_a != 0, trans_b != 0, Obj(bias), Obj(group_list),
+                                               static_cast<GmmSplitType>(group_type), static_cast<GmmListType>(group_list_type)));
+      },
+      static_cast<dvm_obj *>(nullptr));
+}
+
 // RtKernelPy::Clone (src/pybind_api.cc:923-993): rebuilds `base`'s graph in `rt`, with shapes, axis lists and
 // scalars of its own, and translates the n handles in `items` (kinds: 0 operator, 1 shape, 2 scalar) to the
 // clone's handles in `out`.

@@ -397,6 +397,7 @@ class Compiler {
   bool cube_mode_ = false;
   VCubeMem cmems_[DVM_CUBE_MAXMEM];
   const NDObject *cube_out_ = nullptr;
+  int gmm_bias_node_ = -1;  // the [groups, n] bias of a grouped matmul (its row goes with the group, not with the output's dims)
   bool SimpleOperand(int v);
   void EmitOperandInsn(uint32_t op, uint32_t sub, uint32_t rnd, int v);
   void EmitValue(int v);

@@ -86,7 +86,10 @@ std::string &VKernel::DumpGraph(bool ref_shapes) {
       case kObjConcatPart: os << "ConcatPart"; break;
       case kObjConcat: os << "Concat"; break;
       case kObjCopy: os << "Copy"; break;
-      case kObjMatMul: os << "MatMul" << (o->trans_a ? "T" : "N") << (o->trans_b ? "T" : "N"); break;
+      case kObjMatMul:
+        os << (o->gmm_type != 0 ? "GroupedMatMul" : "MatMul") << (o->trans_a ? "T" : "N") << (o->trans_b ? "T" : "N");
+        if (o->gmm_type != 0) os << "<group_type=" << (o->gmm_type == 1 ? 0 : 2) << ", group_list_type=" << (o->gmm_sizes ? 1 : 0) << ", list=%" << o->group_list->id << ">";
+        break;
       case kObjPack64: os << "Pack"; break;
       case kObjOneHot: os << "OneHot<" << o->slice_dim << ">"; break;
       case kObjGather: os << "GatherLoad<" << o->slice_dim << ", gather_mode(" << static_cast<int>(o->op) << ")>"; break;
@@ -232,6 +235,10 @@ std::string &VKernel::DisAssemble() {
       if (c->epi_flags & VCF_DUMP16) os << " tile-as-16-bit";
       if (c->epi_flags & VCF_SPLITK_PARTIAL) os << " split-k partials " << c->k_split << " x " << c->k_chunk;
       if (c->epi_flags & VCF_SPLITK_COMBINE) os << " split-k sum of " << c->k_split;
+      if (c->group_mode != VCG_NONE) {
+        static const char *gm[] = {"", "rows by bounds", "rows by sizes", "k by bounds", "k by sizes"};
+        os << " groups=" << c->nb1 << " (" << gm[c->group_mode <= VCG_K_SIZE ? c->group_mode : 0] << ", " << (c->group_i32 ? "int32" : "int64") << " list)";
+      }
       os << "\n";
       const VCubeMem *cm = reinterpret_cast<const VCubeMem *>(p.blob.w + c->mem_off);
       for (uint32_t i = 0; i < c->n_mem; ++i) {

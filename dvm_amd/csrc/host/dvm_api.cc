@@ -643,6 +643,9 @@ void Kernel::Clone(const Kernel &base, CloneHelper &helper) {
       c->aux_ref = o->aux_ref != nullptr ? helper.GetClone(o->aux_ref) : nullptr;
     }
     c->elem_any = o->elem_any;
+    c->gmm_type = o->gmm_type;
+    c->gmm_sizes = o->gmm_sizes;
+    c->group_list = o->group_list != nullptr ? helper.GetClone(o->group_list) : nullptr;
     c->pad_size = o->pad_size;
     c->scalar2.imm = o->scalar2.imm;
     c->scalar2.ref = o->scalar2.ref != nullptr ? helper.GetClone(o->scalar2.ref) : nullptr;
@@ -1027,8 +1030,21 @@ NDObject *Kernel::ElemAny(NDObject *input) {
   o->elem_any = true;
   return o;
 }
-NDObject *Kernel::GroupedMatMul(NDObject *, NDObject *, bool, bool, NDObject *, NDObject *, GmmSplitType, GmmListType) {
-  Unsupported("GroupedMatMul");
+// GroupedMatMul (include/dvm.h:510-522, src/ops_m.cc:698-800 of the reference; tests/ut/test_gmm.py): the groups are
+// ranges of the rows of lhs (kSplit_M: rhs is [groups, k, n], the result [m, n]) or of the k axis (kSplit_K: the result
+// is [groups, m, n]); the list holds their upper bounds or their sizes and is read on the device at every launch.
+NDObject *Kernel::GroupedMatMul(NDObject *lhs, NDObject *rhs, bool trans_a, bool trans_b, NDObject *bias, NDObject *group_list,
+                                GmmSplitType group_type, GmmListType group_list_type) {
+  if (group_type != kSplit_M && group_type != kSplit_K) Unsupported("GroupedMatMul over the n axis");
+  if (group_list == nullptr || group_list->kind != kObjLoad || group_list->strided ||
+      (group_list->type_id_ != kInt64 && group_list->type_id_ != kInt32)) {
+    Throw("GroupedMatMul needs its group list as a plain Load of int64 or int32 values");
+  }
+  NDObject *o = MatMul(lhs, rhs, trans_a, trans_b, bias);
+  o->gmm_type = group_type == kSplit_M ? 1 : 2;
+  o->gmm_sizes = group_list_type == kListSize;
+  o->group_list = group_list;
+  return o;
 }
 NDObject *Kernel::_AllReduce(int, NDObject *, const Comm *) { Unsupported("AllReduce (single-GPU backend)"); }
 NDObject *Kernel::AllGather(NDObject *, const Comm *) { Unsupported("AllGather (single-GPU backend)"); }

@@ -24,7 +24,13 @@ int Compiler::CubeMemIndex(int v) {
   m.dtype = MemDType(n.dtype);
   const int R = cube_out_->rank();
   int64_t stride = 1;
-  for (int d = n.rank - 1; d >= 0; --d) {
+  if (v == gmm_bias_node_) {
+    // the bias of a grouped product is [groups, n]: one row per group, and the groups are the kernel's inner batch axis
+    if (n.view != nullptr || n.rank != 2) Fail("the bias of a grouped matmul must be a dense [groups, n] tensor");
+    m.stride_n = 1;
+    m.stride_b1 = static_cast<uint32_t>(n.dims[1]);
+  }
+  for (int d = n.rank - 1; d >= 0 && v != gmm_bias_node_; --d) {
     const int od = d + R - n.rank;
     if (n.dims[d] != 1) {
       if (od < 0 || n.dims[d] != cube_out_->dim(od)) Fail("epilogue operand does not broadcast to the matmul result");
@@ -137,6 +143,8 @@ void Compiler::CompileCube(int a) {
   const int R = mm->rank();
   const int br = R - 2;
   if (br > 2) Fail("matmul with more than two batch dimensions");
+  const int gmm = mm->gmm_type;  // 0: a plain product; 1: groups of rows; 2: groups along k
+  gmm_bias_node_ = -1;
   VCubeHeader h;
   std::memset(&h, 0, sizeof(h));
   h.entry = VE_CUBE;
@@ -149,6 +157,16 @@ void Compiler::CompileCube(int a) {
   h.k = static_cast<uint32_t>(K);
   h.nb0 = br == 2 ? static_cast<uint32_t>(mm->dim(0)) : 1;
   h.nb1 = br >= 1 ? static_cast<uint32_t>(mm->dim(br - 1)) : 1;
+  if (gmm != 0) {
+    // the groups are the inner batch axis: matrix g of B with the rows of group g (the output has no batch axis
+    // then), or the k range of group g into matrix g of the output
+    const int64_t groups = mm->group_list->dim(0);
+    if (groups > static_cast<int64_t>(DVM_CUBE_MAX_GROUPS)) Throw("DVM EXCEPTION. reason: a grouped matmul of more than 2048 groups is not supported by the gfx950 backend");
+    h.nb0 = 1;
+    h.nb1 = static_cast<uint32_t>(groups);
+    h.group_mode = gmm == 1 ? (mm->gmm_sizes ? VCG_M_SIZE : VCG_M_BOUND) : (mm->gmm_sizes ? VCG_K_SIZE : VCG_K_BOUND);
+    h.group_i32 = mm->group_list->type_id_ == kInt32 ? 1 : 0;
+  }
   // An operand is a matrix (or a batch of matrices) walked through a leading dimension and up to two batch strides.
   // A dense tensor gives those from its shape; a strided view (a load with strides, a slice, a permute of a stored
   // value: a sliced weight, the heads-first view of a [batch, seq, heads, dim] tensor, a transposed K) gives them
@@ -187,6 +205,13 @@ void Compiler::CompileCube(int a) {
   bool flip_a = false, flip_b = false;
   operand_layout(an, &flip_a, &h.lda, &h.a_sb0, &h.a_sb1);
   operand_layout(bn, &flip_b, &h.ldb, &h.b_sb0, &h.b_sb1);
+  if (gmm == 1) {  // matrix g of B: its outermost dim, whatever the rank of the output
+    int64_t walk = bn.view != nullptr ? bn.view->vstride_[0] : bn.dims[1] * bn.dims[2];
+    if (walk < 0 || walk >= (1ll << 32)) Fail("stride above 2^32");
+    h.b_sb0 = 0;
+    h.b_sb1 = static_cast<uint32_t>(walk);
+    h.a_sb0 = h.a_sb1 = 0;
+  }
   const bool trans_a = mm->trans_a != flip_a, trans_b = mm->trans_b != flip_b;  // as the operands lie in memory
   h.trans_a = trans_a ? 1 : 0;
   h.trans_b = trans_b ? 1 : 0;
@@ -204,7 +229,7 @@ void Compiler::CompileCube(int a) {
       t.cube_splitk = split;
     }
   } restore_tuning{k_->tuning_, k_->tuning_.cube_tile, k_->tuning_.cube_splitk};
-  if (!k_->tuning_.in_tuner && k_->tuning_.cube_tile < 0 && k_->tuning_.cube_splitk < 0 && K > 0) {
+  if (!k_->tuning_.in_tuner && k_->tuning_.cube_tile < 0 && k_->tuning_.cube_splitk < 0 && K > 0 && gmm == 0) {
     CubeProblem q;
     q.m = M;
     q.n = N;
@@ -221,7 +246,8 @@ void Compiler::CompileCube(int a) {
     }
   }
   // block tile: the largest that still gives most compute units a tile
-  const uint64_t batch = static_cast<uint64_t>(h.nb0) * h.nb1;
+  // (groups of rows: a tile is computed once per group that owns rows of it, so about once: the groups do not multiply the work)
+  const uint64_t batch = gmm == 1 ? 1 : static_cast<uint64_t>(h.nb0) * h.nb1;
   auto tiles = [&](int64_t t) { return static_cast<uint64_t>((M + t - 1) / t) * static_cast<uint64_t>((N + t - 1) / t) * batch; };
   const uint64_t cus = g_system.core_num;
   int64_t bt;
@@ -270,7 +296,7 @@ void Compiler::CompileCube(int a) {
   // paying, plus the time the first launch takes to write the partial tiles (some 4 TB/s over the whole chip).
   uint32_t k_split = 1, k_chunk = 0;
   {
-    const int forced = k_->tuning_.cube_splitk;
+    const int forced = gmm != 0 ? 0 : k_->tuning_.cube_splitk;  // (the k axis of a grouped product is never shared)
     const bool user_tile = k_->tuning_.cube_tile == 256 || k_->tuning_.cube_tile == 128 || k_->tuning_.cube_tile == 64;
     auto parts_of = [&](uint32_t want, uint32_t *chunk) -> uint32_t {  // parts actually made when `want` are asked for
       if (want < 2 || K < 128) return 1;
@@ -329,8 +355,9 @@ void Compiler::CompileCube(int a) {
   if (h.tile == 0 && k_->tuning_.cube_waves != 4) h.tile = 3;
   h.tiles_m = static_cast<uint32_t>((M + bt - 1) / bt);
   h.tiles_n = static_cast<uint32_t>((N + bt - 1) / bt);
-  if (tiles(bt) >= (1ull << 31)) Fail("too many matmul tiles");
-  h.fast = (K % 64 == 0 && K > 0 && h.lda < (1u << 22) && h.ldb < (1u << 22) && h.lda % 8 == 0 && h.ldb % 8 == 0 && h.a_sb0 % 8 == 0 &&
+  if (tiles(bt) * (gmm == 1 ? h.nb1 : 1) >= (1ull << 31)) Fail("too many matmul tiles");
+  // (groups along k: every group's range decides for itself on the device whether it is whole 64-steps from an aligned start)
+  h.fast = ((K % 64 == 0 || gmm == 2) && K > 0 && h.lda < (1u << 22) && h.ldb < (1u << 22) && h.lda % 8 == 0 && h.ldb % 8 == 0 && h.a_sb0 % 8 == 0 &&
             h.a_sb1 % 8 == 0 && h.b_sb0 % 8 == 0 && h.b_sb1 % 8 == 0)
                ? 1
                : 0;
@@ -343,6 +370,14 @@ void Compiler::CompileCube(int a) {
     p.ws_slot = x.ws_slot;
     p.byte_offset = x.view != nullptr ? x.view->view_base_ * static_cast<int64_t>(DTypeSize(x.dtype)) : 0;
     p.role = Program::kPatchCubeOperand;
+    prog_->patches.push_back(p);
+  }
+  if (gmm != 0) {
+    Program::Patch p;
+    p.word = static_cast<uint32_t>(offsetof(VCubeHeader, group_addr) / 8);
+    p.op_id = mm->group_list->id;
+    p.ws_slot = -1;
+    p.role = Program::kPatchPlain;
     prog_->patches.push_back(p);
   }
   // the epilogue: one section over values that all live in fragments
@@ -359,6 +394,7 @@ void Compiler::CompileCube(int a) {
   // the tile loop reads A and B itself: they are no values of the epilogue
   const int bias = nodes_[c].nin > 2 ? nodes_[c].in[2] : -1;
   if (bias >= 0 && nodes_[bias].kind != AK_MEM) Fail("matmul bias must come from memory");
+  if (gmm != 0) gmm_bias_node_ = bias;
   nodes_[c].nin = 0;
   nr_ = 0;
   n_sec_ = 1;
@@ -461,8 +497,15 @@ void Compiler::CompileCube(int a) {
   std::memcpy(prog_->blob.w + h.mem_off, cmems_, sizeof(VCubeMem) * n_mem_);
   std::memcpy(prog_->blob.w + h.code_off, code_.data(), 8 * code_.size());
   prog_->threads = h.tile == 3 ? 512 : 256;
-  prog_->lds_bytes = DVM_CUBE_LDS_BYTES(static_cast<uint32_t>(bt));
+  prog_->lds_bytes = DVM_CUBE_LDS_BYTES(static_cast<uint32_t>(bt)) + (gmm != 0 ? 8u * h.nb1 : 0u);
   prog_->grid = static_cast<uint32_t>(tiles(bt));
+  if (gmm == 1) {
+    // The work items are the tiles that have rows of a group to store, counted on the device from the list: at most
+    // one row of tiles more per group than the matrix has (a tile a bound runs through is computed for both sides).
+    // One workgroup per item that can exist; those past the count leave at once.
+    const uint64_t rows_max = static_cast<uint64_t>(h.tiles_m) + std::min<uint64_t>(h.nb1, static_cast<uint64_t>(M));
+    prog_->grid = static_cast<uint32_t>(std::min<uint64_t>(rows_max * h.tiles_n, 1u << 20));
+  }
   // A short k axis (the scores of an attention, an outer product): a 256 tile is then mostly its start-up (program
   // and header into local memory) and its epilogue, and one workgroup per compute unit that walks the tiles pays the
   // start-up once. Measured on MI355X, fp16: [128,1024,64] x [128,1024,64]^T 148 -> 130 us, 8192 x 8192 x 128

@@ -92,6 +92,12 @@ class NDObject {
   NDObject *in[3] = {nullptr, nullptr, nullptr};
   ScalarOperand scalar;
   ScalarOperand scalar2;           // kObjOneHot: the value where the index does not match
+  // kObjMatMul made by GroupedMatMul (src/ops_m.h:143-159 of the reference): 1 = the groups split the rows of the left
+  // operand (right operand [groups, k, n], result [m, n]), 2 = they split the k axis (result [groups, m, n]);
+  // group_list = the Load of the int64 (or int32) list of bounds (gmm_sizes: of sizes); a bias is [groups, n]
+  uint8_t gmm_type = 0;
+  bool gmm_sizes = false;
+  NDObject *group_list = nullptr;
   bool elem_any = false;           // kObjReduce made by ElemAny: a reduce to one element, result of shape [1]
   int64_t pad_size = -1;           // kObjStore made by PadStore: rows of the buffer are this many elements longer than the value's
   int64_t gather_extent = 0, gather_stride = 0;  // kObjGather: extent and element stride of the gathered dim of the source

@@ -391,6 +391,26 @@ void VKernel::Normalize() {
         const int64_t kb = o->trans_b ? b->dim(rb - 1) : b->dim(rb - 2);
         const int64_t n = o->trans_b ? b->dim(rb - 2) : b->dim(rb - 1);
         if (ka != kb) Throw("matmul inner dimensions differ");
+        if (o->gmm_type != 0) {  // src/ops_m.cc:721-762 of the reference
+          const NDObject *gl = o->group_list;
+          if (gl->rank() != 1) Throw("GroupedMatMul needs a list of one dim");
+          const int64_t groups = gl->dim(0);
+          if (o->gmm_type == 1) {
+            if (ra != 2 || rb != 3 || b->dim(0) != groups) Throw("GroupedMatMul over rows needs lhs [m, k] and rhs [groups, k, n]");
+            o->shape_[0] = m;
+            o->shape_[1] = n;
+            o->own_ref_.size = 2;
+          } else {
+            if (ra != 2 || rb != 2) Throw("GroupedMatMul over the k axis needs lhs [m, k] and rhs [k, n]");
+            o->shape_[0] = groups;
+            o->shape_[1] = m;
+            o->shape_[2] = n;
+            o->own_ref_.size = 3;
+          }
+          const NDObject *bias = o->nin > 2 ? o->in[2] : nullptr;
+          if (bias != nullptr && (bias->rank() != 2 || bias->dim(0) != groups || bias->dim(1) != n)) Throw("GroupedMatMul needs a bias of [groups, n]");
+          break;
+        }
         const size_t ba = ra - 2, bb = rb - 2, br = std::max(ba, bb);
         if (br + 2 > static_cast<size_t>(kMaxRank)) Throw("tensor rank above 10");
         for (size_t i = 0; i < br; ++i) {

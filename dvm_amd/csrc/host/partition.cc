@@ -529,7 +529,7 @@ void Compiler::DetectAttention() {
   for (int i = 0; i < n_; ++i) {
     if (!live_[i]) continue;
     NDObject *m2 = k_->ops_[i];
-    if (m2->kind != kObjMatMul || m2->trans_a || m2->trans_b || m2->in[2] != nullptr) continue;
+    if (m2->kind != kObjMatMul || m2->gmm_type != 0 || m2->trans_a || m2->trans_b || m2->in[2] != nullptr) continue;
     if (m2->type_id_ != kFloat16 && m2->type_id_ != kBFloat16) continue;
     NDObject *p = m2->in[0], *v = m2->in[1];
     if (p->kind != kObjCast || p->in[0]->type_id_ != kFloat32 || uses[p->id] != 1) continue;
@@ -563,7 +563,7 @@ void Compiler::DetectAttention() {
       const uint32_t bits = ScalarToContainer(sc->scalar.Get(), sc->in[0]->type_id_);
       std::memcpy(&scale, &bits, 4);
     }
-    if (m1->kind != kObjMatMul || m1->trans_a || !m1->trans_b || m1->in[2] != nullptr || uses[m1->id] != 1) continue;
+    if (m1->kind != kObjMatMul || m1->gmm_type != 0 || m1->trans_a || !m1->trans_b || m1->in[2] != nullptr || uses[m1->id] != 1) continue;
     if (m1->type_id_ != m2->type_id_) continue;
     NDObject *q = m1->in[0], *kk = m1->in[1];
     // q, k, v: loads, or views of loads the kernel can walk in place (a heads-first view of a [batch, seq, heads, d]

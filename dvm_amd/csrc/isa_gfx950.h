@@ -290,7 +290,18 @@ typedef struct {
   uint32_t k_split;    // VCF_SPLITK_*: parts the k axis is cut into (>= 2), each k_chunk long (a multiple of 64; the last
   uint32_t k_chunk;    // may be shorter), and the fp32 partial tiles: [k_split][tiles][tile vectors][lanes] of 16 bytes
   uint64_t part_addr;
+  // Grouped products (VCG_*; nb0 = 1, nb1 = the number of groups): a list of nb1 int64 (group_i32: int32) values in
+  // device memory, the upper bounds of the groups' ranges (VCG_*_BOUND: ascending) or their sizes (VCG_*_SIZE), read
+  // by the kernel when it starts. VCG_M_*: group g owns the rows [bound[g-1], bound[g]) of A and of the output and
+  // multiplies them with matrix g of B; the output has no batch axis, and a tile that crosses a bound is computed
+  // once per group that owns rows of it, each storing only its rows. VCG_K_*: group g multiplies the columns
+  // [bound[g-1], bound[g]) of A with the same rows of B into matrix g of the output (zeros for an empty range).
+  uint64_t group_addr;
+  uint32_t group_mode;
+  uint32_t group_i32;
 } VCubeHeader;
+enum { VCG_NONE = 0, VCG_M_BOUND = 1, VCG_M_SIZE = 2, VCG_K_BOUND = 3, VCG_K_SIZE = 4 };
+#define DVM_CUBE_MAX_GROUPS 2048u
 
 // VCubeHeader::epi_flags
 // Every store of the epilogue writes fp16 or bf16 and the program holds only operators that are continuous in
@@ -329,6 +340,7 @@ typedef struct {
 #define DVM_CUBE_MAX2(a, b) ((a) > (b) ? (a) : (b))
 #define DVM_CUBE_LDS_BYTES(bt) \
   DVM_CUBE_MAX2(DVM_CUBE_LDS_LOOP_BYTES(bt), DVM_CUBE_MAX2(DVM_CUBE_LDS_DUMP32_BYTES(bt), DVM_CUBE_LDS_DUMP16_BYTES(bt)))
+// (a grouped product keeps its tables behind that: 8 bytes per group)
 
 // ---- fused attention programs (VE_ATTN) -------------------------------------------
 // O[b] = softmax(Q[b] K[b]^T * scale) V[b] for nb independent (batch, head) pairs, all operands row

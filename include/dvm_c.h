@@ -71,6 +71,13 @@ dvm_obj *dvm_rt_gather_load(dvm_rt *rt, dvm_shape *shape, dvm_obj *index, int dt
 dvm_obj *dvm_rt_pad_store(dvm_rt *rt, dvm_obj *x, long long pad_size);
 dvm_obj *dvm_rt_one_hot(dvm_rt *rt, dvm_obj *indices, dvm_shape *depth, int axis, double on_value, double off_value, int dtype);
 dvm_obj *dvm_rt_element_any(dvm_rt *rt, dvm_obj *x);
+// Kernel::GroupedMatMul (include/dvm.h:510-522 of the reference; KernelPy grouped_matmul, include/dvm_py.h:198-205):
+// group_type 0: the groups are ranges of lhs's rows, rhs is [groups, k, n] ([groups, n, k] transposed), the result
+// [m, n]; group_type 2: ranges of the k axis, the result [groups, m, n]. group_list is a load of int64 (or int32)
+// values, one per group, read on the device at every launch: the ranges' upper bounds (group_list_type 0, ascending)
+// or their sizes (1). bias (may be null) is [groups, n]. Rows past the last bound are not written.
+dvm_obj *dvm_rt_grouped_matmul(dvm_rt *rt, dvm_obj *lhs, dvm_obj *rhs, int trans_a, int trans_b, dvm_obj *bias, dvm_obj *group_list,
+                               int group_type, int group_list_type);
 int dvm_rt_set_store_inplace(dvm_rt *rt, dvm_obj *store);
 // Kernel::SetStoreTemp / SetLoadBind / SpecNext (include/dvm.h:352-353, 544 of the reference; KernelPy set_store_temp /
 // set_load_bind, include/dvm_py.h:207-208, RtKernelPy spec_next): a Store that is no output of the kernel, a Load that

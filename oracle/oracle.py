@@ -29,8 +29,8 @@ import numpy as np
 _DIR = os.path.dirname(os.path.abspath(__file__))
 _SO = os.path.join(_DIR, "libdvm_oracle.so")
 
-BOOL, F16, BF16, F32, I32 = 0, 1, 2, 3, 4
-_NAMES = {"bool": BOOL, "float16": F16, "bfloat16": BF16, "float32": F32, "int32": I32}
+BOOL, F16, BF16, F32, I32, I64 = 0, 1, 2, 3, 4, 5
+_NAMES = {"bool": BOOL, "float16": F16, "bfloat16": BF16, "float32": F32, "int32": I32, "int64": I64}
 
 SQRT, ABS, LOG, EXP, RECIP, ISFINITE, LNOT, ROUND, FLOOR, CEIL, TRUNC = range(11)
 EQ, NE, GT, GE, LT, LE, ADD, SUB, MUL, DIV, POW, MAXIMUM, MINIMUM, LAND, LOR = range(15)
@@ -247,7 +247,9 @@ class OracleKernel:
     def load(self, array, dtype=None):
         a = np.asarray(array)
         t = _tid(dtype) if dtype is not None else _NAMES[str(a.dtype)]
-        if t == BOOL:
+        if t == I64:  # carried as it is: only the group list of a grouped matmul has this type here
+            v = a.astype(np.int64)
+        elif t == BOOL:
             v = a.astype(np.bool_)
         elif t == I32:
             v = a.astype(np.int32)
@@ -577,6 +579,37 @@ class OracleKernel:
 
     def matmul(self, lhs, rhs, trans_a, trans_b, bias=None):
         return OVal(matmul(lhs.a, rhs.a, bias.a if bias is not None else None, trans_a, trans_b, lhs.t), lhs.t)
+
+    def grouped_matmul(self, lhs, rhs, trans_a, trans_b, bias, group_list, group_type, group_list_type=0):
+        """One product per group (include/dvm.h:510-522, src/ops_m.cc:721-762 of the reference; expected values of
+        tests/ut/test_gmm.py:25-76): the list holds the groups' upper bounds (group_list_type 0) or sizes (1).
+        group_type 0: rows [lo, hi) of lhs times matrix g of rhs (+ row g of the bias) are rows [lo, hi) of the
+        result; rows past the last bound are left at zero here (the product does not write them). group_type 2:
+        columns [lo, hi) of lhs times rows [lo, hi) of rhs (+ row g of the bias) are matrix g of the result. Every
+        product is the matmul of this module: fp32 accumulation, bias added in fp32, one rounding."""
+        a = lhs.a.T if trans_a else lhs.a
+        b = np.swapaxes(rhs.a, -1, -2) if trans_b else rhs.a
+        gl = np.asarray(group_list.a, np.int64)
+        if group_list_type == 1:
+            gl = np.cumsum(gl)
+        m, k = a.shape
+        lim = m if group_type == 0 else k
+        gl = np.clip(gl, 0, lim)
+        n = b.shape[-1]
+        out = np.zeros((m, n) if group_type == 0 else (len(gl), m, n), np.float32)
+        lo = 0
+        for g, hi in enumerate(gl):
+            hi = max(int(hi), lo)
+            bg = bias.a[g] if bias is not None else None
+            if group_type == 0:
+                if hi > lo:
+                    out[lo:hi] = matmul(np.ascontiguousarray(a[lo:hi]), np.ascontiguousarray(b[g]), bg, False, False, lhs.t)
+            elif hi > lo:
+                out[g] = matmul(np.ascontiguousarray(a[:, lo:hi]), np.ascontiguousarray(b[lo:hi]), bg, False, False, lhs.t)
+            elif bg is not None:
+                out[g] = np.broadcast_to(round_to(lhs.t, bg.astype(np.float32)), (m, n))
+            lo = hi
+        return OVal(out, lhs.t)
 
     # -- outputs --
     def store(self, x, dtype=None):

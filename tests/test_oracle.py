@@ -377,3 +377,43 @@ def test_gather_onehot_pad_any_against_numpy_and_the_reference_rule():
     assert k.output(k.element_any(k.load(m))).tolist() == [0.0]
     m[3, 7] = 1
     assert k.output(k.element_any(k.load(m))).tolist() == [1.0]
+
+
+def test_grouped_matmul_against_float64_rule():
+    # the reference's own expectation (tests/ut/test_gmm.py:25-76) in float64: per group, rows [lo, hi) of x times
+    # matrix g of w (groups of rows), or columns [lo, hi) of x times rows [lo, hi) of w (groups along k), + bias row g
+    rng = np.random.default_rng(21)
+    k = OracleKernel()
+    m, n, kk, g = 37, 24, 50, 4
+    x = rng.normal(0, 0.5, (m, kk)).astype(np.float16)
+    wm = rng.normal(0, 0.5, (g, kk, n)).astype(np.float16)
+    wk = rng.normal(0, 0.5, (kk, n)).astype(np.float16)
+    b = rng.normal(0, 0.5, (g, n)).astype(np.float16)
+    for bounds, sizes in [([5, 5, 20, 37], False), ([5, 0, 15, 17], True), ([3, 30, 37, 37], False)]:
+        ends = np.cumsum(bounds) if sizes else np.array(bounds)
+        want = np.zeros((m, n))
+        lo = 0
+        for i, hi in enumerate(ends):
+            want[lo:hi] = x[lo:hi].astype(np.float64) @ wm[i].astype(np.float64) + b[i].astype(np.float64)
+            lo = hi
+        got = k.output(k.grouped_matmul(k.load(x), k.load(wm), False, False, k.load(b), k.load(np.array(bounds, np.int64)), 0, int(sizes)))
+        assert got.dtype == np.float16 and np.allclose(got, want, rtol=2e-3, atol=2e-3)
+        # transposed operands give the same product
+        got_t = k.output(k.grouped_matmul(k.load(np.ascontiguousarray(x.T)), k.load(np.ascontiguousarray(wm.transpose(0, 2, 1))), True, True,
+                                          k.load(b), k.load(np.array(bounds, np.int64)), 0, int(sizes)))
+        assert np.array_equal(got_t, got)
+    for bounds, sizes in [([0, 7, 7, 50], False), ([10, 0, 25, 15], True)]:
+        ends = np.cumsum(bounds) if sizes else np.array(bounds)
+        want = np.zeros((g, m, n))
+        lo = 0
+        for i, hi in enumerate(ends):
+            want[i] = x[:, lo:hi].astype(np.float64) @ wk[lo:hi].astype(np.float64) + b[i].astype(np.float64)
+            lo = hi
+        got = k.output(k.grouped_matmul(k.load(x), k.load(wk), False, False, k.load(b), k.load(np.array(bounds, np.int64)), 2, int(sizes)))
+        assert got.shape == (g, m, n) and np.allclose(got, want, rtol=2e-3, atol=2e-3)
+    # rows past the last bound are not written (zeros here); bounds past the axis are clipped
+    got = k.output(k.grouped_matmul(k.load(x), k.load(wm), False, False, None, k.load(np.array([5, 9, 9, 12], np.int64)), 0))
+    assert not got[12:].any() and got[:12].any()
+    a = k.output(k.grouped_matmul(k.load(x), k.load(wm), False, False, None, k.load(np.array([5, 9, 20, 99], np.int64)), 0))
+    c = k.output(k.grouped_matmul(k.load(x), k.load(wm), False, False, None, k.load(np.array([5, 9, 20, 37], np.int64)), 0))
+    assert np.array_equal(a, c)
