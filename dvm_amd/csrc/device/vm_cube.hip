@@ -1312,7 +1312,6 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
         k_fast = (k_lo & 7u) == 0u && k_hi > k_lo && ((k_hi - k_lo) & 63u) == 0u;
       }
     }
-    const uint32_t nk = (k_hi - k_lo + BK - 1) / BK;
     if (h.fast) {
       if (m0 + BM > h.m && h.m >= BM && (A_KC || (h.m & 7u) == 0)) m0 = h.m - BM;
       if (n0 + BN > h.n && h.n >= BN && (h.n & 7u) == 0) n0 = h.n - BN;
@@ -1332,6 +1331,48 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
     constexpr bool a_clamps = !RING && A_KC && (BM * BK / 8 / NTHR) <= 2, b_clamps = !RING && B_KC && (BN * BK / 8 / NTHR) <= 2;
     const uint32_t a_rows = h.m - m0 < static_cast<uint32_t>(BM) ? h.m - m0 : static_cast<uint32_t>(BM);
     const uint32_t b_rows = h.n - n0 < static_cast<uint32_t>(BN) ? h.n - n0 : static_cast<uint32_t>(BN);
+    // The guarded walk over a part of the k axis: any start, any length, rows and columns past the edges read as zero.
+    const uint32_t a_vec = ((h.lda & 7u) == 0u && (a_base & 15u) == 0u) ? 1u : 0u;
+    const uint32_t b_vec = ((h.ldb & 7u) == 0u && (b_base & 15u) == 0u) ? 1u : 0u;
+    auto guarded_walk = [&](uint32_t from, uint32_t to) {
+      for (uint32_t k0 = from; k0 < to; k0 += BK) {
+        stage_generic<BM, NTHR>(lds, a_base, h.lda, m0, k0, h.m, to, A_KC ? 1u : 0u, a_vec, tid);
+        stage_generic<BN, NTHR>(lds + kBBase, b_base, h.ldb, n0, k0, h.n, to, B_KC ? 1u : 0u, b_vec, tid);
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+          vu4 af[TM], bf[TN];
+#pragma unroll
+          for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const vu4 *>(lds + frag_off(a_row, a_x, i, kk));
+#pragma unroll
+          for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const vu4 *>(lds + frag_off(b_row, b_x, j, kk));
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j) acc[i][j] = mfma<IS_BF16>(af[i], bf[j], acc[i][j]);
+        }
+        __syncthreads();
+      }
+    };
+    // A group's part of the k axis that is not whole steps from an aligned start: the vector path takes the steps in
+    // its middle, the guarded walk the few k in front (up to the next multiple of 8) and behind (less than a step).
+    uint32_t tail_lo = 0, tail_hi = 0;
+    if constexpr (!COMB) {
+      if (!g_rows && gmode != VCG_NONE && !k_fast && h.fast && k_hi > k_lo && (m0 + BM <= h.m || a_clamps) && (n0 + BN <= h.n || b_clamps)) {
+        const uint32_t up8 = (k_lo + 7u) & ~7u;
+        const uint32_t f_lo = up8 < k_hi ? up8 : k_hi;
+        const uint32_t f_hi = f_lo + ((k_hi - f_lo) & ~63u);
+        if (f_hi > f_lo) {
+          if (f_lo > k_lo) guarded_walk(k_lo, f_lo);
+          tail_lo = f_hi;
+          tail_hi = k_hi;
+          k_lo = f_lo;
+          k_hi = f_hi;
+          k_fast = true;
+        }
+      }
+    }
+    const uint32_t nk = (k_hi - k_lo + BK - 1) / BK;
     // address of element (row0, k_lo) of each operand
     const uint64_t a_org = a_base + (A_KC ? static_cast<uint64_t>(m0) * h.lda + k_lo : static_cast<uint64_t>(k_lo) * h.lda + m0) * 2;
     const uint64_t b_org = b_base + (B_KC ? static_cast<uint64_t>(n0) * h.ldb + k_lo : static_cast<uint64_t>(k_lo) * h.ldb + n0) * 2;
@@ -1518,27 +1559,9 @@ __device__ __forceinline__ void vm_cube(const VmParam &p) {
       __syncthreads();
      }
     } else {
-      const uint32_t a_vec = ((h.lda & 7u) == 0u && (a_base & 15u) == 0u) ? 1u : 0u;
-      const uint32_t b_vec = ((h.ldb & 7u) == 0u && (b_base & 15u) == 0u) ? 1u : 0u;
-      for (uint32_t kt = 0; kt < nk; ++kt) {
-        stage_generic<BM, NTHR>(lds, a_base, h.lda, m0, k_lo + kt * BK, h.m, k_hi, A_KC ? 1u : 0u, a_vec, tid);
-        stage_generic<BN, NTHR>(lds + kBBase, b_base, h.ldb, n0, k_lo + kt * BK, h.n, k_hi, B_KC ? 1u : 0u, b_vec, tid);
-        __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < BK / 16; ++kk) {
-          vu4 af[TM], bf[TN];
-#pragma unroll
-          for (int i = 0; i < TM; ++i) af[i] = *reinterpret_cast<const vu4 *>(lds + frag_off(a_row, a_x, i, kk));
-#pragma unroll
-          for (int j = 0; j < TN; ++j) bf[j] = *reinterpret_cast<const vu4 *>(lds + frag_off(b_row, b_x, j, kk));
-#pragma unroll
-          for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j) acc[i][j] = mfma<IS_BF16>(af[i], bf[j], acc[i][j]);
-        }
-        __syncthreads();
-      }
+      guarded_walk(k_lo, k_hi);
     }
+    if (tail_hi > tail_lo) guarded_walk(tail_lo, tail_hi);
     }
 
     if (split_part) {
