@@ -229,6 +229,7 @@ struct Tuning {
   int vec_unirun = -1;  // DVM_VEC_UNIRUN=0: every wave executes the per-output runs
   int vec_reread = -1;  // DVM_VEC_REREAD=0: nothing parked, no reversed sweeps; 2: parked rounds only; 3: reversed sweeps only
   int vec_sweeps = -1;  // DVM_VEC_SWEEPS=0: never the sweep build of the vector VM
+  int vec_gather_tile = -1;  // DVM_VEC_GATHER_TILE=0: pointwise programs with a gathered operand keep the plain slab order
   int cube_tile = -1;   // DVM_CUBE_TILE=256|128|64
   int cube_waves = -1;  // DVM_CUBE_WAVES=4|8
   int red_split_turn = -1;  // DVM_RED_SPLIT_TURN=0: the reduce over the parts of a shared reduce walks them outermost, as they lie in memory

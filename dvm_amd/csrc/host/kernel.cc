@@ -31,6 +31,7 @@ void Tuning::Read() {
   vec_unirun = num("DVM_VEC_UNIRUN");
   vec_reread = num("DVM_VEC_REREAD");
   vec_sweeps = num("DVM_VEC_SWEEPS");
+  vec_gather_tile = num("DVM_VEC_GATHER_TILE");
   cube_tile = num("DVM_CUBE_TILE");
   cube_waves = num("DVM_CUBE_WAVES");
   cube_exact = num("DVM_CUBE_EXACT");

@@ -526,7 +526,7 @@ void Compiler::ChooseSchedule() {
     // innermost axis walked in tiles of 64 elements (8 slabs) and the next axis inside that, a workgroup covers
     // 64 x 64 elements and uses every line it fetches in full:
     // kept dims [8 slabs][the other dims ...][innermost extent / 64].
-    static const bool tile_gather = !(std::getenv("DVM_VEC_GATHER_TILE") != nullptr && std::getenv("DVM_VEC_GATHER_TILE")[0] == '0');
+    const bool tile_gather = k_->tuning_.vec_gather_tile != 0;
     if (tile_gather && nk_ >= 2 && nk_ < DVM_VEC_MAXR && klist_[0] == inner && dims_[inner].extent % (8 * E) == 0) {
       for (int i = 0; i < nn_ && !split_inner_; ++i) {
         const ANode &n = nodes_[i];

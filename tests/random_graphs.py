@@ -6,7 +6,9 @@ pointwise_reduce_graph  fp32 arithmetic over fp32/fp16/bf16 inputs with broadcas
 typed_graph             values kept in their own types (fp32/fp16/bf16/int32/bool): compares, logic, selects, casts
 matmul_graph            one matmul (transposes, batches, shared operands) with a computed operand and an epilogue chain
 dynamic_case            one graph and three sets of input shapes for a kernel object built with -1 extents
-view_graph              permute / slice / split / concat / copy chains mixed with pointwise operators and reduces"""
+view_graph              permute / slice / split / concat / copy chains mixed with pointwise operators and reduces
+index_graph             one_hot / gather_load (both modes, computed indices) / pad_store / element_any around pointwise
+                        operators, reduces, permutes and slices"""
 import numpy as np
 
 from dvm_amd.tester import Tester
@@ -372,6 +374,107 @@ def view_graph(case):
 
 
 
+def index_graph(case):
+    rng = np.random.default_rng(case)
+    rank = int(rng.integers(1, 4))
+    shape = [int(rng.choice([1, 2, 3, 5, 8, 17, 40])) for _ in range(rank)]
+    shape[-1] = int(rng.choice([1, 3, 8, 24, 64, 100, 257]))
+    dt = str(rng.choice(["float32", "float32", "float16", "bfloat16", "int32"]))
+    kind = str(rng.choice(["onehot", "take", "along"]))
+    axis = int(rng.integers(0, rank + (1 if kind == "onehot" else 0)))
+    if rng.random() < 0.3:
+        axis -= rank + (1 if kind == "onehot" else 0)
+    depth = int(rng.choice([1, 2, 7, 16, 100, 300]))
+    ix_shape = [int(rng.choice([1, 2, 4, 9, 33])) for _ in range(int(rng.integers(1, 3)))]
+    src = rng.integers(-50, 50, shape).astype(np.int32) if dt == "int32" else rng.uniform(-2, 2, shape).astype(np.float32)
+    if dt == "float16": src = src.astype(np.float16)
+    if kind == "onehot":
+        ix = rng.integers(-2, depth + 2, shape).astype(np.int32)
+    elif kind == "take":
+        n = shape[axis]
+        ix = rng.integers(-n - 3, n + 3, ix_shape).astype(np.int32)
+    else:
+        n = shape[axis]
+        sh = list(shape)
+        sh[axis] = int(rng.choice([1, 2, 5, 19]))
+        ix = rng.integers(-n, n, sh).astype(np.int32)
+    computed_ix = bool(rng.integers(0, 2))
+    tail = [(str(rng.choice(["add", "mul", "sum", "max", "permute", "slice_dim", "any", "pad", "neg"])), int(rng.integers(0, 1 << 30)))
+            for _ in range(int(rng.integers(0, 4)))]
+
+    def head(k):
+        i = k.load(ix)
+        if computed_ix:
+            i = k.sub(k.add(i, 3), 3)
+        if kind == "onehot":
+            if dt == "int32":
+                return k.one_hot(i, depth, axis, 3, -1, dt)
+            x = k.one_hot(i, depth, axis, 1.5, -0.25, dt)
+            return x if dt == "float32" else k.cast(x, "float32")
+        x = k.gather_load(src, i, axis=axis, dtype=dt, gather_mode=1 if kind == "take" else 0)
+        return x if dt in ("float32", "int32") else k.cast(x, "float32")
+
+    is_int = dt == "int32"
+
+    def step(k, x, stores, op):
+        name = op[0]
+        if name == "add":
+            return k.add(x, 2 if is_int else 0.5)
+        if name == "mul":
+            return k.mul(x, x)
+        if name == "neg":
+            return k.mul(x, -1 if is_int else -1.0)
+        if name in ("sum", "max"):
+            return (k.sum if name == "sum" else k.max)(x, (op[1],), op[2])
+        if name == "permute":
+            return k.permute(x, list(op[1]))
+        if name == "slice_dim":
+            return k.slice_dim(x, op[1], op[2], op[3])
+        if name == "any":
+            stores.append(k.store(k.element_any(k.abs(x))))
+        elif name == "pad":
+            stores.append(k.pad_store(k.add(x, 1 if is_int else 1.0), op[1]))
+        return x
+
+    # the graph is planned on the oracle, whose shapes are known while it is built, and recorded as a tape
+    tape = []
+    with np.errstate(all="ignore"):
+        ko = OracleKernel()
+        x = head(ko)
+        for name, seed in tail:
+            r = np.random.default_rng(seed)
+            shp = list(x.shape())
+            rk = len(shp)
+            op = None
+            if name in ("add", "mul", "neg"):
+                op = (name,)
+            elif name in ("sum", "max") and rk > 0 and not (name == "sum" and is_int):
+                op = (name, int(r.integers(0, rk)), bool(r.integers(0, 2)))
+            elif name == "permute" and rk > 1:
+                op = (name, [int(p) for p in r.permutation(rk)])
+            elif name == "slice_dim" and rk > 0:
+                d = int(r.integers(0, rk)); n = shp[d]
+                if n >= 1:
+                    b0 = int(r.integers(0, n)); e0 = int(r.integers(b0 + 1, n + 1))
+                    op = (name, d, b0, e0)
+            elif name == "any" and not is_int and rk > 0:
+                op = (name,)
+            elif name == "pad" and rk > 0:
+                op = (name, int(r.integers(0, 9)))
+            if op is not None:
+                tape.append(op)
+                x = step(ko, x, [], op)
+
+    def build(k):
+        x = head(k)
+        stores = []
+        for op in tape:
+            x = step(k, x, stores, op)
+        stores.append(k.store(x))
+        return stores
+    return build
+
+
 def compile_in_das_mode(seeds):
     """The host compiler alone on `seeds` cases of every generator, in disassembly mode (no GPU): what `make
     asan-check` runs against the sanitizer build. A compile error with one of the documented messages is a valid
@@ -380,7 +483,7 @@ def compile_in_das_mode(seeds):
     from oracle.oracle import OracleKernel
     done = refused = 0
     for case in range(seeds):
-        for gen, ker in ((lambda c: pointwise_reduce_graph(c, True), ""), (typed_graph, ""), (matmul_graph, "mix"), (view_graph, "")):
+        for gen, ker in ((lambda c: pointwise_reduce_graph(c, True), ""), (typed_graph, ""), (matmul_graph, "mix"), (view_graph, ""), (index_graph, "")):
             build = gen(case)
             if gen is not matmul_graph:
                 try:  # (the plan of a graph is made on the oracle; a case it rejects is no case)

@@ -148,3 +148,11 @@ def test_attention_shapes(first):
         want = np_attention(q, k, v)
         assert got.shape == want.shape, (case, got.shape, want.shape)
         assert np.allclose(got, want, rtol=1e-2, atol=1e-2), (case, batch, sq, skv, d, dt, float(np.abs(got - want).max()))
+
+
+@gpu
+@pytest.mark.parametrize("first", range(0, 4 * CHUNK, CHUNK))
+def test_index_graphs(first):
+    for case in range(first, first + CHUNK):
+        build = R.index_graph(case)
+        _check(case, build, "", _oracle(build), skip=("needs a Copy",))
