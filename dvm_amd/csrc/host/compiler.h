@@ -243,6 +243,11 @@ class Compiler {
     NDObject *m1, *m2, *q, *k, *v;
     float scale;
     int area;
+    // The result goes straight into a Store through strides (a Store with a stride list, or the dense Store of a
+    // Permute of the result that keeps the head dimension innermost): no dense copy of the result exists then.
+    NDObject *out_store = nullptr;
+    uint32_t out_row = 0, out_outer = 0, out_inner = 0, out_nb_inner = 1;
+    int64_t out_base = 0;
   };
   // How an operand of a fused attention lies in memory (VAttnHeader: strides in elements). `ok`: the kernel can
   // read it in place (a load, or a permute / slice of a load; head dimension contiguous; at most two batch axes

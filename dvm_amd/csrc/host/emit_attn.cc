@@ -32,6 +32,7 @@ void Compiler::CompileAttn(int gi) {
     if (!l.ok) Fail("attention operand layout");
     if (l.nb_inner != 1) nb_inner = l.nb_inner;
   }
+  if (g.out_store != nullptr && g.out_nb_inner != 1) nb_inner = g.out_nb_inner;
   h.nb_inner = nb_inner;
   for (int i = 0; i < 3; ++i) {
     const NDObject *t = i == 0 ? g.q : (i == 1 ? g.k : g.v);
@@ -45,10 +46,20 @@ void Compiler::CompileAttn(int gi) {
       h.inner_stride[i] = lay[i].inner;
     }
   }
-  // the result is dense: [nb][sq][d]
+  // the result is dense, [nb][sq][d], unless it goes into a Store through strides
   h.row_stride[3] = h.d;
   h.inner_stride[3] = nb_inner != 1 ? h.sq * h.d : 0;
   h.outer_stride[3] = h.sq * h.d * nb_inner;
+  if (g.out_store != nullptr) {
+    h.row_stride[3] = g.out_row;
+    if (g.out_nb_inner == 1 && nb_inner != 1) {  // one batch stride beside operands with two: split it
+      h.inner_stride[3] = g.out_outer;
+      h.outer_stride[3] = g.out_outer * nb_inner;
+    } else {
+      h.inner_stride[3] = g.out_inner;
+      h.outer_stride[3] = g.out_outer;
+    }
+  }
   if (static_cast<uint64_t>(h.nb) * h.q_blocks >= (1ull << 31)) Fail("too many attention blocks");
   std::memset(&prog_->blob, 0, sizeof(VmParam));
   std::memcpy(prog_->blob.w, &h, sizeof(h));
@@ -66,7 +77,9 @@ void Compiler::CompileAttn(int gi) {
   patch(offsetof(VAttnHeader, v_addr), lay[2].root->id, -1, lay[2].base);
   // the result goes to the user's store when there is one in this sub-kernel, else to workspace
   const int m2 = g.m2->id;
-  if (store_of_[m2] >= 0 && area_[store_of_[m2]] == area_[m2]) {
+  if (g.out_store != nullptr) {
+    patch(offsetof(VAttnHeader, o_addr), g.out_store->id, -1, g.out_base);
+  } else if (store_of_[m2] >= 0 && area_[store_of_[m2]] == area_[m2]) {
     patch(offsetof(VAttnHeader, o_addr), store_of_[m2], -1);
   } else if (ws_slot_[m2] >= 0) {
     patch(offsetof(VAttnHeader, o_addr), -1, ws_slot_[m2]);

@@ -96,7 +96,7 @@ bool Compiler::CanJoin(int a, const NDObject *o) {
   if (o->kind == kObjReduce && LevelIn(a, o) < 8 && ai.red_at_level[LevelIn(a, o)] >= 2) return false;
   if (o->kind == kObjMatMul) return false;
   if (ai.n_ops >= kMaxAreaOps && !IsStoreLike(o)) return false;  // long graphs are cut into several launches
-  if (ai.attn >= 0) return o->kind == kObjStore && o->in[0] == attn_groups_[ai.attn].m2;
+  if (ai.attn >= 0) return o->kind == kObjStore && (o->in[0] == attn_groups_[ai.attn].m2 || o == attn_groups_[ai.attn].out_store);
   if (ai.cube) {
     if (!IsPointwiseKind(o->kind)) return false;
     if (mode_ >= 2 && !(o->kind == kObjStore && o->in[0] == ai.cube_op)) return false;  // plain matmul, epilogue on its own
@@ -448,6 +448,7 @@ void Compiler::PlanMaterialisation() {
       if (v == nullptr) continue;
       const NDObject *root = ViewRoot(v);
       if (IsLeaf(root) || root->kind == kObjLoad) continue;
+      if (attn_of_[i] >= 0 && attn_groups_[attn_of_[i]].out_store == o) continue;  // (the attention kernel writes it through strides)
       const int user_area = IsView(o) ? -2 : area_[i];
       if (IsView(v) || (user_area != -2 && area_[root->id] != user_area)) mat_[root->id] = 1;
     }
@@ -594,9 +595,85 @@ void Compiler::DetectAttention() {
     for (int d = 0; d < r - 2 && ok; ++d) ok = q->dim(d) == kk->dim(d) && q->dim(d) == v->dim(d) && q->dim(d) > 0;
     if (!ok || q->numel() >= (1ll << 31) || kk->numel() >= (1ll << 31)) continue;
     AttnGroup g = {m1, m2, q, kk, v, scale, -1};
+    // Where the result goes when its one consumer is a Store through strides, or a Permute (head dimension still
+    // innermost) whose one consumer is a dense Store: the kernel writes rows of d elements through a row stride and
+    // two batch strides, so the [batch, seq, heads, d] layout of a [batch, heads, seq, d] result costs no copy.
+    NDObject *out_store = nullptr;
+    if (uses[m2->id] == 1 && r >= 2 && r <= 4) {
+      NDObject *c1 = nullptr;
+      for (int j = i + 1; j < n_ && c1 == nullptr; ++j) {
+        NDObject *o = k_->ops_[j];
+        if (!live_[j]) continue;
+        for (int t = 0; t < o->nin; ++t)
+          if (o->in[t] == m2) c1 = o;
+      }
+      int64_t st[kMaxRank];
+      bool have = false;
+      int64_t base = 0;
+      if (c1 != nullptr && c1->kind == kObjStore && c1->strided && c1->pad_size < 0 && c1->type_id_ == m2->type_id_ && c1->stride_ref != nullptr) {
+        for (int d = 0; d < r; ++d) st[d] = c1->vstride_[d];
+        base = c1->view_base_;
+        out_store = c1;
+        have = true;
+      } else if (c1 != nullptr && c1->kind == kObjPermute && uses[c1->id] == 1 && c1->aux_ref != nullptr && static_cast<int>(c1->aux_ref->size) == r) {
+        NDObject *c2 = nullptr;
+        for (int j = c1->id + 1; j < n_ && c2 == nullptr; ++j) {
+          NDObject *o = k_->ops_[j];
+          if (live_[j] && o->nin >= 1 && o->in[0] == c1) c2 = o;
+        }
+        if (c2 != nullptr && c2->kind == kObjStore && !c2->strided && !c2->temp && !c2->inplace && c2->type_id_ == m2->type_id_) {
+          // result dim perm[i] lies at the dense stride of dim i of the permuted value
+          int64_t dense = 1;
+          for (int d = r - 1; d >= 0; --d) {
+            int64_t src = c1->aux_ref->data[d];
+            if (src < 0) src += r;
+            st[src] = dense;
+            dense *= c1->dim(d);
+          }
+          out_store = c2;
+          have = true;
+        }
+      }
+      if (have) {
+        auto fits = [](int64_t v) { return v >= 0 && v < (1ll << 32) && v % 8 == 0; };
+        const int64_t d = m2->dim(r - 1), rows = m2->dim(r - 2);
+        const int64_t row = rows == 1 ? d : st[r - 2];
+        bool ok_out = (d == 1 || st[r - 1] == 1) && row >= d && row < (1ll << 22) && row % 8 == 0 && base >= 0 && base % 8 == 0;
+        int64_t outer = 0, inner = 0, nbi = 1;
+        if (r == 3) {
+          outer = m2->dim(0) == 1 ? 0 : st[0];
+        } else if (r == 4) {
+          outer = m2->dim(0) == 1 ? 0 : st[0];
+          inner = m2->dim(1) == 1 ? 0 : st[1];
+          nbi = m2->dim(1);
+        }
+        ok_out = ok_out && fits(outer) && fits(inner);
+        // the operands must split their (batch, head) pairs the same way: views with two batch axes already do, or
+        // they are dense rank-4 tensors whose second dim is the inner extent
+        if (ok_out && nbi != 1) {
+          for (const AttnLayout *l : {&lq, &lk, &lv}) {
+            const NDObject *t = l == &lq ? q : (l == &lk ? kk : v);
+            if (l->nb_inner != 1 ? l->nb_inner != static_cast<uint32_t>(nbi) : (t->rank() != 4 || t->dim(1) != nbi)) ok_out = false;
+          }
+        } else if (ok_out) {
+          for (const AttnLayout *l : {&lq, &lk, &lv})
+            if (l->nb_inner != 1) ok_out = false;  // (rank 4 with one head: the operands' split decides; keep it simple)
+        }
+        if (ok_out) {
+          g.out_store = out_store;
+          g.out_row = static_cast<uint32_t>(row);
+          g.out_outer = static_cast<uint32_t>(outer);
+          g.out_inner = static_cast<uint32_t>(inner);
+          g.out_nb_inner = static_cast<uint32_t>(nbi);
+          g.out_base = base;
+        } else {
+          out_store = nullptr;
+        }
+      }
+    }
     const int gi = static_cast<int>(attn_groups_.size());
     attn_groups_.push_back(g);
-    NDObject *members[] = {m1, mul, x, mul32, mx, sb, e, sm, dv, p, m2};
+    NDObject *members[] = {m1, mul, x, mul32, mx, sb, e, sm, dv, p, m2, g.out_store};
     for (NDObject *mbr : members)
       if (mbr != nullptr) attn_of_[mbr->id] = gi;
   }

@@ -204,3 +204,62 @@ def test_attention_views_the_kernel_cannot_walk_run_unfused():
     t.run()
     assert "entry attention" not in t.das(), t.das()
     assert np.allclose(t.output(out), np_attention(q, kt.transpose(0, 2, 1), v), rtol=1e-2, atol=1e-2)
+
+
+# ---- the result written through strides: no dense copy of it exists ----
+
+@pytest.mark.parametrize("b,s,h,d", [(2, 320, 4, 128), (1, 200, 3, 64), (2, 512, 2, 128)])
+@pytest.mark.parametrize("how", ["permute_store", "view_store"])
+@pytest.mark.parametrize("operands", ["dense", "views"])
+def test_attention_result_written_sequence_major(b, s, h, d, how, operands):
+    # the result [batch, heads, seq, d] goes to memory as [batch, seq, heads, d] (what the projection behind an
+    # attention reads), as the dense Store of a Permute or as a Store with a stride list: one launch either way
+    rng = np.random.default_rng(b * 1000 + s + h + 5)
+    t = Tester("mix")
+    if operands == "dense":
+        q, k, v = (rng.standard_normal((b, h, s, d)).astype(np.float16) for _ in range(3))
+        lq, lk, lv = (t.load(x) for x in (q, k, v))
+        want = np_attention(q, k, v)
+    else:
+        q, k, v = (rng.standard_normal((b, s, h, d)).astype(np.float16) for _ in range(3))
+        lq, lk, lv = (t.permute(t.load(x), [0, 2, 1, 3]) for x in (q, k, v))
+        want = np_attention(q.transpose(0, 2, 1, 3), k.transpose(0, 2, 1, 3), v.transpose(0, 2, 1, 3))
+    o = attention_graph(t, lq, lk, lv, 1.0 / math.sqrt(d), 4)
+    if how == "permute_store":
+        out = t.store(t.permute(o, [0, 2, 1, 3]))
+        t.run()
+        got = t.output(out)
+    else:
+        out = t.view_store(o, [s * h * d, d, h * d, 1], b * s * h * d)
+        t.run()
+        got = t.output(out, (b, s, h, d))
+    assert "entry attention" in t.das() and "o: view, strides row=%d" % (h * d) in t.das() and t.num_launches() == 1, t.das()
+    assert got.shape == (b, s, h, d) and np.allclose(got, want.transpose(0, 2, 1, 3), rtol=1e-2, atol=1e-2)
+
+
+def test_attention_result_into_a_padded_buffer_and_results_the_kernel_cannot_place():
+    rng = np.random.default_rng(91)
+    hds, s, d = 3, 200, 128
+    q, k, v = (rng.standard_normal((hds, s, d)).astype(np.float16) for _ in range(3))
+    want = np_attention(q, k, v)
+    # rows 160 elements apart, heads a whole number of rows apart: the kernel writes it in place
+    t = Tester("mix")
+    out = t.view_store(attention_graph(t, t.load(q), t.load(k), t.load(v), 1.0 / math.sqrt(d), 3), [s * 160, 160, 1], hds * s * 160)
+    t.run()
+    assert t.num_launches() == 1 and "o: view, strides row=160" in t.das(), t.das()
+    got = t.output(out, (hds, s, 160))
+    assert np.allclose(got[:, :, :d], want, rtol=1e-2, atol=1e-2) and not got[:, :, d:].any()
+    # a transposing permute of the result (the head dimension no longer innermost) is a copy behind the kernel
+    t = Tester("mix")
+    out = t.store(t.permute(attention_graph(t, t.load(q), t.load(k), t.load(v), 1.0 / math.sqrt(d), 3), [0, 2, 1]))
+    t.run()
+    assert "entry attention" in t.das() and t.num_launches() == 2, t.das()
+    assert np.allclose(t.output(out), want.transpose(0, 2, 1), rtol=1e-2, atol=1e-2)
+    # a result with a second consumer keeps its dense copy
+    t = Tester("mix")
+    o = attention_graph(t, t.load(q), t.load(k), t.load(v), 1.0 / math.sqrt(d), 3)
+    out1 = t.store(t.permute(o, [1, 0, 2]))
+    out2 = t.store(t.mul(o, 2.0))
+    t.run()
+    assert np.allclose(t.output(out1), want.transpose(1, 0, 2), rtol=1e-2, atol=1e-2)
+    assert np.allclose(t.output(out2), want * 2, rtol=1e-2, atol=2e-2)
