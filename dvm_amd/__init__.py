@@ -14,5 +14,13 @@ float32 = DataType.float32
 int32 = DataType.int32
 int64 = DataType.int64
 
-__all__ = ["DataType", "Device", "Kernel", "PyKernel", "NDObject", "IntArrayRef", "ScalarRef", "kernel",
+
+
+def lazy_fusion(ktype="eager"):
+    """Eager fusion without graphs for PyTorch tensors on the GPU (dvm_amd/lazy.py); imports torch on first use."""
+    from .lazy import lazy_fusion as _lazy_fusion
+    return _lazy_fusion(ktype)
+
+
+__all__ = ["lazy_fusion", "DataType", "Device", "Kernel", "PyKernel", "NDObject", "IntArrayRef", "ScalarRef", "kernel",
            "bool_", "float16", "bfloat16", "float32", "int32", "int64"]

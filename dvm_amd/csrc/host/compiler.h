@@ -402,6 +402,8 @@ class Compiler {
   bool cube_mode_ = false;
   VCubeMem cmems_[DVM_CUBE_MAXMEM];
   const NDObject *cube_out_ = nullptr;
+  uint32_t pw_threads_cap_ = 256;     // lanes of a pointwise workgroup in this attempt (128 doubles the V register slots a lane has)
+  int area_ops_limit_ = kMaxAreaOps;  // operators per sub-kernel in this attempt (RunModes lowers it when a sub-kernel runs out of registers)
   int gmm_bias_node_ = -1;  // the [groups, n] bias of a grouped matmul (its row goes with the group, not with the output's dims)
   bool SimpleOperand(int v);
   void EmitOperandInsn(uint32_t op, uint32_t sub, uint32_t rnd, int v);

@@ -283,6 +283,8 @@ class VKernel {
   void *ws_base_ = nullptr;
   std::string name_, fullname_;
   int part_mode_ = 0;             // partition mode that compiled last time (see Compiler::Run)
+  int ops_limit_ = 0;             // ... and, when that took fewer operators per sub-kernel or pointwise workgroups of
+  uint32_t pw_cap_ = 0;           // fewer lanes than the defaults, those (0: the defaults)
   double last_codegen_us_ = 0.0;  // wall time of the last Normalize+CodeGen, for JIT latency reports
 
  private:

@@ -1,10 +1,12 @@
 // VKernel::CodeGen / BindAddresses / Launch and the loop over partition modes.
 #include <algorithm>
+#include <cstdio>
 #include <cstdlib>
 #include <cmath>
 #include <cstddef>
 #include <cstring>
 #include <stdexcept>
+#include <string>
 
 #include "compiler.h"
 
@@ -70,12 +72,60 @@ size_t Compiler::Run() {
 size_t Compiler::RunModes() {
   n_ = static_cast<int>(k_->ops_.size());
   const int first_mode = k_->part_mode_;
+  area_ops_limit_ = kMaxAreaOps;
+  pw_threads_cap_ = 256;
+  if (k_->ops_limit_ != 0) {  // what this kernel needed last time
+    area_ops_limit_ = k_->ops_limit_;
+    pw_threads_cap_ = k_->pw_cap_;
+    try {
+      const size_t ws = RunOnce(first_mode);
+      area_ops_limit_ = kMaxAreaOps;
+      pw_threads_cap_ = 256;
+      return ws;
+    } catch (const std::runtime_error &) {
+      k_->ops_limit_ = 0;
+      k_->pw_cap_ = 0;
+      area_ops_limit_ = kMaxAreaOps;
+      pw_threads_cap_ = 256;
+    }
+  }
   for (int mode = first_mode; mode < 3; ++mode) {
     try {
       const size_t ws = RunOnce(mode);
       k_->part_mode_ = mode;
       return ws;
-    } catch (const std::runtime_error &) {
+    } catch (const std::runtime_error &e) {
+      if (k_->tuning_.debug) std::fprintf(stderr, "dvm: partition mode %d does not compile: %s\n", mode, e.what());
+      // A sub-kernel that holds more values at once than it has registers (a wide expression tree), more operands than
+      // descriptors or more code than a blob: the same rules with fewer operators per sub-kernel, before the rules
+      // themselves get stricter. (The cut values cross launches through the workspace.)
+      const std::string why = e.what();
+      const bool resources = why.find("out of V register slots") != std::string::npos || why.find("out of S registers") != std::string::npos ||
+                             why.find("too many memory operands") != std::string::npos || why.find("program larger than 4 KB") != std::string::npos;
+      if (resources && mode == first_mode) {
+        // (first with pointwise workgroups of 128 lanes, which have twice the V register slots per lane)
+        struct Restore {
+          Compiler *c;
+          ~Restore() {
+            c->area_ops_limit_ = kMaxAreaOps;
+            c->pw_threads_cap_ = 256;
+          }
+        } restore{this};
+        pw_threads_cap_ = 128;
+        for (int limit : {kMaxAreaOps, 40, 20, 10, 5}) {
+          if (limit != kMaxAreaOps && limit >= n_) continue;
+          area_ops_limit_ = limit;
+          try {
+            const size_t ws = RunOnce(mode);
+            k_->part_mode_ = mode;
+            k_->ops_limit_ = limit;
+            k_->pw_cap_ = pw_threads_cap_;
+            return ws;
+          } catch (const std::runtime_error &e2) {
+            if (k_->tuning_.debug) std::fprintf(stderr, "dvm: partition mode %d, %d operators a sub-kernel: %s\n", mode, limit, e2.what());
+          }
+        }
+      }
     }
   }
   k_->part_mode_ = 3;

@@ -95,7 +95,7 @@ bool Compiler::CanJoin(int a, const NDObject *o) {
   if (ai.over_parts != 0 && o->numel() > ai.over_parts) return false;
   if (o->kind == kObjReduce && LevelIn(a, o) < 8 && ai.red_at_level[LevelIn(a, o)] >= 2) return false;
   if (o->kind == kObjMatMul) return false;
-  if (ai.n_ops >= kMaxAreaOps && !IsStoreLike(o)) return false;  // long graphs are cut into several launches
+  if (ai.n_ops >= area_ops_limit_ && !IsStoreLike(o)) return false;  // long graphs are cut into several launches
   if (ai.attn >= 0) return o->kind == kObjStore && (o->in[0] == attn_groups_[ai.attn].m2 || o == attn_groups_[ai.attn].out_store);
   if (ai.cube) {
     if (!IsPointwiseKind(o->kind)) return false;

@@ -546,6 +546,7 @@ void Compiler::ChooseSchedule() {
     hdr_.sched = VS_POINTWISE;
     if (n_k <= 64 * U) threads = 64;
     else if (n_k <= 128 * U) threads = 128;
+    if (threads > pw_threads_cap_) threads = pw_threads_cap_;  // (fewer lanes: more V register slots for each)
     hdr_.n_items = static_cast<uint32_t>((n_k + static_cast<uint64_t>(threads) * U - 1) / (threads * U));
     n_sec_ = 1;
   } else if (inner_red) {

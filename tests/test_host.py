@@ -731,3 +731,32 @@ def test_clone_carries_gathers_onehots_padded_stores_and_element_any():
     strip = lambda d: "\n".join(x for x in d.splitlines() if "@0x" not in x)
     assert strip(t2.das()) == strip(t.das()), t2.das()
     assert "r[1,32]" in t2.das() and "gather_load.fp32" in t2.das() and "positions" in t2.das(), t2.das()
+
+
+def test_a_wide_expression_tree_gets_more_registers_before_it_is_cut():
+    # a pointwise graph that holds more values at once than a 256-lane workgroup has V register slots for: compiled
+    # again with workgroups of 128 lanes (twice the slots per lane), and only if that fails with fewer operators per
+    # sub-kernel; never one launch per operator
+    t = Tester("eager", run_mode="das")
+    x = t.load(np.zeros([300, 257], np.float32))
+    sig = lambda v: t.div(1.0, t.add(t.exp(t.mul(v, -1.0)), 1.0))
+    tanh = lambda v: t.sub(1.0, t.div(2.0, t.add(t.exp(t.mul(v, 2.0)), 1.0)))
+    a = t.add(t.mul(x, sig(x)), t.mul(sig(x), tanh(x)))
+    b = t.add(t.sub(t.mul(t.mul(x, 0.5), t.add(tanh(t.mul(x, 0.8)), 1.0)), t.maximum(x, 0.0)), t.select(t.greater(x, 0.0), x, t.mul(x, 0.1)))
+    c = t.select(t.greater(x, 0.5), a, t.mul(b, 2.0))
+    t.store(t.sub(t.div(t.maximum(c, t.mul(x, -1.0)), t.add(t.abs(x), 1.0)), t.sub(1.5, x)))
+    t.store(t.less_equal(x, 0.0))
+    t.codegen()
+    assert t.num_launches() == 1 and "threads=128" in t.das(), t.das()
+    t.codegen()  # (the kernel remembers what it needed)
+    assert t.num_launches() == 1
+    # forty values alive at once do not fit any workgroup: a few launches, not forty
+    t = Tester("eager", run_mode="das")
+    x = t.load(np.zeros([64, 256], np.float32))
+    vals = [t.exp(t.mul(x, float(i + 1))) for i in range(40)]
+    acc = vals[0]
+    for i in range(39, 0, -1):
+        acc = t.add(t.mul(acc, vals[i]), vals[(i * 7) % 40])
+    t.store(acc)
+    t.codegen()
+    assert 1 < t.num_launches() <= 16, t.num_launches()
