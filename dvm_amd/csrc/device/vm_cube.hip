@@ -852,8 +852,9 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
             case VB_MUL: acc = acc * src; break;
             case VB_DIV: acc = acc / src; break;
             case VB_RDIV: acc = src / acc; break;
-            case VB_DIV_APPROX: FOR_SE acc[q] = __fdividef(acc[q], src[q]); break;
-            case VB_RDIV_APPROX: FOR_SE acc[q] = __fdividef(src[q], acc[q]); break;
+            // (v_rcp_f32 and a multiply; the library's __fdividef is the full IEEE division, ten instructions)
+            case VB_DIV_APPROX: FOR_SE acc[q] = acc[q] * __builtin_amdgcn_rcpf(src[q]); break;
+            case VB_RDIV_APPROX: FOR_SE acc[q] = src[q] * __builtin_amdgcn_rcpf(acc[q]); break;
             case VB_MIN: FOR_SE acc[q] = acc[q] < src[q] ? acc[q] : src[q]; break;
             case VB_MAX: FOR_SE acc[q] = acc[q] > src[q] ? acc[q] : src[q]; break;
             case VB_AND: if constexpr (!SLIM) FOR_SE acc[q] = (acc[q] != 0.0f && src[q] != 0.0f) ? 1.0f : 0.0f; break;
@@ -922,7 +923,7 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
           case VU_SQRT_APPROX: FOR_SE acc[q] = __builtin_amdgcn_sqrtf(acc[q]); break;
           case VU_ABS: FOR_SE acc[q] = fabsf(acc[q]); break;
           case VU_LOG: if constexpr (!SLIM) acc = by_halves<SL>(acc, math_log); break;
-          case VU_LOG_APPROX: FOR_SE acc[q] = __logf(acc[q]); break;
+          case VU_LOG_APPROX: FOR_SE acc[q] = __builtin_amdgcn_logf(acc[q]) * 0.6931471805599453f; break;  // (v_log_f32 is log2; the library's __logf is the exact one)
           case VU_EXP: if constexpr (!SLIM) acc = by_halves<SL>(acc, math_exp); break;
           case VU_EXP_SCALED:  // the product is a value of its own: rounded to fp32, never contracted into what follows
             if constexpr (!SLIM) {
@@ -940,6 +941,17 @@ __device__ __forceinline__ void run_epilogue(typename SlabVec<SL>::type acc, con
               float y = acc[q] * __uint_as_float(imm);
               asm volatile("" : "+v"(y));
               acc[q] = __expf(y);
+            }
+            break;
+          case VU_SILU_APPROX:
+          case VU_SIGMOID_APPROX:
+            FOR_SE {
+              float y = acc[q] * __uint_as_float(imm);
+              asm volatile("" : "+v"(y));  // (the product is a value of its own, as in the separate instructions)
+              float d = __expf(y) + 1.0f;
+              asm volatile("" : "+v"(d));
+              const float r = __builtin_amdgcn_rcpf(d);
+              acc[q] = sub == VU_SILU_APPROX ? acc[q] * r : r;
             }
             break;
           case VU_ISFINITE: if constexpr (!SLIM) FOR_SE acc[q] = isfinite(acc[q]) ? 1.0f : 0.0f; break;

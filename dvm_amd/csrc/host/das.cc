@@ -39,7 +39,7 @@ void PrintShape(std::ostringstream &os, const NDObject *o) {
 const char *kMemTypes[] = {"bool", "fp16", "bf16", "fp32", "int32", "positions"};
 const char *kBinF[] = {"Add", "Sub", "RSub", "Mul", "Div", "RDiv", "Min", "Max", "And", "Or", "Pow", "RPow", "Div~", "RDiv~"};
 const char *kBinI[] = {"Add", "Sub", "RSub", "Mul", "Min", "Max", "WrapIndex"};
-const char *kUn[] = {"Sqrt", "Abs", "Log", "Exp", "IsFinite", "Round", "Floor", "Ceil", "Trunc", "Abs", "Exp", "Exp~", "Exp~", "Log~", "Sqrt~"};
+const char *kUn[] = {"Sqrt", "Abs", "Log", "Exp", "IsFinite", "Round", "Floor", "Ceil", "Trunc", "Abs", "Exp", "Exp~", "Exp~", "Log~", "Sqrt~", "SiLU~", "Sigmoid~"};
 const char *kCmp[] = {"Eq", "Ne", "Gt", "Ge", "Lt", "Le"};
 const char *kRnd[] = {"fp32", "fp16", "bf16", "?"};
 const char *kRed[] = {"sum", "max", "min"};
@@ -142,6 +142,10 @@ std::string &VKernel::DisAssemble() {
             if (static_cast<uint32_t>(w) & VI_ENDS) os << "  ; endsweep";
             break;
           case VOP_UN:
+            if (sub == VU_SILU_APPROX || sub == VU_SIGMOID_APPROX) {
+              os << kUn[sub] << "." << kRnd[VI_RND(w)] << (sub == VU_SILU_APPROX ? " acc / (exp(acc * #0x" : " 1 / (exp(acc * #0x") << std::hex << VI_IMM(w) << std::dec << ") + 1)";
+              break;
+            }
             if (sub == VU_EXP_SCALED || sub == VU_EXP_SCALED_APPROX) {
               os << kUn[sub] << "." << kRnd[VI_RND(w)] << " acc * #0x" << std::hex << VI_IMM(w) << std::dec;
               break;

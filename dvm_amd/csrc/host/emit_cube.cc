@@ -125,6 +125,41 @@ uint32_t Compiler::FuseCubeEpilogue() {
     }
     w = (w & ~0xff00ull) | (static_cast<uint64_t>(sub) << 8);
   }
+  // x / (exp(x * c) + 1) and 1 / (exp(x * c) + 1), all in fp32: one dispatch instead of four / three (SiLU, sigmoid)
+  if (k_->tuning_.cube_fuse_act != 0) {
+    std::vector<uint64_t> &out2 = scratch_code_;
+    out2.clear();
+    auto is_exp = [](uint64_t w) { return VI_OP(w) == VOP_UN && VI_SUB(w) == VU_EXP_SCALED_APPROX && VI_RND(w) == 0; };
+    auto is_add1 = [](uint64_t w) { return VI_OP(w) == VOP_BINF && VI_SUB(w) == VB_ADD && VI_KIND(w) == VK_IMM && VI_RND(w) == 0 && VI_IMM(w) == 0x3f800000u; };
+    for (size_t i = 0; i < code_.size(); ++i) {
+      const uint64_t w = code_[i];
+      if (i + 3 < code_.size() && VI_OP(w) == VOP_STR && is_exp(code_[i + 1]) && is_add1(code_[i + 2])) {
+        const uint64_t d = code_[i + 3];
+        // the parked value must not be read again later (it is only this division's numerator)
+        bool reread = false;
+        for (size_t j = i + 4; j < code_.size() && !reread; ++j) {
+          const uint64_t v = code_[j];
+          if (VI_OP(v) == VOP_STR && VI_A(v) == VI_A(w)) break;
+          if ((VI_OP(v) == VOP_LDR || (VI_OP(v) >= VOP_SRC_BASE && VI_KIND(v) == VK_REG)) && VI_A(v) == VI_A(w)) reread = true;
+        }
+        if (!reread && VI_OP(d) == VOP_BINF && VI_SUB(d) == VB_RDIV_APPROX && VI_KIND(d) == VK_REG && VI_A(d) == VI_A(w) && VI_RND(d) == 0) {
+          out2.push_back(VI_MAKE(VOP_UN, VU_SILU_APPROX, 0, 0, 0, VI_IMM(code_[i + 1])));
+          i += 3;
+          continue;
+        }
+      }
+      if (i + 2 < code_.size() && is_exp(w) && is_add1(code_[i + 1])) {
+        const uint64_t d = code_[i + 2];
+        if (VI_OP(d) == VOP_BINF && VI_SUB(d) == VB_RDIV_APPROX && VI_KIND(d) == VK_IMM && VI_RND(d) == 0 && VI_IMM(d) == 0x3f800000u) {
+          out2.push_back(VI_MAKE(VOP_UN, VU_SIGMOID_APPROX, 0, 0, 0, VI_IMM(w)));
+          i += 2;
+          continue;
+        }
+      }
+      out2.push_back(w);
+    }
+    code_.swap(out2);
+  }
   return VCF_APPROX_MATH;
 }
 
@@ -447,7 +482,8 @@ void Compiler::CompileCube(int a) {
           if (sub != VC_RND) slim = false;
           break;
         case VOP_UN:
-          if (sub != VU_ABS && sub != VU_EXP_APPROX && sub != VU_EXP_SCALED_APPROX && sub != VU_LOG_APPROX && sub != VU_SQRT_APPROX) slim = false;
+          if (sub != VU_ABS && sub != VU_EXP_APPROX && sub != VU_EXP_SCALED_APPROX && sub != VU_LOG_APPROX && sub != VU_SQRT_APPROX &&
+              sub != VU_SILU_APPROX && sub != VU_SIGMOID_APPROX) slim = false;
           break;
         case VOP_BINF: {
           const uint32_t b = sub & 0x3fu;

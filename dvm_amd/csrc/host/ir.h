@@ -236,6 +236,7 @@ struct Tuning {
   int red_split = -1;    // DVM_RED_SPLIT=0: never share a reduce between workgroups; N >= 2: N parts whenever the graph allows
   int cube_splitk = -1;  // DVM_CUBE_SPLITK=0: never split the k axis; N >= 2: split it N ways whenever the shape allows
   int cube_dump16 = -1; // DVM_CUBE_DUMP16=0: the matmul epilogue always reads the tile back as fp32, half a tile per pass
+  int cube_fuse_act = -1;  // DVM_CUBE_FUSE_ACT=0: x / (exp(x * c) + 1) and 1 / (exp(x * c) + 1) of a matmul epilogue stay separate instructions
   int cube_exact = -1;  // DVM_CUBE_EXACT=1: never the hardware approximations of exp, log, sqrt, division in a matmul epilogue
   int attn_waves = -1;  // DVM_ATTN_WAVES=4
   bool debug = false;   // DVM_DEBUG: node dump in compile errors

@@ -42,6 +42,7 @@ void Tuning::Read() {
   red_split = num("DVM_RED_SPLIT");
   red_split_turn = num("DVM_RED_SPLIT_TURN");
   attn_waves = num("DVM_ATTN_WAVES");
+  cube_fuse_act = num("DVM_CUBE_FUSE_ACT");
   debug = std::getenv("DVM_DEBUG") != nullptr;
 }
 

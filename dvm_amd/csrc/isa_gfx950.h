@@ -128,6 +128,10 @@ enum {
   // of a multiply by a constant followed by Exp). The _APPROX forms use the hardware approximations (v_exp_f32,
   // v_log_f32, v_sqrt_f32: one ulp of fp32); the host picks them under VCF_APPROX_MATH.
   VU_EXP_SCALED, VU_EXP_APPROX, VU_EXP_SCALED_APPROX, VU_LOG_APPROX, VU_SQRT_APPROX,
+  // matmul epilogues under VCF_APPROX_MATH only: the four (three) instructions of x / (exp(x * imm) + 1) and of
+  // 1 / (exp(x * imm) + 1) in one dispatch, every intermediate rounded to fp32 as the separate instructions do
+  // (SiLU and the logistic function with imm = -1); the host joins them when none of the four rounds to a 16-bit type
+  VU_SILU_APPROX, VU_SIGMOID_APPROX,
 };
 // compare sub-ops (same order as dvm::BinaryType kEqual..kLessEqual); +VCMP_INT for int32 operands
 enum { VCMP_EQ = 0, VCMP_NE, VCMP_GT, VCMP_GE, VCMP_LT, VCMP_LE, VCMP_INT = 8 };

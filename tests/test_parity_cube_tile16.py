@@ -85,3 +85,44 @@ def test_split_k_sum_goes_the_one_pass_route_too(monkeypatch):
     ref, _, _ = _run(monkeypatch, False, "bfloat16", 1024, 1024, 16384, "float32", "relu")
     assert "split-k sum" in das_on and "tile-as-16-bit" in das_on, das_on
     assert np.array_equal(got, ref), das_on
+
+
+@pytest.mark.parametrize("act", ["silu", "sigmoid", "silu_as_product"])
+@pytest.mark.parametrize("dt", ["float16", "bfloat16"])
+@pytest.mark.parametrize("shape", [(512, 384, 128), (300, 520, 64), (2048, 1024, 256)])
+def test_fused_activation_instructions_give_the_bits_of_the_separate_ones(monkeypatch, act, dt, shape):
+    # x / (exp(-x) + 1) and 1 / (exp(-x) + 1) behind a matmul are one epilogue instruction each (VU_SILU_APPROX,
+    # VU_SIGMOID_APPROX): the same fp32 operations in the same order as the three or four they replace
+    m, n, k = shape
+    rng = np.random.default_rng(m + n + k)
+    a = (rng.standard_normal([m, k]) * 0.3).astype(np.float32)
+    b = (rng.standard_normal([k, n]) * 0.3).astype(np.float32)
+    bias = rng.standard_normal([n]).astype(np.float32)
+
+    def run():
+        t = Tester("mix")
+        la, lb = (t.load(v.astype(np.float16)) if dt == "float16" else t.load(v, dt) for v in (a, b))
+        h = t.add(t.cast(t.matmul(la, lb, False, False), "float32"), t.load(bias))
+        if act == "silu":
+            y = t.div(h, t.add(t.exp(t.mul(h, -1.0)), 1.0))
+        elif act == "sigmoid":
+            y = t.div(1.0, t.add(t.exp(t.mul(h, -1.0)), 1.0))
+        else:
+            y = t.mul(h, t.div(1.0, t.add(t.exp(t.mul(h, -1.0)), 1.0)))
+        out = t.store(t.cast(y, dt))
+        t.run()
+        return t.output(out), t.das()
+
+    fused, das = run()
+    assert ("SiLU~" in das) == (act == "silu") and ("Sigmoid~" in das) == (act != "silu"), das
+    monkeypatch.setenv("DVM_CUBE_FUSE_ACT", "0")
+    apart, das0 = run()
+    assert "SiLU~" not in das0 and "Sigmoid~" not in das0 and "RDiv~" in das0, das0
+    assert np.array_equal(fused.view(np.uint16), apart.view(np.uint16))
+    # and against float64
+    h64 = a.astype(np.float64) @ b.astype(np.float64)
+    ref = None
+    if dt == "float16":
+        h64 = (a.astype(np.float16).astype(np.float64) @ b.astype(np.float16).astype(np.float64)).astype(np.float16).astype(np.float64) + bias
+        ref = h64 / (np.exp(-h64) + 1) if act != "sigmoid" else 1 / (np.exp(-h64) + 1)
+        assert np.allclose(fused.astype(np.float64), ref, rtol=3e-3, atol=3e-3)
