@@ -227,8 +227,8 @@ def test_matmul_epilogue_is_one_cube_program():
     t.codegen()
     das = t.das()
     assert das.count("== sub-kernel") == 1 and "entry cube bf16 m=512 n=384 k=256" in das, das
-    # exp(-h) is one instruction, and with a 16-bit store and continuous operators it is the hardware's exp
-    assert "mmad acc, A, B" in das and "Exp~.fp32 acc * #0xbf800000" in das and "RDiv~.fp32" in das, das
+    # with a 16-bit store and continuous operators x / (exp(-x) + 1) is one instruction on the hardware's exp and reciprocal
+    assert "mmad acc, A, B" in das and "SiLU~.fp32 acc / (exp(acc * #0xbf800000) + 1)" in das, das
     assert "store.bf16" in das and "strides n=1 m=0" in das, das
     # the fp32 accumulators are rounded to the operand type before the epilogue sees them (src/vm_aic.cce:34-470)
     assert das.index("cast.round.bf16") < das.index("Add.fp32"), das
