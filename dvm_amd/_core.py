@@ -596,7 +596,13 @@ class PyKernel(Kernel):
 
     def codegen(self, pass_names=None):
         """Normalize + CodeGen. `pass_names` is the reference's argument (src/pybind_api.cc:616): the pipeline here is
-        fixed and the generated code does not depend on it (Tester.set_passes checks the names)."""
+        fixed and the generated code does not depend on it (Tester.set_passes checks the names).
+
+        A dynamic kernel whose placeholder loads have no shape yet (negative dims, nothing bound) has nothing to
+        generate code for: the call returns and the run that follows the inputs generates it. (The reference's
+        graph kernel compiles symbolic shapes at this point, tests/ut/test_split_sym_graph.py:193-214.)"""
+        if any(d < 0 for ref in self._load_shape.values() for d in ref.shape()):
+            return
         _check(_lib.dvm_rt_codegen(self._rt))
 
     def jit_us(self):

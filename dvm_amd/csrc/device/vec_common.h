@@ -74,7 +74,9 @@ __device__ __forceinline__ float exp_f32(float x) {
   const float kLog2eHi = 1.44269502162933349609375f, kLog2eLo = 1.925963033500011e-08f, kLn2 = 0.693147182464599609375f;
   const float hi = x * kLog2eHi;
   float lo = __builtin_fmaf(x, kLog2eLo, __builtin_fmaf(x, kLog2eHi, -hi));
-  lo = __builtin_fabsf(x) < __builtin_huge_valf() ? lo : 0.0f;  // (inf - inf above)
+  // (inf - inf above when the product overflows, which a finite x beyond 2.4e38 does as well as an infinite one:
+  // the lowest float a masked softmax fills in)
+  lo = __builtin_fabsf(hi) < __builtin_huge_valf() ? lo : 0.0f;
   const float p = __builtin_amdgcn_exp2f(hi);
   return p < __builtin_huge_valf() ? __builtin_fmaf(p * kLn2, lo, p) : p;  // (inf * lo; a NaN passes through)
 }

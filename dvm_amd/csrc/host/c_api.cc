@@ -176,6 +176,9 @@ void ParseKernelType(const std::string &s, KernelType *type, uint32_t *flags) {
       *flags |= kSpeculate;
     } else if (f == "priv1" && *type == kVector) {  // with "spec": the stages are found automatically (no SpecNext calls)
       *flags |= kPrivate1;
+    } else if (f == "priv1" || f == "priv2" || f == "opt_fractal") {
+      // The reference picks between implementations of one kernel type with these (src/dvm.cc:1059-1106: the graph
+      // kernel behind "split:priv1"; a fractal layout of its matrix unit), never between meanings: accepted, no effect.
     } else if (!f.empty()) {
       throw std::runtime_error("DVM EXCEPTION. reason: kernel flag '" + f + "' is not supported by the gfx950 backend");
     }

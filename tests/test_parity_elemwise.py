@@ -19,6 +19,25 @@ def test_unary(dt):  # tests/ut/test_elemwise.py:24-35
                golden=[np.sqrt(x), np.abs(x), np.log(x), np.exp(x), np.reciprocal(x)])
 
 
+def test_exp_at_the_ends_of_the_range():
+    # the lowest float is what a masked softmax fills in (tests/ut/test_pass_insert_removepad.py:99): its product
+    # with log2(e) overflows although the value is finite; results below the smallest normal number may come out as 0
+    fmax = np.finfo(np.float32).max
+    vals = np.array([-fmax, fmax, -3e38, -2.4e38, -2.3e38, 2.4e38, -np.inf, np.inf, np.nan, -104.0, -103.0, -88.0,
+                     -87.3, 0.0, -0.0, 88.0, 88.7, 89.0, 1e-30, -1e-30], np.float32)
+    x = np.tile(vals, 64).reshape(64, -1)
+    with np.errstate(over="ignore"):
+        gold = np.exp(x)
+
+    masked = np.tile(np.array([-fmax, -3e38, -2.4e38, -104.0, -88.0, 0.0, 1.0, 5.0], np.float32), 512).reshape(4, -1)
+    with np.errstate(over="ignore"):
+        soft = np.exp(masked - masked.max(axis=1, keepdims=True))
+
+    def g(k, a, m):  # alone, after an arithmetic operator, and in the sweep behind a row maximum
+        return [k.exp(a), k.exp(k.mul(a, 1.0)), k.exp(k.sub(m, k.max(m, (1,), True)))]
+    run_parity(g, [x, masked], golden=[gold, gold, soft], golden_eps=1e-5)
+
+
 @pytest.mark.parametrize("dt", [np.float16, np.float32])
 def test_binary(dt):  # tests/ut/test_elemwise.py:38-54
     x, y = np.full([32, 1024], 0.5, dt), np.full([32, 1024], 0.4, dt)
