@@ -220,8 +220,17 @@ void ora_select_32(const uint32_t *cond, const uint32_t *a, const uint32_t *b, u
 void ora_round_f(int t, const float *x, float *y, size_t n) {
   for (size_t i = 0; i < n; ++i) y[i] = round_to(t, x[i]);
 }
+/* The reference's functor is a C cast (src/vm_gpu.cu:299-301). Its device compiler turns that into the saturating
+ * conversion of the PTX ISA (cvt.rzi.s32.f32: truncation toward zero, a value beyond the range gives the nearest end
+ * of the range, NaN gives 0); the same cast on the host is undefined for those inputs, so they are spelled out. */
+static int32_t f_to_i32(float x) {
+  if (x != x) return 0;
+  if (x >= 2147483648.0f) return INT32_MAX;
+  if (x <= -2147483648.0f) return INT32_MIN;
+  return (int32_t)x;
+}
 void ora_f_to_i32(const float *x, int32_t *y, size_t n) {
-  for (size_t i = 0; i < n; ++i) y[i] = (int32_t)x[i]; /* C truncation, src/vm_gpu.cu:299-301 */
+  for (size_t i = 0; i < n; ++i) y[i] = f_to_i32(x[i]);
 }
 void ora_i32_to_f(int t, const int32_t *x, float *y, size_t n) {
   for (size_t i = 0; i < n; ++i) y[i] = round_to(t, (float)x[i]);

@@ -130,6 +130,15 @@ def test_int32_wraparound_and_casts():
     assert np.array_equal(k.output(k.cast(k.load(x[0]), "float32")), x[0].astype(np.float32))
     h = rng.normal(0, 10, 10000).astype(np.float16)
     assert np.array_equal(k.output(k.cast(k.load(h), "int32")), np.trunc(h.astype(np.float32)).astype(np.int32))
+    # beyond the range of int32 the conversion saturates and NaN gives 0: what the reference's C cast
+    # (src/vm_gpu.cu:299-301) means on its device (PTX cvt.rzi.s32.f32); known answers, not a host cast (undefined there)
+    edge = np.array([np.inf, -np.inf, np.nan, 3e9, -3e9, 2147483648.0, 2147483520.0, -2147483648.0, -2147483904.0,
+                     1.9, -1.9, -0.0], np.float32)
+    want = np.array([2 ** 31 - 1, -2 ** 31, 0, 2 ** 31 - 1, -2 ** 31, 2 ** 31 - 1, 2147483520, -2 ** 31, -2 ** 31, 1, -1, 0],
+                    np.int64).astype(np.int32)
+    assert np.array_equal(k.output(k.cast(k.load(edge), "int32")), want)
+    assert np.array_equal(k.output(k.cast(k.load(np.array([np.inf, -np.inf, np.nan, 65504.0], np.float16)), "int32")),
+                          np.array([2 ** 31 - 1, -2 ** 31, 0, 65504], np.int64).astype(np.int32))
     r = np.array([0.5, 1.5, 2.5, -0.5, -1.5, 2.4999, 3.5001], np.float32)
     assert np.array_equal(k.output(k.round(k.load(r))), np.round(r))
     assert np.array_equal(k.output(k.floor(k.load(f))), np.floor(f))

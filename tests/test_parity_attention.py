@@ -66,6 +66,20 @@ def test_attention_fused(monkeypatch, shape, dt, waves):
     assert np.allclose(got, want, rtol=1e-2, atol=1e-2), np.abs(got - want).max()
 
 
+@pytest.mark.parametrize("dt", ["float16", "bfloat16"])
+@pytest.mark.parametrize("spread,d", [(20.0, 128), (20.0, 64), (0.0, 128), (6.0, 64)])
+def test_attention_sharp_and_flat_softmax(dt, spread, d):
+    # scores hundreds apart (the weights of a row are one key's, the rest underflow) and scores all equal
+    rng = np.random.default_rng(int(spread) + d)
+    conv = (lambda x: x.astype(np.float16)) if dt == "float16" else _bf16
+    q, k, v = (conv(rng.standard_normal((2, n, d)) * s) for n, s in ((300, spread), (520, spread), (520, 1.0)))
+    if spread > 0:
+        k[:, 7, :] = q[:, 0, :]  # query 0 has one key far above the rest
+    got, want = _fused(q, k, v, dt), np_attention(q, k, v)
+    assert not np.isnan(got).any()
+    assert np.allclose(got, want, rtol=2e-2, atol=2e-2), np.abs(got - want).max()
+
+
 def test_attention_fused_constant_values_and_key_order():
     # softmax weights sum to one: with every row of V equal to c the output rows are c, at any size;
     # and the result does not depend on the order of the keys

@@ -190,6 +190,18 @@ def test_casts():  # tests/ut/test_cast.py:26-165
                golden=(h.astype(np.float32) + np.float32(0.5)).astype(np.int32).astype(np.float16), eps=0)
 
 
+def test_float_to_int_beyond_the_range_saturates():
+    # src/vm_gpu.cu:299-301 on the reference's device: the nearest end of the range, 0 for NaN
+    edge = np.tile(np.array([np.inf, -np.inf, np.nan, 3e9, -3e9, 2147483648.0, 2147483520.0, -2147483648.0, -2147483904.0,
+                             1.9, -1.9, -0.0], np.float32), 100)
+    want = np.tile(np.array([2 ** 31 - 1, -2 ** 31, 0, 2 ** 31 - 1, -2 ** 31, 2 ** 31 - 1, 2147483520, -2 ** 31, -2 ** 31, 1, -1, 0],
+                            np.int64).astype(np.int32), 100)
+    half = np.tile(np.array([np.inf, -np.inf, np.nan, 65504.0, -1.5], np.float16), 100)
+    want_half = np.tile(np.array([2 ** 31 - 1, -2 ** 31, 0, 65504, -1], np.int64).astype(np.int32), 100)
+    run_parity(lambda k, a, h: [k.cast(a, "int32"), k.cast(h, "int32"), k.cast(k.mul(a, 1.0), "int32")], [edge, half],
+               golden=[want, want_half, want], golden_eps=0)
+
+
 @pytest.mark.parametrize("shape", [(32, 32), (1024, 32), (1024, 2000)])
 @pytest.mark.parametrize("dt", [np.int32, np.float32, np.float16, np.bool_])
 def test_compare(shape, dt):  # tests/ut/test_cmp.py:24-170
