@@ -4,6 +4,7 @@ bf16 operands). NumPy expectations as there, the CPU oracle as second opinion; i
 import numpy as np
 import pytest
 
+from dvm_amd.tester import Tester
 from tests.util import run_graph
 
 pytestmark = pytest.mark.gpu
@@ -65,3 +66,33 @@ def test_broadcast_then_reduce():  # :279-288 (the tile hint there is advice for
     a = np.random.default_rng(6).normal(0, 0.1, [40, 20, 17, 1]).astype(np.float32)
     run_graph("", lambda k: [(k.store(k.sum(k.broadcast(k.load(a), [40, 20, 17, 32]), (1,), True)),
                               np.sum(np.broadcast_to(a, [40, 20, 17, 32]), (1,), keepdims=True), 1e-5)])
+
+
+@pytest.mark.parametrize("lead", [1024, 511])
+@pytest.mark.parametrize("src,dst,tiles", [
+    ([2, 1, 1], [2, 96, 1], [(2, 2, 2), (1, 1, 48)]),
+    ([2, 1, 4], [2, 3, 4], [(2, 2, 2), (1, 1, 3), (0, 0, 4)]),
+    ([2, 1, 4, 1, 1], [2, 3, 4, 6, 1], [(4, 4, 2), (3, 3, 3), (2, 2, 4), (1, 1, 3)]),
+    ([2, 1, 4, 1, 2], [2, 3, 4, 5, 2], [(4, 4, 2), (3, 3, 3), (2, 2, 4), (1, 1, 5), (0, 1, 2)]),
+])
+def test_value_stored_before_and_after_its_broadcast(lead, src, dst, tiles):  # :184-256 (innermost extent a multiple of `lead`)
+    src, dst = src[:-1] + [src[-1] * lead], dst[:-1] + [dst[-1] * lead]
+    a = np.random.default_rng(lead + len(src)).standard_normal(src, dtype=np.float32)
+
+    def g(k):
+        v = k.add(k.load(a), 0.5)
+        out = [(k.store(v), a + np.float32(0.5), 0), (k.store(k.broadcast(v, dst)), np.broadcast_to(a + np.float32(0.5), dst), 0)]
+        for h in tiles:  # the reference's tests fix a tiling by hand here: accepted, without effect
+            if hasattr(k, "tile"):
+                k.tile(*h)
+        return out
+    run_graph("", g)
+
+
+@pytest.mark.parametrize("src,dst", [((8, 1, 257, 1), (8, 5, 257, 129)), ((1, 9, 1, 257), (6, 9, 33, 257)),
+                                     ((4, 1, 8, 1, 129), (4, 3, 8, 17, 129))])
+def test_broadcast_of_64_bit_integers_along_two_axes(src, dst):  # :93-105
+    a = np.random.default_rng(len(src)).integers(0x10000000, 0x2000000000, size=src, dtype=np.int64)
+    t = Tester("")
+    t.store_expect(t.broadcast(t.load(a), list(dst)), np.broadcast_to(a, dst))
+    assert t.run_check()

@@ -67,3 +67,71 @@ def test_seventeen_inputs_sixteen_outputs():  # :81-95
             out.append((k.store(x), result, None))
         return out
     run_graph("", g)
+
+
+def test_three_stores_of_two_expressions_in_reverse_order():  # tests/ut/test_codegen.py:66-82
+    rng = np.random.default_rng(1)
+    a0, a1 = rng.standard_normal([1024, 1024], dtype=np.float32), rng.standard_normal([1024, 1024], dtype=np.float32)
+
+    def g(k):
+        x0, x1 = k.load(a0), k.load(a1)
+        b, a, f = k.sub(x0, x1), k.sub(x0, x1), k.sub(x1, x0)
+        return [(k.store(a), a0 - a1, 0), (k.store(f), a1 - a0, 0), (k.store(b), a0 - a1, 0)]
+    run_graph("vector", g)
+
+
+def test_value_with_three_readers_of_different_age():  # tests/ut/test_codegen.py:102-113 (run here, listed there)
+    rng = np.random.default_rng(2)
+    x = np.abs(rng.standard_normal([32, 1024])).astype(np.float16) + np.float16(0.5)
+
+    def g(k):
+        v = k.load(x)
+        root, mag = k.sqrt(v), k.abs(v)
+        return [(k.store(k.add(k.add(root, mag), k.reciprocal(mag))), np.sqrt(x) + np.abs(x) + np.reciprocal(np.abs(x)), 2e-3)]
+    run_graph("vector", g)
+
+
+def test_tensor_without_elements():  # tests/ut/test_codegen.py:116-138
+    t = Tester("vector")
+    out = t.store(t.mul(t.load(np.full([10, 0, 2], 0.1, np.float32)), 0.1))
+    t.run()
+    assert out.shape() == (10, 0, 2) and t.output(out).shape == (10, 0, 2)
+    t = Tester("vector")
+    out = t.store_expect(t.sum(t.add(t.load(np.full([10, 0, 2], 0.01, np.float32)), 0.1), (1,), True), 0.0)
+    assert t.run_check()
+    assert out.shape() == (10, 1, 2)
+
+
+def test_dynamic_load_that_changes_rank_and_loses_its_elements():  # tests/ut/test_codegen.py:141-165
+    t = Tester("vector:dyn")
+    x1 = t.load([-1], "float32")
+    out = t.store(t.sum(t.add(x1, 0.1), (1,), True))
+    t.input(x1, np.full([10, 0, 20], 0.01, np.float32))
+    t.run()
+    assert t.check(out, 0.0) and out.shape() == (10, 1, 20)
+    t.input(x1, np.full([0, 10, 20], 0.01, np.float32))
+    t.run()
+    assert out.shape() == (0, 1, 20)
+    t.input(x1, np.full([10, 40, 20], 0.01, np.float32))
+    t.run()
+    assert t.check(out, (np.float32(0.01) + np.float32(0.1)) * 40) and out.shape() == (10, 1, 20)
+
+
+def test_dynamic_rows_of_4096_around_a_multiple_of_the_workgroup_count():  # tests/ut/test_dynamic_shape.py:136-162
+    t = Tester("vector:dyn")
+    p0, p1 = t.load([-1], "float16"), t.load([-1], "float16")
+    y0 = t.add(p0, p1)
+    out0 = t.store(y0)
+    y1 = t.cast(y0, "float32")
+    out1 = t.store(y1)
+    out2 = t.store(t.sum(t.mul(y1, y1), [2], True))
+    np.random.seed(3)
+    for rows in (2685, 2686, 2687):
+        a = Tester.fast_random_normal(0, 1, [1, rows, 4096]).astype(np.float16)
+        b = Tester.fast_random_normal(0, 1, [1, rows, 4096]).astype(np.float16)
+        t.input(p0, a)
+        t.input(p1, b)
+        t.run()
+        s = (a + b).astype(np.float32)
+        assert t.check(out0, a + b) and t.check(out1, s)
+        assert t.check(out2, np.sum(s * s, (2,), keepdims=True), 1e-4)
