@@ -282,3 +282,31 @@ def test_operators_on_a_value_of_rank_zero():  # src/ops.cc:3080-3117: a reduce 
     assert outs[0].shape == () and outs[1].shape == () and outs[2].shape == (257,)
     bf = Tester.convert_from_bf16(Tester.convert_to_bf16(np.float32(1.5)))
     assert bf.shape == () and float(bf) == 1.5
+
+
+@pytest.mark.parametrize("n,hint", [(256 * 50 + 100, (0, 0, 51, 256)), (249 * 50 + 223, (0, 0, 51, 249)), (501 * 20, (0, 0, 20, 501))])
+def test_sum_of_a_long_vector_with_a_tiling_hint(n, hint):  # tests/ut/test_reduce.py:310-325 (the hint fixes the reference's tiles)
+    a = np.random.default_rng(n).standard_normal([n], dtype=np.float32)
+    t = Tester()
+    t.store_expect(t.sum(t.load(a), (0,), True), np.sum(a.astype(np.float64), axis=(0,), keepdims=True), 1e-4)
+    t.tile(*hint)
+    assert t.run_check()
+
+
+def test_sum_over_both_axes_of_rows_of_two():  # tests/ut/test_reduce.py:328-338
+    rng = np.random.default_rng(8002)
+    a0, a1 = rng.standard_normal([8002, 2], dtype=np.float32), rng.standard_normal([8002, 1], dtype=np.float32)
+    t = Tester()
+    t.store_expect(t.sum(t.add(t.load(a0), t.load(a1)), [0, 1], False), np.sum((a0 + a1).astype(np.float64), axis=(0, 1)), 1e-4)
+    t.tile(1, 1, 8)
+    assert t.run_check()
+
+
+def test_sum_of_a_broadcast_stored_beside_its_input():  # tests/ut/test_reduce.py:296-307
+    a = (np.random.default_rng(12).standard_normal([32, 12, 1, 1]) * 0.5 - 0.5).astype(np.float32)
+    wide = np.broadcast_to(a, [32, 12, 111, 111]) + np.float32(0.1)
+    t = Tester()
+    x = t.add(t.broadcast(t.load(a), [32, 12, 111, 111]), 0.1)
+    t.store_expect(t.sum(x, [0, 2, 3], False), np.sum(wide.astype(np.float64), axis=(0, 2, 3)), 1e-4)
+    t.store_expect(x, wide)
+    assert t.run_check()
