@@ -309,13 +309,21 @@ def _back(k, n, x):
     return x if int(x.dtype()) == int(_DT[n.dtype]) else k.cast(x, _DT[n.dtype])
 
 
-def _scalar_binary(name):
+def _scalar_binary(name, widen=False):
+    """widen: arithmetic of a 16-bit tensor with a number happens in fp32 with the number as it is and is rounded
+    once, as torch's kernels do it (the DVM operator alone would first round the number to the tensor's type);
+    compares take the number in the tensor's type on both sides."""
     def build(k, n, a):
         fn = getattr(k, name)
         if len(a) == 2:
             return fn(a[0], a[1])
         side, s = n.const
-        return fn(s, a[0]) if side == "l" else fn(a[0], s)
+        x = a[0]
+        narrow = widen and int(x.dtype()) in (int(DataType.float16), int(DataType.bfloat16))
+        if narrow:
+            x = k.cast(x, DataType.float32)
+        out = fn(s, x) if side == "l" else fn(x, s)
+        return k.cast(out, _DT[n.dtype]) if narrow else out
     return build
 
 
@@ -327,8 +335,9 @@ def _in_f32(body):
 
 
 _BUILD = {
-    "add": _scalar_binary("add"), "sub": _scalar_binary("sub"), "mul": _scalar_binary("mul"), "div": _scalar_binary("div"),
-    "maximum": _scalar_binary("maximum"), "minimum": _scalar_binary("minimum"), "pow": _scalar_binary("pow"),
+    "add": _scalar_binary("add", True), "sub": _scalar_binary("sub", True), "mul": _scalar_binary("mul", True),
+    "div": _scalar_binary("div", True), "pow": _scalar_binary("pow", True),
+    "maximum": _scalar_binary("maximum"), "minimum": _scalar_binary("minimum"),
     "eq": _scalar_binary("equal"), "ne": _scalar_binary("not_equal"), "gt": _scalar_binary("greater"),
     "ge": _scalar_binary("greater_equal"), "lt": _scalar_binary("less"), "le": _scalar_binary("less_equal"),
     "abs": lambda k, n, a: k.abs(a[0]),
@@ -339,7 +348,7 @@ _BUILD = {
     "reciprocal": lambda k, n, a: k.reciprocal(a[0]),
     "rsqrt": _in_f32(lambda k, n, x: k.div(1.0, k.sqrt(x))),
     "relu": lambda k, n, a: k.maximum(a[0], 0.0),
-    "leaky_relu": lambda k, n, a: k.select(k.greater(a[0], 0.0), a[0], k.mul(a[0], float(n.const[0]))),
+    "leaky_relu": _in_f32(lambda k, n, x: k.select(k.greater(x, 0.0), x, k.mul(x, float(n.const[0])))),
     "sigmoid": _in_f32(lambda k, n, x: k.div(1.0, k.add(k.exp(k.mul(x, -1.0)), 1.0))),
     "silu": _in_f32(lambda k, n, x: k.div(x, k.add(k.exp(k.mul(x, -1.0)), 1.0))),
     # 1 - 2 / (exp(2x) + 1): finite at both ends (exp overflows to inf, 2 / inf is 0)

@@ -120,6 +120,20 @@ for i in range(4):
 assert lf.stats["compiled"] == 1 and lf.stats["flushes"] == 4, lf.stats
 print("cache: ok")
 
+# ---- a 16-bit tensor and a number: torch computes in fp32 with the number as it is and rounds once ----
+for dt in (torch.bfloat16, torch.float16):
+    h = rnd(300, 257, dtype=dt)
+    def numbers(h):
+        return [(h.abs() + 0.6762023455442653) * 0.9084074272936424, 2.0 - h, h / 3.0, F.leaky_relu(h, 0.1), h ** 2,
+                torch.where(h > 0.3, h, h * 1.3137085138672244)]
+    want = numbers(h)
+    with dvm.lazy_fusion() as lf:
+        got = numbers(h)
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        assert a.dtype == b.dtype and torch.equal(a, b), (dt, (a.float() - b.float()).abs().max())
+print("numbers: ok")
+
 # ---- long expressions are cut into segments; an exception inside the block leaves nothing pending ----
 t = rnd(1000)
 with dvm.lazy_fusion() as lf:
@@ -147,5 +161,5 @@ def test_lazy_fusion_of_eager_torch_programs():
     env = dict(os.environ, PYTHONPATH=root + os.pathsep + os.environ.get("PYTHONPATH", ""))
     done = subprocess.run([sys.executable, "-c", _SCRIPT], cwd=root, env=env, capture_output=True, text=True, timeout=280)
     assert done.returncode == 0, done.stdout + "\n" + done.stderr
-    for line in ("example: ok", "activations: ok", "rmsnorm: ok", "matmul: ok", "fallbacks: ok", "views: ok", "cache: ok", "segments: ok"):
+    for line in ("example: ok", "activations: ok", "rmsnorm: ok", "matmul: ok", "fallbacks: ok", "views: ok", "cache: ok", "numbers: ok", "segments: ok"):
         assert line in done.stdout, done.stdout + "\n" + done.stderr
