@@ -237,6 +237,13 @@ void Compiler::CompileCube(int a) {
       else *s0 = static_cast<uint32_t>(walk[d]);
     }
   };
+  if (M == 0 || N == 0 || h.nb0 == 0 || h.nb1 == 0) {  // an empty result: nothing to launch
+    prog_->skip = true;
+    return;
+  }
+  if (K == 0 && gmm == 0) {
+    Throw("DVM EXCEPTION. reason: a matmul over an empty k axis is not supported by the gfx950 backend (its result is the bias alone)");
+  }
   bool flip_a = false, flip_b = false;
   operand_layout(an, &flip_a, &h.lda, &h.a_sb0, &h.a_sb1);
   operand_layout(bn, &flip_b, &h.ldb, &h.b_sb0, &h.b_sb1);
@@ -250,10 +257,6 @@ void Compiler::CompileCube(int a) {
   const bool trans_a = mm->trans_a != flip_a, trans_b = mm->trans_b != flip_b;  // as the operands lie in memory
   h.trans_a = trans_a ? 1 : 0;
   h.trans_b = trans_b ? 1 : 0;
-  if (M == 0 || N == 0 || h.nb0 == 0 || h.nb1 == 0) {
-    prog_->skip = true;
-    return;
-  }
   // A measured choice of tile and split for this product shape (the online tuner, host/tuner.cc) stands in for the
   // two tuning switches for the rest of this function; a switch the user has set wins.
   struct RestoreTuning {

@@ -106,7 +106,10 @@ bool Config::IsInitialized() const { return g_system.IsInit(); }
 void Throw(const std::string &msg) { DvmException(msg.c_str()); }
 
 void DvmException(const char *error_str) {
-  throw std::runtime_error(std::string("DVM EXCEPTION. reason: ") + error_str);
+  static const char kPrefix[] = "DVM EXCEPTION. reason: ";
+  const std::string msg(error_str);
+  // (some callers spell the prefix out themselves: it appears once either way)
+  throw std::runtime_error(msg.compare(0, sizeof(kPrefix) - 1, kPrefix) == 0 ? msg : kPrefix + msg);
 }
 
 }  // namespace dvm

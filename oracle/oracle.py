@@ -173,9 +173,10 @@ def matmul(a, b, bias, trans_a, trans_b, t):
     k = a.shape[-2] if trans_a else a.shape[-1]
     n = b.shape[-2] if trans_b else b.shape[-1]
     batch = np.broadcast_shapes(a.shape[:-2], b.shape[:-2])
-    ab = np.broadcast_to(a, batch + a.shape[-2:]).reshape((-1,) + a.shape[-2:])
-    bb = np.broadcast_to(b, batch + b.shape[-2:]).reshape((-1,) + b.shape[-2:])
-    out = np.empty((ab.shape[0], m, n), np.float32)
+    nb = int(np.prod(batch, dtype=np.int64))  # (spelled out: a -1 cannot be inferred next to an empty matrix)
+    ab = np.broadcast_to(a, batch + a.shape[-2:]).reshape((nb,) + a.shape[-2:])
+    bb = np.broadcast_to(b, batch + b.shape[-2:]).reshape((nb,) + b.shape[-2:])
+    out = np.empty((nb, m, n), np.float32)
     bias_c = _c(bias, np.float32) if bias is not None else None
     for i in range(ab.shape[0]):
         ai, bi, oi = np.ascontiguousarray(ab[i]), np.ascontiguousarray(bb[i]), out[i]

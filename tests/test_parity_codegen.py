@@ -135,3 +135,28 @@ def test_dynamic_rows_of_4096_around_a_multiple_of_the_workgroup_count():  # tes
         s = (a + b).astype(np.float32)
         assert t.check(out0, a + b) and t.check(out1, s)
         assert t.check(out2, np.sum(s * s, (2,), keepdims=True), 1e-4)
+
+
+@pytest.mark.parametrize("ker", ["vector", "split", "eager"])
+@pytest.mark.parametrize("shape", [[0], [0, 5], [5, 0], [3, 0, 4], [0, 3, 4], [3, 4, 0], [2, 0, 0], [1, 0, 1]])
+def test_an_extent_of_zero_anywhere(ker, shape):
+    # elementwise, casts, reduces over each axis (the sum of nothing is 0), layout operators, a broadcast partner,
+    # and a second output that does have elements, in one kernel each
+    rng = np.random.default_rng(len(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    partner = rng.standard_normal([1 if d == 0 else d for d in shape]).astype(np.float32)
+    full = rng.standard_normal([4, 8]).astype(np.float32)
+    graphs = [lambda k: [k.exp(k.load(x))], lambda k: [k.add(k.mul(k.load(x), 2.0), 1.0)],
+              lambda k: [k.cast(k.load(x), "float16"), k.cast(k.load(x), "int32")],
+              lambda k: [k.sum(k.load(x), tuple(range(len(shape))), True)],
+              lambda k: [k.add(k.load(x), k.load(partner))],
+              lambda k: [k.exp(k.load(x)), k.add(k.load(full), 1.0)],
+              lambda k: [k.select(k.greater(k.load(x), 0.0), k.load(x), k.mul(k.load(x), 2.0))]]
+    for ax in range(len(shape)):
+        graphs += [lambda k, ax=ax: [k.sum(k.load(x), (ax,), True)], lambda k, ax=ax: [k.sum(k.load(x), (ax,), False)]]
+    if len(shape) >= 2:
+        graphs.append(lambda k: [k.add(k.permute(k.load(x), list(range(len(shape)))[::-1]), 1.0)])
+        flat = [int(np.prod(shape[:-1])), shape[-1]] if shape[-1] != 0 else [0]
+        graphs.append(lambda k: [k.mul(k.reshape(k.load(x), flat), 2.0)])
+    for g in graphs:
+        run_graph(ker, lambda k, g=g: [(k.store(v), None, None) for v in g(k)])

@@ -273,3 +273,22 @@ def test_dyn_shape_tuning(mix):  # tests/ut/test_matmul.py:697-718: a dynamic ke
             assert t.check(x3, expect, 2e-3)
     finally:
         Tester.set_lazy_tuning(False)
+
+
+@pytest.mark.parametrize("ker", ["mix", "split"])
+@pytest.mark.parametrize("m,n,k,batch", [(0, 8, 16, ()), (8, 0, 16, ()), (0, 0, 16, ()), (0, 8, 0, ()), (8, 8, 16, (0,))])
+def test_matmul_with_an_empty_result(ker, m, n, k, batch):
+    a, b = np.ones(batch + (m, k), np.float16), np.ones(batch + (k, n), np.float16)
+    t = Tester(ker)
+    plain = t.store(t.matmul(t.load(a), t.load(b), False, False))
+    fused = t.store(t.add(t.cast(t.matmul(t.load(a), t.load(b), False, False), "float32"), 1.0))
+    t.run()
+    assert t.output(plain).shape == batch + (m, n) and t.output(fused).shape == batch + (m, n)
+    assert plain.shape() == batch + (m, n)
+
+
+def test_matmul_over_an_empty_k_axis_is_refused_by_name():
+    t = Tester("mix")
+    t.store(t.matmul(t.load(np.ones([8, 0], np.float16)), t.load(np.ones([0, 8], np.float16)), False, False))
+    with pytest.raises(RuntimeError, match="empty k axis"):
+        t.codegen()
