@@ -310,3 +310,36 @@ def test_sum_of_a_broadcast_stored_beside_its_input():  # tests/ut/test_reduce.p
     t.store_expect(t.sum(x, [0, 2, 3], False), np.sum(wide.astype(np.float64), axis=(0, 2, 3)), 1e-4)
     t.store_expect(x, wide)
     assert t.run_check()
+
+
+def test_tensors_beyond_four_gigabytes():
+    # byte offsets past 2^32 in each schedule: row sums and a normalise sweep (reduce over the innermost axis), column sums
+    # (the innermost axis kept, shared between workgroups), a matmul operand; expectations in closed form
+    rows, cols = 40960, 32768
+    x = np.empty([rows, cols], np.float32)
+    x[:] = (np.arange(rows) % 13).astype(np.float32)[:, None]
+    x[:, ::2] *= -0.5
+    row_sum = ((np.arange(rows) % 13).astype(np.float64) * (cols / 2) * 0.5)[:, None]
+    t = Tester("split")
+    st = t.store(t.sum(t.load(x), (1,), True))
+    t.run()
+    assert np.allclose(t.output(st), row_sum, rtol=1e-5)
+    t = Tester("split")
+    xl = t.load(x)
+    st = t.store(t.sub(xl, t.mul(t.sum(xl, (1,), True), 1.0 / cols)))
+    t.run()
+    assert np.allclose(t.output(st), x - (row_sum / cols).astype(np.float32), rtol=1e-5, atol=1e-4)
+    tall = x.reshape(rows * 2, cols // 2)
+    t = Tester("split")
+    st = t.store(t.sum(t.load(tall), (0,), True))
+    t.run()
+    assert np.allclose(t.output(st), tall.astype(np.float64).sum(0, keepdims=True), rtol=1e-4)
+    del x, tall
+    m, k, n = 65536, 40960, 128
+    a = np.empty([m, k], np.float16)
+    a[:] = (np.arange(m) % 7).astype(np.float16)[:, None]
+    t = Tester("mix")
+    st = t.store(t.matmul(t.load(a), t.load(np.full([k, n], 0.125, np.float16)), False, False))
+    t.run()
+    want = ((np.arange(m) % 7) * k * 0.125).astype(np.float32)[:, None] * np.ones([1, n], np.float32)
+    assert np.array_equal(t.output(st).astype(np.float32), want)
