@@ -301,3 +301,77 @@ def test_slice_mixed_with_casts():  # :104-123 (the reference's [1, 14, 41850, 4
         z = k.add(k.cast(k.load(c), "float32"), k.mul(x, y))
         return [(k.store(k.cast(z, "float16")), g, 1e-3)]
     run_graph("", build)
+
+
+# ---- transposes read through strides, tests/ut/test_view_sch.py:22-106, 221-243, 777-785 (the kernel flag there picks the
+# reference's fractal transpose; the tile counts in its comments are its own) ----
+
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+@pytest.mark.parametrize("h,w", [(1024, 2048), (38, 1024), (1024, 38), (100, 70), (2000, 900), (300, 10), (7, 300), (7, 12)])
+def test_transpose_through_a_strided_load_and_a_strided_store(dtype, h, w):
+    a = rng(h + w).normal(0, 1, (w, h)).astype(dtype)
+    e = np.ascontiguousarray(a.T)
+    run_graph("vector:opt_fractal", lambda k: [(k.view_store_expect(k.view_load([h, w], [1, h], a), [w, 1], e), e, 0)])
+
+
+@pytest.mark.parametrize("shape1,swap1,shape2,swap2,strided_store", [
+    ([10, 64, 200], (1, 2), [10, 64, 200], (1, 2), True), ([4, 70, 20, 200], (1, 3), [1, 70, 20, 200], (1, 3), False),
+    ([10, 1, 200], (1, 2), [10, 128, 200], (1, 2), True), ([10, 200, 1], (1, 2), [10, 200, 128], (1, 2), False),
+    ([5, 3, 32, 1], (2, 3), [5, 3, 32, 129], (2, 3), True)])
+def test_sum_of_two_transposing_loads(shape1, swap1, shape2, swap2, strided_store):
+    a, b = rng(31).normal(0, 1, shape1).astype(np.float32), rng(32).normal(0, 1, shape2).astype(np.float32)
+    ta, tb = np.swapaxes(a, *swap1), np.swapaxes(b, *swap2)
+    s1, s2 = row_major(shape1), row_major(shape2)
+    s1[swap1[0]], s1[swap1[1]] = s1[swap1[1]], s1[swap1[0]]
+    s2[swap2[0]], s2[swap2[1]] = s2[swap2[1]], s2[swap2[0]]
+    e = np.ascontiguousarray(ta + tb)
+
+    def g(k):
+        v = k.add(k.view_load(list(ta.shape), s1, a), k.view_load(list(tb.shape), s2, b))
+        return [(k.view_store_expect(v, row_major(list(e.shape)), e) if strided_store else k.store(v), e, 0)]
+    run_graph("vector:opt_fractal", g)
+
+
+def test_transposed_column_plus_transposed_rows_of_23():
+    lhs = rng(33).normal(0, 1, [1, 1, 2, 1]).astype(np.float16)
+    rhs = rng(34).normal(0, 1, [4, 1, 23, 257]).astype(np.float16)
+    e = np.swapaxes(lhs, 1, 2) + np.swapaxes(rhs, 2, 3)
+
+    def g(k):
+        x = k.view_load([1, 2, 1, 1], [2, 1, 2, 1], lhs)
+        y = k.view_load([4, 1, 257, 23], [5911, 5911, 1, 257], rhs)
+        return [(k.store(k.copy(k.add(x, y))), e, 0)]
+    run_graph("", g)
+
+
+@pytest.mark.parametrize("shape,swap", [([4, 70, 20, 200], (1, 3)), ([2, 2048, 16, 128], (2, 3)), ([129, 128], (0, 1))])
+def test_transpose_of_two_axes_of_a_larger_tensor(shape, swap):
+    a = rng(35).normal(0, 1, shape).astype(np.float16)
+    e = np.ascontiguousarray(np.swapaxes(a, *swap))
+    s = row_major(shape)
+    s[swap[0]], s[swap[1]] = s[swap[1]], s[swap[0]]
+    run_graph("vector:opt_fractal", lambda k: [(k.view_store_expect(k.view_load(list(e.shape), s, a), row_major(list(e.shape)), e), e, 0)])
+
+
+@pytest.mark.parametrize("shape1,shape2", [([3, 18911], [3, 1]), ([2, 18911, 3], [2, 1, 3]), ([3, 15401, 3], [3, 1, 1])])
+@pytest.mark.parametrize("through_strides", [True, False])
+def test_long_odd_rows_plus_a_broadcast_operand(shape1, shape2, through_strides):
+    a, b = rng(36).normal(0, 1, shape1).astype(np.float32), rng(37).normal(0, 1, shape2).astype(np.float32)
+    e = a + b
+
+    def g(k):
+        if through_strides:
+            v = k.add(k.view_load(shape1, row_major(shape1), a), k.view_load(shape2, row_major(shape2), b))
+            return [(k.view_store_expect(v, row_major(list(e.shape)), e), e, 0)]
+        return [(k.store(k.add(k.load(a), k.load(b))), e, 0)]
+    run_graph("", g)
+
+
+def test_split_and_slice_of_a_load_with_gaps_meet_again():
+    a0 = np.arange(64, dtype=np.float32).reshape(8, 8)
+
+    def g(k):
+        vl = k.view_load([8, 4], [8, 2], a0)
+        _, second = k.split(vl, 1, 2, 2)
+        return [(k.store(k.add(second, k.slice(vl, [0, 2], [8, 2]))), 2 * a0[:, [4, 6]], 0)]
+    run_graph("", g)
