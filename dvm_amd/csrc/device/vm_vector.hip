@@ -370,6 +370,12 @@ __device__ __forceinline__ void vm_vector(const VmParam &p) {
               default: FOR_U FOR_E acc.v[u][e] = __int_as_float(__float_as_int(acc.v[u][e]) <= si ? 1 : 0); break;
             }
           }
+          if constexpr (SCHED == VS_REDX) {
+            if (park_slot != 0u) {  // this was the instruction behind a load that parks its round (x * c, x + c)
+              vreg_store(keep_lds, park_slot - 1u, park_fmt, nthreads, tid, acc);
+              park_slot = 0u;
+            }
+          }
           continue;
         }
         // ---- fetch a full-width source operand ----

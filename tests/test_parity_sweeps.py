@@ -168,3 +168,29 @@ def test_unaligned_rows_and_addresses_fall_back_to_the_generic_kernel(monkeypatc
     a, das_on = _run(monkeypatch, True, build)
     assert "reduce-x sweeps" not in das_on, das_on
     assert np.allclose(a[0], x - x.astype(np.float64).mean(1, keepdims=True), rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("sweeps", [True, False])
+@pytest.mark.parametrize("first", ["times a number", "plus a number", "plus a tensor"])
+@pytest.mark.parametrize("n", [40000, 70001])
+def test_parked_rounds_hold_the_value_behind_the_first_instruction(monkeypatch, sweeps, first, n):
+    # Both sweeps open with [load x] [one float binary]: the rounds that stay in local memory hold that binary's
+    # result, whatever its operand is. (With a number as the operand the generic kernel once parked the value behind
+    # the instruction after it.) A store of a V register between the sweeps keeps the program off the sweep build.
+    rng = np.random.default_rng(n)
+    x, y = rng.uniform(0.25, 2.0, [n]).astype(np.float32), rng.uniform(0.25, 2.0, [n]).astype(np.float32)
+    head = {"times a number": lambda k, a, b: k.mul(a, -1.0), "plus a number": lambda k, a, b: k.add(a, 0.75),
+            "plus a tensor": lambda k, a, b: k.add(a, b)}[first]
+    h64 = {"times a number": -x.astype(np.float64), "plus a number": x.astype(np.float64) + 0.75,
+           "plus a tensor": x.astype(np.float64) + y}[first]
+    v64 = h64 * x
+    want = v64.max() - v64 / (np.abs(v64) + 0.5)
+
+    def build(k):
+        a, b = k.load(x), k.load(y)
+        v = k.mul(head(k, a, b), a)
+        top = k.max(v, (0,), True)
+        return [k.store(k.sub(top, k.div(v, k.add(k.abs(v), 0.5))))]
+    (out,), das = _run(monkeypatch, sweeps, build)
+    assert "parks its first" in das, das
+    assert np.allclose(out, want, rtol=1e-5, atol=1e-6), (np.abs(out - want).max(), das)
