@@ -38,8 +38,7 @@ def _check(case, build, ker, refs, skip=()):
 
 
 @gpu
-@pytest.mark.parametrize("first", range(0, 4 * CHUNK, CHUNK))
-@pytest.mark.parametrize("big", [False, True])
+@pytest.mark.parametrize("first,big", [(f, False) for f in range(0, 4 * CHUNK, CHUNK)] + [(f, True) for f in range(0, 12 * CHUNK, CHUNK)])
 def test_pointwise_and_reduce_graphs(first, big):
     for case in range(first, first + CHUNK):
         build = R.pointwise_reduce_graph(case, big)
