@@ -197,10 +197,16 @@ void Compiler::MarkUniformRuns() {
   out.clear();
   out.reserve(code_.size() + 8);
   bool in_sweep = false;
+  // The waves that skip a run never compute the offsets of its memory operands: the first memory instruction behind
+  // the run that would reuse them (VI_SAME_OFFS) computes its own instead.
+  bool offsets_stale = false;
   for (size_t i = 0; i < code_.size();) {
-    const uint64_t w = code_[i];
+    uint64_t w = code_[i];
     const uint32_t op = VI_OP(w);
-    if (op == VOP_SWEEP) in_sweep = true;
+    if (op == VOP_SWEEP) {
+      in_sweep = true;
+      offsets_stale = false;  // (a sweep starts from offsets of its own)
+    }
     if (static_cast<uint32_t>(w) & VI_ENDS) {
       in_sweep = false;
     }
@@ -211,8 +217,17 @@ void Compiler::MarkUniformRuns() {
         out.push_back(VI_MAKE(VOP_UNI_BEGIN, 0, 0, 0, 0, static_cast<uint32_t>(j - i + 1)));
         out.insert(out.end(), code_.begin() + i, code_.begin() + j);
         out.push_back(VI_MAKE(VOP_UNI_END, 0, 0, 0, 0, 0));
+        for (size_t q = i; q < j; ++q) offsets_stale = offsets_stale || (VI_OP(code_[q]) >= VOP_SRC_BASE && VI_KIND(code_[q]) == VK_MEM);
         i = j;
         continue;
+      }
+    }
+    if (offsets_stale && (op == VOP_ST || (op >= VOP_SRC_BASE && VI_KIND(w) == VK_MEM))) {
+      if (static_cast<uint32_t>(w) & VI_SAME_OFFS) {
+        w &= ~static_cast<uint64_t>(VI_SAME_OFFS);
+        offsets_stale = false;
+      } else if (!(static_cast<uint32_t>(w) & VI_OFFS_ASIDE)) {
+        offsets_stale = false;  // offsets of its own, current from here on
       }
     }
     out.push_back(w);

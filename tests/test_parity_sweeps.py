@@ -194,3 +194,27 @@ def test_parked_rounds_hold_the_value_behind_the_first_instruction(monkeypatch, 
     (out,), das = _run(monkeypatch, sweeps, build)
     assert "parks its first" in das, das
     assert np.allclose(out, want, rtol=1e-5, atol=1e-6), (np.abs(out - want).max(), das)
+
+
+@pytest.mark.parametrize("sweeps", [True, False])
+@pytest.mark.parametrize("rows,cols", [(500, 4096), (37, 1000), (3, 20000)])
+def test_operand_read_inside_a_per_output_run_and_again_behind_it(monkeypatch, sweeps, rows, cols):
+    # A per-row value is loaded inside a run that only the first wave of the workgroup executes, stored, and loaded
+    # again behind the run: the waves that skipped the run have to compute that operand's offsets themselves.
+    # (They once reused offsets they never had, and every row but the first read the first row's value.)
+    rng = np.random.default_rng(rows)
+    c = rng.uniform(0.25, 2.0, [rows, 1]).astype(np.float32)
+    x = rng.uniform(0.25, 2.0, [rows, cols]).astype(np.float16)
+    e = np.exp(c.astype(np.float64) * 0.125)
+    d = x.astype(np.float64) - e * c
+
+    def build(k):
+        cv = k.load(c)
+        ev = k.exp(k.mul(cv, 0.125))
+        diff = k.sub(k.cast(k.load(x), "float32"), k.mul(ev, cv))
+        return [k.store(k.cast(k.cast(ev, "float16"), "float32")), k.store(diff), k.store(k.sum(diff, (1,), True))]
+    (o0, o1, o2), das = _run(monkeypatch, sweeps, build)
+    assert "per-output run" in das, das
+    assert np.allclose(o0, e.astype(np.float16).astype(np.float32), rtol=1e-3)
+    assert np.allclose(o1, d, rtol=1e-5, atol=1e-5), np.abs(o1 - d).max()
+    assert np.allclose(o2, d.sum(1, keepdims=True), rtol=1e-4, atol=1e-3)
