@@ -78,6 +78,17 @@ void Compiler::PairLoads() {
       const uint64_t w = code_[i], nx = code_[i + 1];
       if (VI_OP(code_[i - 1]) != VOP_SWEEP || VI_OP(w) != VOP_LD || (static_cast<uint32_t>(w) & (VI_UNIFORM | VI_LD_PAIR))) continue;
       if (VI_OP(nx) != VOP_RED || !(static_cast<uint32_t>(nx) & VI_ENDS) || (VI_SUB(nx) & VRF_INT)) continue;
+      // The fused path leaves no particular round in the accumulator. What follows the sweep may read it (an
+      // operand that does not vary along the reduced axes is taken from the last round instead of being loaded
+      // again): then the load stays an ordinary one.
+      bool acc_dead = false;
+      for (size_t q = i + 2; q < code_.size(); ++q) {
+        const uint32_t qop = VI_OP(code_[q]);
+        if (qop == VOP_UNI_BEGIN || qop == VOP_SWEEP || qop == VOP_ENDSWEEP) continue;
+        acc_dead = qop == VOP_END || qop == VOP_FIN || qop == VOP_LDS || qop == VOP_LDI || qop == VOP_LD;
+        break;
+      }
+      if (!acc_dead) continue;
       code_[i] = w | VI_LD_RED2;
     }
   }

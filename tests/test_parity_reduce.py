@@ -343,3 +343,20 @@ def test_tensors_beyond_four_gigabytes():
     t.run()
     want = ((np.arange(m) % 7) * k * 0.125).astype(np.float32)[:, None] * np.ones([1, n], np.float32)
     assert np.array_equal(t.output(st).astype(np.float32), want)
+
+
+@pytest.mark.parametrize("rows,cols", [(7, 8), (300, 4096), (33, 1000)])
+@pytest.mark.parametrize("red", ["min", "max", "sum"])
+def test_reduce_over_the_repeats_of_a_broadcast_that_is_used_again(rows, cols, red):
+    # The value that is reduced over axis 0 does not vary along it (a row repeated): what follows takes it from the
+    # accumulator of the last round instead of loading it again, so the load of that sweep must leave it there.
+    # (The load that fetches several rounds per trip and reduces them itself did not.)
+    x = np.random.default_rng(rows).uniform(0.25, 2.0, [1, cols]).astype(np.float32)
+    want = {"min": x, "max": x, "sum": x * np.float32(rows)}[red] + np.broadcast_to(x, (rows, cols))
+
+    def g(k, a):
+        b = k.broadcast(a, [rows, cols])
+        m = getattr(k, red)(b, (0,), True)
+        picked = k.select(k.greater(m, a), a, m)  # (the reduce result either way for min; keeps the graph of the failing case)
+        return k.add(picked if red == "min" else m, b)
+    run_parity(g, [x], ker="split", golden=want, eps=1e-5)
