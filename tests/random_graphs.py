@@ -30,7 +30,12 @@ def close_enough(out, ref, exact):
         return not bad.any() or (bad.mean() < 0.01 and np.nanmax(np.where(bad, d / (np.abs(b) + 1e-3), 0)) < 1e-2)
 
 
-def pointwise_reduce_graph(case, big=False):
+# further operators of the generator below (more=True): reduces to the minimum, over two axes and without keepdims,
+# logarithm, reciprocal square root, minimum, numbers on either side
+MORE_OPS = ["min", "sum2", "sumnk", "log", "abs", "rsqrt", "minimum", "square", "recip", "maxnk", "mulc", "subc"]
+
+
+def pointwise_reduce_graph(case, big=False, more=False):
     rng = np.random.default_rng(case)
     rank = int(rng.integers(1, 4))
     big = int(big)
@@ -46,7 +51,7 @@ def pointwise_reduce_graph(case, big=False):
         dt = str(rng.choice(["float32", "float32", "float16", "bfloat16"]))
         arr = rng.uniform(0.25, 2.0, sh).astype(np.float32)
         ins.append((arr, dt))
-    prog = [(str(rng.choice(["add", "mul", "sub", "div", "exp", "sqrt", "cast16", "castbf", "cast32", "sum", "max", "bcast", "select", "neg", "maximum", "reshape", "addc"])), int(rng.integers(0, 1 << 30))) for _ in range(int(rng.integers(2, 9 + 6 * big)))]
+    prog = [(str(rng.choice(["add", "mul", "sub", "div", "exp", "sqrt", "cast16", "castbf", "cast32", "sum", "max", "bcast", "select", "neg", "maximum", "reshape", "addc"] + (MORE_OPS if more else []))), int(rng.integers(0, 1 << 30))) for _ in range(int(rng.integers(2, 9 + 6 * big)))]
     n_out = int(rng.integers(1, 3 + big))
     # plan the graph on the oracle (its shapes are known at once) and record it as a tape both builders replay
     tape = []
@@ -64,7 +69,11 @@ def pointwise_reduce_graph(case, big=False):
                 compat = False
             step = None
             if name in ("add", "mul", "sub", "div", "maximum") and compat: step = (name, xi, yi, None)
-            elif name in ("exp", "sqrt", "cast16", "castbf", "cast32", "neg"): step = (name, xi, None, None)
+            elif name in ("exp", "sqrt", "cast16", "castbf", "cast32", "neg", "log", "abs", "rsqrt", "square", "recip"): step = (name, xi, None, None)
+            elif name == "minimum" and compat: step = (name, xi, yi, None)
+            elif name in ("mulc", "subc"): step = (name, xi, None, float(r.random()) + 0.5)
+            elif name in ("min", "sumnk", "maxnk") and len(xs) > 0: step = (name, xi, None, int(r.integers(0, len(xs))))
+            elif name == "sum2" and len(xs) > 1: step = (name, xi, None, tuple(sorted({int(r.integers(0, len(xs))), int(r.integers(0, len(xs)))})))
             elif name == "addc": step = (name, xi, None, float(r.random()))
             elif name in ("sum", "max") and len(xs) > 0: step = (name, xi, None, int(r.integers(0, len(xs))))
             elif name == "bcast" and len(xs) > 0:
@@ -90,6 +99,18 @@ def pointwise_reduce_graph(case, big=False):
         if name == "castbf": return f32(k.cast(x, "bfloat16"))
         if name == "cast32": return f32(x)
         if name in ("sum", "max"): return getattr(k, name)(x, (prm,), True)
+        if name == "min": return k.min(x, (prm,), True)
+        if name == "sumnk": return k.sum(x, (prm,), False)
+        if name == "maxnk": return k.max(x, (prm,), False)
+        if name == "sum2": return k.sum(x, prm, True)
+        if name == "log": return k.log(k.add(k.abs(x), 0.25))
+        if name == "abs": return k.abs(x)
+        if name == "rsqrt": return k.div(1.0, k.sqrt(k.add(k.abs(x), 0.25)))
+        if name == "square": return k.mul(x, x)
+        if name == "recip": return k.reciprocal(k.add(k.abs(x), 0.5))
+        if name == "minimum": return k.minimum(x, y)
+        if name == "mulc": return k.mul(x, prm)
+        if name == "subc": return k.sub(prm, x)
         if name == "bcast": return k.broadcast(x, prm)
         if name == "select": return k.select(k.greater(x, y), x, y)
         if name == "neg": return k.mul(x, -1.0)

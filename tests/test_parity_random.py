@@ -38,10 +38,11 @@ def _check(case, build, ker, refs, skip=()):
 
 
 @gpu
-@pytest.mark.parametrize("first,big", [(f, False) for f in range(0, 4 * CHUNK, CHUNK)] + [(f, True) for f in range(0, 12 * CHUNK, CHUNK)])
-def test_pointwise_and_reduce_graphs(first, big):
+@pytest.mark.parametrize("first,big,more", [(f, False, False) for f in range(0, 4 * CHUNK, CHUNK)] +
+                         [(f, True, False) for f in range(0, 12 * CHUNK, CHUNK)] + [(f, True, True) for f in range(0, 12 * CHUNK, CHUNK)])
+def test_pointwise_and_reduce_graphs(first, big, more):
     for case in range(first, first + CHUNK):
-        build = R.pointwise_reduce_graph(case, big)
+        build = R.pointwise_reduce_graph(case, big, more)
         try:
             refs = _oracle(build)
         except Exception:
